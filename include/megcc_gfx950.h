@@ -1,0 +1,373 @@
+/*
+ * megcc_gfx950.h -- C ABI of libmegcc_gfx950.so: MI355X (gfx950) implementations of the
+ * per-operator kernels MegCC's KernelGen emits and its TinyNN VM calls.
+ *
+ * Boundary being replaced (all citations relative to the MegCC tree):
+ *   - every generated kernel has the uniform signature
+ *         TinyNNStatus S(Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+ *                        const Workspace* workspace, const RuntimeOpt* opt);
+ *     with companions S_init / S_workspace (runtime/src/data_struct.h:131-153, emitted by
+ *     compiler/lib/KernelGen/KernelGen.cpp:130-153) and is called from execute_single_opr
+ *     (runtime/src/vm/op.c:161-163) and init_model_weights (runtime/src/init.c:29-131).
+ *   - everything that is *not* a run-time tensor (window, stride, padding, layout format,
+ *     activation ...) is baked into the generated symbol S at compile time. Here those
+ *     attributes travel in a small constant "attr" struct placed in front of the uniform
+ *     argument list; the KernelGen target for this arch emits, per symbol S, a three-line C
+ *     shim `S(...) { static const MegccConvAttr a = {...}; return megcc_gfx950_conv2d(&a, ...); }`.
+ *
+ * All Tensor.ptr / Workspace.ptr / out_weights->ptr are DEVICE pointers obtained through the
+ * Device.malloc hook installed by megcc_gfx950_init_device(). Kernels are launched
+ * asynchronously on one library-owned stream, in call order; results are visible to the host
+ * after megcc_gfx950_wait() or a megcc_gfx950_memcpy_d2h().
+ *
+ * There is no CPU fallback anywhere in the library: an operator / layout / dtype combination that
+ * has no gfx950 kernel returns TinyNN_ERROR_NO_IMPLEMENT.
+ */
+#ifndef MEGCC_GFX950_H
+#define MEGCC_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * Run-time ABI types. Field order, widths and enum values are those of
+ * runtime/src/tinynn.h:7-54, runtime/src/device.h:8-21 and runtime/src/data_struct.h:12-59 so
+ * that a Tensor built by the TinyNN runtime can be handed over unchanged. When the reference's
+ * own data_struct.h has been included first, its definitions are used instead.
+ * ---------------------------------------------------------------------------------------- */
+#ifndef DATA_STRUCT_H
+
+#define MAX_DIM (7)
+
+typedef enum {
+    TinyNN_SUCCESS = 0,
+    TinyNN_ERROR_NULL_PTR = 1,
+    TinyNN_ERROR_STANDER = 2,
+    TinyNN_ERROR_RUNTIME = 3,
+    TinyNN_ERROR_OUT_OF_RANGE = 4,
+    TinyNN_ERROR_NO_FOUND = 5,
+    TinyNN_ERROR_NO_IMPLEMENT = 6,
+    TinyNN_ERROR_MODEL_PARSE = 7,
+    TinyNN_ERROR_OPEN_FILE_ERROR = 8,
+    TinyNN_ERROR_MEMORY_MALLOC = 9,
+    TinyNN_ERROR_UNSUPPORTED_INSTRUCTION_TYPE = 10,
+    TinyNN_ERROR_UNSUPPORTED_DTYPE_TYPE = 11,
+    TinyNN_ERROR_INVALID_LAYOUT = 12,
+    TinyNN_ERROR = 13
+} TinyNNStatus;
+
+typedef enum {
+    TinyNN_FLOAT = 0,
+    TinyNN_FLOAT16 = 1,
+    TinyNN_INT = 2,
+    TinyNN_INT8 = 3,
+    TinyNN_INT16 = 4,
+    TinyNN_UINT8 = 5,
+    TinyNN_QINT8 = 100,
+    TinyNN_QINT32 = 101,
+    TinyNN_QUINT8 = 102
+} TinyNNDType;
+
+typedef enum { TinyNN_NCHW = 0, TinyNN_NHWC, TinyNN_NCHW4, TinyNN_NCHW8, TinyNN_OIHW } TinyNNFormat;
+
+typedef enum {
+    TinyNN_BARE_METAL = 0,
+    TinyNN_ARM64,
+    TinyNN_ARM32,
+    TinyNN_ARM64_V82,
+    TinyNN_ARM32_V82,
+    TinyNN_OPENCL_MALI,
+    TinyNN_WEB_ASSEMBLY
+} TinyNNDevice;
+
+typedef struct {
+    int alignment;
+    TinyNNDevice device_type;
+    void* (*malloc)(size_t length);
+    void (*free)(void* ptr);
+} Device;
+
+typedef struct RuntimeOpt {
+    const Device* device;
+} RuntimeOpt;
+
+typedef struct {
+    float scale;
+    uint8_t zero_point;
+} DTypeParam;
+
+typedef struct {
+    TinyNNDType type_enum;
+    DTypeParam param;
+} DType;
+
+typedef struct {
+    int nr_dim;
+    uint32_t dims[MAX_DIM];
+    int stride[MAX_DIM]; /* in elements */
+    TinyNNFormat format;
+} Layout;
+
+typedef struct Tensor {
+    char* name;
+    DType dtype;
+    Layout layout;
+    void* ptr;
+    size_t offset;
+    int use_count;
+    int is_weight;
+    int is_dynamic;
+    uint32_t checksum;
+    size_t size;
+    int is_shared;
+    int is_input;
+} Tensor;
+
+typedef struct {
+    void* ptr;
+    size_t size;
+    size_t offset;
+} Workspace;
+
+#endif /* DATA_STRUCT_H */
+
+/* Value of Device.device_type reported by megcc_gfx950_init_device(): the next free slot after
+ * runtime/src/tinynn.h:46-54 (TinyNN_WEB_ASSEMBLY = 6). */
+#define TinyNN_GFX950 ((TinyNNDevice)7)
+
+/* ------------------------------------------------------------------------------------------
+ * Compile-time attributes (what the reference bakes into the kernel symbol).
+ * ---------------------------------------------------------------------------------------- */
+typedef enum {
+    MEGCC_FMT_NCHW = 0,        /* "NCHW"  : [N,C,H,W]                                      */
+    MEGCC_FMT_NCHW44 = 1,      /* "NCHW44": [N,C/4,H,W,4]                                  */
+    MEGCC_FMT_NCHW_NCHW44 = 2  /* "NCHW44" with a 4-D source: NCHW in, NCHW44 out (first layer) */
+} MegccFormat;
+
+typedef enum { MEGCC_SPARSE_DENSE = 0, MEGCC_SPARSE_GROUP = 1 } MegccSparse;
+
+typedef enum {
+    MEGCC_NONLINE_IDENTITY = 0,
+    MEGCC_NONLINE_RELU = 1,
+    MEGCC_NONLINE_H_SWISH = 2,
+    MEGCC_NONLINE_SIGMOID = 3
+} MegccNonline;
+
+/* ConvBias attributes: the keys KernelMaterialization hands to KernelGen
+ * (compiler/test/kernel/common/src/cc_fill_attr.cpp:253-274). */
+typedef struct {
+    uint32_t kernel_h, kernel_w;
+    uint32_t stride_h, stride_w;
+    uint32_t pad_h, pad_w;
+    uint32_t dilate_h, dilate_w;
+    MegccFormat format;
+    MegccSparse sparse;
+    MegccNonline nonline;
+    int with_bias; /* Common/ConvKernel.h:10-13 "is_bias" */
+} MegccConvAttr;
+
+typedef enum {
+    MEGCC_POOL_MAX = 0,
+    MEGCC_POOL_AVERAGE = 1,
+    MEGCC_POOL_AVERAGE_COUNT_EXCLUDE_PADDING = 2
+} MegccPoolMode;
+
+/* cc_fill_attr.cpp:276-292 */
+typedef struct {
+    uint32_t window_h, window_w;
+    uint32_t stride_h, stride_w;
+    uint32_t pad_h, pad_w;
+    MegccFormat format; /* NCHW or NCHW44 */
+    MegccPoolMode mode;
+} MegccPoolAttr;
+
+/* cc_fill_attr.cpp:304-317; only format DEFAULT (row-major) is on this path */
+typedef struct {
+    int transpose_a;
+    int transpose_b;
+} MegccMatMulAttr;
+
+typedef enum {
+    MEGCC_Q_ADD = 0,
+    MEGCC_Q_FUSE_ADD_RELU = 1,
+    MEGCC_Q_MUL = 2,
+    MEGCC_Q_RELU = 3
+} MegccMultiTypeMode;
+
+typedef enum {
+    MEGCC_EW_RELU = 0,
+    MEGCC_EW_EXP = 1,
+    MEGCC_EW_SIGMOID = 2,
+    MEGCC_EW_H_SWISH = 3,
+    MEGCC_EW_NEGATE = 4,
+    MEGCC_EW_ADD = 16,
+    MEGCC_EW_SUB = 17,
+    MEGCC_EW_MUL = 18,
+    MEGCC_EW_TRUE_DIV = 19,
+    MEGCC_EW_MAX = 20,
+    MEGCC_EW_MIN = 21,
+    MEGCC_EW_FUSE_ADD_RELU = 22
+} MegccElemwiseMode;
+
+typedef enum {
+    MEGCC_REDUCE_SUM = 0,
+    MEGCC_REDUCE_MEAN = 1,
+    MEGCC_REDUCE_MAX = 2,
+    MEGCC_REDUCE_MIN = 3
+} MegccReduceMode;
+
+typedef struct {
+    MegccReduceMode mode;
+    int axis;
+} MegccReduceAttr;
+
+/* ------------------------------------------------------------------------------------------
+ * Operator entry points. After the attr pointer the argument lists are exactly KernelFunc /
+ * InitFunc / WorkspaceFunc of runtime/src/data_struct.h:131-153.
+ * ---------------------------------------------------------------------------------------- */
+
+/* ConvBias. Replaces BareMetal::ConvGeneral (compiler/lib/KernelGen/BareMetal/ConvKernel.cpp:
+ * 178-389) for qsi8 x qsi8 (+qsi32 bias) -> qsi8 and f32, formats NCHW / NCHW44 / NCHW->NCHW44,
+ * DENSE and GROUP, and GeneralIntrinsic::ConvIm2colFloat (GeneralIntrinsic/ConvKernel/
+ * Fp32Im2col.cpp:88-218) for f32 NCHW DENSE.
+ * inputs = {src, filter[, bias]}, outputs = {dst}. qsi8 results are bit-identical with the
+ * reference: int32 accumulate, + int32 bias, (float)acc * src_scale * flt_scale / dst_scale in
+ * IEEE fp32, activation, roundf, saturate (BareMetal/Activation.cpp:47-56,105-114). */
+TinyNNStatus megcc_gfx950_conv2d(
+        const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace* workspace, const RuntimeOpt* opt);
+/* Three-phase weight pre-processing protocol of Utils/StringTemplate.cpp:106-135 /
+ * runtime/src/init.c:94-131: (out_weights==NULL) -> *nr_out_weight = number of processed weights;
+ * (nr_out_weight==NULL) -> fill out_weights[i].layout/dtype/name; both non-NULL -> write the
+ * processed weights into out_weights[i].ptr (device memory allocated by the caller). Dense qsi8
+ * NCHW44 / NCHW convolutions that run on the MFMA kernel repack the filter into K-major 32-byte
+ * rows; every other case reports 0 processed weights. */
+TinyNNStatus megcc_gfx950_conv2d_init(
+        const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor* out_weights,
+        int* nr_out_weight, const RuntimeOpt* opt);
+/* Always 0 bytes: padding and im2col are folded into the LDS loads (the reference's optimised
+ * paths copy a padded source into workspace, e.g. GeneralIntrinsic/ConvKernel/Im2colCommon.cpp:
+ * 326-377). Plain C semantics, no side effects, so the compiler may evaluate it at compile time
+ * as compiler/lib/KernelGen/Jit/JitExe.cpp:67-123 does. */
+TinyNNStatus megcc_gfx950_conv2d_workspace(
+        const MegccConvAttr* attr, Tensor** inputs, int nr_input, int nr_thread,
+        size_t* workspace);
+
+/* f32 MatrixMul, row-major, C = op(A) * op(B), no bias. Replaces GeneralIntrinsic::
+ * Fp32MatMulM4N12 (GeneralIntrinsic/MatMulKernel/Fp32MatMulM4N12.cpp:9-158), Fp32GevmKernel
+ * (GeneralIntrinsic/MatMulKernel/Fp32Gevm.cpp:50-119) and BareMetal::MatrixMulKernel
+ * (BareMetal/MatrixMul.cpp:13-120). Leading dimensions are layout.stride[0].
+ * (The reference has no qsi8 MatrixMul on this arch: a quantized FullyConnected is the 1x1 NCHW
+ * convolution above on [M,K,1,1] x [N,K,1,1].) */
+TinyNNStatus megcc_gfx950_matmul(
+        const MegccMatMulAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs,
+        int nr_output, const Workspace* workspace, const RuntimeOpt* opt);
+TinyNNStatus megcc_gfx950_matmul_workspace(
+        const MegccMatMulAttr* attr, Tensor** inputs, int nr_input, int nr_thread,
+        size_t* workspace);
+
+/* Pooling qsi8 / f32. Replaces BareMetal::PoolingKernel (BareMetal/Pooling.cpp:166-273, NCHW) and
+ * GeneralIntrinsic::PoolingNchw44QInt8 (GeneralIntrinsic/PoolingKernel/QInt8PoolingNCHW44.cpp:
+ * 116-216, NCHW44). inputs = {src}, outputs = {dst}. */
+TinyNNStatus megcc_gfx950_pooling(
+        const MegccPoolAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace* workspace, const RuntimeOpt* opt);
+
+/* Quantized elementwise QADD / QFUSE_ADD_RELU / QMUL (inputs = {a, b}) and QRELU (inputs = {a});
+ * b may equal a in shape, be [1,C,1,1...] or a single element. Replaces
+ * BareMetal::ElemwiseMultiTypeKernel (BareMetal/ElemwiseMultiType.cpp:16-213). */
+TinyNNStatus megcc_gfx950_elemwise_multitype(
+        const MegccMultiTypeMode* mode, Tensor** inputs, int nr_input, Tensor** outputs,
+        int nr_output, const Workspace* workspace, const RuntimeOpt* opt);
+
+/* f32 elementwise, unary or binary with the same broadcast rules as above plus a trailing-axis
+ * vector ([M,N] op [N], the FullyConnected bias). Replaces GeneralIntrinsic::ElemwiseKernel
+ * (GeneralIntrinsic/Elemwise/Elemwise.cpp:10-36) / BareMetal::ElmwiseKernel
+ * (BareMetal/ElemwiseKernel.cpp:35-66,413-431). */
+TinyNNStatus megcc_gfx950_elemwise(
+        const MegccElemwiseMode* mode, Tensor** inputs, int nr_input, Tensor** outputs,
+        int nr_output, const Workspace* workspace, const RuntimeOpt* opt);
+
+/* TypeCvt f32->qsi8, qsi8->f32, qsi8->qsi8 (GeneralIntrinsic/Typecvt.cpp:71-295: one premultiplied
+ * scale = src_scale/dst_scale) and qsi32->qsi8 (BareMetal/Typecvt.cpp:43-105: val*src/dst).
+ * Directions are taken from the tensors' dtype; no attr. */
+TinyNNStatus megcc_gfx950_typecvt(
+        Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace* workspace, const RuntimeOpt* opt);
+
+/* f32 reduce over one axis of a contiguous tensor viewed as [A,B,C] (BareMetal/Reduce.cpp:73-134,
+ * GeneralIntrinsic/Reduce.cpp:605-613). */
+TinyNNStatus megcc_gfx950_reduce(
+        const MegccReduceAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs,
+        int nr_output, const Workspace* workspace, const RuntimeOpt* opt);
+
+/* ------------------------------------------------------------------------------------------
+ * Dispatch by the reference's kernel symbol: lets a caller that only knows the generated name
+ * (e.g. "kernel_conv2d_3x3_NCHW44_DENSE_p1x1_s1x1_d1x1_qsi8qsi8qsi32qsi8_bias_RELU",
+ * BareMetal/ConvKernel.cpp:144-176; "kernel_pooling_MAX_NCHW_p0x0_s2x2_w2x2_qsi8qsi8",
+ * BareMetal/Pooling.cpp:31-44; GI_* aliases of the same operators) reach the entry points above.
+ * ---------------------------------------------------------------------------------------- */
+typedef enum {
+    MEGCC_KERN_CONV = 1,
+    MEGCC_KERN_MATMUL = 2,
+    MEGCC_KERN_POOLING = 3,
+    MEGCC_KERN_ELEMWISE_MULTITYPE = 4,
+    MEGCC_KERN_ELEMWISE = 5,
+    MEGCC_KERN_TYPECVT = 6,
+    MEGCC_KERN_REDUCE = 7
+} MegccKernelKind;
+
+typedef struct {
+    MegccKernelKind kind;
+    union {
+        MegccConvAttr conv;
+        MegccMatMulAttr matmul;
+        MegccPoolAttr pool;
+        MegccMultiTypeMode multitype;
+        MegccElemwiseMode elemwise;
+        MegccReduceAttr reduce;
+    } attr;
+} MegccKernelDesc;
+
+/* TinyNN_ERROR_NO_FOUND when the symbol is not one of this path's operators. */
+TinyNNStatus megcc_gfx950_parse_symbol(const char* symbol, MegccKernelDesc* desc);
+TinyNNStatus megcc_gfx950_call(
+        const MegccKernelDesc* desc, Tensor** inputs, int nr_input, Tensor** outputs,
+        int nr_output, const Workspace* workspace, const RuntimeOpt* opt);
+TinyNNStatus megcc_gfx950_call_init(
+        const MegccKernelDesc* desc, Tensor** inputs, int nr_input, Tensor* out_weights,
+        int* nr_out_weight, const RuntimeOpt* opt);
+TinyNNStatus megcc_gfx950_call_workspace(
+        const MegccKernelDesc* desc, Tensor** inputs, int nr_input, int nr_thread,
+        size_t* workspace);
+
+/* ------------------------------------------------------------------------------------------
+ * Device seam: what runtime/src/device.c:29-43 (init_device) and the Lite C API's staging points
+ * (runtime/src/lite/tensor.c:93-112 LITE_reset_tensor_memory, lite/network.c:229-232 LITE_wait)
+ * need from a GPU device.
+ * ---------------------------------------------------------------------------------------- */
+/* Fills alignment (256), device_type and the HBM malloc/free hooks. */
+TinyNNStatus megcc_gfx950_init_device(Device* device);
+/* The hooks themselves (plain hipMalloc/hipFree: the TinyNN runtime asks for ONE arena per model,
+ * runtime/src/init.c:437-487, plus one block per weight). */
+void* megcc_gfx950_malloc(size_t length);
+void megcc_gfx950_free(void* ptr);
+/* Stream-ordered copies on the library stream (input staging / output fetch). d2h waits. */
+TinyNNStatus megcc_gfx950_memcpy_h2d(void* dst_device, const void* src_host, size_t length);
+TinyNNStatus megcc_gfx950_memcpy_d2h(void* dst_host, const void* src_device, size_t length);
+TinyNNStatus megcc_gfx950_memset(void* dst_device, int value, size_t length);
+/* Blocks until every kernel launched so far has finished (LITE_wait). */
+TinyNNStatus megcc_gfx950_wait(void);
+/* The hipStream_t all kernels are launched on, for callers that time with HIP events. */
+void* megcc_gfx950_stream(void);
+/* Text of the most recent error on the calling thread ("" if none). */
+const char* megcc_gfx950_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MEGCC_GFX950_H */

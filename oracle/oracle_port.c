@@ -1,0 +1,408 @@
+/*
+ * TEST INFRASTRUCTURE ONLY -- CPU restatement ("port") of the arithmetic of MegCC's generated
+ * x86/BAREMETAL kernels for the conv / matmul / pooling / elemwise / typecvt path. It exists to
+ * check the gfx950 kernels and to serve as bench.py's cpu_baseline leg; nothing in the product
+ * library includes, links or calls it.
+ *
+ * Every function cites the generator it restates (paths relative to the MegCC tree,
+ * compiler/lib/KernelGen/...). Integer accumulation is exact, so loop order is free there; every
+ * *float* expression keeps the reference's operand order and is compiled with
+ * -ffp-contract=off -fno-fast-math (see oracle/Makefile) so that no FMA or re-association can
+ * change a result.
+ *
+ * Pinning: tests/test_oracle.py runs each function against the reference's own generated C
+ * (oracle/_ref/libmegcc_ref.so, built by `make ref` where the reference tree exists) and against
+ * the fixtures under tests/golden/ that were produced from it. Functions without such a check:
+ * none.  Known limit: `int r = roundf(x)` for |x| >= 2^31 is undefined behaviour in the
+ * reference (BareMetal/Activation.cpp:50); it is unreachable with int8 data and sane scales and is
+ * not restated.
+ *
+ * Threads: orc_set_threads(n) lets the *tests* spread the outer loop over n cores; the default
+ * and the cpu_baseline use 1 (the reference runtime is single-threaded).
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+static int g_threads = 1;
+void orc_set_threads(int n) {
+    g_threads = n < 1 ? 1 : n;
+}
+
+enum { FMT_NCHW = 0, FMT_NCHW44 = 1, FMT_NCHW_NCHW44 = 2 };
+enum { ACT_IDENTITY = 0, ACT_RELU = 1, ACT_H_SWISH = 2, ACT_SIGMOID = 3 };
+
+/* BareMetal/Activation.cpp:9-42 -- the helper functions the generator pastes in front of a
+ * kernel; `min`/`max` there are `a > b ? b : a` and `a > b ? a : b`. */
+static inline float act_apply(int act, float x) {
+    switch (act) {
+        case ACT_RELU:
+            return x > 0 ? x : 0;
+        case ACT_H_SWISH: {
+            float t = x + 3;
+            float mx = t > 0.f ? t : 0.f;
+            float mn = mx > 6.f ? 6.f : mx;
+            return x * mn * (1.f / 6.f);
+        }
+        case ACT_SIGMOID:
+            return 1.f / (expf(-x) + 1.f);
+        default:
+            return x;
+    }
+}
+
+/* BareMetal/Activation.cpp:47-56 fp32_to_int8 */
+static inline int8_t fp32_to_int8(float src) {
+    int res = roundf(src);
+    res = res > 127 ? 127 : res;
+    res = res < -128 ? -128 : res;
+    return (int8_t)res;
+}
+
+/* element offset of (n, c, h, w): BareMetal/FormatHelper.cpp:12-36 on a contiguous tensor */
+static inline size_t off_nchw(int C, int H, int W, int n, int c, int h, int w) {
+    return (((size_t)n * C + c) * H + h) * W + w;
+}
+static inline size_t off_nchw44(int C, int H, int W, int n, int c, int h, int w) {
+    return ((((size_t)n * (C / 4) + c / 4) * H + h) * W + w) * 4 + (c % 4);
+}
+
+/* filter offset: BareMetal/ConvKernel.cpp:48-76 (strides) and :78-113 (address) */
+static inline size_t flt_off(
+        int fmt, int group_conv, int g, int oc, int ic, int fh, int fw, int ocpg, int icpg,
+        int FH, int FW) {
+    if (fmt == FMT_NCHW) {
+        /* [G,] OCpg, ICpg, FH, FW */
+        return ((((size_t)g * ocpg + oc) * icpg + ic) * FH + fh) * FW + fw;
+    } else if (fmt == FMT_NCHW_NCHW44) {
+        /* OC/4, FH, FW, IC, 4oc */
+        return ((((size_t)(oc / 4) * FH + fh) * FW + fw) * icpg + ic) * 4 + (oc % 4);
+    } else if (!group_conv) {
+        /* OC/4, IC/4, FH, FW, 4ic, 4oc */
+        return (((((size_t)(oc / 4) * (icpg / 4) + ic / 4) * FH + fh) * FW + fw) * 4 + (ic % 4)) *
+                       4 +
+               (oc % 4);
+    } else {
+        /* channel-wise: G/4, 1, 1, FH, FW, 4 */
+        return (((size_t)(g / 4) * FH + fh) * FW + fw) * 4 + (g % 4);
+    }
+}
+
+/* BareMetal::ConvGeneral, qsi8 x qsi8 (+qsi32 bias) -> qsi8:
+ * BareMetal/ConvKernel.cpp:305-344 (loops, `uint32 idx < ih` zero padding), :374-380 (bias added
+ * to the int accumulator), BareMetal/Activation.cpp:105-114 (dval*scale*flt_scale/dst_scale,
+ * activation applied to the fully scaled value, then fp32_to_int8).
+ * groups == 1: DENSE; groups > 1: GROUP with ocpg = OC/groups, icpg = IC/groups. */
+void orc_conv_q8(
+        const int8_t* src, const int8_t* flt, const int32_t* bias, int8_t* dst, int fmt,
+        int groups, int N, int IC, int IH, int IW, int OC, int OH, int OW, int FH, int FW, int SH,
+        int SW, int PH, int PW, int DH, int DW, int act, float scale, float flt_scale,
+        float dst_scale) {
+    const int ocpg = OC / groups, icpg = IC / groups;
+    const int src44 = (fmt == FMT_NCHW44);
+    const int dst44 = (fmt != FMT_NCHW);
+    const int is_group = groups > 1;
+    const long total = (long)N * OC;
+#pragma omp parallel for schedule(dynamic) num_threads(g_threads) if (g_threads > 1)
+    for (long job = 0; job < total; ++job) {
+        const int n = (int)(job / OC), oc = (int)(job % OC);
+        const int g = oc / ocpg, ocl = oc % ocpg;
+        for (int oh = 0; oh < OH; ++oh)
+            for (int ow = 0; ow < OW; ++ow) {
+                int dval = 0;
+                for (int fh = 0; fh < FH; ++fh)
+                    for (int fw = 0; fw < FW; ++fw) {
+                        uint32_t ih = (uint32_t)(oh * SH + fh * DH - PH);
+                        uint32_t iw = (uint32_t)(ow * SW + fw * DW - PW);
+                        if (ih < (uint32_t)IH && iw < (uint32_t)IW) {
+                            for (int icl = 0; icl < icpg; ++icl) {
+                                int ic = g * icpg + icl;
+                                int sval = src44 ? src[off_nchw44(IC, IH, IW, n, ic, ih, iw)]
+                                                 : src[off_nchw(IC, IH, IW, n, ic, ih, iw)];
+                                int fval = flt[flt_off(
+                                        fmt, is_group, g, ocl, icl, fh, fw, ocpg, icpg, FH, FW)];
+                                dval += sval * fval;
+                            }
+                        }
+                    }
+                if (bias)
+                    dval += bias[oc];
+                size_t o = dst44 ? off_nchw44(OC, OH, OW, n, oc, oh, ow)
+                                 : off_nchw(OC, OH, OW, n, oc, oh, ow);
+                dst[o] = fp32_to_int8(act_apply(act, dval * scale * flt_scale / dst_scale));
+            }
+    }
+}
+
+/* Same template with acc_specifier = "float" (BareMetal/ConvKernel.cpp:199-207): accumulation
+ * order fh -> fw -> ic, bias added last, activation on the sum. The kernel MegCC actually selects
+ * for f32 NCHW DENSE on x86 is GI im2col + 4x12 GEMM (GeneralIntrinsic/ConvKernel/Fp32Im2col.cpp:
+ * 88-218), which sums in a different order; the two agree to ~1e-6 relative and the product is
+ * held to 1e-4 against either. */
+void orc_conv_f32(
+        const float* src, const float* flt, const float* bias, float* dst, int fmt, int groups,
+        int N, int IC, int IH, int IW, int OC, int OH, int OW, int FH, int FW, int SH, int SW,
+        int PH, int PW, int DH, int DW, int act) {
+    const int ocpg = OC / groups, icpg = IC / groups;
+    const int src44 = (fmt == FMT_NCHW44);
+    const int dst44 = (fmt != FMT_NCHW);
+    const int is_group = groups > 1;
+    const long total = (long)N * OC;
+#pragma omp parallel for schedule(dynamic) num_threads(g_threads) if (g_threads > 1)
+    for (long job = 0; job < total; ++job) {
+        const int n = (int)(job / OC), oc = (int)(job % OC);
+        const int g = oc / ocpg, ocl = oc % ocpg;
+        for (int oh = 0; oh < OH; ++oh)
+            for (int ow = 0; ow < OW; ++ow) {
+                float dval = 0;
+                for (int fh = 0; fh < FH; ++fh)
+                    for (int fw = 0; fw < FW; ++fw) {
+                        uint32_t ih = (uint32_t)(oh * SH + fh * DH - PH);
+                        uint32_t iw = (uint32_t)(ow * SW + fw * DW - PW);
+                        if (ih < (uint32_t)IH && iw < (uint32_t)IW) {
+                            for (int icl = 0; icl < icpg; ++icl) {
+                                int ic = g * icpg + icl;
+                                float sval = src44 ? src[off_nchw44(IC, IH, IW, n, ic, ih, iw)]
+                                                   : src[off_nchw(IC, IH, IW, n, ic, ih, iw)];
+                                float fval = flt[flt_off(
+                                        fmt, is_group, g, ocl, icl, fh, fw, ocpg, icpg, FH, FW)];
+                                dval += sval * fval;
+                            }
+                        }
+                    }
+                if (bias)
+                    dval += bias[oc];
+                size_t o = dst44 ? off_nchw44(OC, OH, OW, n, oc, oh, ow)
+                                 : off_nchw(OC, OH, OW, n, oc, oh, ow);
+                dst[o] = act_apply(act, dval);
+            }
+    }
+}
+
+/* f32 MatrixMul, row-major, no bias. BareMetal/MatrixMul.cpp:25-120 (naive m,n,k loops) --
+ * GI 4x12 (GeneralIntrinsic/MatMulKernel/Fp32MatMulM4N12.cpp) and gevm
+ * (GeneralIntrinsic/MatMulKernel/Fp32Gevm.cpp:50-91) differ only in summation order. */
+void orc_matmul_f32(
+        const float* A, const float* B, float* C, int M, int N, int K, int lda, int ldb, int ldc,
+        int trans_a, int trans_b) {
+#pragma omp parallel for schedule(static) num_threads(g_threads) if (g_threads > 1)
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            float acc = 0.f;
+            for (int k = 0; k < K; ++k) {
+                float a = trans_a ? A[(size_t)k * lda + m] : A[(size_t)m * lda + k];
+                float b = trans_b ? B[(size_t)n * ldb + k] : B[(size_t)k * ldb + n];
+                acc += a * b;
+            }
+            C[(size_t)m * ldc + n] = acc;
+        }
+}
+
+enum { POOL_MAX = 0, POOL_AVG = 1, POOL_AVG_EXCL = 2 };
+
+/* qsi8 pooling.
+ * NCHW  : BareMetal/Pooling.cpp:84-148,219-245 -- MAX over in-bounds taps starting from -128;
+ *         AVERAGE `sum = roundf((float)sum / (wh*ww))`, COUNT_EXCLUDE_PADDING `/ count`; the int
+ *         is stored to int8 without a clamp.
+ * NCHW44: GeneralIntrinsic/PoolingKernel/QInt8PoolingNCHW44.cpp:34-113 -- AVERAGE is
+ *         `float count_div = 1.0 / window_count;` then saturate(round((float)sum * count_div))
+ *         (the non-SSE4.2 branch of GiCvtFromFloat32ToInt8, immigration/include/gi_int.h:
+ *         1145-1160: round(), clamp to [-128,127]). */
+void orc_pool_q8(
+        const int8_t* src, int8_t* dst, int fmt, int mode, int N, int C, int IH, int IW, int OH,
+        int OW, int WH, int WW, int SH, int SW, int PH, int PW) {
+    const long total = (long)N * C;
+#pragma omp parallel for schedule(static) num_threads(g_threads) if (g_threads > 1)
+    for (long job = 0; job < total; ++job) {
+        const int n = (int)(job / C), c = (int)(job % C);
+        for (int oh = 0; oh < OH; ++oh)
+            for (int ow = 0; ow < OW; ++ow) {
+                int8_t res = -128;
+                int sum = 0, count = 0;
+                for (int fh = 0; fh < WH; ++fh)
+                    for (int fw = 0; fw < WW; ++fw) {
+                        uint32_t ih = (uint32_t)(-PH + oh * SH + fh);
+                        uint32_t iw = (uint32_t)(-PW + ow * SW + fw);
+                        if (ih < (uint32_t)IH && iw < (uint32_t)IW) {
+                            int8_t v = fmt == FMT_NCHW44
+                                             ? src[off_nchw44(C, IH, IW, n, c, ih, iw)]
+                                             : src[off_nchw(C, IH, IW, n, c, ih, iw)];
+                            res = res > v ? res : v;
+                            sum += v;
+                            ++count;
+                        }
+                    }
+                int8_t out;
+                if (mode == POOL_MAX) {
+                    out = res;
+                } else if (fmt == FMT_NCHW44) {
+                    uint32_t window_count = mode == POOL_AVG ? (uint32_t)(WH * WW) : (uint32_t)count;
+                    float count_div = 1.0 / window_count;
+                    double r = round((float)sum * count_div);
+                    r = r > 127 ? 127 : r;
+                    r = r < -128 ? -128 : r;
+                    out = (int8_t)r;
+                } else {
+                    int s = mode == POOL_AVG ? (int)roundf((float)sum / (WH * WW))
+                                             : (int)roundf((float)sum / count);
+                    out = (int8_t)s;
+                }
+                size_t o = fmt == FMT_NCHW44 ? off_nchw44(C, OH, OW, n, c, oh, ow)
+                                             : off_nchw(C, OH, OW, n, c, oh, ow);
+                dst[o] = out;
+            }
+    }
+}
+
+enum { Q_ADD = 0, Q_FUSE_ADD_RELU = 1, Q_MUL = 2, Q_RELU = 3 };
+
+/* BareMetal/ElemwiseMultiType.cpp:16-55 (expressions) and :102-213 (three broadcast cases).
+ * bcast: 0 same shape, 1 b is one element, 2 b is [1,C,1,1..] against a = [outer,C,inner]. */
+void orc_multitype_q8(
+        const int8_t* a, const int8_t* b, int8_t* dst, int mode, size_t n, int bcast, int C,
+        size_t inner, float scale_0, float scale_1, float scale_dst) {
+    float scale_div = 1.f / scale_dst;
+    float scale_mul = scale_0 * scale_1 * scale_div;
+    for (size_t i = 0; i < n; ++i) {
+        int8_t val_0 = a[i];
+        int8_t val_1 = 0;
+        if (mode != Q_RELU)
+            val_1 = bcast == 0 ? b[i] : bcast == 1 ? b[0] : b[(i / inner) % C];
+        int8_t out;
+        if (mode == Q_ADD) {
+            out = fp32_to_int8((scale_0 * val_0 + scale_1 * val_1) * scale_div);
+        } else if (mode == Q_FUSE_ADD_RELU) {
+            float val0 = scale_0 * val_0;
+            float val1 = scale_1 * val_1;
+            out = fp32_to_int8(((val0 + val1) > 0 ? (val0 + val1) : 0) * scale_div);
+        } else if (mode == Q_MUL) {
+            out = fp32_to_int8(val_0 * val_1 * scale_mul);
+        } else {
+            out = fp32_to_int8(((scale_0 * val_0) > 0 ? (scale_0 * val_0) : 0) * scale_div);
+        }
+        dst[i] = out;
+    }
+}
+
+/* GeneralIntrinsic/Typecvt.cpp:227-295: `scale = src_scale/dst_scale` with 1 substituted on a float
+ * side, then x*scale; the 16-wide body and the scalar tail round identically on a host without
+ * SSE4.2 (gi_int.h:1145-1160 round() vs roundf(), both half away from zero; both clamp). */
+static inline int8_t sat_q8(float v) {
+    int d = roundf(v);
+    d = d >= 127 ? 127 : d;
+    d = d <= -128 ? -128 : d;
+    return (int8_t)d;
+}
+void orc_typecvt_f32_q8(const float* src, int8_t* dst, size_t n, float dst_scale) {
+    float scale = 1.f / dst_scale;
+    for (size_t i = 0; i < n; ++i)
+        dst[i] = sat_q8(src[i] * scale);
+}
+void orc_typecvt_q8_f32(const int8_t* src, float* dst, size_t n, float src_scale) {
+    float scale = src_scale / 1.f;
+    for (size_t i = 0; i < n; ++i)
+        dst[i] = src[i] * scale;
+}
+void orc_typecvt_q8_q8(const int8_t* src, int8_t* dst, size_t n, float src_scale, float dst_scale) {
+    float scale = src_scale / dst_scale;
+    for (size_t i = 0; i < n; ++i)
+        dst[i] = sat_q8(src[i] * scale);
+}
+/* BareMetal/Typecvt.cpp:43-105: qsi32 -> qsi8 is `staturate(val * src_scale / dst_scale)` */
+void orc_typecvt_q32_q8(
+        const int32_t* src, int8_t* dst, size_t n, float src_scale, float dst_scale) {
+    for (size_t i = 0; i < n; ++i)
+        dst[i] = sat_q8(src[i] * src_scale / dst_scale);
+}
+
+enum {
+    EW_RELU = 0,
+    EW_EXP = 1,
+    EW_SIGMOID = 2,
+    EW_H_SWISH = 3,
+    EW_NEGATE = 4,
+    EW_ADD = 16,
+    EW_SUB = 17,
+    EW_MUL = 18,
+    EW_TRUE_DIV = 19,
+    EW_MAX = 20,
+    EW_MIN = 21,
+    EW_FUSE_ADD_RELU = 22
+};
+
+/* f32 elementwise, BareMetal/ElemwiseKernel.cpp:35-110 expressions.
+ * bcast: 0 same shape, 1 scalar b, 2 b indexed by (i / inner) % C, i.e. [1,C,1,1] or a trailing
+ * vector when inner == 1. */
+void orc_elemwise_f32(
+        const float* a, const float* b, float* dst, int mode, size_t n, int bcast, int C,
+        size_t inner) {
+    for (size_t i = 0; i < n; ++i) {
+        float x = a[i], y = 0.f, r;
+        if (mode >= EW_ADD)
+            y = bcast == 0 ? b[i] : bcast == 1 ? b[0] : b[(i / inner) % C];
+        switch (mode) {
+            case EW_RELU:
+                r = x > 0 ? x : 0;
+                break;
+            case EW_EXP:
+                r = expf(x);
+                break;
+            case EW_SIGMOID:
+                r = 1.f / (1.f + expf(-x));
+                break;
+            case EW_H_SWISH: {
+                float t = x + 3.f;
+                t = t > 6.f ? 6.f : t;
+                t = t < 0.f ? 0.f : t;
+                r = x * t / 6.f;
+                break;
+            }
+            case EW_NEGATE:
+                r = -x;
+                break;
+            case EW_ADD:
+                r = x + y;
+                break;
+            case EW_SUB:
+                r = x - y;
+                break;
+            case EW_MUL:
+                r = x * y;
+                break;
+            case EW_TRUE_DIV:
+                r = x / y;
+                break;
+            case EW_MAX:
+                r = x > y ? x : y;
+                break;
+            case EW_MIN:
+                r = x < y ? x : y;
+                break;
+            default: /* FUSE_ADD_RELU */
+                r = (x + y) > 0 ? (x + y) : 0;
+                break;
+        }
+        dst[i] = r;
+    }
+}
+
+enum { RED_SUM = 0, RED_MEAN = 1, RED_MAX = 2, RED_MIN = 3 };
+
+/* BareMetal/Reduce.cpp:98-131: view as [A,B,C], reduce over B in ascending j. */
+void orc_reduce_f32(const float* src, float* dst, int mode, int A, int B, int C) {
+    for (int i = 0; i < A; ++i)
+        for (int k = 0; k < C; ++k) {
+            float acc = mode == RED_MAX ? -__FLT_MAX__ : mode == RED_MIN ? __FLT_MAX__ : 0.f;
+            for (int j = 0; j < B; ++j) {
+                float v = src[((size_t)i * B + j) * C + k];
+                if (mode == RED_MAX)
+                    acc = acc > v ? acc : v;
+                else if (mode == RED_MIN)
+                    acc = acc < v ? acc : v;
+                else
+                    acc = acc + v;
+            }
+            dst[(size_t)i * C + k] = mode == RED_MEAN ? acc / B : acc;
+        }
+}

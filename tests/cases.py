@@ -1,0 +1,373 @@
+"""Operator test cases shared by the CPU (oracle) and GPU (parity) tests.
+
+A case knows (1) the reference kernel symbol MegCC would generate for it, (2) how to draw seeded
+inputs in the reference's layouts, (3) how to evaluate it on the CPU port (oracle/port.py) and on
+the reference's generated C (oracle/ref.py), and (4) the Tensor list the uniform kernel ABI takes.
+The GPU side (tests/gpu_util.py) consumes the same description.
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from megcc_amd import abi  # noqa: E402
+from oracle import port, ref  # noqa: E402
+
+FMT_NAME = {abi.FMT_NCHW: "NCHW", abi.FMT_NCHW44: "NCHW44", abi.FMT_NCHW_NCHW44: "NCHW_NCHW44"}
+
+
+def rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+def _op(shape, dtype, scale=None):
+    """operand text of oracle/ref_kernels.spec: dims|dtype|scale"""
+    return "o:%s|%s|%s" % ("x".join(str(int(d)) for d in shape), dtype,
+                           "" if scale is None else repr(float(scale)))
+
+
+class TensorSpec:
+    """name, numpy array (inputs) or shape (outputs), TinyNN dtype enum, scale"""
+
+    def __init__(self, name, shape, type_enum, scale=1.0, array=None):
+        self.name, self.shape, self.type_enum, self.scale, self.array = (
+            name, tuple(shape), type_enum, scale, array)
+
+    @property
+    def nbytes(self):
+        return int(np.prod(self.shape, dtype=np.int64)) * abi.np_dtype(self.type_enum).itemsize
+
+
+class ConvCase:
+    def __init__(self, fmt, sparse, n, ic, ih, iw, oc, k, stride=1, pad=0, act=abi.IDENTITY,
+                 dtype="qsi8", scales=(0.02, 0.01, 0.05), bias=True, dilate=1,
+                 src_range=(-128, 127), flt_range=(-127, 127), bias_range=(-1000, 1000)):
+        self.fmt, self.sparse = fmt, sparse
+        self.n, self.ic, self.ih, self.iw, self.oc = n, ic, ih, iw, oc
+        self.fh = self.fw = k
+        self.sh = self.sw = stride
+        self.ph = self.pw = pad
+        self.dh = self.dw = dilate
+        self.act, self.dtype, self.scales, self.bias = act, dtype, scales, bias
+        self.src_range, self.flt_range, self.bias_range = src_range, flt_range, bias_range
+        self.groups = ic if sparse == abi.GROUP else 1
+        if sparse == abi.GROUP:
+            assert ic == oc, "only channel-wise GROUP cases are described here"
+        self.oh, self.ow = port.conv_out_hw(ih, iw, k, k, stride, stride, pad, pad, dilate, dilate)
+
+    def __repr__(self):
+        return "%s[n%d c%d->%d %dx%d %s]" % (self.symbol(), self.n, self.ic, self.oc, self.ih,
+                                             self.iw, "x".join("%g" % s for s in self.scales))
+
+    # -- shapes in the reference's layouts (BareMetal/ConvKernel.cpp:48-113) -------------------
+    def src_shape(self):
+        if self.fmt == abi.FMT_NCHW44:
+            return (self.n, self.ic // 4, self.ih, self.iw, 4)
+        return (self.n, self.ic, self.ih, self.iw)
+
+    def dst_shape(self):
+        if self.fmt == abi.FMT_NCHW:
+            return (self.n, self.oc, self.oh, self.ow)
+        return (self.n, self.oc // 4, self.oh, self.ow, 4)
+
+    def flt_shape(self):
+        k = self.fh
+        if self.fmt == abi.FMT_NCHW:
+            if self.sparse == abi.GROUP:
+                return (self.groups, 1, 1, k, k)
+            return (self.oc, self.ic, k, k)
+        if self.fmt == abi.FMT_NCHW_NCHW44:
+            return (self.oc // 4, k, k, self.ic, 4)
+        if self.sparse == abi.GROUP:
+            return (self.groups // 4, 1, 1, k, k, 4)
+        return (self.oc // 4, self.ic // 4, k, k, 4, 4)
+
+    def bias_shape(self):
+        if self.fmt == abi.FMT_NCHW:
+            return (1, self.oc, 1, 1)
+        return (1, self.oc // 4, 1, 1, 4)
+
+    def symbol(self):
+        """ConvImpl::GetKernelSymbol, BareMetal/ConvKernel.cpp:144-176 (GI_ prefix and suffix
+        order of GeneralIntrinsic/ConvKernel/Fp32Im2col.cpp for the f32 NCHW dense case)."""
+        q = self.dtype == "qsi8"
+        io = "qsi8qsi8qsi32qsi8" if q else "f32f32f32f32"
+        if not self.bias:
+            io = "qsi8qsi8qsi8" if q else "f32f32f32"
+        s = "kernel_conv2d_%dx%d_%s_%s_p%dx%d_s%dx%d_d%dx%d_%s" % (
+            self.fh, self.fw, FMT_NAME[self.fmt], "GROUP" if self.sparse == abi.GROUP else "DENSE",
+            self.ph, self.pw, self.sh, self.sw, self.dh, self.dw, io)
+        if self.bias:
+            s += "_bias"
+        if self.act != abi.IDENTITY:
+            s += "_" + abi.NONLINE_NAMES[self.act]
+        return s
+
+    def spec_line(self):
+        """the attribute bag the reference compiler hands to KernelGen for this operator
+        (compiler/test/kernel/common/src/cc_fill_attr.cpp:253-274), in ref_dump's text form"""
+        q = self.dtype == "qsi8"
+        sd, bd = ("qsi8", "qsi32") if q else ("f32", "f32")
+        ss, fs, ds = self.scales if q else (None, None, None)
+        src_shape = self.src_shape()
+        a = ["ConvKernel", "format=s:" + ("NCHW" if self.fmt == abi.FMT_NCHW else "NCHW44"),
+             "sparse=s:" + ("GROUP" if self.sparse == abi.GROUP else "DENSE"),
+             "mode=s:CROSS_CORRELATION", "nonlineMode=s:" + abi.NONLINE_NAMES[self.act],
+             "kernel_h=u:%d" % self.fh, "kernel_w=u:%d" % self.fw, "stride_h=u:%d" % self.sh,
+             "stride_w=u:%d" % self.sw, "pad_h=u:%d" % self.ph, "pad_w=u:%d" % self.pw,
+             "dilate_h=u:%d" % self.dh, "dilate_w=u:%d" % self.dw,
+             "nr_operands=i:%d" % (4 if self.bias else 3),
+             "operand:0=" + _op(src_shape, sd, ss), "operand:1=" + _op(self.flt_shape(), sd, fs)]
+        if self.bias:
+            a.append("operand:2=" + _op(self.bias_shape(), bd, ss * fs if q else None))
+        a.append("operand:%d=%s" % (3 if self.bias else 2, _op(self.dst_shape(), sd, ds)))
+        return " ".join(a)
+
+    def attr(self):
+        return abi.ConvAttr(self.fh, self.fw, self.sh, self.sw, self.ph, self.pw, self.dh, self.dw,
+                            self.fmt, self.sparse, self.act, int(self.bias))
+
+    def gen(self, seed=0):
+        r = rng(seed)
+        if self.dtype == "qsi8":
+            src = r.integers(self.src_range[0], self.src_range[1] + 1, self.src_shape()).astype(np.int8)
+            flt = r.integers(self.flt_range[0], self.flt_range[1] + 1, self.flt_shape()).astype(np.int8)
+            b = r.integers(self.bias_range[0], self.bias_range[1] + 1, self.bias_shape()).astype(np.int32)
+        else:
+            src = r.uniform(-1, 1, self.src_shape()).astype(np.float32)
+            flt = r.uniform(-1, 1, self.flt_shape()).astype(np.float32)
+            b = r.uniform(-0.1, 0.1, self.bias_shape()).astype(np.float32)
+        return {"src": src, "flt": flt, "bias": b if self.bias else None}
+
+    def specs(self, arrays):
+        q = self.dtype == "qsi8"
+        ss, fs, ds = self.scales if q else (1.0, 1.0, 1.0)
+        ins = [TensorSpec(b"src", self.src_shape(), abi.QINT8 if q else abi.FLOAT, ss, arrays["src"]),
+               TensorSpec(b"flt", self.flt_shape(), abi.QINT8 if q else abi.FLOAT, fs, arrays["flt"])]
+        if self.bias:
+            ins.append(TensorSpec(b"bias", self.bias_shape(), abi.QINT32 if q else abi.FLOAT,
+                                  ss * fs, arrays["bias"]))
+        outs = [TensorSpec(b"dst", self.dst_shape(), abi.QINT8 if q else abi.FLOAT, ds)]
+        return ins, outs
+
+    def run_port(self, arrays):
+        return port.conv(arrays["src"], arrays["flt"], arrays["bias"], self.fmt, self.groups,
+                         self.oc, self.fh, self.fw, (self.sh, self.sw), (self.ph, self.pw),
+                         (self.dh, self.dw), self.act,
+                         self.scales if self.dtype == "qsi8" else None)
+
+    def ops(self):
+        return 2 * self.n * self.oc * self.oh * self.ow * (self.ic // self.groups) * self.fh * self.fw
+
+    def min_bytes(self):
+        e = 1 if self.dtype == "qsi8" else 4
+        return (int(np.prod(self.src_shape())) * e + int(np.prod(self.flt_shape())) * e +
+                self.oc * 4 + int(np.prod(self.dst_shape())) * e)
+
+
+class PoolCase:
+    def __init__(self, fmt, mode, n, c, ih, iw, window, stride, pad, scale=0.05):
+        self.fmt, self.mode, self.n, self.c, self.ih, self.iw = fmt, mode, n, c, ih, iw
+        self.window, self.stride, self.pad, self.scale = window, stride, pad, scale
+        self.oh = (ih + 2 * pad - window) // stride + 1
+        self.ow = (iw + 2 * pad - window) // stride + 1
+
+    def __repr__(self):
+        return "%s[n%d c%d %dx%d]" % (self.symbol(), self.n, self.c, self.ih, self.iw)
+
+    def src_shape(self):
+        return ((self.n, self.c // 4, self.ih, self.iw, 4) if self.fmt == abi.FMT_NCHW44
+                else (self.n, self.c, self.ih, self.iw))
+
+    def dst_shape(self):
+        return ((self.n, self.c // 4, self.oh, self.ow, 4) if self.fmt == abi.FMT_NCHW44
+                else (self.n, self.c, self.oh, self.ow))
+
+    def symbol(self):
+        """PoolingImpl::GetKernelSymbol (BareMetal/Pooling.cpp:31-44); the NCHW44 kernel comes
+        from GI with its extra io-string and _fallback suffix
+        (GeneralIntrinsic/PoolingKernel/QInt8PoolingNCHW44.cpp:25-31)."""
+        s = "kernel_pooling_%s_%s_p%dx%d_s%dx%d_w%dx%d_qsi8qsi8" % (
+            abi.POOL_NAMES[self.mode], FMT_NAME[self.fmt], self.pad, self.pad, self.stride,
+            self.stride, self.window, self.window)
+        if self.fmt == abi.FMT_NCHW44:
+            s = "GI_" + s + "_qsi8qsi8_fallback"
+        return s
+
+    def spec_line(self):
+        return " ".join([
+            "PoolingKernel", "format=s:" + FMT_NAME[self.fmt], "mode=s:" + abi.POOL_NAMES[self.mode],
+            "window_h=u:%d" % self.window, "window_w=u:%d" % self.window,
+            "stride_h=u:%d" % self.stride, "stride_w=u:%d" % self.stride,
+            "pad_h=u:%d" % self.pad, "pad_w=u:%d" % self.pad, "nr_operands=i:2",
+            "operand:0=" + _op(self.src_shape(), "qsi8", self.scale),
+            "operand:1=" + _op(self.dst_shape(), "qsi8", self.scale)])
+
+    def attr(self):
+        return abi.PoolAttr(self.window, self.window, self.stride, self.stride, self.pad, self.pad,
+                            self.fmt, self.mode)
+
+    def gen(self, seed=0):
+        return {"src": rng(seed).integers(-128, 128, self.src_shape()).astype(np.int8)}
+
+    def specs(self, arrays):
+        return ([TensorSpec(b"src", self.src_shape(), abi.QINT8, self.scale, arrays["src"])],
+                [TensorSpec(b"dst", self.dst_shape(), abi.QINT8, self.scale)])
+
+    def run_port(self, arrays):
+        return port.pool_q8(arrays["src"], self.fmt, self.mode, (self.window,) * 2,
+                            (self.stride,) * 2, (self.pad,) * 2)
+
+
+class MultiTypeCase:
+    def __init__(self, mode, shape, scales=(0.05, 0.01, 0.05), bshape=None):
+        self.mode, self.shape, self.scales = mode, tuple(shape), scales
+        self.bshape = tuple(bshape) if bshape is not None else self.shape
+
+    def __repr__(self):
+        return "%s%s%s" % (self.symbol(), list(self.shape), list(self.bshape))
+
+    def symbol(self):
+        """BareMetal/ElemwiseMultiType.cpp:94-100"""
+        io = "qsi8qsi8" if self.mode == abi.Q_RELU else "qsi8qsi8qsi8"
+        return "kernel_elementwise_multitype_%s_%s" % (abi.MULTITYPE_NAMES[self.mode], io)
+
+    def spec_line(self):
+        ops = [_op(self.shape, "qsi8", self.scales[0])]
+        if self.mode != abi.Q_RELU:
+            ops.append(_op(self.bshape, "qsi8", self.scales[1]))
+        ops.append(_op(self.shape, "qsi8", self.scales[2]))
+        return " ".join(["ElemwiseMultiKernel", "mode=s:" + abi.MULTITYPE_NAMES[self.mode],
+                         "nr_operands=i:%d" % len(ops)] +
+                        ["operand:%d=%s" % (i, o) for i, o in enumerate(ops)])
+
+    def gen(self, seed=0):
+        r = rng(seed)
+        a = r.integers(-128, 128, self.shape).astype(np.int8)
+        b = None if self.mode == abi.Q_RELU else r.integers(-128, 128, self.bshape).astype(np.int8)
+        return {"a": a, "b": b}
+
+    def specs(self, arrays):
+        ins = [TensorSpec(b"a", self.shape, abi.QINT8, self.scales[0], arrays["a"])]
+        if self.mode != abi.Q_RELU:
+            ins.append(TensorSpec(b"b", self.bshape, abi.QINT8, self.scales[1], arrays["b"]))
+        return ins, [TensorSpec(b"dst", self.shape, abi.QINT8, self.scales[2])]
+
+    def run_port(self, arrays):
+        return port.multitype_q8(arrays["a"], arrays["b"], self.mode, *self.scales)
+
+
+_KIND_ENUM = {"f32": abi.FLOAT, "qsi8": abi.QINT8, "qsi32": abi.QINT32}
+
+
+class TypeCvtCase:
+    def __init__(self, src_kind, dst_kind, shape, src_scale=1.0, dst_scale=1.0, span=None):
+        self.src_kind, self.dst_kind, self.shape = src_kind, dst_kind, tuple(shape)
+        self.src_scale, self.dst_scale, self.span = src_scale, dst_scale, span
+
+    def __repr__(self):
+        return "%s%s" % (self.symbol(), list(self.shape))
+
+    def symbol(self):
+        """GI for q8<->f32 and q8->q8 (GeneralIntrinsic/Typecvt.cpp:36-41), BareMetal otherwise
+        (BareMetal/Typecvt.cpp:36-41)."""
+        gi = (self.src_kind, self.dst_kind) != ("qsi32", "qsi8")
+        return ("GI_" if gi else "") + "kernel_typecvt_%s%s" % (self.src_kind, self.dst_kind)
+
+    def spec_line(self):
+        return " ".join([
+            "TypeCvtKernel", "nr_operands=i:2",
+            "operand:0=" + _op(self.shape, self.src_kind,
+                               None if self.src_kind == "f32" else self.src_scale),
+            "operand:1=" + _op(self.shape, self.dst_kind,
+                               None if self.dst_kind == "f32" else self.dst_scale)])
+
+    def gen(self, seed=0):
+        r = rng(seed)
+        if self.src_kind == "f32":
+            span = self.span or 140 * self.dst_scale
+            src = r.uniform(-span, span, self.shape).astype(np.float32)
+            # exact .5 ties, which round half away from zero
+            flat = src.reshape(-1)
+            k = min(flat.size, 64)
+            flat[:k] = (np.arange(k, dtype=np.float32) - k // 2 + 0.5) * np.float32(self.dst_scale)
+        elif self.src_kind == "qsi8":
+            src = r.integers(-128, 128, self.shape).astype(np.int8)
+        else:
+            span = int(self.span or 140 * self.dst_scale / self.src_scale)
+            src = r.integers(-span, span + 1, self.shape).astype(np.int32)
+        return {"src": src}
+
+    def specs(self, arrays):
+        return ([TensorSpec(b"src", self.shape, _KIND_ENUM[self.src_kind], self.src_scale,
+                            arrays["src"])],
+                [TensorSpec(b"dst", self.shape, _KIND_ENUM[self.dst_kind], self.dst_scale)])
+
+    def run_port(self, arrays):
+        return port.typecvt(arrays["src"], self.src_kind, self.dst_kind, self.src_scale,
+                            self.dst_scale)
+
+
+class MatMulCase:
+    def __init__(self, m, k, n, trans_a=False, trans_b=False):
+        self.m, self.k, self.n, self.trans_a, self.trans_b = m, k, n, trans_a, trans_b
+
+    def __repr__(self):
+        return "%s[%dx%dx%d]" % (self.symbol(), self.m, self.k, self.n)
+
+    def symbol(self):
+        """GeneralIntrinsic/MatMulKernel/Fp32Gevm.cpp:109-135 (M<=4, A not transposed) else
+        Fp32MatMulM4N12.cpp:9-45"""
+        t = ("t" if self.trans_a else "n") + ("t" if self.trans_b else "n")
+        if self.m <= 4 and not self.trans_a:
+            return "GI_kernel_gevm_" + t
+        return "GI_kernel_fp32_matmul_4x12_" + t
+
+    def spec_line(self):
+        ashape = (self.k, self.m) if self.trans_a else (self.m, self.k)
+        bshape = (self.n, self.k) if self.trans_b else (self.k, self.n)
+        return " ".join([
+            "MatrixMulKernel", "transposeA=b:%d" % self.trans_a, "transposeB=b:%d" % self.trans_b,
+            "format=s:DEFAULT", "compute_mode=s:DEFAULT", "nr_operands=i:3",
+            "operand:0=" + _op(ashape, "f32"), "operand:1=" + _op(bshape, "f32"),
+            "operand:2=" + _op((self.m, self.n), "f32")])
+
+    def attr(self):
+        return abi.MatMulAttr(int(self.trans_a), int(self.trans_b))
+
+    def gen(self, seed=0):
+        r = rng(seed)
+        ashape = (self.k, self.m) if self.trans_a else (self.m, self.k)
+        bshape = (self.n, self.k) if self.trans_b else (self.k, self.n)
+        return {"a": r.uniform(-1, 1, ashape).astype(np.float32),
+                "b": r.uniform(-1, 1, bshape).astype(np.float32)}
+
+    def specs(self, arrays):
+        return ([TensorSpec(b"a", arrays["a"].shape, abi.FLOAT, 1.0, arrays["a"]),
+                 TensorSpec(b"b", arrays["b"].shape, abi.FLOAT, 1.0, arrays["b"])],
+                [TensorSpec(b"c", (self.m, self.n), abi.FLOAT)])
+
+    def run_port(self, arrays):
+        return port.matmul_f32(arrays["a"], arrays["b"], self.trans_a, self.trans_b)
+
+
+def run_ref(case, arrays):
+    """Evaluate `case` with the reference's generated C kernel; returns the output array."""
+    ins, outs = case.specs(arrays)
+    out_arr = np.zeros(outs[0].shape, abi.np_dtype(outs[0].type_enum))
+    tin = [abi.host_tensor(s.array, s.type_enum, s.scale, s.name) for s in ins]
+    tout = [abi.host_tensor(out_arr, outs[0].type_enum, outs[0].scale, outs[0].name)]
+    ref.run(case.symbol(), tin, tout)
+    return out_arr
+
+
+def max_rel_err(got, want):
+    """|a-b| / max(1, min(|a|,|b|)): the reference's model-level metric (ci/compare_output_bin.py)."""
+    got = got.astype(np.float64)
+    want = want.astype(np.float64)
+    d = np.abs(got - want) / np.maximum(1.0, np.minimum(np.abs(got), np.abs(want)))
+    return float(d.max()) if d.size else 0.0

@@ -1,0 +1,90 @@
+"""The small cases whose reference outputs are committed under tests/golden/ (see
+tests/golden/make_golden.py). Shapes follow the reference's own kernel tests
+(compiler/test/kernel/opr/naive/conv.cpp:53-264, pool.cpp:6-66, elemwise_multitype.cpp:6-64,
+typecvt.cpp:5-70): odd sizes, k in {1,3}, stride in {1,2}, pad in {0,k/2}, every activation, the
+small-magnitude tie case and the 30..50 overflow case."""
+from megcc_amd import abi
+from cases import ConvCase, MatMulCase, MultiTypeCase, PoolCase, TypeCvtCase
+
+A = abi
+
+
+def unsat(k_taps):
+    """dst scale that keeps outputs inside [-128,127] for full-range int8 data: the accumulator's
+    std is about 74*73*sqrt(K); put 3 sigma near 100."""
+    return 0.02 * 0.01 * 5.4e3 * (k_taps ** 0.5) / 35.0
+
+
+def golden_cases():
+    c = {}
+    # --- qsi8 dense NCHW44 3x3 (headline kernel), every activation, saturating and not
+    for act in (A.IDENTITY, A.RELU, A.H_SWISH, A.SIGMOID):
+        c["conv44_3x3_s1_%s" % A.NONLINE_NAMES[act]] = ConvCase(
+            A.FMT_NCHW44, A.DENSE, 2, 8, 7, 9, 12, 3, 1, 1, act, scales=(0.02, 0.01, unsat(72)))
+    c["conv44_3x3_s1_RELU_baseline_scales"] = ConvCase(
+        A.FMT_NCHW44, A.DENSE, 1, 16, 9, 11, 16, 3, 1, 1, A.RELU, scales=(0.02, 0.01, 0.05))
+    # rounding ties: acc * 0.5 * 0.5 / 0.5 = acc / 2 -> every odd accumulator is an exact .5
+    c["conv44_3x3_s1_ties"] = ConvCase(
+        A.FMT_NCHW44, A.DENSE, 1, 8, 6, 5, 8, 3, 1, 1, A.IDENTITY, scales=(0.5, 0.5, 0.5),
+        src_range=(-3, 3), flt_range=(-3, 3), bias_range=(-3, 3))
+    # overflow case of the reference tests: all-positive 30..50 -> clamps at 127
+    c["conv44_3x3_s1_overflow"] = ConvCase(
+        A.FMT_NCHW44, A.DENSE, 1, 8, 6, 5, 8, 3, 1, 1, A.IDENTITY, scales=(1.0, 1.0, 1.0),
+        src_range=(30, 50), flt_range=(30, 50), bias_range=(30, 50))
+    c["conv44_3x3_s2_RELU"] = ConvCase(
+        A.FMT_NCHW44, A.DENSE, 2, 8, 9, 8, 8, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(72)))
+    c["conv44_3x3_s1_p0"] = ConvCase(
+        A.FMT_NCHW44, A.DENSE, 1, 8, 7, 7, 8, 3, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(72)))
+    c["conv44_1x1_RELU"] = ConvCase(
+        A.FMT_NCHW44, A.DENSE, 2, 16, 5, 7, 24, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(16)))
+    # (a qsi8 conv without bias does not exist in the reference: ConvGeneral::IsAvailable wants
+    #  operand:2 to be qsi32, BareMetal/ConvKernel.cpp:25-29)
+    # --- qsi8 NCHW dense: FullyConnected (1x1 on [M,K,1,1]) and 3x3
+    c["fc_q8_5x40x13"] = ConvCase(
+        A.FMT_NCHW, A.DENSE, 5, 40, 1, 1, 13, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(40) / 2))
+    c["fc_q8_1x64x10_RELU"] = ConvCase(
+        A.FMT_NCHW, A.DENSE, 1, 64, 1, 1, 10, 1, 1, 0, A.RELU, scales=(0.01, 0.01, 0.1))
+    c["conv_nchw_3x3_s1"] = ConvCase(
+        A.FMT_NCHW, A.DENSE, 2, 5, 7, 6, 7, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(45)))
+    c["conv_nchw_3x3_s2"] = ConvCase(
+        A.FMT_NCHW, A.DENSE, 1, 5, 9, 9, 6, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(45)))
+    # --- depthwise
+    for s in (1, 2):
+        c["dw44_3x3_s%d_RELU" % s] = ConvCase(
+            A.FMT_NCHW44, A.GROUP, 2, 8, 9, 7, 8, 3, s, 1, A.RELU, scales=(0.02, 0.01, unsat(9)))
+        c["dw_nchw_3x3_s%d_RELU" % s] = ConvCase(
+            A.FMT_NCHW, A.GROUP, 2, 6, 9, 7, 6, 3, s, 1, A.RELU, scales=(0.02, 0.01, unsat(9)))
+    c["dw44_3x3_s1_IDENTITY_baseline_scales"] = ConvCase(
+        A.FMT_NCHW44, A.GROUP, 1, 8, 6, 6, 8, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, 0.05))
+    # --- first layer NCHW -> NCHW44
+    c["conv_hybrid_3x3_s2_RELU"] = ConvCase(
+        A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 11, 9, 8, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27)))
+    # --- f32 (tolerance-based)
+    c["conv_f32_3x3_RELU"] = ConvCase(A.FMT_NCHW, A.DENSE, 1, 6, 9, 8, 5, 3, 1, 1, A.RELU, dtype="f32")
+    c["matmul_f32_11x8x13"] = MatMulCase(11, 8, 13)
+    c["gevm_f32_1x37x29"] = MatMulCase(1, 37, 29)
+    # --- pooling
+    c["pool_max_nchw_2x2"] = PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 3, 8, 6, 2, 2, 0)
+    c["pool_max_nchw44_2x2"] = PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 8, 8, 6, 2, 2, 0)
+    c["pool_max_nchw_3x3_p1"] = PoolCase(A.FMT_NCHW, A.POOL_MAX, 1, 3, 9, 7, 3, 2, 1)
+    c["pool_max_nchw44_3x3_p1"] = PoolCase(A.FMT_NCHW44, A.POOL_MAX, 1, 8, 9, 7, 3, 2, 1)
+    c["pool_avg_nchw_7x7"] = PoolCase(A.FMT_NCHW, A.POOL_AVERAGE, 2, 5, 7, 7, 7, 7, 0)
+    c["pool_avg_nchw44_7x7"] = PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE, 2, 8, 7, 7, 7, 7, 0)
+    c["pool_avg_nchw_3x3_p1"] = PoolCase(A.FMT_NCHW, A.POOL_AVERAGE, 1, 3, 9, 7, 3, 2, 1)
+    c["pool_avgx_nchw_3x3_p1"] = PoolCase(
+        A.FMT_NCHW, A.POOL_AVERAGE_COUNT_EXCLUDE_PADDING, 1, 3, 9, 7, 3, 2, 1)
+    # --- quantized elemwise: three broadcast modes
+    for mode in (A.Q_ADD, A.Q_FUSE_ADD_RELU, A.Q_MUL):
+        nm = A.MULTITYPE_NAMES[mode]
+        sc = (0.05, 0.01, 0.05) if mode != A.Q_MUL else (0.05, 0.04, 0.3)
+        c["%s_vec" % nm] = MultiTypeCase(mode, (2, 3, 5, 7), sc)
+        c["%s_chan" % nm] = MultiTypeCase(mode, (2, 3, 5, 7), sc, bshape=(1, 3, 1, 1))
+        c["%s_scalar" % nm] = MultiTypeCase(mode, (2, 3, 5, 7), sc, bshape=(1,))
+    c["QRELU"] = MultiTypeCase(A.Q_RELU, (2, 3, 5, 7), (0.05, 0.01, 0.03))
+    c["QADD_ties"] = MultiTypeCase(A.Q_ADD, (4, 1, 8, 8), (0.5, 0.5, 1.0))
+    # --- typecvt (37 elements: SIMD body of 16 + scalar tail)
+    c["cvt_f32_q8"] = TypeCvtCase("f32", "qsi8", (3, 37), dst_scale=0.02)
+    c["cvt_q8_f32"] = TypeCvtCase("qsi8", "f32", (3, 37), src_scale=0.05)
+    c["cvt_q8_q8"] = TypeCvtCase("qsi8", "qsi8", (3, 37), src_scale=0.05, dst_scale=0.02)
+    c["cvt_q32_q8"] = TypeCvtCase("qsi32", "qsi8", (3, 37), src_scale=0.0002, dst_scale=0.05)
+    return c

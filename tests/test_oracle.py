@@ -1,0 +1,175 @@
+"""CPU tests of the checker itself: the C restatement (oracle/oracle_port.c) against
+(1) the committed fixtures produced by the reference's own generated kernels (tests/golden/),
+(2) the same generated kernels run live where oracle/_ref has been built, on larger seeded cases,
+(3) what the mathematics fixes independently of either (exact integer correlation via numpy,
+    zero-weight and identity-weight closed forms)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import cases
+from cases import ConvCase, MultiTypeCase, PoolCase, TypeCvtCase, MatMulCase
+from golden_cases import golden_cases, unsat
+from megcc_amd import abi
+from oracle import port, ref
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLD = np.load(os.path.join(HERE, "golden", "golden.npz"))
+with open(os.path.join(HERE, "golden", "symbols.json")) as f:
+    SYMBOLS = json.load(f)
+CASES = golden_cases()
+F32_TOL = 1e-4  # max |a-b| / max(1, min(|a|,|b|)), the north star's fp32 bar
+
+
+def golden_arrays(name):
+    out = {}
+    for key in GOLD.files:
+        if key.startswith(name + "/"):
+            out[key.split("/", 1)[1]] = GOLD[key]
+    return out
+
+
+def is_float_case(case):
+    _, outs = case.specs(case.gen(0))
+    return outs[0].type_enum == abi.FLOAT
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_port_matches_golden(name):
+    case = CASES[name]
+    g = golden_arrays(name)
+    arrays = {k: g.get(k) for k in case.gen(0).keys()}
+    got = case.run_port(arrays)
+    if got.dtype == np.float32:
+        assert cases.max_rel_err(got, g["expect"]) <= F32_TOL
+    else:
+        np.testing.assert_array_equal(got, g["expect"])
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_symbol_mirror(name):
+    """our reading of the reference's symbol scheme against what its registry actually chose"""
+    case = CASES[name]
+    if isinstance(case, ConvCase) and case.dtype == "f32":
+        assert SYMBOLS[name].startswith("GI_kernel_conv2d_im2col_3x3_NCHW_DENSE")
+    else:
+        assert case.symbol() == SYMBOLS[name]
+
+
+def test_golden_not_degenerate():
+    """the fixtures must exercise rounding, not just the clamps"""
+    for name in ("conv44_3x3_s1_IDENTITY", "conv44_1x1_RELU", "fc_q8_5x40x13", "dw44_3x3_s1_RELU"):
+        e = GOLD[name + "/expect"]
+        sat = np.mean((e == 127) | (e == -128))
+        assert sat < 0.2, (name, sat)
+        assert len(np.unique(e)) > 40, name
+    e = GOLD["conv44_3x3_s1_overflow/expect"]
+    assert (e == 127).all()
+
+
+LIVE = [
+    ConvCase(abi.FMT_NCHW44, abi.DENSE, 2, 64, 14, 14, 64, 3, 1, 1, abi.RELU, scales=(0.02, 0.01, unsat(576))),
+    ConvCase(abi.FMT_NCHW44, abi.DENSE, 1, 32, 12, 13, 48, 3, 1, 1, abi.IDENTITY, scales=(0.02, 0.01, 0.05)),
+    ConvCase(abi.FMT_NCHW44, abi.DENSE, 1, 32, 9, 9, 32, 3, 1, 1, abi.H_SWISH, scales=(0.02, 0.01, unsat(288))),
+    ConvCase(abi.FMT_NCHW44, abi.DENSE, 1, 32, 9, 9, 32, 3, 1, 1, abi.SIGMOID, scales=(0.02, 0.01, unsat(288) * 40)),
+    ConvCase(abi.FMT_NCHW44, abi.DENSE, 2, 64, 7, 7, 128, 1, 1, 0, abi.RELU, scales=(0.02, 0.01, unsat(64))),
+    ConvCase(abi.FMT_NCHW, abi.DENSE, 16, 256, 1, 1, 100, 1, 1, 0, abi.IDENTITY, scales=(0.01, 0.01, unsat(256) / 2)),
+    ConvCase(abi.FMT_NCHW44, abi.GROUP, 2, 32, 20, 18, 32, 3, 1, 1, abi.RELU, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(abi.FMT_NCHW44, abi.GROUP, 2, 32, 20, 18, 32, 3, 2, 1, abi.RELU, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(abi.FMT_NCHW_NCHW44, abi.DENSE, 1, 3, 32, 32, 32, 3, 2, 1, abi.RELU, scales=(0.02, 0.01, unsat(27))),
+    PoolCase(abi.FMT_NCHW44, abi.POOL_MAX, 2, 16, 14, 14, 2, 2, 0),
+    PoolCase(abi.FMT_NCHW44, abi.POOL_AVERAGE, 3, 64, 7, 7, 7, 7, 0),
+    PoolCase(abi.FMT_NCHW, abi.POOL_AVERAGE, 3, 64, 7, 7, 7, 7, 0),
+    MultiTypeCase(abi.Q_FUSE_ADD_RELU, (4, 32, 14, 14), (0.05, 0.01, 0.05)),
+    MultiTypeCase(abi.Q_ADD, (4, 32, 14, 14), (0.031, 0.017, 0.023)),
+    TypeCvtCase("f32", "qsi8", (5, 1001), dst_scale=0.0173),
+    TypeCvtCase("qsi8", "qsi8", (5, 1001), src_scale=0.0173, dst_scale=0.0291),
+]
+
+
+@pytest.mark.skipif(not ref.available(), reason="oracle/_ref not built (needs /root/reference)")
+@pytest.mark.parametrize("case", LIVE, ids=[repr(c) for c in LIVE])
+def test_port_matches_reference_live(case):
+    if not ref.has(case.symbol()):
+        pytest.skip("symbol not in this _ref build")
+    arrays = case.gen(seed=7)
+    want = cases.run_ref(case, arrays)
+    got = case.run_port(arrays)
+    np.testing.assert_array_equal(got, want)
+
+
+# ---- checks that do not involve the reference at all ----------------------------------------
+def _acc_numpy_nchw44_dense(src, flt, bias, pad, stride):
+    """exact int64 correlation, written against the layout definition (not the port's loops)"""
+    n, c4, ih, iw, _ = src.shape
+    oc4 = flt.shape[0]
+    x = src.transpose(0, 1, 4, 2, 3).reshape(n, c4 * 4, ih, iw).astype(np.int64)
+    # flt[oc/4, ic/4, fh, fw, ic%4, oc%4] -> w[oc, ic, fh, fw]
+    w = flt.transpose(0, 5, 1, 4, 2, 3).reshape(oc4 * 4, c4 * 4, flt.shape[2], flt.shape[3]).astype(np.int64)
+    xp = np.pad(x, ((0, 0), (0, 0), (pad, pad), (pad, pad)))
+    fh, fw = w.shape[2:]
+    oh = (ih + 2 * pad - fh) // stride + 1
+    ow = (iw + 2 * pad - fw) // stride + 1
+    acc = np.zeros((n, oc4 * 4, oh, ow), np.int64)
+    for a in range(fh):
+        for b in range(fw):
+            win = xp[:, :, a:a + stride * oh:stride, b:b + stride * ow:stride]
+            acc += np.einsum("nchw,oc->nohw", win, w[:, :, a, b])
+    acc += bias.reshape(1, -1, 1, 1)
+    return acc
+
+
+def _requant_numpy(acc, s0, s1, s2, relu):
+    v = acc.astype(np.int32).astype(np.float32) * np.float32(s0) * np.float32(s1) / np.float32(s2)
+    if relu:
+        v = np.where(v > 0, v, np.float32(0))
+    r = np.sign(v) * np.floor(np.abs(v) + np.float32(0.5))  # half away from zero
+    # floor(|v|+0.5) in fp32 can differ from roundf for |v| just below .5: compare via float64
+    r = np.sign(v) * np.floor(np.abs(v.astype(np.float64)) + 0.5)
+    return np.clip(r, -128, 127).astype(np.int8)
+
+
+@pytest.mark.parametrize("stride,relu", [(1, False), (1, True), (2, True)])
+def test_port_conv_vs_numpy_closed_form(stride, relu):
+    case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 2, 16, 10, 9, 24, 3, stride, 1,
+                    abi.RELU if relu else abi.IDENTITY, scales=(0.02, 0.01, unsat(144)))
+    a = case.gen(3)
+    acc = _acc_numpy_nchw44_dense(a["src"], a["flt"], a["bias"].reshape(-1), 1, stride)
+    want = _requant_numpy(acc, *case.scales, relu)
+    want44 = want.reshape(2, 6, 4, case.oh, case.ow).transpose(0, 1, 3, 4, 2)
+    np.testing.assert_array_equal(case.run_port(a), want44)
+
+
+def test_port_conv_zero_weight_gives_bias_only():
+    case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 1, 8, 5, 5, 8, 3, 1, 1, abi.IDENTITY,
+                    scales=(0.5, 0.5, 0.25), bias_range=(-100, 100))
+    a = case.gen(1)
+    a["flt"][:] = 0
+    got = case.run_port(a)
+    want = np.clip(a["bias"].reshape(1, 2, 1, 1, 4), -128, 127).astype(np.int8)  # 0.5*0.5/0.25 = 1
+    np.testing.assert_array_equal(got, np.broadcast_to(want, got.shape))
+
+
+def test_port_fc_identity_weight():
+    k = 16
+    case = ConvCase(abi.FMT_NCHW, abi.DENSE, 7, k, 1, 1, k, 1, 1, 0, abi.IDENTITY,
+                    scales=(1.0, 1.0, 1.0), bias_range=(0, 0))
+    a = case.gen(2)
+    a["flt"][:] = np.eye(k, dtype=np.int8).reshape(k, k, 1, 1)
+    np.testing.assert_array_equal(case.run_port(a), a["src"])
+
+
+def test_port_maxpool_vs_numpy():
+    case = PoolCase(abi.FMT_NCHW, abi.POOL_MAX, 2, 3, 8, 6, 2, 2, 0)
+    a = case.gen(5)
+    want = a["src"].reshape(2, 3, 4, 2, 3, 2).max(axis=(3, 5))
+    np.testing.assert_array_equal(case.run_port(a), want)
+
+
+def test_port_matmul_vs_float64():
+    case = MatMulCase(9, 33, 17)
+    a = case.gen(4)
+    want = a["a"].astype(np.float64) @ a["b"].astype(np.float64)
+    assert cases.max_rel_err(case.run_port(a), want) <= 1e-5

@@ -1,0 +1,76 @@
+// Shared host-side helpers of libmegcc_gfx950.so: error reporting, the library stream, Tensor
+// inspection. Everything here is host code; device helpers live in epilogue.cuh.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "megcc_gfx950.h"
+
+namespace mg {
+
+// One stream for every launch and copy, default priority, created on first use.
+hipStream_t stream();
+
+// Records a message for megcc_gfx950_last_error() and returns `st`.
+TinyNNStatus fail(TinyNNStatus st, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define MG_REQUIRE(cond, st, ...)          \
+    do {                                   \
+        if (!(cond))                       \
+            return ::mg::fail(st, __VA_ARGS__); \
+    } while (0)
+
+// After a kernel launch: surfaces launch-configuration errors as TinyNN_ERROR_RUNTIME.
+TinyNNStatus check_launch(const char* what);
+
+inline size_t nr_elem(const Layout& l) {
+    size_t n = 1;
+    for (int i = 0; i < l.nr_dim; ++i)
+        n *= l.dims[i];
+    return n;
+}
+
+// Dense row-major strides (dims of extent 1 may carry any stride).
+inline bool is_contiguous(const Layout& l) {
+    long expect = 1;
+    for (int i = l.nr_dim - 1; i >= 0; --i) {
+        if (l.dims[i] != 1 && l.stride[i] != expect)
+            return false;
+        expect *= l.dims[i];
+    }
+    return true;
+}
+
+inline bool is_q8(const Tensor* t) {
+    return t->dtype.type_enum == TinyNN_QINT8 || t->dtype.type_enum == TinyNN_INT8;
+}
+inline bool is_q32(const Tensor* t) {
+    return t->dtype.type_enum == TinyNN_QINT32 || t->dtype.type_enum == TinyNN_INT;
+}
+inline bool is_f32(const Tensor* t) {
+    return t->dtype.type_enum == TinyNN_FLOAT;
+}
+inline size_t dtype_size(const Tensor* t) {
+    switch (t->dtype.type_enum) {
+        case TinyNN_FLOAT:
+        case TinyNN_INT:
+        case TinyNN_QINT32:
+            return 4;
+        case TinyNN_FLOAT16:
+        case TinyNN_INT16:
+            return 2;
+        default:
+            return 1;
+    }
+}
+
+inline unsigned ceil_div(size_t a, size_t b) {
+    return (unsigned)((a + b - 1) / b);
+}
+
+// NULL / pointer checks shared by every entry point (the reference kernels TINYNN_ASSERT these).
+TinyNNStatus check_io(
+        Tensor** inputs, int nr_input, int want_in_min, int want_in_max, Tensor** outputs,
+        int nr_output, const char* who);
+
+}  // namespace mg

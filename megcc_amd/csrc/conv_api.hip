@@ -1,0 +1,236 @@
+// ConvBias entry points: derive the geometry from the Tensor layouts exactly as the reference's
+// generated kernel does at run time (BareMetal/ConvKernel.cpp:262-287), validate what that kernel
+// would TINYNN_ASSERT, and route to the kernel for the case:
+//   qsi8 NCHW44 DENSE, qsi8 FullyConnected (1x1 NCHW on [M,K,1,1])  -> conv_mfma_i8.hip
+//   qsi8 NCHW44 depthwise                                           -> dwconv.hip
+//   f32 NCHW DENSE                                                  -> gemm_f32.hip
+//   everything else ConvGeneral accepts                             -> conv_direct.hip
+#include "common.h"
+#include "conv_geom.h"
+
+namespace mg {
+bool conv_mfma_supported(const ConvGeom& g);
+size_t conv_mfma_packed_bytes(const ConvGeom& g);
+TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed);
+TinyNNStatus conv_mfma_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+bool dwconv44_supported(const ConvGeom& g);
+TinyNNStatus dwconv44_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+bool conv_f32_gemm_supported(const ConvGeom& g);
+TinyNNStatus conv_f32_gemm_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+TinyNNStatus conv_direct_launch(const ConvGeom&, bool, const void*, const void*, const void*, void*);
+
+// A filter that went through megcc_gfx950_conv2d_init is a 1-d byte tensor.
+static bool is_packed_filter(const Tensor* flt) {
+    return flt->layout.nr_dim == 1;
+}
+
+// Fills `g` from (attr, src, filter, dst). `dst` may be NULL (init / workspace time): the output
+// extent is then computed from the convolution formula.
+static TinyNNStatus make_geom(
+        const MegccConvAttr* a, const Tensor* src, const Tensor* flt, const Tensor* dst,
+        bool filter_is_packed, int oc_hint, ConvGeom* g) {
+    const int fmt = a->format;
+    MG_REQUIRE(fmt == MEGCC_FMT_NCHW || fmt == MEGCC_FMT_NCHW44 || fmt == MEGCC_FMT_NCHW_NCHW44,
+               TinyNN_ERROR_NO_IMPLEMENT, "conv2d: format %d", fmt);
+    const int src_dims = fmt == MEGCC_FMT_NCHW44 ? 5 : 4;
+    MG_REQUIRE(src->layout.nr_dim == src_dims && is_contiguous(src->layout),
+               TinyNN_ERROR_INVALID_LAYOUT, "conv2d: source must be a contiguous %d-d tensor",
+               src_dims);
+    MG_REQUIRE(a->kernel_h && a->kernel_w && a->stride_h && a->stride_w && a->dilate_h &&
+                       a->dilate_w,
+               TinyNN_ERROR_OUT_OF_RANGE, "conv2d: zero kernel / stride / dilation");
+    const int ic_ratio = fmt == MEGCC_FMT_NCHW44 ? 4 : 1;
+    const int oc_ratio = fmt == MEGCC_FMT_NCHW ? 1 : 4;
+    g->fmt = fmt;
+    g->act = a->nonline;
+    g->has_bias = a->with_bias;
+    g->n = src->layout.dims[0];
+    g->ic = src->layout.dims[1] * ic_ratio;
+    g->ih = src->layout.dims[2];
+    g->iw = src->layout.dims[3];
+    g->fh = a->kernel_h; g->fw = a->kernel_w;
+    g->sh = a->stride_h; g->sw = a->stride_w;
+    g->ph = a->pad_h; g->pw = a->pad_w;
+    g->dh = a->dilate_h; g->dw = a->dilate_w;
+    if (dst) {
+        const int dst_dims = fmt == MEGCC_FMT_NCHW ? 4 : 5;
+        MG_REQUIRE(dst->layout.nr_dim == dst_dims && is_contiguous(dst->layout),
+                   TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: destination must be a contiguous %d-d tensor", dst_dims);
+        g->oc = dst->layout.dims[1] * oc_ratio;
+        g->oh = dst->layout.dims[2];
+        g->ow = dst->layout.dims[3];
+        MG_REQUIRE(dst->layout.dims[0] == (uint32_t)g->n, TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: batch of source and destination differ");
+    } else {
+        g->oc = oc_hint;
+        g->oh = g->ow = -1;
+    }
+    const int eh = g->dh * (g->fh - 1) + 1, ew = g->dw * (g->fw - 1) + 1;
+    const int want_oh = g->ih + 2 * g->ph >= eh ? (g->ih + 2 * g->ph - eh) / g->sh + 1 : 0;
+    const int want_ow = g->iw + 2 * g->pw >= ew ? (g->iw + 2 * g->pw - ew) / g->sw + 1 : 0;
+    if (dst)
+        MG_REQUIRE(g->oh == want_oh && g->ow == want_ow, TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: destination is %dx%d, the convolution yields %dx%d", g->oh, g->ow,
+                   want_oh, want_ow);
+    g->oh = want_oh;
+    g->ow = want_ow;
+
+    // group count and filter shape (BareMetal/ConvKernel.cpp:209-236, 48-76)
+    g->groups = 1;
+    if (!filter_is_packed) {
+        const Layout& fl = flt->layout;
+        if (a->sparse == MEGCC_SPARSE_GROUP) {
+            MG_REQUIRE(fmt != MEGCC_FMT_NCHW_NCHW44, TinyNN_ERROR_NO_IMPLEMENT,
+                       "conv2d: NCHW->NCHW44 is DENSE only");
+            g->groups = fl.dims[0] * (fmt == MEGCC_FMT_NCHW44 ? 4 : 1);
+        }
+        if (!dst && a->sparse == MEGCC_SPARSE_DENSE) {
+            g->oc = fl.dims[0] * oc_ratio;
+        } else if (!dst) {
+            g->oc = fmt == MEGCC_FMT_NCHW ? fl.dims[0] * fl.dims[1] : g->groups;
+        }
+        MG_REQUIRE(g->groups > 0 && g->oc % g->groups == 0 && g->ic % g->groups == 0,
+                   TinyNN_ERROR_INVALID_LAYOUT, "conv2d: %d groups do not divide ic=%d / oc=%d",
+                   g->groups, g->ic, g->oc);
+        const int ocpg = g->oc / g->groups, icpg = g->ic / g->groups;
+        size_t want;
+        if (fmt == MEGCC_FMT_NCHW44 && a->sparse == MEGCC_SPARSE_GROUP) {
+            MG_REQUIRE(ocpg == 1 && icpg == 1, TinyNN_ERROR_NO_IMPLEMENT,
+                       "conv2d: NCHW44 GROUP is implemented for channel-wise filters only");
+            want = (size_t)g->groups * g->fh * g->fw;
+        } else {
+            want = (size_t)g->groups * ocpg * icpg * g->fh * g->fw;
+        }
+        MG_REQUIRE(nr_elem(fl) == want && is_contiguous(fl), TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: filter has %zu elements, expected %zu", nr_elem(fl), want);
+    } else {
+        MG_REQUIRE(a->sparse == MEGCC_SPARSE_DENSE, TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: packed filter with a GROUP convolution");
+    }
+    if (fmt != MEGCC_FMT_NCHW)
+        MG_REQUIRE(g->oc % 4 == 0, TinyNN_ERROR_INVALID_LAYOUT, "conv2d: oc %% 4 != 0");
+    g->s_src = src->dtype.param.scale;
+    g->s_flt = flt->dtype.param.scale;
+    g->s_dst = dst ? dst->dtype.param.scale : 1.f;
+    return TinyNN_SUCCESS;
+}
+
+static bool aligned4(const void* p) {
+    return ((uintptr_t)p & 3) == 0;
+}
+static bool aligned16(const void* p) {
+    return ((uintptr_t)p & 15) == 0;
+}
+
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" TinyNNStatus megcc_gfx950_conv2d(
+        const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace*, const RuntimeOpt*) {
+    MG_REQUIRE(attr, TinyNN_ERROR_NULL_PTR, "conv2d: NULL attr");
+    const int want_in = attr->with_bias ? 3 : 2;
+    // the test harness of the reference passes an extra empty `z` operand after the bias
+    TinyNNStatus st = check_io(inputs, nr_input < want_in ? nr_input : want_in, want_in, want_in,
+                               outputs, nr_output, "conv2d");
+    if (st != TinyNN_SUCCESS)
+        return st;
+    MG_REQUIRE(nr_input <= want_in + 1, TinyNN_ERROR_OUT_OF_RANGE, "conv2d: %d inputs", nr_input);
+    const Tensor *src = inputs[0], *flt = inputs[1], *dst = outputs[0];
+    const Tensor* bias = attr->with_bias ? inputs[2] : nullptr;
+    const bool q8 = is_q8(src) && is_q8(flt) && is_q8(dst) && (!bias || is_q32(bias));
+    const bool f32 = is_f32(src) && is_f32(flt) && is_f32(dst) && (!bias || is_f32(bias));
+    MG_REQUIRE(q8 || f32, TinyNN_ERROR_UNSUPPORTED_DTYPE_TYPE,
+               "conv2d: operands must be qsi8,qsi8[,qsi32]->qsi8 or all f32");
+    const bool packed = is_packed_filter(flt);
+    ConvGeom g;
+    st = make_geom(attr, src, flt, dst, packed, 0, &g);
+    if (st != TinyNN_SUCCESS)
+        return st;
+    if (bias) {
+        MG_REQUIRE(nr_elem(bias->layout) == (size_t)g.oc, TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: bias must be per output channel (%zu elements, oc=%d)",
+                   nr_elem(bias->layout), g.oc);
+        if (q8) {
+            // ConvGeneral::IsAvailable, BareMetal/ConvKernel.cpp:37-42
+            float d = g.s_src * g.s_flt - bias->dtype.param.scale;
+            MG_REQUIRE((d < 0 ? -d : d) < 1e-5f, TinyNN_ERROR_UNSUPPORTED_DTYPE_TYPE,
+                       "conv2d: bias scale %g != src scale * filter scale %g",
+                       bias->dtype.param.scale, g.s_src * g.s_flt);
+        }
+    }
+    if (q8)
+        MG_REQUIRE(g.s_dst > 0.f, TinyNN_ERROR_UNSUPPORTED_DTYPE_TYPE, "conv2d: dst scale <= 0");
+    const void* b = bias ? bias->ptr : nullptr;
+    if ((size_t)g.n * g.oc * g.oh * g.ow == 0)
+        return TinyNN_SUCCESS;
+
+    if (packed) {
+        MG_REQUIRE(q8 && conv_mfma_supported(g), TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: a packed filter was passed to a convolution the MFMA kernel does not cover");
+        MG_REQUIRE(nr_elem(flt->layout) == conv_mfma_packed_bytes(g), TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: packed filter has %zu bytes, expected %zu", nr_elem(flt->layout),
+                   conv_mfma_packed_bytes(g));
+        MG_REQUIRE(aligned4(src->ptr) && aligned4(dst->ptr) && aligned16(flt->ptr) &&
+                           (!b || aligned4(b)),
+                   TinyNN_ERROR_INVALID_LAYOUT, "conv2d: misaligned operand");
+        return conv_mfma_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+    }
+    if (q8 && dwconv44_supported(g) && aligned4(src->ptr) && aligned4(flt->ptr) &&
+        aligned4(dst->ptr))
+        return dwconv44_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+    if (f32 && conv_f32_gemm_supported(g))
+        return conv_f32_gemm_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+    return conv_direct_launch(g, f32, src->ptr, flt->ptr, b, dst->ptr);
+}
+
+extern "C" TinyNNStatus megcc_gfx950_conv2d_init(
+        const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor* out_weights,
+        int* nr_out_weight, const RuntimeOpt*) {
+    MG_REQUIRE(attr && inputs && nr_input >= 2 && inputs[0] && inputs[1], TinyNN_ERROR_NULL_PTR,
+               "conv2d_init: NULL argument");
+    const Tensor *src = inputs[0], *flt = inputs[1];
+    ConvGeom g;
+    bool pack = false;
+    if (is_q8(src) && is_q8(flt) && attr->sparse == MEGCC_SPARSE_DENSE &&
+        !is_packed_filter(flt)) {
+        TinyNNStatus st = make_geom(attr, src, flt, nullptr, false, 0, &g);
+        if (st != TinyNN_SUCCESS)
+            return st;
+        pack = conv_mfma_supported(g);
+    }
+    if (!out_weights) {  // phase 1: how many
+        MG_REQUIRE(nr_out_weight, TinyNN_ERROR_NULL_PTR, "conv2d_init: both outputs NULL");
+        *nr_out_weight = pack ? 1 : 0;
+        return TinyNN_SUCCESS;
+    }
+    if (!pack) {
+        if (nr_out_weight)
+            *nr_out_weight = 0;
+        return TinyNN_SUCCESS;
+    }
+    if (!nr_out_weight) {  // phase 2: describe
+        out_weights->layout.nr_dim = 1;
+        out_weights->layout.dims[0] = (uint32_t)conv_mfma_packed_bytes(g);
+        out_weights->layout.stride[0] = 1;
+        out_weights->layout.format = flt->layout.format;
+        out_weights->dtype = flt->dtype;
+        out_weights->name = flt->name;  // identity by name pointer: runtime/src/init.c:64,88
+        return TinyNN_SUCCESS;
+    }
+    // phase 3: transform into the caller-allocated device buffer
+    MG_REQUIRE(out_weights->ptr && flt->ptr, TinyNN_ERROR_NULL_PTR, "conv2d_init: NULL weight");
+    MG_REQUIRE(aligned16(out_weights->ptr), TinyNN_ERROR_INVALID_LAYOUT,
+               "conv2d_init: processed weight must be 16-byte aligned");
+    *nr_out_weight = 1;
+    return conv_mfma_pack(g, flt->ptr, out_weights->ptr);
+}
+
+extern "C" TinyNNStatus megcc_gfx950_conv2d_workspace(
+        const MegccConvAttr*, Tensor**, int, int, size_t* workspace) {
+    MG_REQUIRE(workspace, TinyNN_ERROR_NULL_PTR, "conv2d_workspace: NULL size");
+    *workspace = 0;
+    return TinyNN_SUCCESS;
+}

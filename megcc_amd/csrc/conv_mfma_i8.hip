@@ -1,0 +1,453 @@
+// qsi8 dense convolution / FullyConnected as an implicit GEMM on the gfx950 matrix cores
+// (v_mfma_i32_32x32x32_i8): rows = output channels, columns = output pixels, K = (tap, ic).
+//
+// Replaces, for format NCHW44 + sparse DENSE and for the 1x1 NCHW convolution on [M,K,1,1] that
+// MegCC uses as quantized FullyConnected, the scalar seven-deep loop of BareMetal::ConvGeneral
+// (compiler/lib/KernelGen/BareMetal/ConvKernel.cpp:305-344). int8 x int8 products are summed
+// exactly in int32, so any summation order gives the reference's accumulator; the epilogue is the
+// reference's float sequence (epilogue.cuh).
+//
+// Data movement per workgroup (256 threads = 4 waves in a 2x2 grid, tile BM oc x 128 pixels):
+//   * the filter is pre-packed once by the _init entry point into rows of 32 consecutive input
+//     channels per (ic-chunk, tap, oc): a tile is a straight 16-byte-vector copy into LDS;
+//   * the activations needed by ALL taps of the tile (the tile's pixels plus their halo, in a
+//     zero-padded "virtual" image) are gathered once per ic-chunk from the NCHW44 planes into LDS
+//     rows of 32 channels per pixel -- im2col happens only as an LDS address offset per tap, and
+//     padding is a predicated zero at load time, so there is no workspace and no 9x re-read;
+//   * both LDS tiles swap the two 16-byte halves of a row on every other group of 8 rows, which
+//     makes the 64-lane ds_read_b128 of an MFMA operand (stride 32 bytes between lanes) hit every
+//     bank once;
+//   * the MFMA result layout (lane = pixel, 4 consecutive registers = 4 consecutive oc) is exactly
+//     one NCHW44 dword per pixel, so 32 lanes store 128 contiguous bytes.
+#include "common.h"
+#include "conv_geom.h"
+#include "epilogue.cuh"
+
+namespace mg {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+static constexpr int BN = 128;       // pixels per workgroup
+static constexpr int THREADS = 256;  // 4 waves
+static constexpr int KROW = 32;      // input channels per LDS row = K of one MFMA
+static constexpr int MAX_TAPS_STAGE = 9;
+static constexpr int MAX_B_ITEMS = 8;  // 16-byte gather items per thread per stage
+static constexpr int OC_PAD = 128;
+
+// unsigned division by a run-time constant: q = (x * mul) >> (32 + shift), exact for x < 2^31
+struct FastDiv {
+    uint32_t mul, shift, d;
+};
+static FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    if (d == 1) {
+        f.mul = 0;
+        f.shift = 0;
+        return f;
+    }
+    uint32_t s = 0;
+    while ((1u << s) < d)
+        ++s;  // ceil(log2 d)
+    uint64_t m = ((uint64_t(1) << (32 + s - 1)) + d - 1) / d;  // fits 32 bits for x < 2^31
+    f.mul = (uint32_t)m;
+    f.shift = s - 1;
+    return f;
+}
+__device__ __forceinline__ uint32_t fdiv(uint32_t x, const FastDiv& f) {
+    return f.d == 1 ? x : (__umulhi(x, f.mul) >> f.shift);
+}
+
+struct MfmaParams {
+    const int8_t* src;
+    const int8_t* wp;
+    const int32_t* bias;
+    int8_t* dst;
+    int P, OH, OW, OHW, N;
+    int OC, OCP, C4;
+    int stages, KS, taps, FH, FW;
+    int VW, VH, IH, IW, PH, PW, SH, SW, DH, DW;
+    int image_stride, plane_stride, row_stride, pix_stride;  // bytes
+    int Lmax;    // LDS patch slots (multiple of 64)
+    int dst_fc;  // 0: NCHW44, 1: [P][OC] row-major
+    int act;
+    float s_src, s_flt, s_dst;
+    FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
+};
+
+// virtual pixel index of output pixel p at tap (0,0): rows of the zero-padded images stacked
+__device__ __forceinline__ int vp_of(const MfmaParams& q, int p) {
+    int g = fdiv(p, q.dOW), ow = p - g * q.OW;
+    int n = fdiv(g, q.dOH), oh = g - n * q.OH;
+    return (n * q.VH + oh * q.SH) * q.VW + ow * q.SW;
+}
+
+template <int BM>
+__global__ void __launch_bounds__(THREADS) conv_mfma_i8_kernel(MfmaParams q) {
+    constexpr int WM = BM / 2;          // rows per wave
+    constexpr int MT = WM / 32;         // 32x32 tiles per wave along oc
+    constexpr int NT = 2;               // 64 pixels per wave
+    constexpr int A_ROW_CHUNKS = BM * 2;  // 16-byte chunks per tap
+    constexpr int MAX_A_ITEMS = MAX_TAPS_STAGE * A_ROW_CHUNKS / THREADS;
+
+    extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+    const int taps_stage = q.taps * q.KS;
+    int8_t* ldsA = lds;
+    int8_t* ldsB = lds + taps_stage * BM * KROW;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int p0 = blockIdx.x * BN, oc0 = blockIdx.y * BM;
+    const int plast = min(p0 + BN, q.P) - 1;
+    const int vp0 = vp_of(q, p0);
+    const int L = vp_of(q, plast) + ((q.FH - 1) * q.DH) * q.VW + (q.FW - 1) * q.DW - vp0 + 1;
+
+    // ---- gather items of this thread: (patch slot, 16-byte half of a 32-channel row, sub-chunk)
+    int b_goff[MAX_B_ITEMS];   // byte offset of the pixel in plane 0 of its image, -1 = zero fill
+    int b_loff[MAX_B_ITEMS];   // LDS byte offset of the 16-byte destination, -1 = no item
+    int b_plane[MAX_B_ITEMS];  // first of the 4 planes, relative to the stage
+    const int n_items = 2 * q.KS * q.Lmax;
+#pragma unroll
+    for (int j = 0; j < MAX_B_ITEMS; ++j) {
+        int i = tid + j * THREADS;
+        b_goff[j] = -1;
+        b_loff[j] = -1;
+        b_plane[j] = 0;
+        if (i < n_items) {
+            int h = fdiv(i, q.dL), slot = i - h * q.Lmax;  // h = ks*2 + half
+            b_loff[j] = (h >> 1) * (q.Lmax * KROW) + slot * KROW + (((h ^ (slot >> 3)) & 1) << 4);
+            b_plane[j] = (h >> 1) * 8 + (h & 1) * 4;
+            if (slot < L) {
+                int vp = vp0 + slot;
+                int v = fdiv(vp, q.dVW), vc = vp - v * q.VW;
+                int n = fdiv(v, q.dVH), vh = v - n * q.VH;
+                int ih = vh - q.PH, iw = vc - q.PW;
+                if (n < q.N && (unsigned)ih < (unsigned)q.IH && (unsigned)iw < (unsigned)q.IW)
+                    b_goff[j] = n * q.image_stride + ih * q.row_stride + iw * q.pix_stride;
+            }
+        }
+    }
+
+    // ---- MFMA operand addresses of this lane
+    const int kg = lane >> 5;  // which 16 of the 32 K values this lane feeds
+    int a_off[MT];
+#pragma unroll
+    for (int mi = 0; mi < MT; ++mi) {
+        int r = wm * WM + mi * 32 + (lane & 31);
+        a_off[mi] = r * KROW + (((kg ^ (r >> 3)) & 1) << 4);
+    }
+    int b_slot[NT];
+#pragma unroll
+    for (int ni = 0; ni < NT; ++ni) {
+        int p = p0 + wn * 64 + ni * 32 + (lane & 31);
+        b_slot[ni] = p <= plast ? vp_of(q, p) - vp0 : 0;
+    }
+
+    v16i acc[MT][NT];
+#pragma unroll
+    for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NT; ++ni)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                acc[mi][ni][e] = 0;
+
+    v4i ra[MAX_A_ITEMS];
+    v4i rb[MAX_B_ITEMS];
+    const int a_items = taps_stage * A_ROW_CHUNKS;  // 16-byte chunks of filter per stage
+
+    auto prefetch = [&](int st) {
+#pragma unroll
+        for (int j = 0; j < MAX_A_ITEMS; ++j) {
+            int i = tid + j * THREADS;
+            if (i < a_items) {
+                int t = i / A_ROW_CHUNKS, c = i - t * A_ROW_CHUNKS;
+                const int8_t* g = q.wp + ((size_t)(st * taps_stage + t) * q.OCP + oc0) * KROW + c * 16;
+                ra[j] = *(const v4i*)g;
+            }
+        }
+        const int plane0 = st * q.KS * 8;
+#pragma unroll
+        for (int j = 0; j < MAX_B_ITEMS; ++j) {
+            v4i v = {0, 0, 0, 0};
+            if (b_goff[j] >= 0) {
+                int pl = plane0 + b_plane[j];
+                const int8_t* g = q.src + b_goff[j] + (size_t)pl * q.plane_stride;
+                // planes past the last one meet zero filter rows, so their value is irrelevant;
+                // they are only kept from reading out of bounds
+                if (pl + 0 < q.C4) v[0] = *(const int*)(g);
+                if (pl + 1 < q.C4) v[1] = *(const int*)(g + q.plane_stride);
+                if (pl + 2 < q.C4) v[2] = *(const int*)(g + 2 * q.plane_stride);
+                if (pl + 3 < q.C4) v[3] = *(const int*)(g + 3 * q.plane_stride);
+            }
+            rb[j] = v;
+        }
+    };
+
+    prefetch(0);
+    for (int st = 0; st < q.stages; ++st) {
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < MAX_A_ITEMS; ++j) {
+            int i = tid + j * THREADS;
+            if (i < a_items)
+                *(v4i*)(ldsA + i * 16) = ra[j];
+        }
+#pragma unroll
+        for (int j = 0; j < MAX_B_ITEMS; ++j)
+            if (b_loff[j] >= 0)
+                *(v4i*)(ldsB + b_loff[j]) = rb[j];
+        __syncthreads();
+        if (st + 1 < q.stages)
+            prefetch(st + 1);
+
+        for (int ks = 0; ks < q.KS; ++ks) {
+            const int8_t* bks = ldsB + ks * (q.Lmax * KROW);
+            int t = ks * q.taps;
+            for (int fh = 0; fh < q.FH; ++fh) {
+                for (int fw = 0; fw < q.FW; ++fw, ++t) {
+                    const int tap_off = fh * q.DH * q.VW + fw * q.DW;
+                    v4i a[MT], b[NT];
+#pragma unroll
+                    for (int mi = 0; mi < MT; ++mi)
+                        a[mi] = *(const v4i*)(ldsA + t * (BM * KROW) + a_off[mi]);
+#pragma unroll
+                    for (int ni = 0; ni < NT; ++ni) {
+                        int s = b_slot[ni] + tap_off;
+                        b[ni] = *(const v4i*)(bks + s * KROW + (((kg ^ (s >> 3)) & 1) << 4));
+                    }
+#pragma unroll
+                    for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+                        for (int ni = 0; ni < NT; ++ni)
+                            acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                    a[mi], b[ni], acc[mi][ni], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // ---- epilogue: register e of a 32x32 tile holds row 8*(e/4) + 4*(lane/32) + e%4, col lane%32
+#pragma unroll
+    for (int ni = 0; ni < NT; ++ni) {
+        const int p = p0 + wn * 64 + ni * 32 + (lane & 31);
+        if (p > plast)
+            continue;
+        const int n = fdiv(p, q.dOHW), rem = p - n * q.OHW;
+#pragma unroll
+        for (int mi = 0; mi < MT; ++mi) {
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int oc = oc0 + wm * WM + mi * 32 + e4 * 8 + kg * 4;
+                if (oc >= q.OC)
+                    continue;
+                int r[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    int a = acc[mi][ni][e4 * 4 + e];
+                    if (q.bias && oc + e < q.OC)
+                        a += q.bias[oc + e];
+                    r[e] = requant_conv_rt(q.act, a, q.s_src, q.s_flt, q.s_dst);
+                }
+                if (!q.dst_fc) {
+                    size_t o = ((size_t)n * (q.OC >> 2) + (oc >> 2)) * q.OHW + rem;
+                    ((uint32_t*)q.dst)[o] = pack4(r[0], r[1], r[2], r[3]);
+                } else {
+                    int8_t* o = q.dst + (size_t)p * q.OC + oc;
+                    if (((q.OC & 3) == 0)) {
+                        *(uint32_t*)o = pack4(r[0], r[1], r[2], r[3]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (oc + e < q.OC)
+                                o[e] = (int8_t)r[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---- filter packing ---------------------------------------------------------------------
+// packed[(chunk*taps + tap)*OCP + oc][pos], pos in 0..31 holds input channel
+// chunk*32 + (pos ^ 16*((oc>>3)&1)); zero beyond IC / OC.
+__global__ void __launch_bounds__(256) pack_filter_kernel(
+        const int8_t* __restrict__ flt, int8_t* __restrict__ out, size_t total, int taps, int FW,
+        int OC, int OCP, int IC, int fmt) {
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        int pos = i & 31;
+        size_t r = i >> 5;
+        int oc = r % OCP;
+        r /= OCP;
+        int tap = r % taps;
+        int chunk = (int)(r / taps);
+        int ic = chunk * 32 + (pos ^ (((oc >> 3) & 1) << 4));
+        int8_t v = 0;
+        if (oc < OC && ic < IC) {
+            int fh = tap / FW, fw = tap - fh * FW;
+            int FH = taps / FW;
+            size_t o;
+            if (fmt == MEGCC_FMT_NCHW44)  // [OC/4][IC/4][FH][FW][4 ic][4 oc]
+                o = (((((size_t)(oc >> 2) * (IC >> 2) + (ic >> 2)) * FH + fh) * FW + fw) * 4 +
+                     (ic & 3)) * 4 + (oc & 3);
+            else  // NCHW [OC][IC][FH][FW]
+                o = (((size_t)oc * IC + ic) * FH + fh) * FW + fw;
+            v = flt[o];
+        }
+        out[i] = v;
+    }
+}
+
+static int round_up(int a, int b) {
+    return (a + b - 1) / b * b;
+}
+
+static bool is_fc(const ConvGeom& g) {
+    return g.fmt == MEGCC_FMT_NCHW && g.ih == 1 && g.iw == 1 && g.fh == 1 && g.fw == 1 &&
+           g.oh == 1 && g.ow == 1 && g.ph == 0 && g.pw == 0;
+}
+
+static int choose_ks(int taps) {
+    return taps <= 2 ? 4 : taps <= 4 ? 2 : 1;
+}
+
+struct TilePlan {
+    int Lmax;
+    int VW, VH;
+};
+
+// largest patch any tile needs; mirrors vp_of() / L in the kernel
+static TilePlan plan_tiles(const ConvGeom& g) {
+    TilePlan t;
+    t.VW = g.iw + 2 * g.pw;
+    t.VH = g.ih + 2 * g.ph;
+    long P = (long)g.n * g.oh * g.ow;
+    auto vp = [&](long p) {
+        long gi = p / g.ow, ow = p % g.ow;
+        long n = gi / g.oh, oh = gi % g.oh;
+        return (n * t.VH + oh * g.sh) * t.VW + ow * g.sw;
+    };
+    long lmax = 1;
+    for (long p0 = 0; p0 < P; p0 += BN) {
+        long pl = (p0 + BN < P ? p0 + BN : P) - 1;
+        long L = vp(pl) + (long)(g.fh - 1) * g.dh * t.VW + (g.fw - 1) * g.dw - vp(p0) + 1;
+        if (L > lmax)
+            lmax = L;
+    }
+    t.Lmax = round_up((int)(lmax > (1 << 20) ? (1 << 20) : lmax), 64);
+    return t;
+}
+
+bool conv_mfma_supported(const ConvGeom& g) {
+    if (g.groups != 1)
+        return false;
+    bool fc = is_fc(g);
+    if (!(g.fmt == MEGCC_FMT_NCHW44 || fc))
+        return false;
+    if ((g.ic & 3) || g.fh * g.fw > MAX_TAPS_STAGE)
+        return false;
+    if (g.fmt == MEGCC_FMT_NCHW44 && (g.oc & 3))
+        return false;
+    long P = (long)g.n * g.oh * g.ow;
+    long src_bytes = (long)g.n * g.ic * g.ih * g.iw;
+    long vmax = ((long)g.n * (g.ih + 2 * g.ph) + 2L * g.fh * g.dh) * (g.iw + 2 * g.pw);
+    if (P <= 0 || P >= (1L << 31) - BN || src_bytes >= (1L << 31) || vmax >= (1L << 31))
+        return false;
+    TilePlan t = plan_tiles(g);
+    int ks = choose_ks(g.fh * g.fw);
+    if (2L * ks * t.Lmax > (long)MAX_B_ITEMS * THREADS)
+        return false;
+    return true;
+}
+
+size_t conv_mfma_packed_bytes(const ConvGeom& g) {
+    int taps = g.fh * g.fw, ks = choose_ks(taps);
+    int chunks = round_up((g.ic + 31) / 32, ks);
+    return (size_t)chunks * taps * round_up(g.oc, OC_PAD) * KROW;
+}
+
+TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed) {
+    size_t total = conv_mfma_packed_bytes(g);
+    unsigned blocks = (unsigned)((total + 255) / 256);
+    if (blocks > 65536u)
+        blocks = 65536u;
+    hipLaunchKernelGGL(pack_filter_kernel, dim3(blocks), dim3(256), 0, stream(),
+                       (const int8_t*)flt, (int8_t*)packed, total, g.fh * g.fw, g.fw, g.oc,
+                       round_up(g.oc, OC_PAD), g.ic, g.fmt);
+    return check_launch("pack_filter");
+}
+
+TinyNNStatus conv_mfma_launch(
+        const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst) {
+    MfmaParams q;
+    TilePlan t = plan_tiles(g);
+    bool fc = is_fc(g);
+    q.src = (const int8_t*)src;
+    q.wp = (const int8_t*)packed;
+    q.bias = (const int32_t*)bias;
+    q.dst = (int8_t*)dst;
+    q.N = g.n;
+    q.OH = g.oh;
+    q.OW = g.ow;
+    q.OHW = g.oh * g.ow;
+    q.P = g.n * q.OHW;
+    q.OC = g.oc;
+    q.OCP = round_up(g.oc, OC_PAD);
+    q.C4 = g.ic / 4;
+    q.taps = g.fh * g.fw;
+    q.FH = g.fh;
+    q.FW = g.fw;
+    q.KS = choose_ks(q.taps);
+    q.stages = round_up((g.ic + 31) / 32, q.KS) / q.KS;
+    q.VW = t.VW;
+    q.VH = t.VH;
+    q.IH = g.ih;
+    q.IW = g.iw;
+    q.PH = g.ph;
+    q.PW = g.pw;
+    q.SH = g.sh;
+    q.SW = g.sw;
+    q.DH = g.dh;
+    q.DW = g.dw;
+    if (fc) {
+        q.image_stride = g.ic;
+        q.plane_stride = 4;
+        q.row_stride = 0;
+        q.pix_stride = 0;
+    } else {
+        q.image_stride = g.ic * g.ih * g.iw;
+        q.plane_stride = g.ih * g.iw * 4;
+        q.row_stride = g.iw * 4;
+        q.pix_stride = 4;
+    }
+    q.Lmax = t.Lmax;
+    q.dst_fc = fc ? 1 : 0;
+    q.act = g.act;
+    q.s_src = g.s_src;
+    q.s_flt = g.s_flt;
+    q.s_dst = g.s_dst;
+    q.dOW = make_fastdiv(q.OW);
+    q.dOH = make_fastdiv(q.OH);
+    q.dVW = make_fastdiv(q.VW);
+    q.dVH = make_fastdiv(q.VH);
+    q.dL = make_fastdiv(q.Lmax);
+    q.dOHW = make_fastdiv(q.OHW);
+
+    const int bm = g.oc <= 64 ? 64 : 128;
+    const size_t lds = (size_t)q.taps * q.KS * bm * KROW + (size_t)q.KS * q.Lmax * KROW;
+    MG_REQUIRE(lds <= 160 * 1024, TinyNN_ERROR_OUT_OF_RANGE, "conv_mfma: %zu bytes of LDS", lds);
+    dim3 grid((q.P + BN - 1) / BN, (g.oc + bm - 1) / bm);
+    auto kern = bm == 64 ? conv_mfma_i8_kernel<64> : conv_mfma_i8_kernel<128>;
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(
+                (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_mfma: LDS attribute: %s",
+                   hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(THREADS), lds, stream(), q);
+    return check_launch("conv_mfma_i8");
+}
+
+}  // namespace mg

@@ -1,0 +1,126 @@
+// Device seam: the hooks a TinyNN `Device` needs from a GPU (runtime/src/device.c:29-43 fills the
+// same struct for the CPU), the staging copies of the Lite API, the library stream and the
+// per-thread error text.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include <mutex>
+
+#include "common.h"
+
+namespace mg {
+
+static hipStream_t g_stream = nullptr;
+static std::once_flag g_stream_once;
+static thread_local char g_error[512] = "";
+
+hipStream_t stream() {
+    std::call_once(g_stream_once, [] {
+        if (hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking) != hipSuccess)
+            g_stream = nullptr;  // falls back to the null stream; launches still work
+    });
+    return g_stream;
+}
+
+TinyNNStatus fail(TinyNNStatus st, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return st;
+}
+
+TinyNNStatus check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+        return fail(TinyNN_ERROR_RUNTIME, "%s: launch failed: %s", what, hipGetErrorString(e));
+    return TinyNN_SUCCESS;
+}
+
+TinyNNStatus check_io(
+        Tensor** inputs, int nr_input, int want_in_min, int want_in_max, Tensor** outputs,
+        int nr_output, const char* who) {
+    MG_REQUIRE(inputs && outputs, TinyNN_ERROR_NULL_PTR, "%s: NULL tensor list", who);
+    MG_REQUIRE(nr_input >= want_in_min && nr_input <= want_in_max, TinyNN_ERROR_OUT_OF_RANGE,
+               "%s: %d inputs, expected %d..%d", who, nr_input, want_in_min, want_in_max);
+    MG_REQUIRE(nr_output == 1, TinyNN_ERROR_OUT_OF_RANGE, "%s: %d outputs, expected 1", who,
+               nr_output);
+    for (int i = 0; i < nr_input; ++i)
+        MG_REQUIRE(inputs[i] && inputs[i]->ptr, TinyNN_ERROR_NULL_PTR, "%s: input %d is NULL", who, i);
+    MG_REQUIRE(outputs[0] && outputs[0]->ptr, TinyNN_ERROR_NULL_PTR, "%s: output is NULL", who);
+    return TinyNN_SUCCESS;
+}
+
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+void* megcc_gfx950_malloc(size_t length) {
+    void* p = nullptr;
+    if (length == 0)
+        length = 1;
+    if (hipMalloc(&p, length) != hipSuccess) {
+        fail(TinyNN_ERROR_MEMORY_MALLOC, "hipMalloc(%zu) failed", length);
+        return nullptr;
+    }
+    return p;
+}
+
+void megcc_gfx950_free(void* ptr) {
+    if (ptr)
+        (void)hipFree(ptr);
+}
+
+TinyNNStatus megcc_gfx950_init_device(Device* device) {
+    MG_REQUIRE(device, TinyNN_ERROR_NULL_PTR, "init_device: NULL device");
+    int n = 0;
+    MG_REQUIRE(hipGetDeviceCount(&n) == hipSuccess && n > 0, TinyNN_ERROR_RUNTIME,
+               "init_device: no HIP device");
+    device->alignment = 256;
+    device->device_type = TinyNN_GFX950;
+    device->malloc = megcc_gfx950_malloc;
+    device->free = megcc_gfx950_free;
+    return TinyNN_SUCCESS;
+}
+
+TinyNNStatus megcc_gfx950_memcpy_h2d(void* dst, const void* src, size_t length) {
+    MG_REQUIRE(dst && src, TinyNN_ERROR_NULL_PTR, "memcpy_h2d: NULL pointer");
+    hipError_t e = hipMemcpyAsync(dst, src, length, hipMemcpyHostToDevice, stream());
+    // pageable source: the copy is staged before the call returns, so `src` may be reused
+    MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "memcpy_h2d: %s", hipGetErrorString(e));
+    return TinyNN_SUCCESS;
+}
+
+TinyNNStatus megcc_gfx950_memcpy_d2h(void* dst, const void* src, size_t length) {
+    MG_REQUIRE(dst && src, TinyNN_ERROR_NULL_PTR, "memcpy_d2h: NULL pointer");
+    hipError_t e = hipMemcpyAsync(dst, src, length, hipMemcpyDeviceToHost, stream());
+    if (e == hipSuccess)
+        e = hipStreamSynchronize(stream());
+    MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "memcpy_d2h: %s", hipGetErrorString(e));
+    return TinyNN_SUCCESS;
+}
+
+TinyNNStatus megcc_gfx950_memset(void* dst, int value, size_t length) {
+    MG_REQUIRE(dst, TinyNN_ERROR_NULL_PTR, "memset: NULL pointer");
+    hipError_t e = hipMemsetAsync(dst, value, length, stream());
+    MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "memset: %s", hipGetErrorString(e));
+    return TinyNN_SUCCESS;
+}
+
+TinyNNStatus megcc_gfx950_wait(void) {
+    hipError_t e = hipStreamSynchronize(stream());
+    MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "wait: %s", hipGetErrorString(e));
+    return TinyNN_SUCCESS;
+}
+
+void* megcc_gfx950_stream(void) {
+    return (void*)stream();
+}
+
+const char* megcc_gfx950_last_error(void) {
+    return g_error;
+}
+
+}  // extern "C"

@@ -1,0 +1,72 @@
+// Device-side arithmetic shared by every kernel that produces qsi8: the exact float sequence of
+// the reference's generated C, so that outputs are bit-identical.
+//
+//   conv / FullyConnected : fp32_to_int8(act((float)acc * src_scale * flt_scale / dst_scale))
+//                           (BareMetal/Activation.cpp:47-56,105-114; ConvKernel.cpp:374-380)
+//   fp32_to_int8          : int r = roundf(x); clamp to [-128,127]   (half away from zero)
+//
+// Built with -ffp-contract=off: no multiply may fuse with a following add, and the division is the
+// correctly rounded IEEE one (hipcc's default for fp32 `/`); int->float conversion rounds to
+// nearest even exactly like the host's cvtsi2ss.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "megcc_gfx950.h"
+
+namespace mg {
+
+template <int ACT>
+__device__ __forceinline__ float act_apply(float x) {
+    if (ACT == MEGCC_NONLINE_RELU) {
+        return x > 0 ? x : 0;
+    } else if (ACT == MEGCC_NONLINE_H_SWISH) {
+        // res * min(max(res + 3, 0.f), 6.f) * (1.f / 6.f) with the generated min/max helpers
+        float t = x + 3;
+        float mx = t > 0.f ? t : 0.f;
+        float mn = mx > 6.f ? 6.f : mx;
+        return x * mn * (1.f / 6.f);
+    } else if (ACT == MEGCC_NONLINE_SIGMOID) {
+        return 1.f / (expf(-x) + 1.f);
+    }
+    return x;
+}
+
+__device__ __forceinline__ int fp32_to_int8(float v) {
+    int r = (int)roundf(v);
+    r = r > 127 ? 127 : r;
+    r = r < -128 ? -128 : r;
+    return r;
+}
+
+// acc already includes the int32 bias.
+template <int ACT>
+__device__ __forceinline__ int requant_conv(int acc, float s_src, float s_flt, float s_dst) {
+    float v = (float)acc * s_src * s_flt / s_dst;
+    return fp32_to_int8(act_apply<ACT>(v));
+}
+
+// run-time activation selector (a uniform branch) for kernels that are not templated on it
+__device__ __forceinline__ int requant_conv_rt(int act, int acc, float s0, float s1, float s2) {
+    switch (act) {
+        case MEGCC_NONLINE_RELU:
+            return requant_conv<MEGCC_NONLINE_RELU>(acc, s0, s1, s2);
+        case MEGCC_NONLINE_H_SWISH:
+            return requant_conv<MEGCC_NONLINE_H_SWISH>(acc, s0, s1, s2);
+        case MEGCC_NONLINE_SIGMOID:
+            return requant_conv<MEGCC_NONLINE_SIGMOID>(acc, s0, s1, s2);
+        default:
+            return requant_conv<MEGCC_NONLINE_IDENTITY>(acc, s0, s1, s2);
+    }
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) |
+           ((uint32_t)(d & 0xff) << 24);
+}
+
+__device__ __forceinline__ int sbyte(uint32_t w, int i) {
+    return (int)(int8_t)(w >> (8 * i));
+}
+
+}  // namespace mg

@@ -1,0 +1,264 @@
+// f32 GEMM on the matrix cores (v_mfma_f32_32x32x2_f32), shared by
+//   * MatrixMul C = op(A) op(B)   (GeneralIntrinsic/MatMulKernel/Fp32MatMulM4N12.cpp:9-158,
+//                                  Fp32Gevm.cpp:50-119, BareMetal/MatrixMul.cpp:25-120), and
+//   * f32 NCHW dense convolution as an implicit GEMM: rows = oc, columns = output pixels,
+//     K = (ic, fh, fw) (GeneralIntrinsic/ConvKernel/Fp32Im2col.cpp:88-218 does the same product
+//     through an explicit im2col + pack into workspace; here the gather happens while the B tile
+//     is staged into LDS, so there is no workspace), bias + activation fused into the store.
+// Workgroup: 256 threads (2x2 waves), tile 128 x 128 x 16; LDS tiles are K-major with the row
+// padded by 4 floats so both the staging writes and the MFMA operand reads are bank-conflict free.
+// fp32 sums are formed in a different order from the reference's 4x12 micro-kernel; results are
+// held to 1e-4 relative, not bit-exactness.
+#include "common.h"
+#include "conv_geom.h"
+#include "epilogue.cuh"
+
+namespace mg {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+static constexpr int GBM = 128, GBN = 128, GBK = 16, GPAD = 4;
+
+struct GemmArgs {
+    const float* A;
+    const float* B;
+    float* C;
+    const float* bias;
+    int M, N, K;
+    long a_rs, a_cs;  // element strides of A(m,k)
+    long b_rs, b_cs;  // element strides of B(k,n)  (matmul only)
+    long ldc;
+    int act;
+    ConvGeom g;  // convolution only
+    int is_conv;
+};
+
+__device__ __forceinline__ float act_rt(int act, float x) {
+    switch (act) {
+        case MEGCC_NONLINE_RELU: return act_apply<MEGCC_NONLINE_RELU>(x);
+        case MEGCC_NONLINE_H_SWISH: return act_apply<MEGCC_NONLINE_H_SWISH>(x);
+        case MEGCC_NONLINE_SIGMOID: return act_apply<MEGCC_NONLINE_SIGMOID>(x);
+        default: return x;
+    }
+}
+
+// B(k, p) of the implicit GEMM: source pixel of output pixel p under filter tap k
+__device__ __forceinline__ float conv_b(const GemmArgs& q, int k, int p) {
+    const ConvGeom& g = q.g;
+    int taps = g.fh * g.fw;
+    int ic = k / taps, t = k - ic * taps;
+    int fh = t / g.fw, fw = t - fh * g.fw;
+    int ohw = g.oh * g.ow;
+    int n = p / ohw, r = p - n * ohw;
+    int oh = r / g.ow, ow = r - oh * g.ow;
+    unsigned ih = (unsigned)(oh * g.sh + fh * g.dh - g.ph);
+    unsigned iw = (unsigned)(ow * g.sw + fw * g.dw - g.pw);
+    if (ih >= (unsigned)g.ih || iw >= (unsigned)g.iw)
+        return 0.f;
+    return q.B[(((size_t)n * g.ic + ic) * g.ih + ih) * g.iw + iw];
+}
+
+// A_KFAST: A(m,k) has k contiguous (row-major, not transposed) -> lanes walk k when staging.
+// B_NFAST: B(k,n) has n contiguous -> lanes walk n.
+template <bool A_KFAST, bool B_NFAST, bool CONV>
+__global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
+    __shared__ float As[GBK][GBM + GPAD];
+    __shared__ float Bs[GBK][GBN + GPAD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * GBM, n0 = blockIdx.x * GBN;
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                acc[i][j][e] = 0.f;
+
+    for (int k0 = 0; k0 < q.K; k0 += GBK) {
+        // ---- stage A tile (GBM x GBK) and B tile (GBK x GBN): 8 elements per thread each
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            int m, k;
+            if (A_KFAST) {
+                k = tid & 15;
+                m = (tid >> 4) + it * 16;
+            } else {
+                m = tid & 127;
+                k = (tid >> 7) + it * 2;
+            }
+            float v = 0.f;
+            if (m0 + m < q.M && k0 + k < q.K)
+                v = q.A[(size_t)(m0 + m) * q.a_rs + (size_t)(k0 + k) * q.a_cs];
+            As[k][m] = v;
+        }
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            int n, k;
+            if (B_NFAST) {
+                n = tid & 127;
+                k = (tid >> 7) + it * 2;
+            } else {
+                k = tid & 15;
+                n = (tid >> 4) + it * 16;
+            }
+            float v = 0.f;
+            if (n0 + n < q.N && k0 + k < q.K) {
+                if (CONV)
+                    v = conv_b(q, k0 + k, n0 + n);
+                else
+                    v = q.B[(size_t)(k0 + k) * q.b_rs + (size_t)(n0 + n) * q.b_cs];
+            }
+            Bs[k][n] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < GBK; kk += 2) {
+            const int k = kk + (lane >> 5);
+            float a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                a[i] = As[k][wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                b[j] = Bs[k][wn * 64 + j * 32 + (lane & 31)];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // register e of a tile: row 8*(e/4) + 4*(lane/32) + e%4, column lane%32
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+        if (n >= q.N)
+            continue;
+        size_t col_off;
+        int img = 0, rem = 0;
+        if (CONV) {
+            int ohw = q.g.oh * q.g.ow;
+            img = n / ohw;
+            rem = n - img * ohw;
+            col_off = 0;
+        } else {
+            col_off = n;
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                if (m >= q.M)
+                    continue;
+                float v = acc[i][j][e];
+                if (CONV) {
+                    if (q.bias)
+                        v += q.bias[m];
+                    v = act_rt(q.act, v);
+                    q.C[((size_t)img * q.M + m) * (q.g.oh * q.g.ow) + rem] = v;
+                } else {
+                    q.C[(size_t)m * q.ldc + col_off] = v;
+                }
+            }
+    }
+}
+
+bool conv_f32_gemm_supported(const ConvGeom& g) {
+    long P = (long)g.n * g.oh * g.ow;
+    return g.fmt == MEGCC_FMT_NCHW && g.groups == 1 && P < (1L << 31) &&
+           (long)g.ic * g.fh * g.fw < (1L << 31);
+}
+
+TinyNNStatus conv_f32_gemm_launch(
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, void* dst) {
+    GemmArgs q;
+    q.A = (const float*)flt;  // [OC][IC*FH*FW]
+    q.B = (const float*)src;
+    q.C = (float*)dst;
+    q.bias = (const float*)bias;
+    q.M = g.oc;
+    q.N = g.n * g.oh * g.ow;
+    q.K = g.ic * g.fh * g.fw;
+    q.a_rs = q.K;
+    q.a_cs = 1;
+    q.b_rs = q.b_cs = 0;
+    q.ldc = 0;
+    q.act = g.act;
+    q.g = g;
+    q.is_conv = 1;
+    if (q.M == 0 || q.N == 0)
+        return TinyNN_SUCCESS;
+    dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM);
+    hipLaunchKernelGGL((gemm_f32_kernel<true, true, true>), grid, dim3(256), 0, stream(), q);
+    return check_launch("conv_f32_gemm");
+}
+
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" TinyNNStatus megcc_gfx950_matmul(
+        const MegccMatMulAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs,
+        int nr_output, const Workspace*, const RuntimeOpt*) {
+    MG_REQUIRE(attr, TinyNN_ERROR_NULL_PTR, "matmul: NULL attr");
+    TinyNNStatus st = check_io(inputs, nr_input, 2, 2, outputs, nr_output, "matmul");
+    if (st != TinyNN_SUCCESS)
+        return st;
+    const Tensor *a = inputs[0], *b = inputs[1], *c = outputs[0];
+    // the reference has no quantized MatrixMul for row-major operands on this arch
+    // (BareMetal/MatrixMul.cpp:13-23 is f32/f16 only); a qsi8 FullyConnected is a 1x1 conv
+    MG_REQUIRE(is_f32(a) && is_f32(b) && is_f32(c), TinyNN_ERROR_UNSUPPORTED_DTYPE_TYPE,
+               "matmul: only f32 is implemented (quantized FullyConnected goes through conv2d)");
+    MG_REQUIRE(a->layout.nr_dim == 2 && b->layout.nr_dim == 2 && c->layout.nr_dim == 2,
+               TinyNN_ERROR_INVALID_LAYOUT, "matmul: expects 2-d tensors");
+    MG_REQUIRE(a->layout.stride[1] == 1 && b->layout.stride[1] == 1 && c->layout.stride[1] == 1,
+               TinyNN_ERROR_INVALID_LAYOUT, "matmul: innermost stride must be 1");
+    GemmArgs q;
+    const int ta = attr->transpose_a != 0, tb = attr->transpose_b != 0;
+    q.M = c->layout.dims[0];
+    q.N = c->layout.dims[1];
+    q.K = ta ? a->layout.dims[0] : a->layout.dims[1];
+    MG_REQUIRE((int)(ta ? a->layout.dims[1] : a->layout.dims[0]) == q.M &&
+                       (int)(tb ? b->layout.dims[1] : b->layout.dims[0]) == q.K &&
+                       (int)(tb ? b->layout.dims[0] : b->layout.dims[1]) == q.N,
+               TinyNN_ERROR_INVALID_LAYOUT, "matmul: shapes do not agree");
+    const long lda = a->layout.stride[0], ldb = b->layout.stride[0];
+    q.A = (const float*)a->ptr;
+    q.B = (const float*)b->ptr;
+    q.C = (float*)c->ptr;
+    q.bias = nullptr;
+    q.a_rs = ta ? 1 : lda;
+    q.a_cs = ta ? lda : 1;
+    q.b_rs = tb ? 1 : ldb;
+    q.b_cs = tb ? ldb : 1;
+    q.ldc = c->layout.stride[0];
+    q.act = 0;
+    q.is_conv = 0;
+    if (q.M == 0 || q.N == 0)
+        return TinyNN_SUCCESS;
+    dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM);
+    if (!ta && !tb)
+        hipLaunchKernelGGL((gemm_f32_kernel<true, true, false>), grid, dim3(256), 0, stream(), q);
+    else if (!ta && tb)
+        hipLaunchKernelGGL((gemm_f32_kernel<true, false, false>), grid, dim3(256), 0, stream(), q);
+    else if (ta && !tb)
+        hipLaunchKernelGGL((gemm_f32_kernel<false, true, false>), grid, dim3(256), 0, stream(), q);
+    else
+        hipLaunchKernelGGL((gemm_f32_kernel<false, false, false>), grid, dim3(256), 0, stream(), q);
+    return check_launch("matmul");
+}
+
+// No scratch: tiles are staged straight from the operands (the reference packs A and B into
+// workspace, GeneralIntrinsic/MatMulKernel/Fp32MatMulM4N12.cpp:47-66).
+extern "C" TinyNNStatus megcc_gfx950_matmul_workspace(
+        const MegccMatMulAttr*, Tensor**, int, int, size_t* workspace) {
+    MG_REQUIRE(workspace, TinyNN_ERROR_NULL_PTR, "matmul_workspace: NULL size");
+    *workspace = 0;
+    return TinyNN_SUCCESS;
+}

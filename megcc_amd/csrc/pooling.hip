@@ -1,0 +1,161 @@
+// qsi8 pooling, bandwidth-bound, no MFMA.
+//   NCHW   : BareMetal::PoolingKernel (BareMetal/Pooling.cpp:84-148,219-245): MAX of the in-bounds
+//            taps starting from -128; AVERAGE roundf((float)sum / (wh*ww)); COUNT_EXCLUDE_PADDING
+//            roundf((float)sum / count); stored without clamp.
+//   NCHW44 : GeneralIntrinsic::PoolingNchw44QInt8 (GeneralIntrinsic/PoolingKernel/
+//            QInt8PoolingNCHW44.cpp:34-113): AVERAGE is saturate(round((float)sum * count_div)) with
+//            `float count_div = 1.0 / window_count` (a double quotient rounded to float).
+// NCHW44: one thread per output dword (4 channels of a pixel), lanes walk W -> coalesced dwords.
+// NCHW  : one thread per output byte, lanes walk W.
+#include "common.h"
+#include "epilogue.cuh"
+
+namespace mg {
+
+struct PoolGeom {
+    int n, c, ih, iw, oh, ow;
+    int wh, ww, sh, sw, ph, pw;
+    int mode;
+    float count_div;  // 1.0 / (wh*ww) rounded to float, for NCHW44 AVERAGE
+};
+
+__global__ void __launch_bounds__(256) pool44_q8_kernel(
+        PoolGeom g, const uint32_t* __restrict__ src, uint32_t* __restrict__ dst) {
+    const int c4n = g.c >> 2;
+    const size_t total = (size_t)g.n * c4n * g.oh * g.ow;
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        size_t r = i;
+        int ow = r % g.ow; r /= g.ow;
+        int oh = r % g.oh; r /= g.oh;
+        const uint32_t* plane = src + r * g.ih * g.iw;
+        int mx[4] = {-128, -128, -128, -128};
+        int sum[4] = {0, 0, 0, 0};
+        int count = 0;
+        for (int fh = 0; fh < g.wh; ++fh) {
+            unsigned ih = (unsigned)(oh * g.sh + fh - g.ph);
+            if (ih >= (unsigned)g.ih)
+                continue;
+            for (int fw = 0; fw < g.ww; ++fw) {
+                unsigned iw = (unsigned)(ow * g.sw + fw - g.pw);
+                if (iw >= (unsigned)g.iw)
+                    continue;
+                uint32_t v = plane[ih * g.iw + iw];
+                ++count;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    int b = sbyte(v, c);
+                    mx[c] = max(mx[c], b);
+                    sum[c] += b;
+                }
+            }
+        }
+        int o[4];
+        if (g.mode == MEGCC_POOL_MAX) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                o[c] = mx[c];
+        } else {
+            float div = g.mode == MEGCC_POOL_AVERAGE ? g.count_div : (float)(1.0 / (double)(uint32_t)count);
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                o[c] = fp32_to_int8((float)sum[c] * div);
+        }
+        dst[i] = pack4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+__global__ void __launch_bounds__(256) pool_nchw_q8_kernel(
+        PoolGeom g, const int8_t* __restrict__ src, int8_t* __restrict__ dst) {
+    const size_t total = (size_t)g.n * g.c * g.oh * g.ow;
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        size_t r = i;
+        int ow = r % g.ow; r /= g.ow;
+        int oh = r % g.oh; r /= g.oh;
+        const int8_t* plane = src + r * g.ih * g.iw;
+        int mx = -128, sum = 0, count = 0;
+        for (int fh = 0; fh < g.wh; ++fh) {
+            unsigned ih = (unsigned)(oh * g.sh + fh - g.ph);
+            if (ih >= (unsigned)g.ih)
+                continue;
+            for (int fw = 0; fw < g.ww; ++fw) {
+                unsigned iw = (unsigned)(ow * g.sw + fw - g.pw);
+                if (iw >= (unsigned)g.iw)
+                    continue;
+                int b = plane[ih * g.iw + iw];
+                mx = max(mx, b);
+                sum += b;
+                ++count;
+            }
+        }
+        int o;
+        if (g.mode == MEGCC_POOL_MAX)
+            o = mx;
+        else if (g.mode == MEGCC_POOL_AVERAGE)
+            o = (int)roundf((float)sum / (float)(g.wh * g.ww));
+        else
+            o = (int)roundf((float)sum / (float)count);
+        dst[i] = (int8_t)o;
+    }
+}
+
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" TinyNNStatus megcc_gfx950_pooling(
+        const MegccPoolAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace*, const RuntimeOpt*) {
+    MG_REQUIRE(attr, TinyNN_ERROR_NULL_PTR, "pooling: NULL attr");
+    TinyNNStatus st = check_io(inputs, nr_input, 1, 1, outputs, nr_output, "pooling");
+    if (st != TinyNN_SUCCESS)
+        return st;
+    const Tensor* src = inputs[0];
+    const Tensor* dst = outputs[0];
+    MG_REQUIRE(is_q8(src) && is_q8(dst), TinyNN_ERROR_UNSUPPORTED_DTYPE_TYPE,
+               "pooling: only qsi8 -> qsi8 is implemented");
+    // "quant pooling only support same scale" (BareMetal/Pooling.cpp:22-27)
+    MG_REQUIRE(src->dtype.param.scale == dst->dtype.param.scale, TinyNN_ERROR_UNSUPPORTED_DTYPE_TYPE,
+               "pooling: source and destination scales differ");
+    const bool f44 = attr->format == MEGCC_FMT_NCHW44;
+    MG_REQUIRE(f44 || attr->format == MEGCC_FMT_NCHW, TinyNN_ERROR_NO_IMPLEMENT,
+               "pooling: format %d", (int)attr->format);
+    const int want_dim = f44 ? 5 : 4;
+    MG_REQUIRE(src->layout.nr_dim == want_dim && dst->layout.nr_dim == want_dim &&
+                       is_contiguous(src->layout) && is_contiguous(dst->layout),
+               TinyNN_ERROR_INVALID_LAYOUT, "pooling: expects contiguous %d-d tensors", want_dim);
+    PoolGeom g;
+    g.n = src->layout.dims[0];
+    g.c = src->layout.dims[1] * (f44 ? 4 : 1);
+    g.ih = src->layout.dims[2];
+    g.iw = src->layout.dims[3];
+    g.oh = dst->layout.dims[2];
+    g.ow = dst->layout.dims[3];
+    g.wh = attr->window_h; g.ww = attr->window_w;
+    g.sh = attr->stride_h; g.sw = attr->stride_w;
+    g.ph = attr->pad_h; g.pw = attr->pad_w;
+    g.mode = attr->mode;
+    MG_REQUIRE(g.wh > 0 && g.ww > 0 && g.sh > 0 && g.sw > 0, TinyNN_ERROR_OUT_OF_RANGE,
+               "pooling: empty window or stride");
+    MG_REQUIRE(dst->layout.dims[0] == (uint32_t)g.n && dst->layout.dims[1] == src->layout.dims[1] &&
+                       g.oh == (g.ih + 2 * g.ph - g.wh) / g.sh + 1 &&
+                       g.ow == (g.iw + 2 * g.pw - g.ww) / g.sw + 1,
+               TinyNN_ERROR_INVALID_LAYOUT, "pooling: destination shape does not match");
+    g.count_div = (float)(1.0 / (double)(uint32_t)(g.wh * g.ww));
+    size_t total = (size_t)g.n * g.c * g.oh * g.ow;
+    if (total == 0)
+        return TinyNN_SUCCESS;
+    if (f44) {
+        MG_REQUIRE(((uintptr_t)src->ptr & 3) == 0 && ((uintptr_t)dst->ptr & 3) == 0,
+                   TinyNN_ERROR_INVALID_LAYOUT, "pooling: NCHW44 tensors must be 4-byte aligned");
+        unsigned blocks = min(ceil_div(total / 4, 256), 1u << 20);
+        hipLaunchKernelGGL(pool44_q8_kernel, dim3(blocks), dim3(256), 0, stream(), g,
+                           (const uint32_t*)src->ptr, (uint32_t*)dst->ptr);
+    } else {
+        unsigned blocks = min(ceil_div(total, 256), 1u << 20);
+        hipLaunchKernelGGL(pool_nchw_q8_kernel, dim3(blocks), dim3(256), 0, stream(), g,
+                           (const int8_t*)src->ptr, (int8_t*)dst->ptr);
+    }
+    return check_launch("pooling");
+}

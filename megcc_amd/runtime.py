@@ -1,0 +1,191 @@
+"""ctypes front-end of libmegcc_gfx950.so: prototypes, device buffers, and a helper that runs one
+operator through the uniform kernel ABI (workspace -> three-phase init -> kernel), the calling
+sequence of the TinyNN runtime (runtime/src/init.c:29-131, runtime/src/vm/op.c:67-172)."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import LIB_PATH, abi
+
+_lib = None
+
+
+class MegccError(RuntimeError):
+    pass
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise MegccError(
+                "%s is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(there is no CPU fallback)" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        kern = abi.KERNEL_ARGS
+        L.megcc_gfx950_conv2d.argtypes = [C.POINTER(abi.ConvAttr)] + kern
+        L.megcc_gfx950_conv2d_init.argtypes = [C.POINTER(abi.ConvAttr)] + abi.INIT_ARGS
+        L.megcc_gfx950_conv2d_workspace.argtypes = [C.POINTER(abi.ConvAttr)] + abi.WORKSPACE_ARGS
+        L.megcc_gfx950_matmul.argtypes = [C.POINTER(abi.MatMulAttr)] + kern
+        L.megcc_gfx950_matmul_workspace.argtypes = [C.POINTER(abi.MatMulAttr)] + abi.WORKSPACE_ARGS
+        L.megcc_gfx950_pooling.argtypes = [C.POINTER(abi.PoolAttr)] + kern
+        L.megcc_gfx950_elemwise_multitype.argtypes = [C.POINTER(C.c_int)] + kern
+        L.megcc_gfx950_elemwise.argtypes = [C.POINTER(C.c_int)] + kern
+        L.megcc_gfx950_typecvt.argtypes = kern
+        L.megcc_gfx950_reduce.argtypes = [C.POINTER(abi.ReduceAttr)] + kern
+        L.megcc_gfx950_parse_symbol.argtypes = [C.c_char_p, C.POINTER(abi.KernelDesc)]
+        L.megcc_gfx950_call.argtypes = [C.POINTER(abi.KernelDesc)] + kern
+        L.megcc_gfx950_call_init.argtypes = [C.POINTER(abi.KernelDesc)] + abi.INIT_ARGS
+        L.megcc_gfx950_call_workspace.argtypes = [C.POINTER(abi.KernelDesc)] + abi.WORKSPACE_ARGS
+        L.megcc_gfx950_init_device.argtypes = [C.POINTER(abi.Device)]
+        L.megcc_gfx950_malloc.argtypes = [C.c_size_t]
+        L.megcc_gfx950_malloc.restype = C.c_void_p
+        L.megcc_gfx950_free.argtypes = [C.c_void_p]
+        L.megcc_gfx950_free.restype = None
+        L.megcc_gfx950_memcpy_h2d.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        L.megcc_gfx950_memcpy_d2h.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        L.megcc_gfx950_memset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
+        L.megcc_gfx950_wait.argtypes = []
+        L.megcc_gfx950_stream.argtypes = []
+        L.megcc_gfx950_stream.restype = C.c_void_p
+        L.megcc_gfx950_last_error.argtypes = []
+        L.megcc_gfx950_last_error.restype = C.c_char_p
+        _lib = L
+    return _lib
+
+
+EXPORTS = [
+    "megcc_gfx950_conv2d", "megcc_gfx950_conv2d_init", "megcc_gfx950_conv2d_workspace",
+    "megcc_gfx950_matmul", "megcc_gfx950_matmul_workspace", "megcc_gfx950_pooling",
+    "megcc_gfx950_elemwise_multitype", "megcc_gfx950_elemwise", "megcc_gfx950_typecvt",
+    "megcc_gfx950_reduce", "megcc_gfx950_parse_symbol", "megcc_gfx950_call",
+    "megcc_gfx950_call_init", "megcc_gfx950_call_workspace", "megcc_gfx950_init_device",
+    "megcc_gfx950_malloc", "megcc_gfx950_free", "megcc_gfx950_memcpy_h2d",
+    "megcc_gfx950_memcpy_d2h", "megcc_gfx950_memset", "megcc_gfx950_wait",
+    "megcc_gfx950_stream", "megcc_gfx950_last_error",
+]
+
+
+def check(status, what=""):
+    if status != abi.SUCCESS:
+        raise MegccError("%s: TinyNNStatus %d: %s" % (
+            what, status, lib().megcc_gfx950_last_error().decode()))
+
+
+class DeviceBuffer:
+    """HBM allocation made through the Device.malloc hook of the library."""
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        self.ptr = lib().megcc_gfx950_malloc(max(self.nbytes, 1))
+        if not self.ptr:
+            raise MegccError("device malloc of %d bytes failed" % self.nbytes)
+
+    @classmethod
+    def from_array(cls, arr):
+        arr = np.ascontiguousarray(arr)
+        buf = cls(arr.nbytes)
+        if arr.nbytes:
+            check(lib().megcc_gfx950_memcpy_h2d(buf.ptr, arr.ctypes.data, arr.nbytes), "h2d")
+            check(lib().megcc_gfx950_wait(), "wait")
+        return buf
+
+    def to_array(self, shape, dtype):
+        out = np.empty(shape, dtype)
+        assert out.nbytes <= self.nbytes
+        if out.nbytes:
+            check(lib().megcc_gfx950_memcpy_d2h(out.ctypes.data, self.ptr, out.nbytes), "d2h")
+        return out
+
+    def fill(self, value):
+        check(lib().megcc_gfx950_memset(self.ptr, value, self.nbytes), "memset")
+
+    def free(self):
+        if self.ptr:
+            lib().megcc_gfx950_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def wait():
+    check(lib().megcc_gfx950_wait(), "wait")
+
+
+def parse_symbol(symbol):
+    desc = abi.KernelDesc()
+    check(lib().megcc_gfx950_parse_symbol(symbol.encode(), C.byref(desc)), "parse_symbol " + symbol)
+    return desc
+
+
+class PreparedOp:
+    """One operator instance: device tensors, the processed weight from the init protocol, ready
+    to be launched repeatedly (what one `Opr` instruction of the TinyNN VM holds)."""
+
+    def __init__(self, desc, in_specs, out_specs):
+        L = lib()
+        self.desc = desc
+        self.keep = []
+        self.in_tensors = []
+        for s in in_specs:
+            buf = DeviceBuffer.from_array(s.array)
+            self.keep.append(buf)
+            self.in_tensors.append(abi.make_tensor(buf.ptr, s.shape, s.type_enum, s.scale, s.name))
+        self.out_bufs, self.out_tensors, self.out_specs = [], [], out_specs
+        for s in out_specs:
+            buf = DeviceBuffer(s.nbytes)
+            buf.fill(0x5A)  # poison: an element the kernel fails to write shows up in the compare
+            self.out_bufs.append(buf)
+            self.out_tensors.append(abi.make_tensor(buf.ptr, s.shape, s.type_enum, s.scale, s.name))
+        # workspace
+        size = C.c_size_t(0)
+        ins = abi.tensor_array(self.in_tensors)
+        check(L.megcc_gfx950_call_workspace(C.byref(desc), ins, len(self.in_tensors), 1,
+                                            C.byref(size)), "workspace")
+        self.ws = abi.Workspace()
+        self.ws_buf = DeviceBuffer(size.value) if size.value else None
+        self.ws.ptr = self.ws_buf.ptr if self.ws_buf else None
+        self.ws.size = size.value
+        # three-phase init
+        n_out = C.c_int(0)
+        check(L.megcc_gfx950_call_init(C.byref(desc), ins, len(self.in_tensors), None,
+                                       C.byref(n_out), None), "init(count)")
+        self.n_processed = n_out.value
+        if n_out.value:
+            assert n_out.value == 1
+            w = abi.Tensor()
+            check(L.megcc_gfx950_call_init(C.byref(desc), ins, len(self.in_tensors), C.byref(w),
+                                           None, None), "init(describe)")
+            nbytes = abi.np_dtype(w.dtype.type_enum).itemsize
+            for i in range(w.layout.nr_dim):
+                nbytes *= w.layout.dims[i]
+            wbuf = DeviceBuffer(nbytes)
+            self.keep.append(wbuf)
+            w.ptr = wbuf.ptr
+            check(L.megcc_gfx950_call_init(C.byref(desc), ins, len(self.in_tensors), C.byref(w),
+                                           C.byref(n_out), None), "init(transform)")
+            for i, t in enumerate(self.in_tensors):
+                if t.name == w.name:
+                    self.in_tensors[i] = w
+        self.ins = abi.tensor_array(self.in_tensors)
+        self.outs = abi.tensor_array(self.out_tensors)
+
+    def launch(self):
+        check(lib().megcc_gfx950_call(C.byref(self.desc), self.ins, len(self.in_tensors), self.outs,
+                                      len(self.out_tensors), C.byref(self.ws), None), "kernel")
+
+    def result(self, i=0):
+        s = self.out_specs[i]
+        return self.out_bufs[i].to_array(s.shape, abi.np_dtype(s.type_enum))
+
+
+def run_symbol(symbol, in_specs, out_specs):
+    """Run the operator the reference calls `symbol` once and fetch its (first) output."""
+    op = PreparedOp(parse_symbol(symbol), in_specs, out_specs)
+    op.launch()
+    return op.result()

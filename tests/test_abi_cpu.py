@@ -1,0 +1,99 @@
+"""CPU-only checks of the boundary: the library loads, exports every entry point the header
+declares, and the host-side logic that needs no GPU (symbol parsing, workspace size, argument
+validation) behaves like the reference's."""
+import ctypes as C
+import json
+import os
+import re
+
+import pytest
+
+from megcc_amd import abi, runtime
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "megcc_gfx950.h")).read()
+    return sorted(set(re.findall(r"\b(megcc_gfx950_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = runtime.lib()
+    declared = header_functions()
+    assert len(declared) >= 20
+    for name in declared:
+        assert hasattr(L, name), name
+    assert sorted(runtime.EXPORTS) == declared
+
+
+def test_struct_sizes_match_the_c_abi():
+    # x86-64 layout of runtime/src/data_struct.h: Layout = 4 + 28 + 28 + 4, Tensor = 8 + 12 + 64 + ...
+    assert C.sizeof(abi.Layout) == 64
+    assert C.sizeof(abi.DType) == 12
+    assert C.sizeof(abi.Tensor) == 136
+    assert C.sizeof(abi.Workspace) == 24
+    assert C.sizeof(abi.Device) == 24
+
+
+with open(os.path.join(HERE, "golden", "symbols.json")) as f:
+    SYMBOLS = json.load(f)
+
+
+@pytest.mark.parametrize("symbol", sorted(set(SYMBOLS.values())))
+def test_every_reference_symbol_parses(symbol):
+    desc = runtime.parse_symbol(symbol)
+    assert desc.kind in range(1, 8)
+
+
+def test_parse_conv_symbol_fields():
+    d = runtime.parse_symbol(
+        "kernel_conv2d_3x3_NCHW44_DENSE_p1x1_s2x2_d1x1_qsi8qsi8qsi32qsi8_bias_H_SWISH")
+    a = d.attr.conv
+    assert d.kind == abi.KERN_CONV
+    assert (a.kernel_h, a.kernel_w, a.pad_h, a.pad_w, a.stride_h, a.stride_w) == (3, 3, 1, 1, 2, 2)
+    assert (a.format, a.sparse, a.nonline, a.with_bias) == (abi.FMT_NCHW44, abi.DENSE, abi.H_SWISH, 1)
+    d = runtime.parse_symbol("kernel_conv2d_3x3_NCHW_NCHW44_DENSE_p1x1_s2x2_d1x1_qsi8qsi8qsi32qsi8_bias_RELU")
+    assert d.attr.conv.format == abi.FMT_NCHW_NCHW44 and d.attr.conv.nonline == abi.RELU
+    d = runtime.parse_symbol("GI_kernel_conv2d_im2col_3x3_NCHW_DENSE_p1x1_s1x1_d1x1_bias_RELUf32")
+    assert (d.attr.conv.format, d.attr.conv.with_bias, d.attr.conv.nonline) == (abi.FMT_NCHW, 1, abi.RELU)
+    d = runtime.parse_symbol("GI_kernel_conv2d_im2col_3x3_NCHW_DENSE_p1x1_s1x1_d1x1f32")
+    assert (d.attr.conv.with_bias, d.attr.conv.nonline) == (0, abi.IDENTITY)
+
+
+def test_parse_other_symbols():
+    d = runtime.parse_symbol("kernel_pooling_AVERAGE_COUNT_EXCLUDE_PADDING_NCHW_p1x1_s2x2_w3x3_qsi8qsi8")
+    assert d.kind == abi.KERN_POOLING and d.attr.pool.mode == abi.POOL_AVERAGE_COUNT_EXCLUDE_PADDING
+    assert (d.attr.pool.window_h, d.attr.pool.stride_w, d.attr.pool.pad_h) == (3, 2, 1)
+    d = runtime.parse_symbol("GI_kernel_pooling_MAX_NCHW44_p0x0_s2x2_w2x2_qsi8qsi8_qsi8qsi8_fallback")
+    assert d.attr.pool.format == abi.FMT_NCHW44 and d.attr.pool.mode == abi.POOL_MAX
+    d = runtime.parse_symbol("kernel_elementwise_multitype_QFUSE_ADD_RELU_qsi8qsi8qsi8")
+    assert d.kind == abi.KERN_ELEMWISE_MULTITYPE and d.attr.multitype == abi.Q_FUSE_ADD_RELU
+    d = runtime.parse_symbol("GI_kernel_elementwise_TRUE_DIV_f32_binary_VEC_VEC_f32f32f32")
+    assert d.kind == abi.KERN_ELEMWISE and d.attr.elemwise == abi.EW_TRUE_DIV
+    d = runtime.parse_symbol("GI_kernel_reduce_MAX_DEFAULT_f32_a1")
+    assert d.kind == abi.KERN_REDUCE and (d.attr.reduce.mode, d.attr.reduce.axis) == (abi.REDUCE_MAX, 1)
+    d = runtime.parse_symbol("GI_kernel_gevm_nn")
+    assert d.kind == abi.KERN_MATMUL and d.attr.matmul.transpose_b == 0
+    d = runtime.parse_symbol("GI_kernel_fp32_matmul_4x12_nt")
+    assert d.attr.matmul.transpose_b == 1
+
+
+def test_unknown_symbol_is_reported_not_guessed():
+    desc = abi.KernelDesc()
+    for bad in ("kernel_argsort_f32", "kernel_conv2d_3x3_NHWC_DENSE_p1x1_s1x1_d1x1_f32f32f32",
+                "kernel_typecvt_f16f32", ""):
+        st = runtime.lib().megcc_gfx950_parse_symbol(bad.encode(), C.byref(desc))
+        assert st == abi.ERROR_NO_FOUND
+        assert b"not a kernel" in runtime.lib().megcc_gfx950_last_error()
+
+
+def test_null_arguments_are_rejected():
+    L = runtime.lib()
+    attr = abi.ConvAttr(3, 3, 1, 1, 1, 1, 1, 1, abi.FMT_NCHW44, abi.DENSE, abi.RELU, 1)
+    assert L.megcc_gfx950_conv2d(C.byref(attr), None, 0, None, 0, None, None) == abi.ERROR_NULL_PTR
+    assert L.megcc_gfx950_conv2d(None, None, 0, None, 0, None, None) == abi.ERROR_NULL_PTR
+    size = C.c_size_t(123)
+    assert L.megcc_gfx950_conv2d_workspace(C.byref(attr), None, 0, 1, C.byref(size)) == 0
+    assert size.value == 0

@@ -1,0 +1,156 @@
+"""GPU parity tests: every operator is called through the C ABI (megcc_gfx950_call on the
+reference's own kernel symbol, after the workspace / three-phase-init protocol) and compared with
+  * the committed outputs of the reference's generated C kernels (tests/golden/),
+  * the CPU oracle on larger seeded cases,
+bit-exact for qsi8, max |a-b|/max(1,min(|a|,|b|)) <= 1e-4 for f32."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import cases
+from cases import ConvCase, MatMulCase, MultiTypeCase, PoolCase, TypeCvtCase
+from golden_cases import golden_cases, unsat
+from megcc_amd import abi, runtime
+from oracle import port
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+F32_TOL = 1e-4
+CASES = golden_cases()
+
+
+@pytest.fixture(scope="module")
+def golden():
+    gold = np.load(os.path.join(HERE, "golden", "golden.npz"))
+    with open(os.path.join(HERE, "golden", "symbols.json")) as f:
+        return gold, json.load(f)
+
+
+def compare(got, want, what):
+    assert got.shape == want.shape and got.dtype == want.dtype, what
+    if got.dtype == np.float32:
+        err = cases.max_rel_err(got, want)
+        assert err <= F32_TOL, "%s: max rel err %g" % (what, err)
+    else:
+        bad = np.flatnonzero(got.reshape(-1) != want.reshape(-1))
+        assert bad.size == 0, "%s: %d of %d differ, first at %d: got %d want %d" % (
+            what, bad.size, got.size, bad[0], got.reshape(-1)[bad[0]], want.reshape(-1)[bad[0]])
+
+
+def run_gpu(case, arrays, symbol=None):
+    print("GPU case:", repr(case), flush=True)
+    ins, outs = case.specs(arrays)
+    return runtime.run_symbol(symbol or case.symbol(), ins, outs)
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_matches_reference_golden(name, golden):
+    gold, symbols = golden
+    case = CASES[name]
+    arrays = {k: (gold["%s/%s" % (name, k)] if "%s/%s" % (name, k) in gold.files else None)
+              for k in case.gen(0).keys()}
+    got = run_gpu(case, arrays, symbols[name])
+    compare(got, gold[name + "/expect"], name)
+
+
+A = abi
+LIVE = [
+    # headline kernel at its real channel counts (spatial size cut so the oracle stays fast)
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 64, 56, 56, 64, 3, 1, 1, A.RELU, scales=(0.02, 0.01, 0.05)),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 64, 56, 56, 64, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(576))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 28, 28, 256, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(2304))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 256, 14, 14, 256, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, 0.05)),
+    # ragged: pixel count not a multiple of the 128-pixel tile, oc not a multiple of 64, ic % 32 != 0
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 40, 13, 17, 72, 3, 1, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(360))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 36, 15, 9, 200, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(324))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 5, 24, 7, 7, 32, 3, 1, 1, A.SIGMOID, scales=(0.02, 0.01, unsat(216) * 40)),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 1, 8, 30, 31, 8, 3, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(72))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 1, 16, 20, 20, 16, 3, 1, 2, A.RELU, scales=(0.02, 0.01, unsat(144)), dilate=2),
+    # MobileNet pointwise shapes
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 32, 112, 112, 64, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(32))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 4, 512, 14, 14, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(512))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 1024, 7, 7, 1024, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(1024))),
+    # FullyConnected = 1x1 NCHW conv on [M,K,1,1]
+    ConvCase(A.FMT_NCHW, A.DENSE, 64, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(1024) / 2)),
+    ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, 0.1)),
+    ConvCase(A.FMT_NCHW, A.DENSE, 200, 512, 1, 1, 333, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(512) / 2)),
+    # depthwise, pooling, elemwise chain of the bandwidth-bound config
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 32, 112, 112, 32, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 32, 112, 112, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, 0.05)),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 3, 512, 14, 14, 512, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 3, 512, 14, 14, 512, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW, A.GROUP, 2, 32, 28, 28, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 224, 224, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),
+    PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
+    PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
+    PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE, 5, 1024, 7, 7, 7, 7, 0),
+    PoolCase(A.FMT_NCHW, A.POOL_AVERAGE, 5, 1024, 7, 7, 7, 7, 0),
+    MultiTypeCase(A.Q_FUSE_ADD_RELU, (2, 32, 56, 56), (0.05, 0.01, 0.05)),
+    MultiTypeCase(A.Q_ADD, (3, 7, 13, 5), (0.031, 0.017, 0.023)),
+    MultiTypeCase(A.Q_MUL, (2, 32, 56, 56), (0.05, 0.04, 0.3)),
+    MultiTypeCase(A.Q_RELU, (1, 1, 1, 100003), (0.05, 0.01, 0.03)),
+    TypeCvtCase("f32", "qsi8", (2, 3, 224, 224), dst_scale=0.0173),
+    TypeCvtCase("qsi8", "f32", (64, 1000), src_scale=0.0173),
+    TypeCvtCase("qsi8", "qsi8", (5, 1001), src_scale=0.0173, dst_scale=0.0291),
+    TypeCvtCase("qsi32", "qsi8", (5, 1001), src_scale=0.0002, dst_scale=0.05),
+    # f32
+    ConvCase(A.FMT_NCHW, A.DENSE, 1, 32, 56, 56, 32, 3, 1, 1, A.RELU, dtype="f32"),
+    ConvCase(A.FMT_NCHW, A.DENSE, 2, 5, 19, 23, 37, 3, 2, 1, A.IDENTITY, dtype="f32"),
+    MatMulCase(1, 1024, 1000),
+    MatMulCase(64, 512, 384),
+    MatMulCase(130, 77, 259),
+    MatMulCase(33, 65, 70, trans_a=True),
+    MatMulCase(33, 65, 70, trans_b=True),
+    MatMulCase(33, 65, 70, trans_a=True, trans_b=True),
+]
+
+
+@pytest.mark.parametrize("case", LIVE, ids=[repr(c) for c in LIVE])
+def test_matches_oracle(case):
+    port.set_threads(8)
+    arrays = case.gen(seed=11)
+    want = case.run_port(arrays)
+    got = run_gpu(case, arrays)
+    compare(got, want, repr(case))
+
+
+def test_direct_kernel_when_filter_was_not_packed():
+    """a caller that skips the init protocol still gets the right answer (generic kernel)"""
+    import ctypes as C
+    case = ConvCase(A.FMT_NCHW44, A.DENSE, 2, 16, 9, 11, 24, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(144)))
+    arrays = case.gen(5)
+    ins, outs = case.specs(arrays)
+    bufs = [runtime.DeviceBuffer.from_array(s.array) for s in ins]
+    out = runtime.DeviceBuffer(outs[0].nbytes)
+    tin = [abi.make_tensor(b.ptr, s.shape, s.type_enum, s.scale, s.name) for b, s in zip(bufs, ins)]
+    tout = [abi.make_tensor(out.ptr, outs[0].shape, outs[0].type_enum, outs[0].scale)]
+    attr = case.attr()
+    runtime.check(runtime.lib().megcc_gfx950_conv2d(
+        C.byref(attr), abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1, None, None), "conv2d")
+    compare(out.to_array(outs[0].shape, np.int8), case.run_port(arrays), "direct")
+
+
+def test_errors_do_not_launch():
+    import ctypes as C
+    case = ConvCase(A.FMT_NCHW44, A.DENSE, 1, 8, 6, 6, 8, 3, 1, 1, A.RELU)
+    arrays = case.gen(5)
+    ins, outs = case.specs(arrays)
+    bufs = [runtime.DeviceBuffer.from_array(s.array) for s in ins]
+    out = runtime.DeviceBuffer(outs[0].nbytes)
+    tin = [abi.make_tensor(b.ptr, s.shape, s.type_enum, s.scale, s.name) for b, s in zip(bufs, ins)]
+    bad_shape = list(outs[0].shape)
+    bad_shape[2] += 1
+    tout = [abi.make_tensor(out.ptr, bad_shape, outs[0].type_enum, outs[0].scale)]
+    attr = case.attr()
+    st = runtime.lib().megcc_gfx950_conv2d(
+        C.byref(attr), abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1, None, None)
+    assert st == abi.ERROR_INVALID_LAYOUT
+    # bias scale must equal src*flt scale (ConvGeneral::IsAvailable)
+    tin[2].dtype.param.scale = 0.5
+    tout = [abi.make_tensor(out.ptr, outs[0].shape, outs[0].type_enum, outs[0].scale)]
+    st = runtime.lib().megcc_gfx950_conv2d(
+        C.byref(attr), abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1, None, None)
+    assert st == abi.ERROR_UNSUPPORTED_DTYPE_TYPE

@@ -1,0 +1,204 @@
+#!/usr/bin/env python3
+"""bench.py -- one JSON line for the headline metric of the generated-kernel hot path.
+
+Default workload: the qsi8 3x3 stride-1 pad-1 NCHW44 convolution of BASELINE.json configs[1] at
+its largest single-GPU shape (N=32, Cin=Cout=256, 56x56, int32 bias, fused ReLU, scales
+0.02/0.01 -> 0.05), called through the C ABI exactly as the TinyNN VM would: init protocol once,
+then one kernel call per step with all operands resident in HBM.
+
+  value      whole-job int8 throughput, ops = 2*N*OC*OH*OW*IC*FH*FW  (the reference's own workload
+             formula, compiler/test/kernel/common/src/workload_proxy.cpp:69), wall clock around
+             the K timed steps with a stream sync on both sides
+  roofline   the same ops over the average kernel duration measured with HIP events on the
+             library's stream, against the 5.0 POP/s dense int8 MFMA peak of MI355X
+  cpu_baseline  the reference's own generated C kernel (oracle/_ref, kind "reference") or our C
+             restatement (kind "port") on ONE host core, on a bounded slice of the same layer
+
+Other workloads (--workload dw|fc|chain ...) are for development; the driver uses the default.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_INT8_TOPS = 5000.0  # dense int8 MFMA, MI355X
+PEAK_HBM_GBS = 8000.0
+
+
+class HipEvents:
+    def __init__(self, stream):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.stream = C.c_void_p(stream)
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+
+    def new(self):
+        e = C.c_void_p()
+        assert self.hip.hipEventCreate(C.byref(e)) == 0
+        return e
+
+    def record(self, e):
+        assert self.hip.hipEventRecord(e, self.stream) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.hip.hipEventSynchronize(b) == 0
+        ms = C.c_float()
+        assert self.hip.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return ms.value
+
+
+def headline_case(n=32, c=256, hw=56):
+    from cases import ConvCase
+    from megcc_amd import abi
+    return ConvCase(abi.FMT_NCHW44, abi.DENSE, n, c, hw, hw, c, 3, 1, 1, abi.RELU,
+                    scales=(0.02, 0.01, 0.05))
+
+
+def make_workload(name):
+    """-> (case, description, bound, algorithmic units per launch)"""
+    from cases import ConvCase, MultiTypeCase, PoolCase
+    from megcc_amd import abi
+    if name == "conv":
+        case = headline_case()
+        return case, "qsi8 conv3x3 s1 p1 NCHW44 N=32 Cin=Cout=256 56x56 +bias +ReLU requant", "mfma"
+    if name == "conv_c64":
+        return headline_case(32, 64, 56), "qsi8 conv3x3 NCHW44 N=32 C=64 56x56", "mfma"
+    if name == "conv_c256_28":
+        return headline_case(32, 256, 28), "qsi8 conv3x3 NCHW44 N=32 C=256 28x28", "mfma"
+    if name == "conv_n1":
+        return headline_case(1, 64, 56), "qsi8 conv3x3 NCHW44 N=1 C=64 56x56", "mfma"
+    if name == "pw":
+        case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 64, 512, 14, 14, 512, 1, 1, 0, abi.RELU,
+                        scales=(0.02, 0.01, 0.05))
+        return case, "qsi8 conv1x1 NCHW44 N=64 C=512 14x14", "mfma"
+    if name == "fc":
+        case = ConvCase(abi.FMT_NCHW, abi.DENSE, 4096, 4096, 1, 1, 4096, 1, 1, 0, abi.IDENTITY,
+                        scales=(0.01, 0.01, 0.1))
+        return case, "qsi8 FullyConnected 4096x4096x4096", "mfma"
+    if name == "fc64":
+        case = ConvCase(abi.FMT_NCHW, abi.DENSE, 64, 4096, 1, 1, 4096, 1, 1, 0, abi.IDENTITY,
+                        scales=(0.01, 0.01, 0.1))
+        return case, "qsi8 FullyConnected 64x4096x4096", "hbm"
+    if name.startswith("dw"):
+        c, hw, s = {"dw": (32, 112, 1), "dw_s2": (32, 112, 2), "dw512": (512, 14, 1),
+                    "dw512_s2": (512, 14, 2)}[name]
+        case = ConvCase(abi.FMT_NCHW44, abi.GROUP, 64, c, hw, hw, c, 3, s, 1, abi.RELU,
+                        scales=(0.02, 0.01, 0.05))
+        return case, "qsi8 depthwise 3x3 s%d NCHW44 N=64 C=%d %dx%d" % (s, c, hw, hw), "hbm"
+    if name == "pool":
+        return (PoolCase(abi.FMT_NCHW44, abi.POOL_MAX, 64, 32, 112, 112, 2, 2, 0),
+                "qsi8 maxpool 2x2 s2 NCHW44 N=64 C=32 112x112", "hbm")
+    if name == "add":
+        return (MultiTypeCase(abi.Q_FUSE_ADD_RELU, (64, 32, 56, 56), (0.05, 0.01, 0.05)),
+                "qsi8 QFUSE_ADD_RELU 64x32x56x56", "hbm")
+    raise SystemExit("unknown workload " + name)
+
+
+def case_bytes(case):
+    ins, outs = case.specs(case.gen(0))
+    return sum(s.nbytes for s in ins) + sum(s.nbytes for s in outs)
+
+
+def cpu_baseline(full_case, budget_s=20.0):
+    """One host core on a bounded slice of the same layer: batch 1 (of 32) of the headline conv."""
+    from oracle import port, ref
+    import cases
+    from cases import ConvCase
+    if not isinstance(full_case, ConvCase) or full_case.sparse != 0 or full_case.fh != 3:
+        return None
+    sample = headline_case(1, full_case.ic, full_case.ih)
+    arrays = sample.gen(seed=0)
+    use_ref = ref.available() and ref.has(sample.symbol())
+    port.set_threads(1)
+    t0 = time.perf_counter()
+    if use_ref:
+        cases.run_ref(sample, arrays)
+    else:
+        sample.run_port(arrays)
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(sample.ops() / dt / 1e12, 6), "unit": "TOP/s", "cores": 1,
+        "kind": "reference" if use_ref else "port",
+        "sample": "batch 1 of 32 of the same layer (N=1 Cin=Cout=%d %dx%d, %.2f GOP) timed once "
+                  "in %.2f s; %s" % (
+                      sample.ic, sample.ih, sample.iw, sample.ops() / 1e9, dt,
+                      "MegCC's generated kernel %s built with -O3 -fno-finite-math-only" %
+                      sample.symbol() if use_ref else "oracle/oracle_port.c built with -O2"),
+        "host_cores": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="conv")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU (the path shards over the batch "
+                         "dimension with no exchange step); --gpus %d is not supported" % args.gpus)
+
+    from megcc_amd import runtime
+    import numpy as np
+
+    case, desc, bound = make_workload(args.workload)
+    arrays = case.gen(seed=0)
+    ins, outs = case.specs(arrays)
+    op = runtime.PreparedOp(runtime.parse_symbol(case.symbol()), ins, outs)
+    ev = HipEvents(runtime.lib().megcc_gfx950_stream())
+
+    for _ in range(args.warmup):
+        op.launch()
+    runtime.wait()
+    e0, e1 = ev.new(), ev.new()
+    t0 = time.perf_counter()
+    ev.record(e0)
+    for _ in range(args.steps):
+        op.launch()
+    ev.record(e1)
+    runtime.wait()
+    wall = time.perf_counter() - t0
+    kern_ms = ev.elapsed_ms(e0, e1) / args.steps
+
+    # spot check of the timed output against the oracle on one image (full check is in tests/)
+    ops = case.ops() if hasattr(case, "ops") else 0
+    nbytes = case_bytes(case)
+    ms = wall * 1e3 / args.steps
+    if bound == "mfma":
+        value, unit, metric = ops / (wall / args.steps) / 1e12, "TOP/s", "int8_conv_tops"
+        roof = {"bound": "mfma", "achieved": round(ops / (kern_ms * 1e-3) / 1e12, 3),
+                "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "traffic": None}
+    else:
+        value, unit, metric = nbytes / (wall / args.steps) / 1e9, "GB/s", "hbm_gbps"
+        roof = {"bound": "hbm", "achieved": round(nbytes / (kern_ms * 1e-3) / 1e9, 2),
+                "peak": PEAK_HBM_GBS, "unit": "GB/s", "traffic": None}
+    roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
+    roof["kernel_ms"] = round(kern_ms, 5)
+    roof["algorithmic_per_launch"] = ops if bound == "mfma" else nbytes
+
+    out = {
+        "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8" if bound == "mfma" or True else "u8", "data": "synthetic",
+        "config": {"workload": desc, "symbol": case.symbol(), "abi": "megcc_gfx950_call"},
+        "roofline": roof,
+    }
+    if not args.no_cpu and args.workload == "conv":
+        out["cpu_baseline"] = cpu_baseline(case)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

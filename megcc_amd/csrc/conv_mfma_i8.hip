@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(THREADS) conv_mfma_i8_kernel(MfmaParams q) {
     constexpr int MT = WM / 32;         // 32x32 tiles per wave along oc
     constexpr int NT = 2;               // 64 pixels per wave
     constexpr int A_ROW_CHUNKS = BM * 2;  // 16-byte chunks per tap
-    constexpr int MAX_A_ITEMS = MAX_TAPS_STAGE * A_ROW_CHUNKS / THREADS;
+    constexpr int MAX_A_ITEMS = (MAX_TAPS_STAGE * A_ROW_CHUNKS + THREADS - 1) / THREADS;
 
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];
     const int taps_stage = q.taps * q.KS;

@@ -19,71 +19,17 @@
 //     bank once;
 //   * the MFMA result layout (lane = pixel, 4 consecutive registers = 4 consecutive oc) is exactly
 //     one NCHW44 dword per pixel, so 32 lanes store 128 contiguous bytes.
-#include "common.h"
-#include "conv_geom.h"
-#include "epilogue.cuh"
+#include <stdlib.h>
+
+#include "conv_mfma_i8.h"
 
 namespace mg {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
+static constexpr int ACT_RUNTIME = -1;
 
-static constexpr int BN = 128;       // pixels per workgroup
-static constexpr int THREADS = 256;  // 4 waves
-static constexpr int KROW = 32;      // input channels per LDS row = K of one MFMA
-static constexpr int MAX_TAPS_STAGE = 9;
-static constexpr int MAX_B_ITEMS = 8;  // 16-byte gather items per thread per stage
-static constexpr int OC_PAD = 128;
-
-// unsigned division by a run-time constant: q = (x * mul) >> (32 + shift), exact for x < 2^31
-struct FastDiv {
-    uint32_t mul, shift, d;
-};
-static FastDiv make_fastdiv(uint32_t d) {
-    FastDiv f;
-    f.d = d;
-    if (d == 1) {
-        f.mul = 0;
-        f.shift = 0;
-        return f;
-    }
-    uint32_t s = 0;
-    while ((1u << s) < d)
-        ++s;  // ceil(log2 d)
-    uint64_t m = ((uint64_t(1) << (32 + s - 1)) + d - 1) / d;  // fits 32 bits for x < 2^31
-    f.mul = (uint32_t)m;
-    f.shift = s - 1;
-    return f;
-}
-__device__ __forceinline__ uint32_t fdiv(uint32_t x, const FastDiv& f) {
-    return f.d == 1 ? x : (__umulhi(x, f.mul) >> f.shift);
-}
-
-struct MfmaParams {
-    const int8_t* src;
-    const int8_t* wp;
-    const int32_t* bias;
-    int8_t* dst;
-    int P, OH, OW, OHW, N;
-    int OC, OCP, C4;
-    int stages, KS, taps, FH, FW;
-    int VW, VH, IH, IW, PH, PW, SH, SW, DH, DW;
-    int image_stride, plane_stride, row_stride, pix_stride;  // bytes
-    int Lmax;    // LDS patch slots (multiple of 64)
-    int dst_fc;  // 0: NCHW44, 1: [P][OC] row-major
-    int act;
-    float s_src, s_flt, s_dst;
-    FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
-};
-
-// virtual pixel index of output pixel p at tap (0,0): rows of the zero-padded images stacked
-__device__ __forceinline__ int vp_of(const MfmaParams& q, int p) {
-    int g = fdiv(p, q.dOW), ow = p - g * q.OW;
-    int n = fdiv(g, q.dOH), oh = g - n * q.OH;
-    return (n * q.VH + oh * q.SH) * q.VW + ow * q.SW;
-}
-
-template <int BM>
+// ACT: MEGCC_NONLINE_IDENTITY / MEGCC_NONLINE_RELU compile the epilogue for that activation;
+// ACT_RUNTIME selects by q.act per element (H_SWISH, SIGMOID).
+template <int BM, int ACT>
 __global__ void __launch_bounds__(THREADS) conv_mfma_i8_kernel(MfmaParams q) {
     constexpr int WM = BM / 2;          // rows per wave
     constexpr int MT = WM / 32;         // 32x32 tiles per wave along oc
@@ -228,40 +174,60 @@ __global__ void __launch_bounds__(THREADS) conv_mfma_i8_kernel(MfmaParams q) {
         }
     }
 
-    // ---- epilogue: register e of a 32x32 tile holds row 8*(e/4) + 4*(lane/32) + e%4, col lane%32
+    // ---- epilogue: register e of a 32x32 tile holds row 8*(e/4) + 4*(lane/32) + e%4, col lane%32.
+    //      The 4 bias values of a register group are fetched once and reused for all pixels.
+    int pix_n[NT], pix_rem[NT];
 #pragma unroll
     for (int ni = 0; ni < NT; ++ni) {
         const int p = p0 + wn * 64 + ni * 32 + (lane & 31);
-        if (p > plast)
-            continue;
-        const int n = fdiv(p, q.dOHW), rem = p - n * q.OHW;
+        pix_n[ni] = p <= plast ? (int)fdiv(p, q.dOHW) : -1;
+        pix_rem[ni] = p - pix_n[ni] * q.OHW;
+    }
 #pragma unroll
-        for (int mi = 0; mi < MT; ++mi) {
+    for (int mi = 0; mi < MT; ++mi) {
 #pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4) {
-                const int oc = oc0 + wm * WM + mi * 32 + e4 * 8 + kg * 4;
-                if (oc >= q.OC)
-                    continue;
-                int r[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    int a = acc[mi][ni][e4 * 4 + e];
-                    if (q.bias && oc + e < q.OC)
-                        a += q.bias[oc + e];
-                    r[e] = requant_conv_rt(q.act, a, q.s_src, q.s_flt, q.s_dst);
-                }
-                if (!q.dst_fc) {
-                    size_t o = ((size_t)n * (q.OC >> 2) + (oc >> 2)) * q.OHW + rem;
-                    ((uint32_t*)q.dst)[o] = pack4(r[0], r[1], r[2], r[3]);
-                } else {
-                    int8_t* o = q.dst + (size_t)p * q.OC + oc;
-                    if (((q.OC & 3) == 0)) {
-                        *(uint32_t*)o = pack4(r[0], r[1], r[2], r[3]);
+        for (int e4 = 0; e4 < 4; ++e4) {
+            const int oc = oc0 + wm * WM + mi * 32 + e4 * 8 + kg * 4;
+            if (oc < q.OC) {
+                int bv[4] = {0, 0, 0, 0};
+                if (q.bias) {
+                    if (oc + 3 < q.OC && q.bias_vec4) {
+                        const int4 t4 = *(const int4*)(q.bias + oc);
+                        bv[0] = t4.x; bv[1] = t4.y; bv[2] = t4.z; bv[3] = t4.w;
                     } else {
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                             if (oc + e < q.OC)
-                                o[e] = (int8_t)r[e];
+                                bv[e] = q.bias[oc + e];
+                    }
+                }
+#pragma unroll
+                for (int ni = 0; ni < NT; ++ni) {
+                    if (pix_n[ni] >= 0) {
+                        int r[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int a = acc[mi][ni][e4 * 4 + e] + bv[e];
+                            if (ACT == ACT_RUNTIME)
+                                r[e] = requant_conv_rt(q.act, a, q.s_src, q.s_flt, q.s_dst);
+                            else
+                                r[e] = requant_conv<ACT>(a, q.s_src, q.s_flt, q.s_dst);
+                        }
+                        if (!q.dst_fc) {
+                            size_t o = ((size_t)pix_n[ni] * (q.OC >> 2) + (oc >> 2)) * q.OHW + pix_rem[ni];
+                            ((uint32_t*)q.dst)[o] = pack4(r[0], r[1], r[2], r[3]);
+                        } else {
+                            const int p = p0 + wn * 64 + ni * 32 + (lane & 31);
+                            int8_t* o = q.dst + (size_t)p * q.OC + oc;
+                            if (((q.OC & 3) == 0)) {
+                                *(uint32_t*)o = pack4(r[0], r[1], r[2], r[3]);
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    if (oc + e < q.OC)
+                                        o[e] = (int8_t)r[e];
+                            }
+                        }
                     }
                 }
             }
@@ -300,6 +266,19 @@ __global__ void __launch_bounds__(256) pack_filter_kernel(
     }
 }
 
+static int num_cus() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            n = prop.multiProcessorCount;
+        if (n <= 0)
+            n = 256;
+    }
+    return n;
+}
+
 static int round_up(int a, int b) {
     return (a + b - 1) / b * b;
 }
@@ -318,8 +297,8 @@ struct TilePlan {
     int VW, VH;
 };
 
-// largest patch any tile needs; mirrors vp_of() / L in the kernel
-static TilePlan plan_tiles(const ConvGeom& g) {
+// largest patch any tile of `bn` pixels needs; mirrors vp_of() / L in the kernels
+static TilePlan plan_tiles(const ConvGeom& g, int bn = BN, long range_len = 0) {
     TilePlan t;
     t.VW = g.iw + 2 * g.pw;
     t.VH = g.ih + 2 * g.ph;
@@ -330,8 +309,12 @@ static TilePlan plan_tiles(const ConvGeom& g) {
         return (n * t.VH + oh * g.sh) * t.VW + ow * g.sw;
     };
     long lmax = 1;
-    for (long p0 = 0; p0 < P; p0 += BN) {
-        long pl = (p0 + BN < P ? p0 + BN : P) - 1;
+    if (range_len <= 0)
+        range_len = P;
+    for (long r0 = 0; r0 < P; r0 += range_len)
+    for (long p0 = r0; p0 < (r0 + range_len < P ? r0 + range_len : P); p0 += bn) {
+        long r1 = r0 + range_len < P ? r0 + range_len : P;
+        long pl = (p0 + bn < r1 ? p0 + bn : r1) - 1;
         long L = vp(pl) + (long)(g.fh - 1) * g.dh * t.VW + (g.fw - 1) * g.dw - vp(p0) + 1;
         if (L > lmax)
             lmax = L;
@@ -364,7 +347,8 @@ bool conv_mfma_supported(const ConvGeom& g) {
 
 size_t conv_mfma_packed_bytes(const ConvGeom& g) {
     int taps = g.fh * g.fw, ks = choose_ks(taps);
-    int chunks = round_up((g.ic + 31) / 32, ks);
+    (void)ks;
+    int chunks = round_up((g.ic + 31) / 32, CHUNK_PAD);
     return (size_t)chunks * taps * round_up(g.oc, OC_PAD) * KROW;
 }
 
@@ -379,10 +363,33 @@ TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed) {
     return check_launch("pack_filter");
 }
 
+bool conv_mfma_pipe_config(const ConvGeom& g, PipeConfig* c);
+TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
+
 TinyNNStatus conv_mfma_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst) {
     MfmaParams q;
-    TilePlan t = plan_tiles(g);
+    PipeConfig pc;
+    bool pipe = conv_mfma_pipe_config(g, &pc) && !getenv("MEGCC_NOPIPE");
+    long range_len = 0;
+    if (pipe) {
+        // one pixel range per free workgroup slot, so that the whole grid is resident at once and
+        // every CU finishes at the same time (no partial last round)
+        const long P = (long)g.n * g.oh * g.ow;
+        const long slots = (long)num_cus() * pc.blocks_per_cu;
+        const long oc_tiles = (g.oc + pc.bm - 1) / pc.bm;
+        long ranges = slots / oc_tiles > 0 ? slots / oc_tiles : 1;
+        range_len = ((P + ranges - 1) / ranges + 31) / 32 * 32;
+        if (range_len < pc.bn / 2)
+            pipe = false;  // too few pixels per workgroup to fill the 256-pixel tile
+    }
+    TilePlan t = plan_tiles(g, pipe ? pc.bn : BN, range_len);
+    if (pipe && (2L * pc.ks * t.Lmax > (long)pc.maxb * THREADS ||
+                 3L * pc.bm * KROW + 2L * pc.ks * t.Lmax * KROW > 160 * 1024)) {
+        pipe = false;
+        t = plan_tiles(g, BN);
+    }
+    q.range_len = (int)range_len;
     bool fc = is_fc(g);
     q.src = (const int8_t*)src;
     q.wp = (const int8_t*)packed;
@@ -399,7 +406,7 @@ TinyNNStatus conv_mfma_launch(
     q.taps = g.fh * g.fw;
     q.FH = g.fh;
     q.FW = g.fw;
-    q.KS = choose_ks(q.taps);
+    q.KS = pipe ? pc.ks : choose_ks(q.taps);
     q.stages = round_up((g.ic + 31) / 32, q.KS) / q.KS;
     q.VW = t.VW;
     q.VH = t.VH;
@@ -424,6 +431,7 @@ TinyNNStatus conv_mfma_launch(
     }
     q.Lmax = t.Lmax;
     q.dst_fc = fc ? 1 : 0;
+    q.bias_vec4 = bias && ((uintptr_t)bias & 15) == 0;
     q.act = g.act;
     q.s_src = g.s_src;
     q.s_flt = g.s_flt;
@@ -435,11 +443,22 @@ TinyNNStatus conv_mfma_launch(
     q.dL = make_fastdiv(q.Lmax);
     q.dOHW = make_fastdiv(q.OHW);
 
+    if (pipe)
+        return conv_mfma_pipe_launch(pc, q);
+
     const int bm = g.oc <= 64 ? 64 : 128;
     const size_t lds = (size_t)q.taps * q.KS * bm * KROW + (size_t)q.KS * q.Lmax * KROW;
     MG_REQUIRE(lds <= 160 * 1024, TinyNN_ERROR_OUT_OF_RANGE, "conv_mfma: %zu bytes of LDS", lds);
     dim3 grid((q.P + BN - 1) / BN, (g.oc + bm - 1) / bm);
-    auto kern = bm == 64 ? conv_mfma_i8_kernel<64> : conv_mfma_i8_kernel<128>;
+    void (*kern)(MfmaParams);
+    if (g.act == MEGCC_NONLINE_IDENTITY)
+        kern = bm == 64 ? conv_mfma_i8_kernel<64, MEGCC_NONLINE_IDENTITY>
+                        : conv_mfma_i8_kernel<128, MEGCC_NONLINE_IDENTITY>;
+    else if (g.act == MEGCC_NONLINE_RELU)
+        kern = bm == 64 ? conv_mfma_i8_kernel<64, MEGCC_NONLINE_RELU>
+                        : conv_mfma_i8_kernel<128, MEGCC_NONLINE_RELU>;
+    else
+        kern = bm == 64 ? conv_mfma_i8_kernel<64, ACT_RUNTIME> : conv_mfma_i8_kernel<128, ACT_RUNTIME>;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(
                 (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

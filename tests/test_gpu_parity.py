@@ -69,6 +69,14 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.DENSE, 5, 24, 7, 7, 32, 3, 1, 1, A.SIGMOID, scales=(0.02, 0.01, unsat(216) * 40)),
     ConvCase(A.FMT_NCHW44, A.DENSE, 1, 8, 30, 31, 8, 3, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(72))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 1, 16, 20, 20, 16, 3, 1, 2, A.RELU, scales=(0.02, 0.01, unsat(144)), dilate=2),
+    # large enough for the software-pipelined kernel (256x256 and 128x256 tiles), ragged edges
+    ConvCase(A.FMT_NCHW44, A.DENSE, 6, 32, 56, 56, 160, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(288))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 6, 64, 55, 57, 256, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(576))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 11, 36, 56, 56, 128, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(324))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 6, 136, 56, 56, 264, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(136))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 11, 64, 56, 56, 128, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(64))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 70, 256, 14, 14, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(256))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 16500, 96, 1, 1, 200, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(96) / 2)),
     # MobileNet pointwise shapes
     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 32, 112, 112, 64, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(32))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 4, 512, 14, 14, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(512))),

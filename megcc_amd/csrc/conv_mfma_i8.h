@@ -70,7 +70,7 @@ __device__ __forceinline__ int vp_of(const MfmaParams& q, int p) {
 
 
 struct PipeConfig {
-    int bm, bn, ks, maxb, blocks_per_cu;
+    int bm, bn, ks, maxb, blocks_per_cu, threads, a_bytes;
     const void* kernel;
 };
 

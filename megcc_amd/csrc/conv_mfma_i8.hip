@@ -370,7 +370,7 @@ TinyNNStatus conv_mfma_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst) {
     MfmaParams q;
     PipeConfig pc;
-    bool pipe = conv_mfma_pipe_config(g, &pc) && !getenv("MEGCC_NOPIPE");
+    bool pipe = conv_mfma_pipe_config(g, &pc) && !getenv("MEGCC_NOWIDE");
     long range_len = 0;
     if (pipe) {
         // one pixel range per free workgroup slot, so that the whole grid is resident at once and
@@ -384,8 +384,8 @@ TinyNNStatus conv_mfma_launch(
             pipe = false;  // too few pixels per workgroup to fill the 256-pixel tile
     }
     TilePlan t = plan_tiles(g, pipe ? pc.bn : BN, range_len);
-    if (pipe && (2L * pc.ks * t.Lmax > (long)pc.maxb * THREADS ||
-                 3L * pc.bm * KROW + 2L * pc.ks * t.Lmax * KROW > 160 * 1024)) {
+    if (pipe && (2L * pc.ks * t.Lmax > (long)pc.maxb * pc.threads ||
+                 2L * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) > 160 * 1024)) {
         pipe = false;
         t = plan_tiles(g, BN);
     }

@@ -59,6 +59,8 @@ struct MfmaParams {
     int act;
     float s_src, s_flt, s_dst;
     FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
+    int G, RG;       // 16-byte gather: pixel groups per row, groups per plane of the largest patch
+    FastDiv dG, dRG;
 };
 
 // virtual pixel index of output pixel p at tap (0,0): rows of the zero-padded images stacked
@@ -70,7 +72,7 @@ __device__ __forceinline__ int vp_of(const MfmaParams& q, int p) {
 
 
 struct PipeConfig {
-    int bm, bn, ks, maxb, blocks_per_cu, threads, a_bytes;
+    int bm, bn, ks, maxb, blocks_per_cu, threads, a_bytes, g4;
     const void* kernel;
 };
 

@@ -295,6 +295,7 @@ static int choose_ks(int taps) {
 struct TilePlan {
     int Lmax;
     int VW, VH;
+    int rows_max;  // most virtual rows any patch touches
 };
 
 // largest patch any tile of `bn` pixels needs; mirrors vp_of() / L in the kernels
@@ -308,7 +309,7 @@ static TilePlan plan_tiles(const ConvGeom& g, int bn = BN, long range_len = 0) {
         long n = gi / g.oh, oh = gi % g.oh;
         return (n * t.VH + oh * g.sh) * t.VW + ow * g.sw;
     };
-    long lmax = 1;
+    long lmax = 1, rmax = 1;
     if (range_len <= 0)
         range_len = P;
     for (long r0 = 0; r0 < P; r0 += range_len)
@@ -318,8 +319,12 @@ static TilePlan plan_tiles(const ConvGeom& g, int bn = BN, long range_len = 0) {
         long L = vp(pl) + (long)(g.fh - 1) * g.dh * t.VW + (g.fw - 1) * g.dw - vp(p0) + 1;
         if (L > lmax)
             lmax = L;
+        long rows = (vp(p0) + L - 1) / t.VW - vp(p0) / t.VW + 1;
+        if (rows > rmax)
+            rmax = rows;
     }
     t.Lmax = round_up((int)(lmax > (1 << 20) ? (1 << 20) : lmax), 64);
+    t.rows_max = (int)rmax;
     return t;
 }
 
@@ -363,14 +368,15 @@ TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed) {
     return check_launch("pack_filter");
 }
 
-bool conv_mfma_pipe_config(const ConvGeom& g, PipeConfig* c);
+bool conv_mfma_pipe_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
 
 TinyNNStatus conv_mfma_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst) {
     MfmaParams q;
     PipeConfig pc;
-    bool pipe = conv_mfma_pipe_config(g, &pc) && !getenv("MEGCC_NOWIDE");
+    const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;
+    bool pipe = conv_mfma_pipe_config(g, g4_ok, &pc) && !getenv("MEGCC_NOWIDE");
     long range_len = 0;
     if (pipe) {
         // one pixel range per free workgroup slot, so that the whole grid is resident at once and
@@ -384,7 +390,9 @@ TinyNNStatus conv_mfma_launch(
             pipe = false;  // too few pixels per workgroup to fill the 256-pixel tile
     }
     TilePlan t = plan_tiles(g, pipe ? pc.bn : BN, range_len);
-    if (pipe && (2L * pc.ks * t.Lmax > (long)pc.maxb * pc.threads ||
+    const long gather_items =
+            !pipe ? 0 : pc.g4 ? 8L * pc.ks * t.rows_max * (g.iw / 4) : 2L * pc.ks * t.Lmax;
+    if (pipe && (gather_items > (long)pc.maxb * pc.threads ||
                  2L * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) > 160 * 1024)) {
         pipe = false;
         t = plan_tiles(g, BN);
@@ -442,6 +450,10 @@ TinyNNStatus conv_mfma_launch(
     q.dVH = make_fastdiv(q.VH);
     q.dL = make_fastdiv(q.Lmax);
     q.dOHW = make_fastdiv(q.OHW);
+    q.G = g.iw / 4 > 0 ? g.iw / 4 : 1;
+    q.RG = t.rows_max * q.G;
+    q.dG = make_fastdiv(q.G);
+    q.dRG = make_fastdiv(q.RG);
 
     if (pipe)
         return conv_mfma_pipe_launch(pc, q);

@@ -48,7 +48,15 @@ static constexpr int WTHREADS = 512;
 // FH x FW: 3x3 or 1x1 (taps unrolled); KS: 32-channel sub-chunks per stage.
 // ACT: MEGCC_NONLINE_IDENTITY / _RELU compile the epilogue for that activation, ACT_RT selects by
 // q.act per element.
-template <int WGM, int WGN, int MT, int NT, int FH, int FW, int KS, int ACT>
+//
+// G4 selects how the activation patch is gathered from the NCHW44 planes:
+//   G4 = false: one dword (4 channels of one pixel) per lane and load, 4 loads -> one 16-byte LDS
+//               write; works for any layout the one-stage kernel accepts.
+//   G4 = true : one 16-byte load = 4 horizontally adjacent pixels x 4 channels of one plane,
+//               scattered as four dword LDS writes (a quarter of the load instructions); needs
+//               IW % 4 == 0 and a 16-byte aligned source. Padding slots are never written by
+//               the gather: they are zeroed once per sub-tile.
+template <int WGM, int WGN, int MT, int NT, int FH, int FW, int KS, int ACT, bool G4, int MAXB>
 __global__ void __launch_bounds__(WTHREADS) conv_mfma_i8_wide_kernel(MfmaParams q) {
     constexpr int BM = WGM * MT * 32;
     constexpr int BNP = WGN * NT * 32;
@@ -57,7 +65,6 @@ __global__ void __launch_bounds__(WTHREADS) conv_mfma_i8_wide_kernel(MfmaParams 
     constexpr int A_BYTES = TS * BM * KROW;
     constexpr int A_CHUNKS = A_BYTES / 16;
     constexpr int A_ITEMS = (A_CHUNKS + WTHREADS - 1) / WTHREADS;
-    constexpr int MAXB = 4;
     static_assert(WGM * WGN * 64 == WTHREADS, "8 waves");
 
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];
@@ -84,29 +91,62 @@ __global__ void __launch_bounds__(WTHREADS) conv_mfma_i8_wide_kernel(MfmaParams 
         const int vp0 = vp_of(q, p0);
         const int L = vp_of(q, plast) + ((FH - 1) * q.DH) * q.VW + (FW - 1) * q.DW - vp0 + 1;
 
-        // ---- gather items of this thread (see conv_mfma_i8.hip)
+        // ---- gather items of this thread
         int b_goff[MAXB], b_loff[MAXB], b_plane[MAXB];
-        const int n_items = 2 * KS * q.Lmax;
+        if (!G4) {
+            // (patch slot, 16-byte half of a 32-channel row, sub-chunk), see conv_mfma_i8.hip
+            const int n_items = 2 * KS * q.Lmax;
 #pragma unroll
-        for (int j = 0; j < MAXB; ++j) {
-            int i = tid + j * WTHREADS;
-            b_goff[j] = -1;
-            b_loff[j] = -1;
-            b_plane[j] = 0;
-            if (i < n_items) {
-                int h = fdiv(i, q.dL), slot = i - h * q.Lmax;
-                b_loff[j] = A_BYTES + (h >> 1) * (q.Lmax * KROW) + slot * KROW +
-                            (((h ^ (slot >> 3)) & 1) << 4);
-                b_plane[j] = (h >> 1) * 8 + (h & 1) * 4;
-                if (slot < L) {
-                    int vp = vp0 + slot;
-                    int v = fdiv(vp, q.dVW), vc = vp - v * q.VW;
-                    int n = fdiv(v, q.dVH), vh = v - n * q.VH;
-                    int ih = vh - q.PH, iw = vc - q.PW;
-                    if (n < q.N && (unsigned)ih < (unsigned)q.IH && (unsigned)iw < (unsigned)q.IW)
-                        b_goff[j] = n * q.image_stride + ih * q.row_stride + iw * q.pix_stride;
+            for (int j = 0; j < MAXB; ++j) {
+                int i = tid + j * WTHREADS;
+                b_goff[j] = -1;
+                b_loff[j] = -1;
+                b_plane[j] = 0;
+                if (i < n_items) {
+                    int h = fdiv(i, q.dL), slot = i - h * q.Lmax;
+                    b_loff[j] = A_BYTES + (h >> 1) * (q.Lmax * KROW) + slot * KROW +
+                                (((h ^ (slot >> 3)) & 1) << 4);
+                    b_plane[j] = (h >> 1) * 8 + (h & 1) * 4;
+                    if (slot < L) {
+                        int vp = vp0 + slot;
+                        int v = fdiv(vp, q.dVW), vc = vp - v * q.VW;
+                        int n = fdiv(v, q.dVH), vh = v - n * q.VH;
+                        int ih = vh - q.PH, iw = vc - q.PW;
+                        if (n < q.N && (unsigned)ih < (unsigned)q.IH && (unsigned)iw < (unsigned)q.IW)
+                            b_goff[j] = n * q.image_stride + ih * q.row_stride + iw * q.pix_stride;
+                    }
                 }
             }
+        } else {
+            // (plane of the stage, patch row, group of 4 pixels): b_goff = byte offset of the
+            // group in plane 0 (-1: no such item / padding row), b_loff = patch slot of its first
+            // pixel (may be negative at the ragged start of the patch), b_plane = plane in stage
+            const int v_first = fdiv(vp0, q.dVW);
+            const int rows = (int)fdiv(vp0 + L - 1, q.dVW) - v_first + 1;
+            const int slot_base = q.PW - (vp0 - v_first * q.VW);
+#pragma unroll
+            for (int j = 0; j < MAXB; ++j) {
+                int i = tid + j * WTHREADS;
+                int pl = fdiv(i, q.dRG), rem = i - pl * q.RG;
+                int r = fdiv(rem, q.dG), g4 = rem - r * q.G;
+                b_goff[j] = -1;
+                b_plane[j] = pl;
+                b_loff[j] = r * q.VW + slot_base + 4 * g4;
+                if (pl < KS * 8 && r < rows) {
+                    int v = v_first + r;
+                    int n = fdiv(v, q.dVH), vh = v - n * q.VH;
+                    int ih = vh - q.PH;
+                    if (n < q.N && (unsigned)ih < (unsigned)q.IH)
+                        b_goff[j] = n * q.image_stride + ih * q.row_stride + g4 * 16;
+                }
+            }
+            // padding slots stay zero for the whole sub-tile, in both buffers
+            const v4i zero = {0, 0, 0, 0};
+            for (int i = tid; i < b_bytes / 16; i += WTHREADS) {
+                *(v4i*)(lds + A_BYTES + i * 16) = zero;
+                *(v4i*)(lds + buf_bytes + A_BYTES + i * 16) = zero;
+            }
+            lds_barrier();
         }
         int b_slot[NT];
 #pragma unroll
@@ -140,17 +180,26 @@ __global__ void __launch_bounds__(WTHREADS) conv_mfma_i8_wide_kernel(MfmaParams 
             const int last = q.C4 - 1;
 #pragma unroll
             for (int j = 0; j < MAXB; ++j) {
-                // branch-free: padding pixels read pixel 0 and are zeroed by a select; planes past
-                // the last one are clamped (they meet zero filter rows: their value is irrelevant)
-                const bool ok = b_goff[j] >= 0;
-                const int8_t* g = q.src + (ok ? b_goff[j] : 0);
-                const int pl = plane0 + b_plane[j];
-                v4i v;
-                v[0] = *(const int*)(g + (size_t)min(pl + 0, last) * q.plane_stride);
-                v[1] = *(const int*)(g + (size_t)min(pl + 1, last) * q.plane_stride);
-                v[2] = *(const int*)(g + (size_t)min(pl + 2, last) * q.plane_stride);
-                v[3] = *(const int*)(g + (size_t)min(pl + 3, last) * q.plane_stride);
-                rb[j] = ok ? v : v4i{0, 0, 0, 0};
+                if (G4) {
+                    // planes past the last one are clamped: they meet zero filter rows
+                    if (b_goff[j] >= 0)
+                        rb[j] = *(const v4i*)(q.src + b_goff[j] +
+                                                   (size_t)min(plane0 + b_plane[j], last) * q.plane_stride);
+                } else {
+                    // whole waves have no item j (wave-uniform branch); inside an item the loads
+                    // are branch-free: padding pixels read pixel 0 and are zeroed by a select
+                    if (b_loff[j] < 0)
+                        continue;
+                    const bool ok = b_goff[j] >= 0;
+                    const int8_t* g = q.src + (ok ? b_goff[j] : 0);
+                    const int pl = plane0 + b_plane[j];
+                    v4i v;
+                    v[0] = *(const int*)(g + (size_t)min(pl + 0, last) * q.plane_stride);
+                    v[1] = *(const int*)(g + (size_t)min(pl + 1, last) * q.plane_stride);
+                    v[2] = *(const int*)(g + (size_t)min(pl + 2, last) * q.plane_stride);
+                    v[3] = *(const int*)(g + (size_t)min(pl + 3, last) * q.plane_stride);
+                    rb[j] = ok ? v : v4i{0, 0, 0, 0};
+                }
             }
         };
         auto stage_to_lds = [&](int st) {
@@ -162,18 +211,25 @@ __global__ void __launch_bounds__(WTHREADS) conv_mfma_i8_wide_kernel(MfmaParams 
                     *(v4i*)(buf + i * 16) = ra[j];
             }
 #pragma unroll
-            for (int j = 0; j < MAXB; ++j)
-                if (b_loff[j] >= 0)
+            for (int j = 0; j < MAXB; ++j) {
+                if (G4) {
+                    if (b_goff[j] >= 0) {
+                        const int pl = b_plane[j];
+                        int8_t* row = buf + A_BYTES + (pl >> 3) * (q.Lmax * KROW) + (pl & 3) * 4;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const int slot = b_loff[j] + k;
+                            if ((unsigned)slot < (unsigned)L)
+                                *(int*)(row + slot * KROW + ((((pl >> 2) ^ (slot >> 3)) & 1) << 4)) =
+                                        rb[j][k];
+                        }
+                    }
+                } else if (b_loff[j] >= 0) {
                     *(v4i*)(buf + b_loff[j]) = rb[j];
+                }
+            }
         };
-
-        prefetch(0);
-        stage_to_lds(0);
-        lds_barrier();
-
-        for (int st = 0; st < q.stages; ++st) {
-            if (st + 1 < q.stages)
-                prefetch(st + 1);
+        auto compute = [&](int st) {
             const int8_t* bufA = lds + (st & 1) * buf_bytes;
             const int8_t* bufB = bufA + A_BYTES;
             static_for<TS>([&](auto tc) {
@@ -198,6 +254,15 @@ __global__ void __launch_bounds__(WTHREADS) conv_mfma_i8_wide_kernel(MfmaParams 
                         acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
                                 a[mi], b[ni], acc[mi][ni], 0, 0, 0);
             });
+        };
+        prefetch(0);
+        stage_to_lds(0);
+        lds_barrier();
+
+        for (int st = 0; st < q.stages; ++st) {
+            if (st + 1 < q.stages)
+                prefetch(st + 1);
+            compute(st);
             if (st + 1 < q.stages)
                 stage_to_lds(st + 1);
             lds_barrier();
@@ -261,41 +326,48 @@ __global__ void __launch_bounds__(WTHREADS) conv_mfma_i8_wide_kernel(MfmaParams 
 }
 
 // ---- configurations --------------------------------------------------------------------------
-template <int WGM, int WGN, int MT, int NT, int FH, int FW, int KS>
+template <int WGM, int WGN, int MT, int NT, int FH, int FW, int KS, bool G4, int MAXB>
 static PipeConfig make_config(int act) {
     PipeConfig c;
     c.bm = WGM * MT * 32;
     c.bn = WGN * NT * 32;
     c.ks = KS;
-    c.maxb = 4;
+    c.maxb = MAXB;
+    c.g4 = G4;
     c.threads = WTHREADS;
     c.blocks_per_cu = 1;
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     if (act == MEGCC_NONLINE_IDENTITY)
-        c.kernel = (const void*)conv_mfma_i8_wide_kernel<WGM, WGN, MT, NT, FH, FW, KS, MEGCC_NONLINE_IDENTITY>;
+        c.kernel = (const void*)conv_mfma_i8_wide_kernel<WGM, WGN, MT, NT, FH, FW, KS,
+                                                         MEGCC_NONLINE_IDENTITY, G4, MAXB>;
     else if (act == MEGCC_NONLINE_RELU)
-        c.kernel = (const void*)conv_mfma_i8_wide_kernel<WGM, WGN, MT, NT, FH, FW, KS, MEGCC_NONLINE_RELU>;
+        c.kernel = (const void*)conv_mfma_i8_wide_kernel<WGM, WGN, MT, NT, FH, FW, KS,
+                                                         MEGCC_NONLINE_RELU, G4, MAXB>;
     else
-        c.kernel = (const void*)conv_mfma_i8_wide_kernel<WGM, WGN, MT, NT, FH, FW, KS, ACT_RT>;
+        c.kernel = (const void*)conv_mfma_i8_wide_kernel<WGM, WGN, MT, NT, FH, FW, KS, ACT_RT, G4, MAXB>;
     return c;
 }
 
 // Picks the tile for (filter size, oc); returns false when the shape is better served by the
-// one-stage kernel (small problems, filter sizes other than 1x1 and 3x3).
-bool conv_mfma_pipe_config(const ConvGeom& g, PipeConfig* c) {
+// one-stage kernel (small problems, filter sizes other than 1x1 and 3x3). `g4_ok`: the source
+// allows 16-byte gathers (NCHW44, IW % 4 == 0, 16-byte aligned).
+bool conv_mfma_pipe_config(const ConvGeom& g, bool g4_ok, PipeConfig* c) {
     const long P = (long)g.n * g.oh * g.ow;
     const bool k3 = g.fh == 3 && g.fw == 3, k1 = g.fh == 1 && g.fw == 1;
     if (!(k3 || k1) || g.oc < 128 || P < 8192)
         return false;
-    *c = k3 ? make_config<2, 4, 2, 2, 3, 3, 1>(g.act) : make_config<2, 4, 2, 2, 1, 1, 4>(g.act);
+    if (k3)
+        *c = g4_ok ? make_config<2, 4, 2, 2, 3, 3, 1, true, 3>(g.act)
+                   : make_config<2, 4, 2, 2, 3, 3, 1, false, 2>(g.act);
+    else
+        *c = g4_ok ? make_config<2, 4, 2, 2, 1, 1, 4, true, 7>(g.act)
+                   : make_config<2, 4, 2, 2, 1, 1, 4, false, 4>(g.act);
     return true;
 }
 
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q) {
     const size_t lds = 2 * ((size_t)c.a_bytes + (size_t)c.ks * q.Lmax * KROW);
     MG_REQUIRE(lds <= 160 * 1024, TinyNN_ERROR_OUT_OF_RANGE, "conv_mfma_wide: %zu bytes of LDS", lds);
-    MG_REQUIRE(2L * c.ks * q.Lmax <= (long)c.maxb * c.threads, TinyNN_ERROR_OUT_OF_RANGE,
-               "conv_mfma_wide: patch of %d slots exceeds the gather registers", q.Lmax);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(c.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_mfma_wide: LDS attribute: %s",

@@ -367,6 +367,48 @@ void* megcc_gfx950_stream(void);
 /* Text of the most recent error on the calling thread ("" if none). */
 const char* megcc_gfx950_last_error(void);
 
+/* ------------------------------------------------------------------------------------------
+ * In-memory model runtime: MegCC's static memory plan on one HBM arena. The calls mirror what the
+ * TinyNN runtime does with a parsed `.tiny` model -- tensors with offsets into one buffer, weights,
+ * a list of Opr instructions (runtime/schema/model.fbs:63-124) -- for a caller that builds the
+ * model in memory the way runtime/test/common/common.h:46-123 does:
+ *   add_* / add_opr   describe tensors, weights (uploaded to HBM at once) and instructions; an
+ *                     instruction names its kernel by the generated symbol
+ *   add_alias         a MemForward / reshape view sharing another tensor's memory
+ *   finalize          liveness -> offsets (the [def, last use] intervals of
+ *                     compiler/lib/Dialect/Kernel/Transforms/StaticMemoryPlanning.cpp:88-96), one
+ *                     Device.malloc for the arena (runtime/src/init.c:437-487), three-phase kernel
+ *                     init on the weights (init.c:29-131)
+ *   set_input         LITE_reset_tensor_memory + staging copy (runtime/src/lite/tensor.c:93-112)
+ *   forward           LITE_forward: one asynchronous launch per Opr (lite/network.c:171-227)
+ *   get_output        waits, then copies back (LITE_get_tensor_memory)
+ * Tensor ids are the return values of the add_* calls (-1 on error).
+ * ---------------------------------------------------------------------------------------- */
+void* megcc_gfx950_model_create(void);
+void megcc_gfx950_model_destroy(void* model);
+int megcc_gfx950_model_add_tensor(
+        void* model, const char* name, int nr_dim, const uint32_t* dims, TinyNNDType dtype,
+        float scale);
+int megcc_gfx950_model_add_weight(
+        void* model, const char* name, int nr_dim, const uint32_t* dims, TinyNNDType dtype,
+        float scale, const void* host_data);
+int megcc_gfx950_model_add_alias(
+        void* model, const char* name, int of_tensor, int nr_dim, const uint32_t* dims);
+TinyNNStatus megcc_gfx950_model_add_opr(
+        void* model, const char* symbol, const int* inputs, int nr_input, const int* outputs,
+        int nr_output);
+TinyNNStatus megcc_gfx950_model_mark_io(void* model, int tensor, int is_output);
+TinyNNStatus megcc_gfx950_model_finalize(void* model);
+size_t megcc_gfx950_model_arena_bytes(void* model);
+void* megcc_gfx950_model_tensor_ptr(void* model, int tensor);
+TinyNNStatus megcc_gfx950_model_set_input(void* model, int tensor, const void* host, size_t bytes);
+TinyNNStatus megcc_gfx950_model_get_output(void* model, int tensor, void* host, size_t bytes);
+TinyNNStatus megcc_gfx950_model_forward(void* model);
+int megcc_gfx950_model_nr_opr(void* model);
+/* one instruction only: per-layer timing / tensor dumps (the TINYNN_PROFILE_KERNEL and
+ * TINYNN_DUMP_TENSOR hooks of runtime/src/lite/network.c:187-224) */
+TinyNNStatus megcc_gfx950_model_run_opr(void* model, int index);
+
 #ifdef __cplusplus
 }
 #endif

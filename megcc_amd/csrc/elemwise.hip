@@ -244,6 +244,12 @@ static TinyNNStatus classify_bcast(const Tensor* a, const Tensor* b, EwArgs* p, 
         p->bcast = BC_CHANNEL;
         p->C = (int)nb;
         p->inner = 1;
+    } else if (a->layout.nr_dim == 2 && b->layout.nr_dim == 2 &&
+               b->layout.dims[0] == a->layout.dims[0] && b->layout.dims[1] == 1) {
+        // [A,N] op [A,1]: one value per row (softmax: x - max, e / sum)
+        p->bcast = BC_CHANNEL;
+        p->C = a->layout.dims[0];
+        p->inner = a->layout.dims[1];
     } else {
         return fail(TinyNN_ERROR_INVALID_LAYOUT, "%s: unsupported broadcast", who);
     }

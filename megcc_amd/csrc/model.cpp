@@ -1,0 +1,409 @@
+// In-memory model runtime: the seam between MegCC's static memory plan and one HBM arena.
+//
+// A MegCC model is a list of tensors with byte offsets into ONE buffer, a list of weights and a
+// list of `Opr` instructions, each naming a kernel and its tensors (runtime/schema/model.fbs:63-124,
+// runtime/src/vm/instruction.h:61-76). The TinyNN runtime allocates that buffer once through
+// Device.malloc and points every tensor at base + offset (runtime/src/init.c:437-487), runs the
+// kernels' three-phase init on the weights (init.c:29-131) and then simply walks the instruction
+// list (runtime/src/lite/network.c:171-227, vm/op.c:67-172). This file is that sequence with the
+// gfx950 Device: weights are uploaded to HBM and repacked there by the kernels' init, the arena is
+// one hipMalloc, input staging is a stream-ordered hipMemcpyAsync, and forward() is one
+// asynchronous launch per Opr on the library stream.
+//
+// The MegCC compiler (and with it StaticMemoryPlanning) cannot be built without MLIR, so the plan
+// is produced here from the same inputs it uses: per tensor the interval [defining opr, last
+// using opr + 1) (compiler/lib/Dialect/Kernel/Transforms/StaticMemoryPlanning.cpp:88-96) and the
+// byte size; tensors whose intervals overlap get disjoint offset ranges.
+#include <string.h>
+
+#include <algorithm>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+using namespace mg;
+
+namespace {
+
+struct ModelTensor {
+    Tensor t;
+    std::string name;
+    bool is_weight = false, is_input = false, is_output = false;
+    int alias_of = -1;  // MemForward / reshape: shares the memory of another tensor
+    int def = -1, last = -1;
+    void* owned = nullptr;  // weights: device allocation owned by the model
+};
+
+struct ModelOpr {
+    MegccKernelDesc desc;
+    std::string symbol;
+    std::vector<int> in, out;
+    std::vector<Tensor*> in_ptrs, out_ptrs;
+    Tensor processed;  // weight produced by the kernel's init, replaces one input
+    bool has_processed = false;
+    void* processed_mem = nullptr;
+    Workspace ws;
+};
+
+struct Model {
+    Device dev;
+    RuntimeOpt opt;
+    std::vector<ModelTensor*> tensors;
+    std::vector<ModelOpr*> oprs;
+    void* arena = nullptr;
+    size_t arena_bytes = 0;
+    bool finalized = false;
+};
+
+size_t tensor_bytes(const Tensor& t) {
+    return nr_elem(t.layout) * dtype_size(&t);
+}
+
+size_t align_up(size_t v, size_t a) {
+    return (v + a - 1) / a * a;
+}
+
+int root_of(const Model* m, int id) {
+    while (m->tensors[id]->alias_of >= 0)
+        id = m->tensors[id]->alias_of;
+    return id;
+}
+
+// Offsets for the arena: largest tensors first, each at the lowest offset that does not collide
+// with an already placed tensor whose lifetime overlaps.
+void plan_memory(Model* m) {
+    struct Item {
+        int id;
+        size_t size, offset;
+        int begin, end;
+    };
+    std::vector<Item> items;
+    for (size_t i = 0; i < m->tensors.size(); ++i) {
+        ModelTensor* t = m->tensors[i];
+        if (t->is_weight || t->alias_of >= 0 || t->def < 0)
+            continue;
+        Item it;
+        it.id = (int)i;
+        it.size = align_up(tensor_bytes(t->t), m->dev.alignment);
+        it.begin = t->def;
+        it.end = t->last + 1;
+        if (t->is_output)
+            it.end = (int)m->oprs.size() + 1;  // outputs stay valid after forward()
+        it.offset = 0;
+        items.push_back(it);
+    }
+    // model inputs are staged into the arena as well and live from before the first opr
+    std::vector<Item*> order;
+    for (auto& it : items)
+        order.push_back(&it);
+    std::sort(order.begin(), order.end(), [](const Item* a, const Item* b) {
+        return a->size != b->size ? a->size > b->size : a->id < b->id;
+    });
+    std::vector<Item*> placed;
+    size_t total = 0;
+    for (Item* it : order) {
+        std::vector<std::pair<size_t, size_t>> busy;
+        for (Item* p : placed)
+            if (p->begin < it->end && it->begin < p->end)
+                busy.emplace_back(p->offset, p->offset + p->size);
+        std::sort(busy.begin(), busy.end());
+        size_t off = 0;
+        for (auto& b : busy) {
+            if (off + it->size <= b.first)
+                break;
+            off = std::max(off, b.second);
+        }
+        it->offset = off;
+        total = std::max(total, off + it->size);
+        placed.push_back(it);
+    }
+    for (auto& it : items)
+        m->tensors[it.id]->t.offset = it.offset;
+    m->arena_bytes = total;
+}
+
+}  // namespace
+
+extern "C" {
+
+void* megcc_gfx950_model_create(void) {
+    Model* m = new Model();
+    if (megcc_gfx950_init_device(&m->dev) != TinyNN_SUCCESS) {
+        delete m;
+        return nullptr;
+    }
+    m->opt.device = &m->dev;
+    return m;
+}
+
+void megcc_gfx950_model_destroy(void* model) {
+    Model* m = (Model*)model;
+    if (!m)
+        return;
+    (void)hipStreamSynchronize(stream());
+    for (auto* o : m->oprs) {
+        if (o->processed_mem)
+            m->dev.free(o->processed_mem);
+        delete o;
+    }
+    for (auto* t : m->tensors) {
+        if (t->owned)
+            m->dev.free(t->owned);
+        delete t;
+    }
+    if (m->arena)
+        m->dev.free(m->arena);
+    delete m;
+}
+
+static int add_tensor(
+        Model* m, const char* name, int nr_dim, const uint32_t* dims, TinyNNDType dtype,
+        float scale) {
+    if (!m || m->finalized || nr_dim < 1 || nr_dim > MAX_DIM || !dims)
+        return -1;
+    ModelTensor* t = new ModelTensor();
+    memset(&t->t, 0, sizeof(Tensor));
+    t->name = name ? name : "";
+    t->t.dtype.type_enum = dtype;
+    t->t.dtype.param.scale = scale;
+    t->t.layout.nr_dim = nr_dim;
+    int stride = 1;
+    for (int i = nr_dim - 1; i >= 0; --i) {
+        t->t.layout.dims[i] = dims[i];
+        t->t.layout.stride[i] = stride;
+        stride *= dims[i];
+    }
+    t->t.size = tensor_bytes(t->t);
+    m->tensors.push_back(t);
+    t->t.name = (char*)m->tensors.back()->name.c_str();
+    return (int)m->tensors.size() - 1;
+}
+
+int megcc_gfx950_model_add_tensor(
+        void* model, const char* name, int nr_dim, const uint32_t* dims, TinyNNDType dtype,
+        float scale) {
+    return add_tensor((Model*)model, name, nr_dim, dims, dtype, scale);
+}
+
+int megcc_gfx950_model_add_weight(
+        void* model, const char* name, int nr_dim, const uint32_t* dims, TinyNNDType dtype,
+        float scale, const void* host_data) {
+    Model* m = (Model*)model;
+    int id = add_tensor(m, name, nr_dim, dims, dtype, scale);
+    if (id < 0 || !host_data)
+        return -1;
+    ModelTensor* t = m->tensors[id];
+    t->is_weight = true;
+    t->t.is_weight = 1;
+    t->owned = m->dev.malloc(t->t.size);
+    if (!t->owned)
+        return -1;
+    t->t.ptr = t->owned;
+    if (megcc_gfx950_memcpy_h2d(t->owned, host_data, t->t.size) != TinyNN_SUCCESS)
+        return -1;
+    return id;
+}
+
+int megcc_gfx950_model_add_alias(
+        void* model, const char* name, int of, int nr_dim, const uint32_t* dims) {
+    Model* m = (Model*)model;
+    if (!m || of < 0 || of >= (int)m->tensors.size())
+        return -1;
+    const Tensor& src = m->tensors[of]->t;
+    int id = add_tensor(m, name, nr_dim, dims, src.dtype.type_enum, src.dtype.param.scale);
+    if (id < 0)
+        return -1;
+    if (tensor_bytes(m->tensors[id]->t) != tensor_bytes(src)) {
+        fail(TinyNN_ERROR_INVALID_LAYOUT, "model_add_alias: byte sizes differ");
+        return -1;
+    }
+    m->tensors[id]->alias_of = of;
+    return id;
+}
+
+TinyNNStatus megcc_gfx950_model_add_opr(
+        void* model, const char* symbol, const int* inputs, int nr_input, const int* outputs,
+        int nr_output) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && symbol && inputs && outputs && !m->finalized, TinyNN_ERROR_NULL_PTR,
+               "model_add_opr: bad argument");
+    ModelOpr* o = new ModelOpr();
+    TinyNNStatus st = megcc_gfx950_parse_symbol(symbol, &o->desc);
+    if (st != TinyNN_SUCCESS) {
+        delete o;
+        return st;
+    }
+    o->symbol = symbol;
+    memset(&o->ws, 0, sizeof(o->ws));
+    const int idx = (int)m->oprs.size();
+    for (int i = 0; i < nr_input; ++i) {
+        if (inputs[i] < 0 || inputs[i] >= (int)m->tensors.size()) {
+            delete o;
+            return fail(TinyNN_ERROR_OUT_OF_RANGE, "model_add_opr: input id %d", inputs[i]);
+        }
+        o->in.push_back(inputs[i]);
+        ModelTensor* t = m->tensors[root_of(m, inputs[i])];
+        t->last = std::max(t->last, idx);
+    }
+    for (int i = 0; i < nr_output; ++i) {
+        if (outputs[i] < 0 || outputs[i] >= (int)m->tensors.size()) {
+            delete o;
+            return fail(TinyNN_ERROR_OUT_OF_RANGE, "model_add_opr: output id %d", outputs[i]);
+        }
+        o->out.push_back(outputs[i]);
+        ModelTensor* t = m->tensors[root_of(m, outputs[i])];
+        if (t->def < 0)
+            t->def = idx;
+        t->last = std::max(t->last, idx);
+    }
+    m->oprs.push_back(o);
+    return TinyNN_SUCCESS;
+}
+
+TinyNNStatus megcc_gfx950_model_mark_io(void* model, int tensor, int is_output) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && tensor >= 0 && tensor < (int)m->tensors.size(), TinyNN_ERROR_OUT_OF_RANGE,
+               "model_mark_io: tensor id");
+    ModelTensor* t = m->tensors[root_of(m, tensor)];
+    if (is_output) {
+        t->is_output = true;
+    } else {
+        t->is_input = true;
+        t->def = 0;  // staged before the first opr
+        if (t->last < 0)
+            t->last = 0;
+    }
+    return TinyNN_SUCCESS;
+}
+
+// parse_model + init_model_weights + init_model_memory of the TinyNN runtime
+TinyNNStatus megcc_gfx950_model_finalize(void* model) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && !m->finalized, TinyNN_ERROR_NULL_PTR, "model_finalize: bad model");
+    for (auto* t : m->tensors)
+        if (t->is_input && t->def != 0)
+            t->def = 0;
+    plan_memory(m);
+    m->arena = m->dev.malloc(m->arena_bytes ? m->arena_bytes : 1);
+    MG_REQUIRE(m->arena, TinyNN_ERROR_MEMORY_MALLOC, "model_finalize: arena of %zu bytes",
+               m->arena_bytes);
+    for (auto* t : m->tensors)
+        if (!t->is_weight && t->alias_of < 0)
+            t->t.ptr = (char*)m->arena + t->t.offset;
+    for (size_t i = 0; i < m->tensors.size(); ++i)
+        if (m->tensors[i]->alias_of >= 0) {
+            const Tensor& r = m->tensors[root_of(m, (int)i)]->t;
+            m->tensors[i]->t.ptr = r.ptr;
+            m->tensors[i]->t.offset = r.offset;
+        }
+    for (auto* o : m->oprs) {
+        for (int id : o->in)
+            o->in_ptrs.push_back(&m->tensors[id]->t);
+        for (int id : o->out)
+            o->out_ptrs.push_back(&m->tensors[id]->t);
+        // three-phase init (runtime/src/init.c:94-131)
+        int n = 0;
+        TinyNNStatus st = megcc_gfx950_call_init(
+                &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), nullptr, &n, &m->opt);
+        if (st != TinyNN_SUCCESS)
+            return st;
+        MG_REQUIRE(n <= 1, TinyNN_ERROR_NO_IMPLEMENT, "model_finalize: %d processed weights", n);
+        if (n == 1) {
+            memset(&o->processed, 0, sizeof(Tensor));
+            st = megcc_gfx950_call_init(
+                    &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), &o->processed, nullptr,
+                    &m->opt);
+            if (st != TinyNN_SUCCESS)
+                return st;
+            size_t bytes = tensor_bytes(o->processed);
+            o->processed_mem = m->dev.malloc(bytes);
+            MG_REQUIRE(o->processed_mem, TinyNN_ERROR_MEMORY_MALLOC,
+                       "model_finalize: processed weight of %zu bytes", bytes);
+            o->processed.ptr = o->processed_mem;
+            o->processed.size = bytes;
+            o->processed.is_weight = 1;
+            st = megcc_gfx950_call_init(
+                    &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), &o->processed, &n,
+                    &m->opt);
+            if (st != TinyNN_SUCCESS)
+                return st;
+            // the processed weight replaces the input with the same name (init.c:60-91)
+            for (size_t j = 0; j < o->in_ptrs.size(); ++j)
+                if (o->in_ptrs[j]->name == o->processed.name) {
+                    o->in_ptrs[j] = &o->processed;
+                    o->has_processed = true;
+                    break;
+                }
+            MG_REQUIRE(o->has_processed, TinyNN_ERROR_NO_FOUND,
+                       "model_finalize: %s: processed weight matches no input", o->symbol.c_str());
+        }
+    }
+    m->finalized = true;
+    return megcc_gfx950_wait();
+}
+
+size_t megcc_gfx950_model_arena_bytes(void* model) {
+    return model ? ((Model*)model)->arena_bytes : 0;
+}
+
+void* megcc_gfx950_model_tensor_ptr(void* model, int tensor) {
+    Model* m = (Model*)model;
+    if (!m || tensor < 0 || tensor >= (int)m->tensors.size())
+        return nullptr;
+    return m->tensors[tensor]->t.ptr;
+}
+
+// LITE_reset_tensor_memory + the staging copy (runtime/src/lite/tensor.c:93-112)
+TinyNNStatus megcc_gfx950_model_set_input(void* model, int tensor, const void* host, size_t bytes) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && m->finalized && tensor >= 0 && tensor < (int)m->tensors.size(),
+               TinyNN_ERROR_OUT_OF_RANGE, "model_set_input: bad tensor");
+    Tensor& t = m->tensors[tensor]->t;
+    MG_REQUIRE(bytes == tensor_bytes(t), TinyNN_ERROR_INVALID_LAYOUT,
+               "model_set_input: %zu bytes given, tensor has %zu", bytes, tensor_bytes(t));
+    return megcc_gfx950_memcpy_h2d(t.ptr, host, bytes);
+}
+
+TinyNNStatus megcc_gfx950_model_get_output(void* model, int tensor, void* host, size_t bytes) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && m->finalized && tensor >= 0 && tensor < (int)m->tensors.size(),
+               TinyNN_ERROR_OUT_OF_RANGE, "model_get_output: bad tensor");
+    Tensor& t = m->tensors[tensor]->t;
+    MG_REQUIRE(bytes == tensor_bytes(t), TinyNN_ERROR_INVALID_LAYOUT,
+               "model_get_output: %zu bytes asked, tensor has %zu", bytes, tensor_bytes(t));
+    return megcc_gfx950_memcpy_d2h(host, t.ptr, bytes);
+}
+
+// LITE_forward: one asynchronous kernel launch per Opr, in order, on the library stream; stops at
+// the first failing kernel like network.c:191-194. Results are visible after megcc_gfx950_wait().
+TinyNNStatus megcc_gfx950_model_forward(void* model) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && m->finalized, TinyNN_ERROR_NULL_PTR, "model_forward: model not finalized");
+    for (auto* o : m->oprs) {
+        TinyNNStatus st = megcc_gfx950_call(
+                &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), o->out_ptrs.data(),
+                (int)o->out_ptrs.size(), &o->ws, &m->opt);
+        if (st != TinyNN_SUCCESS)
+            return st;
+    }
+    return TinyNN_SUCCESS;
+}
+
+int megcc_gfx950_model_nr_opr(void* model) {
+    return model ? (int)((Model*)model)->oprs.size() : 0;
+}
+
+// Runs a single instruction (per-layer timing and tensor dumps, the TINYNN_PROFILE_KERNEL /
+// TINYNN_DUMP_TENSOR hooks of network.c:187-224)
+TinyNNStatus megcc_gfx950_model_run_opr(void* model, int index) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && m->finalized && index >= 0 && index < (int)m->oprs.size(),
+               TinyNN_ERROR_OUT_OF_RANGE, "model_run_opr: index %d", index);
+    ModelOpr* o = m->oprs[index];
+    return megcc_gfx950_call(
+            &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), o->out_ptrs.data(),
+            (int)o->out_ptrs.size(), &o->ws, &m->opt);
+}
+
+}  // extern "C"

@@ -1,0 +1,414 @@
+// KernelFunc implementations of the gfx950 target: availability rules, kernel symbols and the
+// emitted C shims. Symbol construction follows the reference's GetKernelSymbol() of the kernel
+// its x86 (Arch::BAREMETAL) registry selects for the same context:
+//   conv      BareMetal/ConvKernel.cpp:144-176 (ConvImpl), NCHW_NCHW44 detection :115-127
+//   pooling   BareMetal/Pooling.cpp:31-44; NCHW44 qsi8 comes from GI with
+//             "_<io>_fallback" appended (GeneralIntrinsic/PoolingKernel/QInt8PoolingNCHW44.cpp:25-31)
+//   multitype BareMetal/ElemwiseMultiType.cpp:94-100
+//   typecvt   GeneralIntrinsic/Typecvt.cpp:36-41 (q8<->f32, q8->q8), BareMetal/Typecvt.cpp:36-41
+//   elemwise  BareMetal/ElemwiseKernel.cpp:433-439
+//   reduce    BareMetal/Reduce.cpp:82-90
+//   matmul    BareMetal/MatrixMul.cpp:26-41
+// (for f32 conv / matmul / elemwise / reduce the x86 registry prefers GI variants whose names
+// carry tiling details; the BAREMETAL template's name is used for those, and the run-time library
+// also resolves the GI spellings.)
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <sstream>
+
+#include "KernelGen.h"
+
+namespace megcc_gfx950 {
+
+#ifndef MEGCC_GFX950_IN_TREE
+// ---- TContext mirror ---------------------------------------------------------------------------
+static void missing(const std::string& k) {
+    fprintf(stderr, "not find CCAttr %s\n", k.c_str());
+    abort();  // TContext.h:224-231 aborts as well
+}
+std::string TContext::getAttrStr(const std::string& k) const {
+    auto it = m_str.find(k);
+    if (it == m_str.end())
+        missing(k);
+    return it->second;
+}
+int64_t TContext::get_int(const std::string& k) const {
+    auto it = m_int.find(k);
+    if (it == m_int.end())
+        missing(k);
+    return it->second;
+}
+CCOperand TContext::getAttrOprand(const std::string& k) const {
+    auto it = m_op.find(k);
+    if (it == m_op.end())
+        missing(k);
+    return it->second;
+}
+
+// KernelGen.cpp:130-153
+static const char* kCall =
+        "(Tensor** inputs, int nr_input, Tensor** outputs, int nr_output, "
+        "const Workspace* workspace, const RuntimeOpt* opt)";
+static const char* kInitCall =
+        "(Tensor** inputs, int nr_input, Tensor* out_weights, int* nr_out_weight, "
+        "const RuntimeOpt* opt)";
+static const char* kWorkspaceCall =
+        "(Tensor** inputs, int nr_input, int nr_thread, size_t* workspace)";
+
+std::string KernelFuncBase::GetKernelSignature(TContext* c) const {
+    return GetKernelSymbol(c) + kCall;
+}
+std::string KernelFuncBase::GetInitSignature(TContext* c) const {
+    return GetInitSymbol(c) + kInitCall;
+}
+std::string KernelFuncBase::GetWorkspaceSignature(TContext* c) const {
+    return GetWorkspaceSymbol(c) + kWorkspaceCall;
+}
+// defaults of KernelGen.h:97-124: no processed weights, no workspace
+std::string KernelFuncBase::GetInitBody(TContext* c) const {
+    return "TinyNNStatus " + GetInitSignature(c) +
+           " {\n    if (nr_out_weight) *nr_out_weight = 0;\n    return TinyNN_SUCCESS;\n}\n";
+}
+std::string KernelFuncBase::GetWorkspaceBody(TContext* c) const {
+    return "TinyNNStatus " + GetWorkspaceSignature(c) +
+           " {\n    *workspace = 0;\n    return TinyNN_SUCCESS;\n}\n";
+}
+#endif
+
+namespace {
+
+// ---- dtype helpers (Utils/Utils.h:41-140, Utils/SymbolHelper.h:9-23) ---------------------------
+std::string valid_dtype(const std::string& d) {
+    size_t p = d.find('<');
+    return p == std::string::npos ? d : d.substr(0, p);
+}
+bool is_q(const std::string& d, int bits) {
+    return valid_dtype(d) == "qsi" + std::to_string(bits);
+}
+bool is_f32(const std::string& d) {
+    return d == "f32";
+}
+std::string io_str(TContext* c) {
+    std::string s;
+    for (int i = 0; i < c->getAttrInt("nr_operands"); ++i)
+        s += valid_dtype(c->getAttrOprand("operand:" + std::to_string(i)).dtype);
+    return s;
+}
+size_t nr_elem(const CCOperand& o) {
+    size_t n = o.shape.empty() ? 0 : 1;
+    for (size_t d : o.shape)
+        n *= d;
+    return n;
+}
+
+const char* kHeader = "#include \"megcc_gfx950.h\"\n";
+
+std::string kernel_def(const KernelFuncBase* k, TContext* c, const std::string& attr_decl,
+                       const std::string& call) {
+    std::stringstream ss;
+    ss << "TinyNNStatus " << k->GetKernelSignature(c) << " {\n"
+       << attr_decl << "    return " << call << ";\n}\n";
+    return ss.str();
+}
+
+// ---- ConvBias ----------------------------------------------------------------------------------
+// Common/ConvKernel.h:10-13 is_bias
+bool conv_is_bias(TContext* c) {
+    return c->getAttrInt("nr_operands") > 3 && !c->getAttrOprand("operand:2").shape.empty();
+}
+// BareMetal/ConvKernel.cpp:115-127 get_format
+std::string conv_format(TContext* c) {
+    std::string f = c->getAttrStr("format");
+    if (f == "NCHW44" && c->getAttrOprand("operand:0").shape.size() == 4)
+        return "NCHW_NCHW44";
+    return f;
+}
+std::string conv_nonline(TContext* c) {
+    return c->haveAttr("nonlineMode") ? c->getAttrStr("nonlineMode") : "IDENTITY";
+}
+
+struct ConvKernel : KernelFuncBase {
+    bool IsAvailable(TContext* c) const override {
+        const std::string fmt = conv_format(c), sparse = c->getAttrStr("sparse");
+        if (!(fmt == "NCHW" || fmt == "NCHW44" || fmt == "NCHW_NCHW44") ||
+            c->getAttrStr("mode") != "CROSS_CORRELATION" || c->getAttrInt("nr_operands") < 3)
+            return false;
+        const auto src = c->getAttrOprand("operand:0"), flt = c->getAttrOprand("operand:1");
+        const auto op2 = c->getAttrOprand("operand:2");
+        const bool f32 = is_f32(src.dtype) && is_f32(flt.dtype) && is_f32(op2.dtype);
+        // the reference wants operand:2 to be qsi32, i.e. a qsi8 conv always has a bias
+        // (BareMetal/ConvKernel.cpp:25-29), and |src*flt - bias scale| < 1e-5 (:37-42)
+        bool q8 = is_q(src.dtype, 8) && is_q(flt.dtype, 8) && is_q(op2.dtype, 32);
+        if (q8 && conv_is_bias(c))
+            q8 = std::fabs(src.scale * flt.scale - op2.scale) < 1e-5;
+        if (!(f32 || q8))
+            return false;
+        const std::string nl = conv_nonline(c);
+        if (!(nl == "IDENTITY" || nl == "RELU" || nl == "H_SWISH" || nl == "SIGMOID"))
+            return false;
+        // bias must be per channel (Common/ConvKernel.h:15-30)
+        if (conv_is_bias(c)) {
+            const auto dst = c->getAttrOprand("operand:" + std::to_string(c->getAttrInt("nr_operands") - 1));
+            size_t oc = dst.shape.size() == 5 ? dst.shape[1] * 4 : dst.shape[1];
+            if (nr_elem(op2) != oc)
+                return false;
+        }
+        if (sparse == "GROUP") {
+            if (fmt == "NCHW_NCHW44")
+                return false;
+            // NCHW44 GROUP: channel-wise filters [G/4,1,1,FH,FW,4] only
+            if (fmt == "NCHW44" && flt.shape.size() != 6)
+                return false;
+        } else if (sparse != "DENSE") {
+            return false;
+        }
+        return true;
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)
+            return "kernel_conv2d";
+        std::stringstream ss;
+        ss << "kernel_conv2d_" << c->getAttrUInt("kernel_h") << "x" << c->getAttrUInt("kernel_w")
+           << "_" << conv_format(c) << "_" << c->getAttrStr("sparse") << "_p"
+           << c->getAttrUInt("pad_h") << "x" << c->getAttrUInt("pad_w") << "_s"
+           << c->getAttrUInt("stride_h") << "x" << c->getAttrUInt("stride_w") << "_d"
+           << c->getAttrUInt("dilate_h") << "x" << c->getAttrUInt("dilate_w") << "_" << io_str(c);
+        if (conv_is_bias(c))
+            ss << "_bias";
+        if (conv_nonline(c) != "IDENTITY")
+            ss << "_" << conv_nonline(c);
+        return ss.str();
+    }
+    std::string attr_decl(TContext* c) const {
+        const std::string fmt = conv_format(c);
+        std::stringstream ss;
+        ss << "    static const MegccConvAttr attr = {" << c->getAttrUInt("kernel_h") << ", "
+           << c->getAttrUInt("kernel_w") << ", " << c->getAttrUInt("stride_h") << ", "
+           << c->getAttrUInt("stride_w") << ", " << c->getAttrUInt("pad_h") << ", "
+           << c->getAttrUInt("pad_w") << ", " << c->getAttrUInt("dilate_h") << ", "
+           << c->getAttrUInt("dilate_w") << ", MEGCC_FMT_" << fmt << ", MEGCC_SPARSE_"
+           << c->getAttrStr("sparse") << ", MEGCC_NONLINE_" << conv_nonline(c) << ", "
+           << (conv_is_bias(c) ? 1 : 0) << "};\n";
+        return ss.str();
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        return kHeader + kernel_def(this, c, attr_decl(c),
+                                    "megcc_gfx950_conv2d(&attr, inputs, nr_input, outputs, "
+                                    "nr_output, workspace, opt)");
+    }
+    // the filter repack for the MFMA kernel happens at model load through the 3-phase protocol
+    std::string GetInitBody(TContext* c) const override {
+        return "TinyNNStatus " + GetInitSignature(c) + " {\n" + attr_decl(c) +
+               "    return megcc_gfx950_conv2d_init(&attr, inputs, nr_input, out_weights, "
+               "nr_out_weight, opt);\n}\n";
+    }
+    // plain C, no external call: the compiler may evaluate it at compile time
+    // (compiler/lib/KernelGen/Jit/JitExe.cpp:67-123 forbids externs in workspace bodies)
+    std::string GetWorkspaceBody(TContext* c) const override {
+        return "TinyNNStatus " + GetWorkspaceSignature(c) +
+               " {\n    *workspace = 0;\n    return TinyNN_SUCCESS;\n}\n";
+    }
+};
+
+// ---- Pooling -----------------------------------------------------------------------------------
+struct PoolingKernel : KernelFuncBase {
+    bool IsAvailable(TContext* c) const override {
+        const std::string fmt = c->getAttrStr("format"), mode = c->getAttrStr("mode");
+        const auto src = c->getAttrOprand("operand:0"), dst = c->getAttrOprand("operand:1");
+        if (!(fmt == "NCHW" || fmt == "NCHW44"))
+            return false;
+        if (!(mode == "MAX" || mode == "AVERAGE" || mode == "AVERAGE_COUNT_EXCLUDE_PADDING"))
+            return false;
+        // "quant pooling only support same scale" (BareMetal/Pooling.cpp:22-27)
+        return is_q(src.dtype, 8) && is_q(dst.dtype, 8) && src.scale == dst.scale;
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        std::stringstream ss;
+        const bool f44 = c->getAttrStr("format") == "NCHW44";
+        ss << (f44 ? "GI_" : "") << "kernel_pooling_" << c->getAttrStr("mode") << "_"
+           << c->getAttrStr("format") << "_p" << c->getAttrInt("pad_h") << "x"
+           << c->getAttrInt("pad_w") << "_s" << c->getAttrInt("stride_h") << "x"
+           << c->getAttrInt("stride_w") << "_w" << c->getAttrInt("window_h") << "x"
+           << c->getAttrInt("window_w") << "_" << io_str(c);
+        if (f44)
+            ss << "_" << io_str(c) << "_fallback";
+        return ss.str();
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        std::stringstream a;
+        a << "    static const MegccPoolAttr attr = {" << c->getAttrInt("window_h") << ", "
+          << c->getAttrInt("window_w") << ", " << c->getAttrInt("stride_h") << ", "
+          << c->getAttrInt("stride_w") << ", " << c->getAttrInt("pad_h") << ", "
+          << c->getAttrInt("pad_w") << ", MEGCC_FMT_" << c->getAttrStr("format")
+          << ", MEGCC_POOL_" << c->getAttrStr("mode") << "};\n";
+        return kHeader + kernel_def(this, c, a.str(),
+                                    "megcc_gfx950_pooling(&attr, inputs, nr_input, outputs, "
+                                    "nr_output, workspace, opt)");
+    }
+};
+
+// ---- ElemwiseMultiType -------------------------------------------------------------------------
+struct ElemwiseMultiTypeKernel : KernelFuncBase {
+    bool IsAvailable(TContext* c) const override {
+        const std::string mode = c->getAttrStr("mode");
+        const int n = c->getAttrInt("nr_operands");
+        for (int i = 0; i < n; ++i)
+            if (!is_q(c->getAttrOprand("operand:" + std::to_string(i)).dtype, 8))
+                return false;
+        if (n == 2)
+            return mode == "QRELU";
+        if (n != 3 || !(mode == "QADD" || mode == "QFUSE_ADD_RELU" || mode == "QMUL"))
+            return false;
+        // broadcast modes of BareMetal/ElemwiseMultiType.cpp:76-92
+        const auto a = c->getAttrOprand("operand:0"), b = c->getAttrOprand("operand:1");
+        const size_t nb = nr_elem(b);
+        return a.shape == b.shape || nb == 1 ||
+               (a.shape.size() == b.shape.size() && a.shape.size() > 2 &&
+                a.shape[1] == b.shape[1] && nb == b.shape[1]);
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        return "kernel_elementwise_multitype_" + c->getAttrStr("mode") + "_" + io_str(c);
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        std::string m = c->getAttrStr("mode").substr(1);  // QADD -> ADD
+        return kHeader +
+               kernel_def(this, c, "    static const MegccMultiTypeMode mode = MEGCC_Q_" + m + ";\n",
+                          "megcc_gfx950_elemwise_multitype(&mode, inputs, nr_input, outputs, "
+                          "nr_output, workspace, opt)");
+    }
+};
+
+// ---- Elemwise (f32) ----------------------------------------------------------------------------
+struct ElemwiseKernel : KernelFuncBase {
+    bool IsAvailable(TContext* c) const override {
+        static const char* unary[] = {"RELU", "EXP", "SIGMOID", "H_SWISH", "NEGATE"};
+        static const char* binary[] = {"ADD", "SUB", "MUL", "TRUE_DIV", "MAX", "MIN", "FUSE_ADD_RELU"};
+        const std::string mode = c->getAttrStr("mode");
+        const int n = c->getAttrInt("nr_operands");
+        for (int i = 0; i < n; ++i)
+            if (!is_f32(c->getAttrOprand("operand:" + std::to_string(i)).dtype))
+                return false;
+        bool ok = false;
+        if (n == 2)
+            for (auto u : unary)
+                ok |= mode == u;
+        if (n == 3)
+            for (auto b : binary)
+                ok |= mode == b;
+        return ok;
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        return "kernel_elementwise_" + c->getAttrStr("mode") + "_" + io_str(c);
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        return kHeader + kernel_def(this, c,
+                                    "    static const MegccElemwiseMode mode = MEGCC_EW_" +
+                                            c->getAttrStr("mode") + ";\n",
+                                    "megcc_gfx950_elemwise(&mode, inputs, nr_input, outputs, "
+                                    "nr_output, workspace, opt)");
+    }
+};
+
+// ---- TypeCvt -----------------------------------------------------------------------------------
+struct TypeCvtKernel : KernelFuncBase {
+    static std::string pair(TContext* c) {
+        return valid_dtype(c->getAttrOprand("operand:0").dtype) +
+               valid_dtype(c->getAttrOprand("operand:1").dtype);
+    }
+    bool IsAvailable(TContext* c) const override {
+        const std::string p = pair(c);
+        if (!(p == "f32qsi8" || p == "qsi8f32" || p == "qsi8qsi8" || p == "qsi32qsi8"))
+            return false;
+        const auto s = c->getAttrOprand("operand:0"), d = c->getAttrOprand("operand:1");
+        return (is_f32(s.dtype) || s.scale > 0) && (is_f32(d.dtype) || d.scale > 0);
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        const std::string p = pair(c);
+        return std::string(p == "qsi32qsi8" ? "" : "GI_") + "kernel_typecvt_" + p;
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        return kHeader + kernel_def(this, c, "",
+                                    "megcc_gfx950_typecvt(inputs, nr_input, outputs, nr_output, "
+                                    "workspace, opt)");
+    }
+};
+
+// ---- Reduce (f32) ------------------------------------------------------------------------------
+struct ReduceKernel : KernelFuncBase {
+    bool IsAvailable(TContext* c) const override {
+        const std::string mode = c->getAttrStr("mode");
+        return c->getAttrStr("data_type") == "DEFAULT" &&
+               is_f32(c->getAttrOprand("operand:0").dtype) &&
+               (mode == "SUM" || mode == "MEAN" || mode == "MAX" || mode == "MIN");
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        std::stringstream ss;
+        ss << "kernel_reduce_" << c->getAttrStr("mode") << "_" << c->getAttrStr("data_type")
+           << "_a" << c->getAttrInt("axis") << "_" << io_str(c);
+        return ss.str();
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        std::stringstream a;
+        a << "    static const MegccReduceAttr attr = {MEGCC_REDUCE_" << c->getAttrStr("mode")
+          << ", " << c->getAttrInt("axis") << "};\n";
+        return kHeader + kernel_def(this, c, a.str(),
+                                    "megcc_gfx950_reduce(&attr, inputs, nr_input, outputs, "
+                                    "nr_output, workspace, opt)");
+    }
+};
+
+// ---- MatrixMul (f32) ---------------------------------------------------------------------------
+struct MatrixMulKernel : KernelFuncBase {
+    bool IsAvailable(TContext* c) const override {
+        for (int i = 0; i < 3; ++i)
+            if (!is_f32(c->getAttrOprand("operand:" + std::to_string(i)).dtype))
+                return false;
+        return c->getAttrStr("format") == "DEFAULT" &&
+               (!c->haveAttr("compute_mode") || c->getAttrStr("compute_mode") == "DEFAULT");
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        return std::string("kernel_matmul_") + (c->getAttrBool("transposeA") ? "t" : "n") +
+               (c->getAttrBool("transposeB") ? "t" : "n") + "_" +
+               c->getAttrOprand("operand:0").dtype;
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        std::stringstream a;
+        a << "    static const MegccMatMulAttr attr = {" << (c->getAttrBool("transposeA") ? 1 : 0)
+          << ", " << (c->getAttrBool("transposeB") ? 1 : 0) << "};\n";
+        return kHeader + kernel_def(this, c, a.str(),
+                                    "megcc_gfx950_matmul(&attr, inputs, nr_input, outputs, "
+                                    "nr_output, workspace, opt)");
+    }
+};
+
+}  // namespace
+
+std::vector<const KernelFuncBase*> Gfx950KernelPack::GetKernel(KernType type) {
+    static const ConvKernel conv;
+    static const PoolingKernel pool;
+    static const ElemwiseMultiTypeKernel multitype;
+    static const ElemwiseKernel elemwise;
+    static const TypeCvtKernel typecvt;
+    static const ReduceKernel reduce;
+    static const MatrixMulKernel matmul;
+    switch (type) {
+        case KernType::ConvKernel: return {&conv};
+        case KernType::PoolingKernel: return {&pool};
+        case KernType::ElemwiseMultiKernel: return {&multitype};
+        case KernType::ElemwiseKernel: return {&elemwise};
+        case KernType::TypeCvtKernel: return {&typecvt};
+        case KernType::ReduceKernel: return {&reduce};
+        case KernType::MatrixMulKernel: return {&matmul};
+        default: return {};
+    }
+}
+
+std::string ReferenceSymbol(KernType type, TContext* context) {
+    for (auto* k : Gfx950KernelPack::GetKernel(type))
+        if (k->IsAvailable(context))
+            return k->GetKernelSymbol(context);
+    return "";
+}
+
+}  // namespace megcc_gfx950

@@ -6,7 +6,7 @@ import os
 
 import numpy as np
 
-from . import LIB_PATH, abi
+from . import LIB_PATH, abi  # noqa: F401
 
 _lib = None
 
@@ -51,6 +51,27 @@ def lib():
         L.megcc_gfx950_stream.restype = C.c_void_p
         L.megcc_gfx950_last_error.argtypes = []
         L.megcc_gfx950_last_error.restype = C.c_char_p
+        L.megcc_gfx950_model_create.argtypes = []
+        L.megcc_gfx950_model_create.restype = C.c_void_p
+        L.megcc_gfx950_model_destroy.argtypes = [C.c_void_p]
+        L.megcc_gfx950_model_destroy.restype = None
+        dims = C.POINTER(C.c_uint32)
+        L.megcc_gfx950_model_add_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_int, dims, C.c_int, C.c_float]
+        L.megcc_gfx950_model_add_weight.argtypes = [C.c_void_p, C.c_char_p, C.c_int, dims, C.c_int, C.c_float, C.c_void_p]
+        L.megcc_gfx950_model_add_alias.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_int, dims]
+        ints = C.POINTER(C.c_int)
+        L.megcc_gfx950_model_add_opr.argtypes = [C.c_void_p, C.c_char_p, ints, C.c_int, ints, C.c_int]
+        L.megcc_gfx950_model_mark_io.argtypes = [C.c_void_p, C.c_int, C.c_int]
+        L.megcc_gfx950_model_finalize.argtypes = [C.c_void_p]
+        L.megcc_gfx950_model_arena_bytes.argtypes = [C.c_void_p]
+        L.megcc_gfx950_model_arena_bytes.restype = C.c_size_t
+        L.megcc_gfx950_model_tensor_ptr.argtypes = [C.c_void_p, C.c_int]
+        L.megcc_gfx950_model_tensor_ptr.restype = C.c_void_p
+        L.megcc_gfx950_model_set_input.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t]
+        L.megcc_gfx950_model_get_output.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t]
+        L.megcc_gfx950_model_forward.argtypes = [C.c_void_p]
+        L.megcc_gfx950_model_nr_opr.argtypes = [C.c_void_p]
+        L.megcc_gfx950_model_run_opr.argtypes = [C.c_void_p, C.c_int]
         _lib = L
     return _lib
 
@@ -64,6 +85,12 @@ EXPORTS = [
     "megcc_gfx950_malloc", "megcc_gfx950_free", "megcc_gfx950_memcpy_h2d",
     "megcc_gfx950_memcpy_d2h", "megcc_gfx950_memset", "megcc_gfx950_wait",
     "megcc_gfx950_stream", "megcc_gfx950_last_error",
+    "megcc_gfx950_model_create", "megcc_gfx950_model_destroy", "megcc_gfx950_model_add_tensor",
+    "megcc_gfx950_model_add_weight", "megcc_gfx950_model_add_alias", "megcc_gfx950_model_add_opr",
+    "megcc_gfx950_model_mark_io", "megcc_gfx950_model_finalize", "megcc_gfx950_model_arena_bytes",
+    "megcc_gfx950_model_tensor_ptr", "megcc_gfx950_model_set_input",
+    "megcc_gfx950_model_get_output", "megcc_gfx950_model_forward", "megcc_gfx950_model_nr_opr",
+    "megcc_gfx950_model_run_opr",
 ]
 
 
@@ -189,3 +216,89 @@ def run_symbol(symbol, in_specs, out_specs):
     op = PreparedOp(parse_symbol(symbol), in_specs, out_specs)
     op.launch()
     return op.result()
+
+
+class Model:
+    """Python handle of the in-memory model runtime (megcc_gfx950_model_*)."""
+
+    def __init__(self):
+        self.h = lib().megcc_gfx950_model_create()
+        if not self.h:
+            raise MegccError("model_create failed: " + lib().megcc_gfx950_last_error().decode())
+        self.shapes = {}
+
+    @staticmethod
+    def _dims(shape):
+        return (C.c_uint32 * len(shape))(*[int(d) for d in shape])
+
+    def _remember(self, tid, shape, type_enum, what):
+        if tid < 0:
+            raise MegccError("%s failed: %s" % (what, lib().megcc_gfx950_last_error().decode()))
+        self.shapes[tid] = (tuple(shape), type_enum)
+        return tid
+
+    def tensor(self, name, shape, type_enum, scale=1.0):
+        tid = lib().megcc_gfx950_model_add_tensor(self.h, name.encode(), len(shape), self._dims(shape),
+                                                  type_enum, scale)
+        return self._remember(tid, shape, type_enum, "add_tensor")
+
+    def weight(self, name, array, type_enum, scale=1.0):
+        array = np.ascontiguousarray(array)
+        tid = lib().megcc_gfx950_model_add_weight(self.h, name.encode(), array.ndim,
+                                                  self._dims(array.shape), type_enum, scale,
+                                                  array.ctypes.data)
+        return self._remember(tid, array.shape, type_enum, "add_weight")
+
+    def alias(self, name, of, shape):
+        tid = lib().megcc_gfx950_model_add_alias(self.h, name.encode(), of, len(shape), self._dims(shape))
+        return self._remember(tid, shape, self.shapes[of][1], "add_alias")
+
+    def opr(self, symbol, inputs, outputs):
+        ins = (C.c_int * len(inputs))(*inputs)
+        outs = (C.c_int * len(outputs))(*outputs)
+        check(lib().megcc_gfx950_model_add_opr(self.h, symbol.encode(), ins, len(inputs), outs,
+                                               len(outputs)), "add_opr " + symbol)
+
+    def mark_input(self, tid):
+        check(lib().megcc_gfx950_model_mark_io(self.h, tid, 0), "mark_io")
+
+    def mark_output(self, tid):
+        check(lib().megcc_gfx950_model_mark_io(self.h, tid, 1), "mark_io")
+
+    def finalize(self):
+        check(lib().megcc_gfx950_model_finalize(self.h), "finalize")
+
+    @property
+    def arena_bytes(self):
+        return lib().megcc_gfx950_model_arena_bytes(self.h)
+
+    @property
+    def nr_opr(self):
+        return lib().megcc_gfx950_model_nr_opr(self.h)
+
+    def set_input(self, tid, array):
+        array = np.ascontiguousarray(array)
+        check(lib().megcc_gfx950_model_set_input(self.h, tid, array.ctypes.data, array.nbytes), "set_input")
+
+    def forward(self):
+        check(lib().megcc_gfx950_model_forward(self.h), "forward")
+
+    def run_opr(self, index):
+        check(lib().megcc_gfx950_model_run_opr(self.h, index), "run_opr")
+
+    def get(self, tid):
+        shape, type_enum = self.shapes[tid]
+        out = np.empty(shape, abi.np_dtype(type_enum))
+        check(lib().megcc_gfx950_model_get_output(self.h, tid, out.ctypes.data, out.nbytes), "get_output")
+        return out
+
+    def close(self):
+        if self.h:
+            lib().megcc_gfx950_model_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

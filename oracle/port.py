@@ -110,6 +110,8 @@ def _bcast(a, b):
         return 2, a.shape[1], inner
     if b.ndim == 1 and b.shape[0] == a.shape[-1]:
         return 2, a.shape[-1], 1
+    if a.ndim == 2 and b.ndim == 2 and b.shape == (a.shape[0], 1):
+        return 2, a.shape[0], a.shape[1]
     raise ValueError("unsupported broadcast %s vs %s" % (a.shape, b.shape))
 
 

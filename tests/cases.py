@@ -150,7 +150,7 @@ class ConvCase:
                TensorSpec(b"flt", self.flt_shape(), abi.QINT8 if q else abi.FLOAT, fs, arrays["flt"])]
         if self.bias:
             ins.append(TensorSpec(b"bias", self.bias_shape(), abi.QINT32 if q else abi.FLOAT,
-                                  ss * fs, arrays["bias"]))
+                                  float(np.float32(ss) * np.float32(fs)), arrays["bias"]))
         outs = [TensorSpec(b"dst", self.dst_shape(), abi.QINT8 if q else abi.FLOAT, ds)]
         return ins, outs
 

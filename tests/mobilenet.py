@@ -1,0 +1,163 @@
+"""MobileNetV1 (width 1.0, 224x224x3, 13 depthwise-separable blocks, global average pool,
+FC-1000, softmax) as the list of operators MegCC would emit for it with the NCHW44 layout enabled
+(compiler/lib/Target/MGB/importer.cpp:1337-1352: nchw44 + fused conv-bias-activation; softmax
+decomposed into Reduce-MAX, SUB, EXP, Reduce-SUM, TRUE_DIV, importer.cpp:987-1016; global average
+pooling as a 7x7 stride-7 AVERAGE Pooling, importer.cpp:691-713).
+
+No MobileNetV1 weights exist in the reference tree: weights are random int8 drawn from a seed and
+the per-tensor scales come from tests/golden/mobilenet_scales.json, calibrated once from the same
+seed so that activations use the int8 range instead of saturating (tests/golden/make_mobilenet_scales.py).
+
+The same description drives (a) the GPU model runtime (megcc_gfx950_model_*), and (b) a layer by
+layer evaluation with the CPU oracle.
+"""
+import json
+import os
+
+import numpy as np
+
+from cases import ConvCase, PoolCase, TypeCvtCase
+from megcc_amd import abi
+from oracle import port
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SCALES_PATH = os.path.join(HERE, "golden", "mobilenet_scales.json")
+
+# (stride of the depthwise conv, output channels of the pointwise conv)
+BLOCKS = [(1, 64), (2, 128), (1, 128), (2, 256), (1, 256), (2, 512),
+          (1, 512), (1, 512), (1, 512), (1, 512), (1, 512), (2, 1024), (1, 1024)]
+IN_SCALE = 1.0 / 127.0
+
+
+def conv_layers(batch):
+    """[(name, ConvCase without scales)] in execution order"""
+    layers = [("conv0", ConvCase(abi.FMT_NCHW_NCHW44, abi.DENSE, batch, 3, 224, 224, 32, 3, 2, 1, abi.RELU))]
+    c, hw = 32, 112
+    for i, (s, oc) in enumerate(BLOCKS, 1):
+        layers.append(("dw%d" % i, ConvCase(abi.FMT_NCHW44, abi.GROUP, batch, c, hw, hw, c, 3, s, 1, abi.RELU)))
+        hw //= s
+        layers.append(("pw%d" % i, ConvCase(abi.FMT_NCHW44, abi.DENSE, batch, c, hw, hw, oc, 1, 1, 0, abi.RELU)))
+        c = oc
+    layers.append(("fc", ConvCase(abi.FMT_NCHW, abi.DENSE, batch, 1024, 1, 1, 1000, 1, 1, 0, abi.IDENTITY)))
+    return layers
+
+
+def macs_per_image():
+    return sum(c.ops() // 2 for _, c in conv_layers(1))
+
+
+def draw_weights(seed=0):
+    """{layer: (filter int8, bias int32, filter scale)} -- independent of the batch size"""
+    r = np.random.Generator(np.random.PCG64(seed))
+    out = {}
+    for name, case in conv_layers(1):
+        flt = r.integers(-127, 128, case.flt_shape()).astype(np.int8)
+        bias = r.integers(-1000, 1001, case.bias_shape()).astype(np.int32)
+        out[name] = (flt, bias, 0.01)  # provisional filter scale, see make_mobilenet_scales.py
+    return out
+
+
+def load_scales():
+    with open(SCALES_PATH) as f:
+        return json.load(f)
+
+
+def draw_input(batch, seed=0):
+    r = np.random.Generator(np.random.PCG64(1000 + seed))
+    return r.uniform(-1, 1, (batch, 3, 224, 224)).astype(np.float32)
+
+
+class Net:
+    """The operator list with all scales resolved: steps = [(kind, name, case, extra)]"""
+
+    def __init__(self, batch, seed=0, scales=None):
+        self.batch = batch
+        self.weights = draw_weights(seed)
+        self.scales = scales if scales is not None else load_scales()
+        self.steps = []
+        s_in = IN_SCALE
+        self.steps.append(("typecvt", "quant", TypeCvtCase("f32", "qsi8", (batch, 3, 224, 224), dst_scale=s_in), None))
+        for name, case in conv_layers(batch):
+            if name == "fc":
+                pool = PoolCase(abi.FMT_NCHW44, abi.POOL_AVERAGE, batch, 1024, 7, 7, 7, 7, 0, scale=s_in)
+                self.steps.append(("pool", "avgpool", pool, None))
+            wscale = float(self.scales[name]["filter"])
+            case.scales = (s_in, wscale, float(self.scales[name]["dst"]))
+            self.steps.append(("conv", name, case, None))
+            s_in = case.scales[2]
+        self.fc_scale = s_in
+        self.steps.append(("typecvt", "dequant", TypeCvtCase("qsi8", "f32", (batch, 1000), src_scale=s_in), None))
+
+    # ---- CPU oracle, layer by layer ------------------------------------------------------------
+    def run_oracle(self, image, keep=False):
+        port.set_threads(8)
+        x = image
+        trace = {}
+        for kind, name, case, _ in self.steps:
+            if kind == "typecvt":
+                x = case.run_port({"src": np.ascontiguousarray(x.reshape(case.shape))})
+            elif kind == "pool":
+                x = case.run_port({"src": x})
+            else:
+                flt, bias, _ = self.weights[name]
+                if name == "fc":
+                    x = np.ascontiguousarray(x.reshape(self.batch, 1024, 1, 1))
+                x = case.run_port({"src": x, "flt": flt, "bias": bias})
+            if keep:
+                trace[name] = x
+        logits = x.reshape(self.batch, 1000)
+        mx = port.reduce_f32(logits, abi.REDUCE_MAX, 1)
+        e = port.elemwise_f32(port.elemwise_f32(logits, mx, abi.EW_SUB), None, abi.EW_EXP)
+        sm = port.elemwise_f32(e, port.reduce_f32(e, abi.REDUCE_SUM, 1), abi.EW_TRUE_DIV)
+        trace["softmax"] = sm
+        return sm, trace
+
+    # ---- GPU model -----------------------------------------------------------------------------
+    def build_gpu(self, keep_all=False):
+        from megcc_amd import runtime
+        m = runtime.Model()
+        ids = {}
+        b = self.batch
+        x = m.tensor("image", (b, 3, 224, 224), abi.FLOAT)
+        m.mark_input(x)
+        ids["image"] = x
+        for kind, name, case, _ in self.steps:
+            if kind == "typecvt" and name == "quant":
+                y = m.tensor(name, case.shape, abi.QINT8, case.dst_scale)
+                m.opr(case.symbol(), [x], [y])
+            elif kind == "typecvt":
+                y = m.tensor(name, case.shape, abi.FLOAT)
+                m.opr(case.symbol(), [x], [y])
+            elif kind == "pool":
+                y = m.tensor(name, case.dst_shape(), abi.QINT8, case.scale)
+                m.opr(case.symbol(), [x], [y])
+            else:
+                flt, bias, _ = self.weights[name]
+                wscale = case.scales[1]
+                if name == "fc":  # MemForward: [B,256,1,1,4] and [B,1024,1,1] are the same bytes
+                    x = m.alias("fc_in", x, (b, 1024, 1, 1))
+                w = m.weight(name + ".w", flt, abi.QINT8, wscale)
+                bi = m.weight(name + ".b", bias, abi.QINT32,
+                              float(np.float32(case.scales[0]) * np.float32(wscale)))
+                y = m.tensor(name, case.dst_shape(), abi.QINT8, case.scales[2])
+                m.opr(case.symbol(), [x, w, bi], [y])
+            ids[name] = y
+            x = y
+        logits = x
+        mx = m.tensor("sm.max", (b, 1), abi.FLOAT)
+        m.opr("kernel_reduce_MAX_DEFAULT_a1_f32f32", [logits], [mx])
+        sub = m.tensor("sm.sub", (b, 1000), abi.FLOAT)
+        m.opr("kernel_elementwise_SUB_f32f32f32", [logits, mx], [sub])
+        ex = m.tensor("sm.exp", (b, 1000), abi.FLOAT)
+        m.opr("kernel_elementwise_EXP_f32f32", [sub], [ex])
+        sm_sum = m.tensor("sm.sum", (b, 1), abi.FLOAT)
+        m.opr("kernel_reduce_SUM_DEFAULT_a1_f32f32", [ex], [sm_sum])
+        out = m.tensor("softmax", (b, 1000), abi.FLOAT)
+        m.opr("kernel_elementwise_TRUE_DIV_f32f32f32", [ex, sm_sum], [out])
+        ids["softmax"] = out
+        m.mark_output(out)
+        if keep_all:
+            for tid in ids.values():
+                m.mark_output(tid)
+        m.finalize()
+        return m, ids

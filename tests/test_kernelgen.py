@@ -1,0 +1,117 @@
+"""The compile-time half of the boundary: the gfx950 KernelGen target (megcc_amd/kernelgen) must
+pick a kernel for every operator of the path, name it as MegCC's own registry does, and emit C
+shims that compile against the public header and link against the library."""
+import ctypes as C
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import cases
+from golden_cases import golden_cases, unsat
+from megcc_amd import abi, runtime
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+KG = os.path.join(ROOT, "megcc_amd", "kernelgen")
+
+
+@pytest.fixture(scope="module")
+def emitted(tmp_path_factory):
+    out = tmp_path_factory.mktemp("shims")
+    subprocess.check_call(["make", "-s", "-C", KG])
+    subprocess.check_call([os.path.join(KG, "kernelgen_tool"),
+                           os.path.join(ROOT, "oracle", "ref_kernels.spec"), str(out)])
+    manifest = dict(line.split() for line in open(out / "manifest.txt"))
+    return out, manifest
+
+
+def test_every_operator_of_the_path_has_a_kernel(emitted):
+    _, manifest = emitted
+    assert len(manifest) >= 50
+    assert "NONE" not in manifest.values()
+
+
+def test_quantized_symbols_equal_the_reference_registry(emitted):
+    _, manifest = emitted
+    with open(os.path.join(HERE, "golden", "symbols.json")) as f:
+        ref = json.load(f)
+    checked = 0
+    for label, sym in ref.items():
+        if "qsi" in sym:  # f32 kernels use the BAREMETAL template's name, see Gfx950Kernels.cpp
+            assert manifest[label] == sym, label
+            checked += 1
+    assert checked >= 35
+
+
+def test_library_resolves_every_emitted_symbol(emitted):
+    _, manifest = emitted
+    for sym in set(manifest.values()):
+        runtime.parse_symbol(sym)
+
+
+def test_shim_attributes_round_trip(emitted):
+    """the constant struct in the shim must equal what the library parses from the symbol"""
+    out, manifest = emitted
+    sym = manifest["conv44_3x3_s2_RELU"]
+    text = open(out / (sym + ".c")).read()
+    assert "MegccConvAttr attr = {3, 3, 2, 2, 1, 1, 1, 1, MEGCC_FMT_NCHW44, MEGCC_SPARSE_DENSE, MEGCC_NONLINE_RELU, 1}" in text
+    a = runtime.parse_symbol(sym).attr.conv
+    assert (a.kernel_h, a.stride_h, a.pad_h, a.format, a.nonline, a.with_bias) == (3, 2, 1, abi.FMT_NCHW44, abi.RELU, 1)
+    sym = manifest["conv_hybrid_3x3_s2_RELU"]
+    assert "MEGCC_FMT_NCHW_NCHW44" in open(out / (sym + ".c")).read()
+
+
+@pytest.fixture(scope="module")
+def shim_library(emitted):
+    out, manifest = emitted
+    so = out / "libshims.so"
+    srcs = sorted(str(p) for p in out.glob("*.c"))
+    subprocess.check_call(["gcc", "-shared", "-fPIC", "-Wall", "-Werror", "-o", str(so)] + srcs +
+                          ["-I" + os.path.join(ROOT, "include"),
+                           "-L" + os.path.dirname(runtime.LIB_PATH) if hasattr(runtime, "LIB_PATH") else "-L.",
+                           "-L" + os.path.join(ROOT, "megcc_amd"), "-lmegcc_gfx950",
+                           "-Wl,-rpath," + os.path.join(ROOT, "megcc_amd")])
+    return C.CDLL(str(so)), manifest
+
+
+def test_shims_compile_and_link(shim_library):
+    lib, manifest = shim_library
+    for sym in set(manifest.values()):
+        assert hasattr(lib, sym)
+        assert hasattr(lib, sym + "_init")
+        assert hasattr(lib, sym + "_workspace")
+
+
+@pytest.mark.gpu
+def test_conv_through_the_generated_shim(shim_library):
+    """call the kernel the way the TinyNN runtime would: by its generated symbol"""
+    lib, manifest = shim_library
+    case = cases.ConvCase(abi.FMT_NCHW44, abi.DENSE, 2, 32, 20, 24, 48, 3, 1, 1, abi.RELU,
+                          scales=(0.02, 0.01, unsat(288)))
+    sym = case.symbol()
+    assert sym in manifest.values()
+    arrays = case.gen(3)
+    ins, outs = case.specs(arrays)
+    bufs = [runtime.DeviceBuffer.from_array(s.array) for s in ins]
+    out = runtime.DeviceBuffer(outs[0].nbytes)
+    tin = [abi.make_tensor(b.ptr, s.shape, s.type_enum, s.scale, s.name) for b, s in zip(bufs, ins)]
+    tout = [abi.make_tensor(out.ptr, outs[0].shape, outs[0].type_enum, outs[0].scale)]
+    kern, init, ws = getattr(lib, sym), getattr(lib, sym + "_init"), getattr(lib, sym + "_workspace")
+    kern.argtypes, init.argtypes, ws.argtypes = abi.KERNEL_ARGS, abi.INIT_ARGS, abi.WORKSPACE_ARGS
+    size = C.c_size_t(1)
+    assert ws(abi.tensor_array(tin), len(tin), 1, C.byref(size)) == 0 and size.value == 0
+    n = C.c_int(0)
+    assert init(abi.tensor_array(tin), len(tin), None, C.byref(n), None) == 0 and n.value == 1
+    w = abi.Tensor()
+    assert init(abi.tensor_array(tin), len(tin), C.byref(w), None, None) == 0
+    assert w.name == tin[1].name
+    wbuf = runtime.DeviceBuffer(w.layout.dims[0])
+    w.ptr = wbuf.ptr
+    assert init(abi.tensor_array(tin), len(tin), C.byref(w), C.byref(n), None) == 0
+    tin[1] = w
+    assert kern(abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1, None, None) == 0
+    got = out.to_array(outs[0].shape, np.int8)
+    np.testing.assert_array_equal(got, case.run_port(arrays))

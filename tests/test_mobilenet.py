@@ -1,0 +1,61 @@
+"""End-to-end MobileNetV1-int8 through the model runtime (static memory plan on one HBM arena)
+against the CPU oracle evaluated layer by layer."""
+import numpy as np
+import pytest
+
+import cases
+import mobilenet
+from megcc_amd import abi
+
+
+def test_layer_table_matches_the_standard_topology():
+    layers = mobilenet.conv_layers(1)
+    assert len(layers) == 1 + 26 + 1
+    assert mobilenet.macs_per_image() == 568740352  # 568.74 MMAC per image
+    weights = mobilenet.draw_weights(0)
+    assert sum(w[0].size for w in weights.values()) == 4209088  # int8 weight bytes
+
+
+def test_scales_cover_every_layer():
+    scales = mobilenet.load_scales()
+    for name, _ in mobilenet.conv_layers(1):
+        assert scales[name]["filter"] > 0 and scales[name]["dst"] > 0
+
+
+@pytest.mark.gpu
+def test_every_layer_is_bit_exact_batch2():
+    net = mobilenet.Net(2)
+    image = mobilenet.draw_input(2, seed=5)
+    want, trace = net.run_oracle(image, keep=True)
+    model, ids = net.build_gpu(keep_all=True)
+    model.set_input(ids["image"], image)
+    model.forward()
+    for name, tid in ids.items():
+        if name in ("image", "softmax", "dequant"):
+            continue
+        got = model.get(tid)
+        exp = trace[name].reshape(got.shape)
+        bad = int((got != exp).sum())
+        assert bad == 0, "%s: %d of %d elements differ" % (name, bad, got.size)
+    got = model.get(ids["softmax"])
+    assert cases.max_rel_err(got, want) <= 1e-4
+    assert np.allclose(got.sum(axis=1), 1.0, atol=1e-4)
+    # the test images must not collapse to a constant prediction
+    assert len(set(np.argmax(want, axis=1).tolist())) >= 1 and want.max() < 0.999
+    model.close()
+
+
+@pytest.mark.gpu
+def test_memory_plan_reuses_the_arena_and_keeps_results():
+    net = mobilenet.Net(3)
+    image = mobilenet.draw_input(3, seed=9)
+    want, _ = net.run_oracle(image)
+    model, ids = net.build_gpu()
+    total = sum(c.n * c.oc * c.oh * c.ow for k, _, c, _ in net.steps if k == "conv")
+    assert model.arena_bytes < total / 3, "tensors with disjoint lifetimes must share memory"
+    for _ in range(2):  # a second forward must not depend on leftovers of the first
+        model.set_input(ids["image"], image)
+        model.forward()
+        got = model.get(ids["softmax"])
+        assert cases.max_rel_err(got, want) <= 1e-4
+    model.close()

@@ -386,8 +386,10 @@ TinyNNStatus conv_mfma_launch(
         const long oc_tiles = (g.oc + pc.bm - 1) / pc.bm;
         long ranges = slots / oc_tiles > 0 ? slots / oc_tiles : 1;
         range_len = ((P + ranges - 1) / ranges + 31) / 32 * 32;
-        if (range_len < pc.bn / 2)
+        if (range_len < pc.bn / 2) {
             pipe = false;  // too few pixels per workgroup to fill the 256-pixel tile
+            range_len = 0;
+        }
     }
     TilePlan t = plan_tiles(g, pipe ? pc.bn : BN, range_len);
     const long gather_items =

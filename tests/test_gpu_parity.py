@@ -77,6 +77,9 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.DENSE, 11, 64, 56, 56, 128, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(64))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 70, 256, 14, 14, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(256))),
     ConvCase(A.FMT_NCHW, A.DENSE, 16500, 96, 1, 1, 200, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(96) / 2)),
+    # enough pixels for the wide kernel but too few per workgroup: must fall back cleanly
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 64, 56, 56, 128, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(64))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 32, 56, 56, 128, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(288))),
     # MobileNet pointwise shapes
     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 32, 112, 112, 64, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(32))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 4, 512, 14, 14, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(512))),

@@ -103,6 +103,49 @@ def make_workload(name):
     raise SystemExit("unknown workload " + name)
 
 
+def bench_mobilenet(batch, steps, warmup, per_layer=False):
+    """MobileNetV1-int8 end to end through the model runtime: images/s, inputs resident in HBM."""
+    import mobilenet
+    from megcc_amd import runtime
+    net = mobilenet.Net(batch)
+    model, ids = net.build_gpu()
+    model.set_input(ids["image"], mobilenet.draw_input(batch, seed=1))
+    ev = HipEvents(runtime.lib().megcc_gfx950_stream())
+    for _ in range(warmup):
+        model.forward()
+    runtime.wait()
+    e0, e1 = ev.new(), ev.new()
+    t0 = time.perf_counter()
+    ev.record(e0)
+    for _ in range(steps):
+        model.forward()
+    ev.record(e1)
+    runtime.wait()
+    wall = time.perf_counter() - t0
+    dev_ms = ev.elapsed_ms(e0, e1) / steps
+    out = {"batch": batch, "images_per_s": round(batch * steps / wall, 1),
+           "ms_per_forward": round(wall * 1e3 / steps, 4), "device_ms_per_forward": round(dev_ms, 4),
+           "arena_bytes": model.arena_bytes, "nr_opr": model.nr_opr,
+           "int8_tops": round(2 * mobilenet.macs_per_image() * batch / (dev_ms * 1e-3) / 1e12, 2)}
+    if per_layer:
+        names = [n for _, n, _, _ in net.steps] + ["sm.max", "sm.sub", "sm.exp", "sm.sum", "softmax"]
+        layers = []
+        for i in range(model.nr_opr):
+            for _ in range(3):
+                model.run_opr(i)
+            runtime.wait()
+            a, b = ev.new(), ev.new()
+            ev.record(a)
+            for _ in range(10):
+                model.run_opr(i)
+            ev.record(b)
+            runtime.wait()
+            layers.append((names[i], round(ev.elapsed_ms(a, b) / 10 * 1e3, 1)))
+        out["layer_us"] = layers
+    model.close()
+    return out
+
+
 def case_bytes(case):
     ins, outs = case.specs(case.gen(0))
     return sum(s.nbytes for s in ins) + sum(s.nbytes for s in outs)
@@ -144,6 +187,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="conv")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--batch", type=int, default=64, help="batch of the mobilenet workload")
+    ap.add_argument("--per-layer", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (the path shards over the batch "
@@ -152,6 +197,9 @@ def main():
     from megcc_amd import runtime
     import numpy as np
 
+    if args.workload == "mobilenet":
+        print(json.dumps(bench_mobilenet(args.batch, args.steps, args.warmup, args.per_layer)))
+        return
     case, desc, bound = make_workload(args.workload)
     arrays = case.gen(seed=0)
     ins, outs = case.specs(arrays)

@@ -58,6 +58,7 @@ struct MfmaParams {
     int range_len;  // pixels per workgroup of the pipelined kernel (multiple of 32)
     int act;
     float s_src, s_flt, s_dst;
+    RequantFast rq;
     FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
     int G, RG;       // 16-byte gather: pixel groups per row, groups per plane of the largest patch
     FastDiv dG, dRG;

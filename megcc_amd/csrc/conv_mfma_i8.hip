@@ -208,10 +208,10 @@ __global__ void __launch_bounds__(THREADS) conv_mfma_i8_kernel(MfmaParams q) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const int a = acc[mi][ni][e4 * 4 + e] + bv[e];
-                            if (ACT == ACT_RUNTIME)
+                            if constexpr (ACT == ACT_RUNTIME)
                                 r[e] = requant_conv_rt(q.act, a, q.s_src, q.s_flt, q.s_dst);
                             else
-                                r[e] = requant_conv<ACT>(a, q.s_src, q.s_flt, q.s_dst);
+                                r[e] = requant_conv_fast<ACT>(a, q.rq);
                         }
                         if (!q.dst_fc) {
                             size_t o = ((size_t)pix_n[ni] * (q.OC >> 2) + (oc >> 2)) * q.OHW + pix_rem[ni];
@@ -446,6 +446,7 @@ TinyNNStatus conv_mfma_launch(
     q.s_src = g.s_src;
     q.s_flt = g.s_flt;
     q.s_dst = g.s_dst;
+    q.rq = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
     q.dOW = make_fastdiv(q.OW);
     q.dOH = make_fastdiv(q.OH);
     q.dVW = make_fastdiv(q.VW);

@@ -298,10 +298,10 @@ __global__ void __launch_bounds__(WTHREADS) conv_mfma_i8_wide_kernel(MfmaParams 
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int a = acc[mi][ni][e4 * 4 + e] + bv[e];
-                    if (ACT == ACT_RT)
+                    if constexpr (ACT == ACT_RT)
                         r[e] = requant_conv_rt(q.act, a, q.s_src, q.s_flt, q.s_dst);
                     else
-                        r[e] = requant_conv<ACT>(a, q.s_src, q.s_flt, q.s_dst);
+                        r[e] = requant_conv_fast<ACT>(a, q.rq);
                 }
                 if (pix_n[ni] >= 0 && oc < q.OC) {
                     if (!q.dst_fc) {

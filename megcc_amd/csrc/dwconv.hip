@@ -10,8 +10,9 @@
 
 namespace mg {
 
+template <int ACT>
 __global__ void __launch_bounds__(256) dwconv44_q8_kernel(
-        ConvGeom g, const uint32_t* __restrict__ src, const uint32_t* __restrict__ flt,
+        ConvGeom g, RequantFast rq, const uint32_t* __restrict__ src, const uint32_t* __restrict__ flt,
         const int32_t* __restrict__ bias, uint32_t* __restrict__ dst) {
     const int c4n = g.oc >> 2;
     const size_t total = (size_t)g.n * c4n * g.oh * g.ow;
@@ -44,7 +45,10 @@ __global__ void __launch_bounds__(256) dwconv44_q8_kernel(
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             int a = acc[c] + (bias ? bias[c4 * 4 + c] : 0);
-            o[c] = requant_conv_rt(g.act, a, g.s_src, g.s_flt, g.s_dst);
+            if (ACT < 0)
+                o[c] = requant_conv_rt(g.act, a, g.s_src, g.s_flt, g.s_dst);
+            else
+                o[c] = requant_conv_fast<(ACT < 0 ? 0 : ACT)>(a, rq);
         }
         dst[i] = pack4(o[0], o[1], o[2], o[3]);
     }
@@ -63,9 +67,12 @@ TinyNNStatus dwconv44_launch(
     unsigned blocks = (unsigned)((total + 255) / 256);
     if (blocks > 65536u * 8)
         blocks = 65536u * 8;
-    hipLaunchKernelGGL(dwconv44_q8_kernel, dim3(blocks), dim3(256), 0, stream(), g,
-                       (const uint32_t*)src, (const uint32_t*)flt, (const int32_t*)bias,
-                       (uint32_t*)dst);
+    const RequantFast rq = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
+    auto kern = g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_q8_kernel<MEGCC_NONLINE_IDENTITY>
+              : g.act == MEGCC_NONLINE_RELU     ? dwconv44_q8_kernel<MEGCC_NONLINE_RELU>
+                                                : dwconv44_q8_kernel<-1>;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), 0, stream(), g, rq, (const uint32_t*)src,
+                       (const uint32_t*)flt, (const int32_t*)bias, (uint32_t*)dst);
     return check_launch("dwconv44_q8");
 }
 

@@ -46,6 +46,54 @@ __device__ __forceinline__ int requant_conv(int acc, float s_src, float s_flt, f
     return fp32_to_int8(act_apply<ACT>(v));
 }
 
+// ---- exact requantisation at a third of the instructions ---------------------------------------
+// For IDENTITY and RELU the int8 result only depends on which integer the scaled value rounds to,
+// so it can be taken from ONE multiply by c = fl(fl(s_src*s_flt)/s_dst) whenever that product is
+// safely away from a rounding boundary:
+//     v = fl(fl(fl(a*s_src)*s_flt)/s_dst)  (the reference, three roundings)
+//     g = fl(a*c)                          (three roundings too, c is computed on the host)
+// both are within 3*2^-24 relative of the real quotient, so |v - g| <= 6*2^-24*|v| < 2^-14 for
+// |v| < 129. If the distance of g to the nearest integer r is below 0.5 - 2^-13, v rounds (half
+// away from zero, like roundf) to the same r; beyond +-129 both clamp. Only lanes closer than
+// 2^-13 to a tie (about one in 4000; exact ties included) take the reference's own sequence.
+// RELU commutes with the rounding: roundf(max(v,0)) == max(roundf(v),0).
+struct RequantFast {
+    float c;       // fl(fl(s_src*s_flt)/s_dst); 0 disables the fast path (extreme scales)
+    float s_src, s_flt, s_dst;
+};
+
+// host side: c, or 0 when a scale is so extreme that the error bound above does not hold
+static inline RequantFast make_requant_fast(float s_src, float s_flt, float s_dst) {
+    RequantFast q;
+    q.s_src = s_src;
+    q.s_flt = s_flt;
+    q.s_dst = s_dst;
+    const float p = s_src * s_flt;
+    const float c = p / s_dst;
+    auto mid = [](float x) { return x > 1e-30f && x < 1e30f; };
+    const bool sane = mid(s_src) && mid(s_flt) && mid(p) && mid(s_dst) && mid(c);
+    q.c = sane ? c : 0.f;
+    return q;
+}
+
+template <int ACT>
+__device__ __forceinline__ int requant_conv_fast(int acc, const RequantFast& q) {
+    static_assert(ACT == MEGCC_NONLINE_IDENTITY || ACT == MEGCC_NONLINE_RELU, "monotone only");
+    const float a = (float)acc;
+    const float g = a * q.c;
+    const float r = __builtin_rintf(g);  // nearest, ties to even: ties never use this result
+    const float d = __builtin_fabsf(g - r);
+    int out;
+    if (__builtin_expect((!(d <= 0.5f - 0x1p-13f) && __builtin_fabsf(g) < 129.f) || q.c == 0.f, 0)) {
+        out = requant_conv<ACT>(acc, q.s_src, q.s_flt, q.s_dst);
+    } else {
+        int i = (int)r;  // saturating conversion
+        const int lo = ACT == MEGCC_NONLINE_RELU ? 0 : -128;
+        out = i < lo ? lo : (i > 127 ? 127 : i);
+    }
+    return out;
+}
+
 // run-time activation selector (a uniform branch) for kernels that are not templated on it
 __device__ __forceinline__ int requant_conv_rt(int act, int acc, float s0, float s1, float s2) {
     switch (act) {

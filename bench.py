@@ -30,6 +30,10 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
 
 PEAK_INT8_TOPS = 5000.0  # dense int8 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the default workload's kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (KiB per dispatch, scaled by what a 256 MiB copy reads on the same counters: x2.000 / x1.000);
+# the counter runs and their figures are in profiles/conv_mfma_i8_wide__conv3x3_n32_c256_56x56.txt
+MEASURED_TRAFFIC = {"conv": (77040 * 2.000 + 41720 * 1.000) * 1024}
 
 
 class HipEvents:
@@ -65,7 +69,7 @@ def headline_case(n=32, c=256, hw=56):
 
 def make_workload(name):
     """-> (case, description, bound, algorithmic units per launch)"""
-    from cases import ConvCase, MultiTypeCase, PoolCase
+    from cases import ConvCase, MultiTypeCase, PoolCase, TypeCvtCase
     from megcc_amd import abi
     if name == "conv":
         case = headline_case()
@@ -100,6 +104,9 @@ def make_workload(name):
     if name == "add":
         return (MultiTypeCase(abi.Q_FUSE_ADD_RELU, (64, 32, 56, 56), (0.05, 0.01, 0.05)),
                 "qsi8 QFUSE_ADD_RELU 64x32x56x56", "hbm")
+    if name == "copy":  # same-scale requantise = a plain copy: the counter calibration kernel
+        return (TypeCvtCase("qsi8", "qsi8", (256, 1024, 1024), src_scale=0.05, dst_scale=0.05),
+                "qsi8->qsi8 typecvt, equal scales, 256 MiB in + 256 MiB out", "hbm")
     raise SystemExit("unknown workload " + name)
 
 
@@ -231,6 +238,8 @@ def main():
         value, unit, metric = nbytes / (wall / args.steps) / 1e9, "GB/s", "hbm_gbps"
         roof = {"bound": "hbm", "achieved": round(nbytes / (kern_ms * 1e-3) / 1e9, 2),
                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "traffic": None}
+    if args.workload in MEASURED_TRAFFIC:
+        roof["traffic"] = int(MEASURED_TRAFFIC[args.workload])
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
     roof["kernel_ms"] = round(kern_ms, 5)
     roof["algorithmic_per_launch"] = ops if bound == "mfma" else nbytes
@@ -239,12 +248,16 @@ def main():
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8" if bound == "mfma" or True else "u8", "data": "synthetic",
+        "dtype": "int8", "data": "synthetic",
         "config": {"workload": desc, "symbol": case.symbol(), "abi": "megcc_gfx950_call"},
         "roofline": roof,
     }
     if not args.no_cpu and args.workload == "conv":
         out["cpu_baseline"] = cpu_baseline(case)
+        op = None
+        mb = bench_mobilenet(64, 20, 5)
+        out["extra"] = {"mobilenet_v1_int8_images_per_s_batch64": mb["images_per_s"],
+                        "mobilenet_v1_int8_ms_per_forward_batch64": mb["ms_per_forward"]}
     print(json.dumps(out))
 
 

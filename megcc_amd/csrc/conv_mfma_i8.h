@@ -1,6 +1,8 @@
-// Definitions shared by the two qsi8 MFMA convolution kernels (conv_mfma_i8.hip: one stage at a
-// time, any shape; conv_mfma_i8_pipe.hip: software-pipelined, large shapes).
+// Definitions shared by the two qsi8 MFMA convolution kernels (conv_mfma_i8.hip: one stage at a time,
+// any shape; conv_mfma_i8_wide.hip and conv_mfma_i8_ws.hip: pipelined, large shapes).
 #pragma once
+#include <utility>
+
 #include "common.h"
 #include "conv_geom.h"
 #include "epilogue.cuh"
@@ -57,6 +59,7 @@ struct MfmaParams {
     int bias_vec4;  // bias pointer is 16-byte aligned
     int range_len;  // pixels per workgroup of the pipelined kernel (multiple of 32)
     int act;
+    int dbg;
     float s_src, s_flt, s_dst;
     RequantFast rq;
     FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
@@ -72,8 +75,27 @@ __device__ __forceinline__ int vp_of(const MfmaParams& q, int p) {
 }
 
 
+// compile-time loop: f(std::integral_constant<int, 0>) ... f(<N-1>)
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+// workgroup barrier that orders LDS traffic only (no wait for outstanding global loads)
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 struct PipeConfig {
     int bm, bn, ks, maxb, blocks_per_cu, threads, a_bytes, g4;
+    int gather_threads;  // threads that share the activation gather (maxb items each)
+    int nbuf;            // LDS stage buffers
     const void* kernel;
 };
 

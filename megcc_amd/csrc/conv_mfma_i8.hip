@@ -369,6 +369,7 @@ TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed) {
 }
 
 bool conv_mfma_pipe_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
+bool conv_mfma_ws_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
 
 TinyNNStatus conv_mfma_launch(
@@ -376,9 +377,14 @@ TinyNNStatus conv_mfma_launch(
     MfmaParams q;
     PipeConfig pc;
     const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;
-    bool pipe = conv_mfma_pipe_config(g, g4_ok, &pc) && !getenv("MEGCC_NOWIDE");
+    // development switches: MEGCC_NOWS / MEGCC_NOWIDE force the next kernel in line
+    const bool allow_wide = !getenv("MEGCC_NOWIDE");
+    bool pipe = allow_wide && ((!getenv("MEGCC_NOWS") && conv_mfma_ws_config(g, g4_ok, &pc)) ||
+                               conv_mfma_pipe_config(g, g4_ok, &pc));
     long range_len = 0;
-    if (pipe) {
+    TilePlan t;
+    bool fits = false;
+    for (int attempt = 0; attempt < 2 && pipe && !fits; ++attempt) {
         // one pixel range per free workgroup slot, so that the whole grid is resident at once and
         // every CU finishes at the same time (no partial last round)
         const long P = (long)g.n * g.oh * g.ow;
@@ -386,17 +392,21 @@ TinyNNStatus conv_mfma_launch(
         const long oc_tiles = (g.oc + pc.bm - 1) / pc.bm;
         long ranges = slots / oc_tiles > 0 ? slots / oc_tiles : 1;
         range_len = ((P + ranges - 1) / ranges + 31) / 32 * 32;
-        if (range_len < pc.bn / 2) {
-            pipe = false;  // too few pixels per workgroup to fill the 256-pixel tile
-            range_len = 0;
+        fits = range_len >= pc.bn / 2;  // else too few pixels per workgroup for the tile
+        if (fits) {
+            t = plan_tiles(g, pc.bn, range_len);
+            const long gather_items =
+                    pc.g4 ? 8L * pc.ks * t.rows_max * (g.iw / 4) : 2L * pc.ks * t.Lmax;
+            fits = gather_items <= (long)pc.maxb * pc.gather_threads &&
+                   (long)pc.nbuf * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) <= 160 * 1024;
         }
+        // the wave-specialised kernel declined: try the symmetric wide kernel, then give up
+        if (!fits)
+            pipe = pc.nbuf == 3 && conv_mfma_pipe_config(g, g4_ok, &pc);
     }
-    TilePlan t = plan_tiles(g, pipe ? pc.bn : BN, range_len);
-    const long gather_items =
-            !pipe ? 0 : pc.g4 ? 8L * pc.ks * t.rows_max * (g.iw / 4) : 2L * pc.ks * t.Lmax;
-    if (pipe && (gather_items > (long)pc.maxb * pc.threads ||
-                 2L * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) > 160 * 1024)) {
-        pipe = false;
+    pipe = pipe && fits;
+    if (!pipe) {
+        range_len = 0;
         t = plan_tiles(g, BN);
     }
     q.range_len = (int)range_len;
@@ -443,6 +453,7 @@ TinyNNStatus conv_mfma_launch(
     q.dst_fc = fc ? 1 : 0;
     q.bias_vec4 = bias && ((uintptr_t)bias & 15) == 0;
     q.act = g.act;
+    q.dbg = getenv("MEGCC_WS_DBG") ? atoi(getenv("MEGCC_WS_DBG")) : 0;
     q.s_src = g.s_src;
     q.s_flt = g.s_flt;
     q.s_dst = g.s_dst;

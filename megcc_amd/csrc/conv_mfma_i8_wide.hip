@@ -19,28 +19,9 @@
 // slots on the chip (CUs / oc-tiles), each workgroup walks its range in sub-tiles of 256 pixels:
 // the whole grid is resident at once and all CUs finish together instead of leaving a partial
 // last round.
-#include <utility>
-
 #include "conv_mfma_i8.h"
 
 namespace mg {
-
-// compile-time loop: f(std::integral_constant<int, 0>) ... f(<N-1>)
-template <int... I, typename F>
-__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
-    (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    static_for_impl(std::make_integer_sequence<int, N>{}, f);
-}
-
-// workgroup barrier that orders LDS traffic only (no wait for outstanding global loads)
-__device__ __forceinline__ void lds_barrier() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
 
 static constexpr int ACT_RT = -1;
 static constexpr int WTHREADS = 512;
@@ -335,6 +316,8 @@ static PipeConfig make_config(int act) {
     c.maxb = MAXB;
     c.g4 = G4;
     c.threads = WTHREADS;
+    c.gather_threads = WTHREADS;
+    c.nbuf = 2;
     c.blocks_per_cu = 1;
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     if (act == MEGCC_NONLINE_IDENTITY)
@@ -366,7 +349,7 @@ bool conv_mfma_pipe_config(const ConvGeom& g, bool g4_ok, PipeConfig* c) {
 }
 
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q) {
-    const size_t lds = 2 * ((size_t)c.a_bytes + (size_t)c.ks * q.Lmax * KROW);
+    const size_t lds = c.nbuf * ((size_t)c.a_bytes + (size_t)c.ks * q.Lmax * KROW);
     MG_REQUIRE(lds <= 160 * 1024, TinyNN_ERROR_OUT_OF_RANGE, "conv_mfma_wide: %zu bytes of LDS", lds);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(c.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

@@ -73,6 +73,9 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.DENSE, 6, 32, 56, 56, 160, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(288))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 6, 64, 55, 57, 256, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(576))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 11, 36, 56, 56, 128, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(324))),
+    # several 256-pixel sub-tiles per workgroup and three channel stages (pipelined across sub-tiles)
+    ConvCase(A.FMT_NCHW44, A.DENSE, 24, 96, 56, 56, 128, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(864))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 21, 32, 60, 52, 136, 3, 1, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(288))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 6, 136, 56, 56, 264, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(136))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 11, 64, 56, 56, 128, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(64))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 70, 256, 14, 14, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(256))),

@@ -59,7 +59,6 @@ struct MfmaParams {
     int bias_vec4;  // bias pointer is 16-byte aligned
     int range_len;  // pixels per workgroup of the pipelined kernel (multiple of 32)
     int act;
-    int dbg;
     float s_src, s_flt, s_dst;
     RequantFast rq;
     FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
@@ -96,6 +95,7 @@ struct PipeConfig {
     int bm, bn, ks, maxb, blocks_per_cu, threads, a_bytes, g4;
     int gather_threads;  // threads that share the activation gather (maxb items each)
     int nbuf;            // LDS stage buffers
+    int extra_lds;       // bytes of LDS beyond the stage buffers
     const void* kernel;
 };
 

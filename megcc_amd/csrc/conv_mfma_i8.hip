@@ -398,7 +398,7 @@ TinyNNStatus conv_mfma_launch(
             const long gather_items =
                     pc.g4 ? 8L * pc.ks * t.rows_max * (g.iw / 4) : 2L * pc.ks * t.Lmax;
             fits = gather_items <= (long)pc.maxb * pc.gather_threads &&
-                   (long)pc.nbuf * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) <= 160 * 1024;
+                   (long)pc.nbuf * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) + pc.extra_lds <= 160 * 1024;
         }
         // the wave-specialised kernel declined: try the symmetric wide kernel, then give up
         if (!fits)
@@ -453,7 +453,6 @@ TinyNNStatus conv_mfma_launch(
     q.dst_fc = fc ? 1 : 0;
     q.bias_vec4 = bias && ((uintptr_t)bias & 15) == 0;
     q.act = g.act;
-    q.dbg = getenv("MEGCC_WS_DBG") ? atoi(getenv("MEGCC_WS_DBG")) : 0;
     q.s_src = g.s_src;
     q.s_flt = g.s_flt;
     q.s_dst = g.s_dst;

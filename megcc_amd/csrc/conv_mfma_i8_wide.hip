@@ -318,6 +318,7 @@ static PipeConfig make_config(int act) {
     c.threads = WTHREADS;
     c.gather_threads = WTHREADS;
     c.nbuf = 2;
+    c.extra_lds = 0;
     c.blocks_per_cu = 1;
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     if (act == MEGCC_NONLINE_IDENTITY)
@@ -349,7 +350,7 @@ bool conv_mfma_pipe_config(const ConvGeom& g, bool g4_ok, PipeConfig* c) {
 }
 
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q) {
-    const size_t lds = c.nbuf * ((size_t)c.a_bytes + (size_t)c.ks * q.Lmax * KROW);
+    const size_t lds = c.nbuf * ((size_t)c.a_bytes + (size_t)c.ks * q.Lmax * KROW) + c.extra_lds;
     MG_REQUIRE(lds <= 160 * 1024, TinyNN_ERROR_OUT_OF_RANGE, "conv_mfma_wide: %zu bytes of LDS", lds);
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(c.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

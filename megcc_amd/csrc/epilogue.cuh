@@ -108,6 +108,59 @@ __device__ __forceinline__ int requant_conv_rt(int act, int acc, float s0, float
     }
 }
 
+// ---- exact requantisation by threshold table ---------------------------------------------------
+// For a monotone activation (IDENTITY, RELU) the reference's F(acc) = fp32_to_int8(act(acc * s_src
+// * s_flt / s_dst)) is a non-decreasing step function of the integer accumulator, so it is fully
+// described by 255 thresholds T[j] = max{a : F(a) < j}, j = -127..127:  F(a) = lo + #{j : a > T[j]}.
+// A kernel builds the table once per workgroup with the reference's literal float sequence
+// (binary search over int32, one entry per thread), and then needs only ONE estimate per output:
+// with g = fl((float)a * c), c = fl(fl(s_src*s_flt)/s_dst), the true value is within 2^-14 of g
+// while |g| < 129, so F(a) is floor(g) or floor(g)+1 (clamped), and the table decides which:
+//     m = clamp(floor(g), lo, 126);   F(a) = m + (a > T[m + 1])
+// No rounding-mode reasoning, no near-tie special case, bit-exact by construction.
+static constexpr int REQUANT_TABLE_ENTRIES = 256;  // entry j + 127, last one unused
+
+// entry `idx` (0..254) of the table; every call runs ~32 evaluations of the literal sequence
+template <int ACT>
+__device__ __forceinline__ int requant_threshold(int idx, float s_src, float s_flt, float s_dst) {
+    const int j = idx - 127;
+    long long lo = INT32_MIN, hi = INT32_MAX;
+    if (!(requant_conv<ACT>((int)lo, s_src, s_flt, s_dst) < j))
+        return INT32_MIN;  // F never drops below j: entry not used (j <= lowest output)
+    while (lo < hi) {  // invariant: F(lo) < j
+        const long long mid = lo + (hi - lo + 1) / 2;
+        if (requant_conv<ACT>((int)mid, s_src, s_flt, s_dst) < j)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    return (int)lo;
+}
+
+// table: pointer to entry 0 (LDS). ACT_LO: lowest output (-128, or 0 with RELU).
+template <int ACT>
+__device__ __forceinline__ int requant_conv_table(int acc, float c, const int* table) {
+    static_assert(ACT == MEGCC_NONLINE_IDENTITY || ACT == MEGCC_NONLINE_RELU, "monotone only");
+    constexpr int LO = ACT == MEGCC_NONLINE_RELU ? 0 : -128;
+    const float g = (float)acc * c;
+    int m = (int)__builtin_floorf(g);  // saturating conversion
+    m = m < LO ? LO : (m > 126 ? 126 : m);
+    return m + (acc > table[m + 128] ? 1 : 0);
+}
+
+// host side: the estimate above is valid (else kernels use the literal sequence per element)
+static inline bool requant_table_ok(float s_src, float s_flt, float s_dst) {
+    const RequantFast q = make_requant_fast(s_src, s_flt, s_dst);
+    return q.c != 0.f && q.c * 2147483648.f > 1000.f;
+}
+
+// bytes 0 of a, b, c, d -> one dword
+__device__ __forceinline__ uint32_t pack4_perm(int a, int b, int c, int d) {
+    const uint32_t lo = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+
 __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
     return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) |
            ((uint32_t)(d & 0xff) << 24);

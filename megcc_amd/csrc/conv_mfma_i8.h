@@ -46,6 +46,7 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t x, const FastDiv& f) {
 
 struct MfmaParams {
     const int8_t* src;
+    int src_bytes;
     const int8_t* wp;
     const int32_t* bias;
     int8_t* dst;
@@ -91,11 +92,55 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+#define MG_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define MG_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt = bits 3:0 and
+// 15:14, expcnt = 6:4, lgkmcnt = 11:8)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// LDS-direct loads written as inline assembly: the compiler's wait-count pass treats the builtin
+// forms as possible LDS accesses of unknown order and then drains the LDS counter (lgkmcnt(0)) at
+// every operand wait of the MFMA loop. These are invisible to it; completion is tracked by hand with
+// wait_vmcnt(). `lds_addr` (byte address in LDS of lane 0's data) must be wave-uniform; lane l's
+// data lands at lds_addr + l * size.
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+    return (unsigned)(size_t)MG_LDS_PTR(p);
+}
+__device__ __forceinline__ void dma_global_b128(const void* gptr, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_addr))
+                 : "memory");
+}
+// raw buffer (stride 0): offsets at or beyond num_records read as zero
+__device__ __forceinline__ v4u make_raw_buffer(const void* base, unsigned num_records) {
+    const unsigned long long a = (unsigned long long)base;
+    v4u r;
+    r[0] = (unsigned)a;
+    r[1] = (unsigned)(a >> 32) & 0xffffu;
+    r[2] = num_records;
+    r[3] = 0x00020000u;
+    return r;
+}
+__device__ __forceinline__ void dma_buffer_b32(v4u rsrc, unsigned voffset, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dword %0, %1, 0 offen lds"
+                 :
+                 : "v"(voffset), "s"(rsrc), "s"(__builtin_amdgcn_readfirstlane(lds_addr))
+                 : "memory");
+}
+
 struct PipeConfig {
     int bm, bn, ks, maxb, blocks_per_cu, threads, a_bytes, g4;
     int gather_threads;  // threads that share the activation gather (maxb items each)
     int nbuf;            // LDS stage buffers
     int extra_lds;       // bytes of LDS beyond the stage buffers
+    int fixed_lmax;      // patch slots compiled into the kernel (0: run-time Lmax)
     const void* kernel;
 };
 

@@ -370,6 +370,7 @@ TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed) {
 
 bool conv_mfma_pipe_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
 bool conv_mfma_ws_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
+bool conv_mfma_dma_config(const ConvGeom& g, PipeConfig* c);
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
 
 TinyNNStatus conv_mfma_launch(
@@ -377,14 +378,21 @@ TinyNNStatus conv_mfma_launch(
     MfmaParams q;
     PipeConfig pc;
     const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;
-    // development switches: MEGCC_NOWS / MEGCC_NOWIDE force the next kernel in line
-    const bool allow_wide = !getenv("MEGCC_NOWIDE");
-    bool pipe = allow_wide && ((!getenv("MEGCC_NOWS") && conv_mfma_ws_config(g, g4_ok, &pc)) ||
-                               conv_mfma_pipe_config(g, g4_ok, &pc));
+    // candidates in order of preference; development switches MEGCC_NODMA / MEGCC_NOWS /
+    // MEGCC_NOWIDE skip one
     long range_len = 0;
     TilePlan t;
-    bool fits = false;
-    for (int attempt = 0; attempt < 2 && pipe && !fits; ++attempt) {
+    bool pipe = false;
+    for (int cand = 0; cand < 3 && !pipe; ++cand) {
+        bool have = false;
+        if (cand == 0)
+            have = !getenv("MEGCC_NODMA") && conv_mfma_dma_config(g, &pc);
+        else if (cand == 1)
+            have = !getenv("MEGCC_NOWS") && conv_mfma_ws_config(g, g4_ok, &pc);
+        else
+            have = !getenv("MEGCC_NOWIDE") && conv_mfma_pipe_config(g, g4_ok, &pc);
+        if (!have)
+            continue;
         // one pixel range per free workgroup slot, so that the whole grid is resident at once and
         // every CU finishes at the same time (no partial last round)
         const long P = (long)g.n * g.oh * g.ow;
@@ -392,19 +400,19 @@ TinyNNStatus conv_mfma_launch(
         const long oc_tiles = (g.oc + pc.bm - 1) / pc.bm;
         long ranges = slots / oc_tiles > 0 ? slots / oc_tiles : 1;
         range_len = ((P + ranges - 1) / ranges + 31) / 32 * 32;
-        fits = range_len >= pc.bn / 2;  // else too few pixels per workgroup for the tile
-        if (fits) {
-            t = plan_tiles(g, pc.bn, range_len);
-            const long gather_items =
-                    pc.g4 ? 8L * pc.ks * t.rows_max * (g.iw / 4) : 2L * pc.ks * t.Lmax;
-            fits = gather_items <= (long)pc.maxb * pc.gather_threads &&
-                   (long)pc.nbuf * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) + pc.extra_lds <= 160 * 1024;
+        if (range_len < pc.bn / 2)  // too few pixels per workgroup for the tile
+            continue;
+        t = plan_tiles(g, pc.bn, range_len);
+        if (pc.fixed_lmax) {
+            if (t.Lmax > pc.fixed_lmax)
+                continue;
+            t.Lmax = pc.fixed_lmax;
         }
-        // the wave-specialised kernel declined: try the symmetric wide kernel, then give up
-        if (!fits)
-            pipe = pc.nbuf == 3 && conv_mfma_pipe_config(g, g4_ok, &pc);
+        const long gather_items =
+                pc.g4 ? 8L * pc.ks * t.rows_max * (g.iw / 4) : 2L * pc.ks * t.Lmax;
+        pipe = (pc.gather_threads == 0 || gather_items <= (long)pc.maxb * pc.gather_threads) &&
+               (long)pc.nbuf * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) + pc.extra_lds <= 160 * 1024;
     }
-    pipe = pipe && fits;
     if (!pipe) {
         range_len = 0;
         t = plan_tiles(g, BN);
@@ -412,6 +420,7 @@ TinyNNStatus conv_mfma_launch(
     q.range_len = (int)range_len;
     bool fc = is_fc(g);
     q.src = (const int8_t*)src;
+    q.src_bytes = (int)((long)g.n * g.ic * g.ih * g.iw);
     q.wp = (const int8_t*)packed;
     q.bias = (const int32_t*)bias;
     q.dst = (int8_t*)dst;

@@ -1,0 +1,319 @@
+// qsi8 implicit-GEMM convolution for large layers, third generation (same arithmetic and packed
+// filter as conv_mfma_i8.hip): every byte reaches LDS by LDS-direct loads, so no wave spends
+// registers, VALU work or LDS-write instructions on data movement.
+//
+//   * filter tile of a stage (taps x 128 oc x 32 ic): 16-byte global->LDS loads, 1 KB per wave-load;
+//   * activation patch of a stage: dword buffer->LDS loads. Lane l of a wave-load fetches plane
+//     (l & 3) of patch slot (l >> 2): the 64 dwords land as 16 consecutive 16-byte words, which is
+//     exactly the LDS layout [sub-chunk][16-channel half][virtual pixel][16 bytes] the MFMA operand
+//     reads want (consecutive lanes -> consecutive words, a tap = a wave-uniform byte offset).
+//     Padding pixels use an offset beyond the buffer's num_records: the hardware range check
+//     returns zero for them, so padding costs nothing;
+//   * three LDS stage buffers; the loads of stage g+2 are issued at the start of stage g and waited
+//     for (s_waitcnt vmcnt, loads return in order) at the end of stage g+1; one barrier per stage.
+//     The stage counter runs across the 256-pixel sub-tiles of the workgroup's pixel range.
+//
+// One workgroup = 8 waves (2 x 4) on a 128 oc x 256 pixel tile, 64 accumulators per lane. The
+// loads of the next sub-tile's first stages are already in flight while a sub-tile's epilogue runs.
+//
+// Requantisation uses the exact threshold table (epilogue.cuh) built once per workgroup.
+#include <stdlib.h>
+
+#include "conv_mfma_i8.h"
+
+namespace mg {
+
+static constexpr int ACT_RT = -1;
+static constexpr int DM_THREADS = 512, DM_WAVES = 8, DM_NBUF = 3;
+static constexpr int DM_BM = 128, DM_BNP = 256;
+
+// FH x FW taps, KS 32-channel sub-chunks per stage, LMAX patch slots (compile time, so that the
+// number of loads per stage is a constant the vmcnt waits can be written for).
+template <int FH, int FW, int KS, int LMAX, int ACT>
+__global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams q) {
+    constexpr int MT = 2, NT = 2, WGN = 4;
+    constexpr int TAPS = FH * FW;
+    constexpr int TS = TAPS * KS;
+    constexpr int A_BYTES = TS * DM_BM * KROW;
+    constexpr int A_CHUNKS = A_BYTES / 1024;
+    constexpr int A_PER_WAVE = (A_CHUNKS + DM_WAVES - 1) / DM_WAVES;
+    constexpr int B_BYTES = KS * 2 * LMAX * 16;
+    constexpr int B_WL = B_BYTES / 256;
+    static_assert(B_WL % DM_WAVES == 0 && LMAX % 16 == 0, "whole wave-loads");
+    constexpr int B_PER_WAVE = B_WL / DM_WAVES;
+    constexpr int LW = LMAX / 16;  // wave-loads per (sub-chunk, half)
+    constexpr int N_DMA = A_PER_WAVE + B_PER_WAVE;
+    constexpr int BUF_BYTES = A_BYTES + B_BYTES;
+    static_assert(N_DMA < 64, "vmcnt range");
+
+    extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+    int* const rq_table = (int*)(lds + DM_NBUF * BUF_BYTES);
+    int* const bias_lds = rq_table + REQUANT_TABLE_ENTRIES;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN, kg = lane >> 5;
+    const int oc0 = blockIdx.y * DM_BM;
+    const int range0 = blockIdx.x * q.range_len;
+    const int range1 = min(range0 + q.range_len, q.P);
+    const int stages = q.stages;
+    const int n_tiles = (range1 - range0 + DM_BNP - 1) / DM_BNP;
+    const int G = n_tiles * stages;
+
+    // ---- once per workgroup: requantisation thresholds and the bias slice of this oc tile
+    if constexpr (ACT != ACT_RT) {
+        if (tid < REQUANT_TABLE_ENTRIES)
+            rq_table[tid] = tid < 255 ? requant_threshold<ACT>(tid, q.s_src, q.s_flt, q.s_dst, q.rq.c) : 0;
+    }
+    if (tid >= 256 && tid < 256 + DM_BM) {
+        const int oc = oc0 + tid - 256;
+        bias_lds[tid - 256] = (q.bias && oc < q.OC) ? q.bias[oc] : 0;
+    }
+
+    // ---- load side ---------------------------------------------------------------------------
+    v4u src_rsrc = make_raw_buffer(q.src, (unsigned)q.src_bytes);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        src_rsrc[i] = __builtin_amdgcn_readfirstlane(src_rsrc[i]);
+    // filter: chunk c = wave + 8a (wrapped: the surplus loads repeat a chunk, same bytes to the
+    // same place), c = 4 * tap-step + 1 KB part
+    int a_chunk[A_PER_WAVE];  // wave-uniform
+#pragma unroll
+    for (int a = 0; a < A_PER_WAVE; ++a) {
+        int c = wave + a * DM_WAVES;
+        a_chunk[a] = c >= A_CHUNKS ? c - A_CHUNKS : c;
+    }
+    const int lane16 = lane * 16;
+    // activations: wave-load u = wave + 8j covers 16 slots of (sub-chunk, half) u / LW; this lane
+    // fetches plane (lane & 3) of slot (u % LW) * 16 + (lane >> 2). b_goff = byte offset of that
+    // dword in the first plane group of a stage, or 2^31 (out of range -> zero) for padding.
+    unsigned b_goff[B_PER_WAVE];
+    auto describe = [&](int p0) {
+        const int plast = min(p0 + DM_BNP, range1) - 1;
+        const int vp0 = vp_of(q, p0);
+        const int L = vp_of(q, plast) + ((FH - 1) * q.DH) * q.VW + (FW - 1) * q.DW - vp0 + 1;
+#pragma unroll
+        for (int j = 0; j < B_PER_WAVE; ++j) {
+            const int u = wave + j * DM_WAVES;
+            const int kh = u / LW, slot = (u - kh * LW) * 16 + (lane >> 2);
+            unsigned off = 0x80000000u;
+            if (slot < L) {
+                const int vp = vp0 + slot;
+                const int v = fdiv(vp, q.dVW), vc = vp - v * q.VW;
+                const int n = fdiv(v, q.dVH), vh = v - n * q.VH;
+                const int ih = vh - q.PH, iw = vc - q.PW;
+                if (n < q.N && (unsigned)ih < (unsigned)q.IH && (unsigned)iw < (unsigned)q.IW)
+                    off = n * q.image_stride + ih * q.row_stride + iw * q.pix_stride +
+                          ((kh >> 1) * 8 + (kh & 1) * 4 + (lane & 3)) * q.plane_stride;
+            }
+            b_goff[j] = off;
+        }
+    };
+    int lp0 = range0, lst = 0, lbuf = 0;  // load cursor: sub-tile, stage in it, LDS buffer
+    describe(lp0);
+    auto issue = [&](int8_t* buf) {
+        const int8_t* abase = q.wp + ((size_t)lst * TS * q.OCP + oc0) * KROW;
+#pragma unroll
+        for (int a = 0; a < A_PER_WAVE; ++a)
+            dma_global_b128(abase + ((a_chunk[a] >> 2) * q.OCP * KROW + (a_chunk[a] & 3) * 1024) + lane16,
+                            lds_address(buf + a_chunk[a] * 1024));
+        const unsigned poff = (unsigned)(lst * KS * 8) * (unsigned)q.plane_stride;
+#pragma unroll
+        for (int j = 0; j < B_PER_WAVE; ++j) {
+            const int u = wave + j * DM_WAVES;
+            dma_buffer_b32(src_rsrc, b_goff[j] + poff, lds_address(buf + A_BYTES + u * 256));
+        }
+        if (++lst == stages) {
+            lst = 0;
+            lp0 += DM_BNP;
+            if (lp0 < range1)
+                describe(lp0);
+        }
+        lbuf = lbuf == DM_NBUF - 1 ? 0 : lbuf + 1;
+    };
+
+    // ---- compute side ------------------------------------------------------------------------
+    int a_off[MT];
+#pragma unroll
+    for (int mi = 0; mi < MT; ++mi) {
+        int r = (wm * MT + mi) * 32 + (lane & 31);
+        a_off[mi] = r * KROW + (((kg ^ (r >> 3)) & 1) << 4);
+    }
+
+    v16i acc[MT][NT];
+    const int kg_plane = kg * q.OHW;
+
+    // Epilogue of one 32 oc x 32 pixel MFMA tile (16 outputs per lane = 4 NCHW44 dwords), written
+    // as one straight-line block so that its 4 bias reads and 16 table look-ups are in flight
+    // together. ob: dword index in dst of this lane's pixel in oc-group 0 (-1: lane beyond the
+    // sub-tile, -2: whole 32-pixel column beyond it, wave-uniform).
+    auto emit_tile = [&](auto mic, auto nic, const int ob, const int* tbl) {
+        constexpr int mi = decltype(mic)::value, ni = decltype(nic)::value;
+        if (ob < -1)
+            return;
+        const int ocl = (wm * MT + mi) * 32 + kg * 4;
+        int r[16];
+        if constexpr (ACT == ACT_RT) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                r[e] = requant_conv_rt(q.act, acc[mi][ni][e] + tbl[REQUANT_TABLE_ENTRIES + ocl + (e / 4) * 8 + e % 4],
+                                       q.s_src, q.s_flt, q.s_dst);
+        } else {
+            constexpr int LO = ACT == MEGCC_NONLINE_RELU ? 0 : -128;
+            v4i bv[4];
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4)
+                bv[e4] = *(const v4i*)(tbl + REQUANT_TABLE_ENTRIES + ocl + e4 * 8);
+            int a[16], m[16], t[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                a[e] = acc[mi][ni][e] + bv[e / 4][e % 4];
+                const int f = (int)__builtin_floorf((float)a[e] * q.rq.c);
+                m[e] = f < LO ? LO : (f > 126 ? 126 : f);
+                t[e] = tbl[m[e] + 128];
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                r[e] = m[e] + (a[e] > t[e] ? 1 : 0);
+        }
+        if (ob >= 0) {
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int oc = oc0 + ocl + e4 * 8;
+                if (oc < q.OC) {
+                    const int o = ob + ((oc0 >> 2) + (wm * MT + mi) * 8 + e4 * 2) * q.OHW + kg_plane;
+                    ((uint32_t*)q.dst)[o] =
+                            pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
+                }
+            }
+        }
+    };
+
+    // ---- prologue: two stages in flight, the first one landed
+    issue(lds);
+    if (G > 1) {
+        issue(lds + BUF_BYTES);
+        wait_vmcnt<N_DMA>();
+    } else {
+        wait_vmcnt<0>();
+    }
+    lds_barrier();
+
+    int g = 0, cbuf = 0;
+    for (int p0 = range0; p0 < range1; p0 += DM_BNP) {
+        const int plast = min(p0 + DM_BNP, range1) - 1;
+        const int vp0 = vp_of(q, p0);
+        int b_byte[NT];  // LDS byte offset of this lane's 16 channels at tap (0,0)
+        int cur_o[NT];
+        int cols = 0;    // wave-uniform: 32-pixel columns of this wave with pixels of the sub-tile
+#pragma unroll
+        for (int ni = 0; ni < NT; ++ni) {
+            const int pc = p0 + (wn * NT + ni) * 32;
+            const int p = pc + (lane & 31);
+            b_byte[ni] = (kg * LMAX + (p <= plast ? vp_of(q, p) - vp0 : 0)) * 16;
+            cols += pc <= plast ? 1 : 0;
+            const int pn = (int)fdiv(p, q.dOHW);
+            cur_o[ni] = pc > plast ? -2 : p <= plast ? pn * (q.OC >> 2) * q.OHW + (p - pn * q.OHW) : -1;
+        }
+#pragma unroll
+        for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < NT; ++ni)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    acc[mi][ni][e] = 0;
+
+        auto stage_body = [&](auto cols_c, const int8_t* bufA, int8_t* dma_buf) {
+            constexpr int COLS = decltype(cols_c)::value;
+            if (g + 2 < G)
+                issue(dma_buf);
+            const int8_t* bufB = bufA + A_BYTES;
+            if constexpr (COLS > 0) {
+                v4i fa[2][MT], fb[2][NT];
+                auto fetch = [&](auto tc) {
+                    constexpr int t = decltype(tc)::value;
+                    constexpr int ks = t / TAPS, tap = t % TAPS;
+                    constexpr int fh = tap / FW, fw = tap % FW;
+                    const int tap_off = fh * q.DH * q.VW + fw * q.DW;
+#pragma unroll
+                    for (int mi = 0; mi < MT; ++mi)
+                        fa[t & 1][mi] = *(const v4i*)(bufA + t * (DM_BM * KROW) + a_off[mi]);
+#pragma unroll
+                    for (int ni = 0; ni < COLS; ++ni)
+                        fb[t & 1][ni] = *(const v4i*)(bufB + ks * (2 * LMAX * 16) + b_byte[ni] +
+                                                      tap_off * 16);
+                };
+                fetch(std::integral_constant<int, 0>{});
+                static_for<TS>([&](auto tc) {
+                    constexpr int t = decltype(tc)::value;
+                    if constexpr (t + 1 < TS)
+                        fetch(std::integral_constant<int, t + 1>{});
+                    // keep the compiler from sinking these reads below the MFMAs of step t
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int ni = 0; ni < COLS; ++ni)
+#pragma unroll
+                        for (int mi = 0; mi < MT; ++mi)
+                            acc[mi][ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                    fa[t & 1][mi], fb[t & 1][ni], acc[mi][ni], 0, 0, 0);
+                });
+            }
+        };
+        auto run_stages = [&](auto cols_c) {
+            for (int st = 0; st < stages; ++st, ++g) {
+                stage_body(cols_c, lds + cbuf * BUF_BYTES, lds + lbuf * BUF_BYTES);
+                if (g + 2 < G)
+                    wait_vmcnt<N_DMA>();
+                else
+                    wait_vmcnt<0>();
+                lds_barrier();
+                cbuf = cbuf == DM_NBUF - 1 ? 0 : cbuf + 1;
+            }
+        };
+        if (cols == 2)
+            run_stages(std::integral_constant<int, 2>{});
+        else if (cols == 1)
+            run_stages(std::integral_constant<int, 1>{});
+        else
+            run_stages(std::integral_constant<int, 0>{});
+
+        static_for<MT>([&](auto mic) {
+            static_for<NT>([&](auto nic) { emit_tile(mic, nic, cur_o[decltype(nic)::value], rq_table); });
+        });
+    }
+}
+
+// ---- configurations --------------------------------------------------------------------------
+template <int FH, int FW, int KS, int LMAX>
+static PipeConfig make_dma_config(int act, bool table_ok) {
+    PipeConfig c;
+    c.bm = DM_BM;
+    c.bn = DM_BNP;
+    c.ks = KS;
+    c.maxb = 0;
+    c.g4 = 0;
+    c.threads = DM_THREADS;
+    c.gather_threads = 0;
+    c.nbuf = DM_NBUF;
+    c.blocks_per_cu = 1;
+    c.a_bytes = FH * FW * KS * c.bm * KROW;
+    c.fixed_lmax = LMAX;
+    c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + DM_BM * 4;
+    if (act == MEGCC_NONLINE_IDENTITY && table_ok)
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY>;
+    else if (act == MEGCC_NONLINE_RELU && table_ok)
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU>;
+    else
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT>;
+    return c;
+}
+
+// 3x3 layers (NCHW44) with at least 128 output channels and enough pixels to fill the chip
+bool conv_mfma_dma_config(const ConvGeom& g, PipeConfig* c) {
+    const long P = (long)g.n * g.oh * g.ow;
+    if (!(g.fh == 3 && g.fw == 3) || g.fmt != MEGCC_FMT_NCHW44 || g.oc < 128 || P < 8192)
+        return false;
+    *c = make_dma_config<3, 3, 1, 512>(g.act, requant_table_ok(g.s_src, g.s_flt, g.s_dst));
+    return true;
+}
+
+}  // namespace mg

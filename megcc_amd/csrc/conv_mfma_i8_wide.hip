@@ -319,6 +319,7 @@ static PipeConfig make_config(int act) {
     c.gather_threads = WTHREADS;
     c.nbuf = 2;
     c.extra_lds = 0;
+    c.fixed_lmax = 0;
     c.blocks_per_cu = 1;
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     if (act == MEGCC_NONLINE_IDENTITY)

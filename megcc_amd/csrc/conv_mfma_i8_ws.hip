@@ -36,17 +36,6 @@ static constexpr int WS_THREADS = WS_CONSUMERS + WS_PRODUCERS;
 static constexpr int WS_NBUF = 3;
 static constexpr int WS_BM = 128, WS_BNP = 256;
 
-#define MG_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
-#define MG_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
-
-// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt = bits 3:0 and
-// 15:14, expcnt = 6:4, lgkmcnt = 11:8)
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
 struct WsTile {  // activation patch of one sub-tile
     int vp0, L, v_first, rows, slot_base;
 };
@@ -221,7 +210,7 @@ __global__ void __launch_bounds__(WS_THREADS) conv_mfma_i8_ws_kernel(MfmaParams 
     int* const rq_table = (int*)(lds + WS_NBUF * buf_bytes);
     if constexpr (ACT != ACT_RT) {
         if (tid < REQUANT_TABLE_ENTRIES)
-            rq_table[tid] = tid < 255 ? requant_threshold<ACT>(tid, q.s_src, q.s_flt, q.s_dst) : 0;
+            rq_table[tid] = tid < 255 ? requant_threshold<ACT>(tid, q.s_src, q.s_flt, q.s_dst, q.rq.c) : 0;
     }
     lds_barrier();  // step -3
     lds_barrier();  // step -2
@@ -381,6 +370,7 @@ static PipeConfig make_ws_config(int act, bool table_ok) {
     c.blocks_per_cu = 1;
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     c.extra_lds = REQUANT_TABLE_ENTRIES * 4;
+    c.fixed_lmax = 0;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
         c.kernel = (const void*)conv_mfma_i8_ws_kernel<FH, FW, KS, MEGCC_NONLINE_IDENTITY, MAXB>;
     else if (act == MEGCC_NONLINE_RELU && table_ok)

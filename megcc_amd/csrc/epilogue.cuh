@@ -120,16 +120,29 @@ __device__ __forceinline__ int requant_conv_rt(int act, int acc, float s0, float
 // No rounding-mode reasoning, no near-tie special case, bit-exact by construction.
 static constexpr int REQUANT_TABLE_ENTRIES = 256;  // entry j + 127, last one unused
 
-// entry `idx` (0..254) of the table; every call runs ~32 evaluations of the literal sequence
+// entry `idx` (0..254) of the table: a handful of evaluations of the literal sequence (32 when
+// the estimate from c is useless)
 template <int ACT>
-__device__ __forceinline__ int requant_threshold(int idx, float s_src, float s_flt, float s_dst) {
+__device__ __forceinline__ int requant_threshold(int idx, float s_src, float s_flt, float s_dst, float c) {
     const int j = idx - 127;
+    auto below = [&](long long a) { return requant_conv<ACT>((int)a, s_src, s_flt, s_dst) < j; };
     long long lo = INT32_MIN, hi = INT32_MAX;
-    if (!(requant_conv<ACT>((int)lo, s_src, s_flt, s_dst) < j))
+    if (!below(lo))
         return INT32_MIN;  // F never drops below j: entry not used (j <= lowest output)
-    while (lo < hi) {  // invariant: F(lo) < j
+    // the threshold is next to (j - 0.5) / c: try a bracket of +-8 around it first
+    if (c > 0.f) {
+        const float est = ((float)j - 0.5f) / c;
+        if (est > -2.0e9f && est < 2.0e9f) {
+            const long long e = (long long)est;
+            if (below(e - 8) && !below(e + 8)) {
+                lo = e - 8;
+                hi = e + 7;
+            }
+        }
+    }
+    while (lo < hi) {  // invariant: F(lo) < j, F(hi + 1) >= j or hi == INT32_MAX
         const long long mid = lo + (hi - lo + 1) / 2;
-        if (requant_conv<ACT>((int)mid, s_src, s_flt, s_dst) < j)
+        if (below(mid))
             lo = mid;
         else
             hi = mid - 1;

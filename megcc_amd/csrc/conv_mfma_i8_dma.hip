@@ -29,7 +29,8 @@ static constexpr int DM_BM = 128, DM_BNP = 256;
 
 // FH x FW taps, KS 32-channel sub-chunks per stage, LMAX patch slots (compile time, so that the
 // number of loads per stage is a constant the vmcnt waits can be written for).
-template <int FH, int FW, int KS, int LMAX, int ACT>
+// FC: dst is row-major [pixel][oc] (qsi8 FullyConnected as a 1x1 NCHW convolution on [M,K,1,1]).
+template <int FH, int FW, int KS, int LMAX, int ACT, bool FC>
 __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams q) {
     constexpr int MT = 2, NT = 2, WGN = 4;
     constexpr int TAPS = FH * FW;
@@ -87,12 +88,12 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
     // fetches plane (lane & 3) of slot (u % LW) * 16 + (lane >> 2). b_goff = byte offset of that
     // dword in the first plane group of a stage, or 2^31 (out of range -> zero) for padding.
     unsigned b_goff[B_PER_WAVE];
-    auto describe = [&](int p0) {
+    auto describe = [&](int p0) __attribute__((always_inline)) {
         const int plast = min(p0 + DM_BNP, range1) - 1;
         const int vp0 = vp_of(q, p0);
         const int L = vp_of(q, plast) + ((FH - 1) * q.DH) * q.VW + (FW - 1) * q.DW - vp0 + 1;
-#pragma unroll
-        for (int j = 0; j < B_PER_WAVE; ++j) {
+        static_for<B_PER_WAVE>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
             const int u = wave + j * DM_WAVES;
             const int kh = u / LW, slot = (u - kh * LW) * 16 + (lane >> 2);
             unsigned off = 0x80000000u;
@@ -106,22 +107,22 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
                           ((kh >> 1) * 8 + (kh & 1) * 4 + (lane & 3)) * q.plane_stride;
             }
             b_goff[j] = off;
-        }
+        });
     };
     int lp0 = range0, lst = 0, lbuf = 0;  // load cursor: sub-tile, stage in it, LDS buffer
     describe(lp0);
-    auto issue = [&](int8_t* buf) {
+    auto issue = [&](int8_t* buf) __attribute__((always_inline)) {
         const int8_t* abase = q.wp + ((size_t)lst * TS * q.OCP + oc0) * KROW;
 #pragma unroll
         for (int a = 0; a < A_PER_WAVE; ++a)
             dma_global_b128(abase + ((a_chunk[a] >> 2) * q.OCP * KROW + (a_chunk[a] & 3) * 1024) + lane16,
                             lds_address(buf + a_chunk[a] * 1024));
         const unsigned poff = (unsigned)(lst * KS * 8) * (unsigned)q.plane_stride;
-#pragma unroll
-        for (int j = 0; j < B_PER_WAVE; ++j) {
+        static_for<B_PER_WAVE>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
             const int u = wave + j * DM_WAVES;
             dma_buffer_b32(src_rsrc, b_goff[j] + poff, lds_address(buf + A_BYTES + u * 256));
-        }
+        });
         if (++lst == stages) {
             lst = 0;
             lp0 += DM_BNP;
@@ -146,7 +147,7 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
     // as one straight-line block so that its 4 bias reads and 16 table look-ups are in flight
     // together. ob: dword index in dst of this lane's pixel in oc-group 0 (-1: lane beyond the
     // sub-tile, -2: whole 32-pixel column beyond it, wave-uniform).
-    auto emit_tile = [&](auto mic, auto nic, const int ob, const int* tbl) {
+    auto emit_tile = [&](auto mic, auto nic, const int ob, const int* tbl) __attribute__((always_inline)) {
         constexpr int mi = decltype(mic)::value, ni = decltype(nic)::value;
         if (ob < -1)
             return;
@@ -179,10 +180,22 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
 #pragma unroll
             for (int e4 = 0; e4 < 4; ++e4) {
                 const int oc = oc0 + ocl + e4 * 8;
-                if (oc < q.OC) {
+                if (oc >= q.OC)
+                    continue;
+                const uint32_t w = pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
+                if constexpr (!FC) {
                     const int o = ob + ((oc0 >> 2) + (wm * MT + mi) * 8 + e4 * 2) * q.OHW + kg_plane;
-                    ((uint32_t*)q.dst)[o] =
-                            pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
+                    ((uint32_t*)q.dst)[o] = w;
+                } else {  // ob = pixel (row of the output matrix)
+                    int8_t* o = q.dst + (size_t)ob * q.OC + oc;
+                    if ((q.OC & 3) == 0) {
+                        *(uint32_t*)o = w;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (oc + e < q.OC)
+                                o[e] = (int8_t)(w >> (8 * e));
+                    }
                 }
             }
         }
@@ -212,7 +225,10 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
             b_byte[ni] = (kg * LMAX + (p <= plast ? vp_of(q, p) - vp0 : 0)) * 16;
             cols += pc <= plast ? 1 : 0;
             const int pn = (int)fdiv(p, q.dOHW);
-            cur_o[ni] = pc > plast ? -2 : p <= plast ? pn * (q.OC >> 2) * q.OHW + (p - pn * q.OHW) : -1;
+            cur_o[ni] = pc > plast ? -2
+                        : p > plast ? -1
+                        : FC        ? p
+                                    : pn * (q.OC >> 2) * q.OHW + (p - pn * q.OHW);
         }
 #pragma unroll
         for (int mi = 0; mi < MT; ++mi)
@@ -222,14 +238,14 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
                 for (int e = 0; e < 16; ++e)
                     acc[mi][ni][e] = 0;
 
-        auto stage_body = [&](auto cols_c, const int8_t* bufA, int8_t* dma_buf) {
+        auto stage_body = [&](auto cols_c, const int8_t* bufA, int8_t* dma_buf) __attribute__((always_inline)) {
             constexpr int COLS = decltype(cols_c)::value;
             if (g + 2 < G)
                 issue(dma_buf);
             const int8_t* bufB = bufA + A_BYTES;
             if constexpr (COLS > 0) {
                 v4i fa[2][MT], fb[2][NT];
-                auto fetch = [&](auto tc) {
+                auto fetch = [&](auto tc) __attribute__((always_inline)) {
                     constexpr int t = decltype(tc)::value;
                     constexpr int ks = t / TAPS, tap = t % TAPS;
                     constexpr int fh = tap / FW, fw = tap % FW;
@@ -258,7 +274,7 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
                 });
             }
         };
-        auto run_stages = [&](auto cols_c) {
+        auto run_stages = [&](auto cols_c) __attribute__((always_inline)) {
             for (int st = 0; st < stages; ++st, ++g) {
                 stage_body(cols_c, lds + cbuf * BUF_BYTES, lds + lbuf * BUF_BYTES);
                 if (g + 2 < G)
@@ -283,7 +299,7 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
 }
 
 // ---- configurations --------------------------------------------------------------------------
-template <int FH, int FW, int KS, int LMAX>
+template <int FH, int FW, int KS, int LMAX, bool FC>
 static PipeConfig make_dma_config(int act, bool table_ok) {
     PipeConfig c;
     c.bm = DM_BM;
@@ -299,20 +315,32 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.fixed_lmax = LMAX;
     c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + DM_BM * 4;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC>;
     else if (act == MEGCC_NONLINE_RELU && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC>;
     else
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC>;
     return c;
 }
 
-// 3x3 layers (NCHW44) with at least 128 output channels and enough pixels to fill the chip
-bool conv_mfma_dma_config(const ConvGeom& g, PipeConfig* c) {
+// 3x3 and 1x1 NCHW44 layers and FullyConnected with at least 128 output channels and enough
+// pixels to fill the chip. 1x1: 128 input channels per stage (64 when IC <= 64).
+bool conv_mfma_dma_config(const ConvGeom& g, bool fc, PipeConfig* c) {
     const long P = (long)g.n * g.oh * g.ow;
-    if (!(g.fh == 3 && g.fw == 3) || g.fmt != MEGCC_FMT_NCHW44 || g.oc < 128 || P < 8192)
+    const bool k3 = g.fh == 3 && g.fw == 3, k1 = g.fh == 1 && g.fw == 1;
+    if (!(k3 || k1) || !(g.fmt == MEGCC_FMT_NCHW44 || fc) || g.oc < 128 || P < 8192)
         return false;
-    *c = make_dma_config<3, 3, 1, 512>(g.act, requant_table_ok(g.s_src, g.s_flt, g.s_dst));
+    if ((long)g.n * g.oc * g.oh * g.ow >= (1L << 31))
+        return false;  // 32-bit output offsets
+    const bool ok = requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    if (k3)
+        *c = make_dma_config<3, 3, 1, 512, false>(g.act, ok);
+    else if (fc)
+        *c = make_dma_config<1, 1, 4, 256, true>(g.act, ok);
+    else if (g.ic <= 64)
+        *c = make_dma_config<1, 1, 2, 256, false>(g.act, ok);
+    else
+        *c = make_dma_config<1, 1, 4, 256, false>(g.act, ok);
     return true;
 }
 

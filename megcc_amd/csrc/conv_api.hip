@@ -3,6 +3,7 @@
 // would TINYNN_ASSERT, and route to the kernel for the case:
 //   qsi8 NCHW44 DENSE, qsi8 FullyConnected (1x1 NCHW on [M,K,1,1])  -> conv_mfma_i8.hip
 //   qsi8 NCHW44 depthwise                                           -> dwconv.hip
+//   qsi8 3-channel NCHW -> NCHW44 3x3 stride 2 (first layer)        -> conv_first.hip
 //   f32 NCHW DENSE                                                  -> gemm_f32.hip
 //   everything else ConvGeneral accepts                             -> conv_direct.hip
 #include "common.h"
@@ -13,6 +14,8 @@ bool conv_mfma_supported(const ConvGeom& g);
 size_t conv_mfma_packed_bytes(const ConvGeom& g);
 TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed);
 TinyNNStatus conv_mfma_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+bool conv_first_supported(const ConvGeom& g);
+TinyNNStatus conv_first_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool dwconv44_supported(const ConvGeom& g);
 TinyNNStatus dwconv44_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool conv_f32_gemm_supported(const ConvGeom& g);
@@ -181,6 +184,8 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
     if (q8 && dwconv44_supported(g) && aligned4(src->ptr) && aligned4(flt->ptr) &&
         aligned4(dst->ptr))
         return dwconv44_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+    if (q8 && conv_first_supported(g) && aligned4(src->ptr) && aligned4(dst->ptr) && (!b || aligned4(b)))
+        return conv_first_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     if (f32 && conv_f32_gemm_supported(g))
         return conv_f32_gemm_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     return conv_direct_launch(g, f32, src->ptr, flt->ptr, b, dst->ptr);

@@ -101,6 +101,9 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.GROUP, 3, 512, 14, 14, 512, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW, A.GROUP, 2, 32, 28, 28, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 224, 224, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 3, 3, 64, 48, 24, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(27))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 32, 36, 8, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(27))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 30, 34, 8, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),  # generic path (IW % 4 != 0)
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
     PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE, 5, 1024, 7, 7, 7, 7, 0),

@@ -4,6 +4,8 @@
 // aligned dword each; consecutive lanes walk W, which makes every load and the store coalesced.
 // Bandwidth-bound (18 int ops per byte moved): no MFMA. Same accumulator and epilogue as the
 // reference's generic loop (ConvKernel.cpp:305-344,374-380).
+#include <stdlib.h>
+
 #include "common.h"
 #include "conv_geom.h"
 #include "epilogue.cuh"
@@ -54,6 +56,149 @@ __global__ void __launch_bounds__(256) dwconv44_q8_kernel(
     }
 }
 
+
+// ---- 3x3, pad 1, stride 1 or 2 -----------------------------------------------------------------
+// One thread = 4 horizontally adjacent output pixels x the 4 channels of one NCHW44 plane group.
+// The pixels of an input row arrive as aligned 16-byte loads (4 pixels x 4 channels); a 4x4 byte
+// transpose (8 v_perm) turns them into one dword per channel holding 4 consecutive pixels, so the
+// three horizontal taps of an output pixel are adjacent bytes of one dword (a v_perm / shift away)
+// and meet the weights (w0, w1, w2, 0) of that channel and filter row in ONE v_dot4_i32_i8.
+// All loads are buffer loads: rows above / below the image, the left and right neighbour column
+// and anything past the end of the tensor use an out-of-range offset and read as zero, so padding
+// needs no branches; pixels past the end of a ragged row are masked after the transpose.
+typedef unsigned dw_v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void transpose4x4(const dw_v4u p, unsigned (&t)[4]) {
+    const unsigned lo01 = __builtin_amdgcn_perm(p[1], p[0], 0x05010400u);
+    const unsigned hi01 = __builtin_amdgcn_perm(p[1], p[0], 0x07030602u);
+    const unsigned lo23 = __builtin_amdgcn_perm(p[3], p[2], 0x05010400u);
+    const unsigned hi23 = __builtin_amdgcn_perm(p[3], p[2], 0x07030602u);
+    t[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+    t[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+    t[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+    t[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+}
+
+template <int S, int ACT>
+__global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
+        ConvGeom g, RequantFast rq, const uint32_t* __restrict__ src, const uint32_t* __restrict__ flt,
+        const int32_t* __restrict__ bias, uint32_t* __restrict__ dst, int total, int src_bytes) {
+    const int c4n = g.oc >> 2;
+    const int ogn = (g.ow + 3) >> 2;  // groups of 4 output pixels per row
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, src_bytes, 0x00020000);
+    const int OOB = (int)0x80000000u;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
+        int r = i;
+        const int og = r % ogn; r /= ogn;
+        const int oh = r % g.oh; r /= g.oh;
+        const int c4 = r % c4n;
+        const int n = r / c4n;
+        const int plane_off = ((n * c4n + c4) * g.ih) * g.iw * 4;  // bytes
+        // weights: per filter row one dword per channel = (w(fw=0), w(fw=1), w(fw=2), 0)
+        unsigned wq[3][4];
+#pragma unroll
+        for (int fh = 0; fh < 3; ++fh) {
+            const uint32_t* f = flt + (size_t)c4 * 9 + fh * 3;
+            const dw_v4u fv = {f[0], f[1], f[2], 0u};
+            transpose4x4(fv, wq[fh]);
+        }
+        int acc[4][4];  // [pixel][channel]
+        {
+            int b4[4] = {0, 0, 0, 0};
+            if (bias) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    b4[c] = bias[c4 * 4 + c];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    acc[j][c] = b4[c];
+        }
+        const int iw0 = og * 4 * S;  // first input pixel of the aligned loads
+#pragma unroll
+        for (int fh = 0; fh < 3; ++fh) {
+            const int ih = oh * S - 1 + fh;
+            const bool row_ok = (unsigned)ih < (unsigned)g.ih;
+            const int row_off = plane_off + ih * g.iw * 4;
+            // left neighbour pixel (iw0 - 1), pixel-major dword
+            const unsigned pv = __builtin_amdgcn_raw_buffer_load_b32(
+                    rs, row_ok && iw0 > 0 ? row_off + (iw0 - 1) * 4 : OOB, 0, 0);
+            dw_v4u l0 = __builtin_amdgcn_raw_buffer_load_b128(rs, row_ok ? row_off + iw0 * 4 : OOB, 0, 0);
+            // pixels past the end of the row belong to the next row: zero them
+            const int left = g.iw - iw0;  // valid pixels from iw0 on
+#pragma unroll
+            for (int k = 1; k < 4; ++k)
+                l0[k] = k < left ? l0[k] : 0u;
+            unsigned t0[4];
+            transpose4x4(l0, t0);
+            if (S == 1) {
+                const unsigned nx = __builtin_amdgcn_raw_buffer_load_b32(
+                        rs, row_ok && left > 4 ? row_off + (iw0 + 4) * 4 : OOB, 0, 0);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const unsigned x0 = __builtin_amdgcn_perm(t0[c], pv, 0x06050400u | c);
+                    const unsigned x3 = __builtin_amdgcn_perm(nx, t0[c], 0x0c000302u | ((4u + c) << 16));
+                    acc[0][c] = __builtin_amdgcn_sdot4((int)x0, (int)wq[fh][c], acc[0][c], false);
+                    acc[1][c] = __builtin_amdgcn_sdot4((int)t0[c], (int)wq[fh][c], acc[1][c], false);
+                    acc[2][c] = __builtin_amdgcn_sdot4((int)(t0[c] >> 8), (int)wq[fh][c], acc[2][c], false);
+                    acc[3][c] = __builtin_amdgcn_sdot4((int)x3, (int)wq[fh][c], acc[3][c], false);
+                }
+            } else {
+                dw_v4u l1 = __builtin_amdgcn_raw_buffer_load_b128(
+                        rs, row_ok && left > 4 ? row_off + (iw0 + 4) * 4 : OOB, 0, 0);
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    l1[k] = k + 4 < left ? l1[k] : 0u;
+                unsigned t1[4];
+                transpose4x4(l1, t1);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const unsigned x0 = __builtin_amdgcn_perm(t0[c], pv, 0x06050400u | c);
+                    const unsigned x2 = __builtin_amdgcn_alignbyte(t1[c], t0[c], 3);
+                    acc[0][c] = __builtin_amdgcn_sdot4((int)x0, (int)wq[fh][c], acc[0][c], false);
+                    acc[1][c] = __builtin_amdgcn_sdot4((int)(t0[c] >> 8), (int)wq[fh][c], acc[1][c], false);
+                    acc[2][c] = __builtin_amdgcn_sdot4((int)x2, (int)wq[fh][c], acc[2][c], false);
+                    acc[3][c] = __builtin_amdgcn_sdot4((int)(t1[c] >> 8), (int)wq[fh][c], acc[3][c], false);
+                }
+            }
+        }
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int q[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (ACT < 0)
+                    q[c] = requant_conv_rt(g.act, acc[j][c], g.s_src, g.s_flt, g.s_dst);
+                else
+                    q[c] = requant_conv_fast<(ACT < 0 ? 0 : ACT)>(acc[j][c], rq);
+            }
+            o[j] = pack4_perm(q[0], q[1], q[2], q[3]);
+        }
+        uint32_t* out = dst + ((size_t)(n * c4n + c4) * g.oh + oh) * g.ow + og * 4;
+        if (og * 4 + 4 <= g.ow && (g.ow & 3) == 0) {
+            *(uint4*)out = make_uint4(o[0], o[1], o[2], o[3]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (og * 4 + j < g.ow)
+                    out[j] = o[j];
+        }
+    }
+}
+
+// 3x3, pad 1, no dilation, stride 1 or 2 (square), rows that start 16-byte aligned
+static bool dwconv44_3x3_ok(const ConvGeom& g, const void* src, const void* dst) {
+    const long src_bytes = (long)g.n * g.ic * g.ih * g.iw;
+    const long groups4 = (long)g.n * (g.oc >> 2) * g.oh * ((g.ow + 3) / 4);
+    return g.fh == 3 && g.fw == 3 && g.ph == 1 && g.pw == 1 && g.dh == 1 && g.dw == 1 &&
+           g.sh == g.sw && (g.sh == 1 || g.sh == 2) && (g.iw & 3) == 0 &&
+           ((uintptr_t)src & 15) == 0 && ((uintptr_t)dst & 15) == 0 && src_bytes < (1L << 31) && groups4 < (1L << 31) &&
+           (long)g.n * g.oc * g.oh * g.ow < (1L << 31);
+}
+
 bool dwconv44_supported(const ConvGeom& g) {
     return g.fmt == MEGCC_FMT_NCHW44 && g.groups > 1 && g.groups == g.ic && g.ic == g.oc &&
            (g.ic & 3) == 0;
@@ -64,6 +209,24 @@ TinyNNStatus dwconv44_launch(
     size_t total = (size_t)g.n * (g.oc >> 2) * g.oh * g.ow;
     if (total == 0)
         return TinyNN_SUCCESS;
+    if (dwconv44_3x3_ok(g, src, dst) && !getenv("MEGCC_DW_GENERIC")) {
+        const int groups4 = (int)((long)g.n * (g.oc >> 2) * g.oh * ((g.ow + 3) / 4));
+        unsigned nb = (unsigned)((groups4 + 255) / 256);
+        const RequantFast rq3 = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
+        void (*k3)(ConvGeom, RequantFast, const uint32_t*, const uint32_t*, const int32_t*, uint32_t*, int, int);
+        if (g.sh == 1)
+            k3 = g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_3x3_kernel<1, MEGCC_NONLINE_IDENTITY>
+               : g.act == MEGCC_NONLINE_RELU     ? dwconv44_3x3_kernel<1, MEGCC_NONLINE_RELU>
+                                                 : dwconv44_3x3_kernel<1, -1>;
+        else
+            k3 = g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_3x3_kernel<2, MEGCC_NONLINE_IDENTITY>
+               : g.act == MEGCC_NONLINE_RELU     ? dwconv44_3x3_kernel<2, MEGCC_NONLINE_RELU>
+                                                 : dwconv44_3x3_kernel<2, -1>;
+        hipLaunchKernelGGL(k3, dim3(nb), dim3(256), 0, stream(), g, rq3, (const uint32_t*)src,
+                           (const uint32_t*)flt, (const int32_t*)bias, (uint32_t*)dst, groups4,
+                           (int)((long)g.n * g.ic * g.ih * g.iw));
+        return check_launch("dwconv44_3x3");
+    }
     unsigned blocks = (unsigned)((total + 255) / 256);
     if (blocks > 65536u * 8)
         blocks = 65536u * 8;

@@ -100,6 +100,12 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.GROUP, 3, 512, 14, 14, 512, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW44, A.GROUP, 3, 512, 14, 14, 512, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW, A.GROUP, 2, 32, 28, 28, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    # dot4 depthwise kernel: ragged rows (OW % 4 != 0), odd heights, every activation
+    ConvCase(A.FMT_NCHW44, A.GROUP, 3, 16, 9, 28, 16, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 11, 20, 8, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 24, 13, 12, 24, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 1, 4, 5, 4, 4, 3, 1, 1, A.SIGMOID, scales=(0.02, 0.01, unsat(9) * 40)),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 5, 12, 7, 7, 12, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),  # generic path
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 224, 224, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 3, 3, 64, 48, 24, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(27))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 32, 36, 8, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(27))),

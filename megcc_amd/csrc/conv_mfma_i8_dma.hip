@@ -24,15 +24,20 @@
 namespace mg {
 
 static constexpr int ACT_RT = -1;
-static constexpr int DM_THREADS = 512, DM_WAVES = 8, DM_NBUF = 3;
-static constexpr int DM_BM = 128, DM_BNP = 256;
+static constexpr int DM_THREADS = 512, DM_WAVES = 8;
+static constexpr int DM_BNP = 256;
 
 // FH x FW taps, KS 32-channel sub-chunks per stage, LMAX patch slots (compile time, so that the
 // number of loads per stage is a constant the vmcnt waits can be written for).
 // FC: dst is row-major [pixel][oc] (qsi8 FullyConnected as a 1x1 NCHW convolution on [M,K,1,1]).
-template <int FH, int FW, int KS, int LMAX, int ACT, bool FC>
+// MT: 32-row MFMA tiles per wave along oc; the workgroup tile is 64 * MT output channels.
+// DM_NBUF: LDS stage buffers; the loads of stage g + DM_NBUF - 1 are issued at the start of stage g.
+// More, smaller stages keep more loads in flight per byte of LDS and push the (in-order) wait for
+// the previous sub-tile's output stores further back: what bandwidth-bound 1x1 layers need.
+template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF>
 __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams q) {
-    constexpr int MT = 2, NT = 2, WGN = 4;
+    constexpr int NT = 2, WGN = 4;
+    constexpr int DM_BM = 64 * MT;
     constexpr int TAPS = FH * FW;
     constexpr int TS = TAPS * KS;
     constexpr int A_BYTES = TS * DM_BM * KROW;
@@ -45,7 +50,8 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
     constexpr int LW = LMAX / 16;  // wave-loads per (sub-chunk, half)
     constexpr int N_DMA = A_PER_WAVE + B_PER_WAVE;
     constexpr int BUF_BYTES = A_BYTES + B_BYTES;
-    static_assert(N_DMA < 64, "vmcnt range");
+    constexpr int N_FLIGHT = N_DMA * (DM_NBUF - 2);  // loads allowed in flight at a stage's end
+    static_assert(N_FLIGHT < 64, "vmcnt range");
 
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];
     int* const rq_table = (int*)(lds + DM_NBUF * BUF_BYTES);
@@ -76,12 +82,11 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
     for (int i = 0; i < 4; ++i)
         src_rsrc[i] = __builtin_amdgcn_readfirstlane(src_rsrc[i]);
     // filter: chunk c = wave + 8a (wrapped: the surplus loads repeat a chunk, same bytes to the
-    // same place), c = 4 * tap-step + 1 KB part
+    // same place), c = (DM_BM / 32) * tap-step + 1 KB part
     int a_chunk[A_PER_WAVE];  // wave-uniform
 #pragma unroll
     for (int a = 0; a < A_PER_WAVE; ++a) {
-        int c = wave + a * DM_WAVES;
-        a_chunk[a] = c >= A_CHUNKS ? c - A_CHUNKS : c;
+        a_chunk[a] = (wave + a * DM_WAVES) % A_CHUNKS;
     }
     const int lane16 = lane * 16;
     // activations: wave-load u = wave + 8j covers 16 slots of (sub-chunk, half) u / LW; this lane
@@ -115,7 +120,8 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
         const int8_t* abase = q.wp + ((size_t)lst * TS * q.OCP + oc0) * KROW;
 #pragma unroll
         for (int a = 0; a < A_PER_WAVE; ++a)
-            dma_global_b128(abase + ((a_chunk[a] >> 2) * q.OCP * KROW + (a_chunk[a] & 3) * 1024) + lane16,
+            dma_global_b128(abase + ((a_chunk[a] / (DM_BM / 32)) * q.OCP * KROW +
+                                     (a_chunk[a] % (DM_BM / 32)) * 1024) + lane16,
                             lds_address(buf + a_chunk[a] * 1024));
         const unsigned poff = (unsigned)(lst * KS * 8) * (unsigned)q.plane_stride;
         static_for<B_PER_WAVE>([&](auto jc) {
@@ -201,14 +207,15 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
         }
     };
 
-    // ---- prologue: two stages in flight, the first one landed
-    issue(lds);
-    if (G > 1) {
-        issue(lds + BUF_BYTES);
-        wait_vmcnt<N_DMA>();
-    } else {
+    // ---- prologue: DM_NBUF - 1 stages in flight, the first one landed
+#pragma unroll
+    for (int i = 0; i < DM_NBUF - 1; ++i)
+        if (i < G)
+            issue(lds + i * BUF_BYTES);
+    if (G >= DM_NBUF - 1)
+        wait_vmcnt<N_FLIGHT>();
+    else
         wait_vmcnt<0>();
-    }
     lds_barrier();
 
     int g = 0, cbuf = 0;
@@ -240,7 +247,7 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
 
         auto stage_body = [&](auto cols_c, const int8_t* bufA, int8_t* dma_buf) __attribute__((always_inline)) {
             constexpr int COLS = decltype(cols_c)::value;
-            if (g + 2 < G)
+            if (g + DM_NBUF - 1 < G)
                 issue(dma_buf);
             const int8_t* bufB = bufA + A_BYTES;
             if constexpr (COLS > 0) {
@@ -277,8 +284,10 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
         auto run_stages = [&](auto cols_c) __attribute__((always_inline)) {
             for (int st = 0; st < stages; ++st, ++g) {
                 stage_body(cols_c, lds + cbuf * BUF_BYTES, lds + lbuf * BUF_BYTES);
-                if (g + 2 < G)
-                    wait_vmcnt<N_DMA>();
+                // stage g+1 must have landed; the DM_NBUF - 2 stages issued after it may be in
+                // flight (stores issued in between only make the wait longer, never shorter)
+                if (g + DM_NBUF - 1 < G)
+                    wait_vmcnt<N_FLIGHT>();
                 else
                     wait_vmcnt<0>();
                 lds_barrier();
@@ -299,8 +308,9 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
 }
 
 // ---- configurations --------------------------------------------------------------------------
-template <int FH, int FW, int KS, int LMAX, bool FC>
+template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3>
 static PipeConfig make_dma_config(int act, bool table_ok) {
+    constexpr int DM_BM = 64 * MT;
     PipeConfig c;
     c.bm = DM_BM;
     c.bn = DM_BNP;
@@ -313,23 +323,26 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.blocks_per_cu = 1;
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     c.fixed_lmax = LMAX;
-    c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + DM_BM * 4;
+    c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + 128 * 4;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF>;
     else if (act == MEGCC_NONLINE_RELU && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF>;
     else
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF>;
     return c;
 }
 
-// 3x3 and 1x1 NCHW44 layers and FullyConnected with at least 128 output channels and enough
-// pixels to fill the chip. 1x1: 128 input channels per stage (64 when IC <= 64).
+// 3x3 and 1x1 NCHW44 layers and FullyConnected with at least 128 output channels (64 for the 1x1
+// with 32 input channels) and enough pixels. 1x1: 128 input channels per stage (64 / 32 when
+// IC <= 64 / 32).
 bool conv_mfma_dma_config(const ConvGeom& g, bool fc, PipeConfig* c) {
     const long P = (long)g.n * g.oh * g.ow;
     const bool k3 = g.fh == 3 && g.fw == 3, k1 = g.fh == 1 && g.fw == 1;
-    if (!(k3 || k1) || !(g.fmt == MEGCC_FMT_NCHW44 || fc) || g.oc < 128 || P < 8192)
+    if (!(k3 || k1) || !(g.fmt == MEGCC_FMT_NCHW44 || fc) || g.oc < 64 || P < 2048)
         return false;
+    if (g.oc < 128 && !(k1 && !fc && g.ic <= 32))
+        return false;  // 64-channel tiles: only the bandwidth-bound 1x1 with 32 input channels
     if ((long)g.n * g.oc * g.oh * g.ow >= (1L << 31))
         return false;  // 32-bit output offsets
     const bool ok = requant_table_ok(g.s_src, g.s_flt, g.s_dst);
@@ -337,8 +350,10 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, PipeConfig* c) {
         *c = make_dma_config<3, 3, 1, 512, false>(g.act, ok);
     else if (fc)
         *c = make_dma_config<1, 1, 4, 256, true>(g.act, ok);
-    else if (g.ic <= 64)
-        *c = make_dma_config<1, 1, 2, 256, false>(g.act, ok);
+    else if (g.oc < 128)
+        *c = make_dma_config<1, 1, 1, 256, false, 1, 8>(g.act, ok);
+    else if (g.ic <= 128)
+        *c = make_dma_config<1, 1, 2, 256, false, 2, 6>(g.act, ok);
     else
         *c = make_dma_config<1, 1, 4, 256, false>(g.act, ok);
     return true;

@@ -189,13 +189,13 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
     }
 }
 
-// 3x3, pad 1, no dilation, stride 1 or 2 (square), rows that start 16-byte aligned
+// 3x3, pad 1, no dilation, stride 1 or 2 (square); buffer loads only need dword alignment
 static bool dwconv44_3x3_ok(const ConvGeom& g, const void* src, const void* dst) {
     const long src_bytes = (long)g.n * g.ic * g.ih * g.iw;
     const long groups4 = (long)g.n * (g.oc >> 2) * g.oh * ((g.ow + 3) / 4);
     return g.fh == 3 && g.fw == 3 && g.ph == 1 && g.pw == 1 && g.dh == 1 && g.dw == 1 &&
-           g.sh == g.sw && (g.sh == 1 || g.sh == 2) && (g.iw & 3) == 0 &&
-           ((uintptr_t)src & 15) == 0 && ((uintptr_t)dst & 15) == 0 && src_bytes < (1L << 31) && groups4 < (1L << 31) &&
+           g.sh == g.sw && (g.sh == 1 || g.sh == 2) &&
+           ((uintptr_t)src & 3) == 0 && ((uintptr_t)dst & 15) == 0 && src_bytes < (1L << 31) && groups4 < (1L << 31) &&
            (long)g.n * g.oc * g.oh * g.ow < (1L << 31);
 }
 

@@ -89,6 +89,8 @@ LIVE = [
     # MobileNet pointwise shapes
     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 32, 112, 112, 64, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(32))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 4, 512, 14, 14, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(512))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 16, 512, 14, 14, 1024, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(512))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 5, 32, 56, 56, 64, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(32))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 3, 1024, 7, 7, 1024, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(1024))),
     # FullyConnected = 1x1 NCHW conv on [M,K,1,1]
     ConvCase(A.FMT_NCHW, A.DENSE, 64, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(1024) / 2)),

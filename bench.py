@@ -32,8 +32,8 @@ PEAK_INT8_TOPS = 5000.0  # dense int8 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the default workload's kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by what a 256 MiB copy reads on the same counters: x2.000 / x1.000);
-# the counter runs and their figures are in profiles/conv_mfma_i8_wide__conv3x3_n32_c256_56x56.txt
-MEASURED_TRAFFIC = {"conv": (77040 * 2.000 + 41720 * 1.000) * 1024}
+# the counter runs and their figures are in profiles/conv_mfma_i8_dma__conv3x3_n32_c256_56x56.txt
+MEASURED_TRAFFIC = {"conv": (40920 * 2.000 + 25088 * 1.000) * 1024}
 
 
 class HipEvents:

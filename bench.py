@@ -69,7 +69,7 @@ def headline_case(n=32, c=256, hw=56):
 
 def make_workload(name):
     """-> (case, description, bound, algorithmic units per launch)"""
-    from cases import ConvCase, MultiTypeCase, PoolCase, TypeCvtCase
+    from cases import ConvCase, MatMulCase, MultiTypeCase, PoolCase, TypeCvtCase
     from megcc_amd import abi
     if name == "conv":
         case = headline_case()
@@ -104,6 +104,12 @@ def make_workload(name):
     if name == "add":
         return (MultiTypeCase(abi.Q_FUSE_ADD_RELU, (64, 32, 56, 56), (0.05, 0.01, 0.05)),
                 "qsi8 QFUSE_ADD_RELU 64x32x56x56", "hbm")
+    if name in ("mm", "mm64", "mm1"):
+        m, k, n = {"mm": (4096, 4096, 4096), "mm64": (64, 4096, 4096), "mm1": (1, 1024, 1000)}[name]
+        return MatMulCase(m, k, n), "f32 MatMul %dx%dx%d" % (m, k, n), "mfma_f32"
+    if name == "conv_f32":
+        case = ConvCase(abi.FMT_NCHW, abi.DENSE, 1, 32, 56, 56, 32, 3, 1, 1, abi.RELU, dtype="f32")
+        return case, "f32 conv3x3 NCHW N=1 C=32 56x56 +bias +ReLU", "mfma_f32"
     if name == "copy":  # same-scale requantise = a plain copy: the counter calibration kernel
         return (TypeCvtCase("qsi8", "qsi8", (256, 1024, 1024), src_scale=0.05, dst_scale=0.05),
                 "qsi8->qsi8 typecvt, equal scales, 256 MiB in + 256 MiB out", "hbm")
@@ -230,7 +236,12 @@ def main():
     ops = case.ops() if hasattr(case, "ops") else 0
     nbytes = case_bytes(case)
     ms = wall * 1e3 / args.steps
-    if bound == "mfma":
+    if bound == "mfma_f32":
+        bound = "mfma"
+        value, unit, metric = ops / (wall / args.steps) / 1e12, "TFLOP/s", "f32_tflops"
+        roof = {"bound": "mfma", "achieved": round(ops / (kern_ms * 1e-3) / 1e12, 3),
+                "peak": 157.3, "unit": "TFLOP/s", "traffic": None}
+    elif bound == "mfma":
         value, unit, metric = ops / (wall / args.steps) / 1e12, "TOP/s", "int8_conv_tops"
         roof = {"bound": "mfma", "achieved": round(ops / (kern_ms * 1e-3) / 1e12, 3),
                 "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "traffic": None}
@@ -248,7 +259,7 @@ def main():
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8", "data": "synthetic",
+        "dtype": "f32" if unit == "TFLOP/s" else "int8", "data": "synthetic",
         "config": {"workload": desc, "symbol": case.symbol(), "abi": "megcc_gfx950_call"},
         "roofline": roof,
     }

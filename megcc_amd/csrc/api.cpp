@@ -264,9 +264,10 @@ extern "C" TinyNNStatus megcc_gfx950_call_init(
 extern "C" TinyNNStatus megcc_gfx950_call_workspace(
         const MegccKernelDesc* d, Tensor** inputs, int nr_input, int nr_thread, size_t* workspace) {
     MG_REQUIRE(d && workspace, TinyNN_ERROR_NULL_PTR, "call_workspace: NULL argument");
-    (void)inputs;
-    (void)nr_input;
-    (void)nr_thread;
-    *workspace = 0;  // no kernel of this library needs scratch memory
+    if (d->kind == MEGCC_KERN_CONV)
+        return megcc_gfx950_conv2d_workspace(&d->attr.conv, inputs, nr_input, nr_thread, workspace);
+    if (d->kind == MEGCC_KERN_MATMUL)
+        return megcc_gfx950_matmul_workspace(&d->attr.matmul, inputs, nr_input, nr_thread, workspace);
+    *workspace = 0;  // the other kernels of this library need no scratch memory
     return TinyNN_SUCCESS;
 }

@@ -19,7 +19,9 @@ TinyNNStatus conv_first_launch(const ConvGeom&, const void*, const void*, const 
 bool dwconv44_supported(const ConvGeom& g);
 TinyNNStatus dwconv44_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool conv_f32_gemm_supported(const ConvGeom& g);
-TinyNNStatus conv_f32_gemm_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+TinyNNStatus conv_f32_gemm_launch(const ConvGeom&, const void*, const void*, const void*, void*,
+                                  const Workspace*);
+size_t conv_f32_gemm_workspace_bytes(const ConvGeom& g);
 TinyNNStatus conv_direct_launch(const ConvGeom&, bool, const void*, const void*, const void*, void*);
 
 // A filter that went through megcc_gfx950_conv2d_init is a 1-d byte tensor.
@@ -132,7 +134,7 @@ using namespace mg;
 
 extern "C" TinyNNStatus megcc_gfx950_conv2d(
         const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
-        const Workspace*, const RuntimeOpt*) {
+        const Workspace* workspace, const RuntimeOpt*) {
     MG_REQUIRE(attr, TinyNN_ERROR_NULL_PTR, "conv2d: NULL attr");
     const int want_in = attr->with_bias ? 3 : 2;
     // the test harness of the reference passes an extra empty `z` operand after the bias
@@ -187,7 +189,7 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
     if (q8 && conv_first_supported(g) && aligned4(src->ptr) && aligned4(dst->ptr) && (!b || aligned4(b)))
         return conv_first_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     if (f32 && conv_f32_gemm_supported(g))
-        return conv_f32_gemm_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+        return conv_f32_gemm_launch(g, src->ptr, flt->ptr, b, dst->ptr, workspace);
     return conv_direct_launch(g, f32, src->ptr, flt->ptr, b, dst->ptr);
 }
 
@@ -233,9 +235,20 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d_init(
     return conv_mfma_pack(g, flt->ptr, out_weights->ptr);
 }
 
+// im2col never leaves LDS, so the quantized kernels need no scratch; the f32 implicit GEMM asks
+// for room for split-K partial sums when the layer has too few tiles to fill the chip.
 extern "C" TinyNNStatus megcc_gfx950_conv2d_workspace(
-        const MegccConvAttr*, Tensor**, int, int, size_t* workspace) {
+        const MegccConvAttr* attr, Tensor** inputs, int nr_input, int, size_t* workspace) {
     MG_REQUIRE(workspace, TinyNN_ERROR_NULL_PTR, "conv2d_workspace: NULL size");
     *workspace = 0;
+    if (!attr || !inputs || nr_input < 2 || !inputs[0] || !inputs[1])
+        return TinyNN_SUCCESS;
+    const Tensor *src = inputs[0], *flt = inputs[1];
+    if (is_f32(src) && is_f32(flt)) {
+        ConvGeom g;
+        if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS &&
+            conv_f32_gemm_supported(g))
+            *workspace = conv_f32_gemm_workspace_bytes(g);
+    }
     return TinyNN_SUCCESS;
 }

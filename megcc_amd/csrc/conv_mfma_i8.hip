@@ -411,7 +411,7 @@ TinyNNStatus conv_mfma_launch(
         const long gather_items =
                 pc.g4 ? 8L * pc.ks * t.rows_max * (g.iw / 4) : 2L * pc.ks * t.Lmax;
         pipe = (pc.gather_threads == 0 || gather_items <= (long)pc.maxb * pc.gather_threads) &&
-               (long)pc.nbuf * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) + pc.extra_lds <= 160 * 1024;
+               ((long)pc.nbuf * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) + pc.extra_lds) * pc.blocks_per_cu <= 160 * 1024;
     }
     if (!pipe) {
         range_len = 0;

@@ -24,7 +24,6 @@
 namespace mg {
 
 static constexpr int ACT_RT = -1;
-static constexpr int DM_THREADS = 512, DM_WAVES = 8;
 static constexpr int DM_BNP = 256;
 
 // FH x FW taps, KS 32-channel sub-chunks per stage, LMAX patch slots (compile time, so that the
@@ -34,10 +33,15 @@ static constexpr int DM_BNP = 256;
 // DM_NBUF: LDS stage buffers; the loads of stage g + DM_NBUF - 1 are issued at the start of stage g.
 // More, smaller stages keep more loads in flight per byte of LDS and push the (in-order) wait for
 // the previous sub-tile's output stores further back: what bandwidth-bound 1x1 layers need.
-template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF>
-__global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams q) {
+// WGM: waves along oc (1 or 2; 4 waves along pixels). WGM = 1 gives 256-thread workgroups of which
+// two share a CU (launch bound 2): their phases drift apart, so one's epilogue, barrier and load
+// waits overlap the other's MFMAs.
+// BPC: workgroups per CU the register budget is set for.
+template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC>
+__global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaParams q) {
     constexpr int NT = 2, WGN = 4;
-    constexpr int DM_BM = 64 * MT;
+    constexpr int DM_WAVES = WGM * WGN, DM_THREADS = 64 * DM_WAVES;
+    constexpr int DM_BM = 32 * MT * WGM;
     constexpr int TAPS = FH * FW;
     constexpr int TS = TAPS * KS;
     constexpr int A_BYTES = TS * DM_BM * KROW;
@@ -51,7 +55,7 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
     constexpr int N_DMA = A_PER_WAVE + B_PER_WAVE;
     constexpr int BUF_BYTES = A_BYTES + B_BYTES;
     constexpr int N_FLIGHT = N_DMA * (DM_NBUF - 2);  // loads allowed in flight at a stage's end
-    static_assert(N_FLIGHT < 64, "vmcnt range");
+    static_assert(N_FLIGHT < 64 && DM_NBUF >= 2, "vmcnt range");
 
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];
     int* const rq_table = (int*)(lds + DM_NBUF * BUF_BYTES);
@@ -71,10 +75,8 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
         if (tid < REQUANT_TABLE_ENTRIES)
             rq_table[tid] = tid < 255 ? requant_threshold<ACT>(tid, q.s_src, q.s_flt, q.s_dst, q.rq.c) : 0;
     }
-    if (tid >= 256 && tid < 256 + DM_BM) {
-        const int oc = oc0 + tid - 256;
-        bias_lds[tid - 256] = (q.bias && oc < q.OC) ? q.bias[oc] : 0;
-    }
+    for (int i = tid; i < DM_BM; i += DM_THREADS)
+        bias_lds[i] = (q.bias && oc0 + i < q.OC) ? q.bias[oc0 + i] : 0;
 
     // ---- load side ---------------------------------------------------------------------------
     v4u src_rsrc = make_raw_buffer(q.src, (unsigned)q.src_bytes);
@@ -308,28 +310,28 @@ __global__ void __launch_bounds__(DM_THREADS) conv_mfma_i8_dma_kernel(MfmaParams
 }
 
 // ---- configurations --------------------------------------------------------------------------
-template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3>
+template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3, int WGM = 2, int BPC = 1>
 static PipeConfig make_dma_config(int act, bool table_ok) {
-    constexpr int DM_BM = 64 * MT;
+    constexpr int DM_BM = 32 * MT * WGM;
     PipeConfig c;
     c.bm = DM_BM;
     c.bn = DM_BNP;
     c.ks = KS;
     c.maxb = 0;
     c.g4 = 0;
-    c.threads = DM_THREADS;
+    c.threads = 256 * WGM;
     c.gather_threads = 0;
     c.nbuf = DM_NBUF;
-    c.blocks_per_cu = 1;
+    c.blocks_per_cu = BPC;
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     c.fixed_lmax = LMAX;
     c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + 128 * 4;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC>;
     else if (act == MEGCC_NONLINE_RELU && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF, WGM, BPC>;
     else
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC>;
     return c;
 }
 
@@ -346,6 +348,8 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, PipeConfig* c) {
     if ((long)g.n * g.oc * g.oh * g.ow >= (1L << 31))
         return false;  // 32-bit output offsets
     const bool ok = requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    // measured slower on the 256-channel 56x56 layer (91 us): two 256-thread workgroups per CU
+    // with 64-channel tiles and two buffers (100 us), four waves of 128 oc x 64 pixels (107 us)
     if (k3)
         *c = make_dma_config<3, 3, 1, 512, false>(g.act, ok);
     else if (fc)

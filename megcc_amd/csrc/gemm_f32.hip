@@ -31,6 +31,10 @@ struct GemmArgs {
     int act;
     ConvGeom g;  // convolution only
     int is_conv;
+    // split-K: blockIdx.z handles k in [z*kchunk, (z+1)*kchunk) and writes its partial sums to
+    // partial[z][M][N]; gemm_f32_reduce_kernel adds them in z order (deterministic) and stores
+    int split, kchunk;
+    float* partial;
 };
 
 __device__ __forceinline__ float act_rt(int act, float x) {
@@ -77,7 +81,9 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
             for (int e = 0; e < 16; ++e)
                 acc[i][j][e] = 0.f;
 
-    for (int k0 = 0; k0 < q.K; k0 += GBK) {
+    const int k_begin = blockIdx.z * q.kchunk;
+    const int k_end = min(q.K, k_begin + q.kchunk);
+    for (int k0 = k_begin; k0 < k_end; k0 += GBK) {
         // ---- stage A tile (GBM x GBK) and B tile (GBK x GBN): 8 elements per thread each
 #pragma unroll
         for (int it = 0; it < 8; ++it) {
@@ -90,7 +96,7 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
                 k = (tid >> 7) + it * 2;
             }
             float v = 0.f;
-            if (m0 + m < q.M && k0 + k < q.K)
+            if (m0 + m < q.M && k0 + k < k_end)
                 v = q.A[(size_t)(m0 + m) * q.a_rs + (size_t)(k0 + k) * q.a_cs];
             As[k][m] = v;
         }
@@ -105,7 +111,7 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
                 n = (tid >> 4) + it * 16;
             }
             float v = 0.f;
-            if (n0 + n < q.N && k0 + k < q.K) {
+            if (n0 + n < q.N && k0 + k < k_end) {
                 if (CONV)
                     v = conv_b(q, k0 + k, n0 + n);
                 else
@@ -157,7 +163,9 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
                 if (m >= q.M)
                     continue;
                 float v = acc[i][j][e];
-                if (CONV) {
+                if (q.split > 1) {
+                    q.partial[((size_t)blockIdx.z * q.M + m) * q.N + n] = v;
+                } else if (CONV) {
                     if (q.bias)
                         v += q.bias[m];
                     v = act_rt(q.act, v);
@@ -169,14 +177,83 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
     }
 }
 
+// sums the split-K partials in a fixed order and stores like the unsplit kernel would
+__global__ void __launch_bounds__(256) gemm_f32_reduce_kernel(GemmArgs q) {
+    const size_t total = (size_t)q.M * q.N;
+    for (size_t i = blockIdx.x * (size_t)256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const int m = (int)(i / q.N), n = (int)(i - (size_t)m * q.N);
+        float v = 0.f;
+        for (int z = 0; z < q.split; ++z)
+            v += q.partial[(size_t)z * total + i];
+        if (q.is_conv) {
+            if (q.bias)
+                v += q.bias[m];
+            v = act_rt(q.act, v);
+            const int ohw = q.g.oh * q.g.ow;
+            const int img = n / ohw, rem = n - img * ohw;
+            q.C[((size_t)img * q.M + m) * ohw + rem] = v;
+        } else {
+            q.C[(size_t)m * q.ldc + n] = v;
+        }
+    }
+}
+
+// Split factor for problems with too few 128 x 128 tiles to fill the chip (skinny M: GEVM,
+// batch-64 FullyConnected, the small f32 convolution). A pure function of the shape, so that the
+// _workspace entry point and the kernel agree.
+static int gemm_split(long M, long N, long K) {
+    const long tiles = ((M + GBM - 1) / GBM) * ((N + GBN - 1) / GBN);
+    if (tiles >= 192 || K < 128)
+        return 1;
+    long s = (512 + tiles - 1) / tiles;
+    const long max_s = K / 64;
+    if (s > max_s)
+        s = max_s;
+    if (s > 64)
+        s = 64;
+    return s < 2 ? 1 : (int)s;
+}
+
+size_t gemm_f32_workspace_bytes(long M, long N, long K) {
+    const int s = gemm_split(M, N, K);
+    return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+}
+
+// chooses the split for (q.M, q.N, q.K) if the workspace can hold the partials
+static void gemm_plan_split(GemmArgs& q, const Workspace* ws) {
+    q.split = 1;
+    q.kchunk = (q.K + GBK - 1) / GBK * GBK;
+    q.partial = nullptr;
+    const int s = gemm_split(q.M, q.N, q.K);
+    if (s > 1 && ws && ws->ptr && ws->size >= gemm_f32_workspace_bytes(q.M, q.N, q.K) &&
+        ((uintptr_t)ws->ptr & 3) == 0) {
+        q.split = s;
+        q.kchunk = ((q.K + s - 1) / s + GBK - 1) / GBK * GBK;
+        q.partial = (float*)ws->ptr;
+    }
+}
+
+static void gemm_launch_reduce(const GemmArgs& q) {
+    const size_t total = (size_t)q.M * q.N;
+    unsigned blocks = (unsigned)((total + 255) / 256);
+    if (blocks > 8192)
+        blocks = 8192;
+    hipLaunchKernelGGL(gemm_f32_reduce_kernel, dim3(blocks), dim3(256), 0, stream(), q);
+}
+
 bool conv_f32_gemm_supported(const ConvGeom& g) {
     long P = (long)g.n * g.oh * g.ow;
     return g.fmt == MEGCC_FMT_NCHW && g.groups == 1 && P < (1L << 31) &&
            (long)g.ic * g.fh * g.fw < (1L << 31);
 }
 
+size_t conv_f32_gemm_workspace_bytes(const ConvGeom& g) {
+    return gemm_f32_workspace_bytes(g.oc, (long)g.n * g.oh * g.ow, (long)g.ic * g.fh * g.fw);
+}
+
 TinyNNStatus conv_f32_gemm_launch(
-        const ConvGeom& g, const void* src, const void* flt, const void* bias, void* dst) {
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, void* dst,
+        const Workspace* ws) {
     GemmArgs q;
     q.A = (const float*)flt;  // [OC][IC*FH*FW]
     q.B = (const float*)src;
@@ -194,8 +271,11 @@ TinyNNStatus conv_f32_gemm_launch(
     q.is_conv = 1;
     if (q.M == 0 || q.N == 0)
         return TinyNN_SUCCESS;
-    dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM);
+    gemm_plan_split(q, ws);
+    dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM, q.split);
     hipLaunchKernelGGL((gemm_f32_kernel<true, true, true>), grid, dim3(256), 0, stream(), q);
+    if (q.split > 1)
+        gemm_launch_reduce(q);
     return check_launch("conv_f32_gemm");
 }
 
@@ -205,7 +285,7 @@ using namespace mg;
 
 extern "C" TinyNNStatus megcc_gfx950_matmul(
         const MegccMatMulAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs,
-        int nr_output, const Workspace*, const RuntimeOpt*) {
+        int nr_output, const Workspace* ws, const RuntimeOpt*) {
     MG_REQUIRE(attr, TinyNN_ERROR_NULL_PTR, "matmul: NULL attr");
     TinyNNStatus st = check_io(inputs, nr_input, 2, 2, outputs, nr_output, "matmul");
     if (st != TinyNN_SUCCESS)
@@ -242,7 +322,8 @@ extern "C" TinyNNStatus megcc_gfx950_matmul(
     q.is_conv = 0;
     if (q.M == 0 || q.N == 0)
         return TinyNN_SUCCESS;
-    dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM);
+    gemm_plan_split(q, ws);
+    dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM, q.split);
     if (!ta && !tb)
         hipLaunchKernelGGL((gemm_f32_kernel<true, true, false>), grid, dim3(256), 0, stream(), q);
     else if (!ta && tb)
@@ -251,14 +332,26 @@ extern "C" TinyNNStatus megcc_gfx950_matmul(
         hipLaunchKernelGGL((gemm_f32_kernel<false, true, false>), grid, dim3(256), 0, stream(), q);
     else
         hipLaunchKernelGGL((gemm_f32_kernel<false, false, false>), grid, dim3(256), 0, stream(), q);
+    if (q.split > 1)
+        gemm_launch_reduce(q);
     return check_launch("matmul");
 }
 
-// No scratch: tiles are staged straight from the operands (the reference packs A and B into
-// workspace, GeneralIntrinsic/MatMulKernel/Fp32MatMulM4N12.cpp:47-66).
+// Tiles are staged straight from the operands (the reference packs A and B into workspace,
+// GeneralIntrinsic/MatMulKernel/Fp32MatMulM4N12.cpp:47-66); the only scratch is the split-K partial
+// sums of skinny problems. Without it (NULL or short workspace) the kernel runs unsplit.
 extern "C" TinyNNStatus megcc_gfx950_matmul_workspace(
-        const MegccMatMulAttr*, Tensor**, int, int, size_t* workspace) {
+        const MegccMatMulAttr* attr, Tensor** inputs, int nr_input, int, size_t* workspace) {
     MG_REQUIRE(workspace, TinyNN_ERROR_NULL_PTR, "matmul_workspace: NULL size");
     *workspace = 0;
+    if (!attr || !inputs || nr_input < 2 || !inputs[0] || !inputs[1] ||
+        inputs[0]->layout.nr_dim != 2 || inputs[1]->layout.nr_dim != 2)
+        return TinyNN_SUCCESS;
+    const Tensor *a = inputs[0], *b = inputs[1];
+    const int ta = attr->transpose_a != 0, tb = attr->transpose_b != 0;
+    const long M = ta ? a->layout.dims[1] : a->layout.dims[0];
+    const long K = ta ? a->layout.dims[0] : a->layout.dims[1];
+    const long N = tb ? b->layout.dims[0] : b->layout.dims[1];
+    *workspace = gemm_f32_workspace_bytes(M, N, K);
     return TinyNN_SUCCESS;
 }

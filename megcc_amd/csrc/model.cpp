@@ -53,6 +53,10 @@ struct Model {
     std::vector<ModelOpr*> oprs;
     void* arena = nullptr;
     size_t arena_bytes = 0;
+    // one scratch buffer shared by all operators (they run one after the other on one stream),
+    // sized for the largest request of any operator's _workspace function
+    void* workspace = nullptr;
+    size_t workspace_bytes = 0;
     bool finalized = false;
 };
 
@@ -154,6 +158,8 @@ void megcc_gfx950_model_destroy(void* model) {
     }
     if (m->arena)
         m->dev.free(m->arena);
+    if (m->workspace)
+        m->dev.free(m->workspace);
     delete m;
 }
 
@@ -338,6 +344,24 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
             MG_REQUIRE(o->has_processed, TinyNN_ERROR_NO_FOUND,
                        "model_finalize: %s: processed weight matches no input", o->symbol.c_str());
         }
+    }
+    // workspaces (runtime/src/init.c: the VM shares one workspace region between operators)
+    for (auto* o : m->oprs) {
+        size_t bytes = 0;
+        TinyNNStatus st = megcc_gfx950_call_workspace(
+                &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), 1, &bytes);
+        if (st != TinyNN_SUCCESS)
+            return st;
+        o->ws.size = bytes;
+        if (bytes > m->workspace_bytes)
+            m->workspace_bytes = bytes;
+    }
+    if (m->workspace_bytes) {
+        m->workspace = m->dev.malloc(m->workspace_bytes);
+        MG_REQUIRE(m->workspace, TinyNN_ERROR_MEMORY_MALLOC, "model_finalize: workspace of %zu bytes",
+                   m->workspace_bytes);
+        for (auto* o : m->oprs)
+            o->ws.ptr = o->ws.size ? m->workspace : nullptr;
     }
     m->finalized = true;
     return megcc_gfx950_wait();

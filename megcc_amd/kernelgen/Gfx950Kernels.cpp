@@ -78,6 +78,20 @@ std::string KernelFuncBase::GetWorkspaceBody(TContext* c) const {
 
 namespace {
 
+static const char* kSplitBody =
+        "    /* room for the split-K partial sums of problems with too few 128 x 128 tiles to fill\n"
+        "       the chip; the same formula as the library (gemm_f32.hip, gemm_split) */\n"
+        "    long tiles = ((M + 127) / 128) * ((N + 127) / 128), s = 1;\n"
+        "    if (tiles < 192 && K >= 128) {\n"
+        "        s = (512 + tiles - 1) / tiles;\n"
+        "        if (s > K / 64) s = K / 64;\n"
+        "        if (s > 64) s = 64;\n"
+        "        if (s < 2) s = 1;\n"
+        "    }\n"
+        "    *workspace = s > 1 ? (size_t)s * M * N * 4 : 0;\n"
+        "    return TinyNN_SUCCESS;\n}\n";
+
+
 // ---- dtype helpers (Utils/Utils.h:41-140, Utils/SymbolHelper.h:9-23) ---------------------------
 std::string valid_dtype(const std::string& d) {
     size_t p = d.find('<');
@@ -204,10 +218,27 @@ struct ConvKernel : KernelFuncBase {
                "nr_out_weight, opt);\n}\n";
     }
     // plain C, no external call: the compiler may evaluate it at compile time
-    // (compiler/lib/KernelGen/Jit/JitExe.cpp:67-123 forbids externs in workspace bodies)
+    // (compiler/lib/KernelGen/Jit/JitExe.cpp:67-123 forbids externs in workspace bodies).
+    // Quantized kernels need none (im2col stays in LDS); the f32 implicit GEMM may split K.
     std::string GetWorkspaceBody(TContext* c) const override {
-        return "TinyNNStatus " + GetWorkspaceSignature(c) +
-               " {\n    *workspace = 0;\n    return TinyNN_SUCCESS;\n}\n";
+        if (!is_f32(c->getAttrOprand("operand:0").dtype) || conv_format(c) != "NCHW" ||
+            c->getAttrStr("sparse") != "DENSE")
+            return "TinyNNStatus " + GetWorkspaceSignature(c) +
+                   " {\n    *workspace = 0;\n    return TinyNN_SUCCESS;\n}\n";
+        std::stringstream ss;
+        ss << "TinyNNStatus " << GetWorkspaceSignature(c) << " {\n"
+           << "    const Layout src = inputs[0]->layout, flt = inputs[1]->layout;\n"
+           << "    const long eh = " << c->getAttrUInt("dilate_h") << " * (" << c->getAttrUInt("kernel_h")
+           << " - 1) + 1, ew = " << c->getAttrUInt("dilate_w") << " * (" << c->getAttrUInt("kernel_w")
+           << " - 1) + 1;\n"
+           << "    const long ih = src.dims[2] + 2 * " << c->getAttrUInt("pad_h")
+           << ", iw = src.dims[3] + 2 * " << c->getAttrUInt("pad_w") << ";\n"
+           << "    const long oh = ih >= eh ? (ih - eh) / " << c->getAttrUInt("stride_h")
+           << " + 1 : 0, ow = iw >= ew ? (iw - ew) / " << c->getAttrUInt("stride_w") << " + 1 : 0;\n"
+           << "    const long M = flt.dims[0], N = (long)src.dims[0] * oh * ow, K = (long)src.dims[1] * "
+           << c->getAttrUInt("kernel_h") << " * " << c->getAttrUInt("kernel_w") << ";\n"
+           << kSplitBody;
+        return ss.str();
     }
 };
 
@@ -379,6 +410,16 @@ struct MatrixMulKernel : KernelFuncBase {
         return kHeader + kernel_def(this, c, a.str(),
                                     "megcc_gfx950_matmul(&attr, inputs, nr_input, outputs, "
                                     "nr_output, workspace, opt)");
+    }
+    std::string GetWorkspaceBody(TContext* c) const override {
+        const bool ta = c->getAttrBool("transposeA"), tb = c->getAttrBool("transposeB");
+        std::stringstream ss;
+        ss << "TinyNNStatus " << GetWorkspaceSignature(c) << " {\n"
+           << "    const Layout a = inputs[0]->layout, b = inputs[1]->layout;\n"
+           << "    const long M = a.dims[" << (ta ? 1 : 0) << "], K = a.dims[" << (ta ? 0 : 1)
+           << "], N = b.dims[" << (tb ? 0 : 1) << "];\n"
+           << kSplitBody;
+        return ss.str();
     }
 };
 

@@ -319,6 +319,9 @@ class MatMulCase:
     def __repr__(self):
         return "%s[%dx%dx%d]" % (self.symbol(), self.m, self.k, self.n)
 
+    def ops(self):
+        return 2 * self.m * self.n * self.k
+
     def symbol(self):
         """GeneralIntrinsic/MatMulKernel/Fp32Gevm.cpp:109-135 (M<=4, A not transposed) else
         Fp32MatMulM4N12.cpp:9-45"""

@@ -85,6 +85,37 @@ def test_shims_compile_and_link(shim_library):
         assert hasattr(lib, sym + "_workspace")
 
 
+def test_generated_workspace_functions_agree_with_the_library(shim_library):
+    """the shims compute workspace sizes in plain C (the compiler may run them at compile time);
+    they must ask for exactly what the kernels expect"""
+    lib, manifest = shim_library
+    L = runtime.lib()
+    checked = 0
+    for sym in sorted(set(manifest.values())):
+        desc = runtime.parse_symbol(sym)
+        if desc.kind == 2:  # MatrixMul
+            ta, tb = desc.attr.matmul.transpose_a, desc.attr.matmul.transpose_b
+            shapes = [(1, 1024, 1000), (64, 4096, 4096), (4096, 4096, 4096), (5, 100, 7), (300, 64, 200)]
+            cases_ = [[((k, m) if ta else (m, k)), ((n, k) if tb else (k, n))] for m, k, n in shapes]
+        elif desc.kind == 1 and "f32" in sym and "_NCHW_DENSE_" in sym:
+            k = desc.attr.conv.kernel_h
+            cases_ = [[(1, 32, 56, 56), (32, 32, k, k)], [(2, 5, 19, 23), (37, 5, k, k)],
+                      [(8, 64, 56, 56), (128, 64, k, k)]]
+        else:
+            continue
+        fn = getattr(lib, sym + "_workspace")
+        fn.argtypes = abi.WORKSPACE_ARGS
+        for shapes_ in cases_:
+            tin = [abi.make_tensor(None, s, abi.FLOAT, 1.0) for s in shapes_]
+            a, b = C.c_size_t(7), C.c_size_t(9)
+            assert fn(abi.tensor_array(tin), len(tin), 1, C.byref(a)) == 0
+            assert L.megcc_gfx950_call_workspace(C.byref(desc), abi.tensor_array(tin), len(tin), 1,
+                                                 C.byref(b)) == 0
+            assert a.value == b.value, (sym, shapes_, a.value, b.value)
+            checked += 1
+    assert checked >= 8
+
+
 @pytest.mark.gpu
 def test_conv_through_the_generated_shim(shim_library):
     """call the kernel the way the TinyNN runtime would: by its generated symbol"""

@@ -13,7 +13,9 @@ namespace mg {
 bool conv_mfma_supported(const ConvGeom& g);
 size_t conv_mfma_packed_bytes(const ConvGeom& g);
 TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed);
-TinyNNStatus conv_mfma_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+TinyNNStatus conv_mfma_launch(const ConvGeom&, const void*, const void*, const void*, void*,
+                              const Workspace*);
+size_t conv_mfma_workspace_bytes(const ConvGeom& g);
 bool conv_first_supported(const ConvGeom& g);
 TinyNNStatus conv_first_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool dwconv44_supported(const ConvGeom& g);
@@ -181,7 +183,7 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
         MG_REQUIRE(aligned4(src->ptr) && aligned4(dst->ptr) && aligned16(flt->ptr) &&
                            (!b || aligned4(b)),
                    TinyNN_ERROR_INVALID_LAYOUT, "conv2d: misaligned operand");
-        return conv_mfma_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+        return conv_mfma_launch(g, src->ptr, flt->ptr, b, dst->ptr, workspace);
     }
     if (q8 && dwconv44_supported(g) && aligned4(src->ptr) && aligned4(flt->ptr) &&
         aligned4(dst->ptr))
@@ -244,11 +246,17 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d_workspace(
     if (!attr || !inputs || nr_input < 2 || !inputs[0] || !inputs[1])
         return TinyNN_SUCCESS;
     const Tensor *src = inputs[0], *flt = inputs[1];
+    ConvGeom g;
     if (is_f32(src) && is_f32(flt)) {
-        ConvGeom g;
         if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS &&
             conv_f32_gemm_supported(g))
             *workspace = conv_f32_gemm_workspace_bytes(g);
+    } else if (is_q8(src) && is_q8(flt) && attr->sparse == MEGCC_SPARSE_DENSE &&
+               !is_packed_filter(flt)) {
+        // split-K partial sums of the one-stage MFMA kernel (few pixels, long K)
+        if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS &&
+            conv_mfma_supported(g))
+            *workspace = conv_mfma_workspace_bytes(g);
     }
     return TinyNN_SUCCESS;
 }

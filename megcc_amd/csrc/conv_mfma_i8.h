@@ -62,6 +62,10 @@ struct MfmaParams {
     int act;
     float s_src, s_flt, s_dst;
     RequantFast rq;
+    // split-K of the one-stage kernel: blockIdx.z handles stages [z*sps, (z+1)*sps) and writes raw
+    // int32 sums to partial[z][P][round_up(OC,4)]; conv_mfma_reduce_kernel finishes
+    int split, sps;
+    int32_t* partial;
     FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
     int G, RG;       // 16-byte gather: pixel groups per row, groups per plane of the largest patch
     FastDiv dG, dRG;

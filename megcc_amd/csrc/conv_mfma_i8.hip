@@ -131,8 +131,9 @@ __global__ void __launch_bounds__(THREADS) conv_mfma_i8_kernel(MfmaParams q) {
         }
     };
 
-    prefetch(0);
-    for (int st = 0; st < q.stages; ++st) {
+    const int st_begin = blockIdx.z * q.sps, st_end = min(q.stages, st_begin + q.sps);
+    prefetch(st_begin);
+    for (int st = st_begin; st < st_end; ++st) {
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < MAX_A_ITEMS; ++j) {
@@ -145,7 +146,7 @@ __global__ void __launch_bounds__(THREADS) conv_mfma_i8_kernel(MfmaParams q) {
             if (b_loff[j] >= 0)
                 *(v4i*)(ldsB + b_loff[j]) = rb[j];
         __syncthreads();
-        if (st + 1 < q.stages)
+        if (st + 1 < st_end)
             prefetch(st + 1);
 
         for (int ks = 0; ks < q.KS; ++ks) {
@@ -176,6 +177,26 @@ __global__ void __launch_bounds__(THREADS) conv_mfma_i8_kernel(MfmaParams q) {
 
     // ---- epilogue: register e of a 32x32 tile holds row 8*(e/4) + 4*(lane/32) + e%4, col lane%32.
     //      The 4 bias values of a register group are fetched once and reused for all pixels.
+    if (q.split > 1) {
+        const int ocs = (q.OC + 3) & ~3;
+#pragma unroll
+        for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int oc = oc0 + wm * WM + mi * 32 + e4 * 8 + kg * 4;
+                if (oc >= q.OC)
+                    continue;
+#pragma unroll
+                for (int ni = 0; ni < NT; ++ni) {
+                    const int p = p0 + wn * 64 + ni * 32 + (lane & 31);
+                    if (p <= plast)
+                        *(int4*)(q.partial + ((size_t)blockIdx.z * q.P + p) * ocs + oc) =
+                                make_int4(acc[mi][ni][e4 * 4], acc[mi][ni][e4 * 4 + 1],
+                                          acc[mi][ni][e4 * 4 + 2], acc[mi][ni][e4 * 4 + 3]);
+                }
+            }
+        return;
+    }
     int pix_n[NT], pix_rem[NT];
 #pragma unroll
     for (int ni = 0; ni < NT; ++ni) {
@@ -233,6 +254,67 @@ __global__ void __launch_bounds__(THREADS) conv_mfma_i8_kernel(MfmaParams q) {
             }
         }
     }
+}
+
+// ---- split-K: sum the partial accumulators, then bias + requantise + store -----------------
+__global__ void __launch_bounds__(256) conv_mfma_reduce_kernel(MfmaParams q) {
+    const int ocs = (q.OC + 3) & ~3, oc4n = ocs >> 2;
+    const size_t total = (size_t)q.P * oc4n;
+    for (size_t i = blockIdx.x * (size_t)256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const int p = (int)(i / oc4n), oc = (int)(i - (size_t)p * oc4n) * 4;
+        int a[4] = {0, 0, 0, 0};
+        for (int z = 0; z < q.split; ++z) {
+            const int4 v = *(const int4*)(q.partial + ((size_t)z * q.P + p) * ocs + oc);
+            a[0] += v.x; a[1] += v.y; a[2] += v.z; a[3] += v.w;
+        }
+        int r[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int b = (q.bias && oc + e < q.OC) ? q.bias[oc + e] : 0;
+            r[e] = requant_conv_rt(q.act, a[e] + b, q.s_src, q.s_flt, q.s_dst);
+        }
+        if (!q.dst_fc) {
+            const int n = (int)fdiv(p, q.dOHW), rem = p - n * q.OHW;
+            ((uint32_t*)q.dst)[((size_t)n * (q.OC >> 2) + (oc >> 2)) * q.OHW + rem] =
+                    pack4(r[0], r[1], r[2], r[3]);
+        } else {
+            int8_t* o = q.dst + (size_t)p * q.OC + oc;
+            if ((q.OC & 3) == 0) {
+                *(uint32_t*)o = pack4(r[0], r[1], r[2], r[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (oc + e < q.OC)
+                        o[e] = (int8_t)r[e];
+            }
+        }
+    }
+}
+
+// Split factor of the one-stage kernel for layers with few output pixels and a long K
+// (FullyConnected at small batch, the last pointwise layers): a pure function of the shape, shared
+// by the _workspace entry point, the generated shims and the launch.
+static int conv_mfma_split(const ConvGeom& g) {
+    const long P = (long)g.n * g.oh * g.ow;
+    const int taps = g.fh * g.fw;
+    const int ks = taps <= 2 ? 4 : taps <= 4 ? 2 : 1;
+    const long chunks = (g.ic + 31) / 32, stages = (chunks + ks - 1) / ks;
+    const long bm = g.oc <= 64 ? 64 : 128;
+    const long tiles = ((P + 127) / 128) * ((g.oc + bm - 1) / bm);
+    if (tiles >= 128 || stages < 4)
+        return 1;
+    long s = (256 + tiles - 1) / tiles;
+    if (s > stages / 2)
+        s = stages / 2;
+    if (s > 16)
+        s = 16;
+    return s < 2 ? 1 : (int)s;
+}
+
+size_t conv_mfma_workspace_bytes(const ConvGeom& g) {
+    const int s = conv_mfma_split(g);
+    const long P = (long)g.n * g.oh * g.ow;
+    return s > 1 ? (size_t)s * P * ((g.oc + 3) & ~3) * sizeof(int32_t) : 0;
 }
 
 // ---- filter packing ---------------------------------------------------------------------
@@ -374,7 +456,8 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, PipeConfig* c);
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
 
 TinyNNStatus conv_mfma_launch(
-        const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst) {
+        const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst,
+        const Workspace* ws) {
     MfmaParams q;
     PipeConfig pc;
     const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;
@@ -477,13 +560,23 @@ TinyNNStatus conv_mfma_launch(
     q.dG = make_fastdiv(q.G);
     q.dRG = make_fastdiv(q.RG);
 
+    q.split = 1;
+    q.sps = q.stages;
+    q.partial = nullptr;
     if (pipe)
         return conv_mfma_pipe_launch(pc, q);
+    const int split = conv_mfma_split(g);
+    if (split > 1 && ws && ws->ptr && ws->size >= conv_mfma_workspace_bytes(g) &&
+        ((uintptr_t)ws->ptr & 15) == 0) {
+        q.split = split;
+        q.sps = (q.stages + split - 1) / split;
+        q.partial = (int32_t*)ws->ptr;
+    }
 
     const int bm = g.oc <= 64 ? 64 : 128;
     const size_t lds = (size_t)q.taps * q.KS * bm * KROW + (size_t)q.KS * q.Lmax * KROW;
     MG_REQUIRE(lds <= 160 * 1024, TinyNN_ERROR_OUT_OF_RANGE, "conv_mfma: %zu bytes of LDS", lds);
-    dim3 grid((q.P + BN - 1) / BN, (g.oc + bm - 1) / bm);
+    dim3 grid((q.P + BN - 1) / BN, (g.oc + bm - 1) / bm, q.split);
     void (*kern)(MfmaParams);
     if (g.act == MEGCC_NONLINE_IDENTITY)
         kern = bm == 64 ? conv_mfma_i8_kernel<64, MEGCC_NONLINE_IDENTITY>
@@ -500,6 +593,12 @@ TinyNNStatus conv_mfma_launch(
                    hipGetErrorString(e));
     }
     hipLaunchKernelGGL(kern, grid, dim3(THREADS), lds, stream(), q);
+    if (q.split > 1) {
+        const size_t total = (size_t)q.P * ((q.OC + 3) / 4);
+        unsigned blocks = (unsigned)((total + 255) / 256);
+        hipLaunchKernelGGL(conv_mfma_reduce_kernel, dim3(blocks > 4096 ? 4096 : blocks), dim3(256), 0,
+                           stream(), q);
+    }
     return check_launch("conv_mfma_i8");
 }
 

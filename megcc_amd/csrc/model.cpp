@@ -308,6 +308,18 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
             o->in_ptrs.push_back(&m->tensors[id]->t);
         for (int id : o->out)
             o->out_ptrs.push_back(&m->tensors[id]->t);
+        // workspace size, asked with the original weights like the compiler does
+        // (the VM shares one workspace region between operators)
+        {
+            size_t bytes = 0;
+            TinyNNStatus wst = megcc_gfx950_call_workspace(
+                    &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), 1, &bytes);
+            if (wst != TinyNN_SUCCESS)
+                return wst;
+            o->ws.size = bytes;
+            if (bytes > m->workspace_bytes)
+                m->workspace_bytes = bytes;
+        }
         // three-phase init (runtime/src/init.c:94-131)
         int n = 0;
         TinyNNStatus st = megcc_gfx950_call_init(
@@ -344,17 +356,6 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
             MG_REQUIRE(o->has_processed, TinyNN_ERROR_NO_FOUND,
                        "model_finalize: %s: processed weight matches no input", o->symbol.c_str());
         }
-    }
-    // workspaces (runtime/src/init.c: the VM shares one workspace region between operators)
-    for (auto* o : m->oprs) {
-        size_t bytes = 0;
-        TinyNNStatus st = megcc_gfx950_call_workspace(
-                &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), 1, &bytes);
-        if (st != TinyNN_SUCCESS)
-            return st;
-        o->ws.size = bytes;
-        if (bytes > m->workspace_bytes)
-            m->workspace_bytes = bytes;
     }
     if (m->workspace_bytes) {
         m->workspace = m->dev.malloc(m->workspace_bytes);

@@ -221,8 +221,12 @@ struct ConvKernel : KernelFuncBase {
     // (compiler/lib/KernelGen/Jit/JitExe.cpp:67-123 forbids externs in workspace bodies).
     // Quantized kernels need none (im2col stays in LDS); the f32 implicit GEMM may split K.
     std::string GetWorkspaceBody(TContext* c) const override {
-        if (!is_f32(c->getAttrOprand("operand:0").dtype) || conv_format(c) != "NCHW" ||
-            c->getAttrStr("sparse") != "DENSE")
+        const bool f32 = is_f32(c->getAttrOprand("operand:0").dtype);
+        const std::string fmt = conv_format(c);
+        const bool dense = c->getAttrStr("sparse") == "DENSE";
+        const unsigned taps = c->getAttrUInt("kernel_h") * c->getAttrUInt("kernel_w");
+        const bool q8_mfma = !f32 && dense && (fmt == "NCHW44" || fmt == "NCHW") && taps <= 9;
+        if (!(f32 && fmt == "NCHW" && dense) && !q8_mfma)
             return "TinyNNStatus " + GetWorkspaceSignature(c) +
                    " {\n    *workspace = 0;\n    return TinyNN_SUCCESS;\n}\n";
         std::stringstream ss;
@@ -235,9 +239,37 @@ struct ConvKernel : KernelFuncBase {
            << ", iw = src.dims[3] + 2 * " << c->getAttrUInt("pad_w") << ";\n"
            << "    const long oh = ih >= eh ? (ih - eh) / " << c->getAttrUInt("stride_h")
            << " + 1 : 0, ow = iw >= ew ? (iw - ew) / " << c->getAttrUInt("stride_w") << " + 1 : 0;\n"
-           << "    const long M = flt.dims[0], N = (long)src.dims[0] * oh * ow, K = (long)src.dims[1] * "
-           << c->getAttrUInt("kernel_h") << " * " << c->getAttrUInt("kernel_w") << ";\n"
-           << kSplitBody;
+           ;
+        if (f32) {
+            ss << "    const long M = flt.dims[0], N = (long)src.dims[0] * oh * ow, K = (long)src.dims[1] * "
+               << c->getAttrUInt("kernel_h") << " * " << c->getAttrUInt("kernel_w") << ";\n"
+               << kSplitBody;
+            return ss.str();
+        }
+        // qsi8 dense / FullyConnected: split-K partial sums of the one-stage MFMA kernel
+        // (conv_mfma_i8.hip, conv_mfma_split); it covers NCHW44 and the 1x1 NCHW on [M,K,1,1]
+        const int r = fmt == "NCHW44" ? 4 : 1;
+        const int ks = taps <= 2 ? 4 : taps <= 4 ? 2 : 1;
+        ss << "    const long P = (long)src.dims[0] * oh * ow, oc = (long)flt.dims[0] * " << r
+           << ", ic = (long)src.dims[1] * " << r << ";\n";
+        if (fmt == "NCHW")
+            ss << "    if (!(src.dims[2] == 1 && src.dims[3] == 1 && " << taps << " == 1 && "
+               << c->getAttrUInt("pad_h") << " == 0 && " << c->getAttrUInt("pad_w")
+               << " == 0)) {\n        *workspace = 0;\n        return TinyNN_SUCCESS;\n    }\n";
+        ss << "    *workspace = 0;\n"
+           << "    if ((ic & 3) == 0 && P > 0) {\n"
+           << "        const long stages = ((ic + 31) / 32 + " << ks - 1 << ") / " << ks << ";\n"
+           << "        const long bm = oc <= 64 ? 64 : 128;\n"
+           << "        const long tiles = ((P + 127) / 128) * ((oc + bm - 1) / bm);\n"
+           << "        long s = 1;\n"
+           << "        if (tiles < 128 && stages >= 4) {\n"
+           << "            s = (256 + tiles - 1) / tiles;\n"
+           << "            if (s > stages / 2) s = stages / 2;\n"
+           << "            if (s > 16) s = 16;\n"
+           << "        }\n"
+           << "        if (s > 1) *workspace = (size_t)s * P * ((oc + 3) & ~3L) * 4;\n"
+           << "    }\n"
+           << "    return TinyNN_SUCCESS;\n}\n";
         return ss.str();
     }
 };

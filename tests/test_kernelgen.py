@@ -101,19 +101,27 @@ def test_generated_workspace_functions_agree_with_the_library(shim_library):
             k = desc.attr.conv.kernel_h
             cases_ = [[(1, 32, 56, 56), (32, 32, k, k)], [(2, 5, 19, 23), (37, 5, k, k)],
                       [(8, 64, 56, 56), (128, 64, k, k)]]
+        elif desc.kind == 1 and "qsi8" in sym and "_NCHW44_DENSE_" in sym:
+            k = desc.attr.conv.kernel_h
+            cases_ = [[(64, 256, 7, 7, 4), (256, 256, k, k, 4, 4)], [(2, 8, 20, 24, 4), (12, 8, k, k, 4, 4)],
+                      [(1, 128, 14, 14, 4), (32, 128, k, k, 4, 4)]]
+        elif desc.kind == 1 and "qsi8" in sym and "_1x1_NCHW_DENSE_p0x0_s1x1" in sym:
+            cases_ = [[(64, 1024, 1, 1), (1000, 1024, 1, 1)], [(64, 4096, 1, 1), (4096, 4096, 1, 1)],
+                      [(1, 1024, 1, 1), (1000, 1024, 1, 1)], [(4096, 4096, 1, 1), (4096, 4096, 1, 1)]]
         else:
             continue
         fn = getattr(lib, sym + "_workspace")
         fn.argtypes = abi.WORKSPACE_ARGS
+        dt = abi.FLOAT if "f32" in sym else abi.QINT8
         for shapes_ in cases_:
-            tin = [abi.make_tensor(None, s, abi.FLOAT, 1.0) for s in shapes_]
+            tin = [abi.make_tensor(None, s, dt, 1.0) for s in shapes_]
             a, b = C.c_size_t(7), C.c_size_t(9)
             assert fn(abi.tensor_array(tin), len(tin), 1, C.byref(a)) == 0
             assert L.megcc_gfx950_call_workspace(C.byref(desc), abi.tensor_array(tin), len(tin), 1,
                                                  C.byref(b)) == 0
             assert a.value == b.value, (sym, shapes_, a.value, b.value)
             checked += 1
-    assert checked >= 8
+    assert checked >= 20
 
 
 @pytest.mark.gpu

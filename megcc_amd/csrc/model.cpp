@@ -14,6 +14,7 @@
 // is produced here from the same inputs it uses: per tensor the interval [defining opr, last
 // using opr + 1) (compiler/lib/Dialect/Kernel/Transforms/StaticMemoryPlanning.cpp:88-96) and the
 // byte size; tensors whose intervals overlap get disjoint offset ranges.
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -58,6 +59,14 @@ struct Model {
     void* workspace = nullptr;
     size_t workspace_bytes = 0;
     bool finalized = false;
+    // The operator sequence of a finalized model never changes (static shapes, static memory plan),
+    // so after one eager forward it is captured once into a HIP graph and replayed: one launch per
+    // forward instead of one per operator. 0: not tried yet, 1: graph in use, -1: capture failed
+    // or switched off (MEGCC_NO_GRAPH), stay eager.
+    int graph_state = 0;
+    int forwards = 0;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
 };
 
 size_t tensor_bytes(const Tensor& t) {
@@ -160,6 +169,10 @@ void megcc_gfx950_model_destroy(void* model) {
         m->dev.free(m->arena);
     if (m->workspace)
         m->dev.free(m->workspace);
+    if (m->graph_exec)
+        hipGraphExecDestroy(m->graph_exec);
+    if (m->graph)
+        hipGraphDestroy(m->graph);
     delete m;
 }
 
@@ -402,9 +415,7 @@ TinyNNStatus megcc_gfx950_model_get_output(void* model, int tensor, void* host, 
 
 // LITE_forward: one asynchronous kernel launch per Opr, in order, on the library stream; stops at
 // the first failing kernel like network.c:191-194. Results are visible after megcc_gfx950_wait().
-TinyNNStatus megcc_gfx950_model_forward(void* model) {
-    Model* m = (Model*)model;
-    MG_REQUIRE(m && m->finalized, TinyNN_ERROR_NULL_PTR, "model_forward: model not finalized");
+static TinyNNStatus forward_eager(Model* m) {
     for (auto* o : m->oprs) {
         TinyNNStatus st = megcc_gfx950_call(
                 &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), o->out_ptrs.data(),
@@ -413,6 +424,43 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
             return st;
     }
     return TinyNN_SUCCESS;
+}
+
+TinyNNStatus megcc_gfx950_model_forward(void* model) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && m->finalized, TinyNN_ERROR_NULL_PTR, "model_forward: model not finalized");
+    ++m->forwards;
+    if (m->graph_state == 1) {
+        hipError_t e = hipGraphLaunch(m->graph_exec, stream());
+        MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "model_forward: graph launch: %s",
+                   hipGetErrorString(e));
+        return TinyNN_SUCCESS;
+    }
+    // the first forward runs eagerly (it also warms per-kernel attributes), the second is captured
+    if (m->graph_state == 0 && m->forwards >= 2) {
+        m->graph_state = -1;
+        if (!getenv("MEGCC_NO_GRAPH") &&
+            hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal) == hipSuccess) {
+            TinyNNStatus st = forward_eager(m);
+            hipGraph_t g = nullptr;
+            hipError_t e = hipStreamEndCapture(stream(), &g);
+            if (st == TinyNN_SUCCESS && e == hipSuccess && g &&
+                hipGraphInstantiate(&m->graph_exec, g, nullptr, nullptr, 0) == hipSuccess) {
+                m->graph = g;
+                m->graph_state = 1;
+                e = hipGraphLaunch(m->graph_exec, stream());
+                MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "model_forward: graph launch: %s",
+                           hipGetErrorString(e));
+                return TinyNN_SUCCESS;
+            }
+            if (g)
+                hipGraphDestroy(g);
+            (void)hipGetLastError();  // a failed capture must not poison the eager path
+            if (st != TinyNN_SUCCESS)
+                return st;
+        }
+    }
+    return forward_eager(m);
 }
 
 int megcc_gfx950_model_nr_opr(void* model) {

@@ -59,3 +59,27 @@ def test_memory_plan_reuses_the_arena_and_keeps_results():
         got = model.get(ids["softmax"])
         assert cases.max_rel_err(got, want) <= 1e-4
     model.close()
+
+
+@pytest.mark.gpu
+def test_graph_replays_equal_eager_forwards(monkeypatch):
+    """The model runtime captures its operator sequence into a HIP graph on the second forward.
+    Every replay, with new inputs, host copies and synchronisations in between, must give what an
+    eager forward gives (bit for bit: same kernels, same order)."""
+    net = mobilenet.Net(2)
+    eager, ids = net.build_gpu(keep_all=True)
+    graph, _ = net.build_gpu(keep_all=True)
+    names = ["conv0", "pw1", "pw13", "fc", "softmax"]
+    for it in range(5):
+        image = mobilenet.draw_input(2, seed=20 + it)
+        monkeypatch.setenv("MEGCC_NO_GRAPH", "1")
+        eager.set_input(ids["image"], image)
+        eager.forward()
+        want = {k: eager.get(ids[k]).copy() for k in names}
+        monkeypatch.delenv("MEGCC_NO_GRAPH")
+        graph.set_input(ids["image"], image)
+        graph.forward()  # it == 0: eager, it == 1: capture + first launch, then replays
+        for k in names:
+            np.testing.assert_array_equal(graph.get(ids[k]), want[k], err_msg="%s, forward %d" % (k, it))
+    eager.close()
+    graph.close()

@@ -112,6 +112,39 @@ class Net:
         trace["softmax"] = sm
         return sm, trace
 
+    def run_cpu_timed(self, image, threads=1):
+        """One forward on host cores for the reported CPU baseline: every operator through the
+        reference's own generated kernel when oracle/_ref has it, else through the C restatement.
+        Returns (seconds, {operators run by reference kernels, by the port})."""
+        import time
+        import cases
+        from oracle import ref
+        port.set_threads(threads)
+        x = image
+        used = {"reference": 0, "port": 0}
+        t0 = time.perf_counter()
+        for kind, name, case, _ in self.steps:
+            if kind == "typecvt":
+                arrays = {"src": np.ascontiguousarray(x.reshape(case.shape))}
+            elif kind == "pool":
+                arrays = {"src": x}
+            else:
+                flt, bias, _ = self.weights[name]
+                if name == "fc":
+                    x = np.ascontiguousarray(x.reshape(self.batch, 1024, 1, 1))
+                arrays = {"src": x, "flt": flt, "bias": bias}
+            if ref.available() and ref.has(case.symbol()):
+                x = cases.run_ref(case, arrays)
+                used["reference"] += 1
+            else:
+                x = case.run_port(arrays)
+                used["port"] += 1
+        logits = x.reshape(self.batch, 1000)
+        mx = port.reduce_f32(logits, abi.REDUCE_MAX, 1)
+        e = port.elemwise_f32(port.elemwise_f32(logits, mx, abi.EW_SUB), None, abi.EW_EXP)
+        port.elemwise_f32(e, port.reduce_f32(e, abi.REDUCE_SUM, 1), abi.EW_TRUE_DIV)
+        return time.perf_counter() - t0, used
+
     # ---- GPU model -----------------------------------------------------------------------------
     def build_gpu(self, keep_all=False):
         from megcc_amd import runtime

@@ -66,8 +66,10 @@ __device__ __forceinline__ float conv_b(const GemmArgs& q, int k, int p) {
 // B_NFAST: B(k,n) has n contiguous -> lanes walk n.
 template <bool A_KFAST, bool B_NFAST, bool CONV>
 __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
-    __shared__ float As[GBK][GBM + GPAD];
-    __shared__ float Bs[GBK][GBN + GPAD];
+    // LDS is double buffered: the global loads of step k+1 are in flight (in registers) while
+    // step k is multiplied out of the other buffer; one barrier per step.
+    __shared__ float As[2][GBK][GBM + GPAD];
+    __shared__ float Bs[2][GBK][GBN + GPAD];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int m0 = blockIdx.y * GBM, n0 = blockIdx.x * GBN;
@@ -83,8 +85,9 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
 
     const int k_begin = blockIdx.z * q.kchunk;
     const int k_end = min(q.K, k_begin + q.kchunk);
-    for (int k0 = k_begin; k0 < k_end; k0 += GBK) {
-        // ---- stage A tile (GBM x GBK) and B tile (GBK x GBN): 8 elements per thread each
+    float ra[8], rb[8];
+    // stage A tile (GBM x GBK) and B tile (GBK x GBN): 8 elements per thread each
+    auto load_tiles = [&](int k0) {
 #pragma unroll
         for (int it = 0; it < 8; ++it) {
             int m, k;
@@ -98,7 +101,7 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
             float v = 0.f;
             if (m0 + m < q.M && k0 + k < k_end)
                 v = q.A[(size_t)(m0 + m) * q.a_rs + (size_t)(k0 + k) * q.a_cs];
-            As[k][m] = v;
+            ra[it] = v;
         }
 #pragma unroll
         for (int it = 0; it < 8; ++it) {
@@ -117,25 +120,50 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
                 else
                     v = q.B[(size_t)(k0 + k) * q.b_rs + (size_t)(n0 + n) * q.b_cs];
             }
-            Bs[k][n] = v;
+            rb[it] = v;
         }
-        __syncthreads();
+    };
+    auto store_tiles = [&](int buf) {
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            if (A_KFAST)
+                As[buf][tid & 15][(tid >> 4) + it * 16] = ra[it];
+            else
+                As[buf][(tid >> 7) + it * 2][tid & 127] = ra[it];
+            if (B_NFAST)
+                Bs[buf][(tid >> 7) + it * 2][tid & 127] = rb[it];
+            else
+                Bs[buf][tid & 15][(tid >> 4) + it * 16] = rb[it];
+        }
+    };
+    if (k_begin < k_end) {
+        load_tiles(k_begin);
+        store_tiles(0);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = k_begin; k0 < k_end; k0 += GBK, buf ^= 1) {
+        const bool more = k0 + GBK < k_end;
+        if (more)
+            load_tiles(k0 + GBK);
 #pragma unroll
         for (int kk = 0; kk < GBK; kk += 2) {
             const int k = kk + (lane >> 5);
             float a[2], b[2];
 #pragma unroll
             for (int i = 0; i < 2; ++i)
-                a[i] = As[k][wm * 64 + i * 32 + (lane & 31)];
+                a[i] = As[buf][k][wm * 64 + i * 32 + (lane & 31)];
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-                b[j] = Bs[k][wn * 64 + j * 32 + (lane & 31)];
+                b[j] = Bs[buf][k][wn * 64 + j * 32 + (lane & 31)];
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
         }
+        if (more)
+            store_tiles(buf ^ 1);
         __syncthreads();
     }
 

@@ -294,18 +294,24 @@ __global__ void __launch_bounds__(256) conv_mfma_reduce_kernel(MfmaParams q) {
 // Split factor of the one-stage kernel for layers with few output pixels and a long K
 // (FullyConnected at small batch, the last pointwise layers): a pure function of the shape, shared
 // by the _workspace entry point, the generated shims and the launch.
+// oc tile of the one-stage kernel: 64 rows when 128-row tiles would leave most of the chip idle
+static int conv_mfma_bm(const ConvGeom& g) {
+    const long P = (long)g.n * g.oh * g.ow;
+    return g.oc <= 64 || ((P + 127) / 128) * ((g.oc + 127) / 128) < 64 ? 64 : 128;
+}
+
 static int conv_mfma_split(const ConvGeom& g) {
     const long P = (long)g.n * g.oh * g.ow;
     const int taps = g.fh * g.fw;
     const int ks = taps <= 2 ? 4 : taps <= 4 ? 2 : 1;
     const long chunks = (g.ic + 31) / 32, stages = (chunks + ks - 1) / ks;
-    const long bm = g.oc <= 64 ? 64 : 128;
+    const long bm = conv_mfma_bm(g);
     const long tiles = ((P + 127) / 128) * ((g.oc + bm - 1) / bm);
-    if (tiles >= 128 || stages < 4)
+    if (tiles >= 128 || stages < 2)
         return 1;
-    long s = (256 + tiles - 1) / tiles;
-    if (s > stages / 2)
-        s = stages / 2;
+    long s = (512 + tiles - 1) / tiles;
+    if (s > stages)
+        s = stages;
     if (s > 16)
         s = 16;
     return s < 2 ? 1 : (int)s;
@@ -573,7 +579,7 @@ TinyNNStatus conv_mfma_launch(
         q.partial = (int32_t*)ws->ptr;
     }
 
-    const int bm = g.oc <= 64 ? 64 : 128;
+    const int bm = conv_mfma_bm(g);
     const size_t lds = (size_t)q.taps * q.KS * bm * KROW + (size_t)q.KS * q.Lmax * KROW;
     MG_REQUIRE(lds <= 160 * 1024, TinyNN_ERROR_OUT_OF_RANGE, "conv_mfma: %zu bytes of LDS", lds);
     dim3 grid((q.P + BN - 1) / BN, (g.oc + bm - 1) / bm, q.split);

@@ -259,12 +259,12 @@ struct ConvKernel : KernelFuncBase {
         ss << "    *workspace = 0;\n"
            << "    if ((ic & 3) == 0 && P > 0) {\n"
            << "        const long stages = ((ic + 31) / 32 + " << ks - 1 << ") / " << ks << ";\n"
-           << "        const long bm = oc <= 64 ? 64 : 128;\n"
+           << "        const long bm = oc <= 64 || ((P + 127) / 128) * ((oc + 127) / 128) < 64 ? 64 : 128;\n"
            << "        const long tiles = ((P + 127) / 128) * ((oc + bm - 1) / bm);\n"
            << "        long s = 1;\n"
-           << "        if (tiles < 128 && stages >= 4) {\n"
-           << "            s = (256 + tiles - 1) / tiles;\n"
-           << "            if (s > stages / 2) s = stages / 2;\n"
+           << "        if (tiles < 128 && stages >= 2) {\n"
+           << "            s = (512 + tiles - 1) / tiles;\n"
+           << "            if (s > stages) s = stages;\n"
            << "            if (s > 16) s = 16;\n"
            << "        }\n"
            << "        if (s > 1) *workspace = (size_t)s * P * ((oc + 3) & ~3L) * 4;\n"

@@ -409,6 +409,20 @@ int megcc_gfx950_model_nr_opr(void* model);
  * TINYNN_DUMP_TENSOR hooks of runtime/src/lite/network.c:187-224) */
 TinyNNStatus megcc_gfx950_model_run_opr(void* model, int index);
 
+/* The static memory plan by itself: interval i is alive during time steps [begin[i], end[i]) and
+ * needs size[i] bytes; offset[i] receives its place in one arena of *arena_bytes bytes, every
+ * offset a multiple of `alignment` (a power of two). Replaces, with identical offsets and arena
+ * size, StaticMemAlloc::make(PUSHDOWN) + add() + alignment() + solve() + get_start_addr() /
+ * tot_alloc() / tot_alloc_lower_bound() of compiler/lib/Dialect/Kernel/Transforms/migrate/
+ * static_mem_alloc.h:12-87 as driven by Transforms/StaticMemoryPlanning.cpp:34-96 (time step =
+ * operator index, end = last use + 1). Host code only, no GPU needed. lower_bound may be NULL.
+ * TinyNN_ERROR_INVALID_LAYOUT for a bad alignment or an interval with begin >= end (the reference
+ * asserts on both). Overwrite specs (add_overwrite_spec) are not offered: that pass never adds
+ * one. */
+TinyNNStatus megcc_gfx950_plan_memory(
+        size_t nr_interval, const size_t* begin, const size_t* end, const size_t* size,
+        size_t alignment, size_t* offset, size_t* arena_bytes, size_t* lower_bound);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,6 +22,7 @@
 #include <vector>
 
 #include "common.h"
+#include "memplan.h"
 
 using namespace mg;
 
@@ -83,57 +84,32 @@ int root_of(const Model* m, int id) {
     return id;
 }
 
-// Offsets for the arena: largest tensors first, each at the lowest offset that does not collide
-// with an already placed tensor whose lifetime overlaps.
-void plan_memory(Model* m) {
-    struct Item {
-        int id;
-        size_t size, offset;
-        int begin, end;
-    };
-    std::vector<Item> items;
+// Offsets for the arena from the tensors' lifetimes: time step = operator index, a tensor is
+// alive from the operator that writes it to one past the last operator that reads it
+// (compiler/lib/Dialect/Kernel/Transforms/StaticMemoryPlanning.cpp:88-96); model inputs are staged
+// into the arena before the first operator and outputs stay valid after forward().
+bool plan_memory(Model* m) {
+    std::vector<MemInterval> intervals;
+    std::vector<int> ids;
     for (size_t i = 0; i < m->tensors.size(); ++i) {
         ModelTensor* t = m->tensors[i];
         if (t->is_weight || t->alias_of >= 0 || t->def < 0)
             continue;
-        Item it;
-        it.id = (int)i;
-        it.size = align_up(tensor_bytes(t->t), m->dev.alignment);
-        it.begin = t->def;
-        it.end = t->last + 1;
-        if (t->is_output)
-            it.end = (int)m->oprs.size() + 1;  // outputs stay valid after forward()
-        it.offset = 0;
-        items.push_back(it);
+        MemInterval iv;
+        iv.begin = (size_t)t->def;
+        iv.end = t->is_output ? m->oprs.size() + 1 : (size_t)t->last + 1;
+        iv.size = tensor_bytes(t->t);
+        intervals.push_back(iv);
+        ids.push_back((int)i);
     }
-    // model inputs are staged into the arena as well and live from before the first opr
-    std::vector<Item*> order;
-    for (auto& it : items)
-        order.push_back(&it);
-    std::sort(order.begin(), order.end(), [](const Item* a, const Item* b) {
-        return a->size != b->size ? a->size > b->size : a->id < b->id;
-    });
-    std::vector<Item*> placed;
+    std::vector<size_t> offsets;
     size_t total = 0;
-    for (Item* it : order) {
-        std::vector<std::pair<size_t, size_t>> busy;
-        for (Item* p : placed)
-            if (p->begin < it->end && it->begin < p->end)
-                busy.emplace_back(p->offset, p->offset + p->size);
-        std::sort(busy.begin(), busy.end());
-        size_t off = 0;
-        for (auto& b : busy) {
-            if (off + it->size <= b.first)
-                break;
-            off = std::max(off, b.second);
-        }
-        it->offset = off;
-        total = std::max(total, off + it->size);
-        placed.push_back(it);
-    }
-    for (auto& it : items)
-        m->tensors[it.id]->t.offset = it.offset;
+    if (!plan_memory_pushdown(intervals, m->dev.alignment, &offsets, &total, nullptr))
+        return false;
+    for (size_t k = 0; k < ids.size(); ++k)
+        m->tensors[ids[k]]->t.offset = offsets[k];
     m->arena_bytes = total;
+    return true;
 }
 
 }  // namespace
@@ -303,7 +279,8 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
     for (auto* t : m->tensors)
         if (t->is_input && t->def != 0)
             t->def = 0;
-    plan_memory(m);
+    MG_REQUIRE(plan_memory(m), TinyNN_ERROR_INVALID_LAYOUT,
+               "model_finalize: memory plan (alignment %zu)", (size_t)m->dev.alignment);
     m->arena = m->dev.malloc(m->arena_bytes ? m->arena_bytes : 1);
     MG_REQUIRE(m->arena, TinyNN_ERROR_MEMORY_MALLOC, "model_finalize: arena of %zu bytes",
                m->arena_bytes);
@@ -477,6 +454,27 @@ TinyNNStatus megcc_gfx950_model_run_opr(void* model, int index) {
     return megcc_gfx950_call(
             &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), o->out_ptrs.data(),
             (int)o->out_ptrs.size(), &o->ws, &m->opt);
+}
+
+// The static memory plan on its own, for a caller that has the lifetimes (the compiler side, or a
+// loader that wants to check the offsets stored in a model file).
+TinyNNStatus megcc_gfx950_plan_memory(
+        size_t nr_interval, const size_t* begin, const size_t* end, const size_t* size,
+        size_t alignment, size_t* offset, size_t* arena_bytes, size_t* lower_bound) {
+    MG_REQUIRE(nr_interval == 0 || (begin && end && size && offset), TinyNN_ERROR_NULL_PTR,
+               "plan_memory: null array");
+    MG_REQUIRE(arena_bytes, TinyNN_ERROR_NULL_PTR, "plan_memory: null arena_bytes");
+    std::vector<MemInterval> intervals(nr_interval);
+    for (size_t i = 0; i < nr_interval; ++i)
+        intervals[i] = MemInterval{begin[i], end[i], size[i]};
+    std::vector<size_t> offsets;
+    MG_REQUIRE(plan_memory_pushdown(intervals, alignment, &offsets, arena_bytes, lower_bound),
+               TinyNN_ERROR_INVALID_LAYOUT,
+               "plan_memory: alignment %zu is not a power of two, or an interval is empty",
+               alignment);
+    for (size_t i = 0; i < nr_interval; ++i)
+        offset[i] = offsets[i];
+    return TinyNN_SUCCESS;
 }
 
 }  // extern "C"

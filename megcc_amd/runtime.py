@@ -72,6 +72,9 @@ def lib():
         L.megcc_gfx950_model_forward.argtypes = [C.c_void_p]
         L.megcc_gfx950_model_nr_opr.argtypes = [C.c_void_p]
         L.megcc_gfx950_model_run_opr.argtypes = [C.c_void_p, C.c_int]
+        sizes = C.POINTER(C.c_size_t)
+        L.megcc_gfx950_plan_memory.argtypes = [
+            C.c_size_t, sizes, sizes, sizes, C.c_size_t, sizes, sizes, sizes]
         _lib = L
     return _lib
 
@@ -90,7 +93,7 @@ EXPORTS = [
     "megcc_gfx950_model_mark_io", "megcc_gfx950_model_finalize", "megcc_gfx950_model_arena_bytes",
     "megcc_gfx950_model_tensor_ptr", "megcc_gfx950_model_set_input",
     "megcc_gfx950_model_get_output", "megcc_gfx950_model_forward", "megcc_gfx950_model_nr_opr",
-    "megcc_gfx950_model_run_opr",
+    "megcc_gfx950_model_run_opr", "megcc_gfx950_plan_memory",
 ]
 
 
@@ -98,6 +101,24 @@ def check(status, what=""):
     if status != abi.SUCCESS:
         raise MegccError("%s: TinyNNStatus %d: %s" % (
             what, status, lib().megcc_gfx950_last_error().decode()))
+
+
+def plan_memory(begin, end, size, alignment=1):
+    """Static memory plan (host code only): interval i lives during time steps
+    [begin[i], end[i]) and needs size[i] bytes. Returns (offsets, arena_bytes, lower_bound), the
+    result of the reference's StaticMemAlloc PUSHDOWN solver on the same requests
+    (compiler/lib/Dialect/Kernel/Transforms/migrate/static_mem_alloc.h:26,
+    Transforms/StaticMemoryPlanning.cpp:34-96)."""
+    arrs = [np.ascontiguousarray(a, dtype=np.uint64) for a in (begin, end, size)]
+    n = len(arrs[0])
+    assert all(len(a) == n for a in arrs)
+    off = np.zeros(max(n, 1), np.uint64)
+    total, bound = C.c_size_t(0), C.c_size_t(0)
+    ptr = lambda a: a.ctypes.data_as(C.POINTER(C.c_size_t))
+    check(lib().megcc_gfx950_plan_memory(
+        n, ptr(arrs[0]), ptr(arrs[1]), ptr(arrs[2]), alignment, ptr(off),
+        C.byref(total), C.byref(bound)), "plan_memory")
+    return off[:n].astype(np.int64), int(total.value), int(bound.value)
 
 
 class DeviceBuffer:

@@ -88,3 +88,30 @@ def run(symbol, inputs, outputs):
     st = kern(abi.tensor_array(inputs), len(inputs), abi.tensor_array(outputs), len(outputs),
               C.byref(ws), None)
     assert st == 0, "%s -> %d" % (symbol, st)
+
+
+_MEMPLAN_PATH = os.path.join(_HERE, "_ref", "libmegcc_ref_memplan.so")
+_MEMPLAN = None
+
+
+def memplan_available():
+    return os.path.exists(_MEMPLAN_PATH)
+
+
+def plan_memory(begin, end, size, alignment=1):
+    """The reference's own StaticMemAlloc (PUSHDOWN) on these requests, through
+    oracle/ref_memplan.cpp. Returns (offsets, arena_bytes, lower_bound). The reference aborts the
+    process on requests it rejects (begin >= end, alignment not a power of two)."""
+    global _MEMPLAN
+    if _MEMPLAN is None:
+        _MEMPLAN = C.CDLL(_MEMPLAN_PATH)
+    arrs = [np.ascontiguousarray(a, dtype=np.uint64) for a in (begin, end, size)]
+    n = len(arrs[0])
+    off = np.zeros(max(n, 1), np.uint64)
+    total, bound = C.c_size_t(0), C.c_size_t(0)
+    ptr = lambda a: a.ctypes.data_as(C.POINTER(C.c_size_t))
+    st = _MEMPLAN.ref_plan_memory(
+        C.c_size_t(n), ptr(arrs[0]), ptr(arrs[1]), ptr(arrs[2]), C.c_size_t(alignment), ptr(off),
+        C.byref(total), C.byref(bound))
+    assert st == 0
+    return off[:n].astype(np.int64), int(total.value), int(bound.value)

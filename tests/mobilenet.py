@@ -67,6 +67,74 @@ def draw_input(batch, seed=0):
     return r.uniform(-1, 1, (batch, 3, 224, 224)).astype(np.float32)
 
 
+class Lifetimes:
+    """Stands in for runtime.Model on a machine without a GPU: records tensors and operators and
+    derives the memory-plan requests the model runtime makes from them - time step = operator
+    index; a tensor is alive from the operator that writes it (inputs: from step 0) to one past the
+    last operator that touches it (outputs: one past the last operator + 1); views share their
+    root's request; weights are not planned."""
+
+    def __init__(self):
+        self.sizes, self.root, self.first, self.last = [], [], [], []
+        self.is_weight, self.is_output, self.dtype = [], [], []
+        self.nr_opr = 0
+
+    def _add(self, shape, type_enum, root=-1, weight=False):
+        self.sizes.append(int(np.prod(shape)) * abi.np_dtype(type_enum).itemsize)
+        self.root.append(root)
+        self.first.append(-1)
+        self.last.append(-1)
+        self.is_weight.append(weight)
+        self.is_output.append(False)
+        self.dtype.append(type_enum)
+        return len(self.sizes) - 1
+
+    def _root(self, t):
+        while self.root[t] >= 0:
+            t = self.root[t]
+        return t
+
+    def tensor(self, name, shape, type_enum, scale=1.0):
+        return self._add(shape, type_enum)
+
+    def weight(self, name, array, type_enum, scale=1.0):
+        return self._add(array.shape, type_enum, weight=True)
+
+    def alias(self, name, of, shape):
+        return self._add(shape, self.dtype[of], root=of)
+
+    def opr(self, symbol, inputs, outputs):
+        k = self.nr_opr
+        for t in inputs:
+            r = self._root(t)
+            self.last[r] = max(self.last[r], k)
+        for t in outputs:
+            r = self._root(t)
+            if self.first[r] < 0:
+                self.first[r] = k
+            self.last[r] = max(self.last[r], k)
+        self.nr_opr += 1
+
+    def mark_input(self, t):
+        r = self._root(t)
+        self.first[r] = 0
+        self.last[r] = max(self.last[r], 0)
+
+    def mark_output(self, t):
+        self.is_output[self._root(t)] = True
+
+    def finalize(self):
+        pass
+
+    def requests(self):
+        """(tensor ids, begin, end, size) in tensor-id order"""
+        ids = [t for t in range(len(self.sizes))
+               if not self.is_weight[t] and self.root[t] < 0 and self.first[t] >= 0]
+        begin = [self.first[t] for t in ids]
+        end = [self.nr_opr + 1 if self.is_output[t] else self.last[t] + 1 for t in ids]
+        return ids, begin, end, [self.sizes[t] for t in ids]
+
+
 class Net:
     """The operator list with all scales resolved: steps = [(kind, name, case, extra)]"""
 
@@ -146,9 +214,13 @@ class Net:
         return time.perf_counter() - t0, used
 
     # ---- GPU model -----------------------------------------------------------------------------
-    def build_gpu(self, keep_all=False):
-        from megcc_amd import runtime
-        m = runtime.Model()
+    def build_gpu(self, keep_all=False, model=None):
+        """Describes the network to a runtime.Model (or to anything with the same methods, e.g.
+        the Lifetimes recorder below) and finalizes it."""
+        if model is None:
+            from megcc_amd import runtime
+            model = runtime.Model()
+        m = model
         ids = {}
         b = self.batch
         x = m.tensor("image", (b, 3, 224, 224), abi.FLOAT)

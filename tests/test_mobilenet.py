@@ -5,7 +5,7 @@ import pytest
 
 import cases
 import mobilenet
-from megcc_amd import abi
+from megcc_amd import abi, runtime
 
 
 def test_layer_table_matches_the_standard_topology():
@@ -53,6 +53,16 @@ def test_memory_plan_reuses_the_arena_and_keeps_results():
     model, ids = net.build_gpu()
     total = sum(c.n * c.oc * c.oh * c.ow for k, _, c, _ in net.steps if k == "conv")
     assert model.arena_bytes < total / 3, "tensors with disjoint lifetimes must share memory"
+    # the arena is the reference allocator's plan for this model's lifetimes (stored answer for
+    # batch 1 and 64 in golden/memplan.json; here the same planner on batch 3)
+    lt = mobilenet.Lifetimes()
+    net.build_gpu(model=lt)
+    tids, begin, end, size = lt.requests()
+    off, arena, _ = runtime.plan_memory(begin, end, size, 256)
+    assert model.arena_bytes == arena
+    ptrs = [runtime.lib().megcc_gfx950_model_tensor_ptr(model.h, t) for t in tids]
+    lowest = min(ptrs)
+    assert [p - lowest for p in ptrs] == (off - off.min()).tolist()
     for _ in range(2):  # a second forward must not depend on leftovers of the first
         model.set_input(ids["image"], image)
         model.forward()

@@ -458,7 +458,7 @@ TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed) {
 
 bool conv_mfma_pipe_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
 bool conv_mfma_ws_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
-bool conv_mfma_dma_config(const ConvGeom& g, bool fc, PipeConfig* c);
+bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, PipeConfig* c);
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
 
 TinyNNStatus conv_mfma_launch(
@@ -472,10 +472,13 @@ TinyNNStatus conv_mfma_launch(
     long range_len = 0;
     TilePlan t;
     bool pipe = false;
-    for (int cand = 0; cand < 3 && !pipe; ++cand) {
+    for (int cand = -1; cand < 3 && !pipe; ++cand) {
         bool have = false;
-        if (cand == 0)
-            have = !getenv("MEGCC_NODMA") && conv_mfma_dma_config(g, is_fc(g), &pc);
+        if (cand == -1)
+            have = !getenv("MEGCC_NODMA") && !getenv("MEGCC_NODMA512") &&
+                   conv_mfma_dma_config(g, is_fc(g), 0, &pc);
+        else if (cand == 0)
+            have = !getenv("MEGCC_NODMA") && conv_mfma_dma_config(g, is_fc(g), 1, &pc);
         else if (cand == 1)
             have = !getenv("MEGCC_NOWS") && conv_mfma_ws_config(g, g4_ok, &pc);
         else

@@ -24,7 +24,6 @@
 namespace mg {
 
 static constexpr int ACT_RT = -1;
-static constexpr int DM_BNP = 256;
 
 // FH x FW taps, KS 32-channel sub-chunks per stage, LMAX patch slots (compile time, so that the
 // number of loads per stage is a constant the vmcnt waits can be written for).
@@ -37,9 +36,13 @@ static constexpr int DM_BNP = 256;
 // two share a CU (launch bound 2): their phases drift apart, so one's epilogue, barrier and load
 // waits overlap the other's MFMAs.
 // BPC: workgroups per CU the register budget is set for.
-template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC>
+// NT: 32-pixel MFMA tiles per wave along pixels; the workgroup sub-tile is 128 * NT pixels. NT = 4
+// reads 0.75 KB of LDS per MFMA instead of 1 KB (the 2 x 2 wave tile keeps the LDS port as busy as
+// the matrix core).
+template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT>
 __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaParams q) {
-    constexpr int NT = 2, WGN = 4;
+    constexpr int WGN = 4;
+    constexpr int DM_BNP = 32 * NT * WGN;
     constexpr int DM_WAVES = WGM * WGN, DM_THREADS = 64 * DM_WAVES;
     constexpr int DM_BM = 32 * MT * WGM;
     constexpr int TAPS = FH * FW;
@@ -229,7 +232,9 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
         int cols = 0;    // wave-uniform: 32-pixel columns of this wave with pixels of the sub-tile
 #pragma unroll
         for (int ni = 0; ni < NT; ++ni) {
-            const int pc = p0 + (wn * NT + ni) * 32;
+            // columns are dealt round-robin to the 4 pixel waves, so a partial sub-tile keeps
+            // all of them busy
+            const int pc = p0 + (ni * WGN + wn) * 32;
             const int p = pc + (lane & 31);
             b_byte[ni] = (kg * LMAX + (p <= plast ? vp_of(q, p) - vp0 : 0)) * 16;
             cols += pc <= plast ? 1 : 0;
@@ -296,12 +301,10 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
                 cbuf = cbuf == DM_NBUF - 1 ? 0 : cbuf + 1;
             }
         };
-        if (cols == 2)
-            run_stages(std::integral_constant<int, 2>{});
-        else if (cols == 1)
-            run_stages(std::integral_constant<int, 1>{});
-        else
-            run_stages(std::integral_constant<int, 0>{});
+        static_for<NT + 1>([&](auto cc) {
+            if (cols == decltype(cc)::value)
+                run_stages(cc);
+        });
 
         static_for<MT>([&](auto mic) {
             static_for<NT>([&](auto nic) { emit_tile(mic, nic, cur_o[decltype(nic)::value], rq_table); });
@@ -310,12 +313,12 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
 }
 
 // ---- configurations --------------------------------------------------------------------------
-template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3, int WGM = 2, int BPC = 1>
+template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3, int WGM = 2, int BPC = 1, int NT = 2>
 static PipeConfig make_dma_config(int act, bool table_ok) {
     constexpr int DM_BM = 32 * MT * WGM;
     PipeConfig c;
     c.bm = DM_BM;
-    c.bn = DM_BNP;
+    c.bn = 128 * NT;
     c.ks = KS;
     c.maxb = 0;
     c.g4 = 0;
@@ -327,18 +330,19 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.fixed_lmax = LMAX;
     c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + 128 * 4;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC, NT>;
     else if (act == MEGCC_NONLINE_RELU && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF, WGM, BPC>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF, WGM, BPC, NT>;
     else
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT>;
     return c;
 }
 
 // 3x3 and 1x1 NCHW44 layers and FullyConnected with at least 128 output channels (64 for the 1x1
 // with 32 input channels) and enough pixels. 1x1: 128 input channels per stage (64 / 32 when
 // IC <= 64 / 32).
-bool conv_mfma_dma_config(const ConvGeom& g, bool fc, PipeConfig* c) {
+// variant 0: 512-pixel sub-tiles (3x3 only, two stage buffers); variant 1: 256-pixel sub-tiles.
+bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, PipeConfig* c) {
     const long P = (long)g.n * g.oh * g.ow;
     const bool k3 = g.fh == 3 && g.fw == 3, k1 = g.fh == 1 && g.fw == 1;
     if (!(k3 || k1) || !(g.fmt == MEGCC_FMT_NCHW44 || fc) || g.oc < 64 || P < 2048)
@@ -350,6 +354,12 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, PipeConfig* c) {
     const bool ok = requant_table_ok(g.s_src, g.s_flt, g.s_dst);
     // measured slower on the 256-channel 56x56 layer (91 us): two 256-thread workgroups per CU
     // with 64-channel tiles and two buffers (100 us), four waves of 128 oc x 64 pixels (107 us)
+    if (variant == 0) {
+        if (!k3)
+            return false;
+        *c = make_dma_config<3, 3, 1, 768, false, 2, 2, 2, 1, 4>(g.act, ok);
+        return true;
+    }
     if (k3)
         *c = make_dma_config<3, 3, 1, 512, false>(g.act, ok);
     else if (fc)

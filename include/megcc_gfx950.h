@@ -409,6 +409,28 @@ int megcc_gfx950_model_nr_opr(void* model);
  * TINYNN_DUMP_TENSOR hooks of runtime/src/lite/network.c:187-224) */
 TinyNNStatus megcc_gfx950_model_run_opr(void* model, int index);
 
+/* `.tiny` model files (the FlatBuffers binary of runtime/schema/model.fbs written by the MegCC
+ * compiler, compiler/lib/Target/TinyNN/exporter.cpp).
+ * model_load replaces LITE_load_model_from_mem -> parse_model (runtime/src/parse.c:423-560,
+ * per-instruction loaders runtime/src/vm/op.c:11-65 and vm/memforward.c:24-41) plus
+ * init_model_weights / init_model_memory (runtime/src/init.c): weights go to HBM (fp16-compressed
+ * fp32 weights are widened like parse.c:232-263), tensors sit at the offsets of the file's static
+ * memory plan inside one arena of tensor_memory bytes, model inputs get device buffers of their
+ * own, every Opr instruction is bound by its kernel symbol (Opr.type) to the gfx950 kernel of the
+ * same name, MemForward instructions become views. The device model used is the one compiled for
+ * this device (Device value 7, appended to the schema's enum) or else the BARE_METAL one.
+ * Tensor ids of the loaded model = index in the file's tensor_pool; weight j = nr_tensor + j.
+ * Errors: TinyNN_ERROR_MODEL_PARSE for a truncated / inconsistent file (the reference traps),
+ * TinyNN_ERROR_NO_FOUND when no usable device model or no gfx950 kernel for a symbol,
+ * TinyNN_ERROR_UNSUPPORTED_INSTRUCTION_TYPE for instructions other than Opr and MemForward,
+ * TinyNN_ERROR_NO_IMPLEMENT for dynamic tensors. The buffer may be freed after the call.
+ *
+ * tiny_describe writes one text line per weight, tensor and instruction of the file (every field
+ * the loader reads); *needed receives the length including the NUL. Host code only. */
+TinyNNStatus megcc_gfx950_model_load(const void* buffer, size_t size, void** model);
+TinyNNStatus megcc_gfx950_tiny_describe(
+        const void* buffer, size_t size, char* text, size_t capacity, size_t* needed);
+
 /* The static memory plan by itself: interval i is alive during time steps [begin[i], end[i]) and
  * needs size[i] bytes; offset[i] receives its place in one arena of *arena_bytes bytes, every
  * offset a multiple of `alignment` (a power of two). Replaces, with identical offsets and arena

@@ -23,6 +23,7 @@
 
 #include "common.h"
 #include "memplan.h"
+#include "tiny_reader.h"
 
 using namespace mg;
 
@@ -33,6 +34,7 @@ struct ModelTensor {
     std::string name;
     bool is_weight = false, is_input = false, is_output = false;
     int alias_of = -1;  // MemForward / reshape: shares the memory of another tensor
+    size_t alias_offset = 0;  // MemForward: bytes from the start of that tensor
     int def = -1, last = -1;
     void* owned = nullptr;  // weights: device allocation owned by the model
 };
@@ -60,6 +62,9 @@ struct Model {
     void* workspace = nullptr;
     size_t workspace_bytes = 0;
     bool finalized = false;
+    // offsets and arena size come from a model file (the compiler's static memory plan) instead
+    // of plan_memory(); model inputs then live outside the arena, as in the TinyNN runtime
+    bool preplanned = false;
     // The operator sequence of a finalized model never changes (static shapes, static memory plan),
     // so after one eager forward it is captured once into a HIP graph and replayed: one launch per
     // forward instead of one per operator. 0: not tried yet, 1: graph in use, -1: capture failed
@@ -89,6 +94,8 @@ int root_of(const Model* m, int id) {
 // (compiler/lib/Dialect/Kernel/Transforms/StaticMemoryPlanning.cpp:88-96); model inputs are staged
 // into the arena before the first operator and outputs stay valid after forward().
 bool plan_memory(Model* m) {
+    if (m->preplanned)
+        return true;
     std::vector<MemInterval> intervals;
     std::vector<int> ids;
     for (size_t i = 0; i < m->tensors.size(); ++i) {
@@ -284,14 +291,33 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
     m->arena = m->dev.malloc(m->arena_bytes ? m->arena_bytes : 1);
     MG_REQUIRE(m->arena, TinyNN_ERROR_MEMORY_MALLOC, "model_finalize: arena of %zu bytes",
                m->arena_bytes);
-    for (auto* t : m->tensors)
-        if (!t->is_weight && t->alias_of < 0)
+    for (auto* t : m->tensors) {
+        if (t->is_weight || t->alias_of >= 0)
+            continue;
+        if (m->preplanned && t->is_input) {
+            // user memory in the TinyNN runtime (runtime/src/init.c:456-460); here a device
+            // buffer of its own that set_input fills
+            t->owned = m->dev.malloc(t->t.size ? t->t.size : 1);
+            MG_REQUIRE(t->owned, TinyNN_ERROR_MEMORY_MALLOC, "model_finalize: input of %zu bytes",
+                       (size_t)t->t.size);
+            t->t.ptr = t->owned;
+        } else {
             t->t.ptr = (char*)m->arena + t->t.offset;
+        }
+    }
     for (size_t i = 0; i < m->tensors.size(); ++i)
         if (m->tensors[i]->alias_of >= 0) {
-            const Tensor& r = m->tensors[root_of(m, (int)i)]->t;
-            m->tensors[i]->t.ptr = r.ptr;
-            m->tensors[i]->t.offset = r.offset;
+            // a chain of views adds up its offsets (output->ptr = input->ptr + offset,
+            // runtime/src/vm/memforward.c:43-53)
+            size_t shift = 0;
+            int id = (int)i;
+            while (m->tensors[id]->alias_of >= 0) {
+                shift += m->tensors[id]->alias_offset;
+                id = m->tensors[id]->alias_of;
+            }
+            const Tensor& r = m->tensors[id]->t;
+            m->tensors[i]->t.ptr = (char*)r.ptr + shift;
+            m->tensors[i]->t.offset = r.offset + shift;
         }
     for (auto* o : m->oprs) {
         for (int id : o->in)
@@ -474,6 +500,272 @@ TinyNNStatus megcc_gfx950_plan_memory(
                alignment);
     for (size_t i = 0; i < nr_interval; ++i)
         offset[i] = offsets[i];
+    return TinyNN_SUCCESS;
+}
+
+// ---- `.tiny` model files ------------------------------------------------------------------------
+
+TinyNNStatus megcc_gfx950_tiny_describe(
+        const void* buffer, size_t size, char* text, size_t capacity, size_t* needed) {
+    tiny::ModelInfo info;
+    std::string err;
+    MG_REQUIRE(tiny::read_model(buffer, size, &info, &err), TinyNN_ERROR_MODEL_PARSE,
+               "tiny_describe: %s", err.c_str());
+    const std::string s = tiny::describe(info);
+    if (needed)
+        *needed = s.size() + 1;
+    if (text && capacity) {
+        const size_t n = std::min(capacity - 1, s.size());
+        memcpy(text, s.data(), n);
+        text[n] = 0;
+    }
+    return TinyNN_SUCCESS;
+}
+
+namespace {
+
+float half_to_float(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000) << 16;
+    uint32_t e = (h >> 10) & 31, mant = h & 1023, bits;
+    if (e == 0) {
+        if (mant == 0) {
+            bits = sign;
+        } else {  // subnormal: renormalise
+            int shift = 0;
+            while (!(mant & 1024)) {
+                mant <<= 1;
+                ++shift;
+            }
+            bits = sign | ((uint32_t)(113 - shift) << 23) | ((mant & 1023) << 13);
+        }
+    } else if (e == 31) {
+        bits = sign | 0x7f800000u | (mant << 13);
+    } else {
+        bits = sign | ((e + 112) << 23) | (mant << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+// model tensor from a file entry; false (with the error set) when the entry cannot be used
+bool tensor_from_file(
+        Model* m, const tiny::DType& dt, const tiny::Layout& l, const std::string& name,
+        int* id) {
+    const int nd = (int)l.dims.size();
+    if (nd < 1 || nd > MAX_DIM || l.stride.size() != l.dims.size()) {
+        fail(TinyNN_ERROR_MODEL_PARSE, "model_load: tensor %s has %d dims, %zu strides",
+             name.c_str(), nd, l.stride.size());
+        return false;
+    }
+    uint32_t dims[MAX_DIM];
+    for (int i = 0; i < nd; ++i) {
+        if (l.dims[i] < 0) {
+            fail(TinyNN_ERROR_MODEL_PARSE, "model_load: tensor %s: negative dim", name.c_str());
+            return false;
+        }
+        dims[i] = (uint32_t)l.dims[i];
+    }
+    switch (dt.type) {
+        case tiny::DT_Float32: case tiny::DT_Float16: case tiny::DT_Int32: case tiny::DT_Int8:
+        case tiny::DT_Int16: case tiny::DT_Uint8: case tiny::DT_QInt8: case tiny::DT_QInt32:
+        case tiny::DT_QUint8:
+            break;
+        default:
+            fail(TinyNN_ERROR_UNSUPPORTED_DTYPE_TYPE, "model_load: tensor %s: dtype %d",
+                 name.c_str(), dt.type);
+            return false;
+    }
+    // the schema's enum values are the runtime's (runtime/src/parse.c:33-58)
+    *id = add_tensor(m, name.c_str(), nd, dims, (TinyNNDType)dt.type,
+                     dt.has_param ? dt.scale : 0.0f);
+    if (*id < 0) {
+        fail(TinyNN_ERROR_MODEL_PARSE, "model_load: tensor %s rejected", name.c_str());
+        return false;
+    }
+    Tensor& t = m->tensors[*id]->t;
+    t.dtype.param.zero_point = (uint8_t)dt.zero_point;
+    for (int i = 0; i < nd; ++i)
+        t.layout.stride[i] = l.stride[i];
+    t.layout.format = (TinyNNFormat)l.format;
+    return true;
+}
+
+TinyNNStatus load_into(Model* m, const tiny::ModelInfo& info) {
+    // the device model compiled for this device if there is one, else the BARE_METAL one: its
+    // instructions name the very kernels this library replaces
+    const tiny::DeviceModelInfo* dm = nullptr;
+    for (const auto& d : info.device_models)
+        if (d.device == tiny::DEV_GFX950)
+            dm = &d;
+    if (!dm)
+        for (const auto& d : info.device_models)
+            if (d.device == tiny::DEV_BARE_METAL) {
+                dm = &d;
+                break;
+            }
+    MG_REQUIRE(dm, TinyNN_ERROR_NO_FOUND,
+               "model_load: %zu device models, none for gfx950 or BARE_METAL",
+               info.device_models.size());
+
+    m->preplanned = true;
+    m->arena_bytes = dm->tensor_memory;
+    const int nt = (int)dm->tensors.size(), nw = (int)info.weights.size();
+    for (int i = 0; i < nt; ++i) {
+        const tiny::TensorInfo& ti = dm->tensors[i];
+        MG_REQUIRE(!ti.dynamic, TinyNN_ERROR_NO_IMPLEMENT,
+                   "model_load: tensor %d is dynamic (only static shapes run here)", i);
+        char dflt[32];
+        snprintf(dflt, sizeof(dflt), "tensor:%d", i);  // parse.c:121-127
+        int id = -1;
+        if (!tensor_from_file(m, ti.dtype, ti.layout, ti.name.empty() ? std::string(dflt) : ti.name, &id))
+            return TinyNN_ERROR_MODEL_PARSE;
+        ModelTensor* t = m->tensors[id];
+        t->t.use_count = ti.use_count;
+        MG_REQUIRE(ti.offset >= 0, TinyNN_ERROR_MODEL_PARSE, "model_load: tensor %d: offset", i);
+        t->t.offset = (size_t)ti.offset;
+    }
+    for (int j = 0; j < nw; ++j) {
+        const tiny::WeightInfo& wi = info.weights[j];
+        int id = -1;
+        if (!tensor_from_file(m, wi.dtype, wi.layout, wi.name, &id))
+            return TinyNN_ERROR_MODEL_PARSE;
+        ModelTensor* t = m->tensors[id];
+        t->is_weight = true;
+        t->t.is_weight = 1;
+        t->t.use_count = wi.use_count;
+        t->t.checksum = wi.checksum;
+        const size_t bytes = t->t.size;
+        std::vector<float> wide;
+        const void* host = wi.data;
+        if (wi.dtype.type == tiny::DT_Float32 && bytes && wi.data_bytes == bytes / 2) {
+            // fp32 weight stored as fp16 (parse.c:232-263)
+            wide.resize(bytes / 4);
+            for (size_t k = 0; k < wide.size(); ++k) {
+                uint16_t h;
+                memcpy(&h, wi.data + 2 * k, 2);
+                wide[k] = half_to_float(h);
+            }
+            host = wide.data();
+        } else {
+            MG_REQUIRE(wi.data_bytes == bytes, TinyNN_ERROR_MODEL_PARSE,
+                       "model_load: weight %s holds %zu bytes, its layout needs %zu",
+                       wi.name.c_str(), wi.data_bytes, bytes);
+        }
+        t->owned = m->dev.malloc(bytes ? bytes : 1);
+        MG_REQUIRE(t->owned, TinyNN_ERROR_MEMORY_MALLOC, "model_load: weight of %zu bytes", bytes);
+        t->t.ptr = t->owned;
+        if (bytes) {
+            TinyNNStatus st = megcc_gfx950_memcpy_h2d(t->owned, host, bytes);
+            if (st != TinyNN_SUCCESS)
+                return st;
+        }
+    }
+
+    for (int idx : dm->inputs) {
+        MG_REQUIRE(idx >= 0 && idx < nt, TinyNN_ERROR_MODEL_PARSE, "model_load: input index %d", idx);
+        TinyNNStatus st = megcc_gfx950_model_mark_io(m, idx, 0);
+        if (st != TinyNN_SUCCESS)
+            return st;
+        m->tensors[idx]->t.is_input = 1;
+    }
+    for (int idx : dm->outputs) {
+        MG_REQUIRE(idx >= 0 && idx < nt, TinyNN_ERROR_MODEL_PARSE, "model_load: output index %d", idx);
+        megcc_gfx950_model_mark_io(m, idx, 1);
+    }
+
+    for (size_t k = 0; k < dm->instructions.size(); ++k) {
+        const tiny::Instruction& in = dm->instructions[k];
+        if (in.kind == tiny::INST_Opr) {
+            MG_REQUIRE(in.input_types.size() == in.inputs.size(), TinyNN_ERROR_MODEL_PARSE,
+                       "model_load: instruction %zu: %zu inputs, %zu input types", k,
+                       in.inputs.size(), in.input_types.size());
+            std::vector<int> ins, outs;
+            for (size_t i = 0; i < in.inputs.size(); ++i) {
+                const bool w = in.input_types[i] == tiny::TT_WEIGHT;
+                const int idx = in.inputs[i];
+                MG_REQUIRE(idx >= 0 && idx < (w ? nw : nt), TinyNN_ERROR_MODEL_PARSE,
+                           "model_load: instruction %zu: input index %d", k, idx);
+                ins.push_back(w ? nt + idx : idx);
+            }
+            for (int idx : in.outputs) {
+                MG_REQUIRE(idx >= 0 && idx < nt, TinyNN_ERROR_MODEL_PARSE,
+                           "model_load: instruction %zu: output index %d", k, idx);
+                outs.push_back(idx);
+            }
+            TinyNNStatus st = megcc_gfx950_model_add_opr(
+                    m, in.type.c_str(), ins.data(), (int)ins.size(), outs.data(), (int)outs.size());
+            if (st != TinyNN_SUCCESS)
+                return st == TinyNN_ERROR_NO_FOUND
+                             ? fail(TinyNN_ERROR_NO_FOUND,
+                                    "model_load: instruction %zu: no gfx950 kernel for %s", k,
+                                    in.type.c_str())
+                             : st;
+        } else if (in.kind == tiny::INST_MemForward) {
+            const int src = in.fwd_input, dst = in.fwd_output;
+            MG_REQUIRE(src >= 0 && src < nt && dst >= 0 && dst < nt && src != dst,
+                       TinyNN_ERROR_MODEL_PARSE, "model_load: instruction %zu: MemForward %d -> %d",
+                       k, src, dst);
+            ModelTensor* o = m->tensors[dst];
+            MG_REQUIRE(o->alias_of < 0 && o->def < 0, TinyNN_ERROR_MODEL_PARSE,
+                       "model_load: instruction %zu: tensor %d already has memory", k, dst);
+            MG_REQUIRE(in.fwd_offset >= 0, TinyNN_ERROR_MODEL_PARSE,
+                       "model_load: instruction %zu: negative MemForward offset", k);
+            for (int id = src, hops = 0; id >= 0; id = m->tensors[id]->alias_of)
+                MG_REQUIRE(id != dst && ++hops <= nt, TinyNN_ERROR_MODEL_PARSE,
+                           "model_load: instruction %zu: MemForward cycle", k);
+            o->alias_of = src;
+            o->alias_offset = (size_t)in.fwd_offset;
+        } else {
+            return fail(TinyNN_ERROR_UNSUPPORTED_INSTRUCTION_TYPE,
+                        "model_load: instruction %zu has type %d; this runtime executes Opr and "
+                        "MemForward", k, in.kind);
+        }
+    }
+
+    // every byte a kernel may touch lies inside the arena (or inside the tensor a view points at)
+    for (int i = 0; i < nt; ++i) {
+        ModelTensor* t = m->tensors[i];
+        if (t->alias_of >= 0) {
+            size_t shift = 0;
+            int id = i, hops = 0;
+            while (m->tensors[id]->alias_of >= 0) {
+                shift += m->tensors[id]->alias_offset;
+                id = m->tensors[id]->alias_of;
+                MG_REQUIRE(++hops <= nt, TinyNN_ERROR_MODEL_PARSE, "model_load: MemForward cycle");
+            }
+            MG_REQUIRE(shift + t->t.size <= m->tensors[id]->t.size, TinyNN_ERROR_MODEL_PARSE,
+                       "model_load: tensor %d views bytes %zu..%zu of tensor %d (%zu bytes)", i,
+                       shift, shift + (size_t)t->t.size, id, (size_t)m->tensors[id]->t.size);
+        } else if (!t->is_input) {
+            MG_REQUIRE(t->t.offset + t->t.size <= m->arena_bytes, TinyNN_ERROR_MODEL_PARSE,
+                       "model_load: tensor %d ends at byte %zu of a %zu byte arena", i,
+                       (size_t)(t->t.offset + t->t.size), m->arena_bytes);
+        }
+    }
+    return megcc_gfx950_model_finalize(m);
+}
+
+}  // namespace
+
+// parse_model + init_model_weights + init_model_memory (runtime/src/parse.c:423-560,
+// runtime/src/init.c) for this device. Tensor ids of the returned model: the file's tensor_pool
+// index; weight j of the weight_pool is id nr_tensor + j.
+TinyNNStatus megcc_gfx950_model_load(const void* buffer, size_t size, void** model) {
+    MG_REQUIRE(model, TinyNN_ERROR_NULL_PTR, "model_load: null result pointer");
+    *model = nullptr;
+    tiny::ModelInfo info;
+    std::string err;
+    MG_REQUIRE(tiny::read_model(buffer, size, &info, &err), TinyNN_ERROR_MODEL_PARSE,
+               "model_load: %s", err.c_str());
+    Model* m = (Model*)megcc_gfx950_model_create();
+    MG_REQUIRE(m, TinyNN_ERROR_RUNTIME, "model_load: no device");
+    TinyNNStatus st = load_into(m, info);
+    if (st != TinyNN_SUCCESS) {
+        megcc_gfx950_model_destroy(m);
+        return st;
+    }
+    *model = m;
     return TinyNN_SUCCESS;
 }
 

@@ -72,6 +72,9 @@ def lib():
         L.megcc_gfx950_model_forward.argtypes = [C.c_void_p]
         L.megcc_gfx950_model_nr_opr.argtypes = [C.c_void_p]
         L.megcc_gfx950_model_run_opr.argtypes = [C.c_void_p, C.c_int]
+        L.megcc_gfx950_model_load.argtypes = [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]
+        L.megcc_gfx950_tiny_describe.argtypes = [C.c_void_p, C.c_size_t, C.c_char_p, C.c_size_t,
+                                                 C.POINTER(C.c_size_t)]
         sizes = C.POINTER(C.c_size_t)
         L.megcc_gfx950_plan_memory.argtypes = [
             C.c_size_t, sizes, sizes, sizes, C.c_size_t, sizes, sizes, sizes]
@@ -93,7 +96,8 @@ EXPORTS = [
     "megcc_gfx950_model_mark_io", "megcc_gfx950_model_finalize", "megcc_gfx950_model_arena_bytes",
     "megcc_gfx950_model_tensor_ptr", "megcc_gfx950_model_set_input",
     "megcc_gfx950_model_get_output", "megcc_gfx950_model_forward", "megcc_gfx950_model_nr_opr",
-    "megcc_gfx950_model_run_opr", "megcc_gfx950_plan_memory",
+    "megcc_gfx950_model_run_opr", "megcc_gfx950_plan_memory", "megcc_gfx950_model_load",
+    "megcc_gfx950_tiny_describe",
 ]
 
 
@@ -119,6 +123,16 @@ def plan_memory(begin, end, size, alignment=1):
         n, ptr(arrs[0]), ptr(arrs[1]), ptr(arrs[2]), alignment, ptr(off),
         C.byref(total), C.byref(bound)), "plan_memory")
     return off[:n].astype(np.int64), int(total.value), int(bound.value)
+
+
+def tiny_describe(data):
+    """Text listing of a `.tiny` model file (bytes): one line per weight, tensor, instruction."""
+    data = bytes(data)
+    need = C.c_size_t(0)
+    check(lib().megcc_gfx950_tiny_describe(data, len(data), None, 0, C.byref(need)), "tiny_describe")
+    buf = C.create_string_buffer(need.value)
+    check(lib().megcc_gfx950_tiny_describe(data, len(data), buf, need.value, None), "tiny_describe")
+    return buf.value.decode(errors="replace")
 
 
 class DeviceBuffer:
@@ -247,6 +261,20 @@ class Model:
         if not self.h:
             raise MegccError("model_create failed: " + lib().megcc_gfx950_last_error().decode())
         self.shapes = {}
+
+    @classmethod
+    def load(cls, data, shapes=None):
+        """Model from the bytes of a `.tiny` file (megcc_gfx950_model_load). Tensor ids are the
+        file's tensor_pool indices; `shapes` = {id: (shape, dtype enum)} for the tensors get()
+        will be asked for."""
+        self = cls.__new__(cls)
+        self.h = None
+        self.shapes = dict(shapes or {})
+        data = bytes(data)
+        h = C.c_void_p()
+        check(lib().megcc_gfx950_model_load(data, len(data), C.byref(h)), "model_load")
+        self.h = h.value
+        return self
 
     @staticmethod
     def _dims(shape):

@@ -115,3 +115,16 @@ def plan_memory(begin, end, size, alignment=1):
         C.byref(total), C.byref(bound))
     assert st == 0
     return off[:n].astype(np.int64), int(total.value), int(bound.value)
+
+
+_TINY_DUMP = os.path.join(_HERE, "_ref", "ref_tiny_dump")
+
+
+def tiny_dump_available():
+    return os.path.exists(_TINY_DUMP)
+
+
+def tiny_dump(path):
+    """What the reference's generated FlatBuffers reader sees in the `.tiny` file at `path`
+    (oracle/ref_tiny_dump.c), as text."""
+    return subprocess.run([_TINY_DUMP, path], check=True, capture_output=True, text=True).stdout

@@ -167,25 +167,19 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
         if constexpr (ACT == ACT_RT) {
 #pragma unroll
             for (int e = 0; e < 16; ++e)
-                r[e] = requant_conv_rt(q.act, acc[mi][ni][e] + tbl[REQUANT_TABLE_ENTRIES + ocl + (e / 4) * 8 + e % 4],
-                                       q.s_src, q.s_flt, q.s_dst);
+                r[e] = requant_conv_rt(q.act, acc[mi][ni][e], q.s_src, q.s_flt, q.s_dst);
         } else {
             constexpr int LO = ACT == MEGCC_NONLINE_RELU ? 0 : -128;
-            v4i bv[4];
-#pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4)
-                bv[e4] = *(const v4i*)(tbl + REQUANT_TABLE_ENTRIES + ocl + e4 * 8);
-            int a[16], m[16], t[16];
+            int m[16], t[16];
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                a[e] = acc[mi][ni][e] + bv[e / 4][e % 4];
-                const int f = (int)__builtin_floorf((float)a[e] * q.rq.c);
+                const int f = cvt_floor_i32((float)acc[mi][ni][e] * q.rq.c);
                 m[e] = f < LO ? LO : (f > 126 ? 126 : f);
                 t[e] = tbl[m[e] + 128];
             }
 #pragma unroll
             for (int e = 0; e < 16; ++e)
-                r[e] = m[e] + (a[e] > t[e] ? 1 : 0);
+                r[e] = m[e] + (acc[mi][ni][e] > t[e] ? 1 : 0);
         }
         if (ob >= 0) {
 #pragma unroll
@@ -244,13 +238,20 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
                         : FC        ? p
                                     : pn * (q.OC >> 2) * q.OHW + (p - pn * q.OHW);
         }
+        // the accumulators start from the bias of their output channel (register e of a tile:
+        // channel 8 * (e / 4) + 4 * kg + e % 4)
 #pragma unroll
-        for (int mi = 0; mi < MT; ++mi)
+        for (int mi = 0; mi < MT; ++mi) {
+            v4i bv[4];
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4)
+                bv[e4] = *(const v4i*)(bias_lds + (wm * MT + mi) * 32 + kg * 4 + e4 * 8);
 #pragma unroll
             for (int ni = 0; ni < NT; ++ni)
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
-                    acc[mi][ni][e] = 0;
+                    acc[mi][ni][e] = bv[e / 4][e % 4];
+        }
 
         auto stage_body = [&](auto cols_c, const int8_t* bufA, int8_t* dma_buf) __attribute__((always_inline)) {
             constexpr int COLS = decltype(cols_c)::value;

@@ -167,6 +167,13 @@ static inline bool requant_table_ok(float s_src, float s_flt, float s_dst) {
     return q.c != 0.f && q.c * 2147483648.f > 1000.f;
 }
 
+// (int)floorf(x) in one instruction (saturating like the plain conversion)
+__device__ __forceinline__ int cvt_floor_i32(float x) {
+    int r;
+    asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
+
 // bytes 0 of a, b, c, d -> one dword
 __device__ __forceinline__ uint32_t pack4_perm(int a, int b, int c, int d) {
     const uint32_t lo = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);

@@ -1,6 +1,7 @@
 // Definitions shared by the two qsi8 MFMA convolution kernels (conv_mfma_i8.hip: one stage at a time,
 // any shape; conv_mfma_i8_wide.hip and conv_mfma_i8_ws.hip: pipelined, large shapes).
 #pragma once
+#include <stddef.h>
 #include <utility>
 
 #include "common.h"
@@ -69,7 +70,19 @@ struct MfmaParams {
     FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
     int G, RG;       // 16-byte gather: pixel groups per row, groups per plane of the largest patch
     FastDiv dG, dRG;
+    // exact requantisation thresholds for IDENTITY / RELU (built on the host, epilogue.cuh); only
+    // the kernels that look outputs up in LDS read it
+    RequantTable rq_table;
 };
+
+// Entry i of the threshold table of a kernel whose ONLY argument is an MfmaParams, read straight
+// from the kernel-argument segment (indexing the by-value struct with a run-time index can make
+// the compiler copy all of it to scratch).
+__device__ __forceinline__ int kernarg_rq_table(int i) {
+    typedef const __attribute__((address_space(4))) char* kptr;
+    const kptr base = (kptr)__builtin_amdgcn_kernarg_segment_ptr();
+    return *(const __attribute__((address_space(4))) int*)(base + offsetof(MfmaParams, rq_table) + 4 * i);
+}
 
 // virtual pixel index of output pixel p at tap (0,0): rows of the zero-padded images stacked
 __device__ __forceinline__ int vp_of(const MfmaParams& q, int p) {

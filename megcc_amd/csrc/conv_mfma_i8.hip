@@ -464,7 +464,7 @@ TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
 TinyNNStatus conv_mfma_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst,
         const Workspace* ws) {
-    MfmaParams q;
+    MfmaParams q = {};
     PipeConfig pc;
     const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;
     // candidates in order of preference; development switches MEGCC_NODMA / MEGCC_NOWS /
@@ -558,6 +558,9 @@ TinyNNStatus conv_mfma_launch(
     q.s_flt = g.s_flt;
     q.s_dst = g.s_dst;
     q.rq = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
+    if (pipe && (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
+        requant_table_ok(g.s_src, g.s_flt, g.s_dst))
+        q.rq_table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
     q.dOW = make_fastdiv(q.OW);
     q.dOH = make_fastdiv(q.OH);
     q.dVW = make_fastdiv(q.VW);

@@ -76,7 +76,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     // ---- once per workgroup: requantisation thresholds and the bias slice of this oc tile
     if constexpr (ACT != ACT_RT) {
         if (tid < REQUANT_TABLE_ENTRIES)
-            rq_table[tid] = tid < 255 ? requant_threshold<ACT>(tid, q.s_src, q.s_flt, q.s_dst, q.rq.c) : 0;
+            rq_table[tid] = kernarg_rq_table(tid);
     }
     for (int i = tid; i < DM_BM; i += DM_THREADS)
         bias_lds[i] = (q.bias && oc0 + i < q.OC) ? q.bias[oc0 + i] : 0;

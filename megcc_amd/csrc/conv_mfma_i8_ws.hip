@@ -210,7 +210,7 @@ __global__ void __launch_bounds__(WS_THREADS) conv_mfma_i8_ws_kernel(MfmaParams 
     int* const rq_table = (int*)(lds + WS_NBUF * buf_bytes);
     if constexpr (ACT != ACT_RT) {
         if (tid < REQUANT_TABLE_ENTRIES)
-            rq_table[tid] = tid < 255 ? requant_threshold<ACT>(tid, q.s_src, q.s_flt, q.s_dst, q.rq.c) : 0;
+            rq_table[tid] = kernarg_rq_table(tid);
     }
     lds_barrier();  // step -3
     lds_barrier();  // step -2

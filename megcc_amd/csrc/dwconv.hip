@@ -79,18 +79,29 @@ __device__ __forceinline__ void transpose4x4(const dw_v4u p, unsigned (&t)[4]) {
     t[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
 }
 
-template <int S, int ACT>
+// Two vertically adjacent output rows per thread: their 3 + 3 input rows overlap (4 distinct rows
+// for stride 1, 5 for stride 2), so a row is loaded and transposed once for both, and the weights
+// are rearranged once for 32 outputs.
+template <int S, int ACT, int R>
 __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
         ConvGeom g, RequantFast rq, const uint32_t* __restrict__ src, const uint32_t* __restrict__ flt,
-        const int32_t* __restrict__ bias, uint32_t* __restrict__ dst, int total, int src_bytes) {
+        const int32_t* __restrict__ bias, uint32_t* __restrict__ dst, int total, int src_bytes,
+        RequantTable table) {
+    __shared__ int tbl[REQUANT_TABLE_ENTRIES];
+    if (ACT >= 0) {
+        tbl[threadIdx.x] = table.t[threadIdx.x];
+        __syncthreads();
+    }
+    constexpr int ROWS = (R - 1) * S + 3;   // input rows they need
     const int c4n = g.oc >> 2;
     const int ogn = (g.ow + 3) >> 2;  // groups of 4 output pixels per row
+    const int ohn = (g.oh + R - 1) / R;
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, src_bytes, 0x00020000);
     const int OOB = (int)0x80000000u;
     for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
         int r = i;
         const int og = r % ogn; r /= ogn;
-        const int oh = r % g.oh; r /= g.oh;
+        const int oh = (r % ohn) * R; r /= ohn;
         const int c4 = r % c4n;
         const int n = r / c4n;
         const int plane_off = ((n * c4n + c4) * g.ih) * g.iw * 4;  // bytes
@@ -102,7 +113,7 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
             const dw_v4u fv = {f[0], f[1], f[2], 0u};
             transpose4x4(fv, wq[fh]);
         }
-        int acc[4][4];  // [pixel][channel]
+        int acc[R * 16];  // [row][pixel][channel]
         {
             int b4[4] = {0, 0, 0, 0};
             if (bias) {
@@ -111,15 +122,14 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
                     b4[c] = bias[c4 * 4 + c];
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    acc[j][c] = b4[c];
+            for (int e = 0; e < R * 16; ++e)
+                acc[e] = b4[e & 3];
         }
-        const int iw0 = og * 4 * S;  // first input pixel of the aligned loads
+        const int iw0 = og * 4 * S;   // first input pixel of the aligned loads
+        const int left = g.iw - iw0;  // valid pixels from iw0 on
 #pragma unroll
-        for (int fh = 0; fh < 3; ++fh) {
-            const int ih = oh * S - 1 + fh;
+        for (int ir = 0; ir < ROWS; ++ir) {
+            const int ih = oh * S - 1 + ir;
             const bool row_ok = (unsigned)ih < (unsigned)g.ih;
             const int row_off = plane_off + ih * g.iw * 4;
             // left neighbour pixel (iw0 - 1), pixel-major dword
@@ -127,23 +137,22 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
                     rs, row_ok && iw0 > 0 ? row_off + (iw0 - 1) * 4 : OOB, 0, 0);
             dw_v4u l0 = __builtin_amdgcn_raw_buffer_load_b128(rs, row_ok ? row_off + iw0 * 4 : OOB, 0, 0);
             // pixels past the end of the row belong to the next row: zero them
-            const int left = g.iw - iw0;  // valid pixels from iw0 on
 #pragma unroll
             for (int k = 1; k < 4; ++k)
                 l0[k] = k < left ? l0[k] : 0u;
             unsigned t0[4];
             transpose4x4(l0, t0);
+            // the four 3-pixel windows of each channel in this input row
+            unsigned win[4][4];  // [pixel][channel]
             if (S == 1) {
                 const unsigned nx = __builtin_amdgcn_raw_buffer_load_b32(
                         rs, row_ok && left > 4 ? row_off + (iw0 + 4) * 4 : OOB, 0, 0);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    const unsigned x0 = __builtin_amdgcn_perm(t0[c], pv, 0x06050400u | c);
-                    const unsigned x3 = __builtin_amdgcn_perm(nx, t0[c], 0x0c000302u | ((4u + c) << 16));
-                    acc[0][c] = __builtin_amdgcn_sdot4((int)x0, (int)wq[fh][c], acc[0][c], false);
-                    acc[1][c] = __builtin_amdgcn_sdot4((int)t0[c], (int)wq[fh][c], acc[1][c], false);
-                    acc[2][c] = __builtin_amdgcn_sdot4((int)(t0[c] >> 8), (int)wq[fh][c], acc[2][c], false);
-                    acc[3][c] = __builtin_amdgcn_sdot4((int)x3, (int)wq[fh][c], acc[3][c], false);
+                    win[0][c] = __builtin_amdgcn_perm(t0[c], pv, 0x06050400u | c);
+                    win[1][c] = t0[c];
+                    win[2][c] = t0[c] >> 8;
+                    win[3][c] = __builtin_amdgcn_perm(nx, t0[c], 0x0c000302u | ((4u + c) << 16));
                 }
             } else {
                 dw_v4u l1 = __builtin_amdgcn_raw_buffer_load_b128(
@@ -155,41 +164,57 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
                 transpose4x4(l1, t1);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    const unsigned x0 = __builtin_amdgcn_perm(t0[c], pv, 0x06050400u | c);
-                    const unsigned x2 = __builtin_amdgcn_alignbyte(t1[c], t0[c], 3);
-                    acc[0][c] = __builtin_amdgcn_sdot4((int)x0, (int)wq[fh][c], acc[0][c], false);
-                    acc[1][c] = __builtin_amdgcn_sdot4((int)(t0[c] >> 8), (int)wq[fh][c], acc[1][c], false);
-                    acc[2][c] = __builtin_amdgcn_sdot4((int)x2, (int)wq[fh][c], acc[2][c], false);
-                    acc[3][c] = __builtin_amdgcn_sdot4((int)(t1[c] >> 8), (int)wq[fh][c], acc[3][c], false);
+                    win[0][c] = __builtin_amdgcn_perm(t0[c], pv, 0x06050400u | c);
+                    win[1][c] = t0[c] >> 8;
+                    win[2][c] = __builtin_amdgcn_alignbyte(t1[c], t0[c], 3);
+                    win[3][c] = t1[c] >> 8;
                 }
             }
-        }
-        uint32_t o[4];
+            // input row ir is filter row ir - orow * S of output row orow
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            int q[4];
+            for (int orow = 0; orow < R; ++orow) {
+                const int fh = ir - orow * S;
+                if (fh < 0 || fh > 2)
+                    continue;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if (ACT < 0)
-                    q[c] = requant_conv_rt(g.act, acc[j][c], g.s_src, g.s_flt, g.s_dst);
-                else
-                    q[c] = requant_conv_fast<(ACT < 0 ? 0 : ACT)>(acc[j][c], rq);
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        acc[orow * 16 + j * 4 + c] = __builtin_amdgcn_sdot4(
+                                (int)win[j][c], (int)wq[fh][c], acc[orow * 16 + j * 4 + c], false);
             }
-            o[j] = pack4_perm(q[0], q[1], q[2], q[3]);
         }
-        uint32_t* out = dst + ((size_t)(n * c4n + c4) * g.oh + oh) * g.ow + og * 4;
-        if (og * 4 + 4 <= g.ow && (g.ow & 3) == 0) {
-            *(uint4*)out = make_uint4(o[0], o[1], o[2], o[3]);
+        if (ACT < 0) {
+#pragma unroll
+            for (int e = 0; e < R * 16; ++e)
+                acc[e] = requant_conv_rt(g.act, acc[e], g.s_src, g.s_flt, g.s_dst);
         } else {
 #pragma unroll
+            for (int e = 0; e < R * 16; ++e)
+                acc[e] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[e], rq.c, tbl);
+        }
+#pragma unroll
+        for (int orow = 0; orow < R; ++orow) {
+            if (oh + orow >= g.oh)
+                break;
+            uint32_t o[4];
+#pragma unroll
             for (int j = 0; j < 4; ++j)
-                if (og * 4 + j < g.ow)
-                    out[j] = o[j];
+                o[j] = pack4_perm(acc[orow * 16 + j * 4], acc[orow * 16 + j * 4 + 1],
+                                  acc[orow * 16 + j * 4 + 2], acc[orow * 16 + j * 4 + 3]);
+            uint32_t* out = dst + ((size_t)(n * c4n + c4) * g.oh + oh + orow) * g.ow + og * 4;
+            if (og * 4 + 4 <= g.ow && (g.ow & 3) == 0) {
+                *(uint4*)out = make_uint4(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (og * 4 + j < g.ow)
+                        out[j] = o[j];
+            }
         }
     }
 }
 
-// 3x3, pad 1, no dilation, stride 1 or 2 (square); buffer loads only need dword alignment
 static bool dwconv44_3x3_ok(const ConvGeom& g, const void* src, const void* dst) {
     const long src_bytes = (long)g.n * g.ic * g.ih * g.iw;
     const long groups4 = (long)g.n * (g.oc >> 2) * g.oh * ((g.ow + 3) / 4);
@@ -210,21 +235,33 @@ TinyNNStatus dwconv44_launch(
     if (total == 0)
         return TinyNN_SUCCESS;
     if (dwconv44_3x3_ok(g, src, dst) && !getenv("MEGCC_DW_GENERIC")) {
-        const int groups4 = (int)((long)g.n * (g.oc >> 2) * g.oh * ((g.ow + 3) / 4));
+        // one thread per R output rows x 4 output pixels x 4 channels
+        // (two rows share input rows and the weight set-up: measured faster for stride 1 on
+        // large planes only)
+        const int R = g.sh == 1 && g.oh >= 28 ? 2 : 1;
+        const int groups4 = (int)((long)g.n * (g.oc >> 2) * ((g.oh + R - 1) / R) * ((g.ow + 3) / 4));
         unsigned nb = (unsigned)((groups4 + 255) / 256);
         const RequantFast rq3 = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
-        void (*k3)(ConvGeom, RequantFast, const uint32_t*, const uint32_t*, const int32_t*, uint32_t*, int, int);
+        void (*k3)(ConvGeom, RequantFast, const uint32_t*, const uint32_t*, const int32_t*, uint32_t*, int, int,
+                   RequantTable);
+        // exact thresholds for the monotone activations; anything else (and extreme scales)
+        // evaluates the literal sequence per output
+        const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
+                         requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+        static const RequantTable no_table = {};
+        const RequantTable& table = tab ? requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst) : no_table;
+#define MG_DW_PICK(S_, R_)                                                                      \
+    (tab && g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_IDENTITY, R_> \
+     : tab && g.act == MEGCC_NONLINE_RELU   ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_RELU, R_>     \
+                                            : dwconv44_3x3_kernel<S_, -1, R_>)
         if (g.sh == 1)
-            k3 = g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_3x3_kernel<1, MEGCC_NONLINE_IDENTITY>
-               : g.act == MEGCC_NONLINE_RELU     ? dwconv44_3x3_kernel<1, MEGCC_NONLINE_RELU>
-                                                 : dwconv44_3x3_kernel<1, -1>;
+            k3 = R == 2 ? MG_DW_PICK(1, 2) : MG_DW_PICK(1, 1);
         else
-            k3 = g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_3x3_kernel<2, MEGCC_NONLINE_IDENTITY>
-               : g.act == MEGCC_NONLINE_RELU     ? dwconv44_3x3_kernel<2, MEGCC_NONLINE_RELU>
-                                                 : dwconv44_3x3_kernel<2, -1>;
+            k3 = R == 2 ? MG_DW_PICK(2, 2) : MG_DW_PICK(2, 1);
+#undef MG_DW_PICK
         hipLaunchKernelGGL(k3, dim3(nb), dim3(256), 0, stream(), g, rq3, (const uint32_t*)src,
                            (const uint32_t*)flt, (const int32_t*)bias, (uint32_t*)dst, groups4,
-                           (int)((long)g.n * g.ic * g.ih * g.iw));
+                           (int)((long)g.n * g.ic * g.ih * g.iw), table);
         return check_launch("dwconv44_3x3");
     }
     unsigned blocks = (unsigned)((total + 255) / 256);

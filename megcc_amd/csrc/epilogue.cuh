@@ -17,7 +17,7 @@
 namespace mg {
 
 template <int ACT>
-__device__ __forceinline__ float act_apply(float x) {
+__host__ __device__ __forceinline__ float act_apply(float x) {
     if (ACT == MEGCC_NONLINE_RELU) {
         return x > 0 ? x : 0;
     } else if (ACT == MEGCC_NONLINE_H_SWISH) {
@@ -32,7 +32,7 @@ __device__ __forceinline__ float act_apply(float x) {
     return x;
 }
 
-__device__ __forceinline__ int fp32_to_int8(float v) {
+__host__ __device__ __forceinline__ int fp32_to_int8(float v) {
     int r = (int)roundf(v);
     r = r > 127 ? 127 : r;
     r = r < -128 ? -128 : r;
@@ -41,7 +41,7 @@ __device__ __forceinline__ int fp32_to_int8(float v) {
 
 // acc already includes the int32 bias.
 template <int ACT>
-__device__ __forceinline__ int requant_conv(int acc, float s_src, float s_flt, float s_dst) {
+__host__ __device__ __forceinline__ int requant_conv(int acc, float s_src, float s_flt, float s_dst) {
     float v = (float)acc * s_src * s_flt / s_dst;
     return fp32_to_int8(act_apply<ACT>(v));
 }
@@ -112,8 +112,10 @@ __device__ __forceinline__ int requant_conv_rt(int act, int acc, float s0, float
 // For a monotone activation (IDENTITY, RELU) the reference's F(acc) = fp32_to_int8(act(acc * s_src
 // * s_flt / s_dst)) is a non-decreasing step function of the integer accumulator, so it is fully
 // described by 255 thresholds T[j] = max{a : F(a) < j}, j = -127..127:  F(a) = lo + #{j : a > T[j]}.
-// A kernel builds the table once per workgroup with the reference's literal float sequence
-// (binary search over int32, one entry per thread), and then needs only ONE estimate per output:
+// The table is built with the reference's literal float sequence (binary search over int32) - on
+// the host, once per (activation, scales) and cached, since x86-64 SSE arithmetic and the device's
+// are the same IEEE operations; it travels to the kernel as an argument and each workgroup copies
+// it to LDS. A kernel then needs only ONE estimate per output:
 // with g = fl((float)a * c), c = fl(fl(s_src*s_flt)/s_dst), the true value is within 2^-14 of g
 // while |g| < 129, so F(a) is floor(g) or floor(g)+1 (clamped), and the table decides which:
 //     m = clamp(floor(g), lo, 126);   F(a) = m + (a > T[m + 1])
@@ -123,7 +125,7 @@ static constexpr int REQUANT_TABLE_ENTRIES = 256;  // entry j + 127, last one un
 // entry `idx` (0..254) of the table: a handful of evaluations of the literal sequence (32 when
 // the estimate from c is useless)
 template <int ACT>
-__device__ __forceinline__ int requant_threshold(int idx, float s_src, float s_flt, float s_dst, float c) {
+__host__ __device__ __forceinline__ int requant_threshold(int idx, float s_src, float s_flt, float s_dst, float c) {
     const int j = idx - 127;
     auto below = [&](long long a) { return requant_conv<ACT>((int)a, s_src, s_flt, s_dst) < j; };
     long long lo = INT32_MIN, hi = INT32_MAX;
@@ -150,13 +152,27 @@ __device__ __forceinline__ int requant_threshold(int idx, float s_src, float s_f
     return (int)lo;
 }
 
+// (int)floorf(x) in one instruction (saturating like the plain conversion)
+__device__ __forceinline__ int cvt_floor_i32(float x) {
+    int r;
+    asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
+
+struct RequantTable {
+    int t[REQUANT_TABLE_ENTRIES];
+};
+
+// host: the table for (act in {IDENTITY, RELU}, scales); the reference stays valid for the life of
+// the process (requant_table.hip)
+const RequantTable& requant_table_for(int act, float s_src, float s_flt, float s_dst);
+
 // table: pointer to entry 0 (LDS). ACT_LO: lowest output (-128, or 0 with RELU).
 template <int ACT>
 __device__ __forceinline__ int requant_conv_table(int acc, float c, const int* table) {
     static_assert(ACT == MEGCC_NONLINE_IDENTITY || ACT == MEGCC_NONLINE_RELU, "monotone only");
     constexpr int LO = ACT == MEGCC_NONLINE_RELU ? 0 : -128;
-    const float g = (float)acc * c;
-    int m = (int)__builtin_floorf(g);  // saturating conversion
+    int m = cvt_floor_i32((float)acc * c);  // saturating conversion
     m = m < LO ? LO : (m > 126 ? 126 : m);
     return m + (acc > table[m + 128] ? 1 : 0);
 }
@@ -165,13 +181,6 @@ __device__ __forceinline__ int requant_conv_table(int acc, float c, const int* t
 static inline bool requant_table_ok(float s_src, float s_flt, float s_dst) {
     const RequantFast q = make_requant_fast(s_src, s_flt, s_dst);
     return q.c != 0.f && q.c * 2147483648.f > 1000.f;
-}
-
-// (int)floorf(x) in one instruction (saturating like the plain conversion)
-__device__ __forceinline__ int cvt_floor_i32(float x) {
-    int r;
-    asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(r) : "v"(x));
-    return r;
 }
 
 // bytes 0 of a, b, c, d -> one dword

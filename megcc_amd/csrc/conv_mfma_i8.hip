@@ -21,6 +21,10 @@
 //     one NCHW44 dword per pixel, so 32 lanes store 128 contiguous bytes.
 #include <stdlib.h>
 
+#include <array>
+#include <map>
+#include <mutex>
+
 #include "conv_mfma_i8.h"
 
 namespace mg {
@@ -387,7 +391,26 @@ struct TilePlan {
 };
 
 // largest patch any tile of `bn` pixels needs; mirrors vp_of() / L in the kernels
+static TilePlan plan_tiles_uncached(const ConvGeom& g, int bn, long range_len);
+
+// The plan walks over every tile of the layer: kept per geometry, so that a launch costs the host
+// a map look-up and not a loop over the tensor.
 static TilePlan plan_tiles(const ConvGeom& g, int bn = BN, long range_len = 0) {
+    typedef std::array<long, 16> Key;
+    static std::map<Key, TilePlan> cache;
+    static std::mutex lock;
+    const Key key = {g.n, g.ih, g.iw, g.oh, g.ow, g.fh, g.fw, g.sh, g.sw, g.ph, g.pw, g.dh, g.dw,
+                     bn, range_len, 0};
+    std::lock_guard<std::mutex> guard(lock);
+    auto it = cache.find(key);
+    if (it != cache.end())
+        return it->second;
+    if (cache.size() > 4096)
+        cache.clear();
+    return cache[key] = plan_tiles_uncached(g, bn, range_len);
+}
+
+static TilePlan plan_tiles_uncached(const ConvGeom& g, int bn, long range_len) {
     TilePlan t;
     t.VW = g.iw + 2 * g.pw;
     t.VH = g.ih + 2 * g.ph;
@@ -461,9 +484,16 @@ bool conv_mfma_ws_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
 bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, PipeConfig* c);
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
 
+bool conv_pw_stream_supported(const ConvGeom& g);
+TinyNNStatus conv_pw_stream_launch(
+        const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst);
+
 TinyNNStatus conv_mfma_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst,
         const Workspace* ws) {
+    // pointwise layers with few input channels: the streaming kernel (conv_pw_stream.hip)
+    if (conv_pw_stream_supported(g) && !getenv("MEGCC_NOPWS"))
+        return conv_pw_stream_launch(g, src, packed, bias, dst);
     MfmaParams q = {};
     PipeConfig pc;
     const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;

@@ -1,0 +1,264 @@
+// qsi8 pointwise (1x1, stride 1) NCHW44 convolution with few input channels: a streaming kernel.
+//
+// With K = IC <= 256 a pointwise layer does one to eight MFMAs per 32 x 32 output tile and then
+// requantises 16 outputs per lane: the layer is bound by HBM and by the epilogue's vector
+// instructions, not by the matrix cores, and any staging through LDS (barriers, stage buffers,
+// one workgroup per CU) only adds latency. So nothing is staged:
+//   * a wave owns 64 output channels and keeps their filter rows in registers for its whole life
+//     (2 MFMA row tiles x IC/32 K-chunks x 4 VGPRs, read once from the packed filter);
+//   * it walks over 32-pixel tiles; the MFMA B operand of a tile is exactly what NCHW44 holds per
+//     lane - lane (pixel l & 31, K-half l >> 5) needs 16 consecutive channels = one dword from
+//     each of 4 consecutive channel planes - so it is loaded straight from global memory, 128
+//     contiguous bytes per plane and half wave, the next tile's loads issued before the current
+//     tile's MFMAs;
+//   * results leave like in the tiled kernels: 4 consecutive accumulator registers are the 4
+//     channels of one NCHW44 dword, 32 lanes store 128 contiguous bytes.
+// Waves never synchronise after the set-up (threshold table and bias to LDS), so any number of
+// them can be resident and the memory latency is hidden by occupancy.
+//
+// Same arithmetic as the other qsi8 kernels: int32 accumulators starting from the bias, exact
+// requantisation by threshold table (epilogue.cuh). Reference loop: BareMetal/ConvKernel.cpp:305-344.
+#include <map>
+#include <mutex>
+
+#include "conv_mfma_i8.h"
+
+namespace mg {
+
+static constexpr int PW_THREADS = 256;
+static constexpr int PW_MAX_OC = 1024;
+
+struct PwParams {
+    const int8_t* src;
+    const int8_t* wp;  // packed filter [IC/32][OCP][32], 16-byte halves swapped when (oc >> 3) & 1
+    const int32_t* bias;
+    uint32_t* dst;
+    int src_bytes;
+    int P, OHW, OC, OCP;
+    int tiles;         // ceil(P / 32)
+    int groups;        // OC / 64
+    int image_stride;  // bytes
+    int plane_stride;  // bytes
+    int act;
+    float s_src, s_flt, s_dst, c;
+    FastDiv dOHW;
+    RequantTable table;
+};
+
+__device__ __forceinline__ int pw_kernarg_table(int i) {
+    typedef const __attribute__((address_space(4))) char* kptr;
+    const kptr base = (kptr)__builtin_amdgcn_kernarg_segment_ptr();
+    return *(const __attribute__((address_space(4))) int*)(base + offsetof(PwParams, table) + 4 * i);
+}
+
+// KC: 32-channel K chunks (IC = 32 * KC). ACT: IDENTITY / RELU use the table, -1 evaluates the
+// literal sequence with the run-time activation.
+template <int KC, int ACT>
+__global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) {
+    __shared__ int tbl[REQUANT_TABLE_ENTRIES];
+    __shared__ __attribute__((aligned(16))) int bias_lds[PW_MAX_OC];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, kg = lane >> 5;
+    // wave -> (64-channel group, first tile, tile step); the grid holds a multiple of `groups` waves
+    const int gw = blockIdx.x * (PW_THREADS / 64) + wave;
+    const int nw = gridDim.x * (PW_THREADS / 64);
+    const int og = gw % q.groups;
+    // each wave walks a contiguous run of tiles: its loads and stores stream through every
+    // channel plane in address order
+    const int per = (q.tiles + nw / q.groups - 1) / (nw / q.groups);
+    int t = (gw / q.groups) * per;
+    const int tend = min(t + per, q.tiles);
+
+    v4i A[2][KC];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi) {
+        const int oc = og * 64 + mi * 32 + col;
+#pragma unroll
+        for (int c = 0; c < KC; ++c)
+            A[mi][c] = *(const v4i*)(q.wp + ((size_t)c * q.OCP + oc) * KROW + (((kg ^ (oc >> 3)) & 1) << 4));
+    }
+
+    const __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc((void*)q.src, 0, q.src_bytes, 0x00020000);
+    // one tile's B operand; lanes beyond the last pixel (and tiles beyond the wave's run) read
+    // zeros (offset out of range)
+    auto load_tile = [&](int tile, v4i (&B)[KC]) __attribute__((always_inline)) {
+        const int p = tile * 32 + col;
+        const int n = fdiv(p, q.dOHW);
+        const int rem = p - n * q.OHW;
+        const unsigned base =
+                tile < tend && p < q.P ? (unsigned)(n * q.image_stride + rem * 4) : 0x80000000u;
+#pragma unroll
+        for (int c = 0; c < KC; ++c)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                B[c][j] = (int)__builtin_amdgcn_raw_buffer_load_b32(
+                        rs, (int)(base + (unsigned)((c * 8 + kg * 4 + j) * q.plane_stride)), 0, 0);
+    };
+
+    // D tiles in flight per wave: the memory latency is several times the time a tile takes
+    constexpr int D = KC == 1 ? 4 : KC == 2 ? 3 : KC == 4 ? 2 : 1;
+    v4i B[D][KC];
+    static_for<D>([&](auto dc) { load_tile(t + decltype(dc)::value, B[decltype(dc)::value]); });
+
+    // threshold table and bias to LDS while those loads are in flight
+    if (ACT >= 0)
+        tbl[tid] = pw_kernarg_table(tid);
+    for (int i = tid; i < q.OC; i += PW_THREADS)
+        bias_lds[i] = q.bias ? q.bias[i] : 0;
+    __syncthreads();
+    for (; t < tend; t += D) {
+        static_for<D>([&](auto dc) {
+            constexpr int d = decltype(dc)::value;
+            const int tile = t + d;
+            if (tile < tend) {
+                v16i acc[2];
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi) {
+                    // register e of a tile: channel 8 * (e / 4) + 4 * kg + e % 4
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4) {
+                        const v4i bv = *(const v4i*)(bias_lds + og * 64 + mi * 32 + e4 * 8 + kg * 4);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                            acc[mi][e4 * 4 + k] = bv[k];
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < KC; ++c)
+#pragma unroll
+                    for (int mi = 0; mi < 2; ++mi)
+                        acc[mi] = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[mi][c], B[d][c], acc[mi], 0, 0, 0);
+                // this buffer is free again: fetch the tile D ahead
+                load_tile(tile + D, B[d]);
+
+                const int p = tile * 32 + col;
+                const bool ok = p < q.P;
+                const int n = fdiv(p, q.dOHW);
+                const int obase = n * (q.OC >> 2) * q.OHW + (p - n * q.OHW);
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi) {
+                    int r[16];
+                    if (ACT < 0) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e)
+                            r[e] = requant_conv_rt(q.act, acc[mi][e], q.s_src, q.s_flt, q.s_dst);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e)
+                            r[e] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[mi][e], q.c, tbl);
+                    }
+                    if (ok) {
+#pragma unroll
+                        for (int e4 = 0; e4 < 4; ++e4) {
+                            const int oc4 = og * 16 + mi * 8 + e4 * 2 + kg;
+                            q.dst[obase + oc4 * q.OHW] =
+                                    pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
+                        }
+                    }
+                }
+            }
+        });
+    }
+}
+
+static int pw_num_cus() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            n = prop.multiProcessorCount;
+        if (n <= 0)
+            n = 256;
+    }
+    return n;
+}
+
+// workgroups of `kern` one CU holds at a time
+static int pw_resident_blocks(const void* kern) {
+    static std::map<const void*, int> cache;
+    static std::mutex lock;
+    std::lock_guard<std::mutex> guard(lock);
+    auto it = cache.find(kern);
+    if (it != cache.end())
+        return it->second;
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, PW_THREADS, 0) != hipSuccess || n < 1)
+        n = 2;
+    return cache[kern] = n;
+}
+
+bool conv_pw_stream_supported(const ConvGeom& g) {
+    const long P = (long)g.n * g.oh * g.ow;
+    return g.fmt == MEGCC_FMT_NCHW44 && g.groups == 1 && g.fh == 1 && g.fw == 1 && g.sh == 1 &&
+           g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.ic == 32 || g.ic == 64 || g.ic == 128 || g.ic == 256) &&
+           (g.oc & 63) == 0 && g.oc <= PW_MAX_OC && P >= 2048 &&
+           (long)g.n * g.ic * g.ih * g.iw < (1L << 31) && P * g.oc < (1L << 31);
+}
+
+TinyNNStatus conv_pw_stream_launch(
+        const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst) {
+    PwParams q = {};
+    q.src = (const int8_t*)src;
+    q.wp = (const int8_t*)packed;
+    q.bias = (const int32_t*)bias;
+    q.dst = (uint32_t*)dst;
+    q.src_bytes = (int)((long)g.n * g.ic * g.ih * g.iw);
+    q.OHW = g.oh * g.ow;
+    q.P = g.n * q.OHW;
+    q.OC = g.oc;
+    q.OCP = (g.oc + OC_PAD - 1) / OC_PAD * OC_PAD;
+    q.tiles = (q.P + 31) / 32;
+    q.groups = g.oc / 64;
+    q.image_stride = g.ic * q.OHW;
+    q.plane_stride = q.OHW * 4;
+    q.act = g.act;
+    q.s_src = g.s_src;
+    q.s_flt = g.s_flt;
+    q.s_dst = g.s_dst;
+    q.c = make_requant_fast(g.s_src, g.s_flt, g.s_dst).c;
+    q.dOHW = make_fastdiv(q.OHW);
+    const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
+                     requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    if (tab)
+        q.table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
+    const int act = tab ? g.act : -1;
+
+    const void* kern = nullptr;
+#define MG_PW_PICK(KC_)                                                                      \
+    (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_stream_kernel<KC_, MEGCC_NONLINE_IDENTITY> \
+     : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_stream_kernel<KC_, MEGCC_NONLINE_RELU>     \
+                                   : (const void*)conv_pw_stream_kernel<KC_, -1>)
+    switch (g.ic / 32) {
+        case 1: kern = MG_PW_PICK(1); break;
+        case 2: kern = MG_PW_PICK(2); break;
+        case 4: kern = MG_PW_PICK(4); break;
+        default: kern = MG_PW_PICK(8); break;
+    }
+#undef MG_PW_PICK
+
+    // waves: a multiple of `groups`; as many as are resident at once (every wave pays the set-up
+    // once and then streams), fewer when there are not about four tiles for each
+    const long items = (long)q.tiles * q.groups;
+    long waves = items / 4;
+    const long cap = (long)pw_num_cus() * 4 * pw_resident_blocks(kern);
+    if (waves > cap)
+        waves = cap;
+    long gcd = q.groups, rest = 4;  // unit = lcm(groups, waves per workgroup)
+    while (rest) {
+        const long r = gcd % rest;
+        gcd = rest;
+        rest = r;
+    }
+    const long unit = (long)q.groups * 4 / gcd;
+    waves = (waves + unit - 1) / unit * unit;
+    const unsigned blocks = (unsigned)(waves / 4);
+
+    void* args[] = {&q};
+    hipError_t e = hipLaunchKernel(kern, dim3(blocks), dim3(PW_THREADS), args, 0, stream());
+    MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_pw_stream: %s", hipGetErrorString(e));
+    return check_launch("conv_pw_stream");
+}
+
+}  // namespace mg

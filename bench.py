@@ -84,9 +84,11 @@ def make_workload(name):
         case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 64, 512, 14, 14, 512, 1, 1, 0, abi.RELU,
                         scales=(0.02, 0.01, 0.05))
         return case, "qsi8 conv1x1 NCHW44 N=64 C=512 14x14", "mfma"
-    if name in ("pw1", "pw2", "pw3", "pw4", "pw5", "pw6"):  # MobileNetV1 pointwise layers, batch 64
+    if name in ("pw1", "pw2", "pw3", "pw4", "pw5", "pw6", "pw7", "pw12", "pw13"):
+        # MobileNetV1 pointwise layers, batch 64
         ic, oc, hw = {"pw1": (32, 64, 112), "pw2": (64, 128, 56), "pw3": (128, 128, 56),
-                      "pw4": (128, 256, 28), "pw5": (256, 256, 28), "pw6": (256, 512, 14)}[name]
+                      "pw4": (128, 256, 28), "pw5": (256, 256, 28), "pw6": (256, 512, 14),
+                      "pw7": (512, 512, 14), "pw12": (512, 1024, 7), "pw13": (1024, 1024, 7)}[name]
         case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 64, ic, hw, hw, oc, 1, 1, 0, abi.RELU,
                         scales=(0.02, 0.01, 0.05))
         return case, "qsi8 conv1x1 NCHW44 N=64 %d->%d %dx%d" % (ic, oc, hw, hw), "hbm"

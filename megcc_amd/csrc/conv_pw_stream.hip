@@ -1,11 +1,12 @@
 // qsi8 pointwise (1x1, stride 1) NCHW44 convolution with few input channels: a streaming kernel.
 //
-// With K = IC <= 256 a pointwise layer does one to eight MFMAs per 32 x 32 output tile and then
+// With K = IC <= 512 a pointwise layer does one to sixteen MFMAs per 32 x 32 output tile and then
 // requantises 16 outputs per lane: the layer is bound by HBM and by the epilogue's vector
 // instructions, not by the matrix cores, and any staging through LDS (barriers, stage buffers,
 // one workgroup per CU) only adds latency. So nothing is staged:
-//   * a wave owns 64 output channels and keeps their filter rows in registers for its whole life
-//     (2 MFMA row tiles x IC/32 K-chunks x 4 VGPRs, read once from the packed filter);
+//   * a wave owns 64 output channels (32 with 512 input channels) and keeps their filter rows in
+//     registers for its whole life (MFMA row tiles x IC/32 K-chunks x 4 VGPRs, read once from the
+//     packed filter);
 //   * it walks over 32-pixel tiles; the MFMA B operand of a tile is exactly what NCHW44 holds per
 //     lane - lane (pixel l & 31, K-half l >> 5) needs 16 consecutive channels = one dword from
 //     each of 4 consecutive channel planes - so it is loaded straight from global memory, 128
@@ -36,7 +37,7 @@ struct PwParams {
     int src_bytes;
     int P, OHW, OC, OCP;
     int tiles;         // ceil(P / 32)
-    int groups;        // OC / 64
+    int groups;        // OC / channels per wave
     int image_stride;  // bytes
     int plane_stride;  // bytes
     int act;
@@ -53,7 +54,8 @@ __device__ __forceinline__ int pw_kernarg_table(int i) {
 
 // KC: 32-channel K chunks (IC = 32 * KC). ACT: IDENTITY / RELU use the table, -1 evaluates the
 // literal sequence with the run-time activation.
-template <int KC, int ACT>
+// MT: 32-channel MFMA row tiles per wave (a wave owns 32 * MT output channels).
+template <int KC, int MT, int ACT>
 __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) {
     __shared__ int tbl[REQUANT_TABLE_ENTRIES];
     __shared__ __attribute__((aligned(16))) int bias_lds[PW_MAX_OC];
@@ -69,10 +71,10 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
     int t = (gw / q.groups) * per;
     const int tend = min(t + per, q.tiles);
 
-    v4i A[2][KC];
+    v4i A[MT][KC];
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi) {
-        const int oc = og * 64 + mi * 32 + col;
+    for (int mi = 0; mi < MT; ++mi) {
+        const int oc = og * (32 * MT) + mi * 32 + col;
 #pragma unroll
         for (int c = 0; c < KC; ++c)
             A[mi][c] = *(const v4i*)(q.wp + ((size_t)c * q.OCP + oc) * KROW + (((kg ^ (oc >> 3)) & 1) << 4));
@@ -80,26 +82,37 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
 
     const __amdgpu_buffer_rsrc_t rs =
             __builtin_amdgcn_make_buffer_rsrc((void*)q.src, 0, q.src_bytes, 0x00020000);
-    // one tile's B operand; lanes beyond the last pixel (and tiles beyond the wave's run) read
-    // zeros (offset out of range)
-    auto load_tile = [&](int tile, v4i (&B)[KC]) __attribute__((always_inline)) {
+    // ---- B operand: a ring of RING 32-channel chunks in flight per wave ------------------------
+    // The memory latency is several times the time a tile takes, so chunks are requested RING
+    // positions ahead of their MFMA in the sequence (tile, chunk) -> tile * KC + chunk: four tiles
+    // ahead with 32 input channels, half a tile with 512. The loop is unrolled over U tiles so that
+    // every ring slot and every "which tile, which chunk" below is a compile-time constant.
+    constexpr int RING = KC == 1 ? 4 : KC == 2 ? 6 : 8;
+    constexpr int U = RING > KC ? RING / KC : 1;           // tiles per unrolled step
+    constexpr int AHEAD = (RING + KC - 1) / KC;            // tiles a request can be ahead
+    static_assert(RING % KC == 0 || KC % RING == 0, "slots repeat every U tiles");
+    static_assert(4 * (KC * MT + RING) <= 192, "filter rows and chunks in flight must fit the registers");
+    // byte offset of a tile's pixel in plane 0, or out of range (reads as zero) beyond the
+    // wave's run / the last pixel
+    auto tile_base = [&](int tile) __attribute__((always_inline)) -> unsigned {
         const int p = tile * 32 + col;
         const int n = fdiv(p, q.dOHW);
-        const int rem = p - n * q.OHW;
-        const unsigned base =
-                tile < tend && p < q.P ? (unsigned)(n * q.image_stride + rem * 4) : 0x80000000u;
+        return tile < tend && p < q.P
+                       ? (unsigned)(n * q.image_stride + (p - n * q.OHW) * 4 + kg * 4 * q.plane_stride)
+                       : 0x80000000u;
+    };
+    auto load_chunk = [&](unsigned base, int c, v4i& dst) __attribute__((always_inline)) {
 #pragma unroll
-        for (int c = 0; c < KC; ++c)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                B[c][j] = (int)__builtin_amdgcn_raw_buffer_load_b32(
-                        rs, (int)(base + (unsigned)((c * 8 + kg * 4 + j) * q.plane_stride)), 0, 0);
+        for (int j = 0; j < 4; ++j)
+            dst[j] = (int)__builtin_amdgcn_raw_buffer_load_b32(
+                    rs, (int)(base + (unsigned)((c * 8 + j) * q.plane_stride)), 0, 0);
     };
 
-    // D tiles in flight per wave: the memory latency is several times the time a tile takes
-    constexpr int D = KC == 1 ? 4 : KC == 2 ? 3 : KC == 4 ? 2 : 1;
-    v4i B[D][KC];
-    static_for<D>([&](auto dc) { load_tile(t + decltype(dc)::value, B[decltype(dc)::value]); });
+    v4i ring[RING];
+    static_for<RING>([&](auto sc) {
+        constexpr int s = decltype(sc)::value;
+        load_chunk(tile_base(t + s / KC), s % KC, ring[s]);
+    });
 
     // threshold table and bias to LDS while those loads are in flight
     if (ACT >= 0)
@@ -107,37 +120,45 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
     for (int i = tid; i < q.OC; i += PW_THREADS)
         bias_lds[i] = q.bias ? q.bias[i] : 0;
     __syncthreads();
-    for (; t < tend; t += D) {
-        static_for<D>([&](auto dc) {
-            constexpr int d = decltype(dc)::value;
-            const int tile = t + d;
+
+    for (; t < tend; t += U) {
+        unsigned base[U + AHEAD];  // of tiles t, t + 1, ...: the targets of this step's requests
+        static_for<U + AHEAD>([&](auto kc) {
+            constexpr int k = decltype(kc)::value;
+            base[k] = tile_base(t + k);
+        });
+        static_for<U>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            const int tile = t + u;
             if (tile < tend) {
-                v16i acc[2];
+                v16i acc[MT];
 #pragma unroll
-                for (int mi = 0; mi < 2; ++mi) {
+                for (int mi = 0; mi < MT; ++mi) {
                     // register e of a tile: channel 8 * (e / 4) + 4 * kg + e % 4
 #pragma unroll
                     for (int e4 = 0; e4 < 4; ++e4) {
-                        const v4i bv = *(const v4i*)(bias_lds + og * 64 + mi * 32 + e4 * 8 + kg * 4);
+                        const v4i bv = *(const v4i*)(bias_lds + og * (32 * MT) + mi * 32 + e4 * 8 + kg * 4);
 #pragma unroll
                         for (int k = 0; k < 4; ++k)
                             acc[mi][e4 * 4 + k] = bv[k];
                     }
                 }
+                static_for<KC>([&](auto cc) {
+                    constexpr int c = decltype(cc)::value;
+                    constexpr int s = u * KC + c, slot = s % RING;
 #pragma unroll
-                for (int c = 0; c < KC; ++c)
-#pragma unroll
-                    for (int mi = 0; mi < 2; ++mi)
-                        acc[mi] = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[mi][c], B[d][c], acc[mi], 0, 0, 0);
-                // this buffer is free again: fetch the tile D ahead
-                load_tile(tile + D, B[d]);
+                    for (int mi = 0; mi < MT; ++mi)
+                        acc[mi] = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[mi][c], ring[slot], acc[mi], 0, 0, 0);
+                    // the slot is free again: request the chunk RING positions ahead
+                    load_chunk(base[(s + RING) / KC], (s + RING) % KC, ring[slot]);
+                });
 
                 const int p = tile * 32 + col;
                 const bool ok = p < q.P;
                 const int n = fdiv(p, q.dOHW);
                 const int obase = n * (q.OC >> 2) * q.OHW + (p - n * q.OHW);
 #pragma unroll
-                for (int mi = 0; mi < 2; ++mi) {
+                for (int mi = 0; mi < MT; ++mi) {
                     int r[16];
                     if (ACT < 0) {
 #pragma unroll
@@ -151,7 +172,7 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
                     if (ok) {
 #pragma unroll
                         for (int e4 = 0; e4 < 4; ++e4) {
-                            const int oc4 = og * 16 + mi * 8 + e4 * 2 + kg;
+                            const int oc4 = og * (8 * MT) + mi * 8 + e4 * 2 + kg;
                             q.dst[obase + oc4 * q.OHW] =
                                     pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
                         }
@@ -192,7 +213,7 @@ static int pw_resident_blocks(const void* kern) {
 bool conv_pw_stream_supported(const ConvGeom& g) {
     const long P = (long)g.n * g.oh * g.ow;
     return g.fmt == MEGCC_FMT_NCHW44 && g.groups == 1 && g.fh == 1 && g.fw == 1 && g.sh == 1 &&
-           g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.ic == 32 || g.ic == 64 || g.ic == 128 || g.ic == 256) &&
+           g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.ic == 32 || g.ic == 64 || g.ic == 128 || g.ic == 256 || g.ic == 512) &&
            (g.oc & 63) == 0 && g.oc <= PW_MAX_OC && P >= 2048 &&
            (long)g.n * g.ic * g.ih * g.iw < (1L << 31) && P * g.oc < (1L << 31);
 }
@@ -210,7 +231,7 @@ TinyNNStatus conv_pw_stream_launch(
     q.OC = g.oc;
     q.OCP = (g.oc + OC_PAD - 1) / OC_PAD * OC_PAD;
     q.tiles = (q.P + 31) / 32;
-    q.groups = g.oc / 64;
+    q.groups = g.oc / (g.ic > 256 ? 32 : 64);
     q.image_stride = g.ic * q.OHW;
     q.plane_stride = q.OHW * 4;
     q.act = g.act;
@@ -226,15 +247,16 @@ TinyNNStatus conv_pw_stream_launch(
     const int act = tab ? g.act : -1;
 
     const void* kern = nullptr;
-#define MG_PW_PICK(KC_)                                                                      \
-    (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_stream_kernel<KC_, MEGCC_NONLINE_IDENTITY> \
-     : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_stream_kernel<KC_, MEGCC_NONLINE_RELU>     \
-                                   : (const void*)conv_pw_stream_kernel<KC_, -1>)
+#define MG_PW_PICK(KC_, MT_)                                                                      \
+    (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_IDENTITY> \
+     : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_RELU>     \
+                                   : (const void*)conv_pw_stream_kernel<KC_, MT_, -1>)
     switch (g.ic / 32) {
-        case 1: kern = MG_PW_PICK(1); break;
-        case 2: kern = MG_PW_PICK(2); break;
-        case 4: kern = MG_PW_PICK(4); break;
-        default: kern = MG_PW_PICK(8); break;
+        case 1: kern = MG_PW_PICK(1, 2); break;
+        case 2: kern = MG_PW_PICK(2, 2); break;
+        case 4: kern = MG_PW_PICK(4, 2); break;
+        case 8: kern = MG_PW_PICK(8, 2); break;
+        default: kern = MG_PW_PICK(16, 1); break;  // 512 input channels: 32 output channels per wave
     }
 #undef MG_PW_PICK
 

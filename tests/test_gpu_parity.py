@@ -116,6 +116,9 @@ LIVE = [
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
     PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE, 5, 1024, 7, 7, 7, 7, 0),
     PoolCase(A.FMT_NCHW, A.POOL_AVERAGE, 5, 1024, 7, 7, 7, 7, 0),
+    PoolCase(A.FMT_NCHW44, A.POOL_MAX, 3, 64, 13, 13, 13, 13, 0),  # one output pixel per plane
+    PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE_COUNT_EXCLUDE_PADDING, 3, 64, 13, 13, 13, 13, 0),
+    PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE, 2, 8, 4, 4, 4, 4, 0),
     MultiTypeCase(A.Q_FUSE_ADD_RELU, (2, 32, 56, 56), (0.05, 0.01, 0.05)),
     MultiTypeCase(A.Q_ADD, (3, 7, 13, 5), (0.031, 0.017, 0.023)),
     MultiTypeCase(A.Q_MUL, (2, 32, 56, 56), (0.05, 0.04, 0.3)),

@@ -27,9 +27,13 @@ typedef int cf_v4i __attribute__((ext_vector_type(4)));
 template <int ACT>
 __global__ void __launch_bounds__(CF_THREADS) conv_first_q8_kernel(
         ConvGeom g, RequantFast rq, const int8_t* __restrict__ src, const int8_t* __restrict__ flt,
-        const int32_t* __restrict__ bias, uint32_t* __restrict__ dst, int total_pairs) {
+        const int32_t* __restrict__ bias, uint32_t* __restrict__ dst, int total_pairs,
+        RequantTable table) {
     __shared__ __attribute__((aligned(16))) int wlds[CF_MAX_OC * 9];
     __shared__ __attribute__((aligned(16))) int blds[CF_MAX_OC];
+    __shared__ int tbl[REQUANT_TABLE_ENTRIES];
+    if (ACT >= 0)
+        tbl[threadIdx.x] = table.t[threadIdx.x];
     const int oc4n = g.oc >> 2;
     // packed weight dword (g4, row = ic*3 + fh, o): bytes fw = 0, 1, 2 and a zero
     for (int i = threadIdx.x; i < g.oc * 9; i += CF_THREADS) {
@@ -93,8 +97,8 @@ __global__ void __launch_bounds__(CF_THREADS) conv_first_q8_kernel(
                     ra[o] = requant_conv_rt(g.act, a[o], g.s_src, g.s_flt, g.s_dst);
                     rb[o] = requant_conv_rt(g.act, b[o], g.s_src, g.s_flt, g.s_dst);
                 } else {
-                    ra[o] = requant_conv_fast<(ACT < 0 ? 0 : ACT)>(a[o], rq);
-                    rb[o] = requant_conv_fast<(ACT < 0 ? 0 : ACT)>(b[o], rq);
+                    ra[o] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(a[o], rq.c, tbl);
+                    rb[o] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(b[o], rq.c, tbl);
                 }
             }
             uint2 v;
@@ -122,12 +126,18 @@ TinyNNStatus conv_first_launch(
     if (blocks > 256 * 16)
         blocks = 256 * 16;
     const RequantFast rq = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
-    auto kern = g.act == MEGCC_NONLINE_IDENTITY ? conv_first_q8_kernel<MEGCC_NONLINE_IDENTITY>
-              : g.act == MEGCC_NONLINE_RELU     ? conv_first_q8_kernel<MEGCC_NONLINE_RELU>
-                                                : conv_first_q8_kernel<-1>;
+    // exact thresholds for the monotone activations; anything else (and extreme scales)
+    // evaluates the literal sequence per output
+    const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
+                     requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    static const RequantTable no_table = {};
+    const RequantTable& table = tab ? requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst) : no_table;
+    auto kern = tab && g.act == MEGCC_NONLINE_IDENTITY ? conv_first_q8_kernel<MEGCC_NONLINE_IDENTITY>
+              : tab && g.act == MEGCC_NONLINE_RELU     ? conv_first_q8_kernel<MEGCC_NONLINE_RELU>
+                                                       : conv_first_q8_kernel<-1>;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(CF_THREADS), 0, stream(), g, rq,
                        (const int8_t*)src, (const int8_t*)flt, (const int32_t*)bias, (uint32_t*)dst,
-                       (int)pairs);
+                       (int)pairs, table);
     return check_launch("conv_first_q8");
 }
 

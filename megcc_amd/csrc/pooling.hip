@@ -66,44 +66,43 @@ __global__ void __launch_bounds__(256) pool44_q8_kernel(
 }
 
 // NCHW44, one output pixel per plane (global pooling, e.g. the 7x7 average in front of a
-// classifier): one wave per plane group instead of one thread, so that the plane is read by 64
-// lanes at once; integer max / sum are combined across the wave, the last step is the same
-// expression as above.
+// classifier): 8 lanes per plane group instead of one thread, so that a wave reads 8 consecutive
+// planes as one contiguous stretch; integer max / sum are combined across the 8 lanes, the last
+// step is the same expression as above.
 __global__ void __launch_bounds__(256) pool44_global_q8_kernel(
         PoolGeom g, const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, int planes) {
-    const int lane = threadIdx.x & 63;
+    const int sub = threadIdx.x & 7;
     const int hw = g.ih * g.iw;
-    for (int pl = blockIdx.x * 4 + (threadIdx.x >> 6); pl < planes; pl += gridDim.x * 4) {
+    const bool is_max = g.mode == MEGCC_POOL_MAX;
+    for (int pl = (blockIdx.x * 256 + threadIdx.x) >> 3; pl < planes; pl += gridDim.x * 32) {
         const uint32_t* plane = src + (size_t)pl * hw;
-        int mx[4] = {-128, -128, -128, -128};
-        int sum[4] = {0, 0, 0, 0};
-        for (int i = lane; i < hw; i += 64) {
+        int v4[4] = {is_max ? -128 : 0, is_max ? -128 : 0, is_max ? -128 : 0, is_max ? -128 : 0};
+        for (int i = sub; i < hw; i += 8) {
             const uint32_t v = plane[i];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const int b = sbyte(v, c);
-                mx[c] = max(mx[c], b);
-                sum[c] += b;
+                v4[c] = is_max ? max(v4[c], b) : v4[c] + b;
             }
         }
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
+        for (int off = 4; off > 0; off >>= 1) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                mx[c] = max(mx[c], __shfl_xor(mx[c], off, 64));
-                sum[c] += __shfl_xor(sum[c], off, 64);
+                const int o = __shfl_xor(v4[c], off, 64);
+                v4[c] = is_max ? max(v4[c], o) : v4[c] + o;
             }
         }
-        if (lane == 0) {
+        if (sub == 0) {
             int o[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                if (g.mode == MEGCC_POOL_MAX)
-                    o[c] = mx[c];
+                if (is_max)
+                    o[c] = v4[c];
                 else if (g.mode == MEGCC_POOL_AVERAGE)
-                    o[c] = fp32_to_int8((float)sum[c] * g.count_div);
+                    o[c] = fp32_to_int8((float)v4[c] * g.count_div);
                 else
-                    o[c] = fp32_to_int8((float)sum[c] * (float)(1.0 / (double)(uint32_t)hw));
+                    o[c] = fp32_to_int8((float)v4[c] * (float)(1.0 / (double)(uint32_t)hw));
             }
             dst[pl] = pack4(o[0], o[1], o[2], o[3]);
         }
@@ -197,7 +196,7 @@ extern "C" TinyNNStatus megcc_gfx950_pooling(
         const long planes = (long)g.n * (g.c / 4);
         if (g.oh == 1 && g.ow == 1 && g.ph == 0 && g.pw == 0 && g.wh == g.ih && g.ww == g.iw &&
             g.ih * g.iw >= 16 && planes < (1L << 30)) {
-            unsigned blocks = min(ceil_div((size_t)planes, 4), 1u << 16);
+            unsigned blocks = min(ceil_div((size_t)planes, 32), 1u << 16);
             hipLaunchKernelGGL(pool44_global_q8_kernel, dim3(blocks), dim3(256), 0, stream(), g,
                                (const uint32_t*)src->ptr, (uint32_t*)dst->ptr, (int)planes);
             return check_launch("pooling");

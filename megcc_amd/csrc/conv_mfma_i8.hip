@@ -481,7 +481,7 @@ TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed) {
 
 bool conv_mfma_pipe_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
 bool conv_mfma_ws_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
-bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, PipeConfig* c);
+bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok, PipeConfig* c);
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
 
 bool conv_pw_stream_supported(const ConvGeom& g);
@@ -497,6 +497,7 @@ TinyNNStatus conv_mfma_launch(
     MfmaParams q = {};
     PipeConfig pc;
     const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;
+    const bool b128_ok = ((uintptr_t)src & 15) == 0 && !getenv("MEGCC_NOFCB");
     // candidates in order of preference; development switches MEGCC_NODMA / MEGCC_NOWS /
     // MEGCC_NOWIDE skip one
     long range_len = 0;
@@ -506,9 +507,9 @@ TinyNNStatus conv_mfma_launch(
         bool have = false;
         if (cand == -1)
             have = !getenv("MEGCC_NODMA") && !getenv("MEGCC_NODMA512") &&
-                   conv_mfma_dma_config(g, is_fc(g), 0, &pc);
+                   conv_mfma_dma_config(g, is_fc(g), 0, b128_ok, &pc);
         else if (cand == 0)
-            have = !getenv("MEGCC_NODMA") && conv_mfma_dma_config(g, is_fc(g), 1, &pc);
+            have = !getenv("MEGCC_NODMA") && conv_mfma_dma_config(g, is_fc(g), 1, b128_ok, &pc);
         else if (cand == 1)
             have = !getenv("MEGCC_NOWS") && conv_mfma_ws_config(g, g4_ok, &pc);
         else

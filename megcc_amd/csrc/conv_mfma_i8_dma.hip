@@ -39,8 +39,15 @@ static constexpr int ACT_RT = -1;
 // NT: 32-pixel MFMA tiles per wave along pixels; the workgroup sub-tile is 128 * NT pixels. NT = 4
 // reads 0.75 KB of LDS per MFMA instead of 1 KB (the 2 x 2 wave tile keeps the LDS port as busy as
 // the matrix core).
-template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT>
+// FCB: FullyConnected with K a multiple of 128 and a 16-byte aligned source: the rows of the
+// activation matrix are contiguous in K, so the B tile comes in with 16-byte loads as well - a
+// wave-load is 8 rows x 128 bytes = 8 full cache lines. LDS then holds a pixel's 128 bytes of a
+// stage together; the eight 16-byte pieces of a row are stored at piece ^ (row & 7) (the load
+// fetches the matching piece), which keeps the MFMA operand reads of 8 consecutive rows on
+// different banks.
+template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT, bool FCB>
 __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaParams q) {
+    static_assert(!FCB || (FC && KS == 4 && FH * FW == 1), "FCB: FullyConnected, 128 channels per stage");
     constexpr int WGN = 4;
     constexpr int DM_BNP = 32 * NT * WGN;
     constexpr int DM_WAVES = WGM * WGN, DM_THREADS = 64 * DM_WAVES;
@@ -51,8 +58,9 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     constexpr int A_CHUNKS = A_BYTES / 1024;
     constexpr int A_PER_WAVE = (A_CHUNKS + DM_WAVES - 1) / DM_WAVES;
     constexpr int B_BYTES = KS * 2 * LMAX * 16;
-    constexpr int B_WL = B_BYTES / 256;
+    constexpr int B_WL = B_BYTES / (FCB ? 1024 : 256);
     static_assert(B_WL % DM_WAVES == 0 && LMAX % 16 == 0, "whole wave-loads");
+    static_assert(!FCB || LMAX == 32 * NT * 4, "FCB: one LDS row per pixel of the sub-tile");
     constexpr int B_PER_WAVE = B_WL / DM_WAVES;
     constexpr int LW = LMAX / 16;  // wave-loads per (sub-chunk, half)
     constexpr int N_DMA = A_PER_WAVE + B_PER_WAVE;
@@ -99,6 +107,17 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     // dword in the first plane group of a stage, or 2^31 (out of range -> zero) for padding.
     unsigned b_goff[B_PER_WAVE];
     auto describe = [&](int p0) __attribute__((always_inline)) {
+        if constexpr (FCB) {
+            // wave-load u covers rows 8u .. 8u + 7; rows beyond the matrix repeat the last one
+            // (their columns of the product are never stored)
+            static_for<B_PER_WAVE>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                const int u = wave + j * DM_WAVES;
+                const int row = min(p0 + u * 8 + (lane >> 3), q.P - 1);
+                b_goff[j] = (unsigned)row * (unsigned)q.image_stride + (((lane & 7) ^ (lane >> 3)) << 4);
+            });
+            return;
+        }
         const int plast = min(p0 + DM_BNP, range1) - 1;
         const int vp0 = vp_of(q, p0);
         const int L = vp_of(q, plast) + ((FH - 1) * q.DH) * q.VW + (FW - 1) * q.DW - vp0 + 1;
@@ -132,7 +151,10 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
         static_for<B_PER_WAVE>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             const int u = wave + j * DM_WAVES;
-            dma_buffer_b32(src_rsrc, b_goff[j] + poff, lds_address(buf + A_BYTES + u * 256));
+            if constexpr (FCB)
+                dma_global_b128(q.src + (b_goff[j] + poff), lds_address(buf + A_BYTES + u * 1024));
+            else
+                dma_buffer_b32(src_rsrc, b_goff[j] + poff, lds_address(buf + A_BYTES + u * 256));
         });
         if (++lst == stages) {
             lst = 0;
@@ -230,7 +252,10 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             // all of them busy
             const int pc = p0 + (ni * WGN + wn) * 32;
             const int p = pc + (lane & 31);
-            b_byte[ni] = (kg * LMAX + (p <= plast ? vp_of(q, p) - vp0 : 0)) * 16;
+            if constexpr (FCB)
+                b_byte[ni] = p - p0;  // LDS row of this lane's pixel
+            else
+                b_byte[ni] = (kg * LMAX + (p <= plast ? vp_of(q, p) - vp0 : 0)) * 16;
             cols += pc <= plast ? 1 : 0;
             const int pn = (int)fdiv(p, q.dOHW);
             cur_o[ni] = pc > plast ? -2
@@ -269,9 +294,14 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
                     for (int mi = 0; mi < MT; ++mi)
                         fa[t & 1][mi] = *(const v4i*)(bufA + t * (DM_BM * KROW) + a_off[mi]);
 #pragma unroll
-                    for (int ni = 0; ni < COLS; ++ni)
-                        fb[t & 1][ni] = *(const v4i*)(bufB + ks * (2 * LMAX * 16) + b_byte[ni] +
-                                                      tap_off * 16);
+                    for (int ni = 0; ni < COLS; ++ni) {
+                        if constexpr (FCB)
+                            fb[t & 1][ni] = *(const v4i*)(bufB + b_byte[ni] * 128 +
+                                                          (((ks * 2 + kg) ^ (b_byte[ni] & 7)) << 4));
+                        else
+                            fb[t & 1][ni] = *(const v4i*)(bufB + ks * (2 * LMAX * 16) + b_byte[ni] +
+                                                          tap_off * 16);
+                    }
                 };
                 fetch(std::integral_constant<int, 0>{});
                 static_for<TS>([&](auto tc) {
@@ -314,7 +344,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
 }
 
 // ---- configurations --------------------------------------------------------------------------
-template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3, int WGM = 2, int BPC = 1, int NT = 2>
+template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3, int WGM = 2, int BPC = 1, int NT = 2, bool FCB = false>
 static PipeConfig make_dma_config(int act, bool table_ok) {
     constexpr int DM_BM = 32 * MT * WGM;
     PipeConfig c;
@@ -331,11 +361,11 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.fixed_lmax = LMAX;
     c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + 128 * 4;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC, NT>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC, NT, FCB>;
     else if (act == MEGCC_NONLINE_RELU && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF, WGM, BPC, NT>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF, WGM, BPC, NT, FCB>;
     else
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT, FCB>;
     return c;
 }
 
@@ -343,7 +373,7 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
 // with 32 input channels) and enough pixels. 1x1: 128 input channels per stage (64 / 32 when
 // IC <= 64 / 32).
 // variant 0: 512-pixel sub-tiles (3x3 only, two stage buffers); variant 1: 256-pixel sub-tiles.
-bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, PipeConfig* c) {
+bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok, PipeConfig* c) {
     const long P = (long)g.n * g.oh * g.ow;
     const bool k3 = g.fh == 3 && g.fw == 3, k1 = g.fh == 1 && g.fw == 1;
     if (!(k3 || k1) || !(g.fmt == MEGCC_FMT_NCHW44 || fc) || g.oc < 64 || P < 2048)
@@ -363,6 +393,8 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, PipeConfig* c
     }
     if (k3)
         *c = make_dma_config<3, 3, 1, 512, false>(g.act, ok);
+    else if (fc && (g.ic & 127) == 0 && b128_ok)
+        *c = make_dma_config<1, 1, 4, 256, true, 2, 3, 2, 1, 2, true>(g.act, ok);
     else if (fc)
         *c = make_dma_config<1, 1, 4, 256, true>(g.act, ok);
     else if (g.oc < 128)

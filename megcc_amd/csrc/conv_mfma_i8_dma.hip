@@ -359,7 +359,7 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.blocks_per_cu = BPC;
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     c.fixed_lmax = LMAX;
-    c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + 128 * 4;
+    c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + (DM_BM > 128 ? DM_BM : 128) * 4;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
         c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC, NT, FCB>;
     else if (act == MEGCC_NONLINE_RELU && table_ok)
@@ -393,6 +393,10 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok,
     }
     if (k3)
         *c = make_dma_config<3, 3, 1, 512, false>(g.act, ok);
+    else if (fc && (g.ic & 127) == 0 && b128_ok && g.oc >= 256)
+        // 256 x 256 tile, each wave 128 oc x 64 rows (4 x 2 MFMA tiles: 0.75 KB of LDS per MFMA;
+        // measured 86 us on 4096^3 against 105 us with the 128 x 256 tile)
+        *c = make_dma_config<1, 1, 4, 256, true, 4, 2, 2, 1, 2, true>(g.act, ok);
     else if (fc && (g.ic & 127) == 0 && b128_ok)
         *c = make_dma_config<1, 1, 4, 256, true, 2, 3, 2, 1, 2, true>(g.act, ok);
     else if (fc)

@@ -99,6 +99,7 @@ LIVE = [
     # FullyConnected with K % 128 == 0: 16-byte activation loads, swizzled LDS rows, ragged M and N
     ConvCase(A.FMT_NCHW, A.DENSE, 2500, 384, 1, 1, 200, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(384) / 2)),
     ConvCase(A.FMT_NCHW, A.DENSE, 4099, 256, 1, 1, 131, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(256) / 2)),
+    ConvCase(A.FMT_NCHW, A.DENSE, 2600, 256, 1, 1, 300, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(256) / 2)),  # 256-row tiles
     # depthwise, pooling, elemwise chain of the bandwidth-bound config
     ConvCase(A.FMT_NCHW44, A.GROUP, 2, 32, 112, 112, 32, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW44, A.GROUP, 2, 32, 112, 112, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, 0.05)),

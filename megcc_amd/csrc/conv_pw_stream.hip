@@ -214,7 +214,7 @@ bool conv_pw_stream_supported(const ConvGeom& g) {
     const long P = (long)g.n * g.oh * g.ow;
     return g.fmt == MEGCC_FMT_NCHW44 && g.groups == 1 && g.fh == 1 && g.fw == 1 && g.sh == 1 &&
            g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.ic == 32 || g.ic == 64 || g.ic == 128 || g.ic == 256 || g.ic == 512) &&
-           (g.oc & 63) == 0 && g.oc <= PW_MAX_OC && P >= 2048 &&
+           (g.oc & 63) == 0 && g.oc <= PW_MAX_OC && P >= 32 &&
            (long)g.n * g.ic * g.ih * g.iw < (1L << 31) && P * g.oc < (1L << 31);
 }
 

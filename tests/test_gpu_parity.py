@@ -96,6 +96,10 @@ LIVE = [
     ConvCase(A.FMT_NCHW, A.DENSE, 64, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(1024) / 2)),
     ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, 0.1)),
     ConvCase(A.FMT_NCHW, A.DENSE, 200, 512, 1, 1, 333, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(512) / 2)),
+    # small pointwise layers on the streaming kernel: fewer pixels than one tile per wave, ragged tile
+    ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 7, 7, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(256))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 64, 5, 9, 192, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(64))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 512, 14, 14, 64, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(512))),
     # FullyConnected with K % 128 == 0: 16-byte activation loads, swizzled LDS rows, ragged M and N
     ConvCase(A.FMT_NCHW, A.DENSE, 2500, 384, 1, 1, 200, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(384) / 2)),
     ConvCase(A.FMT_NCHW, A.DENSE, 4099, 256, 1, 1, 131, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(256) / 2)),

@@ -267,6 +267,7 @@ __global__ void __launch_bounds__(256) conv_mfma_reduce_kernel(MfmaParams q) {
     for (size_t i = blockIdx.x * (size_t)256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
         const int p = (int)(i / oc4n), oc = (int)(i - (size_t)p * oc4n) * 4;
         int a[4] = {0, 0, 0, 0};
+#pragma unroll 8
         for (int z = 0; z < q.split; ++z) {
             const int4 v = *(const int4*)(q.partial + ((size_t)z * q.P + p) * ocs + oc);
             a[0] += v.x; a[1] += v.y; a[2] += v.z; a[3] += v.w;
@@ -484,6 +485,9 @@ bool conv_mfma_ws_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
 bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok, PipeConfig* c);
 TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
 
+int fc_stream_split(const ConvGeom& g, const void* src, size_t ws_bytes, int max_split);
+TinyNNStatus fc_stream_launch(
+        const ConvGeom& g, const void* src, const void* packed, int32_t* partial, int split);
 bool conv_pw_stream_supported(const ConvGeom& g);
 TinyNNStatus conv_pw_stream_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst);
@@ -609,6 +613,23 @@ TinyNNStatus conv_mfma_launch(
     if (pipe)
         return conv_mfma_pipe_launch(pc, q);
     const int split = conv_mfma_split(g);
+    // FullyConnected with few rows: stream the weights (fc_stream.hip), finish with the reduce
+    // kernel below
+    if (fc && split > 1 && ws && ws->ptr && ((uintptr_t)ws->ptr & 15) == 0 && !getenv("MEGCC_NOFCS")) {
+        const int fs = fc_stream_split(g, src, ws->size, split);
+        if (fs > 0) {
+            TinyNNStatus st = fc_stream_launch(g, src, packed, (int32_t*)ws->ptr, fs);
+            if (st != TinyNN_SUCCESS)
+                return st;
+            q.split = fs;
+            q.partial = (int32_t*)ws->ptr;
+            const size_t total = (size_t)q.P * ((q.OC + 3) / 4);
+            unsigned blocks = (unsigned)((total + 255) / 256);
+            hipLaunchKernelGGL(conv_mfma_reduce_kernel, dim3(blocks > 4096 ? 4096 : blocks), dim3(256),
+                               0, stream(), q);
+            return check_launch("conv_mfma_reduce");
+        }
+    }
     if (split > 1 && ws && ws->ptr && ws->size >= conv_mfma_workspace_bytes(g) &&
         ((uintptr_t)ws->ptr & 15) == 0) {
         q.split = split;

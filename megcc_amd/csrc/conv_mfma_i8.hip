@@ -136,7 +136,8 @@ __global__ void __launch_bounds__(THREADS) conv_mfma_i8_kernel(MfmaParams q) {
     };
 
     const int st_begin = blockIdx.z * q.sps, st_end = min(q.stages, st_begin + q.sps);
-    prefetch(st_begin);
+    if (st_begin < st_end)
+        prefetch(st_begin);
     for (int st = st_begin; st < st_end; ++st) {
         __syncthreads();
 #pragma unroll
@@ -632,8 +633,11 @@ TinyNNStatus conv_mfma_launch(
     }
     if (split > 1 && ws && ws->ptr && ws->size >= conv_mfma_workspace_bytes(g) &&
         ((uintptr_t)ws->ptr & 15) == 0) {
-        q.split = split;
+        // equal slices of whole stages; no slice may start at or beyond the last stage (it would
+        // fetch filter rows past the packed buffer), so the slice count follows from the slice
+        // length: 8 stages asked in 6 slices are 4 slices of 2
         q.sps = (q.stages + split - 1) / split;
+        q.split = (q.stages + q.sps - 1) / q.sps;
         q.partial = (int32_t*)ws->ptr;
     }
 

@@ -378,8 +378,8 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok,
     const bool k3 = g.fh == 3 && g.fw == 3, k1 = g.fh == 1 && g.fw == 1;
     if (!(k3 || k1) || !(g.fmt == MEGCC_FMT_NCHW44 || fc) || g.oc < 64 || P < 2048)
         return false;
-    if (g.oc < 128 && !(k1 && !fc && g.ic <= 32))
-        return false;  // 64-channel tiles: only the bandwidth-bound 1x1 with 32 input channels
+    if (g.oc < 128 && !(k1 && !fc && g.ic <= 32) && !k3)
+        return false;  // 64-channel tiles: 3x3 layers and the 1x1 with 32 input channels
     if ((long)g.n * g.oc * g.oh * g.ow >= (1L << 31))
         return false;  // 32-bit output offsets
     const bool ok = requant_table_ok(g.s_src, g.s_flt, g.s_dst);
@@ -388,10 +388,15 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok,
     if (variant == 0) {
         if (!k3)
             return false;
-        *c = make_dma_config<3, 3, 1, 768, false, 2, 2, 2, 1, 4>(g.act, ok);
+        if (g.oc < 128)  // 64 oc x 512 px: each wave 32 oc x 128 px
+            *c = make_dma_config<3, 3, 1, 768, false, 1, 2, 2, 1, 4>(g.act, ok);
+        else
+            *c = make_dma_config<3, 3, 1, 768, false, 2, 2, 2, 1, 4>(g.act, ok);
         return true;
     }
-    if (k3)
+    if (k3 && g.oc < 128)
+        *c = make_dma_config<3, 3, 1, 512, false, 1>(g.act, ok);
+    else if (k3)
         *c = make_dma_config<3, 3, 1, 512, false>(g.act, ok);
     else if (fc && (g.ic & 127) == 0 && b128_ok && g.oc >= 256)
         // 256 x 256 tile, each wave 128 oc x 64 rows (4 x 2 MFMA tiles: 0.75 KB of LDS per MFMA;

@@ -96,6 +96,9 @@ LIVE = [
     ConvCase(A.FMT_NCHW, A.DENSE, 64, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(1024) / 2)),
     ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, 0.1)),
     ConvCase(A.FMT_NCHW, A.DENSE, 200, 512, 1, 1, 333, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(512) / 2)),
+    # split-K of the one-stage kernel where the stages do not divide by the split asked for
+    # (8 stages, 100 tiles -> 6 slices asked, 4 slices of 2 stages run)
+    ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 56, 56, 256, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(2304))),
     # small pointwise layers on the streaming kernel: fewer pixels than one tile per wave, ragged tile
     ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 7, 7, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(256))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 3, 64, 5, 9, 192, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(64))),

@@ -96,6 +96,10 @@ def make_workload(name):
         case = ConvCase(abi.FMT_NCHW, abi.DENSE, 4096, 4096, 1, 1, 4096, 1, 1, 0, abi.IDENTITY,
                         scales=(0.01, 0.01, 0.1))
         return case, "qsi8 FullyConnected 4096x4096x4096", "mfma"
+    if name == "fc1":
+        case = ConvCase(abi.FMT_NCHW, abi.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, abi.IDENTITY,
+                        scales=(0.01, 0.01, 0.1))
+        return case, "qsi8 FullyConnected 1x1024x1000", "hbm"
     if name == "fc64":
         case = ConvCase(abi.FMT_NCHW, abi.DENSE, 64, 4096, 1, 1, 4096, 1, 1, 0, abi.IDENTITY,
                         scales=(0.01, 0.01, 0.1))

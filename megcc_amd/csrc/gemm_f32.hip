@@ -5,8 +5,11 @@
 //     K = (ic, fh, fw) (GeneralIntrinsic/ConvKernel/Fp32Im2col.cpp:88-218 does the same product
 //     through an explicit im2col + pack into workspace; here the gather happens while the B tile
 //     is staged into LDS, so there is no workspace), bias + activation fused into the store.
-// Workgroup: 256 threads (2x2 waves), tile 128 x 128 x 16; LDS tiles are K-major with the row
-// padded by 4 floats so both the staging writes and the MFMA operand reads are bank-conflict free.
+// Workgroup: 256 threads, four waves of 64 x 64 outputs each: tile 128 x 128 x 16 (2 x 2 waves) or,
+// for problems with at most 64 rows (GEVM, batch-64 FullyConnected, convolutions with few output
+// channels), 64 x 256 x 16 (1 x 4 waves) so that no wave multiplies rows that do not exist. LDS
+// tiles are K-major with the row padded by 4 floats so both the staging writes and the MFMA
+// operand reads are bank-conflict free.
 // fp32 sums are formed in a different order from the reference's 4x12 micro-kernel; results are
 // held to 1e-4 relative, not bit-exactness.
 #include "common.h"
@@ -64,15 +67,17 @@ __device__ __forceinline__ float conv_b(const GemmArgs& q, int k, int p) {
 
 // A_KFAST: A(m,k) has k contiguous (row-major, not transposed) -> lanes walk k when staging.
 // B_NFAST: B(k,n) has n contiguous -> lanes walk n.
-template <bool A_KFAST, bool B_NFAST, bool CONV>
+template <bool A_KFAST, bool B_NFAST, bool CONV, int BM>
 __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
+    constexpr int BN = GBM * GBN / BM;  // 128 x 128 or 64 x 256
+    constexpr int A_IT = BM / 16, B_IT = BN / 16;
     // LDS is double buffered: the global loads of step k+1 are in flight (in registers) while
     // step k is multiplied out of the other buffer; one barrier per step.
-    __shared__ float As[2][GBK][GBM + GPAD];
-    __shared__ float Bs[2][GBK][GBN + GPAD];
+    __shared__ float As[2][GBK][BM + GPAD];
+    __shared__ float Bs[2][GBK][BN + GPAD];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * GBM, n0 = blockIdx.x * GBN;
+    const int wm = BM == 128 ? wave >> 1 : 0, wn = BM == 128 ? wave & 1 : wave;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
 
     v16f acc[2][2];
 #pragma unroll
@@ -85,18 +90,46 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
 
     const int k_begin = blockIdx.z * q.kchunk;
     const int k_end = min(q.K, k_begin + q.kchunk);
-    float ra[8], rb[8];
-    // stage A tile (GBM x GBK) and B tile (GBK x GBN): 8 elements per thread each
+    float ra[A_IT], rb[B_IT];
+    // implicit GEMM: with B_NFAST a thread stages the same output pixel in every K step, so its
+    // image / row / column are worked out once
+    const int cn = n0 + tid % BN;
+    long c_img = 0;
+    int c_ih0 = 0, c_iw0 = 0;
+    float c_inv_taps = 0.f, c_inv_fw = 0.f;
+    if (CONV) {
+        const ConvGeom& g = q.g;
+        const int ohw = g.oh * g.ow;
+        const int n = cn / ohw, r = cn - n * ohw;
+        const int oh = r / g.ow, ow = r - oh * g.ow;
+        c_img = (long)n * g.ic * g.ih * g.iw;
+        c_ih0 = oh * g.sh - g.ph;
+        c_iw0 = ow * g.sw - g.pw;
+        c_inv_taps = 1.f / (float)(g.fh * g.fw);
+        c_inv_fw = 1.f / (float)g.fw;
+    }
+    // B(k, cn): the quotients are exact for k below 2^22 (k + 0.5 keeps them off the boundaries)
+    auto conv_b_col = [&](int k) __attribute__((always_inline)) -> float {
+        const ConvGeom& g = q.g;
+        const int taps = g.fh * g.fw;
+        const int ic = (int)(((float)k + 0.5f) * c_inv_taps), t = k - ic * taps;
+        const int fh = (int)(((float)t + 0.5f) * c_inv_fw), fw = t - fh * g.fw;
+        const unsigned ih = (unsigned)(c_ih0 + fh * g.dh), iw = (unsigned)(c_iw0 + fw * g.dw);
+        if (ih >= (unsigned)g.ih || iw >= (unsigned)g.iw)
+            return 0.f;
+        return q.B[c_img + ((size_t)ic * g.ih + ih) * g.iw + iw];
+    };
+    // stage A tile (BM x GBK) and B tile (GBK x BN): BM / 16 and BN / 16 elements per thread
     auto load_tiles = [&](int k0) {
 #pragma unroll
-        for (int it = 0; it < 8; ++it) {
+        for (int it = 0; it < A_IT; ++it) {
             int m, k;
             if (A_KFAST) {
                 k = tid & 15;
                 m = (tid >> 4) + it * 16;
             } else {
-                m = tid & 127;
-                k = (tid >> 7) + it * 2;
+                m = tid % BM;
+                k = tid / BM + it * (256 / BM);
             }
             float v = 0.f;
             if (m0 + m < q.M && k0 + k < k_end)
@@ -104,18 +137,20 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
             ra[it] = v;
         }
 #pragma unroll
-        for (int it = 0; it < 8; ++it) {
+        for (int it = 0; it < B_IT; ++it) {
             int n, k;
             if (B_NFAST) {
-                n = tid & 127;
-                k = (tid >> 7) + it * 2;
+                n = tid % BN;
+                k = tid / BN + it * (256 / BN);
             } else {
                 k = tid & 15;
                 n = (tid >> 4) + it * 16;
             }
             float v = 0.f;
             if (n0 + n < q.N && k0 + k < k_end) {
-                if (CONV)
+                if (CONV && B_NFAST)
+                    v = conv_b_col(k0 + k);
+                else if (CONV)
                     v = conv_b(q, k0 + k, n0 + n);
                 else
                     v = q.B[(size_t)(k0 + k) * q.b_rs + (size_t)(n0 + n) * q.b_cs];
@@ -125,13 +160,16 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
     };
     auto store_tiles = [&](int buf) {
 #pragma unroll
-        for (int it = 0; it < 8; ++it) {
+        for (int it = 0; it < A_IT; ++it) {
             if (A_KFAST)
                 As[buf][tid & 15][(tid >> 4) + it * 16] = ra[it];
             else
-                As[buf][(tid >> 7) + it * 2][tid & 127] = ra[it];
+                As[buf][tid / BM + it * (256 / BM)][tid % BM] = ra[it];
+        }
+#pragma unroll
+        for (int it = 0; it < B_IT; ++it) {
             if (B_NFAST)
-                Bs[buf][(tid >> 7) + it * 2][tid & 127] = rb[it];
+                Bs[buf][tid / BN + it * (256 / BN)][tid % BN] = rb[it];
             else
                 Bs[buf][tid & 15][(tid >> 4) + it * 16] = rb[it];
         }
@@ -300,8 +338,13 @@ TinyNNStatus conv_f32_gemm_launch(
     if (q.M == 0 || q.N == 0)
         return TinyNN_SUCCESS;
     gemm_plan_split(q, ws);
-    dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM, q.split);
-    hipLaunchKernelGGL((gemm_f32_kernel<true, true, true>), grid, dim3(256), 0, stream(), q);
+    if (q.M <= 64 && (long)((q.N + 255) / 256) * q.split >= 128) {
+        dim3 grid((q.N + 255) / 256, 1, q.split);
+        hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 64>), grid, dim3(256), 0, stream(), q);
+    } else {
+        dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM, q.split);
+        hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 128>), grid, dim3(256), 0, stream(), q);
+    }
     if (q.split > 1)
         gemm_launch_reduce(q);
     return check_launch("conv_f32_gemm");
@@ -351,15 +394,28 @@ extern "C" TinyNNStatus megcc_gfx950_matmul(
     if (q.M == 0 || q.N == 0)
         return TinyNN_SUCCESS;
     gemm_plan_split(q, ws);
-    dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM, q.split);
+    // 64 x 256 tiles when they still give every CU a workgroup
+    const bool skinny = q.M <= 64 && (long)((q.N + 255) / 256) * q.split >= 128;
+    dim3 grid(skinny ? (q.N + 255) / 256 : (q.N + GBN - 1) / GBN, skinny ? 1 : (q.M + GBM - 1) / GBM,
+              q.split);
+#define MG_GEMM_LAUNCH(AK, BN_)                                                                  \
+    do {                                                                                         \
+        if (skinny)                                                                              \
+            hipLaunchKernelGGL((gemm_f32_kernel<AK, BN_, false, 64>), grid, dim3(256), 0,        \
+                               stream(), q);                                                     \
+        else                                                                                     \
+            hipLaunchKernelGGL((gemm_f32_kernel<AK, BN_, false, 128>), grid, dim3(256), 0,       \
+                               stream(), q);                                                     \
+    } while (0)
     if (!ta && !tb)
-        hipLaunchKernelGGL((gemm_f32_kernel<true, true, false>), grid, dim3(256), 0, stream(), q);
+        MG_GEMM_LAUNCH(true, true);
     else if (!ta && tb)
-        hipLaunchKernelGGL((gemm_f32_kernel<true, false, false>), grid, dim3(256), 0, stream(), q);
+        MG_GEMM_LAUNCH(true, false);
     else if (ta && !tb)
-        hipLaunchKernelGGL((gemm_f32_kernel<false, true, false>), grid, dim3(256), 0, stream(), q);
+        MG_GEMM_LAUNCH(false, true);
     else
-        hipLaunchKernelGGL((gemm_f32_kernel<false, false, false>), grid, dim3(256), 0, stream(), q);
+        MG_GEMM_LAUNCH(false, false);
+#undef MG_GEMM_LAUNCH
     if (q.split > 1)
         gemm_launch_reduce(q);
     return check_launch("matmul");

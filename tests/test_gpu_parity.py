@@ -96,6 +96,9 @@ LIVE = [
     ConvCase(A.FMT_NCHW, A.DENSE, 64, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(1024) / 2)),
     ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, 0.1)),
     ConvCase(A.FMT_NCHW, A.DENSE, 200, 512, 1, 1, 333, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(512) / 2)),
+    # 3x3 layers with 64..127 output channels on the LDS-direct kernel (64-channel tiles, one of them ragged)
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 64, 40, 40, 64, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(576))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 9, 32, 31, 29, 96, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(288))),
     # split-K of the one-stage kernel where the stages do not divide by the split asked for
     # (8 stages, 100 tiles -> 6 slices asked, 4 slices of 2 stages run)
     ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 56, 56, 256, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(2304))),

@@ -8,6 +8,7 @@
 
 #include "common.h"
 #include "conv_geom.h"
+#include "conv_mfma_i8.h"
 #include "epilogue.cuh"
 
 namespace mg {
@@ -82,11 +83,13 @@ __device__ __forceinline__ void transpose4x4(const dw_v4u p, unsigned (&t)[4]) {
 // Two vertically adjacent output rows per thread: their 3 + 3 input rows overlap (4 distinct rows
 // for stride 1, 5 for stride 2), so a row is loaded and transposed once for both, and the weights
 // are rearranged once for 32 outputs.
-template <int S, int ACT, int R>
+// RAGGED: the input width is not a multiple of the pixels a thread loads per row (4, or 8 with
+// stride 2), so the loads of the last group run into the next row and are masked.
+template <int S, int ACT, int R, bool RAGGED>
 __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
         ConvGeom g, RequantFast rq, const uint32_t* __restrict__ src, const uint32_t* __restrict__ flt,
         const int32_t* __restrict__ bias, uint32_t* __restrict__ dst, int total, int src_bytes,
-        RequantTable table) {
+        FastDiv d_ogn, FastDiv d_ohn, FastDiv d_c4n, RequantTable table) {
     __shared__ int tbl[REQUANT_TABLE_ENTRIES];
     if (ACT >= 0) {
         tbl[threadIdx.x] = table.t[threadIdx.x];
@@ -99,11 +102,10 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, src_bytes, 0x00020000);
     const int OOB = (int)0x80000000u;
     for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
-        int r = i;
-        const int og = r % ogn; r /= ogn;
-        const int oh = (r % ohn) * R; r /= ohn;
-        const int c4 = r % c4n;
-        const int n = r / c4n;
+        // i = ((n * c4n + c4) * ohn + row group) * ogn + pixel group; divisions by multiplication
+        const int r1 = fdiv(i, d_ogn), og = i - r1 * ogn;
+        const int r2 = fdiv(r1, d_ohn), oh = (r1 - r2 * ohn) * R;
+        const int n = fdiv(r2, d_c4n), c4 = r2 - n * c4n;
         const int plane_off = ((n * c4n + c4) * g.ih) * g.iw * 4;  // bytes
         // weights: per filter row one dword per channel = (w(fw=0), w(fw=1), w(fw=2), 0)
         unsigned wq[3][4];
@@ -137,9 +139,11 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
                     rs, row_ok && iw0 > 0 ? row_off + (iw0 - 1) * 4 : OOB, 0, 0);
             dw_v4u l0 = __builtin_amdgcn_raw_buffer_load_b128(rs, row_ok ? row_off + iw0 * 4 : OOB, 0, 0);
             // pixels past the end of the row belong to the next row: zero them
+            if (RAGGED) {
 #pragma unroll
-            for (int k = 1; k < 4; ++k)
-                l0[k] = k < left ? l0[k] : 0u;
+                for (int k = 1; k < 4; ++k)
+                    l0[k] = k < left ? l0[k] : 0u;
+            }
             unsigned t0[4];
             transpose4x4(l0, t0);
             // the four 3-pixel windows of each channel in this input row
@@ -157,9 +161,11 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
             } else {
                 dw_v4u l1 = __builtin_amdgcn_raw_buffer_load_b128(
                         rs, row_ok && left > 4 ? row_off + (iw0 + 4) * 4 : OOB, 0, 0);
+                if (RAGGED) {
 #pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    l1[k] = k + 4 < left ? l1[k] : 0u;
+                    for (int k = 0; k < 4; ++k)
+                        l1[k] = k + 4 < left ? l1[k] : 0u;
+                }
                 unsigned t1[4];
                 transpose4x4(l1, t1);
 #pragma unroll
@@ -243,25 +249,29 @@ TinyNNStatus dwconv44_launch(
         unsigned nb = (unsigned)((groups4 + 255) / 256);
         const RequantFast rq3 = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
         void (*k3)(ConvGeom, RequantFast, const uint32_t*, const uint32_t*, const int32_t*, uint32_t*, int, int,
-                   RequantTable);
+                   FastDiv, FastDiv, FastDiv, RequantTable);
         // exact thresholds for the monotone activations; anything else (and extreme scales)
         // evaluates the literal sequence per output
         const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
                          requant_table_ok(g.s_src, g.s_flt, g.s_dst);
         static const RequantTable no_table = {};
         const RequantTable& table = tab ? requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst) : no_table;
-#define MG_DW_PICK(S_, R_)                                                                      \
-    (tab && g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_IDENTITY, R_> \
-     : tab && g.act == MEGCC_NONLINE_RELU   ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_RELU, R_>     \
-                                            : dwconv44_3x3_kernel<S_, -1, R_>)
-        if (g.sh == 1)
-            k3 = R == 2 ? MG_DW_PICK(1, 2) : MG_DW_PICK(1, 1);
+#define MG_DW_PICK(S_, R_, G_)                                                                      \
+    (tab && g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_IDENTITY, R_, G_> \
+     : tab && g.act == MEGCC_NONLINE_RELU   ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_RELU, R_, G_>     \
+                                            : dwconv44_3x3_kernel<S_, -1, R_, G_>)
+        const bool ragged = (g.iw % (4 * g.sh)) != 0;
+        if (g.sh == 1 && R == 2)
+            k3 = ragged ? MG_DW_PICK(1, 2, true) : MG_DW_PICK(1, 2, false);
+        else if (g.sh == 1)
+            k3 = ragged ? MG_DW_PICK(1, 1, true) : MG_DW_PICK(1, 1, false);
         else
-            k3 = R == 2 ? MG_DW_PICK(2, 2) : MG_DW_PICK(2, 1);
+            k3 = ragged ? MG_DW_PICK(2, 1, true) : MG_DW_PICK(2, 1, false);
 #undef MG_DW_PICK
         hipLaunchKernelGGL(k3, dim3(nb), dim3(256), 0, stream(), g, rq3, (const uint32_t*)src,
                            (const uint32_t*)flt, (const int32_t*)bias, (uint32_t*)dst, groups4,
-                           (int)((long)g.n * g.ic * g.ih * g.iw), table);
+                           (int)((long)g.n * g.ic * g.ih * g.iw), make_fastdiv((g.ow + 3) / 4),
+                           make_fastdiv((g.oh + R - 1) / R), make_fastdiv(g.oc >> 2), table);
         return check_launch("dwconv44_3x3");
     }
     unsigned blocks = (unsigned)((total + 255) / 256);

@@ -69,8 +69,23 @@ def headline_case(n=32, c=256, hw=56):
 
 def make_workload(name):
     """-> (case, description, bound, algorithmic units per launch)"""
-    from cases import ConvCase, MatMulCase, MultiTypeCase, PoolCase, TypeCvtCase
+    from cases import (ConcatCase, ConvCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
+                       TypeCvtCase)
     from megcc_amd import abi
+    if name in ("to_nchw4", "from_nchw4"):
+        hw = 56 * 56
+        nchw = (256 * hw, 4 * hw, 56, 1, hw)  # a [N, C/4, H, W, 4] view of NCHW memory
+        shape = (32, 64, 56, 56, 4)
+        if name == "to_nchw4":
+            return (RelayoutCase("qsi8", shape, nchw, slack=0),
+                    "qsi8 relayout NCHW -> NCHW4 N=32 C=256 56x56", "hbm")
+        return (RelayoutCase("qsi8", shape, None, None, nchw, slack=0),
+                "qsi8 relayout NCHW4 -> NCHW N=32 C=256 56x56", "hbm")
+    if name == "transpose":
+        return RelayoutCase("f32", (4096, 4096), (1, 4096), slack=0), "f32 transpose 4096x4096", "hbm"
+    if name == "concat":
+        return (ConcatCase("qsi8", [(32, 32, 56, 56, 4), (32, 32, 56, 56, 4)], 1),
+                "qsi8 concat of two N=32 C=128 56x56 NCHW44 maps along C", "hbm")
     if name == "conv":
         case = headline_case()
         return case, "qsi8 conv3x3 s1 p1 NCHW44 N=32 Cin=Cout=256 56x56 +bias +ReLU requant", "mfma"

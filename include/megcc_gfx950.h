@@ -305,6 +305,24 @@ TinyNNStatus megcc_gfx950_reduce(
         const MegccReduceAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs,
         int nr_output, const Workspace* workspace, const RuntimeOpt* opt);
 
+/* Relayout: copy between two strided views of the same dtype and element count (dimshuffle,
+ * subtensor copies, NCHW <-> NCHW4 changes). Each side is walked in row-major order of its own
+ * dims with its own strides (elements; negative strides and stride-0 sources allowed); element k
+ * of the source becomes element k of the destination. Replaces BareMetal::RelayoutKernel
+ * (BareMetal/Relayout.cpp:13-101, Common/Relayout.h:10-80; symbol kernel_relayout_<dtype>) and
+ * GeneralIntrinsic::RelayoutKernel (GeneralIntrinsic/Relayout.cpp:27-48, GI_kernel_relayout_<dtype>).
+ * inputs = {src}, outputs = {dst}; dtypes of 1, 2 and 4 bytes. */
+TinyNNStatus megcc_gfx950_relayout(
+        Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace* workspace, const RuntimeOpt* opt);
+
+/* Concat along *axis: input i goes to the slice of the output that starts where the inputs
+ * before it end. Inputs and output may be strided. Replaces BareMetal::ConcatKernel
+ * (BareMetal/Concat.cpp:14-76; symbol kernel_concat_byte_<dtype bytes>_axis_<axis>). */
+TinyNNStatus megcc_gfx950_concat(
+        const int* axis, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace* workspace, const RuntimeOpt* opt);
+
 /* ------------------------------------------------------------------------------------------
  * Dispatch by the reference's kernel symbol: lets a caller that only knows the generated name
  * (e.g. "kernel_conv2d_3x3_NCHW44_DENSE_p1x1_s1x1_d1x1_qsi8qsi8qsi32qsi8_bias_RELU",
@@ -318,7 +336,9 @@ typedef enum {
     MEGCC_KERN_ELEMWISE_MULTITYPE = 4,
     MEGCC_KERN_ELEMWISE = 5,
     MEGCC_KERN_TYPECVT = 6,
-    MEGCC_KERN_REDUCE = 7
+    MEGCC_KERN_REDUCE = 7,
+    MEGCC_KERN_RELAYOUT = 8,
+    MEGCC_KERN_CONCAT = 9
 } MegccKernelKind;
 
 typedef struct {
@@ -330,6 +350,7 @@ typedef struct {
         MegccMultiTypeMode multitype;
         MegccElemwiseMode elemwise;
         MegccReduceAttr reduce;
+        int concat_axis;
     } attr;
 } MegccKernelDesc;
 
@@ -394,6 +415,15 @@ int megcc_gfx950_model_add_weight(
         float scale, const void* host_data);
 int megcc_gfx950_model_add_alias(
         void* model, const char* name, int of_tensor, int nr_dim, const uint32_t* dims);
+/* A strided window into `of_tensor`: dims and strides (in elements, may be negative or 0) of the
+ * view, whose first element lies offset_bytes after the start of `of_tensor`. This is what a
+ * MemForward instruction of type SUBTENSOR or DIMSHUFFLE leaves behind (runtime/schema/
+ * model.fbs:119-140, runtime/src/vm/memforward.c:43-53); operators that take strided tensors
+ * (Relayout, Concat, MatMul row strides) read it as it is. -1 when an element would lie outside
+ * of_tensor. */
+int megcc_gfx950_model_add_view(
+        void* model, const char* name, int of_tensor, int nr_dim, const uint32_t* dims,
+        const int* strides, size_t offset_bytes);
 TinyNNStatus megcc_gfx950_model_add_opr(
         void* model, const char* symbol, const int* inputs, int nr_input, const int* outputs,
         int nr_output);

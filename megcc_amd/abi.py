@@ -42,6 +42,7 @@ REDUCE_SUM, REDUCE_MEAN, REDUCE_MAX, REDUCE_MIN = 0, 1, 2, 3
 # MegccKernelKind
 KERN_CONV, KERN_MATMUL, KERN_POOLING, KERN_ELEMWISE_MULTITYPE = 1, 2, 3, 4
 KERN_ELEMWISE, KERN_TYPECVT, KERN_REDUCE = 5, 6, 7
+KERN_RELAYOUT, KERN_CONCAT = 8, 9
 
 
 class Device(C.Structure):
@@ -127,6 +128,7 @@ class _KernelAttrUnion(C.Union):
     _fields_ = [
         ("conv", ConvAttr), ("matmul", MatMulAttr), ("pool", PoolAttr),
         ("multitype", C.c_int), ("elemwise", C.c_int), ("reduce", ReduceAttr),
+        ("concat_axis", C.c_int),
     ]
 
 
@@ -173,10 +175,12 @@ def make_tensor(ptr, shape, type_enum, scale=1.0, name=b"t", strides=None):
     return t
 
 
-def host_tensor(arr, type_enum, scale=1.0, name=b"t"):
-    """Tensor over a C-contiguous numpy array (kept alive by the caller)."""
+def host_tensor(arr, type_enum, scale=1.0, name=b"t", shape=None, strides=None, offset=0):
+    """Tensor over a C-contiguous numpy array (kept alive by the caller). With `shape`, a view
+    into it: `strides` and `offset` (where the view's first element lies) count elements."""
     assert arr.flags["C_CONTIGUOUS"]
-    return make_tensor(arr.ctypes.data, arr.shape, type_enum, scale, name)
+    return make_tensor(arr.ctypes.data + offset * arr.itemsize,
+                       arr.shape if shape is None else shape, type_enum, scale, name, strides)
 
 
 def tensor_array(tensors):

@@ -211,6 +211,21 @@ extern "C" TinyNNStatus megcc_gfx950_parse_symbol(const char* symbol, MegccKerne
                 return TinyNN_SUCCESS;
             }
         }
+    } else if (eat(s, "GI_kernel_relayout_") || eat(s, "kernel_relayout_")) {
+        if (s == "f32" || s == "qsi8" || s == "si8" || s == "i8" || s == "ui8" || s == "qsi32" ||
+            s == "i32" || s == "i16" || s == "ui16" || s == "f16") {
+            desc->kind = MEGCC_KERN_RELAYOUT;
+            return TinyNN_SUCCESS;
+        }
+    } else if (eat(s, "kernel_concat_byte_")) {
+        int bytes = 0, axis = -1;
+        char tail = 0;
+        if (sscanf(s.c_str(), "%d_axis_%d%c", &bytes, &axis, &tail) == 2 &&
+            (bytes == 1 || bytes == 2 || bytes == 4) && axis >= 0 && axis < MAX_DIM) {
+            desc->kind = MEGCC_KERN_CONCAT;
+            desc->attr.concat_axis = axis;
+            return TinyNN_SUCCESS;
+        }
     } else if (eat(s, "GI_kernel_fp32_matmul_4x12_") || eat(s, "GI_kernel_gevm_") ||
                eat(s, "GI_kernel_gemv_") || eat(s, "kernel_matmul_")) {
         if (s.size() >= 2 && (s[0] == 'n' || s[0] == 't') && (s[1] == 'n' || s[1] == 't') &&
@@ -244,6 +259,11 @@ extern "C" TinyNNStatus megcc_gfx950_call(
             return megcc_gfx950_typecvt(inputs, nr_input, outputs, nr_output, ws, opt);
         case MEGCC_KERN_REDUCE:
             return megcc_gfx950_reduce(&d->attr.reduce, inputs, nr_input, outputs, nr_output, ws, opt);
+        case MEGCC_KERN_RELAYOUT:
+            return megcc_gfx950_relayout(inputs, nr_input, outputs, nr_output, ws, opt);
+        case MEGCC_KERN_CONCAT:
+            return megcc_gfx950_concat(&d->attr.concat_axis, inputs, nr_input, outputs, nr_output,
+                                       ws, opt);
         default:
             return fail(TinyNN_ERROR_NO_FOUND, "call: unknown kernel kind %d", (int)d->kind);
     }

@@ -41,6 +41,19 @@ inline bool is_contiguous(const Layout& l) {
     return true;
 }
 
+// Lowest and highest element offset a layout touches, relative to its first element; false when
+// it has no elements.
+inline bool view_span(const Layout& l, long long* lo, long long* hi) {
+    *lo = *hi = 0;
+    for (int i = 0; i < l.nr_dim; ++i) {
+        if (l.dims[i] == 0)
+            return false;
+        const long long reach = (long long)(l.dims[i] - 1) * l.stride[i];
+        (reach < 0 ? *lo : *hi) += reach;
+    }
+    return true;
+}
+
 inline bool is_q8(const Tensor* t) {
     return t->dtype.type_enum == TinyNN_QINT8 || t->dtype.type_enum == TinyNN_INT8;
 }

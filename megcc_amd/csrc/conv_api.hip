@@ -157,7 +157,8 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
     if (st != TinyNN_SUCCESS)
         return st;
     if (bias) {
-        MG_REQUIRE(nr_elem(bias->layout) == (size_t)g.oc, TinyNN_ERROR_INVALID_LAYOUT,
+        MG_REQUIRE(nr_elem(bias->layout) == (size_t)g.oc && is_contiguous(bias->layout),
+                   TinyNN_ERROR_INVALID_LAYOUT,
                    "conv2d: bias must be per output channel (%zu elements, oc=%d)",
                    nr_elem(bias->layout), g.oc);
         if (q8) {

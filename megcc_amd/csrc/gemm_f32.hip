@@ -380,6 +380,11 @@ extern "C" TinyNNStatus megcc_gfx950_matmul(
                        (int)(tb ? b->layout.dims[0] : b->layout.dims[1]) == q.N,
                TinyNN_ERROR_INVALID_LAYOUT, "matmul: shapes do not agree");
     const long lda = a->layout.stride[0], ldb = b->layout.stride[0];
+    // rows may be padded (a leading dimension larger than the row), never overlapping or reversed
+    MG_REQUIRE((a->layout.dims[0] <= 1 || lda >= (long)a->layout.dims[1]) &&
+                       (b->layout.dims[0] <= 1 || ldb >= (long)b->layout.dims[1]) &&
+                       (c->layout.dims[0] <= 1 || c->layout.stride[0] >= (long)c->layout.dims[1]),
+               TinyNN_ERROR_INVALID_LAYOUT, "matmul: a leading stride is shorter than its row");
     q.A = (const float*)a->ptr;
     q.B = (const float*)b->ptr;
     q.C = (float*)c->ptr;

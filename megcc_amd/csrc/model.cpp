@@ -224,6 +224,40 @@ int megcc_gfx950_model_add_alias(
     return id;
 }
 
+// A strided window into tensor `of` (what the compiler's SUBTENSOR / DIMSHUFFLE MemForward
+// leaves in a model, runtime/schema/model.fbs:125-140): dims and strides (elements) of the view,
+// its first element `offset_bytes` after the start of `of`. Every element must lie inside `of`.
+int megcc_gfx950_model_add_view(
+        void* model, const char* name, int of, int nr_dim, const uint32_t* dims,
+        const int* strides, size_t offset_bytes) {
+    Model* m = (Model*)model;
+    if (!m || !strides || of < 0 || of >= (int)m->tensors.size())
+        return -1;
+    const Tensor& src = m->tensors[of]->t;
+    if (m->tensors[of]->alias_of >= 0 && !is_contiguous(src.layout)) {
+        fail(TinyNN_ERROR_INVALID_LAYOUT, "model_add_view: a view of a strided view");
+        return -1;
+    }
+    int id = add_tensor(m, name, nr_dim, dims, src.dtype.type_enum, src.dtype.param.scale);
+    if (id < 0)
+        return -1;
+    Tensor& t = m->tensors[id]->t;
+    for (int i = 0; i < nr_dim; ++i)
+        t.layout.stride[i] = strides[i];
+    long long lo, hi;
+    const long long es = (long long)dtype_size(&t);
+    if (view_span(t.layout, &lo, &hi) &&
+        ((long long)offset_bytes + lo * es < 0 ||
+         (long long)offset_bytes + (hi + 1) * es > (long long)tensor_bytes(src))) {
+        fail(TinyNN_ERROR_OUT_OF_RANGE, "model_add_view: view leaves the %zu bytes of tensor %d",
+             tensor_bytes(src), of);
+        return -1;
+    }
+    m->tensors[id]->alias_of = of;
+    m->tensors[id]->alias_offset = offset_bytes;
+    return id;
+}
+
 TinyNNStatus megcc_gfx950_model_add_opr(
         void* model, const char* symbol, const int* inputs, int nr_input, const int* outputs,
         int nr_output) {
@@ -723,24 +757,34 @@ TinyNNStatus load_into(Model* m, const tiny::ModelInfo& info) {
         }
     }
 
-    // every byte a kernel may touch lies inside the arena (or inside the tensor a view points at)
+    // every byte a kernel may touch lies inside the arena (or inside the tensor a view points at);
+    // only views may be strided
     for (int i = 0; i < nt; ++i) {
         ModelTensor* t = m->tensors[i];
         if (t->alias_of >= 0) {
-            size_t shift = 0;
+            long long shift = 0;
             int id = i, hops = 0;
             while (m->tensors[id]->alias_of >= 0) {
-                shift += m->tensors[id]->alias_offset;
+                shift += (long long)m->tensors[id]->alias_offset;
                 id = m->tensors[id]->alias_of;
                 MG_REQUIRE(++hops <= nt, TinyNN_ERROR_MODEL_PARSE, "model_load: MemForward cycle");
             }
-            MG_REQUIRE(shift + t->t.size <= m->tensors[id]->t.size, TinyNN_ERROR_MODEL_PARSE,
-                       "model_load: tensor %d views bytes %zu..%zu of tensor %d (%zu bytes)", i,
-                       shift, shift + (size_t)t->t.size, id, (size_t)m->tensors[id]->t.size);
-        } else if (!t->is_input) {
-            MG_REQUIRE(t->t.offset + t->t.size <= m->arena_bytes, TinyNN_ERROR_MODEL_PARSE,
-                       "model_load: tensor %d ends at byte %zu of a %zu byte arena", i,
-                       (size_t)(t->t.offset + t->t.size), m->arena_bytes);
+            long long lo, hi;
+            if (!view_span(t->t.layout, &lo, &hi))
+                continue;  // no elements
+            const long long es = (long long)dtype_size(&t->t);
+            MG_REQUIRE(shift + lo * es >= 0 &&
+                               shift + (hi + 1) * es <= (long long)m->tensors[id]->t.size,
+                       TinyNN_ERROR_MODEL_PARSE,
+                       "model_load: tensor %d views bytes %lld..%lld of tensor %d (%zu bytes)", i,
+                       shift + lo * es, shift + (hi + 1) * es, id, (size_t)m->tensors[id]->t.size);
+        } else {
+            MG_REQUIRE(is_contiguous(t->t.layout), TinyNN_ERROR_MODEL_PARSE,
+                       "model_load: tensor %d owns memory but is not dense", i);
+            if (!t->is_input)
+                MG_REQUIRE(t->t.offset + t->t.size <= m->arena_bytes, TinyNN_ERROR_MODEL_PARSE,
+                           "model_load: tensor %d ends at byte %zu of a %zu byte arena", i,
+                           (size_t)(t->t.offset + t->t.size), m->arena_bytes);
         }
     }
     return megcc_gfx950_model_finalize(m);

@@ -9,6 +9,8 @@
 //   elemwise  BareMetal/ElemwiseKernel.cpp:433-439
 //   reduce    BareMetal/Reduce.cpp:82-90
 //   matmul    BareMetal/MatrixMul.cpp:26-41
+//   relayout  GeneralIntrinsic/Relayout.cpp:43-48 (first in the x86 list for 1/2/4-byte dtypes)
+//   concat    BareMetal/Concat.cpp:14-22
 // (for f32 conv / matmul / elemwise / reduce the x86 registry prefers GI variants whose names
 // carry tiling details; the BAREMETAL template's name is used for those, and the run-time library
 // also resolves the GI spellings.)
@@ -421,6 +423,53 @@ struct ReduceKernel : KernelFuncBase {
     }
 };
 
+// ---- Relayout / Concat (dtypes of 1, 2 and 4 bytes) --------------------------------------------
+// Utils/Utils.h:41-84 get_dtype_size
+int dtype_bytes(const std::string& d) {
+    const std::string v = valid_dtype(d);
+    if (v == "f32" || v == "i32" || v == "qsi32")
+        return 4;
+    if (v == "f16" || v == "i16" || v == "ui16")
+        return 2;
+    if (v == "i8" || v == "si8" || v == "ui8" || v == "qsi8")
+        return 1;
+    return 0;
+}
+
+struct RelayoutKernel : KernelFuncBase {
+    bool IsAvailable(TContext* c) const override {
+        const std::string d = c->getAttrOprand("operand:0").dtype;
+        return dtype_bytes(d) != 0 && d == c->getAttrOprand("operand:1").dtype;
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        return "GI_kernel_relayout_" + valid_dtype(c->getAttrOprand("operand:0").dtype);
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        return kHeader + kernel_def(this, c, "",
+                                    "megcc_gfx950_relayout(inputs, nr_input, outputs, nr_output, "
+                                    "workspace, opt)");
+    }
+};
+
+struct ConcatKernel : KernelFuncBase {
+    bool IsAvailable(TContext* c) const override {
+        return dtype_bytes(c->getAttrOprand("operand:0").dtype) != 0 && c->getAttrInt("axis") >= 0;
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        std::stringstream ss;
+        ss << "kernel_concat_byte_" << dtype_bytes(c->getAttrOprand("operand:0").dtype) << "_axis_"
+           << c->getAttrInt("axis");
+        return ss.str();
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        std::stringstream a;
+        a << "    static const int axis = " << c->getAttrInt("axis") << ";\n";
+        return kHeader + kernel_def(this, c, a.str(),
+                                    "megcc_gfx950_concat(&axis, inputs, nr_input, outputs, "
+                                    "nr_output, workspace, opt)");
+    }
+};
+
 // ---- MatrixMul (f32) ---------------------------------------------------------------------------
 struct MatrixMulKernel : KernelFuncBase {
     bool IsAvailable(TContext* c) const override {
@@ -465,6 +514,8 @@ std::vector<const KernelFuncBase*> Gfx950KernelPack::GetKernel(KernType type) {
     static const TypeCvtKernel typecvt;
     static const ReduceKernel reduce;
     static const MatrixMulKernel matmul;
+    static const RelayoutKernel relayout;
+    static const ConcatKernel concat;
     switch (type) {
         case KernType::ConvKernel: return {&conv};
         case KernType::PoolingKernel: return {&pool};
@@ -473,6 +524,8 @@ std::vector<const KernelFuncBase*> Gfx950KernelPack::GetKernel(KernType type) {
         case KernType::TypeCvtKernel: return {&typecvt};
         case KernType::ReduceKernel: return {&reduce};
         case KernType::MatrixMulKernel: return {&matmul};
+        case KernType::RelayoutKernel: return {&relayout};
+        case KernType::ConcatKernel: return {&concat};
         default: return {};
     }
 }

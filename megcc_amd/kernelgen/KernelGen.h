@@ -89,8 +89,10 @@ enum class KernType {
     ElemwiseMultiKernel,
     PoolingKernel,
     MatrixMulKernel,
+    RelayoutKernel = 7,
     ReduceKernel = 8,
     TypeCvtKernel = 13,
+    ConcatKernel = 25,
 };
 
 }  // namespace megcc_gfx950

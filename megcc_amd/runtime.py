@@ -34,6 +34,8 @@ def lib():
         L.megcc_gfx950_elemwise.argtypes = [C.POINTER(C.c_int)] + kern
         L.megcc_gfx950_typecvt.argtypes = kern
         L.megcc_gfx950_reduce.argtypes = [C.POINTER(abi.ReduceAttr)] + kern
+        L.megcc_gfx950_relayout.argtypes = kern
+        L.megcc_gfx950_concat.argtypes = [C.POINTER(C.c_int)] + kern
         L.megcc_gfx950_parse_symbol.argtypes = [C.c_char_p, C.POINTER(abi.KernelDesc)]
         L.megcc_gfx950_call.argtypes = [C.POINTER(abi.KernelDesc)] + kern
         L.megcc_gfx950_call_init.argtypes = [C.POINTER(abi.KernelDesc)] + abi.INIT_ARGS
@@ -59,6 +61,8 @@ def lib():
         L.megcc_gfx950_model_add_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_int, dims, C.c_int, C.c_float]
         L.megcc_gfx950_model_add_weight.argtypes = [C.c_void_p, C.c_char_p, C.c_int, dims, C.c_int, C.c_float, C.c_void_p]
         L.megcc_gfx950_model_add_alias.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_int, dims]
+        L.megcc_gfx950_model_add_view.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_int, dims,
+                                                  C.POINTER(C.c_int), C.c_size_t]
         ints = C.POINTER(C.c_int)
         L.megcc_gfx950_model_add_opr.argtypes = [C.c_void_p, C.c_char_p, ints, C.c_int, ints, C.c_int]
         L.megcc_gfx950_model_mark_io.argtypes = [C.c_void_p, C.c_int, C.c_int]
@@ -86,13 +90,15 @@ EXPORTS = [
     "megcc_gfx950_conv2d", "megcc_gfx950_conv2d_init", "megcc_gfx950_conv2d_workspace",
     "megcc_gfx950_matmul", "megcc_gfx950_matmul_workspace", "megcc_gfx950_pooling",
     "megcc_gfx950_elemwise_multitype", "megcc_gfx950_elemwise", "megcc_gfx950_typecvt",
-    "megcc_gfx950_reduce", "megcc_gfx950_parse_symbol", "megcc_gfx950_call",
+    "megcc_gfx950_reduce", "megcc_gfx950_relayout", "megcc_gfx950_concat",
+    "megcc_gfx950_parse_symbol", "megcc_gfx950_call",
     "megcc_gfx950_call_init", "megcc_gfx950_call_workspace", "megcc_gfx950_init_device",
     "megcc_gfx950_malloc", "megcc_gfx950_free", "megcc_gfx950_memcpy_h2d",
     "megcc_gfx950_memcpy_d2h", "megcc_gfx950_memset", "megcc_gfx950_wait",
     "megcc_gfx950_stream", "megcc_gfx950_last_error",
     "megcc_gfx950_model_create", "megcc_gfx950_model_destroy", "megcc_gfx950_model_add_tensor",
-    "megcc_gfx950_model_add_weight", "megcc_gfx950_model_add_alias", "megcc_gfx950_model_add_opr",
+    "megcc_gfx950_model_add_weight", "megcc_gfx950_model_add_alias", "megcc_gfx950_model_add_view",
+    "megcc_gfx950_model_add_opr",
     "megcc_gfx950_model_mark_io", "megcc_gfx950_model_finalize", "megcc_gfx950_model_arena_bytes",
     "megcc_gfx950_model_tensor_ptr", "megcc_gfx950_model_set_input",
     "megcc_gfx950_model_get_output", "megcc_gfx950_model_forward", "megcc_gfx950_model_nr_opr",
@@ -197,13 +203,17 @@ class PreparedOp:
         for s in in_specs:
             buf = DeviceBuffer.from_array(s.array)
             self.keep.append(buf)
-            self.in_tensors.append(abi.make_tensor(buf.ptr, s.shape, s.type_enum, s.scale, s.name))
+            self.in_tensors.append(abi.make_tensor(
+                buf.ptr + s.offset * s.array.itemsize, s.shape, s.type_enum, s.scale, s.name,
+                s.strides))
         self.out_bufs, self.out_tensors, self.out_specs = [], [], out_specs
         for s in out_specs:
             buf = DeviceBuffer(s.nbytes)
             buf.fill(0x5A)  # poison: an element the kernel fails to write shows up in the compare
             self.out_bufs.append(buf)
-            self.out_tensors.append(abi.make_tensor(buf.ptr, s.shape, s.type_enum, s.scale, s.name))
+            self.out_tensors.append(abi.make_tensor(
+                buf.ptr + s.offset * abi.np_dtype(s.type_enum).itemsize, s.shape, s.type_enum,
+                s.scale, s.name, s.strides))
         # workspace
         size = C.c_size_t(0)
         ins = abi.tensor_array(self.in_tensors)
@@ -243,7 +253,7 @@ class PreparedOp:
 
     def result(self, i=0):
         s = self.out_specs[i]
-        return self.out_bufs[i].to_array(s.shape, abi.np_dtype(s.type_enum))
+        return self.out_bufs[i].to_array(s.storage, abi.np_dtype(s.type_enum))
 
 
 def run_symbol(symbol, in_specs, out_specs):
@@ -301,6 +311,14 @@ class Model:
     def alias(self, name, of, shape):
         tid = lib().megcc_gfx950_model_add_alias(self.h, name.encode(), of, len(shape), self._dims(shape))
         return self._remember(tid, shape, self.shapes[of][1], "add_alias")
+
+    def view(self, name, of, shape, strides, offset=0):
+        """strided window into tensor `of`: element strides, first element `offset` elements in"""
+        es = abi.np_dtype(self.shapes[of][1]).itemsize
+        tid = lib().megcc_gfx950_model_add_view(
+            self.h, name.encode(), of, len(shape), self._dims(shape),
+            (C.c_int * len(shape))(*[int(s) for s in strides]), C.c_size_t(offset * es))
+        return self._remember(tid, shape, self.shapes[of][1], "add_view")
 
     def opr(self, symbol, inputs, outputs):
         ins = (C.c_int * len(inputs))(*inputs)

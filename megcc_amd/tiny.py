@@ -19,6 +19,9 @@ TENSOR, WEIGHT = 0, 1
 MEMFORWARD_RESHAPE, MEMFORWARD_SUBTENSOR, MEMFORWARD_DIMSHUFFLE = 0, 1, 2
 INSTRUCTION_IDS = {"Opr": 1, "DevMemAlloc": 2, "DevMemFree": 3, "MemForward": 4}
 
+_ITEMSIZE = {FLOAT32: 4, FLOAT16: 2, INT32: 4, INT8: 1, INT16: 2, UINT8: 1, QINT8: 1, QINT32: 4,
+             QUINT8: 1}
+
 _SCALARS = {"i8": "<b", "u8": "<B", "bool": "<B", "i32": "<i", "u32": "<I", "i64": "<q",
             "u64": "<Q", "f32": "<f"}
 
@@ -284,6 +287,17 @@ class ModelBuilder:
                                                      type=MEMFORWARD_RESHAPE)))
         return tid
 
+    def view(self, name, of, shape, strides, offset=0, kind=MEMFORWARD_SUBTENSOR):
+        """strided window into tensor `of` (element strides, first element `offset` elements
+        in): the tensor carries the strides, a MemForward of type `kind` the byte offset"""
+        src = self.tensors[of]
+        tid = self.tensor(name, shape, src["dtype"][0], src["dtype"][1] or 1.0)
+        self.tensors[tid]["stride"] = [int(s) for s in strides]
+        self._root[tid] = of
+        self.instructions.append(("MemForward", dict(
+            input=of, output=tid, offset=int(offset) * _ITEMSIZE[src["dtype"][0]], type=kind)))
+        return tid
+
     def _root_of(self, t):
         while self._root[t] >= 0:
             t = self._root[t]
@@ -329,9 +343,7 @@ class ModelBuilder:
         size = []
         for t in planned:
             info = self.tensors[t]
-            item = {FLOAT32: 4, FLOAT16: 2, INT32: 4, INT8: 1, INT16: 2, UINT8: 1, QINT8: 1,
-                    QINT32: 4, QUINT8: 1}[info["dtype"][0]]
-            size.append(int(np.prod(info["dims"])) * item)
+            size.append(int(np.prod(info["dims"])) * _ITEMSIZE[info["dtype"][0]])
         offsets, arena, _ = runtime.plan_memory(begin, end, size, self.alignment)
         for t, off in zip(planned, offsets):
             self.tensors[t]["offset"] = int(off)

@@ -406,3 +406,55 @@ void orc_reduce_f32(const float* src, float* dst, int mode, int A, int B, int C)
             dst[(size_t)i * C + k] = mode == RED_MEAN ? acc / B : acc;
         }
 }
+
+/* Relayout: BareMetal/Relayout.cpp:83-91 (the "fallback to naive" loop, which every faster
+ * branch of that kernel must agree with) over the odometers of Common/Relayout.h:18-40:
+ * element k, counted in the row-major order of each side's own dims, goes from
+ * src[sum idx_s * sstride] to dst[sum idx_d * dstride]. Offsets are in elements of `es` bytes and
+ * relative to the first element of each view. */
+void orc_relayout(
+        const void* src, int snd, const int64_t* sdims, const int64_t* sstr, void* dst, int dnd,
+        const int64_t* ddims, const int64_t* dstr, int es) {
+    int64_t sidx[8] = {0}, didx[8] = {0};
+    int64_t total = 1;
+    for (int i = 0; i < snd; ++i)
+        total *= sdims[i];
+    int64_t so = 0, doff = 0;
+    for (int64_t k = 0; k < total; ++k) {
+        memcpy((char*)dst + doff * es, (const char*)src + so * es, (size_t)es);
+        for (int i = snd - 1; i >= 0; --i) {
+            if (++sidx[i] < sdims[i]) {
+                so += sstr[i];
+                break;
+            }
+            sidx[i] = 0;
+            so -= (sdims[i] - 1) * sstr[i];
+        }
+        for (int i = dnd - 1; i >= 0; --i) {
+            if (++didx[i] < ddims[i]) {
+                doff += dstr[i];
+                break;
+            }
+            didx[i] = 0;
+            doff -= (ddims[i] - 1) * dstr[i];
+        }
+    }
+}
+
+/* Concat of dense tensors, BareMetal/Concat.cpp:35-61: input i, viewed as [outer, len_i * inner],
+ * lands in the output [outer, sum(len) * inner] at column (len of the inputs before it) * inner. */
+void orc_concat(
+        const void* const* srcs, const int64_t* lens, int nr, void* dst, int64_t outer,
+        int64_t inner, int es) {
+    int64_t all = 0;
+    for (int i = 0; i < nr; ++i)
+        all += lens[i];
+    int64_t at = 0;
+    for (int i = 0; i < nr; ++i) {
+        for (int64_t o = 0; o < outer; ++o)
+            for (int64_t j = 0; j < lens[i] * inner; ++j)
+                memcpy((char*)dst + ((o * all + at) * inner + j) * es,
+                       (const char*)srcs[i] + (o * lens[i] * inner + j) * es, (size_t)es);
+        at += lens[i];
+    }
+}

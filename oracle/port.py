@@ -160,3 +160,29 @@ def reduce_f32(src, mode, axis):
     dst = np.empty(shape, np.float32)
     lib().orc_reduce_f32(_p(src), _p(dst), mode, a, b, c)
     return dst
+
+
+def relayout(src, src_off, src_shape, src_strides, dst, dst_off, dst_shape, dst_strides):
+    """dst view <- src view; `src`/`dst` are flat-able dense arrays, offsets/strides count
+    elements. Writes into `dst` in place."""
+    assert src.dtype == dst.dtype and src.flags["C_CONTIGUOUS"] and dst.flags["C_CONTIGUOUS"]
+    i64 = lambda v: np.ascontiguousarray(v, dtype=np.int64)
+    sd, ss, dd, ds = i64(src_shape), i64(src_strides), i64(dst_shape), i64(dst_strides)
+    es = src.itemsize
+    lib().orc_relayout(
+        C.c_void_p(src.ctypes.data + src_off * es), len(sd), _p(sd), _p(ss),
+        C.c_void_p(dst.ctypes.data + dst_off * es), len(dd), _p(dd), _p(ds), es)
+
+
+def concat(arrays, axis):
+    shape = list(arrays[0].shape)
+    shape[axis] = sum(a.shape[axis] for a in arrays)
+    dst = np.empty(shape, arrays[0].dtype)
+    outer = int(np.prod(shape[:axis], dtype=np.int64))
+    inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    arrays = [np.ascontiguousarray(a) for a in arrays]
+    ptrs = (C.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+    lens = np.array([a.shape[axis] for a in arrays], np.int64)
+    lib().orc_concat(ptrs, _p(lens), len(arrays), _p(dst), C.c_int64(outer), C.c_int64(inner),
+                     dst.itemsize)
+    return dst

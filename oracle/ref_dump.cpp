@@ -42,6 +42,8 @@ static const std::map<std::string, KT> kTypes = {
         {"MatrixMulKernel", KT::MatrixMulKernel},
         {"ReduceKernel", KT::ReduceKernel},
         {"TypeCvtKernel", KT::TypeCvtKernel},
+        {"RelayoutKernel", KT::RelayoutKernel},
+        {"ConcatKernel", KT::ConcatKernel},
 };
 
 static CCOperand parse_operand(const std::string& v) {

@@ -31,15 +31,21 @@ def _op(shape, dtype, scale=None):
 
 
 class TensorSpec:
-    """name, numpy array (inputs) or shape (outputs), TinyNN dtype enum, scale"""
+    """name, numpy array (inputs) or shape (outputs), TinyNN dtype enum, scale.
+    A strided view is given by `strides` and `offset` (elements; offset = where the view's first
+    element lies) into a dense buffer: `array` itself for an input, a buffer of shape `storage`
+    for an output (the whole buffer comes back as the result)."""
 
-    def __init__(self, name, shape, type_enum, scale=1.0, array=None):
+    def __init__(self, name, shape, type_enum, scale=1.0, array=None, strides=None, offset=0,
+                 storage=None):
         self.name, self.shape, self.type_enum, self.scale, self.array = (
             name, tuple(shape), type_enum, scale, array)
+        self.strides, self.offset = strides, offset
+        self.storage = tuple(storage) if storage is not None else self.shape
 
     @property
     def nbytes(self):
-        return int(np.prod(self.shape, dtype=np.int64)) * abi.np_dtype(self.type_enum).itemsize
+        return int(np.prod(self.storage, dtype=np.int64)) * abi.np_dtype(self.type_enum).itemsize
 
 
 class ConvCase:
@@ -358,13 +364,172 @@ class MatMulCase:
         return port.matmul_f32(arrays["a"], arrays["b"], self.trans_a, self.trans_b)
 
 
-def run_ref(case, arrays):
+POISON = 0x5A  # byte every output buffer holds before a kernel runs
+
+
+def poisoned(shape, dtype):
+    return np.full(int(np.prod(shape, dtype=np.int64)) * np.dtype(dtype).itemsize, POISON,
+                   np.uint8).view(dtype).reshape(shape)
+
+
+DTYPES = {"f32": (abi.FLOAT, np.float32), "qsi8": (abi.QINT8, np.int8),
+          "qsi32": (abi.QINT32, np.int32)}
+
+
+def dense_strides(shape):
+    st, s = [], 1
+    for d in reversed(shape):
+        st.append(s)
+        s *= int(d)
+    return tuple(reversed(st))
+
+
+def view_of(buf, shape, strides, offset):
+    """numpy view of the flat array `buf`: element strides, first element at `offset`"""
+    return np.lib.stride_tricks.as_strided(
+        buf.reshape(-1)[offset:], shape, [s * buf.itemsize for s in strides], writeable=True)
+
+
+def span_of(shape, strides):
+    """(lowest, highest) element offset a view touches relative to its first element"""
+    lo = sum((d - 1) * s for d, s in zip(shape, strides) if s < 0)
+    hi = sum((d - 1) * s for d, s in zip(shape, strides) if s > 0)
+    return lo, hi
+
+
+class RelayoutCase:
+    """dst view <- src view, both strided views (element strides, None = dense) over dense
+    buffers sized to the views' spans (+ `slack` untouched elements either side)."""
+
+    def __init__(self, dtype, src_shape, src_strides=None, dst_shape=None, dst_strides=None,
+                 slack=3):
+        self.dtype = dtype
+        self.src_shape = tuple(src_shape)
+        self.dst_shape = tuple(dst_shape) if dst_shape is not None else self.src_shape
+        self.src_strides = tuple(src_strides) if src_strides is not None else None
+        self.dst_strides = tuple(dst_strides) if dst_strides is not None else None
+        self.slack = slack
+
+    def __repr__(self):
+        return "relayout_%s%s_%s%s_to_%s%s" % (
+            self.dtype, "" if self.slack == 3 else "_slack%d" % self.slack, "x".join(map(str, self.src_shape)),
+            "" if self.src_strides is None else "s" + ".".join(map(str, self.src_strides)),
+            "x".join(map(str, self.dst_shape)),
+            "" if self.dst_strides is None else "s" + ".".join(map(str, self.dst_strides)))
+
+    def symbol(self):
+        # (GeneralIntrinsic/Relayout.cpp:43-48 comes first in the registry's candidate list;
+        #  BareMetal's kernel_relayout_<dtype> is the same operator)
+        return "GI_kernel_relayout_" + self.dtype
+
+    def spec_line(self):
+        sc = None if self.dtype == "f32" else 0.05
+        return "RelayoutKernel operand:0=%s operand:1=%s" % (
+            _op(self.src_shape, self.dtype, sc), _op(self.dst_shape, self.dtype, sc))
+
+    def _place(self, shape, strides):
+        """(strides, offset, storage elements) of a view inside its buffer"""
+        if strides is None:
+            return None, 0, int(np.prod(shape, dtype=np.int64))
+        lo, hi = span_of(shape, strides)
+        return strides, self.slack - lo, hi - lo + 1 + 2 * self.slack
+
+    def gen(self, seed=0):
+        r = rng(seed)
+        _, _, n = self._place(self.src_shape, self.src_strides)
+        np_dt = DTYPES[self.dtype][1]
+        if self.dtype == "f32":
+            src = r.standard_normal(n).astype(np.float32)
+        else:
+            info = np.iinfo(np_dt)
+            src = r.integers(info.min, info.max, n, endpoint=True).astype(np_dt)
+        return {"src": src}
+
+    def specs(self, arrays):
+        te = DTYPES[self.dtype][0]
+        sc = 1.0 if self.dtype == "f32" else 0.05
+        ss, so, _ = self._place(self.src_shape, self.src_strides)
+        ds, do, dn = self._place(self.dst_shape, self.dst_strides)
+        return ([TensorSpec(b"src", self.src_shape, te, sc, arrays["src"], ss, so)],
+                [TensorSpec(b"dst", self.dst_shape, te, sc, None, ds, do,
+                            storage=(dn,) if ds is not None else None)])
+
+    def run_port(self, arrays):
+        ss, so, _ = self._place(self.src_shape, self.src_strides)
+        ds, do, dn = self._place(self.dst_shape, self.dst_strides)
+        np_dt = DTYPES[self.dtype][1]
+        if ds is None:
+            out = np.zeros(self.dst_shape, np_dt)
+            port.relayout(arrays["src"], so, self.src_shape, ss or dense_strides(self.src_shape),
+                          out, 0, self.dst_shape, dense_strides(self.dst_shape))
+            return out
+        out = poisoned((dn,), np_dt)
+        port.relayout(arrays["src"], so, self.src_shape, ss or dense_strides(self.src_shape),
+                      out, do, self.dst_shape, ds)
+        return out
+
+
+class ConcatCase:
+    """dense inputs of `shapes` joined along `axis`"""
+
+    def __init__(self, dtype, shapes, axis):
+        self.dtype, self.shapes, self.axis = dtype, [tuple(s) for s in shapes], axis
+
+    def __repr__(self):
+        return "concat_%s_a%d_%s" % (self.dtype, self.axis,
+                                     "_".join("x".join(map(str, s)) for s in self.shapes))
+
+    def out_shape(self):
+        o = list(self.shapes[0])
+        o[self.axis] = sum(s[self.axis] for s in self.shapes)
+        return tuple(o)
+
+    def symbol(self):
+        return "kernel_concat_byte_%d_axis_%d" % (np.dtype(DTYPES[self.dtype][1]).itemsize,
+                                                  self.axis)
+
+    def spec_line(self):
+        sc = None if self.dtype == "f32" else 0.05
+        ops = ["operand:%d=%s" % (i, _op(s, self.dtype, sc)) for i, s in enumerate(self.shapes)]
+        ops.append("operand:%d=%s" % (len(self.shapes), _op(self.out_shape(), self.dtype, sc)))
+        return "ConcatKernel axis=i:%d nr_operands=i:%d %s" % (
+            self.axis, len(self.shapes) + 1, " ".join(ops))
+
+    def gen(self, seed=0):
+        r = rng(seed)
+        np_dt = DTYPES[self.dtype][1]
+        out = {}
+        for i, s in enumerate(self.shapes):
+            if self.dtype == "f32":
+                out["in%d" % i] = r.standard_normal(s).astype(np.float32)
+            else:
+                info = np.iinfo(np_dt)
+                out["in%d" % i] = r.integers(info.min, info.max, s, endpoint=True).astype(np_dt)
+        return out
+
+    def specs(self, arrays):
+        te = DTYPES[self.dtype][0]
+        sc = 1.0 if self.dtype == "f32" else 0.05
+        ins = [TensorSpec(b"in%d" % i, s, te, sc, arrays["in%d" % i])
+               for i, s in enumerate(self.shapes)]
+        return ins, [TensorSpec(b"dst", self.out_shape(), te, sc)]
+
+    def run_port(self, arrays):
+        return port.concat([arrays["in%d" % i] for i in range(len(self.shapes))], self.axis)
+
+
+def run_ref(case, arrays, symbol=None):
     """Evaluate `case` with the reference's generated C kernel; returns the output array."""
     ins, outs = case.specs(arrays)
-    out_arr = np.zeros(outs[0].shape, abi.np_dtype(outs[0].type_enum))
-    tin = [abi.host_tensor(s.array, s.type_enum, s.scale, s.name) for s in ins]
-    tout = [abi.host_tensor(out_arr, outs[0].type_enum, outs[0].scale, outs[0].name)]
-    ref.run(case.symbol(), tin, tout)
+    o = outs[0]
+    strided = o.strides is not None
+    out_arr = (poisoned if strided else np.zeros)(o.storage, abi.np_dtype(o.type_enum))
+    tin = [abi.host_tensor(s.array, s.type_enum, s.scale, s.name,
+                           s.shape if s.strides is not None else None, s.strides, s.offset)
+           for s in ins]
+    tout = [abi.host_tensor(out_arr, o.type_enum, o.scale, o.name, o.shape if strided else None,
+                            o.strides, o.offset)]
+    ref.run(symbol or case.symbol(), tin, tout)
     return out_arr
 
 

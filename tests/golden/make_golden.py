@@ -35,11 +35,7 @@ def main():
     for idx, (name, case) in enumerate(golden_cases().items()):
         arrays = case.gen(seed=1000 + idx)
         sym = manifest[name]
-        ins, outs = case.specs(arrays)
-        out = np.zeros(outs[0].shape, cases.abi.np_dtype(outs[0].type_enum))
-        tin = [cases.abi.host_tensor(s.array, s.type_enum, s.scale, s.name) for s in ins]
-        tout = [cases.abi.host_tensor(out, outs[0].type_enum, outs[0].scale, outs[0].name)]
-        ref.run(sym, tin, tout)
+        out = cases.run_ref(case, arrays, sym)
         for k, v in arrays.items():
             if v is not None:
                 blobs["%s/%s" % (name, k)] = v

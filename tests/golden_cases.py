@@ -4,7 +4,8 @@ tests/golden/make_golden.py). Shapes follow the reference's own kernel tests
 typecvt.cpp:5-70): odd sizes, k in {1,3}, stride in {1,2}, pad in {0,k/2}, every activation, the
 small-magnitude tie case and the 30..50 overflow case."""
 from megcc_amd import abi
-from cases import ConvCase, MatMulCase, MultiTypeCase, PoolCase, TypeCvtCase
+from cases import (ConcatCase, ConvCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
+                   TypeCvtCase)
 
 A = abi
 
@@ -87,4 +88,39 @@ def golden_cases():
     c["cvt_q8_f32"] = TypeCvtCase("qsi8", "f32", (3, 37), src_scale=0.05)
     c["cvt_q8_q8"] = TypeCvtCase("qsi8", "qsi8", (3, 37), src_scale=0.05, dst_scale=0.02)
     c["cvt_q32_q8"] = TypeCvtCase("qsi32", "qsi8", (3, 37), src_scale=0.0002, dst_scale=0.05)
+    # --- relayout: the layouts of compiler/test/kernel/opr/naive/relayout.cpp:7-131 (NCHW <->
+    # NCHW4, negative strides, the transposes of RelayoutFast both ways, a strided destination)
+    for dt in ("f32", "qsi8"):
+        n, ch, hw = 3, 8, 5
+        nchw4_as_nchw = (ch * hw * hw, hw * hw * 4, hw, 1, hw * hw)
+        c["relayout_%s_nchw_to_nchw4" % dt] = RelayoutCase(
+            dt, (n, ch // 4, hw, hw, 4), nchw4_as_nchw)
+        c["relayout_%s_nchw4_to_nchw" % dt] = RelayoutCase(
+            dt, (n, ch // 4, hw, hw, 4), None, None, nchw4_as_nchw)
+        c["relayout_%s_neg_w" % dt] = RelayoutCase(dt, (1, 2, 3, 4), (24, 12, 4, -1))
+        c["relayout_%s_neg_h" % dt] = RelayoutCase(dt, (1, 2, 3, 4), (24, 12, -4, 1))
+        n, ch, h, w = 2, 8, 2, 3
+        fast = [
+            ((n, h, w, ch), (ch * h * w, w, 1, h * w), (n, ch, h, w)),
+            ((n, ch, h, w), (ch * h * w, 1, ch * w, ch), (n, h, w, ch)),
+            ((n, ch // 4, h, w, 4), (ch * h * w, h * w * 4, w, 1, h * w), (n, ch // 4, 4, h, w)),
+            ((n, ch // 4, 4, h, w), (ch * h * w, h * w * 4, 1, w * 4, 4), (n, ch // 4, h, w, 4)),
+        ]
+        for i, (shape, strides, other) in enumerate(fast):
+            c["relayout_%s_fast%d" % (dt, i)] = RelayoutCase(dt, shape, strides, other)
+            c["relayout_%s_fast%d_back" % (dt, i)] = RelayoutCase(dt, other, None, shape, strides)
+        c["relayout_%s_into_slice" % dt] = RelayoutCase(
+            dt, (n, ch, h, w), None, None, (ch * 3 * h * w, 3 * h * w, w, 1))
+        c["relayout_%s_step2" % dt] = RelayoutCase(dt, (3, 5, 7), (140, 14, 2), None, (70, 7, 1))
+        c["relayout_%s_views" % dt] = RelayoutCase(dt, (6, 4), (9, 2), (2, 12), (31, 2))
+        c["relayout_%s_broadcast" % dt] = RelayoutCase(dt, (4, 5, 6), (6, 0, 1))
+    # --- concat: compiler/test/kernel/opr/naive/concat.cpp:5-28 (4 inputs, extent i+1 along axis)
+    for dt in ("f32", "qsi8"):
+        for axis in range(4):
+            shapes = []
+            for i in range(4):
+                sh = [3, 4, 5, 6]
+                sh[axis] = i + 1
+                shapes.append(tuple(sh))
+            c["concat_%s_axis%d" % (dt, axis)] = ConcatCase(dt, shapes, axis)
     return c

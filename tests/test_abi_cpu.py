@@ -44,7 +44,7 @@ with open(os.path.join(HERE, "golden", "symbols.json")) as f:
 @pytest.mark.parametrize("symbol", sorted(set(SYMBOLS.values())))
 def test_every_reference_symbol_parses(symbol):
     desc = runtime.parse_symbol(symbol)
-    assert desc.kind in range(1, 8)
+    assert desc.kind in range(1, 10)
 
 
 def test_parse_conv_symbol_fields():
@@ -78,11 +78,42 @@ def test_parse_other_symbols():
     assert d.kind == abi.KERN_MATMUL and d.attr.matmul.transpose_b == 0
     d = runtime.parse_symbol("GI_kernel_fp32_matmul_4x12_nt")
     assert d.attr.matmul.transpose_b == 1
+    for sym in ("kernel_relayout_f32", "GI_kernel_relayout_qsi8", "kernel_relayout_ui8"):
+        assert runtime.parse_symbol(sym).kind == abi.KERN_RELAYOUT
+    d = runtime.parse_symbol("kernel_concat_byte_4_axis_2")
+    assert d.kind == abi.KERN_CONCAT and d.attr.concat_axis == 2
+
+
+def test_copy_kernels_reject_bad_arguments_before_any_launch():
+    """the checks of Relayout / Concat need no GPU: nothing is launched on a mismatch"""
+    L = runtime.lib()
+    fake = 0x1000  # never dereferenced
+    t = lambda shape, te=abi.FLOAT, strides=None: abi.make_tensor(fake, shape, te, strides=strides)
+    call = lambda fn, ins, out, *pre: fn(*pre, abi.tensor_array(ins), len(ins),
+                                         abi.tensor_array([out]), 1, None, None)
+    assert call(L.megcc_gfx950_relayout, [t((2, 3))], t((2, 3), abi.QINT8)) == \
+        abi.ERROR_UNSUPPORTED_DTYPE_TYPE
+    assert call(L.megcc_gfx950_relayout, [t((2, 3))], t((2, 4))) == abi.ERROR_INVALID_LAYOUT
+    assert call(L.megcc_gfx950_relayout, [t((2, 3))], t((2, 3), strides=(0, 1))) == \
+        abi.ERROR_INVALID_LAYOUT  # two rows written to the same place
+    assert call(L.megcc_gfx950_relayout, [t((0, 3))], t((0, 3))) == 0  # empty: nothing to do
+    axis = C.c_int(1)
+    assert call(L.megcc_gfx950_concat, [t((2, 3)), t((2, 4))], t((2, 8)), C.byref(axis)) == \
+        abi.ERROR_INVALID_LAYOUT
+    assert call(L.megcc_gfx950_concat, [t((2, 3)), t((3, 4))], t((2, 7)), C.byref(axis)) == \
+        abi.ERROR_INVALID_LAYOUT
+    assert call(L.megcc_gfx950_concat, [t((2, 3)), t((2, 4), abi.QINT8)], t((2, 7)),
+                C.byref(axis)) == abi.ERROR_UNSUPPORTED_DTYPE_TYPE
+    axis = C.c_int(2)
+    assert call(L.megcc_gfx950_concat, [t((2, 3))], t((2, 3)), C.byref(axis)) == \
+        abi.ERROR_OUT_OF_RANGE
+    assert L.megcc_gfx950_concat(None, None, 0, None, 0, None, None) == abi.ERROR_NULL_PTR
 
 
 def test_unknown_symbol_is_reported_not_guessed():
     desc = abi.KernelDesc()
-    for bad in ("kernel_argsort_f32", "kernel_conv2d_3x3_NHWC_DENSE_p1x1_s1x1_d1x1_f32f32f32",
+    for bad in ("kernel_argsort_f32", "kernel_relayout_f64", "kernel_concat_byte_8_axis_0",
+                "kernel_concat_byte_4_axis_1x", "kernel_conv2d_3x3_NHWC_DENSE_p1x1_s1x1_d1x1_f32f32f32",
                 "kernel_typecvt_f16f32", ""):
         st = runtime.lib().megcc_gfx950_parse_symbol(bad.encode(), C.byref(desc))
         assert st == abi.ERROR_NO_FOUND

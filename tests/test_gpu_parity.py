@@ -10,7 +10,8 @@ import numpy as np
 import pytest
 
 import cases
-from cases import ConvCase, MatMulCase, MultiTypeCase, PoolCase, TypeCvtCase
+from cases import (ConcatCase, ConvCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
+                   TypeCvtCase)
 from golden_cases import golden_cases, unsat
 from megcc_amd import abi, runtime
 from oracle import port
@@ -141,6 +142,40 @@ LIVE = [
     TypeCvtCase("qsi8", "f32", (64, 1000), src_scale=0.0173),
     TypeCvtCase("qsi8", "qsi8", (5, 1001), src_scale=0.0173, dst_scale=0.0291),
     TypeCvtCase("qsi32", "qsi8", (5, 1001), src_scale=0.0002, dst_scale=0.05),
+    # relayout: NCHW <-> NCHW4 at a model's size, plain and batched transposes, every permutation
+    # class of a 4-d tensor, ragged tiles, views with negative / zero / non-unit strides, rows
+    # that can and cannot be widened to 16-byte elements
+    RelayoutCase("qsi8", (8, 16, 56, 56, 4), (64 * 3136, 4 * 3136, 56, 1, 3136)),
+    RelayoutCase("qsi8", (8, 16, 56, 56, 4), None, None, (64 * 3136, 4 * 3136, 56, 1, 3136)),
+    RelayoutCase("f32", (4, 8, 28, 28, 4), (32 * 784, 4 * 784, 28, 1, 784)),
+    RelayoutCase("f32", (1000, 1023), (1, 1000)),
+    RelayoutCase("f32", (1023, 1000), None, None, (1, 1023)),
+    RelayoutCase("qsi8", (3, 517, 259), (517 * 259, 1, 517)),
+    RelayoutCase("qsi32", (5, 70, 3, 66), (70 * 3 * 66, 1, 70 * 66, 70)),
+    RelayoutCase("f32", (6, 10, 14, 18), (1, 6, 60, 840)),
+    RelayoutCase("f32", (6, 10, 14, 18), (18, 108, 1080, 1)),
+    RelayoutCase("qsi8", (6, 10, 14, 18), (140, 14, 1, 840)),
+    RelayoutCase("qsi8", (2, 3, 1, 2, 3, 2, 5), (180, 5, 7, 30, 60, 15, 1)),
+    RelayoutCase("f32", (7, 9, 33), (9 * 33, -33, 1)),
+    RelayoutCase("qsi8", (7, 9, 33), (9 * 33, 33, -1)),
+    RelayoutCase("f32", (40, 50), (-50, -1), None, (1, 40)),
+    RelayoutCase("f32", (16, 3, 64), (64, 0, 1)),
+    RelayoutCase("qsi8", (5, 1000), (0, 1)),
+    RelayoutCase("qsi8", (64, 4096), (8192, 1), slack=0),
+    RelayoutCase("qsi8", (64, 4096), (8192, 1), slack=5),
+    RelayoutCase("qsi8", (64, 4090), (8190, 1), slack=0),
+    RelayoutCase("f32", (32, 100, 64), None, None, (100 * 192, 192, 1), slack=4),
+    RelayoutCase("f32", (32, 100, 64), (2 * 6400, 2 * 64, 2), None, (7000, 70, 1)),
+    RelayoutCase("qsi8", (60, 40), (90, 2), (20, 120), (310, 2)),
+    RelayoutCase("f32", (1, 1, 1), None),
+    RelayoutCase("f32", (2, 3, 1, 5), (1, 2, 77, 6)),
+    # concat: compiler/test/kernel/opr/naive/concat.cpp:5-28 and the channel join of NCHW44 maps
+    ConcatCase("f32", [(12, 13, i + 1, 15) for i in range(4)], 2),
+    ConcatCase("qsi8", [(12, i + 1, 14, 15) for i in range(4)], 1),
+    ConcatCase("qsi8", [(i + 1, 13, 14, 15) for i in range(4)], 0),
+    ConcatCase("qsi32", [(12, 13, 14, i + 1) for i in range(4)], 3),
+    ConcatCase("qsi8", [(8, 16, 28, 28, 4), (8, 8, 28, 28, 4), (8, 24, 28, 28, 4)], 1),
+    ConcatCase("f32", [(64, 1000)], 1),
     # f32
     ConvCase(A.FMT_NCHW, A.DENSE, 1, 32, 56, 56, 32, 3, 1, 1, A.RELU, dtype="f32"),
     ConvCase(A.FMT_NCHW, A.DENSE, 2, 5, 19, 23, 37, 3, 2, 1, A.IDENTITY, dtype="f32"),

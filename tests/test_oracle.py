@@ -101,6 +101,46 @@ def test_port_matches_reference_live(case):
 
 
 # ---- checks that do not involve the reference at all ----------------------------------------
+@pytest.mark.parametrize("name", sorted(n for n in CASES if n.startswith("relayout_")))
+def test_port_relayout_vs_numpy_views(name):
+    """numpy's own strided views (as_strided + reshape) define the same copy"""
+    case = CASES[name]
+    arrays = case.gen(3)
+    ins, outs = case.specs(arrays)
+    s, o = ins[0], outs[0]
+    src_view = cases.view_of(arrays["src"], s.shape, s.strides or cases.dense_strides(s.shape),
+                             s.offset)
+    want = cases.poisoned(o.storage, arrays["src"].dtype) if o.strides else \
+        np.zeros(o.storage, arrays["src"].dtype)
+    dst_view = cases.view_of(want, o.shape, o.strides or cases.dense_strides(o.shape), o.offset)
+    dst_view[...] = np.ascontiguousarray(src_view).reshape(o.shape)
+    np.testing.assert_array_equal(case.run_port(arrays), want)
+
+
+def test_port_relayout_known_answers():
+    """transpose, flip and NCHW -> NCHW4 written with numpy's own operators"""
+    x = np.arange(2 * 8 * 3 * 5, dtype=np.int32).reshape(2, 8, 3, 5)
+    out = np.zeros((2, 2, 3, 5, 4), np.int32)
+    port.relayout(x, 0, (2, 2, 3, 5, 4), (120, 60, 5, 1, 15), out, 0, out.shape,
+                  cases.dense_strides(out.shape))
+    np.testing.assert_array_equal(out, x.reshape(2, 2, 4, 3, 5).transpose(0, 1, 3, 4, 2))
+    m = np.arange(35, dtype=np.int8).reshape(5, 7)
+    out = np.zeros((7, 5), np.int8)
+    port.relayout(m, 0, (7, 5), (1, 7), out, 0, (7, 5), (5, 1))
+    np.testing.assert_array_equal(out, m.T)
+    out = np.zeros((5, 7), np.int8)
+    port.relayout(m, 6, (5, 7), (7, -1), out, 0, (5, 7), (7, 1))
+    np.testing.assert_array_equal(out, m[:, ::-1])
+
+
+@pytest.mark.parametrize("name", sorted(n for n in CASES if n.startswith("concat_")))
+def test_port_concat_vs_numpy(name):
+    case = CASES[name]
+    arrays = case.gen(3)
+    want = np.concatenate([arrays["in%d" % i] for i in range(len(case.shapes))], case.axis)
+    np.testing.assert_array_equal(case.run_port(arrays), want)
+
+
 def _acc_numpy_nchw44_dense(src, flt, bias, pad, stride):
     """exact int64 correlation, written against the layout definition (not the port's loops)"""
     n, c4, ih, iw, _ = src.shape

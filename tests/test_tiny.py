@@ -140,3 +140,81 @@ def test_loader_refuses_what_it_cannot_run():
         runtime.Model.load(tiny.write_model(d))
     with pytest.raises(runtime.MegccError, match="model_load"):
         runtime.Model.load(small_bytes()[:100])
+
+
+# ---- strided views (SUBTENSOR / DIMSHUFFLE MemForward) + Relayout + Concat ----------------------
+def test_view_file_carries_strides_and_byte_offsets():
+    b = tiny.ModelBuilder("views")
+    net = tiny_cases.ViewNet()
+    ids = net.build(b)
+    text = runtime.tiny_describe(b.to_bytes())
+    lines = text.splitlines()
+    view = [l for l in lines if "name=image.as_nchw4" in l][0]
+    assert "dims=[2,2,6,6,4]" in view and "stride=[288,144,6,1,36]" in view
+    tail = [l for l in lines if "name=cat.tail" in l][0]
+    assert "stride=[144,36,12,4,1]" in tail
+    fwd = [l for l in lines if " MemForward " in l]
+    assert len(fwd) == 2 and "offset=0" in fwd[0] and "offset=72" in fwd[1]
+    assert ids["out"] == 7
+
+
+@pytest.mark.skipif(not ref.tiny_dump_available(), reason="oracle/_ref not built (needs the reference tree)")
+def test_view_file_reads_the_same_with_the_reference_reader(tmp_path):
+    b = tiny.ModelBuilder("views")
+    tiny_cases.ViewNet().build(b)
+    path = tmp_path / "views.tiny"
+    path.write_bytes(b.to_bytes())
+    assert runtime.tiny_describe(b.to_bytes()) == ref.tiny_dump(str(path))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("how", ["built", "loaded"])
+def test_views_relayout_and_concat_inside_a_model(how):
+    net = tiny_cases.ViewNet()
+    if how == "built":
+        model = runtime.Model()
+        ids = net.build(model)
+    else:
+        b = tiny.ModelBuilder("views")
+        ids = net.build(b)
+        half = (net.N, net.C // 4, net.H // 2, net.W // 2, 4)
+        both = (net.N, net.C // 2, net.H // 2, net.W // 2, 4)
+        model = runtime.Model.load(b.to_bytes(), {
+            ids["image"]: ((net.N, net.C, net.H, net.W), abi.QINT8),
+            ids["cat"]: (both, abi.QINT8), ids["out"]: (half, abi.QINT8)})
+    assert model.nr_opr == 5
+    for seed in (1, 2, 3):  # eager, captured, replayed
+        image = net.draw_input(seed)
+        cat, out = net.run_oracle(image)
+        model.set_input(ids["image"], image)
+        model.forward()
+        assert np.array_equal(model.get(ids["cat"]), cat)
+        assert np.array_equal(model.get(ids["out"]), out)
+    model.close()
+
+
+@pytest.mark.gpu
+def test_views_that_leave_their_tensor_are_refused():
+    m = runtime.Model()
+    x = m.tensor("x", (4, 6), abi.QINT8, 0.05)
+    m.view("ok", x, (6, 4), (1, 6))
+    m.view("ok.reversed", x, (4, 6), (6, -1), offset=5)
+    with pytest.raises(runtime.MegccError, match="leaves"):
+        m.view("long", x, (4, 7), (6, 1))
+    with pytest.raises(runtime.MegccError, match="leaves"):
+        m.view("before", x, (4, 6), (6, -1), offset=4)
+    m.close()
+    b = tiny.ModelBuilder("bad")
+    x = b.tensor("x", (4, 6), abi.QINT8, 0.05)
+    b.mark_input(x)
+    v = b.view("long", x, (4, 7), (6, 1))
+    y = b.tensor("y", (4, 7), abi.QINT8, 0.05)
+    b.opr("kernel_relayout_qsi8", [v], [y])
+    b.mark_output(y)
+    with pytest.raises(runtime.MegccError, match="views bytes 0..25 of tensor 0"):
+        runtime.Model.load(b.to_bytes())
+    d = b.to_dict()
+    d["device_models"][0]["tensors"][2]["stride"] = [1, 4]  # an owning tensor must be dense
+    d["device_models"][0]["tensors"][1]["dims"] = [4, 6]
+    with pytest.raises(runtime.MegccError, match="not dense"):
+        runtime.Model.load(tiny.write_model(d))

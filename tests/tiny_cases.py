@@ -46,3 +46,63 @@ def small_model():
                   instructions=instructions[:1], inputs=[0], outputs=[1])
     return dict(name="small", model_id=0x1234567890abcdef, const_shape=False, weights=weights,
                 device_models=[first, second])
+
+
+class ViewNet:
+    """A network that needs strided views: an NCHW qsi8 image is read through a DIMSHUFFLE view
+    as [N, C/4, H, W, 4] and made dense by Relayout (how an NCHW model enters NCHW44 kernels),
+    max- and average-pooled, the two results joined by Concat along the channel blocks, and the
+    last two blocks taken out again through a SUBTENSOR view + Relayout."""
+    N, C, H, W = 2, 8, 6, 6
+    SCALE = 0.05
+
+    def __init__(self):
+        from cases import PoolCase
+        from megcc_amd import abi
+        self.pool_max = PoolCase(abi.FMT_NCHW44, abi.POOL_MAX, self.N, self.C, self.H, self.W,
+                                 2, 2, 0, scale=self.SCALE)
+        self.pool_avg = PoolCase(abi.FMT_NCHW44, abi.POOL_AVERAGE, self.N, self.C, self.H, self.W,
+                                 2, 2, 0, scale=self.SCALE)
+
+    def build(self, m):
+        """m: runtime.Model or tiny.ModelBuilder"""
+        from megcc_amd import abi
+        n, c, h, w = self.N, self.C, self.H, self.W
+        q = lambda name, shape: m.tensor(name, shape, abi.QINT8, self.SCALE)
+        ids = {}
+        ids["image"] = q("image", (n, c, h, w))
+        m.mark_input(ids["image"])
+        blocked = (n, c // 4, h, w, 4)
+        v = m.view("image.as_nchw4", ids["image"], blocked, (c * h * w, 4 * h * w, w, 1, h * w))
+        ids["x4"] = q("x4", blocked)
+        m.opr("GI_kernel_relayout_qsi8", [v], [ids["x4"]])
+        half = (n, c // 4, h // 2, w // 2, 4)
+        ids["max"], ids["avg"] = q("max", half), q("avg", half)
+        m.opr(self.pool_max.symbol(), [ids["x4"]], [ids["max"]])
+        m.opr(self.pool_avg.symbol(), [ids["x4"]], [ids["avg"]])
+        both = (n, c // 2, h // 2, w // 2, 4)
+        ids["cat"] = q("cat", both)
+        m.opr("kernel_concat_byte_1_axis_1", [ids["max"], ids["avg"]], [ids["cat"]])
+        plane = (h // 2) * (w // 2) * 4
+        tail = m.view("cat.tail", ids["cat"], half,
+                      (c // 2 * plane, plane, (w // 2) * 4, 4, 1), offset=(c // 4) * plane)
+        ids["out"] = q("out", half)
+        m.opr("GI_kernel_relayout_qsi8", [tail], [ids["out"]])
+        m.mark_output(ids["cat"])
+        m.mark_output(ids["out"])
+        m.finalize()
+        return ids
+
+    def draw_input(self, seed):
+        return np.random.default_rng(seed).integers(
+            -128, 128, (self.N, self.C, self.H, self.W)).astype(np.int8)
+
+    def run_oracle(self, image):
+        """-> (cat, out), from the pooling port and numpy's own transpose / concatenate"""
+        from oracle import port
+        n, c, h, w = image.shape
+        x4 = np.ascontiguousarray(image.reshape(n, c // 4, 4, h, w).transpose(0, 1, 3, 4, 2))
+        a = self.pool_max.run_port({"src": x4})
+        b = self.pool_avg.run_port({"src": x4})
+        cat = np.concatenate([a, b], 1)
+        return cat, np.ascontiguousarray(cat[:, c // 4:])

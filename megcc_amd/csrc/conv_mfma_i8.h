@@ -152,12 +152,22 @@ __device__ __forceinline__ void dma_buffer_b32(v4u rsrc, unsigned voffset, unsig
                  : "memory");
 }
 
+// 16 bytes per lane from a raw buffer straight into LDS (64 lanes -> 1 KB at lds_addr); offsets at
+// or beyond num_records read as zero
+__device__ __forceinline__ void dma_buffer_b128(v4u rsrc, unsigned voffset, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds"
+                 :
+                 : "v"(voffset), "s"(rsrc), "s"(__builtin_amdgcn_readfirstlane(lds_addr))
+                 : "memory");
+}
+
 struct PipeConfig {
     int bm, bn, ks, maxb, blocks_per_cu, threads, a_bytes, g4;
     int gather_threads;  // threads that share the activation gather (maxb items each)
     int nbuf;            // LDS stage buffers
     int extra_lds;       // bytes of LDS beyond the stage buffers
     int fixed_lmax;      // patch slots compiled into the kernel (0: run-time Lmax)
+    int pm = 0;          // plane-major activation patch (virtual rows padded to a multiple of 4)
     const void* kernel;
 };
 

@@ -393,28 +393,30 @@ struct TilePlan {
 };
 
 // largest patch any tile of `bn` pixels needs; mirrors vp_of() / L in the kernels
-static TilePlan plan_tiles_uncached(const ConvGeom& g, int bn, long range_len);
+static TilePlan plan_tiles_uncached(const ConvGeom& g, int bn, long range_len, int pm);
 
 // The plan walks over every tile of the layer: kept per geometry, so that a launch costs the host
 // a map look-up and not a loop over the tensor.
-static TilePlan plan_tiles(const ConvGeom& g, int bn = BN, long range_len = 0) {
+static TilePlan plan_tiles(const ConvGeom& g, int bn = BN, long range_len = 0, int pm = 0) {
     typedef std::array<long, 16> Key;
     static std::map<Key, TilePlan> cache;
     static std::mutex lock;
     const Key key = {g.n, g.ih, g.iw, g.oh, g.ow, g.fh, g.fw, g.sh, g.sw, g.ph, g.pw, g.dh, g.dw,
-                     bn, range_len, 0};
+                     bn, range_len, pm};
     std::lock_guard<std::mutex> guard(lock);
     auto it = cache.find(key);
     if (it != cache.end())
         return it->second;
     if (cache.size() > 4096)
         cache.clear();
-    return cache[key] = plan_tiles_uncached(g, bn, range_len);
+    return cache[key] = plan_tiles_uncached(g, bn, range_len, pm);
 }
 
-static TilePlan plan_tiles_uncached(const ConvGeom& g, int bn, long range_len) {
+// pm: the slot space of the plane-major patch (rows padded on the right only, to a multiple of 4;
+// a patch starts pw slots before its first window, rounded down to 4)
+static TilePlan plan_tiles_uncached(const ConvGeom& g, int bn, long range_len, int pm) {
     TilePlan t;
-    t.VW = g.iw + 2 * g.pw;
+    t.VW = pm ? round_up(g.iw + g.pw, 4) : g.iw + 2 * g.pw;
     t.VH = g.ih + 2 * g.ph;
     long P = (long)g.n * g.oh * g.ow;
     auto vp = [&](long p) {
@@ -430,6 +432,8 @@ static TilePlan plan_tiles_uncached(const ConvGeom& g, int bn, long range_len) {
         long r1 = r0 + range_len < P ? r0 + range_len : P;
         long pl = (p0 + bn < r1 ? p0 + bn : r1) - 1;
         long L = vp(pl) + (long)(g.fh - 1) * g.dh * t.VW + (g.fw - 1) * g.dw - vp(p0) + 1;
+        if (pm)
+            L += (vp(p0) - g.pw) & 3;  // the slots between the rounded-down start and the window
         if (L > lmax)
             lmax = L;
         long rows = (vp(p0) + L - 1) / t.VW - vp(p0) / t.VW + 1;
@@ -503,22 +507,27 @@ TinyNNStatus conv_mfma_launch(
     PipeConfig pc;
     const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;
     const bool b128_ok = ((uintptr_t)src & 15) == 0 && !getenv("MEGCC_NOFCB");
-    // candidates in order of preference; development switches MEGCC_NODMA / MEGCC_NOWS /
-    // MEGCC_NOWIDE skip one
+    // candidates in order of preference; development switches (MEGCC_NO...) skip one
     long range_len = 0;
     TilePlan t;
     bool pipe = false;
-    for (int cand = -1; cand < 3 && !pipe; ++cand) {
+    // DMA kernel variants in order of preference (see conv_mfma_dma_config), then the two older
+    // generations
+    static const int kDmaVariants[] = {2, 3, 0, 4, 1};
+    static const char* const kDmaSwitch[] = {"MEGCC_NOPM768", "MEGCC_NOPM", "MEGCC_NODMA512",
+                                             "MEGCC_NOPM256", "MEGCC_NODMA"};
+    for (int cand = 0; cand < 7 && !pipe; ++cand) {
         bool have = false;
-        if (cand == -1)
-            have = !getenv("MEGCC_NODMA") && !getenv("MEGCC_NODMA512") &&
-                   conv_mfma_dma_config(g, is_fc(g), 0, b128_ok, &pc);
-        else if (cand == 0)
-            have = !getenv("MEGCC_NODMA") && conv_mfma_dma_config(g, is_fc(g), 1, b128_ok, &pc);
-        else if (cand == 1)
+        if (cand < 5) {
+            const int v = kDmaVariants[cand];
+            have = !getenv("MEGCC_NODMA") && !getenv(kDmaSwitch[cand]) &&
+                   !((v == 2 || v == 4) && getenv("MEGCC_NOPM")) &&
+                   conv_mfma_dma_config(g, is_fc(g), v, b128_ok, &pc);
+        } else if (cand == 5) {
             have = !getenv("MEGCC_NOWS") && conv_mfma_ws_config(g, g4_ok, &pc);
-        else
+        } else {
             have = !getenv("MEGCC_NOWIDE") && conv_mfma_pipe_config(g, g4_ok, &pc);
+        }
         if (!have)
             continue;
         // one pixel range per free workgroup slot, so that the whole grid is resident at once and
@@ -530,7 +539,7 @@ TinyNNStatus conv_mfma_launch(
         range_len = ((P + ranges - 1) / ranges + 31) / 32 * 32;
         if (range_len < pc.bn / 2)  // too few pixels per workgroup for the tile
             continue;
-        t = plan_tiles(g, pc.bn, range_len);
+        t = plan_tiles(g, pc.bn, range_len, pc.pm);
         if (pc.fixed_lmax) {
             if (t.Lmax > pc.fixed_lmax)
                 continue;

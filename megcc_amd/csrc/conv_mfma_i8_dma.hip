@@ -45,7 +45,7 @@ static constexpr int ACT_RT = -1;
 // stage together; the eight 16-byte pieces of a row are stored at piece ^ (row & 7) (the load
 // fetches the matching piece), which keeps the MFMA operand reads of 8 consecutive rows on
 // different banks.
-template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT, bool FCB>
+template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT, bool FCB, bool PM>
 __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaParams q) {
     static_assert(!FCB || (FC && KS == 4 && FH * FW == 1), "FCB: FullyConnected, 128 channels per stage");
     constexpr int WGN = 4;
@@ -58,8 +58,10 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     constexpr int A_CHUNKS = A_BYTES / 1024;
     constexpr int A_PER_WAVE = (A_CHUNKS + DM_WAVES - 1) / DM_WAVES;
     constexpr int B_BYTES = KS * 2 * LMAX * 16;
-    constexpr int B_WL = B_BYTES / (FCB ? 1024 : 256);
+    constexpr int B_WL = B_BYTES / (FCB || PM ? 1024 : 256);
     static_assert(B_WL % DM_WAVES == 0 && LMAX % 16 == 0, "whole wave-loads");
+    static_assert(!PM || (!FC && LMAX % 256 == 0), "PM: planes of whole 1 KB wave-loads");
+    constexpr int PM_PARTS = LMAX / 256;  // wave-loads per plane
     static_assert(!FCB || LMAX == 32 * NT * 4, "FCB: one LDS row per pixel of the sub-tile");
     constexpr int B_PER_WAVE = B_WL / DM_WAVES;
     constexpr int LW = LMAX / 16;  // wave-loads per (sub-chunk, half)
@@ -106,6 +108,12 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     // fetches plane (lane & 3) of slot (u % LW) * 16 + (lane >> 2). b_goff = byte offset of that
     // dword in the first plane group of a stage, or 2^31 (out of range -> zero) for padding.
     unsigned b_goff[B_PER_WAVE];
+    // PM: first slot of a sub-tile's patch. Slot space = rows of VW (a multiple of 4) slots per
+    // padded image row, image column x at slot x: the left padding of a row is the tail of the
+    // row before it. The patch starts PW slots before the first pixel's window, rounded down to 4.
+    auto pm_base = [&](int p0) __attribute__((always_inline)) {
+        return (vp_of(q, p0) - q.PW) & ~3;  // (arithmetic: also right below zero)
+    };
     auto describe = [&](int p0) __attribute__((always_inline)) {
         if constexpr (FCB) {
             // wave-load u covers rows 8u .. 8u + 7; rows beyond the matrix repeat the last one
@@ -115,6 +123,27 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
                 const int u = wave + j * DM_WAVES;
                 const int row = min(p0 + u * 8 + (lane >> 3), q.P - 1);
                 b_goff[j] = (unsigned)row * (unsigned)q.image_stride + (((lane & 7) ^ (lane >> 3)) << 4);
+            });
+            return;
+        }
+        if constexpr (PM) {
+            // wave-load u = plane u / PM_PARTS, slots (u % PM_PARTS) * 256 + 4 * lane .. + 3: four
+            // neighbours of one image row (rows are 4-aligned in slot space) or four padding slots
+            const int vbase = pm_base(p0);
+            static_for<B_PER_WAVE>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                const int u = wave + j * DM_WAVES;
+                const int pl = u / PM_PARTS;
+                const int vs = vbase + (u - pl * PM_PARTS) * 256 + lane * 4;
+                unsigned off = 0x80000000u;
+                if (vs >= 0) {
+                    const int v = fdiv(vs, q.dVW), vc = vs - v * q.VW;
+                    const int n = fdiv(v, q.dVH), ih = v - n * q.VH - q.PH;
+                    if (n < q.N && (unsigned)ih < (unsigned)q.IH && vc < q.IW)
+                        off = n * q.image_stride + ih * q.row_stride + vc * q.pix_stride +
+                              pl * q.plane_stride;
+                }
+                b_goff[j] = off;
             });
             return;
         }
@@ -153,6 +182,8 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             const int u = wave + j * DM_WAVES;
             if constexpr (FCB)
                 dma_global_b128(q.src + (b_goff[j] + poff), lds_address(buf + A_BYTES + u * 1024));
+            else if constexpr (PM)
+                dma_buffer_b128(src_rsrc, b_goff[j] + poff, lds_address(buf + A_BYTES + u * 1024));
             else
                 dma_buffer_b32(src_rsrc, b_goff[j] + poff, lds_address(buf + A_BYTES + u * 256));
         });
@@ -242,7 +273,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     int g = 0, cbuf = 0;
     for (int p0 = range0; p0 < range1; p0 += DM_BNP) {
         const int plast = min(p0 + DM_BNP, range1) - 1;
-        const int vp0 = vp_of(q, p0);
+        const int vp0 = PM ? pm_base(p0) + q.PW : vp_of(q, p0);
         int b_byte[NT];  // LDS byte offset of this lane's 16 channels at tap (0,0)
         int cur_o[NT];
         int cols = 0;    // wave-uniform: 32-pixel columns of this wave with pixels of the sub-tile
@@ -254,6 +285,8 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             const int p = pc + (lane & 31);
             if constexpr (FCB)
                 b_byte[ni] = p - p0;  // LDS row of this lane's pixel
+            else if constexpr (PM)  // dword of the pixel in the lane's first plane
+                b_byte[ni] = (kg * 4 * LMAX + (p <= plast ? vp_of(q, p) - vp0 : 0)) * 4;
             else
                 b_byte[ni] = (kg * LMAX + (p <= plast ? vp_of(q, p) - vp0 : 0)) * 16;
             cols += pc <= plast ? 1 : 0;
@@ -298,7 +331,12 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
                         if constexpr (FCB)
                             fb[t & 1][ni] = *(const v4i*)(bufB + b_byte[ni] * 128 +
                                                           (((ks * 2 + kg) ^ (b_byte[ni] & 7)) << 4));
-                        else
+                        else if constexpr (PM) {
+                            const int8_t* b0 = bufB + ks * (8 * LMAX * 4) + b_byte[ni] + tap_off * 4;
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                fb[t & 1][ni][i] = *(const int*)(b0 + i * (LMAX * 4));
+                        } else
                             fb[t & 1][ni] = *(const v4i*)(bufB + ks * (2 * LMAX * 16) + b_byte[ni] +
                                                           tap_off * 16);
                     }
@@ -344,7 +382,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
 }
 
 // ---- configurations --------------------------------------------------------------------------
-template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3, int WGM = 2, int BPC = 1, int NT = 2, bool FCB = false>
+template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3, int WGM = 2, int BPC = 1, int NT = 2, bool FCB = false, bool PM = false>
 static PipeConfig make_dma_config(int act, bool table_ok) {
     constexpr int DM_BM = 32 * MT * WGM;
     PipeConfig c;
@@ -359,20 +397,22 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.blocks_per_cu = BPC;
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     c.fixed_lmax = LMAX;
+    c.pm = PM ? 1 : 0;
     c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + (DM_BM > 128 ? DM_BM : 128) * 4;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC, NT, FCB>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
     else if (act == MEGCC_NONLINE_RELU && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF, WGM, BPC, NT, FCB>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
     else
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT, FCB>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
     return c;
 }
 
 // 3x3 and 1x1 NCHW44 layers and FullyConnected with at least 128 output channels (64 for the 1x1
 // with 32 input channels) and enough pixels. 1x1: 128 input channels per stage (64 / 32 when
 // IC <= 64 / 32).
-// variant 0: 512-pixel sub-tiles (3x3 only, two stage buffers); variant 1: 256-pixel sub-tiles.
+// variant 0: 512-pixel sub-tiles (3x3 only, two stage buffers); variant 1: 256-pixel sub-tiles;
+// variants 2 / 3: variant 0 with the plane-major patch of 768 / 1024 slots.
 bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok, PipeConfig* c) {
     const long P = (long)g.n * g.oh * g.ow;
     const bool k3 = g.fh == 3 && g.fw == 3, k1 = g.fh == 1 && g.fw == 1;
@@ -385,6 +425,33 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok,
     const bool ok = requant_table_ok(g.s_src, g.s_flt, g.s_dst);
     // measured slower on the 256-channel 56x56 layer (91 us): two 256-thread workgroups per CU
     // with 64-channel tiles and two buffers (100 us), four waves of 128 oc x 64 pixels (107 us)
+    if (variant == 2 || variant == 3) {
+        // plane-major patch, 16-byte activation loads: needs whole 16-byte groups per image row
+        if (!k3 || g.sw != 1 || (g.iw & 3) || !b128_ok || fc ||
+            ((long)g.n * (g.ih + 2 * g.ph) + 2L * g.fh * g.dh) * (g.iw + g.pw + 3) >= (1L << 31))
+            return false;
+        // 768 slots hold a 512-pixel sub-tile of rows up to ~60 slots inside one image; a sub-tile
+        // that crosses into the next image also spans the padding rows between them
+        if (g.oc < 128 && variant == 2)
+            *c = make_dma_config<3, 3, 1, 768, false, 1, 2, 2, 1, 4, false, true>(g.act, ok);
+        else if (g.oc < 128)
+            *c = make_dma_config<3, 3, 1, 1024, false, 1, 2, 2, 1, 4, false, true>(g.act, ok);
+        else if (variant == 2)
+            *c = make_dma_config<3, 3, 1, 768, false, 2, 2, 2, 1, 4, false, true>(g.act, ok);
+        else
+            *c = make_dma_config<3, 3, 1, 1024, false, 2, 2, 2, 1, 4, false, true>(g.act, ok);
+        return true;
+    }
+    if (variant == 4) {  // variant 1 (256-pixel sub-tiles, three buffers) with the plane-major patch
+        if (!k3 || g.sw != 1 || (g.iw & 3) || !b128_ok || fc ||
+            ((long)g.n * (g.ih + 2 * g.ph) + 2L * g.fh * g.dh) * (g.iw + g.pw + 3) >= (1L << 31))
+            return false;
+        if (g.oc < 128)
+            *c = make_dma_config<3, 3, 1, 512, false, 1, 3, 2, 1, 2, false, true>(g.act, ok);
+        else
+            *c = make_dma_config<3, 3, 1, 512, false, 2, 3, 2, 1, 2, false, true>(g.act, ok);
+        return true;
+    }
     if (variant == 0) {
         if (!k3)
             return false;

@@ -33,7 +33,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the default workload's kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by what a 256 MiB copy reads on the same counters: x2.000 / x1.000);
 # the counter runs and their figures are in profiles/conv_mfma_i8_dma__conv3x3_n32_c256_56x56.txt
-MEASURED_TRAFFIC = {"conv": (37684 * 2.000 + 25088 * 1.000) * 1024}
+MEASURED_TRAFFIC = {"conv": (37675 * 2.000 + 25088 * 1.000) * 1024}
 
 
 class HipEvents:
@@ -223,8 +223,10 @@ def cpu_baseline(full_case, budget_s=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=500,
+                    help="untimed launches first (the GPU takes a few hundred 70 us launches to "
+                         "reach its sustained clocks)")
     ap.add_argument("--workload", default="conv")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--batch", type=int, default=64, help="batch of the mobilenet workload")
@@ -293,7 +295,7 @@ def main():
     if not args.no_cpu and args.workload == "conv":
         out["cpu_baseline"] = cpu_baseline(case)
         op = None
-        mb = bench_mobilenet(64, 20, 5)
+        mb = bench_mobilenet(64, 200, 100)
         import mobilenet
         cpu_s, used = mobilenet.Net(1).run_cpu_timed(mobilenet.draw_input(1, seed=1), threads=1)
         out["extra"] = {"mobilenet_v1_int8_images_per_s_batch64": mb["images_per_s"],

@@ -39,6 +39,14 @@ static constexpr int ACT_RT = -1;
 // NT: 32-pixel MFMA tiles per wave along pixels; the workgroup sub-tile is 128 * NT pixels. NT = 4
 // reads 0.75 KB of LDS per MFMA instead of 1 KB (the 2 x 2 wave tile keeps the LDS port as busy as
 // the matrix core).
+// PM: plane-major activation patch for 3x3 stride-1 layers whose rows are a multiple of 4 pixels:
+// the activation loads are 16 bytes per lane as well (the cost of LDS-direct loads goes with their
+// number, not their bytes). Slot space = VW = round_up(IW + PW, 4) slots per padded image row,
+// image column x at slot x, so the left padding of a row is the tail of the row before; a patch
+// starts at a multiple of 4 and every group of 4 slots is 4 neighbouring pixels of one plane or 4
+// padding slots (offset beyond num_records -> zeros). LDS holds [plane][slot][4 bytes], a
+// wave-load = 256 consecutive slots of one plane, and the MFMA B operand (16 channels = 4 planes)
+// is read as four dwords LMAX * 4 bytes apart (two ds_read2st64_b32).
 // FCB: FullyConnected with K a multiple of 128 and a 16-byte aligned source: the rows of the
 // activation matrix are contiguous in K, so the B tile comes in with 16-byte loads as well - a
 // wave-load is 8 rows x 128 bytes = 8 full cache lines. LDS then holds a pixel's 128 bytes of a
@@ -130,13 +138,17 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             // wave-load u = plane u / PM_PARTS, slots (u % PM_PARTS) * 256 + 4 * lane .. + 3: four
             // neighbours of one image row (rows are 4-aligned in slot space) or four padding slots
             const int vbase = pm_base(p0);
+            // slots the sub-tile's windows reach; the rest of the LMAX slots is not fetched
+            const int L = vp_of(q, min(p0 + DM_BNP, range1) - 1) - q.PW +
+                          ((FH - 1) * q.DH) * q.VW + (FW - 1) * q.DW - vbase + 1;
             static_for<B_PER_WAVE>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 const int u = wave + j * DM_WAVES;
                 const int pl = u / PM_PARTS;
-                const int vs = vbase + (u - pl * PM_PARTS) * 256 + lane * 4;
+                const int slot = (u - pl * PM_PARTS) * 256 + lane * 4;
+                const int vs = vbase + slot;
                 unsigned off = 0x80000000u;
-                if (vs >= 0) {
+                if (vs >= 0 && slot < L) {
                     const int v = fdiv(vs, q.dVW), vc = vs - v * q.VW;
                     const int n = fdiv(v, q.dVH), ih = v - n * q.VH - q.PH;
                     if (n < q.N && (unsigned)ih < (unsigned)q.IH && vc < q.IW)

@@ -516,14 +516,15 @@ TinyNNStatus conv_mfma_launch(
     static const int kDmaVariants[] = {2, 3, 0, 4, 1};
     static const char* const kDmaSwitch[] = {"MEGCC_NOPM768", "MEGCC_NOPM", "MEGCC_NODMA512",
                                              "MEGCC_NOPM256", "MEGCC_NODMA"};
-    for (int cand = 0; cand < 7 && !pipe; ++cand) {
+    constexpr int N_DMA_VARIANTS = 5;
+    for (int cand = 0; cand < N_DMA_VARIANTS + 2 && !pipe; ++cand) {
         bool have = false;
-        if (cand < 5) {
+        if (cand < N_DMA_VARIANTS) {
             const int v = kDmaVariants[cand];
             have = !getenv("MEGCC_NODMA") && !getenv(kDmaSwitch[cand]) &&
                    !((v == 2 || v == 4) && getenv("MEGCC_NOPM")) &&
                    conv_mfma_dma_config(g, is_fc(g), v, b128_ok, &pc);
-        } else if (cand == 5) {
+        } else if (cand == N_DMA_VARIANTS) {
             have = !getenv("MEGCC_NOWS") && conv_mfma_ws_config(g, g4_ok, &pc);
         } else {
             have = !getenv("MEGCC_NOWIDE") && conv_mfma_pipe_config(g, g4_ok, &pc);

@@ -153,9 +153,9 @@ void megcc_gfx950_model_destroy(void* model) {
     if (m->workspace)
         m->dev.free(m->workspace);
     if (m->graph_exec)
-        hipGraphExecDestroy(m->graph_exec);
+        (void)hipGraphExecDestroy(m->graph_exec);
     if (m->graph)
-        hipGraphDestroy(m->graph);
+        (void)hipGraphDestroy(m->graph);
     delete m;
 }
 
@@ -491,7 +491,7 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
                 return TinyNN_SUCCESS;
             }
             if (g)
-                hipGraphDestroy(g);
+                (void)hipGraphDestroy(g);
             (void)hipGetLastError();  // a failed capture must not poison the eager path
             if (st != TinyNN_SUCCESS)
                 return st;

@@ -1,8 +1,8 @@
 /*
  * TEST INFRASTRUCTURE ONLY -- CPU restatement ("port") of the arithmetic of MegCC's generated
- * x86/BAREMETAL kernels for the conv / matmul / pooling / elemwise / typecvt path. It exists to
- * check the gfx950 kernels and to serve as bench.py's cpu_baseline leg; nothing in the product
- * library includes, links or calls it.
+ * x86/BAREMETAL kernels for the conv / matmul / pooling / elemwise / typecvt / relayout / concat
+ * path. It exists to check the gfx950 kernels and to serve as bench.py's cpu_baseline leg; nothing
+ * in the product library includes, links or calls it.
  *
  * Every function cites the generator it restates (paths relative to the MegCC tree,
  * compiler/lib/KernelGen/...). Integer accumulation is exact, so loop order is free there; every

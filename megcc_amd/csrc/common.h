@@ -11,6 +11,9 @@ namespace mg {
 // One stream for every launch and copy, default priority, created on first use.
 hipStream_t stream();
 
+// Compute units of the current device (256 when the query fails).
+int num_cus();
+
 // Records a message for megcc_gfx950_last_error() and returns `st`.
 TinyNNStatus fail(TinyNNStatus st, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 

@@ -360,19 +360,6 @@ __global__ void __launch_bounds__(256) pack_filter_kernel(
     }
 }
 
-static int num_cus() {
-    static int n = 0;
-    if (!n) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            n = prop.multiProcessorCount;
-        if (n <= 0)
-            n = 256;
-    }
-    return n;
-}
-
 static int round_up(int a, int b) {
     return (a + b - 1) / b * b;
 }

@@ -183,18 +183,6 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
     }
 }
 
-static int pw_num_cus() {
-    static int n = 0;
-    if (!n) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-            n = prop.multiProcessorCount;
-        if (n <= 0)
-            n = 256;
-    }
-    return n;
-}
 
 // workgroups of `kern` one CU holds at a time
 static int pw_resident_blocks(const void* kern) {
@@ -264,7 +252,7 @@ TinyNNStatus conv_pw_stream_launch(
     // once and then streams), fewer when there are not about four tiles for each
     const long items = (long)q.tiles * q.groups;
     long waves = items / 4;
-    const long cap = (long)pw_num_cus() * 4 * pw_resident_blocks(kern);
+    const long cap = (long)num_cus() * 4 * pw_resident_blocks(kern);
     if (waves > cap)
         waves = cap;
     long gcd = q.groups, rest = 4;  // unit = lcm(groups, waves per workgroup)

@@ -37,6 +37,19 @@ TinyNNStatus check_launch(const char* what) {
     return TinyNN_SUCCESS;
 }
 
+int num_cus() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            n = prop.multiProcessorCount;
+        if (n <= 0)
+            n = 256;
+    }
+    return n;
+}
+
 TinyNNStatus check_io(
         Tensor** inputs, int nr_input, int want_in_min, int want_in_max, Tensor** outputs,
         int nr_output, const char* who) {

@@ -197,6 +197,40 @@ def test_matches_oracle(case):
     compare(got, want, repr(case))
 
 
+def _plane_major_sweep():
+    """seeded random 3x3 stride-1 layers whose rows are a multiple of 4 pixels and that are large
+    enough for the LDS-direct kernels: batches whose sub-tiles cross image borders, ragged last
+    sub-tiles, padding 0 / 1 / 2 (with dilation 2), channel counts that leave partial tiles"""
+    r = np.random.Generator(np.random.PCG64(2024))
+    out = []
+    while len(out) < 14:
+        iw = int(r.integers(2, 17)) * 4
+        ih = int(r.integers(6, 70))
+        pad, dil = [(1, 1), (0, 1), (2, 2), (1, 1)][int(r.integers(0, 4))]
+        oh, ow = ih + 2 * pad - 2 * dil, iw + 2 * pad - 2 * dil
+        if oh < 1 or ow < 1:
+            continue
+        n = int(r.integers(1, 9))
+        if n * oh * ow < 2048 or n * oh * ow > 60000:
+            continue
+        ic = int(r.choice([32, 64, 96, 128]))
+        oc = int(r.choice([64, 96, 128, 192, 256]))
+        act = [A.RELU, A.IDENTITY][int(r.integers(0, 2))]
+        out.append(ConvCase(A.FMT_NCHW44, A.DENSE, n, ic, ih, iw, oc, 3, 1, pad, act,
+                            scales=(0.02, 0.01, unsat(9 * ic)), dilate=dil))
+    return out
+
+
+SWEEP = _plane_major_sweep()
+
+
+@pytest.mark.parametrize("case", SWEEP, ids=[repr(c) for c in SWEEP])
+def test_plane_major_patch_sweep(case):
+    port.set_threads(8)
+    arrays = case.gen(seed=23)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+
+
 def test_direct_kernel_when_filter_was_not_packed():
     """a caller that skips the init protocol still gets the right answer (generic kernel)"""
     import ctypes as C

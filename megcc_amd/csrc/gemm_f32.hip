@@ -13,6 +13,7 @@
 // fp32 sums are formed in a different order from the reference's 4x12 micro-kernel; results are
 // held to 1e-4 relative, not bit-exactness.
 #include "common.h"
+#include "gevm_f32.h"
 #include "conv_geom.h"
 #include "epilogue.cuh"
 
@@ -398,6 +399,11 @@ extern "C" TinyNNStatus megcc_gfx950_matmul(
     q.is_conv = 0;
     if (q.M == 0 || q.N == 0)
         return TinyNN_SUCCESS;
+    if (q.M <= 4 && q.K > 0 && !getenv("MEGCC_NOGEVM")) {  // the reference's gevm case: one pass over B
+        const GevmArgs v = {q.A, q.B, q.C, q.M, q.N, q.K, q.a_rs, q.a_cs, q.b_rs, q.b_cs, q.ldc};
+        if (gevm_f32_supported(v))
+            return gevm_f32_launch(v);
+    }
     gemm_plan_split(q, ws);
     // 64 x 256 tiles when they still give every CU a workgroup
     const bool skinny = q.M <= 64 && (long)((q.N + 255) / 256) * q.split >= 128;

@@ -480,6 +480,9 @@ TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
 int fc_stream_split(const ConvGeom& g, const void* src, size_t ws_bytes, int max_split);
 TinyNNStatus fc_stream_launch(
         const ConvGeom& g, const void* src, const void* packed, int32_t* partial, int split);
+bool fc_gevm_q8_supported(const ConvGeom& g);
+TinyNNStatus fc_gevm_q8_launch(
+        const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst);
 bool conv_pw_stream_supported(const ConvGeom& g);
 TinyNNStatus conv_pw_stream_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst);
@@ -490,6 +493,9 @@ TinyNNStatus conv_mfma_launch(
     // pointwise layers with few input channels: the streaming kernel (conv_pw_stream.hip)
     if (conv_pw_stream_supported(g) && !getenv("MEGCC_NOPWS"))
         return conv_pw_stream_launch(g, src, packed, bias, dst);
+    // FullyConnected with at most 4 rows: one pass over the weights (fc_gevm_q8.hip)
+    if (is_fc(g) && fc_gevm_q8_supported(g) && !getenv("MEGCC_NOGEVM"))
+        return fc_gevm_q8_launch(g, src, packed, bias, dst);
     MfmaParams q = {};
     PipeConfig pc;
     const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;

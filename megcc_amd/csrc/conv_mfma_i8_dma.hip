@@ -489,6 +489,7 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok,
         *c = make_dma_config<1, 1, 1, 256, false, 1, 8>(g.act, ok);
     else if (g.ic <= 128)
         *c = make_dma_config<1, 1, 2, 256, false, 2, 6>(g.act, ok);
+
     else
         *c = make_dma_config<1, 1, 4, 256, false>(g.act, ok);
     return true;

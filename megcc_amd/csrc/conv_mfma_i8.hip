@@ -506,16 +506,16 @@ TinyNNStatus conv_mfma_launch(
     bool pipe = false;
     // DMA kernel variants in order of preference (see conv_mfma_dma_config), then the two older
     // generations
-    static const int kDmaVariants[] = {2, 3, 0, 4, 1};
-    static const char* const kDmaSwitch[] = {"MEGCC_NOPM768", "MEGCC_NOPM", "MEGCC_NODMA512",
-                                             "MEGCC_NOPM256", "MEGCC_NODMA"};
-    constexpr int N_DMA_VARIANTS = 5;
+    static const int kDmaVariants[] = {6, 7, 2, 3, 0, 4, 1};
+    static const char* const kDmaSwitch[] = {"MEGCC_NOSMALL", "MEGCC_NOSMALL", "MEGCC_NOPM768", "MEGCC_NOPM",
+                                             "MEGCC_NODMA512", "MEGCC_NOPM256", "MEGCC_NODMA"};
+    constexpr int N_DMA_VARIANTS = 7;
     for (int cand = 0; cand < N_DMA_VARIANTS + 2 && !pipe; ++cand) {
         bool have = false;
         if (cand < N_DMA_VARIANTS) {
             const int v = kDmaVariants[cand];
             have = !getenv("MEGCC_NODMA") && !getenv(kDmaSwitch[cand]) &&
-                   !((v == 2 || v == 4) && getenv("MEGCC_NOPM")) &&
+                   !((v == 2 || v == 4 || v == 6) && getenv("MEGCC_NOPM")) &&
                    conv_mfma_dma_config(g, is_fc(g), v, b128_ok, &pc);
         } else if (cand == N_DMA_VARIANTS) {
             have = !getenv("MEGCC_NOWS") && conv_mfma_ws_config(g, g4_ok, &pc);
@@ -531,8 +531,11 @@ TinyNNStatus conv_mfma_launch(
         const long oc_tiles = (g.oc + pc.bm - 1) / pc.bm;
         long ranges = slots / oc_tiles > 0 ? slots / oc_tiles : 1;
         range_len = ((P + ranges - 1) / ranges + 31) / 32 * 32;
-        if (range_len < pc.bn / 2)  // too few pixels per workgroup for the tile
-            continue;
+        if (range_len < pc.bn / 2) {  // too few pixels per workgroup for the tile
+            if (pc.bm != 32)
+                continue;
+            range_len = pc.bn;  // the small-layer tiles: one tile per workgroup, not every CU busy
+        }
         t = plan_tiles(g, pc.bn, range_len, pc.pm);
         if (pc.fixed_lmax) {
             if (t.Lmax > pc.fixed_lmax)

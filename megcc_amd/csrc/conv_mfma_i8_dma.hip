@@ -428,6 +428,27 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
 bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok, PipeConfig* c) {
     const long P = (long)g.n * g.oh * g.ow;
     const bool k3 = g.fh == 3 && g.fw == 3, k1 = g.fh == 1 && g.fw == 1;
+    if (variant == 6 || variant == 7) {
+        // small 3x3 layers (batch 1): 32 oc x 128 px tiles of four waves, one 32 x 32 MFMA tile
+        // each, so that a few thousand pixels still give every CU a workgroup; variant 6 with the
+        // plane-major patch
+        // (only while the 128-channel tiles of the other variants would get fewer than 64 pixels per
+        //  CU: measured cross-over between 49 and 98)
+        if (!k3 || fc || g.fmt != MEGCC_FMT_NCHW44 || P < 512 ||
+            P * ((g.oc + 127) / 128) >= 64L * num_cus() || g.oc < 32 || (g.ic & 31) ||
+            (long)g.n * g.oc * g.oh * g.ow >= (1L << 31))
+            return false;
+        const bool okt = requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+        if (variant == 6) {
+            if (g.sw != 1 || (g.iw & 3) || !b128_ok ||
+                ((long)g.n * (g.ih + 2 * g.ph) + 2L * g.fh * g.dh) * (g.iw + g.pw + 3) >= (1L << 31))
+                return false;
+            *c = make_dma_config<3, 3, 1, 512, false, 1, 3, 1, 1, 1, false, true>(g.act, okt);
+        } else {
+            *c = make_dma_config<3, 3, 1, 384, false, 1, 3, 1, 1, 1>(g.act, okt);
+        }
+        return true;
+    }
     if (!(k3 || k1) || !(g.fmt == MEGCC_FMT_NCHW44 || fc) || g.oc < 64 || P < 2048)
         return false;
     if (g.oc < 128 && !(k1 && !fc && g.ic <= 32) && !k3)

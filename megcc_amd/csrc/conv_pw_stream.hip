@@ -87,7 +87,7 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
     // positions ahead of their MFMA in the sequence (tile, chunk) -> tile * KC + chunk: four tiles
     // ahead with 32 input channels, half a tile with 512. The loop is unrolled over U tiles so that
     // every ring slot and every "which tile, which chunk" below is a compile-time constant.
-    constexpr int RING = KC == 1 ? 4 : KC == 2 ? 6 : 8;
+    constexpr int RING = KC == 1 ? 4 : KC == 2 ? 6 : KC == 16 ? 16 : 8;
     constexpr int U = RING > KC ? RING / KC : 1;           // tiles per unrolled step
     constexpr int AHEAD = (RING + KC - 1) / KC;            // tiles a request can be ahead
     static_assert(RING % KC == 0 || KC % RING == 0, "slots repeat every U tiles");

@@ -19,6 +19,8 @@
 //
 // Same arithmetic as the other qsi8 kernels: int32 accumulators starting from the bias, exact
 // requantisation by threshold table (epilogue.cuh). Reference loop: BareMetal/ConvKernel.cpp:305-344.
+#include <stdlib.h>
+
 #include <map>
 #include <mutex>
 
@@ -248,13 +250,12 @@ TinyNNStatus conv_pw_stream_launch(
     }
 #undef MG_PW_PICK
 
-    // waves: a multiple of `groups`; as many as are resident at once (every wave pays the set-up
-    // once and then streams), fewer when there are not about four tiles for each
+    // waves: a multiple of `groups`; one per (tile, channel group) while they are all resident at
+    // once - a small layer is then one memory round trip - and never more than are resident (every
+    // wave pays the set-up once and then streams over its tiles)
     const long items = (long)q.tiles * q.groups;
-    long waves = items / 4;
     const long cap = (long)num_cus() * 4 * pw_resident_blocks(kern);
-    if (waves > cap)
-        waves = cap;
+    long waves = items < cap ? items : cap;
     long gcd = q.groups, rest = 4;  // unit = lcm(groups, waves per workgroup)
     while (rest) {
         const long r = gcd % rest;

@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
     // positions ahead of their MFMA in the sequence (tile, chunk) -> tile * KC + chunk: four tiles
     // ahead with 32 input channels, half a tile with 512. The loop is unrolled over U tiles so that
     // every ring slot and every "which tile, which chunk" below is a compile-time constant.
-    constexpr int RING = KC == 1 ? 4 : KC == 2 ? 6 : KC == 16 ? 16 : 8;
+    constexpr int RING = KC == 1 ? 4 : KC == 2 ? 6 : KC >= 16 ? 16 : 8;
     constexpr int U = RING > KC ? RING / KC : 1;           // tiles per unrolled step
     constexpr int AHEAD = (RING + KC - 1) / KC;            // tiles a request can be ahead
     static_assert(RING % KC == 0 || KC % RING == 0, "slots repeat every U tiles");
@@ -203,7 +203,9 @@ static int pw_resident_blocks(const void* kern) {
 bool conv_pw_stream_supported(const ConvGeom& g) {
     const long P = (long)g.n * g.oh * g.ow;
     return g.fmt == MEGCC_FMT_NCHW44 && g.groups == 1 && g.fh == 1 && g.fw == 1 && g.sh == 1 &&
-           g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.ic == 32 || g.ic == 64 || g.ic == 128 || g.ic == 256 || g.ic == 512) &&
+           g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.ic == 32 || g.ic == 64 || g.ic == 128 || g.ic == 256 || g.ic == 512 ||
+            // (1024: only layers too small for the LDS-staged kernel, where one round trip wins)
+            (g.ic == 1024 && P < 2048)) &&
            (g.oc & 63) == 0 && g.oc <= PW_MAX_OC && P >= 32 &&
            (long)g.n * g.ic * g.ih * g.iw < (1L << 31) && P * g.oc < (1L << 31);
 }
@@ -246,7 +248,8 @@ TinyNNStatus conv_pw_stream_launch(
         case 2: kern = MG_PW_PICK(2, 2); break;
         case 4: kern = MG_PW_PICK(4, 2); break;
         case 8: kern = MG_PW_PICK(8, 2); break;
-        default: kern = MG_PW_PICK(16, 1); break;  // 512 input channels: 32 output channels per wave
+        case 16: kern = MG_PW_PICK(16, 1); break;  // 512 input channels: 32 output channels per wave
+        default: kern = MG_PW_PICK(32, 1); break;  // 1024: the filter rows fill half the registers
     }
 #undef MG_PW_PICK
 

@@ -186,6 +186,116 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
 }
 
 
+// The same layer with the activation tile SHARED by the four waves of a workgroup (512 input
+// channels): the waves own four neighbouring 32-channel groups and the same run of pixel tiles; the
+// MFMA B operand of a tile does not depend on the channel group, so each wave fetches a quarter
+// of a tile's 16 chunks (16 dword loads instead of 64) and parks them in LDS exactly as the lanes
+// will read them back (chunk c, lane l at c * 1 KB + l * 16: consecutive lanes, consecutive 16-byte
+// words, no bank conflicts). Two LDS tiles: the chunks of tile t + 1 are requested before tile t
+// is computed and written after it, one barrier per tile. A quarter of the L2 traffic and of the
+// load instructions of the streaming form.
+template <int KC, int ACT>
+__global__ void __launch_bounds__(PW_THREADS) conv_pw_share_kernel(PwParams q) {
+    static_assert(KC % 4 == 0, "a quarter of the chunks per wave");
+    constexpr int CW = KC / 4;  // chunks a wave fetches per tile
+    __shared__ int tbl[REQUANT_TABLE_ENTRIES];
+    __shared__ __attribute__((aligned(16))) int bias_lds[PW_MAX_OC];
+    __shared__ __attribute__((aligned(16))) int8_t btile[2][KC * 1024];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, kg = lane >> 5;
+    // workgroup -> (block of 4 channel groups, run of tiles)
+    const int gblocks = q.groups >> 2;
+    const int gb = blockIdx.x % gblocks;
+    const int runs = gridDim.x / gblocks;
+    const int og = gb * 4 + wave;
+    const int per = (q.tiles + runs - 1) / runs;
+    const int t0 = (blockIdx.x / gblocks) * per;
+    const int tend = min(t0 + per, q.tiles);
+
+    v4i A[KC];
+    {
+        const int oc = og * 32 + col;
+#pragma unroll
+        for (int c = 0; c < KC; ++c)
+            A[c] = *(const v4i*)(q.wp + ((size_t)c * q.OCP + oc) * KROW + (((kg ^ (oc >> 3)) & 1) << 4));
+    }
+    const __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc((void*)q.src, 0, q.src_bytes, 0x00020000);
+    auto tile_base = [&](int tile) __attribute__((always_inline)) -> unsigned {
+        const int p = tile * 32 + col;
+        const int n = fdiv(p, q.dOHW);
+        return tile < tend && p < q.P
+                       ? (unsigned)(n * q.image_stride + (p - n * q.OHW) * 4 + kg * 4 * q.plane_stride)
+                       : 0x80000000u;
+    };
+    // this wave's chunks wave * CW .. + CW - 1 of `tile`
+    auto request = [&](int tile, v4i (&r)[CW]) __attribute__((always_inline)) {
+        const unsigned base = tile_base(tile);
+#pragma unroll
+        for (int k = 0; k < CW; ++k)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                r[k][j] = (int)__builtin_amdgcn_raw_buffer_load_b32(
+                        rs, (int)(base + (unsigned)(((wave * CW + k) * 8 + j) * q.plane_stride)), 0, 0);
+    };
+    auto park = [&](int buf, const v4i (&r)[CW]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int k = 0; k < CW; ++k)
+            *(v4i*)(btile[buf] + (wave * CW + k) * 1024 + lane * 16) = r[k];
+    };
+
+    v4i nxt[CW];
+    request(t0, nxt);
+    if (ACT >= 0)
+        tbl[tid] = pw_kernarg_table(tid);
+    for (int i = tid; i < q.OC; i += PW_THREADS)
+        bias_lds[i] = q.bias ? q.bias[i] : 0;
+    park(0, nxt);
+    __syncthreads();
+
+    for (int t = t0, buf = 0; t < tend; ++t, buf ^= 1) {
+        if (t + 1 < tend)
+            request(t + 1, nxt);
+        v16i acc;
+#pragma unroll
+        for (int e4 = 0; e4 < 4; ++e4) {
+            const v4i bv = *(const v4i*)(bias_lds + og * 32 + e4 * 8 + kg * 4);
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                acc[e4 * 4 + k] = bv[k];
+        }
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            const v4i b = *(const v4i*)(btile[buf] + c * 1024 + lane * 16);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[c], b, acc, 0, 0, 0);
+        }
+        const int p = t * 32 + col;
+        const bool ok = p < q.P;
+        const int n = fdiv(p, q.dOHW);
+        const int obase = n * (q.OC >> 2) * q.OHW + (p - n * q.OHW);
+        int r[16];
+        if (ACT < 0) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                r[e] = requant_conv_rt(q.act, acc[e], q.s_src, q.s_flt, q.s_dst);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                r[e] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[e], q.c, tbl);
+        }
+        if (ok) {
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int oc4 = og * 8 + e4 * 2 + kg;
+                q.dst[obase + oc4 * q.OHW] = pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
+            }
+        }
+        if (t + 1 < tend)
+            park(buf ^ 1, nxt);
+        __syncthreads();
+    }
+}
+
 // workgroups of `kern` one CU holds at a time
 static int pw_resident_blocks(const void* kern) {
     static std::map<const void*, int> cache;
@@ -253,6 +363,25 @@ TinyNNStatus conv_pw_stream_launch(
     }
 #undef MG_PW_PICK
 
+    // 512 input channels and more tiles than resident waves: the workgroup-shared form
+    if (g.ic == 512 && (q.groups & 3) == 0 && !getenv("MEGCC_NOPWSHARE")) {
+        const void* sk = act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_share_kernel<16, MEGCC_NONLINE_IDENTITY>
+                         : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_share_kernel<16, MEGCC_NONLINE_RELU>
+                                                       : (const void*)conv_pw_share_kernel<16, -1>;
+        const long gblocks = q.groups / 4;
+        const long capb = (long)num_cus() * pw_resident_blocks(sk);
+        if ((long)q.tiles * gblocks >= capb / 2) {
+            long runs = capb / gblocks;
+            if (runs > q.tiles)
+                runs = q.tiles;
+            if (runs < 1)
+                runs = 1;
+            void* sargs[] = {&q};
+            hipError_t e = hipLaunchKernel(sk, dim3((unsigned)(runs * gblocks)), dim3(PW_THREADS), sargs, 0, stream());
+            MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_pw_share: %s", hipGetErrorString(e));
+            return check_launch("conv_pw_share");
+        }
+    }
     // waves: a multiple of `groups`; one per (tile, channel group) while they are all resident at
     // once - a small layer is then one memory round trip - and never more than are resident (every
     // wave pays the set-up once and then streams over its tiles)

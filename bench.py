@@ -33,7 +33,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the default workload's kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by what a 256 MiB copy reads on the same counters: x2.000 / x1.000);
 # the counter runs and their figures are in profiles/conv_mfma_i8_dma__conv3x3_n32_c256_56x56.txt
-MEASURED_TRAFFIC = {"conv": (37675 * 2.000 + 25088 * 1.000) * 1024}
+MEASURED_TRAFFIC = {"conv": (37666 * 2.000 + 25088 * 1.000) * 1024}
 
 
 class HipEvents:

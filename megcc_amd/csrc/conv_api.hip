@@ -20,6 +20,8 @@ bool conv_first_supported(const ConvGeom& g);
 TinyNNStatus conv_first_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool dwconv44_supported(const ConvGeom& g);
 TinyNNStatus dwconv44_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+bool conv_f32_small_supported(const ConvGeom& g);
+TinyNNStatus conv_f32_small_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool conv_f32_gemm_supported(const ConvGeom& g);
 TinyNNStatus conv_f32_gemm_launch(const ConvGeom&, const void*, const void*, const void*, void*,
                                   const Workspace*);
@@ -191,6 +193,8 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
         return dwconv44_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     if (q8 && conv_first_supported(g) && aligned4(src->ptr) && aligned4(dst->ptr) && (!b || aligned4(b)))
         return conv_first_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+    if (f32 && conv_f32_small_supported(g) && !getenv("MEGCC_NOF32SMALL"))
+        return conv_f32_small_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     if (f32 && conv_f32_gemm_supported(g))
         return conv_f32_gemm_launch(g, src->ptr, flt->ptr, b, dst->ptr, workspace);
     return conv_direct_launch(g, f32, src->ptr, flt->ptr, b, dst->ptr);

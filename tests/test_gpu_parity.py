@@ -179,6 +179,9 @@ LIVE = [
     # f32
     ConvCase(A.FMT_NCHW, A.DENSE, 1, 32, 56, 56, 32, 3, 1, 1, A.RELU, dtype="f32"),
     ConvCase(A.FMT_NCHW, A.DENSE, 2, 5, 19, 23, 37, 3, 2, 1, A.IDENTITY, dtype="f32"),
+    # above 2^27 multiply-adds: the implicit GEMM on the matrix cores
+    ConvCase(A.FMT_NCHW, A.DENSE, 4, 64, 56, 56, 64, 3, 1, 1, A.RELU, dtype="f32"),
+    ConvCase(A.FMT_NCHW, A.DENSE, 3, 40, 57, 55, 72, 3, 2, 1, A.H_SWISH, dtype="f32"),
     MatMulCase(1, 1024, 1000),
     MatMulCase(64, 512, 384),
     MatMulCase(130, 77, 259),
@@ -195,6 +198,38 @@ def test_matches_oracle(case):
     want = case.run_port(arrays)
     got = run_gpu(case, arrays)
     compare(got, want, repr(case))
+
+
+OLDER = [
+    # shapes the newer kernels take, forced back (development switches of the library) onto the
+    # kernels that still serve other shapes: one-stage kernel with split-K (slices of 2 stages out
+    # of 8: a sixth slice would start past the packed filter), dword activation loads, the
+    # 256-pixel variant, the tiled FullyConnected
+    ("MEGCC_NOSMALL", ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 56, 56, 256, 3, 1, 1, A.RELU,
+                               scales=(0.02, 0.01, unsat(2304)))),
+    ("MEGCC_NOSMALL", ConvCase(A.FMT_NCHW44, A.DENSE, 3, 256, 14, 14, 256, 3, 1, 1, A.IDENTITY,
+                               scales=(0.02, 0.01, 0.05))),
+    ("MEGCC_NOPM", ConvCase(A.FMT_NCHW44, A.DENSE, 6, 32, 56, 56, 160, 3, 1, 1, A.RELU,
+                            scales=(0.02, 0.01, unsat(288)))),
+    ("MEGCC_NODMA512", ConvCase(A.FMT_NCHW44, A.DENSE, 6, 64, 56, 56, 128, 3, 1, 1, A.RELU,
+                                scales=(0.02, 0.01, unsat(576)))),
+    ("MEGCC_NOGEVM", ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY,
+                              scales=(0.01, 0.01, unsat(1024) / 2))),
+    ("MEGCC_NOGEVM", MatMulCase(3, 301, 79, trans_b=True)),
+    ("MEGCC_NOF32SMALL", ConvCase(A.FMT_NCHW, A.DENSE, 1, 32, 56, 56, 32, 3, 1, 1, A.RELU, dtype="f32")),
+    ("MEGCC_NOPWSHARE", ConvCase(A.FMT_NCHW44, A.DENSE, 70, 512, 14, 14, 512, 1, 1, 0, A.RELU,
+                                 scales=(0.02, 0.01, unsat(512)))),
+    ("MEGCC_NOPWS", ConvCase(A.FMT_NCHW44, A.DENSE, 11, 64, 56, 56, 128, 1, 1, 0, A.IDENTITY,
+                             scales=(0.02, 0.01, unsat(64)))),
+]
+
+
+@pytest.mark.parametrize("switch,case", OLDER, ids=["%s-%r" % (s, c) for s, c in OLDER])
+def test_older_kernels_still_agree(switch, case, monkeypatch):
+    monkeypatch.setenv(switch, "1")
+    port.set_threads(8)
+    arrays = case.gen(seed=29)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
 
 
 def _plane_major_sweep():

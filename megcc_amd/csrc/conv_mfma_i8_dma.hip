@@ -83,7 +83,9 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     int* const bias_lds = rq_table + REQUANT_TABLE_ENTRIES;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WGN, wn = wave % WGN, kg = lane >> 5;
+    // (waves w and w + 4 share a SIMD: give them different pixel columns, so that the wave with
+    //  one column more in a ragged sub-tile does not meet its twin on the same SIMD)
+    const int wm = wave / WGN, wn = (wave + wm) % WGN, kg = lane >> 5;
     const int oc0 = blockIdx.y * DM_BM;
     const int range0 = blockIdx.x * q.range_len;
     const int range1 = min(range0 + q.range_len, q.P);

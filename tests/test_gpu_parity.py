@@ -200,6 +200,49 @@ def test_matches_oracle(case):
     compare(got, want, repr(case))
 
 
+def _random_views():
+    """seeded random strided views: permuted dims, steps of 2, reversed dims, both sides or one"""
+    r = np.random.Generator(np.random.PCG64(77))
+
+    def view(shape):
+        nd = len(shape)
+        perm = r.permutation(nd)
+        step = [int(r.integers(1, 3)) if r.random() < 0.3 else 1 for _ in range(nd)]
+        # dense strides of the permuted, stepped storage
+        st = [0] * nd
+        acc = 1
+        for ax in reversed(perm):
+            st[ax] = acc * step[ax]
+            acc *= shape[ax] * step[ax]
+        if r.random() < 0.25:
+            ax = int(r.integers(0, nd))
+            st[ax] = -st[ax]
+        return tuple(st)
+
+    out = []
+    for i in range(36):
+        nd = int(r.integers(1, 6))
+        big = r.random() < 0.4
+        shape = tuple(int(r.integers(1, 40 if big else 9)) for _ in range(nd))
+        if int(np.prod(shape)) > 300000:
+            shape = shape[:3]
+        dt = ["f32", "qsi8", "qsi32"][i % 3]
+        kind = i % 4
+        src = view(shape) if kind != 1 else None
+        dst = view(shape) if kind in (1, 2) else None
+        out.append(RelayoutCase(dt, shape, src, None, dst, slack=int(r.integers(0, 5))))
+    return out
+
+
+VIEWS = _random_views()
+
+
+@pytest.mark.parametrize("case", VIEWS, ids=["%d-%r" % (i, c) for i, c in enumerate(VIEWS)])
+def test_relayout_random_views(case):
+    arrays = case.gen(seed=31)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+
+
 OLDER = [
     # shapes the newer kernels take, forced back (development switches of the library) onto the
     # kernels that still serve other shapes: one-stage kernel with split-K (slices of 2 stages out

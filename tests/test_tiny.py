@@ -218,3 +218,25 @@ def test_views_that_leave_their_tensor_are_refused():
     d["device_models"][0]["tensors"][1]["dims"] = [4, 6]
     with pytest.raises(runtime.MegccError, match="not dense"):
         runtime.Model.load(tiny.write_model(d))
+
+
+@pytest.mark.gpu
+def test_dense_relayout_is_a_copy_that_replays_in_the_graph():
+    """a Relayout between two dense tensors is a device-to-device copy node of the captured graph:
+    every replay must move the current input"""
+    m = runtime.Model()
+    x = m.tensor("x", (3, 5, 7), abi.QINT8, 0.05)
+    m.mark_input(x)
+    y = m.tensor("y", (3, 5, 7), abi.QINT8, 0.05)
+    m.opr("kernel_relayout_qsi8", [x], [y])
+    z = m.tensor("z", (3, 5, 7), abi.QINT8, 0.05)
+    m.opr("kernel_elementwise_multitype_QRELU_qsi8qsi8", [y], [z])
+    m.mark_output(z)
+    m.finalize()
+    r = np.random.default_rng(3)
+    for _ in range(4):  # eager, captured, replayed twice
+        a = r.integers(-128, 128, (3, 5, 7)).astype(np.int8)
+        m.set_input(x, a)
+        m.forward()
+        assert np.array_equal(m.get(z), np.maximum(a, 0))
+    m.close()

@@ -1,0 +1,249 @@
+// qsi8 NCHW -> NCHW44 ("hybrid" first layer) convolution for any filter up to 8 x 8, stride 1 or 2,
+// 1..4 input channels - the 7x7 stride-2 stem of ResNet-like networks, 5x5 and stride-1 3x3
+// stems. Filter [OC/4, FH, FW, IC, 4 oc], same loop nest and epilogue as
+// BareMetal/ConvKernel.cpp:305-344,374-380 (format detection :115-127).
+//
+// K = IC * FH * FW is at most 147 here, too short for a staged GEMM but long enough that the
+// per-tap VALU kernel of the 3x3 case would spend thousands of instructions per pixel. So the
+// reduction index is re-ordered to make the matrix cores usable without an im2col:
+//     k' = (ic * FH + fh) * 8 + fw          (fw padded to 8, zero weights in the padding)
+// A lane's 16 K-bytes of an MFMA B operand are then two (ic, fh) rows x 8 consecutive input
+// columns: 8 bytes that lie next to each other in an LDS copy of the input rows under a strip of
+// output pixels. They are read as four 2-byte pieces (stride 2: the start column 2 * pixel is
+// even) or eight bytes (stride 1).
+//   * a workgroup walks over strips of 128 output pixels of one output row (a wave: 32 pixels x
+//     all output channels); per strip the IC * FH input row pieces go to LDS as bytes, zero where
+//     the image ends - padding costs nothing later;
+//   * the filter is re-ordered to k' once per workgroup into LDS ([chunk of 32 k'][oc][32 bytes])
+//     and read as MFMA A operands;
+//   * accumulators start from the bias, exact requantisation by threshold table, 4 consecutive
+//     accumulator registers = one NCHW44 dword, 32 lanes store 128 contiguous bytes.
+#include <map>
+#include <mutex>
+
+#include "common.h"
+#include "conv_geom.h"
+#include "conv_mfma_i8.h"
+#include "epilogue.cuh"
+
+namespace mg {
+
+static constexpr int CH_MAX_OC = 128;    // output channels (4 MFMA row tiles)
+static constexpr int CH_MAX_ROWS = 32;   // IC * FH
+static constexpr int CH_STRIP = 128;     // output pixels per strip
+
+struct ChParams {
+    const int8_t* src;
+    const int8_t* flt;
+    const int32_t* bias;
+    uint32_t* dst;
+    int N, IC, IH, IW, OC, OH, OW, FH, FW, PH, PW;
+    int rows;    // IC * FH
+    int chunks;  // ceil(rows / 4)
+    int octiles; // ceil(OC / 32)
+    int pitch;   // bytes per LDS row: (CH_STRIP - 1) * S + 8, rounded up to 4
+    int strips;  // per output row
+    int items;   // N * OH * strips
+    int act;
+    float s_src, s_flt, s_dst, c;
+    RequantTable table;
+};
+
+__device__ __forceinline__ int ch_kernarg_table(int i) {
+    typedef const __attribute__((address_space(4))) char* kptr;
+    const kptr base = (kptr)__builtin_amdgcn_kernarg_segment_ptr();
+    return *(const __attribute__((address_space(4))) int*)(base + offsetof(ChParams, table) + 4 * i);
+}
+
+// S: stride. ACT: IDENTITY / RELU use the table, -1 the literal sequence. OT: MFMA row tiles (OC <= 32 * OT).
+template <int S, int ACT, int OT>
+__global__ void __launch_bounds__(256) conv_hybrid_mfma_kernel(ChParams q) {
+    extern __shared__ __attribute__((aligned(16))) int8_t ch_lds[];
+    __shared__ int tbl[REQUANT_TABLE_ENTRIES];
+    __shared__ __attribute__((aligned(16))) int bias_lds[CH_MAX_OC];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, kg = lane >> 5;
+    const int ocp = OT * 32;
+    int8_t* const wl = ch_lds;                              // [chunk][ocp][32]
+    int8_t* const patch = ch_lds + q.chunks * ocp * 32;     // [chunks * 4 rows][pitch]
+
+    // ---- once per workgroup: filter in k' order, bias, thresholds ------------------------------
+    for (int i = tid; i < q.chunks * ocp * 32; i += 256) {
+        const int b = i & 31, oc = (i >> 5) % ocp, chunk = (i >> 5) / ocp;
+        const int r = chunk * 4 + (b >> 3), fw = b & 7;
+        int8_t v = 0;
+        if (oc < q.OC && r < q.rows && fw < q.FW) {
+            const int ic = r / q.FH, fh = r - ic * q.FH;
+            v = q.flt[((((size_t)(oc >> 2) * q.FH + fh) * q.FW + fw) * q.IC + ic) * 4 + (oc & 3)];
+        }
+        wl[i] = v;
+    }
+    if (ACT >= 0)
+        tbl[tid] = ch_kernarg_table(tid);
+    for (int i = tid; i < ocp; i += 256)
+        bias_lds[i] = (q.bias && i < q.OC) ? q.bias[i] : 0;
+    // rows of the patch beyond IC * FH are multiplied by zero weights: any finite bytes do
+    for (int i = tid; i < q.chunks * 4 * q.pitch; i += 256)
+        patch[i] = 0;
+    __syncthreads();
+
+    const int ohw = q.OH * q.OW;
+    for (int item = blockIdx.x; item < q.items; item += gridDim.x) {
+        const int sx = item % q.strips, row = item / q.strips;
+        const int n = row / q.OH, oh = row - n * q.OH;
+        const int ow0 = sx * CH_STRIP;
+        const int ih0 = oh * S - q.PH, iw0 = ow0 * S - q.PW;
+        // ---- input rows under the strip -> LDS (zero outside the image)
+        const int8_t* img = q.src + (size_t)n * q.IC * q.IH * q.IW;
+        for (int i = tid; i < q.rows * q.pitch; i += 256) {
+            const int r = i / q.pitch, c = i - r * q.pitch;
+            const int ic = r / q.FH, fh = r - ic * q.FH;
+            const unsigned ih = (unsigned)(ih0 + fh), iw = (unsigned)(iw0 + c);
+            patch[i] = ih < (unsigned)q.IH && iw < (unsigned)q.IW
+                               ? img[((size_t)ic * q.IH + ih) * q.IW + iw]
+                               : (int8_t)0;
+        }
+        __syncthreads();
+
+        // ---- this wave's 32 pixels x all output channels
+        v16i acc[OT];
+#pragma unroll
+        for (int t = 0; t < OT; ++t)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const v4i bv = *(const v4i*)(bias_lds + t * 32 + e4 * 8 + kg * 4);
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    acc[t][e4 * 4 + k] = bv[k];
+            }
+        const int px = wave * 32 + col;          // pixel of the strip
+        const int8_t* pb = patch + px * S;       // its window starts here in every row
+        for (int chunk = 0; chunk < q.chunks; ++chunk) {
+            // lane's K-bytes: rows chunk * 4 + 2 kg, + 1; 8 columns each
+            v4i b;
+#pragma unroll
+            for (int rr = 0; rr < 2; ++rr) {
+                const int8_t* p = pb + (chunk * 4 + kg * 2 + rr) * q.pitch;
+                if (S == 2) {
+                    const uint16_t* h = (const uint16_t*)p;
+                    b[rr * 2] = (int)((uint32_t)h[0] | ((uint32_t)h[1] << 16));
+                    b[rr * 2 + 1] = (int)((uint32_t)h[2] | ((uint32_t)h[3] << 16));
+                } else {
+                    const uint8_t* u = (const uint8_t*)p;
+                    b[rr * 2] = (int)((uint32_t)u[0] | ((uint32_t)u[1] << 8) | ((uint32_t)u[2] << 16) |
+                                      ((uint32_t)u[3] << 24));
+                    b[rr * 2 + 1] = (int)((uint32_t)u[4] | ((uint32_t)u[5] << 8) | ((uint32_t)u[6] << 16) |
+                                          ((uint32_t)u[7] << 24));
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < OT; ++t) {
+                const v4i a = *(const v4i*)(wl + ((chunk * ocp + t * 32 + col) * 32 + kg * 16));
+                acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[t], 0, 0, 0);
+            }
+        }
+
+        // ---- epilogue: register e of a tile = channel 8 * (e / 4) + 4 * kg + e % 4, pixel = col
+        const int ow = ow0 + px;
+        const int obase = (n * (q.OC >> 2)) * ohw + oh * q.OW + ow;
+#pragma unroll
+        for (int t = 0; t < OT; ++t) {
+            int r[16];
+            if (ACT < 0) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    r[e] = requant_conv_rt(q.act, acc[t][e], q.s_src, q.s_flt, q.s_dst);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    r[e] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[t][e], q.c, tbl);
+            }
+            if (ow < q.OW) {
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    const int oc4 = t * 8 + e4 * 2 + kg;
+                    if (oc4 * 4 < q.OC)
+                        q.dst[obase + oc4 * ohw] =
+                                pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
+                }
+            }
+        }
+        __syncthreads();  // the patch is rewritten for the next strip
+    }
+}
+
+bool conv_hybrid_mfma_supported(const ConvGeom& g) {
+    return g.fmt == MEGCC_FMT_NCHW_NCHW44 && g.groups == 1 && g.ic >= 1 && g.ic <= 4 && g.fh >= 1 &&
+           g.fw >= 1 && g.fw <= 8 && g.ic * g.fh <= CH_MAX_ROWS && g.sh == g.sw && (g.sh == 1 || g.sh == 2) &&
+           g.dh == 1 && g.dw == 1 && (g.oc & 3) == 0 && g.oc >= 4 && g.oc <= CH_MAX_OC &&
+           (long)g.n * g.ic * g.ih * g.iw < (1L << 31) && (long)g.n * g.oc * g.oh * g.ow < (1L << 31) &&
+           (long)g.n * g.oh * ((g.ow + CH_STRIP - 1) / CH_STRIP) < (1L << 31);
+}
+
+TinyNNStatus conv_hybrid_mfma_launch(
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, void* dst) {
+    ChParams q = {};
+    q.src = (const int8_t*)src;
+    q.flt = (const int8_t*)flt;
+    q.bias = (const int32_t*)bias;
+    q.dst = (uint32_t*)dst;
+    q.N = g.n; q.IC = g.ic; q.IH = g.ih; q.IW = g.iw;
+    q.OC = g.oc; q.OH = g.oh; q.OW = g.ow;
+    q.FH = g.fh; q.FW = g.fw; q.PH = g.ph; q.PW = g.pw;
+    q.rows = g.ic * g.fh;
+    q.chunks = (q.rows + 3) / 4;
+    q.octiles = (g.oc + 31) / 32;
+    q.pitch = ((CH_STRIP - 1) * g.sh + 8 + 3) & ~3;
+    q.strips = (g.ow + CH_STRIP - 1) / CH_STRIP;
+    q.items = g.n * g.oh * q.strips;
+    q.act = g.act;
+    q.s_src = g.s_src; q.s_flt = g.s_flt; q.s_dst = g.s_dst;
+    q.c = make_requant_fast(g.s_src, g.s_flt, g.s_dst).c;
+    const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
+                     requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    if (tab)
+        q.table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
+    const int act = tab ? g.act : -1;
+    const void* kern = nullptr;
+#define MG_CH_PICK(S_, OT_)                                                                             \
+    (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_hybrid_mfma_kernel<S_, MEGCC_NONLINE_IDENTITY, OT_> \
+     : act == MEGCC_NONLINE_RELU   ? (const void*)conv_hybrid_mfma_kernel<S_, MEGCC_NONLINE_RELU, OT_>     \
+                                   : (const void*)conv_hybrid_mfma_kernel<S_, -1, OT_>)
+    const int ot = q.octiles;
+    if (g.sh == 1)
+        kern = ot == 1 ? MG_CH_PICK(1, 1) : ot == 2 ? MG_CH_PICK(1, 2) : ot == 3 ? MG_CH_PICK(1, 3) : MG_CH_PICK(1, 4);
+    else
+        kern = ot == 1 ? MG_CH_PICK(2, 1) : ot == 2 ? MG_CH_PICK(2, 2) : ot == 3 ? MG_CH_PICK(2, 3) : MG_CH_PICK(2, 4);
+#undef MG_CH_PICK
+    const size_t lds = (size_t)q.chunks * ot * 32 * 32 + (size_t)q.chunks * 4 * q.pitch;
+
+    // as many workgroups as are resident at once: the filter set-up is paid once per workgroup
+    static std::map<std::pair<const void*, size_t>, int> per_cu;
+    static std::mutex lock;
+    int blocks_per_cu;
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        auto key = std::make_pair(kern, lds);
+        auto it = per_cu.find(key);
+        if (it == per_cu.end()) {
+            if (lds > 48 * 1024)
+                MG_REQUIRE(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) ==
+                                   hipSuccess,
+                           TinyNN_ERROR_RUNTIME, "conv_hybrid_mfma: LDS attribute");
+            int nb = 0;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kern, 256, lds) != hipSuccess || nb < 1)
+                nb = 1;
+            it = per_cu.emplace(key, nb).first;
+        }
+        blocks_per_cu = it->second;
+    }
+    long blocks = (long)num_cus() * blocks_per_cu;
+    if (blocks > q.items)
+        blocks = q.items;
+    void* args[] = {&q};
+    hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, lds, stream());
+    MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_hybrid_mfma: %s", hipGetErrorString(e));
+    return check_launch("conv_hybrid_mfma");
+}
+
+}  // namespace mg

@@ -243,6 +243,29 @@ def test_relayout_random_views(case):
     compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
 
 
+HYBRID = [
+    # NCHW -> NCHW44 first layers beyond 3x3 stride 2: the matrix-core kernel with the reduction
+    # re-ordered to (ic, fh, fw padded to 8); 1..4 input channels, strips of 128 pixels (one and
+    # several per row), partial channel tiles, every activation
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 64, 64, 64, 7, 2, 3, A.RELU, scales=(0.02, 0.01, unsat(147))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 224, 224, 64, 7, 2, 3, A.RELU, scales=(0.02, 0.01, unsat(147))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 57, 61, 24, 5, 2, 2, A.IDENTITY, scales=(0.02, 0.01, unsat(75))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 33, 47, 32, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 3, 1, 40, 40, 8, 3, 2, 0, A.H_SWISH, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 4, 30, 150, 96, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(36))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 40, 300, 12, 8, 2, 3, A.SIGMOID, scales=(0.02, 0.01, unsat(192) * 30)),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 2, 19, 23, 128, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(2))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 9, 9, 4, 5, 1, 2, A.RELU, scales=(0.02, 0.01, unsat(75))),
+]
+
+
+@pytest.mark.parametrize("case", HYBRID, ids=[repr(c) for c in HYBRID])
+def test_first_layer_shapes(case):
+    port.set_threads(8)
+    arrays = case.gen(seed=37)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+
+
 OLDER = [
     # shapes the newer kernels take, forced back (development switches of the library) onto the
     # kernels that still serve other shapes: one-stage kernel with split-K (slices of 2 stages out

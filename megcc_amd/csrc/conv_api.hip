@@ -196,7 +196,8 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
         return dwconv44_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     if (q8 && conv_first_supported(g) && aligned4(src->ptr) && aligned4(dst->ptr) && (!b || aligned4(b)))
         return conv_first_launch(g, src->ptr, flt->ptr, b, dst->ptr);
-    if (q8 && conv_hybrid_mfma_supported(g) && aligned4(dst->ptr) && !getenv("MEGCC_NOHYBRID"))
+    if (q8 && conv_hybrid_mfma_supported(g) && aligned4(dst->ptr) && aligned4(flt->ptr) && (!b || aligned4(b)) &&
+        !getenv("MEGCC_NOHYBRID"))
         return conv_hybrid_mfma_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     if (f32 && conv_f32_small_supported(g) && !getenv("MEGCC_NOF32SMALL"))
         return conv_f32_small_launch(g, src->ptr, flt->ptr, b, dst->ptr);

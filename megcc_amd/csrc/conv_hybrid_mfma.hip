@@ -11,13 +11,15 @@
 // columns: 8 bytes that lie next to each other in an LDS copy of the input rows under a strip of
 // output pixels. They are read as four 2-byte pieces (stride 2: the start column 2 * pixel is
 // even) or eight bytes (stride 1).
-//   * a workgroup walks over strips of 128 output pixels of one output row (a wave: 32 pixels x
-//     all output channels); per strip the IC * FH input row pieces go to LDS as bytes, zero where
-//     the image ends - padding costs nothing later;
-//   * the filter is re-ordered to k' once per workgroup into LDS ([chunk of 32 k'][oc][32 bytes])
-//     and read as MFMA A operands;
+//   * a workgroup walks over strips of 128 output pixels x R consecutive output rows (a wave: 32
+//     pixels x all output channels, one output row after the other); per strip the
+//     IC * (FH + (R - 1) * S) input row pieces go to LDS once, zero where the image ends - padding
+//     costs nothing later, and neighbouring output rows share most of their input rows;
+//   * the filter is copied to LDS with coalesced loads and re-ordered there to k' once per
+//     workgroup ([chunk of 32 k'][oc][32 bytes]), then read as MFMA A operands;
 //   * accumulators start from the bias, exact requantisation by threshold table, 4 consecutive
 //     accumulator registers = one NCHW44 dword, 32 lanes store 128 contiguous bytes.
+#include <algorithm>
 #include <map>
 #include <mutex>
 
@@ -31,6 +33,7 @@ namespace mg {
 static constexpr int CH_MAX_OC = 128;    // output channels (4 MFMA row tiles)
 static constexpr int CH_MAX_ROWS = 32;   // IC * FH
 static constexpr int CH_STRIP = 128;     // output pixels per strip
+static constexpr int CH_FILL = 4;        // patch dwords a thread has in flight
 
 struct ChParams {
     const int8_t* src;
@@ -43,7 +46,12 @@ struct ChParams {
     int octiles; // ceil(OC / 32)
     int pitch;   // bytes per LDS row: (CH_STRIP - 1) * S + 8, rounded up to 4
     int strips;  // per output row
-    int items;   // N * OH * strips
+    int R;       // output rows per item
+    int RP;      // input rows per channel under R output rows: FH + (R - 1) * S
+    int ohg;     // ceil(OH / R)
+    int items;   // N * ohg * strips
+    int fbytes;  // OC * FH * FW * IC
+    float inv_pitch4, inv_rp;  // 4 / pitch, 1 / RP
     int act;
     float s_src, s_flt, s_dst, c;
     RequantTable table;
@@ -57,54 +65,104 @@ __device__ __forceinline__ int ch_kernarg_table(int i) {
 
 // S: stride. ACT: IDENTITY / RELU use the table, -1 the literal sequence. OT: MFMA row tiles (OC <= 32 * OT).
 template <int S, int ACT, int OT>
-__global__ void __launch_bounds__(256) conv_hybrid_mfma_kernel(ChParams q) {
+__global__ void __launch_bounds__(256, OT <= 2 ? 4 : 2) conv_hybrid_mfma_kernel(ChParams q) {
     extern __shared__ __attribute__((aligned(16))) int8_t ch_lds[];
     __shared__ int tbl[REQUANT_TABLE_ENTRIES];
     __shared__ __attribute__((aligned(16))) int bias_lds[CH_MAX_OC];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, kg = lane >> 5;
     const int ocp = OT * 32;
     int8_t* const wl = ch_lds;                              // [chunk][ocp][32]
-    int8_t* const patch = ch_lds + q.chunks * ocp * 32;     // [chunks * 4 rows][pitch]
+    int8_t* const patch = ch_lds + q.chunks * ocp * 32;     // [IC][RP][pitch]; first the raw filter
 
-    // ---- once per workgroup: filter in k' order, bias, thresholds ------------------------------
-    for (int i = tid; i < q.chunks * ocp * 32; i += 256) {
-        const int b = i & 31, oc = (i >> 5) % ocp, chunk = (i >> 5) / ocp;
-        const int r = chunk * 4 + (b >> 3), fw = b & 7;
-        int8_t v = 0;
-        if (oc < q.OC && r < q.rows && fw < q.FW) {
-            const int ic = r / q.FH, fh = r - ic * q.FH;
-            v = q.flt[((((size_t)(oc >> 2) * q.FH + fh) * q.FW + fw) * q.IC + ic) * 4 + (oc & 3)];
-        }
-        wl[i] = v;
-    }
+    // ---- once per workgroup: filter in k' order, bias, thresholds, row offsets ------------------
+    for (int i = tid; i < (q.fbytes >> 2); i += 256)
+        ((uint32_t*)patch)[i] = ((const uint32_t*)q.flt)[i];
     if (ACT >= 0)
         tbl[tid] = ch_kernarg_table(tid);
     for (int i = tid; i < ocp; i += 256)
         bias_lds[i] = (q.bias && i < q.OC) ? q.bias[i] : 0;
-    // rows of the patch beyond IC * FH are multiplied by zero weights: any finite bytes do
-    for (int i = tid; i < q.chunks * 4 * q.pitch; i += 256)
-        patch[i] = 0;
+    // k' row r = (ic, fh) lies in patch row ic * RP + fh (+ S per output row); rows beyond IC * FH
+    // are multiplied by zero weights: any patch bytes do. Lane r of every wave keeps the offset of
+    // row r; the chunk loop fetches its four rows with v_readlane.
+    int rtab;
+    {
+        const int r = lane & 31, ic = r / q.FH;
+        rtab = r < q.rows ? (ic * q.RP + r - ic * q.FH) * q.pitch : 0;
+    }
     __syncthreads();
+    // a thread makes 4 bytes of wl: one oc, one (ic, fh), fw0 .. fw0 + 3
+    for (int i = tid; i < q.chunks * ocp * 8; i += 256) {
+        const int b4 = i & 7, oc = (i >> 3) % ocp, chunk = (i >> 3) / ocp;
+        const int r = chunk * 4 + (b4 >> 1), fw0 = (b4 & 1) * 4;
+        uint32_t v = 0;
+        if (oc < q.OC && r < q.rows) {
+            const int ic = r / q.FH, fh = r - ic * q.FH;
+            const uint8_t* f = (const uint8_t*)patch +
+                               ((((oc >> 2) * q.FH + fh) * q.FW + fw0) * q.IC + ic) * 4 + (oc & 3);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (fw0 + j < q.FW)
+                    v |= (uint32_t)f[j * q.IC * 4] << (8 * j);
+        }
+        ((uint32_t*)wl)[i] = v;
+    }
+    __syncthreads();  // the raw filter is overwritten by the first patch
 
     const int ohw = q.OH * q.OW;
+    const int pitch4 = q.pitch >> 2;
     for (int item = blockIdx.x; item < q.items; item += gridDim.x) {
-        const int sx = item % q.strips, row = item / q.strips;
-        const int n = row / q.OH, oh = row - n * q.OH;
+        const int sx = item % q.strips, grp = item / q.strips;
+        const int n = grp / q.ohg, oh0 = (grp - n * q.ohg) * q.R;
         const int ow0 = sx * CH_STRIP;
-        const int ih0 = oh * S - q.PH, iw0 = ow0 * S - q.PW;
-        // ---- input rows under the strip -> LDS (zero outside the image)
+        const int ih0 = oh0 * S - q.PH, iw0 = ow0 * S - q.PW;
+        const int nout = min(q.R, q.OH - oh0);
+        // ---- input rows under the strip -> LDS (zero outside the image). Element = 4 columns of
+        // one row; a thread takes elements tid, tid + 256, ... and requests CH_FILL of them (16
+        // byte loads, addresses clamped into the image, bytes outside it masked afterwards)
+        // before it waits for the first.
         const int8_t* img = q.src + (size_t)n * q.IC * q.IH * q.IW;
-        for (int i = tid; i < q.rows * q.pitch; i += 256) {
-            const int r = i / q.pitch, c = i - r * q.pitch;
-            const int ic = r / q.FH, fh = r - ic * q.FH;
-            const unsigned ih = (unsigned)(ih0 + fh), iw = (unsigned)(iw0 + c);
-            patch[i] = ih < (unsigned)q.IH && iw < (unsigned)q.IW
-                               ? img[((size_t)ic * q.IH + ih) * q.IW + iw]
-                               : (int8_t)0;
+        const int need = (nout - 1) * S + q.FH;  // rows per channel that the nout output rows read
+        const int total = q.IC * q.RP * pitch4;
+        for (int e0 = tid; e0 < total; e0 += 256 * CH_FILL) {
+            uint32_t by[CH_FILL][4];
+            bool ok[CH_FILL][4];
+#pragma unroll
+            for (int u = 0; u < CH_FILL; ++u) {
+                const int e = min(e0 + u * 256, total - 1);
+                // e / pitch4 and row / RP by float: (x + 0.5) / d is at least 0.5 / d away from an
+                // integer, far more than the rounding error for these small numbers
+                const int prow = (int)(((float)e + 0.5f) * q.inv_pitch4);
+                const int c4 = e - prow * pitch4;
+                const int ic = (int)(((float)prow + 0.5f) * q.inv_rp);
+                const int j = prow - ic * q.RP;
+                const int ih = ih0 + j, iw = iw0 + c4 * 4;
+                const bool rowok = (unsigned)ih < (unsigned)q.IH && j < need;
+                const uint8_t* srow =
+                        (const uint8_t*)img + ((size_t)ic * q.IH + min(max(ih, 0), q.IH - 1)) * q.IW;
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    ok[u][b] = rowok && (unsigned)(iw + b) < (unsigned)q.IW;
+                    by[u][b] = srow[min(max(iw + b, 0), q.IW - 1)];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < CH_FILL; ++u) {
+                uint32_t v = 0;
+#pragma unroll
+                for (int b = 0; b < 4; ++b)
+                    v |= ok[u][b] ? by[u][b] << (8 * b) : 0u;
+                if (e0 + u * 256 < total)
+                    ((uint32_t*)patch)[e0 + u * 256] = v;
+            }
         }
         __syncthreads();
 
+        const int px = wave * 32 + col;          // pixel of the strip
+        const int ow = ow0 + px;
+        for (int orow = 0; orow < nout; ++orow) {
+        const int oh = oh0 + orow;
         // ---- this wave's 32 pixels x all output channels
         v16i acc[OT];
 #pragma unroll
@@ -116,35 +174,48 @@ __global__ void __launch_bounds__(256) conv_hybrid_mfma_kernel(ChParams q) {
                 for (int k = 0; k < 4; ++k)
                     acc[t][e4 * 4 + k] = bv[k];
             }
-        const int px = wave * 32 + col;          // pixel of the strip
-        const int8_t* pb = patch + px * S;       // its window starts here in every row
-        for (int chunk = 0; chunk < q.chunks; ++chunk) {
-            // lane's K-bytes: rows chunk * 4 + 2 kg, + 1; 8 columns each
+        const int8_t* pb = patch + px * S + orow * S * q.pitch;  // its window starts here in every row
+        // lane's K-bytes of a chunk: rows chunk * 4 + 2 kg, + 1; 8 columns each
+        auto load_b = [&](int chunk) {
+            const int r0 = __builtin_amdgcn_readlane(rtab, chunk * 4), r1 = __builtin_amdgcn_readlane(rtab, chunk * 4 + 1);
+            const int r2 = __builtin_amdgcn_readlane(rtab, chunk * 4 + 2), r3 = __builtin_amdgcn_readlane(rtab, chunk * 4 + 3);
+            const int ro[2] = {kg ? r2 : r0, kg ? r3 : r1};
             v4i b;
 #pragma unroll
             for (int rr = 0; rr < 2; ++rr) {
-                const int8_t* p = pb + (chunk * 4 + kg * 2 + rr) * q.pitch;
-                if (S == 2) {
-                    const uint16_t* h = (const uint16_t*)p;
-                    b[rr * 2] = (int)((uint32_t)h[0] | ((uint32_t)h[1] << 16));
-                    b[rr * 2 + 1] = (int)((uint32_t)h[2] | ((uint32_t)h[3] << 16));
-                } else {
-                    const uint8_t* u = (const uint8_t*)p;
-                    b[rr * 2] = (int)((uint32_t)u[0] | ((uint32_t)u[1] << 8) | ((uint32_t)u[2] << 16) |
-                                      ((uint32_t)u[3] << 24));
-                    b[rr * 2 + 1] = (int)((uint32_t)u[4] | ((uint32_t)u[5] << 8) | ((uint32_t)u[6] << 16) |
-                                          ((uint32_t)u[7] << 24));
-                }
+                const int8_t* p = pb + ro[rr];
+                // 8 neighbouring bytes from any byte address (LDS reads need no alignment)
+                uint32_t lo, hi;
+                __builtin_memcpy(&lo, p, 4);
+                __builtin_memcpy(&hi, p + 4, 4);
+                b[rr * 2] = (int)lo;
+                b[rr * 2 + 1] = (int)hi;
+            }
+            return b;
+        };
+        const int8_t* wa = wl + col * 32 + kg * 16;
+        v4i bn = load_b(0), an[OT];
+#pragma unroll
+        for (int t = 0; t < OT; ++t)
+            an[t] = *(const v4i*)(wa + t * 32 * 32);
+        for (int chunk = 0; chunk < q.chunks; ++chunk) {
+            const v4i b = bn;
+            v4i a[OT];
+#pragma unroll
+            for (int t = 0; t < OT; ++t)
+                a[t] = an[t];
+            if (chunk + 1 < q.chunks) {
+                bn = load_b(chunk + 1);
+#pragma unroll
+                for (int t = 0; t < OT; ++t)
+                    an[t] = *(const v4i*)(wa + ((chunk + 1) * ocp + t * 32) * 32);
             }
 #pragma unroll
-            for (int t = 0; t < OT; ++t) {
-                const v4i a = *(const v4i*)(wl + ((chunk * ocp + t * 32 + col) * 32 + kg * 16));
-                acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[t], 0, 0, 0);
-            }
+            for (int t = 0; t < OT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b, acc[t], 0, 0, 0);
         }
 
         // ---- epilogue: register e of a tile = channel 8 * (e / 4) + 4 * kg + e % 4, pixel = col
-        const int ow = ow0 + px;
         const int obase = (n * (q.OC >> 2)) * ohw + oh * q.OW + ow;
 #pragma unroll
         for (int t = 0; t < OT; ++t) {
@@ -167,6 +238,7 @@ __global__ void __launch_bounds__(256) conv_hybrid_mfma_kernel(ChParams q) {
                                 pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
                 }
             }
+        }
         }
         __syncthreads();  // the patch is rewritten for the next strip
     }
@@ -195,7 +267,17 @@ TinyNNStatus conv_hybrid_mfma_launch(
     q.octiles = (g.oc + 31) / 32;
     q.pitch = ((CH_STRIP - 1) * g.sh + 8 + 3) & ~3;
     q.strips = (g.ow + CH_STRIP - 1) / CH_STRIP;
-    q.items = g.n * g.oh * q.strips;
+    // several output rows per item share their input rows in LDS; fewer when the problem is too
+    // small to fill the chip otherwise
+    q.R = 4;
+    while (q.R > 1 && (long)g.n * ((g.oh + q.R - 1) / q.R) * q.strips < 4L * num_cus())
+        q.R >>= 1;
+    q.RP = g.fh + (q.R - 1) * g.sh;
+    q.ohg = (g.oh + q.R - 1) / q.R;
+    q.items = g.n * q.ohg * q.strips;
+    q.fbytes = g.oc * g.fh * g.fw * g.ic;
+    q.inv_pitch4 = 4.f / (float)q.pitch;
+    q.inv_rp = 1.f / (float)q.RP;
     q.act = g.act;
     q.s_src = g.s_src; q.s_flt = g.s_flt; q.s_dst = g.s_dst;
     q.c = make_requant_fast(g.s_src, g.s_flt, g.s_dst).c;
@@ -215,7 +297,8 @@ TinyNNStatus conv_hybrid_mfma_launch(
     else
         kern = ot == 1 ? MG_CH_PICK(2, 1) : ot == 2 ? MG_CH_PICK(2, 2) : ot == 3 ? MG_CH_PICK(2, 3) : MG_CH_PICK(2, 4);
 #undef MG_CH_PICK
-    const size_t lds = (size_t)q.chunks * ot * 32 * 32 + (size_t)q.chunks * 4 * q.pitch;
+    const size_t lds = (size_t)q.chunks * ot * 32 * 32 +
+                       std::max((size_t)g.ic * q.RP * q.pitch, (size_t)q.fbytes);
 
     // as many workgroups as are resident at once: the filter set-up is paid once per workgroup
     static std::map<std::pair<const void*, size_t>, int> per_cu;
@@ -237,9 +320,10 @@ TinyNNStatus conv_hybrid_mfma_launch(
         }
         blocks_per_cu = it->second;
     }
+    // equal shares: every workgroup gets ceil(items / resident workgroups) items or one fewer
     long blocks = (long)num_cus() * blocks_per_cu;
-    if (blocks > q.items)
-        blocks = q.items;
+    const long per = (q.items + blocks - 1) / blocks;
+    blocks = (q.items + per - 1) / per;
     void* args[] = {&q};
     hipError_t e = hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, lds, stream());
     MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_hybrid_mfma: %s", hipGetErrorString(e));

@@ -256,6 +256,11 @@ HYBRID = [
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 40, 300, 12, 8, 2, 3, A.SIGMOID, scales=(0.02, 0.01, unsat(192) * 30)),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 2, 19, 23, 128, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(2))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 9, 9, 4, 5, 1, 2, A.RELU, scales=(0.02, 0.01, unsat(75))),
+    # enough rows that a workgroup takes 4 / 2 output rows per strip and shares their input rows
+    # in LDS; the last group of rows is incomplete (62 = 15 * 4 + 2, 63 = 31 * 2 + 1)
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 66, 3, 124, 60, 16, 7, 2, 3, A.RELU, scales=(0.02, 0.01, unsat(147))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 34, 3, 126, 50, 8, 7, 2, 3, A.IDENTITY, scales=(0.02, 0.01, unsat(147))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 40, 2, 30, 140, 8, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(18))),
 ]
 
 

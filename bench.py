@@ -70,8 +70,13 @@ def headline_case(n=32, c=256, hw=56):
 def make_workload(name):
     """-> (case, description, bound, algorithmic units per launch)"""
     from cases import (ConcatCase, ConvCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
-                       TypeCvtCase)
+                       ResizeCase, TypeCvtCase)
     from megcc_amd import abi
+    if name in ("resize_linear", "resize_linear44", "resize_nearest"):
+        fmt = abi.FMT_NCHW44 if name == "resize_linear44" else abi.FMT_NCHW
+        c = 64 if name == "resize_linear44" else 256
+        return (ResizeCase(fmt, "NEAREST" if name == "resize_nearest" else "LINEAR", 8, c, 40, 40, 80, 80),
+                "f32 %s x2 N=8 C=256 40x40 -> 80x80" % name, "hbm")
     if name in ("to_nchw4", "from_nchw4"):
         hw = 56 * 56
         nchw = (256 * hw, 4 * hw, 56, 1, hw)  # a [N, C/4, H, W, 4] view of NCHW memory

@@ -225,6 +225,14 @@ typedef struct {
     int axis;
 } MegccReduceAttr;
 
+/* "imode" of Resize (names as in the kernel symbol) */
+typedef enum { MEGCC_IMODE_NEAREST = 0, MEGCC_IMODE_LINEAR = 1 } MegccInterpMode;
+
+typedef struct {
+    MegccFormat format; /* NCHW, or NCHW44 (LINEAR only) */
+    MegccInterpMode imode;
+} MegccResizeAttr;
+
 /* ------------------------------------------------------------------------------------------
  * Operator entry points. After the attr pointer the argument lists are exactly KernelFunc /
  * InitFunc / WorkspaceFunc of runtime/src/data_struct.h:131-153.
@@ -323,6 +331,16 @@ TinyNNStatus megcc_gfx950_concat(
         const int* axis, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
         const Workspace* workspace, const RuntimeOpt* opt);
 
+/* f32 Resize of the two spatial dims: inputs = {src [N,C,IH,IW] or [N,C/4,IH,IW,4] (, target
+ * shape: never read)}, outputs = {dst with OH, OW}. LINEAR: half-pixel centres, edges clamped,
+ * dense tensors; NEAREST: floor(o / (O / I)), the source is read through its strides. Replaces
+ * GeneralIntrinsic::ResizeKernel (GeneralIntrinsic/Resize.cpp:13-83,
+ * GI_kernel_resize_linear_<fmt>_LINEAR_f32) and BareMetal::ResizeKernel (BareMetal/Resize.cpp:15-106,
+ * kernel_resize_linear_<fmt>_<imode>_f32); arithmetic of Common/Resize.h:16-175. */
+TinyNNStatus megcc_gfx950_resize(
+        const MegccResizeAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs,
+        int nr_output, const Workspace* workspace, const RuntimeOpt* opt);
+
 /* ------------------------------------------------------------------------------------------
  * Dispatch by the reference's kernel symbol: lets a caller that only knows the generated name
  * (e.g. "kernel_conv2d_3x3_NCHW44_DENSE_p1x1_s1x1_d1x1_qsi8qsi8qsi32qsi8_bias_RELU",
@@ -338,7 +356,8 @@ typedef enum {
     MEGCC_KERN_TYPECVT = 6,
     MEGCC_KERN_REDUCE = 7,
     MEGCC_KERN_RELAYOUT = 8,
-    MEGCC_KERN_CONCAT = 9
+    MEGCC_KERN_CONCAT = 9,
+    MEGCC_KERN_RESIZE = 10
 } MegccKernelKind;
 
 typedef struct {
@@ -351,6 +370,7 @@ typedef struct {
         MegccElemwiseMode elemwise;
         MegccReduceAttr reduce;
         int concat_axis;
+        MegccResizeAttr resize;
     } attr;
 } MegccKernelDesc;
 

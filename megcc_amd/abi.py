@@ -42,7 +42,8 @@ REDUCE_SUM, REDUCE_MEAN, REDUCE_MAX, REDUCE_MIN = 0, 1, 2, 3
 # MegccKernelKind
 KERN_CONV, KERN_MATMUL, KERN_POOLING, KERN_ELEMWISE_MULTITYPE = 1, 2, 3, 4
 KERN_ELEMWISE, KERN_TYPECVT, KERN_REDUCE = 5, 6, 7
-KERN_RELAYOUT, KERN_CONCAT = 8, 9
+KERN_RELAYOUT, KERN_CONCAT, KERN_RESIZE = 8, 9, 10
+IMODE_NEAREST, IMODE_LINEAR = 0, 1
 
 
 class Device(C.Structure):
@@ -124,11 +125,15 @@ class ReduceAttr(C.Structure):
     _fields_ = [("mode", C.c_int), ("axis", C.c_int)]
 
 
+class ResizeAttr(C.Structure):
+    _fields_ = [("format", C.c_int), ("imode", C.c_int)]
+
+
 class _KernelAttrUnion(C.Union):
     _fields_ = [
         ("conv", ConvAttr), ("matmul", MatMulAttr), ("pool", PoolAttr),
         ("multitype", C.c_int), ("elemwise", C.c_int), ("reduce", ReduceAttr),
-        ("concat_axis", C.c_int),
+        ("concat_axis", C.c_int), ("resize", ResizeAttr),
     ]
 
 

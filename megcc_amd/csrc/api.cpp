@@ -217,6 +217,18 @@ extern "C" TinyNNStatus megcc_gfx950_parse_symbol(const char* symbol, MegccKerne
             desc->kind = MEGCC_KERN_RELAYOUT;
             return TinyNN_SUCCESS;
         }
+    } else if (eat(s, "GI_kernel_resize_linear_") || eat(s, "kernel_resize_linear_")) {
+        // <format>_<imode>_f32
+        const bool p4 = eat(s, "NCHW44_");
+        if (p4 || eat(s, "NCHW_")) {
+            const bool linear = eat(s, "LINEAR_");
+            if ((linear || (!p4 && eat(s, "NEAREST_"))) && s == "f32") {
+                desc->kind = MEGCC_KERN_RESIZE;
+                desc->attr.resize.format = p4 ? MEGCC_FMT_NCHW44 : MEGCC_FMT_NCHW;
+                desc->attr.resize.imode = linear ? MEGCC_IMODE_LINEAR : MEGCC_IMODE_NEAREST;
+                return TinyNN_SUCCESS;
+            }
+        }
     } else if (eat(s, "kernel_concat_byte_")) {
         int bytes = 0, axis = -1;
         char tail = 0;
@@ -261,6 +273,8 @@ extern "C" TinyNNStatus megcc_gfx950_call(
             return megcc_gfx950_reduce(&d->attr.reduce, inputs, nr_input, outputs, nr_output, ws, opt);
         case MEGCC_KERN_RELAYOUT:
             return megcc_gfx950_relayout(inputs, nr_input, outputs, nr_output, ws, opt);
+        case MEGCC_KERN_RESIZE:
+            return megcc_gfx950_resize(&d->attr.resize, inputs, nr_input, outputs, nr_output, ws, opt);
         case MEGCC_KERN_CONCAT:
             return megcc_gfx950_concat(&d->attr.concat_axis, inputs, nr_input, outputs, nr_output,
                                        ws, opt);

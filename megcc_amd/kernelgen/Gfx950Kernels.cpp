@@ -9,6 +9,7 @@
 //   elemwise  BareMetal/ElemwiseKernel.cpp:433-439
 //   reduce    BareMetal/Reduce.cpp:82-90
 //   matmul    BareMetal/MatrixMul.cpp:26-41
+//   resize    GeneralIntrinsic/Resize.cpp:25-33 (LINEAR), BareMetal/Resize.cpp:27-35 (NEAREST)
 //   relayout  GeneralIntrinsic/Relayout.cpp:43-48 (first in the x86 list for 1/2/4-byte dtypes)
 //   concat    BareMetal/Concat.cpp:14-22
 // (for f32 conv / matmul / elemwise / reduce the x86 registry prefers GI variants whose names
@@ -470,6 +471,29 @@ struct ConcatKernel : KernelFuncBase {
     }
 };
 
+// ---- Resize (f32; GeneralIntrinsic/Resize.cpp:13-33 for LINEAR, BareMetal/Resize.cpp:15-35) ----
+struct ResizeKernel : KernelFuncBase {
+    bool IsAvailable(TContext* c) const override {
+        const std::string imode = c->getAttrStr("imode"), fmt = c->getAttrStr("format");
+        return is_f32(c->getAttrOprand("operand:0").dtype) &&
+               ((imode == "LINEAR" && (fmt == "NCHW" || fmt == "NCHW44")) ||
+                (imode == "NEAREST" && fmt == "NCHW"));
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        const std::string imode = c->getAttrStr("imode");
+        return std::string(imode == "LINEAR" ? "GI_" : "") + "kernel_resize_linear_" +
+               c->getAttrStr("format") + "_" + imode + "_" + c->getAttrOprand("operand:0").dtype;
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        std::stringstream a;
+        a << "    static const MegccResizeAttr attr = {MEGCC_FMT_" << c->getAttrStr("format")
+          << ", MEGCC_IMODE_" << c->getAttrStr("imode") << "};\n";
+        return kHeader + kernel_def(this, c, a.str(),
+                                    "megcc_gfx950_resize(&attr, inputs, nr_input, outputs, "
+                                    "nr_output, workspace, opt)");
+    }
+};
+
 // ---- MatrixMul (f32) ---------------------------------------------------------------------------
 struct MatrixMulKernel : KernelFuncBase {
     bool IsAvailable(TContext* c) const override {
@@ -516,6 +540,7 @@ std::vector<const KernelFuncBase*> Gfx950KernelPack::GetKernel(KernType type) {
     static const MatrixMulKernel matmul;
     static const RelayoutKernel relayout;
     static const ConcatKernel concat;
+    static const ResizeKernel resize;
     switch (type) {
         case KernType::ConvKernel: return {&conv};
         case KernType::PoolingKernel: return {&pool};
@@ -526,6 +551,7 @@ std::vector<const KernelFuncBase*> Gfx950KernelPack::GetKernel(KernType type) {
         case KernType::MatrixMulKernel: return {&matmul};
         case KernType::RelayoutKernel: return {&relayout};
         case KernType::ConcatKernel: return {&concat};
+        case KernType::ResizeKernel: return {&resize};
         default: return {};
     }
 }

@@ -92,6 +92,7 @@ enum class KernType {
     RelayoutKernel = 7,
     ReduceKernel = 8,
     TypeCvtKernel = 13,
+    ResizeKernel = 19,
     ConcatKernel = 25,
 };
 

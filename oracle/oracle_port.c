@@ -458,3 +458,72 @@ void orc_concat(
         at += lens[i];
     }
 }
+
+/* Resize, f32. Common/Resize.h:16-40 (get_coord), :42-101 (LINEAR body, NCHW / NCHW44 through
+ * get_offset :209-225), :158-175 (NEAREST, strided NCHW source). scale = (float)O / I. */
+static void orc_resize_coord(float scale, int size, int idx, float* a0, int* i0, float* a1, int* i1) {
+    if (size == 1) {
+        *a0 = 1.f; *i0 = 0; *a1 = 0.f; *i1 = 0;
+        return;
+    }
+    float alpha = (idx + 0.5f) / scale - 0.5f;
+    int origin = (int)floorf(alpha);
+    alpha -= origin;
+    if (origin < 0) {
+        origin = 0;
+        alpha = 0;
+    } else if (origin + 1 >= size) {
+        origin = size - 2;
+        alpha = 1;
+    }
+    *a0 = 1 - alpha; *i0 = origin; *a1 = alpha; *i1 = origin + 1;
+}
+
+static size_t orc_resize_off(int pack4, size_t h, size_t w, size_t c, size_t H, size_t W) {
+    return pack4 ? ((((c >> 2) * H * W + h * W + w) << 2) + (c & 3)) : c * H * W + h * W + w;
+}
+
+/* C counts channels (4 * dims[1] for NCHW44) */
+void orc_resize_linear_f32(
+        const float* src, float* dst, int N, int C, int IH, int IW, int OH, int OW, int pack4) {
+    const float scale_h = (float)OH / IH, scale_w = (float)OW / IW;
+    for (int n = 0; n < N; ++n) {
+        for (int c = 0; c < C; ++c)
+            for (int oh = 0; oh < OH; ++oh) {
+                int ih0, ih1;
+                float ah0, ah1;
+                orc_resize_coord(scale_h, IH, oh, &ah0, &ih0, &ah1, &ih1);
+                for (int ow = 0; ow < OW; ++ow) {
+                    int iw0, iw1;
+                    float aw0, aw1;
+                    orc_resize_coord(scale_w, IW, ow, &aw0, &iw0, &aw1, &iw1);
+                    dst[orc_resize_off(pack4, oh, ow, c, OH, OW)] =
+                            src[orc_resize_off(pack4, ih0, iw0, c, IH, IW)] * ah0 * aw0 +
+                            src[orc_resize_off(pack4, ih0, iw1, c, IH, IW)] * ah0 * aw1 +
+                            src[orc_resize_off(pack4, ih1, iw0, c, IH, IW)] * ah1 * aw0 +
+                            src[orc_resize_off(pack4, ih1, iw1, c, IH, IW)] * ah1 * aw1;
+                }
+            }
+        src += (size_t)C * IH * IW;
+        dst += (size_t)C * OH * OW;
+    }
+}
+
+/* source strides in elements; dense NCHW destination */
+void orc_resize_nearest_f32(
+        const float* src, float* dst, int N, int C, int IH, int IW, int OH, int OW, int64_t s_n,
+        int64_t s_c, int64_t s_h, int64_t s_w) {
+    const float scale_h = (float)OH / IH, scale_w = (float)OW / IW;
+    for (int n = 0; n < N; ++n) {
+        for (int oh = 0; oh < OH; ++oh)
+            for (int ow = 0; ow < OW; ++ow) {
+                int ih = (int)(oh / scale_h), iw = (int)(ow / scale_w);
+                ih = ih < IH - 1 ? ih : IH - 1;
+                iw = iw < IW - 1 ? iw : IW - 1;
+                for (int c = 0; c < C; ++c)
+                    dst[(size_t)c * OH * OW + (size_t)oh * OW + ow] = src[c * s_c + ih * s_h + iw * s_w];
+            }
+        src += s_n;
+        dst += (size_t)C * OH * OW;
+    }
+}

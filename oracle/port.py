@@ -186,3 +186,24 @@ def concat(arrays, axis):
     lib().orc_concat(ptrs, _p(lens), len(arrays), _p(dst), C.c_int64(outer), C.c_int64(inner),
                      dst.itemsize)
     return dst
+
+
+def resize(src, out_hw, imode, nchw44=False, src_strides=None, src_shape=None):
+    """f32 Resize. `src` dense [N,C,H,W] / [N,C/4,H,W,4]; for NEAREST the source may be a
+    strided NCHW view of a dense buffer (`src_shape`, `src_strides` in elements)."""
+    oh, ow = out_hw
+    shape = tuple(src_shape) if src_shape is not None else src.shape
+    n, c, ih, iw = shape[:4]
+    src = np.ascontiguousarray(src, dtype=np.float32)
+    if imode == "LINEAR":
+        assert src_strides is None
+        dst = np.empty((n, c, oh, ow, 4) if nchw44 else (n, c, oh, ow), np.float32)
+        lib().orc_resize_linear_f32(_p(src), _p(dst), n, c * 4 if nchw44 else c, ih, iw, oh, ow,
+                                    1 if nchw44 else 0)
+        return dst
+    assert imode == "NEAREST" and not nchw44
+    st = src_strides if src_strides is not None else (c * ih * iw, ih * iw, iw, 1)
+    dst = np.empty((n, c, oh, ow), np.float32)
+    lib().orc_resize_nearest_f32(_p(src), _p(dst), n, c, ih, iw, oh, ow,
+                                 *[C.c_int64(int(v)) for v in st])
+    return dst

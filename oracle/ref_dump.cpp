@@ -44,6 +44,7 @@ static const std::map<std::string, KT> kTypes = {
         {"TypeCvtKernel", KT::TypeCvtKernel},
         {"RelayoutKernel", KT::RelayoutKernel},
         {"ConcatKernel", KT::ConcatKernel},
+        {"ResizeKernel", KT::ResizeKernel},
 };
 
 static CCOperand parse_operand(const std::string& v) {

@@ -518,6 +518,61 @@ class ConcatCase:
         return port.concat([arrays["in%d" % i] for i in range(len(self.shapes))], self.axis)
 
 
+class ResizeCase:
+    """f32 Resize [N,C,IH,IW] -> [N,C,OH,OW] (NCHW; `c` counts blocks of 4 for NCHW44).
+    NEAREST reads its source through the tensor's strides (Common/Resize.h:158-175):
+    `src_strides` (elements, positive) makes the source a view of a larger dense buffer."""
+
+    def __init__(self, fmt, imode, n, c, ih, iw, oh, ow, src_strides=None):
+        assert fmt in (abi.FMT_NCHW, abi.FMT_NCHW44) and imode in ("LINEAR", "NEAREST")
+        assert src_strides is None or (imode == "NEAREST" and fmt == abi.FMT_NCHW)
+        self.fmt, self.imode = fmt, imode
+        self.n, self.c, self.ih, self.iw, self.oh, self.ow = n, c, ih, iw, oh, ow
+        self.src_strides = None if src_strides is None else tuple(src_strides)
+
+    def _fmt(self):
+        return "NCHW44" if self.fmt == abi.FMT_NCHW44 else "NCHW"
+
+    def __repr__(self):
+        return "resize_%s_%s[n%d c%d %dx%d->%dx%d%s]" % (
+            self._fmt(), self.imode, self.n, self.c, self.ih, self.iw, self.oh, self.ow,
+            "" if self.src_strides is None else " strides " + "x".join(map(str, self.src_strides)))
+
+    def src_shape(self):
+        tail = (4,) if self.fmt == abi.FMT_NCHW44 else ()
+        return (self.n, self.c, self.ih, self.iw) + tail
+
+    def dst_shape(self):
+        tail = (4,) if self.fmt == abi.FMT_NCHW44 else ()
+        return (self.n, self.c, self.oh, self.ow) + tail
+
+    def symbol(self):
+        # GeneralIntrinsic/Resize.cpp:13-33 takes LINEAR, BareMetal/Resize.cpp:15-35 NEAREST
+        return "%skernel_resize_linear_%s_%s_f32" % ("GI_" if self.imode == "LINEAR" else "",
+                                                      self._fmt(), self.imode)
+
+    def spec_line(self):
+        return "ResizeKernel imode=s:%s format=s:%s nr_operands=i:2 operand:0=%s operand:1=%s" % (
+            self.imode, self._fmt(), _op(self.src_shape(), "f32"), _op(self.dst_shape(), "f32"))
+
+    def gen(self, seed=0):
+        r = rng(seed)
+        if self.src_strides is None:
+            return {"src": r.uniform(-30, 30, self.src_shape()).astype(np.float32)}
+        _, hi = span_of(self.src_shape(), self.src_strides)
+        return {"src": r.uniform(-30, 30, hi + 1 + 3).astype(np.float32)}
+
+    def specs(self, arrays):
+        return ([TensorSpec(b"src", self.src_shape(), abi.FLOAT, 1.0, arrays["src"],
+                            self.src_strides, 0)],
+                [TensorSpec(b"dst", self.dst_shape(), abi.FLOAT, 1.0)])
+
+    def run_port(self, arrays):
+        return port.resize(arrays["src"], (self.oh, self.ow), self.imode,
+                           self.fmt == abi.FMT_NCHW44, self.src_strides,
+                           self.src_shape() if self.src_strides is not None else None)
+
+
 def run_ref(case, arrays, symbol=None):
     """Evaluate `case` with the reference's generated C kernel; returns the output array."""
     ins, outs = case.specs(arrays)

@@ -5,7 +5,7 @@ typecvt.cpp:5-70): odd sizes, k in {1,3}, stride in {1,2}, pad in {0,k/2}, every
 small-magnitude tie case and the 30..50 overflow case."""
 from megcc_amd import abi
 from cases import (ConcatCase, ConvCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
-                   TypeCvtCase)
+                   ResizeCase, TypeCvtCase)
 
 A = abi
 
@@ -123,4 +123,19 @@ def golden_cases():
                 sh[axis] = i + 1
                 shapes.append(tuple(sh))
             c["concat_%s_axis%d" % (dt, axis)] = ConcatCase(dt, shapes, axis)
+    # --- resize: the shapes of compiler/test/kernel/opr/naive/resize.cpp:7-35 (up and down, both
+    # at once), then the corners of get_coord: extent 1 in and out, same size, a strided source
+    for i, (n, ch, ih, iw, oh, ow) in enumerate(((1, 1, 5, 6, 7, 13), (1, 4, 5, 6, 9, 12),
+                                                  (2, 3, 15, 16, 9, 12))):
+        c["resize_linear_nchw_%d" % i] = ResizeCase(A.FMT_NCHW, "LINEAR", n, ch, ih, iw, oh, ow)
+        c["resize_linear_nchw44_%d" % i] = ResizeCase(A.FMT_NCHW44, "LINEAR", n, ch, ih, iw, oh, ow)
+        c["resize_nearest_nchw_%d" % i] = ResizeCase(A.FMT_NCHW, "NEAREST", n, ch, ih, iw, oh, ow)
+    c["resize_linear_nchw_from_1x1"] = ResizeCase(A.FMT_NCHW, "LINEAR", 2, 3, 1, 1, 4, 5)
+    c["resize_linear_nchw_row"] = ResizeCase(A.FMT_NCHW, "LINEAR", 1, 2, 1, 7, 3, 10)
+    c["resize_linear_nchw_to_1x1"] = ResizeCase(A.FMT_NCHW, "LINEAR", 1, 2, 6, 9, 1, 1)
+    c["resize_linear_nchw44_same"] = ResizeCase(A.FMT_NCHW44, "LINEAR", 1, 2, 6, 5, 6, 5)
+    c["resize_linear_nchw_x2"] = ResizeCase(A.FMT_NCHW, "LINEAR", 1, 3, 8, 10, 16, 20)
+    c["resize_nearest_nchw_x2"] = ResizeCase(A.FMT_NCHW, "NEAREST", 1, 3, 8, 10, 16, 20)
+    c["resize_nearest_nchw_view"] = ResizeCase(A.FMT_NCHW, "NEAREST", 2, 3, 6, 5, 9, 11,
+                                               src_strides=(400, 120, 20, 2))
     return c

@@ -44,7 +44,7 @@ with open(os.path.join(HERE, "golden", "symbols.json")) as f:
 @pytest.mark.parametrize("symbol", sorted(set(SYMBOLS.values())))
 def test_every_reference_symbol_parses(symbol):
     desc = runtime.parse_symbol(symbol)
-    assert desc.kind in range(1, 10)
+    assert desc.kind in range(1, 11)
 
 
 def test_parse_conv_symbol_fields():
@@ -82,6 +82,11 @@ def test_parse_other_symbols():
         assert runtime.parse_symbol(sym).kind == abi.KERN_RELAYOUT
     d = runtime.parse_symbol("kernel_concat_byte_4_axis_2")
     assert d.kind == abi.KERN_CONCAT and d.attr.concat_axis == 2
+    d = runtime.parse_symbol("GI_kernel_resize_linear_NCHW44_LINEAR_f32")
+    assert d.kind == abi.KERN_RESIZE
+    assert (d.attr.resize.format, d.attr.resize.imode) == (abi.FMT_NCHW44, abi.IMODE_LINEAR)
+    d = runtime.parse_symbol("kernel_resize_linear_NCHW_NEAREST_f32")
+    assert (d.attr.resize.format, d.attr.resize.imode) == (abi.FMT_NCHW, abi.IMODE_NEAREST)
 
 
 def test_copy_kernels_reject_bad_arguments_before_any_launch():
@@ -108,12 +113,25 @@ def test_copy_kernels_reject_bad_arguments_before_any_launch():
     assert call(L.megcc_gfx950_concat, [t((2, 3))], t((2, 3)), C.byref(axis)) == \
         abi.ERROR_OUT_OF_RANGE
     assert L.megcc_gfx950_concat(None, None, 0, None, 0, None, None) == abi.ERROR_NULL_PTR
+    lin = abi.ResizeAttr(abi.FMT_NCHW, abi.IMODE_LINEAR)
+    assert call(L.megcc_gfx950_resize, [t((1, 2, 4, 4))], t((1, 3, 8, 8)), C.byref(lin)) == \
+        abi.ERROR_INVALID_LAYOUT  # channels differ
+    assert call(L.megcc_gfx950_resize, [t((1, 2, 4, 4), strides=(64, 32, 8, 2))], t((1, 2, 8, 8)),
+                C.byref(lin)) == abi.ERROR_INVALID_LAYOUT  # LINEAR reads dense tensors only
+    assert call(L.megcc_gfx950_resize, [t((1, 2, 4, 4), abi.QINT8)], t((1, 2, 8, 8), abi.QINT8),
+                C.byref(lin)) == abi.ERROR_UNSUPPORTED_DTYPE_TYPE
+    assert call(L.megcc_gfx950_resize, [t((1, 2, 4, 4))], t((1, 2, 0, 8)), C.byref(lin)) == 0
+    near44 = abi.ResizeAttr(abi.FMT_NCHW44, abi.IMODE_NEAREST)
+    assert call(L.megcc_gfx950_resize, [t((1, 2, 4, 4, 4))], t((1, 2, 8, 8, 4)),
+                C.byref(near44)) == abi.ERROR_OUT_OF_RANGE  # no such kernel in the reference
+    assert L.megcc_gfx950_resize(None, None, 0, None, 0, None, None) == abi.ERROR_NULL_PTR
 
 
 def test_unknown_symbol_is_reported_not_guessed():
     desc = abi.KernelDesc()
     for bad in ("kernel_argsort_f32", "kernel_relayout_f64", "kernel_concat_byte_8_axis_0",
-                "kernel_concat_byte_4_axis_1x", "kernel_conv2d_3x3_NHWC_DENSE_p1x1_s1x1_d1x1_f32f32f32",
+                "kernel_concat_byte_4_axis_1x", "kernel_resize_linear_NCHW44_NEAREST_f32",
+                "GI_kernel_resize_linear_NHWC_LINEAR_f32", "kernel_resize_linear_NCHW_LINEAR_f16", "kernel_conv2d_3x3_NHWC_DENSE_p1x1_s1x1_d1x1_f32f32f32",
                 "kernel_typecvt_f16f32", ""):
         st = runtime.lib().megcc_gfx950_parse_symbol(bad.encode(), C.byref(desc))
         assert st == abi.ERROR_NO_FOUND

@@ -11,7 +11,7 @@ import pytest
 
 import cases
 from cases import (ConcatCase, ConvCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
-                   TypeCvtCase)
+                   ResizeCase, TypeCvtCase)
 from golden_cases import golden_cases, unsat
 from megcc_amd import abi, runtime
 from oracle import port
@@ -269,6 +269,31 @@ def test_first_layer_shapes(case):
     port.set_threads(8)
     arrays = case.gen(seed=37)
     compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+
+
+RESIZE = [
+    # the 2x upsampling of detection necks, a camera frame scaled down to a network input, odd
+    # ratios, extent 1 either side, a channel slice with a column step as NEAREST source
+    ResizeCase(A.FMT_NCHW, "LINEAR", 2, 16, 40, 52, 80, 104),
+    ResizeCase(A.FMT_NCHW44, "LINEAR", 2, 8, 40, 52, 80, 104),
+    ResizeCase(A.FMT_NCHW, "NEAREST", 2, 16, 40, 52, 80, 104),
+    ResizeCase(A.FMT_NCHW, "LINEAR", 1, 3, 480, 640, 224, 224),
+    ResizeCase(A.FMT_NCHW44, "LINEAR", 3, 2, 37, 53, 111, 29),
+    ResizeCase(A.FMT_NCHW, "LINEAR", 3, 5, 17, 1, 33, 7),
+    ResizeCase(A.FMT_NCHW, "LINEAR", 2, 3, 1, 19, 1, 300),
+    ResizeCase(A.FMT_NCHW, "LINEAR", 1, 2, 5, 700, 3, 2500),  # rows longer than the column table
+    ResizeCase(A.FMT_NCHW, "NEAREST", 3, 7, 31, 45, 17, 101),
+    ResizeCase(A.FMT_NCHW, "NEAREST", 2, 5, 33, 47, 100, 31, src_strides=(40000, 3300, 100, 2)),
+]
+
+
+@pytest.mark.parametrize("case", RESIZE, ids=[repr(c) for c in RESIZE])
+def test_resize(case):
+    arrays = case.gen(seed=41)
+    got, want = run_gpu(case, arrays), case.run_port(arrays)
+    compare(got, want, repr(case))
+    # the kernels keep the reference's order of operations: equal bit for bit
+    assert np.array_equal(got, want), repr(case)
 
 
 OLDER = [

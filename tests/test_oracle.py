@@ -213,3 +213,47 @@ def test_port_matmul_vs_float64():
     a = case.gen(4)
     want = a["a"].astype(np.float64) @ a["b"].astype(np.float64)
     assert cases.max_rel_err(case.run_port(a), want) <= 1e-5
+
+
+def test_port_resize_closed_forms():
+    """what the mathematics fixes for Resize: same size = copy; a constant image stays constant; a
+    plane that is affine in (h, w) is reproduced exactly by bilinear weights wherever the
+    half-pixel source coordinate lies inside the image (no edge clamping); NEAREST equals
+    numpy indexing with floor(o * I / O) for integer ratios."""
+    r = np.random.default_rng(5)
+    x = r.uniform(-30, 30, (2, 3, 6, 5)).astype(np.float32)
+    assert np.array_equal(port.resize(x, (6, 5), "LINEAR"), x)
+    x4 = r.uniform(-30, 30, (1, 2, 6, 5, 4)).astype(np.float32)
+    assert np.array_equal(port.resize(x4, (6, 5), "LINEAR", nchw44=True), x4)
+    const = np.full((1, 2, 4, 7), 3.25, np.float32)
+    # (dyadic weights at ratio 2: no rounding at all; any ratio: within rounding)
+    assert np.array_equal(port.resize(const, (8, 14), "LINEAR"), np.full((1, 2, 8, 14), 3.25, np.float32))
+    np.testing.assert_allclose(port.resize(const, (9, 3), "LINEAR"), 3.25, rtol=1e-6)
+    # affine plane, exactly representable values: 2x upscale of f(h, w) = 8 h + w
+    ih, iw = 8, 8
+    hh, ww = np.meshgrid(np.arange(ih), np.arange(iw), indexing="ij")
+    plane = (8.0 * hh + ww).astype(np.float32)[None, None]
+    got = port.resize(plane, (16, 16), "LINEAR")[0, 0]
+    oh = (np.arange(16) + 0.5) / 2 - 0.5
+    want = 8.0 * oh[:, None] + oh[None, :]
+    inside = (oh >= 0) & (oh <= ih - 1)
+    assert np.array_equal(got[np.ix_(inside, inside)], want[np.ix_(inside, inside)].astype(np.float32))
+    # edges clamp to the border rows / columns
+    assert got[0, 5] == got[0, 5] and np.array_equal(got[0, inside], (8.0 * 0 + oh[inside]).astype(np.float32))
+    # NCHW44 is the same function on interleaved channels
+    y = r.uniform(-30, 30, (2, 8, 5, 6)).astype(np.float32)
+    y44 = np.ascontiguousarray(y.reshape(2, 2, 4, 5, 6).transpose(0, 1, 3, 4, 2))
+    a = port.resize(y, (7, 13), "LINEAR")
+    b = port.resize(y44, (7, 13), "LINEAR", nchw44=True)
+    assert np.array_equal(b.transpose(0, 1, 4, 2, 3).reshape(2, 8, 7, 13), a)
+    # NEAREST, integer ratios up and down
+    z = r.uniform(-30, 30, (1, 2, 6, 8)).astype(np.float32)
+    assert np.array_equal(port.resize(z, (12, 24), "NEAREST"),
+                          z[:, :, np.arange(12) // 2][:, :, :, np.arange(24) // 3])
+    assert np.array_equal(port.resize(z, (3, 4), "NEAREST"), z[:, :, ::2, ::2])
+    # strided source = the same result as on a dense copy of the view
+    buf = r.uniform(-30, 30, 2 * 400 + 8).astype(np.float32)
+    view = np.lib.stride_tricks.as_strided(buf, (2, 3, 6, 5), [4 * s for s in (400, 120, 20, 2)])
+    assert np.array_equal(
+        port.resize(buf, (9, 11), "NEAREST", src_strides=(400, 120, 20, 2), src_shape=(2, 3, 6, 5)),
+        port.resize(np.ascontiguousarray(view), (9, 11), "NEAREST"))

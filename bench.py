@@ -69,9 +69,13 @@ def headline_case(n=32, c=256, hw=56):
 
 def make_workload(name):
     """-> (case, description, bound, algorithmic units per launch)"""
-    from cases import (ConcatCase, ConvCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
-                       ResizeCase, TypeCvtCase)
+    from cases import (ConcatCase, ConvCase, FusedCase, MatMulCase, MultiTypeCase, PoolCase,
+                       RelayoutCase, ResizeCase, TypeCvtCase)
     from megcc_amd import abi
+    if name == "fused":
+        return (FusedCase(["I0,SILU,O0", "O0,I1,MUL,O1", "O1,I2,ADD,D"],
+                          [(8, 256, 80, 80), (1, 256, 1, 1), (1, 256, 1, 1)]),
+                "f32 fused SiLU(x) * scale[c] + shift[c], N=8 C=256 80x80", "hbm")
     if name in ("resize_linear", "resize_linear44", "resize_nearest"):
         fmt = abi.FMT_NCHW44 if name == "resize_linear44" else abi.FMT_NCHW
         c = 64 if name == "resize_linear44" else 256
@@ -250,7 +254,8 @@ def main():
     case, desc, bound = make_workload(args.workload)
     arrays = case.gen(seed=0)
     ins, outs = case.specs(arrays)
-    op = runtime.PreparedOp(runtime.parse_symbol(case.symbol()), ins, outs)
+    kdesc = case.desc() if hasattr(case, "desc") else runtime.parse_symbol(case.symbol())
+    op = runtime.PreparedOp(kdesc, ins, outs)
     ev = HipEvents(runtime.lib().megcc_gfx950_stream())
 
     for _ in range(args.warmup):

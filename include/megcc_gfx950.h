@@ -210,7 +210,20 @@ typedef enum {
     MEGCC_EW_TRUE_DIV = 19,
     MEGCC_EW_MAX = 20,
     MEGCC_EW_MIN = 21,
-    MEGCC_EW_FUSE_ADD_RELU = 22
+    MEGCC_EW_FUSE_ADD_RELU = 22,
+    /* the modes below exist only as steps of a fused elementwise program */
+    MEGCC_EW_ABS = 5,
+    MEGCC_EW_LOG = 6,
+    MEGCC_EW_SILU = 7,
+    MEGCC_EW_ROUND = 8,
+    MEGCC_EW_LT = 23,
+    MEGCC_EW_LEQ = 24,
+    MEGCC_EW_EQ = 25,
+    MEGCC_EW_FLOOR_DIV = 26,
+    MEGCC_EW_FUSE_ADD_SIGMOID = 27,
+    MEGCC_EW_FUSE_ADD_TANH = 28,
+    MEGCC_EW_FUSE_MUL_ADD3 = 32, /* a * b + c         */
+    MEGCC_EW_FUSE_MUL_ADD4 = 33  /* a * b + c * d     */
 } MegccElemwiseMode;
 
 typedef enum {
@@ -224,6 +237,24 @@ typedef struct {
     MegccReduceMode mode;
     int axis;
 } MegccReduceAttr;
+
+/* A fused chain of f32 elementwise steps: the "modes:<i>" attributes of FusedElemwiseKernel
+ * ("I0,I1,ADD,O0", "O0,I2,MUL,D", ...: BareMetal/FusedElemwiseKernel.cpp:126-153,286-306) with the
+ * names resolved to value numbers. Value k < nr_input is input k; value nr_input + j is the
+ * result of step j; the result of the last step is the output. */
+#define MEGCC_FUSED_MAX_STEPS 16
+#define MEGCC_FUSED_MAX_INPUTS 8
+typedef struct {
+    MegccElemwiseMode mode;
+    int nr_arg;  /* 1..4 */
+    int arg[4];  /* value numbers */
+} MegccFusedStep;
+
+typedef struct {
+    int nr_input;
+    int nr_step;
+    MegccFusedStep step[MEGCC_FUSED_MAX_STEPS];
+} MegccFusedElemwiseAttr;
 
 /* "imode" of Resize (names as in the kernel symbol) */
 typedef enum { MEGCC_IMODE_NEAREST = 0, MEGCC_IMODE_LINEAR = 1 } MegccInterpMode;
@@ -341,6 +372,19 @@ TinyNNStatus megcc_gfx950_resize(
         const MegccResizeAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs,
         int nr_output, const Workspace* workspace, const RuntimeOpt* opt);
 
+/* Fused f32 elementwise chain over a dense output: inputs = the attr's nr_input tensors, each
+ * either of the output's element count, a single element, [1,C,1,1] under a >= 4-d output or
+ * [1,C,1,1,4] under a 5-d one (Common/ElemwiseCommon.cpp:7-45; reads as in
+ * BareMetal/FusedElemwiseKernel.cpp:159-219). Replaces BareMetal::FusedElmwiseKernel
+ * (BareMetal/FusedElemwiseKernel.cpp:270-423, kernel_naive_fused_elementwise_*) and
+ * GeneralIntrinsic::FusedElmwiseKernel (GeneralIntrinsic/FusedElemwiseKernel.cpp:680-726,
+ * kernel_gi_fused_elementwise_*). The reference's symbol names only the modes and operand kinds,
+ * not which value feeds which step, so this operator cannot be reached through
+ * megcc_gfx950_parse_symbol: the KernelGen shim carries the attr. */
+TinyNNStatus megcc_gfx950_fused_elemwise(
+        const MegccFusedElemwiseAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs,
+        int nr_output, const Workspace* workspace, const RuntimeOpt* opt);
+
 /* ------------------------------------------------------------------------------------------
  * Dispatch by the reference's kernel symbol: lets a caller that only knows the generated name
  * (e.g. "kernel_conv2d_3x3_NCHW44_DENSE_p1x1_s1x1_d1x1_qsi8qsi8qsi32qsi8_bias_RELU",
@@ -357,7 +401,8 @@ typedef enum {
     MEGCC_KERN_REDUCE = 7,
     MEGCC_KERN_RELAYOUT = 8,
     MEGCC_KERN_CONCAT = 9,
-    MEGCC_KERN_RESIZE = 10
+    MEGCC_KERN_RESIZE = 10,
+    MEGCC_KERN_FUSED_ELEMWISE = 11 /* never produced by parse_symbol; a caller fills the attr */
 } MegccKernelKind;
 
 typedef struct {
@@ -371,6 +416,7 @@ typedef struct {
         MegccReduceAttr reduce;
         int concat_axis;
         MegccResizeAttr resize;
+        MegccFusedElemwiseAttr fused;
     } attr;
 } MegccKernelDesc;
 

@@ -37,12 +37,14 @@ MULTITYPE_NAMES = {0: "QADD", 1: "QFUSE_ADD_RELU", 2: "QMUL", 3: "QRELU"}
 # MegccElemwiseMode
 EW_RELU, EW_EXP, EW_SIGMOID, EW_H_SWISH, EW_NEGATE = 0, 1, 2, 3, 4
 EW_ADD, EW_SUB, EW_MUL, EW_TRUE_DIV, EW_MAX, EW_MIN, EW_FUSE_ADD_RELU = 16, 17, 18, 19, 20, 21, 22
+EW_MODES = {"RELU": 0, "EXP": 1, "SIGMOID": 2, "H_SWISH": 3, "NEGATE": 4, "ADD": 16, "SUB": 17,
+            "MUL": 18, "TRUE_DIV": 19, "MAX": 20, "MIN": 21, "FUSE_ADD_RELU": 22}
 # MegccReduceMode
 REDUCE_SUM, REDUCE_MEAN, REDUCE_MAX, REDUCE_MIN = 0, 1, 2, 3
 # MegccKernelKind
 KERN_CONV, KERN_MATMUL, KERN_POOLING, KERN_ELEMWISE_MULTITYPE = 1, 2, 3, 4
 KERN_ELEMWISE, KERN_TYPECVT, KERN_REDUCE = 5, 6, 7
-KERN_RELAYOUT, KERN_CONCAT, KERN_RESIZE = 8, 9, 10
+KERN_RELAYOUT, KERN_CONCAT, KERN_RESIZE, KERN_FUSED_ELEMWISE = 8, 9, 10, 11
 IMODE_NEAREST, IMODE_LINEAR = 0, 1
 
 
@@ -129,11 +131,54 @@ class ResizeAttr(C.Structure):
     _fields_ = [("format", C.c_int), ("imode", C.c_int)]
 
 
+FUSED_MAX_STEPS, FUSED_MAX_INPUTS = 16, 8
+# modes that exist only as steps of a fused elementwise chain (MegccElemwiseMode)
+FUSED_ONLY_MODES = {"ABS": 5, "LOG": 6, "SILU": 7, "ROUND": 8, "LT": 23, "LEQ": 24, "EQ": 25,
+                    "FLOOR_DIV": 26, "FUSE_ADD_SIGMOID": 27, "FUSE_ADD_TANH": 28,
+                    "FUSE_MUL_ADD3": 32, "FUSE_MUL_ADD4": 33}
+
+
+class FusedStep(C.Structure):
+    _fields_ = [("mode", C.c_int), ("nr_arg", C.c_int), ("arg", C.c_int * 4)]
+
+
+class FusedElemwiseAttr(C.Structure):
+    _fields_ = [("nr_input", C.c_int), ("nr_step", C.c_int), ("step", FusedStep * FUSED_MAX_STEPS)]
+
+
+def parse_fused_modes(modes, nr_input):
+    """["I0,I1,ADD,O0", "O0,I2,MUL,D", ...] -> [(mode enum, [value numbers])]: the naming of
+    compiler/test/kernel/opr/common/fused_elemwise.cpp:67-95 (I<k> input k, O<j> result of step j,
+    the last step's result is the output whatever it is called)."""
+    prog = []
+    for j, text in enumerate(modes):
+        parts = text.split(",")
+        names, mode = parts[:-2], parts[-2]
+        args = []
+        for nm in names:
+            k = int(nm[1:])
+            assert (nm[0] == "I" and k < nr_input) or (nm[0] == "O" and k < j), text
+            args.append(k if nm[0] == "I" else nr_input + k)
+        enum = EW_MODES[mode] if mode in EW_MODES else FUSED_ONLY_MODES[mode]
+        prog.append((enum, args))
+    return prog
+
+
+def fused_attr(prog, nr_input):
+    a = FusedElemwiseAttr()
+    a.nr_input, a.nr_step = nr_input, len(prog)
+    for j, (mode, args) in enumerate(prog):
+        a.step[j].mode, a.step[j].nr_arg = mode, len(args)
+        for i, v in enumerate(args):
+            a.step[j].arg[i] = v
+    return a
+
+
 class _KernelAttrUnion(C.Union):
     _fields_ = [
         ("conv", ConvAttr), ("matmul", MatMulAttr), ("pool", PoolAttr),
         ("multitype", C.c_int), ("elemwise", C.c_int), ("reduce", ReduceAttr),
-        ("concat_axis", C.c_int), ("resize", ResizeAttr),
+        ("concat_axis", C.c_int), ("resize", ResizeAttr), ("fused", FusedElemwiseAttr),
     ]
 
 

@@ -494,6 +494,112 @@ struct ResizeKernel : KernelFuncBase {
     }
 };
 
+// ---- FusedElemwise (f32): the chain "modes:<i>" = "<operands...>,<MODE>,<result>" becomes a
+// constant MegccFusedElemwiseAttr in the shim (names I<k> / O<j> resolved to value numbers). The
+// symbol follows BareMetal/FusedElemwiseKernel.cpp:293-317; like the reference's it names only
+// modes and operand kinds, so - unlike every other operator - the library cannot rebuild the attr
+// from it: the shim is the only carrier.
+struct FusedElemwiseKernel : KernelFuncBase {
+    static std::vector<std::string> split(const std::string& s) {
+        std::vector<std::string> out;
+        std::stringstream ss(s);
+        std::string item;
+        while (std::getline(ss, item, ','))
+            out.push_back(item);
+        return out;
+    }
+    static const char* mode_enum(const std::string& m) {
+        static const char* const known[] = {
+                "RELU", "EXP", "SIGMOID", "H_SWISH", "NEGATE", "ABS", "LOG", "SILU", "ROUND", "ADD",
+                "SUB", "MUL", "TRUE_DIV", "MAX", "MIN", "FUSE_ADD_RELU", "LT", "LEQ", "EQ",
+                "FLOOR_DIV", "FUSE_ADD_SIGMOID", "FUSE_ADD_TANH", "FUSE_MUL_ADD3", "FUSE_MUL_ADD4"};
+        for (const char* k : known)
+            if (m == k)
+                return k;
+        return nullptr;
+    }
+    // 0 VECTOR, 1 SCALAR, 2 BCAST101, 3 BCAST101xX, 4 unknown (Common/ElemwiseCommon.cpp:7-45)
+    static int tensor_type(const CCOperand& dst, const CCOperand& op) {
+        size_t n = 1, m = 1;
+        for (size_t d : dst.shape)
+            n *= d;
+        for (size_t d : op.shape)
+            m *= d;
+        if (n == m)
+            return 0;
+        if (m == 1)
+            return 1;
+        const auto& s = op.shape;
+        if (dst.shape.size() >= 4 && s.size() == 4 && s[0] == 1 && s[2] == 1 && s[3] == 1)
+            return 2;
+        if (dst.shape.size() >= 4 && s.size() == 5 && s[0] == 1 && s[2] == 1 && s[3] == 1 && s[4] == 4)
+            return 3;
+        return 4;
+    }
+    bool IsAvailable(TContext* c) const override {
+        const int steps = c->getAttrInt("modes:size"), nr = c->getAttrInt("nr_operands");
+        if (steps < 1 || steps > 16 || nr < 2 || nr > 9)
+            return false;
+        const CCOperand dst = c->getAttrOprand("operand:" + std::to_string(nr - 1));
+        for (int i = 0; i < nr; ++i) {
+            const CCOperand op = c->getAttrOprand("operand:" + std::to_string(i));
+            if (!is_f32(op.dtype) || tensor_type(dst, op) == 4)
+                return false;
+        }
+        for (int j = 0; j < steps; ++j) {
+            const auto parts = split(c->getAttrStr("modes:" + std::to_string(j)));
+            if (parts.size() < 3 || parts.size() > 6 || !mode_enum(parts[parts.size() - 2]))
+                return false;
+            for (size_t a = 0; a + 2 < parts.size(); ++a) {
+                const std::string& nm = parts[a];
+                if (nm.size() < 2 || (nm[0] != 'I' && nm[0] != 'O'))
+                    return false;
+                const int k = std::atoi(nm.c_str() + 1);
+                if ((nm[0] == 'I' && k >= nr - 1) || (nm[0] == 'O' && k >= j))
+                    return false;
+            }
+        }
+        return true;
+    }
+    std::string GetKernelSymbol(TContext* c) const override {
+        const int steps = c->getAttrInt("modes:size"), nr = c->getAttrInt("nr_operands");
+        const CCOperand dst = c->getAttrOprand("operand:" + std::to_string(nr - 1));
+        std::stringstream ss;
+        ss << "kernel_naive_fused_elementwise";
+        for (int j = 0; j < steps; ++j) {
+            const auto parts = split(c->getAttrStr("modes:" + std::to_string(j)));
+            ss << "_" << parts[parts.size() - 2];
+        }
+        for (int i = 0; i < nr; ++i)
+            ss << "_tensortype" << tensor_type(dst, c->getAttrOprand("operand:" + std::to_string(i)));
+        ss << "_";
+        for (int i = 0; i < nr; ++i)
+            ss << valid_dtype(c->getAttrOprand("operand:" + std::to_string(i)).dtype);
+        return ss.str();
+    }
+    std::string GetKernelBody(TContext* c) const override {
+        const int steps = c->getAttrInt("modes:size"), nr_in = c->getAttrInt("nr_operands") - 1;
+        std::stringstream a;
+        a << "    static const MegccFusedElemwiseAttr attr = {" << nr_in << ", " << steps << ", {\n";
+        for (int j = 0; j < steps; ++j) {
+            const auto parts = split(c->getAttrStr("modes:" + std::to_string(j)));
+            const size_t n = parts.size() - 2;
+            a << "        {MEGCC_EW_" << parts[n] << ", " << n << ", {";
+            for (size_t k = 0; k < 4; ++k) {
+                int v = 0;
+                if (k < n)
+                    v = std::atoi(parts[k].c_str() + 1) + (parts[k][0] == 'O' ? nr_in : 0);
+                a << v << (k < 3 ? ", " : "");
+            }
+            a << "}},\n";
+        }
+        a << "    }};\n";
+        return kHeader + kernel_def(this, c, a.str(),
+                                    "megcc_gfx950_fused_elemwise(&attr, inputs, nr_input, outputs, "
+                                    "nr_output, workspace, opt)");
+    }
+};
+
 // ---- MatrixMul (f32) ---------------------------------------------------------------------------
 struct MatrixMulKernel : KernelFuncBase {
     bool IsAvailable(TContext* c) const override {
@@ -541,6 +647,7 @@ std::vector<const KernelFuncBase*> Gfx950KernelPack::GetKernel(KernType type) {
     static const RelayoutKernel relayout;
     static const ConcatKernel concat;
     static const ResizeKernel resize;
+    static const FusedElemwiseKernel fused;
     switch (type) {
         case KernType::ConvKernel: return {&conv};
         case KernType::PoolingKernel: return {&pool};
@@ -552,6 +659,7 @@ std::vector<const KernelFuncBase*> Gfx950KernelPack::GetKernel(KernType type) {
         case KernType::RelayoutKernel: return {&relayout};
         case KernType::ConcatKernel: return {&concat};
         case KernType::ResizeKernel: return {&resize};
+        case KernType::FusedElemwiseKernel: return {&fused};
         default: return {};
     }
 }

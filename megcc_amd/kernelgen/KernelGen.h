@@ -94,6 +94,7 @@ enum class KernType {
     TypeCvtKernel = 13,
     ResizeKernel = 19,
     ConcatKernel = 25,
+    FusedElemwiseKernel = 28,
 };
 
 }  // namespace megcc_gfx950

@@ -37,6 +37,7 @@ def lib():
         L.megcc_gfx950_relayout.argtypes = kern
         L.megcc_gfx950_concat.argtypes = [C.POINTER(C.c_int)] + kern
         L.megcc_gfx950_resize.argtypes = [C.POINTER(abi.ResizeAttr)] + kern
+        L.megcc_gfx950_fused_elemwise.argtypes = [C.POINTER(abi.FusedElemwiseAttr)] + kern
         L.megcc_gfx950_parse_symbol.argtypes = [C.c_char_p, C.POINTER(abi.KernelDesc)]
         L.megcc_gfx950_call.argtypes = [C.POINTER(abi.KernelDesc)] + kern
         L.megcc_gfx950_call_init.argtypes = [C.POINTER(abi.KernelDesc)] + abi.INIT_ARGS
@@ -91,7 +92,7 @@ EXPORTS = [
     "megcc_gfx950_conv2d", "megcc_gfx950_conv2d_init", "megcc_gfx950_conv2d_workspace",
     "megcc_gfx950_matmul", "megcc_gfx950_matmul_workspace", "megcc_gfx950_pooling",
     "megcc_gfx950_elemwise_multitype", "megcc_gfx950_elemwise", "megcc_gfx950_typecvt",
-    "megcc_gfx950_reduce", "megcc_gfx950_relayout", "megcc_gfx950_concat", "megcc_gfx950_resize",
+    "megcc_gfx950_reduce", "megcc_gfx950_relayout", "megcc_gfx950_concat", "megcc_gfx950_resize", "megcc_gfx950_fused_elemwise",
     "megcc_gfx950_parse_symbol", "megcc_gfx950_call",
     "megcc_gfx950_call_init", "megcc_gfx950_call_workspace", "megcc_gfx950_init_device",
     "megcc_gfx950_malloc", "megcc_gfx950_free", "megcc_gfx950_memcpy_h2d",

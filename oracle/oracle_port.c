@@ -527,3 +527,69 @@ void orc_resize_nearest_f32(
         dst += (size_t)C * OH * OW;
     }
 }
+
+/* Fused f32 elementwise chain, BareMetal/FusedElemwiseKernel.cpp:32-113 (expressions), :159-219
+ * (operand reads), :390-413 (loop). prog: per step {mode, nr_arg, arg0..arg3}; value k < nr_input
+ * is input k, value nr_input + j the result of step j; the last result is stored.
+ * types: 0 VECTOR, 1 SCALAR, 2 BCAST101, 3 BCAST101x4 (Common/ElemwiseCommon.h:8-15). */
+enum {
+    EW_ABS = 5, EW_LOG = 6, EW_SILU = 7, EW_ROUND = 8, EW_LT = 23, EW_LEQ = 24, EW_EQ = 25,
+    EW_FLOOR_DIV = 26, EW_FUSE_ADD_SIGMOID = 27, EW_FUSE_ADD_TANH = 28, EW_FUSE_MUL_ADD3 = 32,
+    EW_FUSE_MUL_ADD4 = 33
+};
+
+static float orc_fused_clip(float val, float min, float max) {
+    if (val < min)
+        val = min;
+    if (val > max)
+        val = max;
+    return val;
+}
+
+void orc_fused_elemwise_f32(
+        const int* prog, int nr_input, int nr_step, const float* const* in, const int* types,
+        float* dst, size_t n, size_t stride1, size_t dims1) {
+    float v[64];
+    for (size_t i = 0; i < n; ++i) {
+        const size_t ch = (i / stride1) % dims1;
+        for (int k = 0; k < nr_input; ++k)
+            v[k] = types[k] == 0   ? in[k][i]
+                   : types[k] == 1 ? in[k][0]
+                   : types[k] == 2 ? in[k][ch]
+                                   : in[k][ch * 4 + i % 4];
+        float r = 0.f;
+        for (int j = 0; j < nr_step; ++j) {
+            const int* s = prog + 6 * j;
+            const float a = v[s[2]], b = s[1] > 1 ? v[s[3]] : 0.f, c = s[1] > 2 ? v[s[4]] : 0.f,
+                        d = s[1] > 3 ? v[s[5]] : 0.f;
+            switch (s[0]) {
+                case EW_RELU: r = a > 0 ? a : 0; break;
+                case EW_EXP: r = expf(a); break;
+                case EW_SIGMOID: r = 1 / (1 + expf(-a)); break;
+                case EW_NEGATE: r = -a; break;
+                case EW_ROUND: r = roundf(a); break;
+                case EW_H_SWISH: r = a * orc_fused_clip(a + 3, 0, 6) / 6; break;
+                case EW_ABS: r = a > 0 ? a : -a; break;
+                case EW_LOG: r = logf(a); break;
+                case EW_SILU: r = a / (1 + expf(-a)); break;
+                case EW_ADD: r = a + b; break;
+                case EW_SUB: r = a - b; break;
+                case EW_MUL: r = a * b; break;
+                case EW_TRUE_DIV: r = a / b; break;
+                case EW_FUSE_ADD_RELU: r = (a + b) > 0 ? (a + b) : 0; break;
+                case EW_FUSE_ADD_SIGMOID: r = 1.f / (1.f + expf(-(a + b))); break;
+                case EW_FUSE_ADD_TANH: r = (float)tanh(a + b); break;
+                case EW_MAX: r = a > b ? a : b; break;
+                case EW_MIN: r = a < b ? a : b; break;
+                case EW_LT: r = (a < b); break;
+                case EW_LEQ: r = (a <= b); break;
+                case EW_EQ: r = (a == b); break;
+                case EW_FLOOR_DIV: r = floorf(a / b); break;
+                case EW_FUSE_MUL_ADD3: r = a * b + c; break;
+                default: r = a * b + c * d; break; /* FUSE_MUL_ADD4 */
+            }
+            v[nr_input + j] = r;
+        }
+        dst[i] = r;
+    }
+}

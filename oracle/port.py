@@ -207,3 +207,22 @@ def resize(src, out_hw, imode, nchw44=False, src_strides=None, src_shape=None):
     lib().orc_resize_nearest_f32(_p(src), _p(dst), n, c, ih, iw, oh, ow,
                                  *[C.c_int64(int(v)) for v in st])
     return dst
+
+
+def fused_elemwise(prog, arrays, types, out_shape):
+    """prog: list of (mode, [value numbers]); arrays: the f32 inputs; types: 0 VECTOR, 1 SCALAR,
+    2 [1,C,1,1], 3 [1,C,1,1,4] per input."""
+    flat = np.zeros((len(prog), 6), np.int32)
+    for j, (mode, args) in enumerate(prog):
+        flat[j, 0], flat[j, 1] = mode, len(args)
+        flat[j, 2:2 + len(args)] = args
+    arrays = [np.ascontiguousarray(a, dtype=np.float32) for a in arrays]
+    ptrs = (C.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+    ty = np.asarray(types, np.int32)
+    dst = np.empty(out_shape, np.float32)
+    n = int(np.prod(out_shape, dtype=np.int64))
+    dims1 = out_shape[1] if len(out_shape) >= 2 else 1
+    stride1 = int(np.prod(out_shape[2:], dtype=np.int64)) if len(out_shape) >= 2 else 1
+    lib().orc_fused_elemwise_f32(_p(flat), len(arrays), len(prog), ptrs, _p(ty), _p(dst),
+                                 C.c_size_t(n), C.c_size_t(stride1), C.c_size_t(dims1))
+    return dst

@@ -45,6 +45,7 @@ static const std::map<std::string, KT> kTypes = {
         {"RelayoutKernel", KT::RelayoutKernel},
         {"ConcatKernel", KT::ConcatKernel},
         {"ResizeKernel", KT::ResizeKernel},
+        {"FusedElemwiseKernel", KT::FusedElemwiseKernel},
 };
 
 static CCOperand parse_operand(const std::string& v) {

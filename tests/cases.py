@@ -573,6 +573,85 @@ class ResizeCase:
                            self.src_shape() if self.src_strides is not None else None)
 
 
+class FusedCase:
+    """a fused chain of f32 elementwise steps (`modes` as the compiler writes them: "I0,I1,ADD,O0",
+    ..., compiler/test/kernel/opr/common/fused_elemwise.cpp:67-112) over inputs of `shapes`; the
+    output has the shape of the largest input. Inputs are small integers as in the reference's
+    test (UniformIntRNG(-10, 10), fused_elemwise.cpp:132), or positive where `positive` says so
+    (LOG, divisors)."""
+
+    GI_MODES = {"RELU", "SIGMOID", "EXP", "H_SWISH", "NEGATE", "ADD", "SUB", "MUL", "MAX", "MIN",
+                "TRUE_DIV", "FUSE_ADD_RELU", "FUSE_ADD_SIGMOID", "FUSE_MUL_ADD3", "FUSE_MUL_ADD4"}
+
+    def __init__(self, modes, shapes, positive=()):
+        self.modes, self.shapes = list(modes), [tuple(s) for s in shapes]
+        self.positive = set(positive)
+        self.out_shape = max(self.shapes, key=lambda sh: int(np.prod(sh)))
+        self.prog = abi.parse_fused_modes(self.modes, len(self.shapes))
+
+    def __repr__(self):
+        return "fused[%s | %s]" % (" ".join(m.split(",")[-2] for m in self.modes),
+                                   " ".join("x".join(map(str, s)) for s in self.shapes))
+
+    def types(self):
+        """Common/ElemwiseCommon.cpp:7-45"""
+        n = int(np.prod(self.out_shape))
+        out = []
+        for sh in self.shapes:
+            ne = int(np.prod(sh))
+            if ne == n:
+                out.append(0)
+            elif ne == 1:
+                out.append(1)
+            elif len(sh) == 4 and sh[0] == 1 and sh[2] == 1 and sh[3] == 1:
+                out.append(2)
+            else:
+                assert len(sh) == 5 and sh[0] == 1 and sh[2] == 1 and sh[3] == 1 and sh[4] == 4, sh
+                out.append(3)
+        return out
+
+    def symbol(self):
+        # GeneralIntrinsic/FusedElemwiseKernel.cpp:680-726 when it knows every mode, else
+        # BareMetal/FusedElemwiseKernel.cpp:270-317; the output counts as one more VECTOR operand
+        names = [m.split(",")[-2] for m in self.modes]
+        # (both availability checks keep only their verdict on the last step)
+        head = "kernel_gi_fused_elementwise" if names[-1] in self.GI_MODES \
+            else "kernel_naive_fused_elementwise"
+        return "%s_%s_%s_%s" % (head, "_".join(names),
+                                "_".join("tensortype%d" % t for t in self.types() + [0]),
+                                "f32" * (len(self.shapes) + 1))
+
+    def spec_line(self):
+        ops = ["operand:%d=%s" % (i, _op(s, "f32")) for i, s in enumerate(self.shapes)]
+        ops.append("operand:%d=%s" % (len(self.shapes), _op(self.out_shape, "f32")))
+        ms = ["modes:%d=s:%s" % (i, m) for i, m in enumerate(self.modes)]
+        return "FusedElemwiseKernel modes:size=i:%d %s nr_operands=i:%d %s" % (
+            len(self.modes), " ".join(ms), len(self.shapes) + 1, " ".join(ops))
+
+    def gen(self, seed=0):
+        r = rng(seed)
+        out = {}
+        for i, sh in enumerate(self.shapes):
+            lo = 1 if i in self.positive else -10
+            out["in%d" % i] = r.integers(lo, 10, sh, endpoint=True).astype(np.float32)
+        return out
+
+    def specs(self, arrays):
+        ins = [TensorSpec(b"in%d" % i, s, abi.FLOAT, 1.0, arrays["in%d" % i])
+               for i, s in enumerate(self.shapes)]
+        return ins, [TensorSpec(b"dst", self.out_shape, abi.FLOAT, 1.0)]
+
+    def desc(self):
+        d = abi.KernelDesc()
+        d.kind = abi.KERN_FUSED_ELEMWISE
+        d.attr.fused = abi.fused_attr(self.prog, len(self.shapes))
+        return d
+
+    def run_port(self, arrays):
+        return port.fused_elemwise(self.prog, [arrays["in%d" % i] for i in range(len(self.shapes))],
+                                   self.types(), self.out_shape)
+
+
 def run_ref(case, arrays, symbol=None):
     """Evaluate `case` with the reference's generated C kernel; returns the output array."""
     ins, outs = case.specs(arrays)

@@ -4,7 +4,7 @@ tests/golden/make_golden.py). Shapes follow the reference's own kernel tests
 typecvt.cpp:5-70): odd sizes, k in {1,3}, stride in {1,2}, pad in {0,k/2}, every activation, the
 small-magnitude tie case and the 30..50 overflow case."""
 from megcc_amd import abi
-from cases import (ConcatCase, ConvCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
+from cases import (ConcatCase, ConvCase, FusedCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
                    ResizeCase, TypeCvtCase)
 
 A = abi
@@ -136,6 +136,37 @@ def golden_cases():
     c["resize_linear_nchw44_same"] = ResizeCase(A.FMT_NCHW44, "LINEAR", 1, 2, 6, 5, 6, 5)
     c["resize_linear_nchw_x2"] = ResizeCase(A.FMT_NCHW, "LINEAR", 1, 3, 8, 10, 16, 20)
     c["resize_nearest_nchw_x2"] = ResizeCase(A.FMT_NCHW, "NEAREST", 1, 3, 8, 10, 16, 20)
+    # --- fused elementwise: the chains and shapes of compiler/test/kernel/opr/naive/fused_elemwise.cpp
+    # (the reference names a kernel by its modes and operand kinds only, so every case here has a
+    # name of its own), then the modes only the BareMetal generator knows
+    two_x_plus = ["I0,I1,ADD,O0", "I2,O0,MUL,O1", "O0,I3,SUB,D"]
+    c["fused_2xy_vec"] = FusedCase(two_x_plus, [(4, 6, 9, 2), (4, 6, 9, 2), (1,), (4, 6, 9, 2)])
+    c["fused_2xy_bcast101"] = FusedCase(two_x_plus, [(1, 6, 1, 1), (4, 6, 9, 2), (1,), (4, 6, 9, 2)])
+    more = ["I0,I1,ADD,O0", "O0,SIGMOID,O1", "O1,I2,MAX,O2", "O2,I2,TRUE_DIV,D"]
+    c["fused_more_101x4_scalar"] = FusedCase(more, [(3, 10, 10, 5, 4), (1, 10, 1, 1, 4), (1,)], positive=(2,))
+    c["fused_more_vec"] = FusedCase(more, [(3, 10, 10, 5, 4)] * 3, positive=(2,))
+    c["fused_more_101x4_twice"] = FusedCase(more, [(3, 10, 10, 5, 4), (1, 10, 1, 1, 4), (1, 10, 1, 1, 4)],
+                                            positive=(2,))
+    c["fused_relu_exp"] = FusedCase(["I0,RELU,O0", "I1,EXP,O1", "O0,O1,FUSE_ADD_RELU,D"],
+                                    [(3, 10, 10, 5, 4), (1, 10, 1, 1, 4)])
+    c["fused_neg_hswish"] = FusedCase(["I0,NEGATE,O0", "I1,H_SWISH,O1", "O0,O1,FUSE_ADD_SIGMOID,D"],
+                                      [(3, 10, 10, 5, 4), (1, 10, 1, 1, 4)])
+    c["fused_mul_add3"] = FusedCase(["I0,I1,I2,FUSE_MUL_ADD3,O0", "O0,RELU,D"],
+                                    [(2, 5, 7, 3), (2, 5, 7, 3), (1, 5, 1, 1)])
+    c["fused_mul_add4"] = FusedCase(["I0,I1,I2,I3,FUSE_MUL_ADD4,O0", "O0,I0,MIN,D"],
+                                    [(2, 5, 7, 3), (1,), (2, 5, 7, 3), (1, 5, 1, 1)])
+    # (the reference's availability checks read operand:<i> for every step i and keep only the
+    # verdict on the last step - BareMetal/FusedElemwiseKernel.cpp:270-290 and the GI twin - so a
+    # chain for the BareMetal generator has no more steps than operands and ends in a mode only
+    # that generator knows)
+    c["fused_naive_unary"] = FusedCase(["I0,I1,I2,FUSE_MUL_ADD3,O0", "O0,SILU,O1", "O1,ABS,O2", "O2,LOG,D"],
+                                       [(2, 3, 4, 5), (2, 3, 4, 5), (1, 3, 1, 1)], positive=(0, 1, 2))
+    c["fused_naive_round"] = FusedCase(["I0,I1,TRUE_DIV,O0", "O0,ROUND,D"], [(2, 3, 4, 5), (1,)],
+                                       positive=(1,))
+    c["fused_naive_compare"] = FusedCase(["I0,I1,LT,O0", "I0,I2,LEQ,O1", "O0,O1,ADD,O2", "O2,I2,FUSE_ADD_TANH,D"],
+                                         [(2, 3, 4, 5), (1, 3, 1, 1), (2, 3, 4, 5)])
+    c["fused_naive_eq_floordiv"] = FusedCase(["I0,I1,EQ,O0", "O0,I0,ADD,O1", "O1,I1,FLOOR_DIV,D"],
+                                             [(2, 3, 4, 5), (2, 3, 4, 5)], positive=(1,))
     c["resize_nearest_nchw_view"] = ResizeCase(A.FMT_NCHW, "NEAREST", 2, 3, 6, 5, 9, 11,
                                                src_strides=(400, 120, 20, 2))
     return c

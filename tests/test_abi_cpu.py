@@ -43,6 +43,12 @@ with open(os.path.join(HERE, "golden", "symbols.json")) as f:
 
 @pytest.mark.parametrize("symbol", sorted(set(SYMBOLS.values())))
 def test_every_reference_symbol_parses(symbol):
+    if "fused_elementwise" in symbol:
+        # the reference names a fused chain by its modes and operand kinds only; which value feeds
+        # which step is not in the name, so the library refuses to guess (the shim carries it)
+        with pytest.raises(runtime.MegccError):
+            runtime.parse_symbol(symbol)
+        return
     desc = runtime.parse_symbol(symbol)
     assert desc.kind in range(1, 11)
 
@@ -125,13 +131,29 @@ def test_copy_kernels_reject_bad_arguments_before_any_launch():
     assert call(L.megcc_gfx950_resize, [t((1, 2, 4, 4, 4))], t((1, 2, 8, 8, 4)),
                 C.byref(near44)) == abi.ERROR_OUT_OF_RANGE  # no such kernel in the reference
     assert L.megcc_gfx950_resize(None, None, 0, None, 0, None, None) == abi.ERROR_NULL_PTR
+    # fused elementwise: the program is checked before anything is launched
+    prog = abi.parse_fused_modes(["I0,I1,ADD,O0", "O0,RELU,D"], 2)
+    ok = abi.fused_attr(prog, 2)
+    x = t((2, 3, 4, 5))
+    assert call(L.megcc_gfx950_fused_elemwise, [x, t((1, 3, 1, 1))], t((0, 3, 4, 5)), C.byref(ok)) == 0
+    assert call(L.megcc_gfx950_fused_elemwise, [x, t((1, 4, 1, 1))], x, C.byref(ok)) == \
+        abi.ERROR_INVALID_LAYOUT  # neither the output's size, a scalar nor [1,C,1,1]
+    assert call(L.megcc_gfx950_fused_elemwise, [x], x, C.byref(ok)) == \
+        abi.ERROR_OUT_OF_RANGE  # 1 input, the program wants 2
+    late = abi.fused_attr([(abi.EW_ADD, [0, 3]), (abi.EW_RELU, [2])], 2)  # reads step 1's result in step 0
+    assert call(L.megcc_gfx950_fused_elemwise, [x, x], x, C.byref(late)) == abi.ERROR_OUT_OF_RANGE
+    arity = abi.fused_attr([(abi.EW_ADD, [0])], 2)
+    assert call(L.megcc_gfx950_fused_elemwise, [x, x], x, C.byref(arity)) == abi.ERROR_OUT_OF_RANGE
+    assert call(L.megcc_gfx950_fused_elemwise, [x, t((2, 3, 4, 5), abi.QINT8)], x, C.byref(ok)) == \
+        abi.ERROR_UNSUPPORTED_DTYPE_TYPE
 
 
 def test_unknown_symbol_is_reported_not_guessed():
     desc = abi.KernelDesc()
     for bad in ("kernel_argsort_f32", "kernel_relayout_f64", "kernel_concat_byte_8_axis_0",
                 "kernel_concat_byte_4_axis_1x", "kernel_resize_linear_NCHW44_NEAREST_f32",
-                "GI_kernel_resize_linear_NHWC_LINEAR_f32", "kernel_resize_linear_NCHW_LINEAR_f16", "kernel_conv2d_3x3_NHWC_DENSE_p1x1_s1x1_d1x1_f32f32f32",
+                "GI_kernel_resize_linear_NHWC_LINEAR_f32",
+                "kernel_gi_fused_elementwise_ADD_RELU_tensortype0_tensortype0_tensortype0_f32f32f32", "kernel_resize_linear_NCHW_LINEAR_f16", "kernel_conv2d_3x3_NHWC_DENSE_p1x1_s1x1_d1x1_f32f32f32",
                 "kernel_typecvt_f16f32", ""):
         st = runtime.lib().megcc_gfx950_parse_symbol(bad.encode(), C.byref(desc))
         assert st == abi.ERROR_NO_FOUND

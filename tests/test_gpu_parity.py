@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import cases
-from cases import (ConcatCase, ConvCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
+from cases import (ConcatCase, ConvCase, FusedCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
                    ResizeCase, TypeCvtCase)
 from golden_cases import golden_cases, unsat
 from megcc_amd import abi, runtime
@@ -44,6 +44,10 @@ def compare(got, want, what):
 def run_gpu(case, arrays, symbol=None):
     print("GPU case:", repr(case), flush=True)
     ins, outs = case.specs(arrays)
+    if hasattr(case, "desc"):  # fused elementwise: the symbol does not say which value feeds which step
+        op = runtime.PreparedOp(case.desc(), ins, outs)
+        op.launch()
+        return op.result()
     return runtime.run_symbol(symbol or case.symbol(), ins, outs)
 
 
@@ -294,6 +298,28 @@ def test_resize(case):
     compare(got, want, repr(case))
     # the kernels keep the reference's order of operations: equal bit for bit
     assert np.array_equal(got, want), repr(case)
+
+
+FUSED = [
+    # chains at the sizes of a detection head (SiLU gating, residual scale + shift, clipped
+    # activations), every operand kind, a chain of the maximum length, a length that is no
+    # multiple of the workgroup
+    FusedCase(["I0,SILU,O0", "O0,I1,MUL,O1", "O1,I2,ADD,D"], [(8, 64, 40, 40), (1, 64, 1, 1), (1, 64, 1, 1)]),
+    FusedCase(["I0,I1,I2,FUSE_MUL_ADD3,O0", "O0,H_SWISH,O1", "O1,I3,FUSE_ADD_RELU,D"],
+              [(4, 16, 28, 28, 4), (1, 16, 1, 1, 4), (1, 16, 1, 1, 4), (4, 16, 28, 28, 4)]),
+    FusedCase(["I0,I1,SUB,O0", "O0,EXP,O1", "O1,I2,TRUE_DIV,D"], [(64, 1000), (1,), (1,)], positive=(2,)),
+    FusedCase(["I0,I1,ADD,O0"] + ["O%d,I1,%s,O%d" % (j, m, j + 1) for j, m in enumerate(
+        ["MUL", "SUB", "MAX", "MIN", "ADD", "MUL", "SUB", "FUSE_ADD_RELU", "ADD", "MAX", "MIN", "SUB", "ADD", "MUL"])]
+        + ["O14,SIGMOID,D"], [(3, 5, 7, 11), (3, 5, 7, 11)]),
+    FusedCase(["I0,ABS,O0", "O0,LOG,O1", "O1,I1,LT,O2", "O2,O1,I0,I1,FUSE_MUL_ADD4,D"],
+              [(1, 3, 1, 331), (1, 3, 1, 1)], positive=(0,)),
+]
+
+
+@pytest.mark.parametrize("case", FUSED, ids=[repr(c) for c in FUSED])
+def test_fused_elemwise(case):
+    arrays = case.gen(seed=43)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
 
 
 OLDER = [

@@ -257,3 +257,29 @@ def test_port_resize_closed_forms():
     assert np.array_equal(
         port.resize(buf, (9, 11), "NEAREST", src_strides=(400, 120, 20, 2), src_shape=(2, 3, 6, 5)),
         port.resize(np.ascontiguousarray(view), (9, 11), "NEAREST"))
+
+
+def test_port_fused_elemwise_vs_numpy():
+    """the chain interpreter against numpy written out by hand: operand kinds (same size, scalar,
+    [1,C,1,1], [1,C,1,1,4]), reuse of an intermediate value, 3- and 4-operand steps"""
+    from megcc_amd import abi
+    r = np.random.default_rng(9)
+    x = r.integers(-10, 10, (3, 10, 10, 5, 4), endpoint=True).astype(np.float32)
+    b = r.integers(-10, 10, (1, 10, 1, 1, 4), endpoint=True).astype(np.float32)
+    z = np.array([3.0], np.float32)
+    prog = abi.parse_fused_modes(["I0,I1,ADD,O0", "O0,SIGMOID,O1", "O1,I2,MAX,O2", "O2,I2,TRUE_DIV,D"], 3)
+    got = port.fused_elemwise(prog, [x, b, z], [0, 3, 1], x.shape)
+    sig = np.float32(1) / (np.float32(1) + np.exp(-(x + b), dtype=np.float32))
+    np.testing.assert_allclose(got, np.maximum(sig, z) / z, rtol=1e-6)
+    y = r.integers(-10, 10, (4, 6, 9, 2), endpoint=True).astype(np.float32)
+    c = r.integers(-10, 10, (1, 6, 1, 1), endpoint=True).astype(np.float32)
+    prog = abi.parse_fused_modes(["I0,I1,ADD,O0", "I2,O0,MUL,O1", "O0,I3,SUB,D"], 4)
+    got = port.fused_elemwise(prog, [c, y, np.array([2.0], np.float32), y], [2, 0, 1, 0], y.shape)
+    assert np.array_equal(got, (c + y) - y)  # step 1's result is computed and not used
+    prog = abi.parse_fused_modes(["I0,I1,I2,I1,FUSE_MUL_ADD4,O0", "O0,I0,LT,O1", "O1,O0,FLOOR_DIV,D"], 3)
+    w = r.integers(1, 10, (4, 6, 9, 2), endpoint=True).astype(np.float32)
+    got = port.fused_elemwise(prog, [y, w, c], [0, 0, 2], y.shape)
+    t0 = y * w + c * w
+    with np.errstate(divide="ignore", invalid="ignore"):
+        want = np.floor((t0 < y).astype(np.float32) / t0)
+    assert np.array_equal(got, want, equal_nan=True)

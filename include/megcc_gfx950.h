@@ -493,6 +493,13 @@ int megcc_gfx950_model_add_view(
 TinyNNStatus megcc_gfx950_model_add_opr(
         void* model, const char* symbol, const int* inputs, int nr_input, const int* outputs,
         int nr_output);
+/* The same with the operator given as a filled MegccKernelDesc instead of its symbol: for the one
+ * operator whose reference symbol does not determine it (fused elementwise chains; `name` is
+ * only a label). What runtime/src/vm/op.c:161-163 does with a function pointer taken from the
+ * generated kernel table. */
+TinyNNStatus megcc_gfx950_model_add_opr_desc(
+        void* model, const MegccKernelDesc* desc, const char* name, const int* inputs, int nr_input,
+        const int* outputs, int nr_output);
 TinyNNStatus megcc_gfx950_model_mark_io(void* model, int tensor, int is_output);
 TinyNNStatus megcc_gfx950_model_finalize(void* model);
 size_t megcc_gfx950_model_arena_bytes(void* model);

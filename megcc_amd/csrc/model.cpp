@@ -258,18 +258,11 @@ int megcc_gfx950_model_add_view(
     return id;
 }
 
-TinyNNStatus megcc_gfx950_model_add_opr(
-        void* model, const char* symbol, const int* inputs, int nr_input, const int* outputs,
-        int nr_output) {
-    Model* m = (Model*)model;
-    MG_REQUIRE(m && symbol && inputs && outputs && !m->finalized, TinyNN_ERROR_NULL_PTR,
-               "model_add_opr: bad argument");
+static TinyNNStatus add_opr(
+        Model* m, const MegccKernelDesc& desc, const char* symbol, const int* inputs, int nr_input,
+        const int* outputs, int nr_output) {
     ModelOpr* o = new ModelOpr();
-    TinyNNStatus st = megcc_gfx950_parse_symbol(symbol, &o->desc);
-    if (st != TinyNN_SUCCESS) {
-        delete o;
-        return st;
-    }
+    o->desc = desc;
     o->symbol = symbol;
     memset(&o->ws, 0, sizeof(o->ws));
     const int idx = (int)m->oprs.size();
@@ -295,6 +288,30 @@ TinyNNStatus megcc_gfx950_model_add_opr(
     }
     m->oprs.push_back(o);
     return TinyNN_SUCCESS;
+}
+
+TinyNNStatus megcc_gfx950_model_add_opr(
+        void* model, const char* symbol, const int* inputs, int nr_input, const int* outputs,
+        int nr_output) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && symbol && inputs && outputs && !m->finalized, TinyNN_ERROR_NULL_PTR,
+               "model_add_opr: bad argument");
+    MegccKernelDesc desc;
+    TinyNNStatus st = megcc_gfx950_parse_symbol(symbol, &desc);
+    if (st != TinyNN_SUCCESS)
+        return st;
+    return add_opr(m, desc, symbol, inputs, nr_input, outputs, nr_output);
+}
+
+TinyNNStatus megcc_gfx950_model_add_opr_desc(
+        void* model, const MegccKernelDesc* desc, const char* name, const int* inputs, int nr_input,
+        const int* outputs, int nr_output) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && desc && name && inputs && outputs && !m->finalized, TinyNN_ERROR_NULL_PTR,
+               "model_add_opr_desc: bad argument");
+    MG_REQUIRE(desc->kind >= MEGCC_KERN_CONV && desc->kind <= MEGCC_KERN_FUSED_ELEMWISE,
+               TinyNN_ERROR_OUT_OF_RANGE, "model_add_opr_desc: kind %d", (int)desc->kind);
+    return add_opr(m, *desc, name, inputs, nr_input, outputs, nr_output);
 }
 
 TinyNNStatus megcc_gfx950_model_mark_io(void* model, int tensor, int is_output) {

@@ -67,6 +67,8 @@ def lib():
                                                   C.POINTER(C.c_int), C.c_size_t]
         ints = C.POINTER(C.c_int)
         L.megcc_gfx950_model_add_opr.argtypes = [C.c_void_p, C.c_char_p, ints, C.c_int, ints, C.c_int]
+        L.megcc_gfx950_model_add_opr_desc.argtypes = [C.c_void_p, C.POINTER(abi.KernelDesc), C.c_char_p,
+                                                      ints, C.c_int, ints, C.c_int]
         L.megcc_gfx950_model_mark_io.argtypes = [C.c_void_p, C.c_int, C.c_int]
         L.megcc_gfx950_model_finalize.argtypes = [C.c_void_p]
         L.megcc_gfx950_model_arena_bytes.argtypes = [C.c_void_p]
@@ -100,7 +102,7 @@ EXPORTS = [
     "megcc_gfx950_stream", "megcc_gfx950_last_error",
     "megcc_gfx950_model_create", "megcc_gfx950_model_destroy", "megcc_gfx950_model_add_tensor",
     "megcc_gfx950_model_add_weight", "megcc_gfx950_model_add_alias", "megcc_gfx950_model_add_view",
-    "megcc_gfx950_model_add_opr",
+    "megcc_gfx950_model_add_opr", "megcc_gfx950_model_add_opr_desc",
     "megcc_gfx950_model_mark_io", "megcc_gfx950_model_finalize", "megcc_gfx950_model_arena_bytes",
     "megcc_gfx950_model_tensor_ptr", "megcc_gfx950_model_set_input",
     "megcc_gfx950_model_get_output", "megcc_gfx950_model_forward", "megcc_gfx950_model_nr_opr",
@@ -327,6 +329,14 @@ class Model:
         outs = (C.c_int * len(outputs))(*outputs)
         check(lib().megcc_gfx950_model_add_opr(self.h, symbol.encode(), ins, len(inputs), outs,
                                                len(outputs)), "add_opr " + symbol)
+
+    def opr_desc(self, desc, name, inputs, outputs):
+        """operator given as a filled KernelDesc (fused elementwise chains have no symbol that
+        determines them)"""
+        ins = (C.c_int * len(inputs))(*inputs)
+        outs = (C.c_int * len(outputs))(*outputs)
+        check(lib().megcc_gfx950_model_add_opr_desc(self.h, C.byref(desc), name.encode(), ins,
+                                                    len(inputs), outs, len(outputs)), "add_opr_desc " + name)
 
     def mark_input(self, tid):
         check(lib().megcc_gfx950_model_mark_io(self.h, tid, 0), "mark_io")

@@ -240,3 +240,39 @@ def test_dense_relayout_is_a_copy_that_replays_in_the_graph():
         m.forward()
         assert np.array_equal(m.get(z), np.maximum(a, 0))
     m.close()
+
+
+@pytest.mark.gpu
+def test_model_with_resize_and_a_fused_chain_replays():
+    """an up-sampling neck in one model: Resize x2 (by symbol), then a fused chain given as a
+    descriptor (its symbol does not determine it): SiLU(up) * scale[c] + skip. Every forward -
+    eager, captured, replayed - must use the current input."""
+    from oracle import port
+    m = runtime.Model()
+    x = m.tensor("x", (2, 6, 9, 11), abi.FLOAT, 1.0)
+    skip = m.tensor("skip", (2, 6, 18, 22), abi.FLOAT, 1.0)
+    m.mark_input(x)
+    m.mark_input(skip)
+    scale = np.linspace(0.5, 1.5, 6, dtype=np.float32).reshape(1, 6, 1, 1)
+    w = m.weight("scale", scale, abi.FLOAT, 1.0)
+    up = m.tensor("up", (2, 6, 18, 22), abi.FLOAT, 1.0)
+    m.opr("GI_kernel_resize_linear_NCHW_LINEAR_f32", [x], [up])
+    out = m.tensor("out", (2, 6, 18, 22), abi.FLOAT, 1.0)
+    prog = abi.parse_fused_modes(["I0,SILU,O0", "O0,I1,I2,FUSE_MUL_ADD3,D"], 3)
+    desc = abi.KernelDesc()
+    desc.kind = abi.KERN_FUSED_ELEMWISE
+    desc.attr.fused = abi.fused_attr(prog, 3)
+    m.opr_desc(desc, "silu_scale_skip", [up, w, skip], [out])
+    m.mark_output(out)
+    m.finalize()
+    r = np.random.default_rng(11)
+    for _ in range(4):
+        a = r.uniform(-4, 4, (2, 6, 9, 11)).astype(np.float32)
+        s = r.uniform(-4, 4, (2, 6, 18, 22)).astype(np.float32)
+        m.set_input(x, a)
+        m.set_input(skip, s)
+        m.forward()
+        want = port.fused_elemwise(prog, [port.resize(a, (18, 22), "LINEAR"), scale, s], [0, 2, 0],
+                                   (2, 6, 18, 22))
+        assert cases.max_rel_err(m.get(out), want) <= 1e-4
+    m.close()

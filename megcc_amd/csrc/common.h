@@ -26,6 +26,10 @@ TinyNNStatus fail(TinyNNStatus st, const char* fmt, ...) __attribute__((format(p
 // After a kernel launch: surfaces launch-configuration errors as TinyNN_ERROR_RUNTIME.
 TinyNNStatus check_launch(const char* what);
 
+// relayout.hip: copies `src` (layout sl) to `dst` (layout dl), elements of `es` bytes; one launch.
+TinyNNStatus strided_copy(
+        const void* src, const Layout& sl, void* dst, const Layout& dl, size_t es, const char* who);
+
 inline size_t nr_elem(const Layout& l) {
     size_t n = 1;
     for (int i = 0; i < l.nr_dim; ++i)

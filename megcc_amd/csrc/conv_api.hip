@@ -135,6 +135,29 @@ static bool aligned16(const void* p) {
     return ((uintptr_t)p & 15) == 0;
 }
 
+// A 1x1 convolution with a stride (the projection shortcut of ResNet-like networks) reads one
+// input pixel per output pixel: it is the stride-1 pointwise convolution of the sub-sampled
+// input. The pixels it keeps are gathered into the workspace by one strided copy (4-byte
+// elements = a pixel's 4 channels), then the pointwise kernels run on dense data.
+static bool strided_pointwise(const ConvGeom& g) {
+    return g.fmt == MEGCC_FMT_NCHW44 && g.groups == 1 && g.fh == 1 && g.fw == 1 && g.ph == 0 &&
+           g.pw == 0 && (g.sh > 1 || g.sw > 1) && (g.ic & 3) == 0;
+}
+static ConvGeom subsampled(const ConvGeom& g) {
+    ConvGeom s = g;
+    s.ih = g.oh;
+    s.iw = g.ow;
+    s.sh = s.sw = 1;
+    return s;
+}
+static size_t round_up256(size_t v) {
+    return (v + 255) & ~(size_t)255;
+}
+// workspace = [partial sums of the stride-1 kernel, rounded up to 256 B][gathered pixels]
+static size_t gather_bytes(const ConvGeom& g) {
+    return (size_t)g.n * g.ic * g.oh * g.ow;
+}
+
 }  // namespace mg
 
 using namespace mg;
@@ -180,6 +203,33 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
     if ((size_t)g.n * g.oc * g.oh * g.ow == 0)
         return TinyNN_SUCCESS;
 
+    if (packed && q8 && strided_pointwise(g) && conv_mfma_supported(subsampled(g))) {
+        const ConvGeom g1 = subsampled(g);
+        MG_REQUIRE(nr_elem(flt->layout) == conv_mfma_packed_bytes(g1), TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: packed filter has %zu bytes, expected %zu", nr_elem(flt->layout),
+                   conv_mfma_packed_bytes(g1));
+        MG_REQUIRE(aligned4(src->ptr) && aligned4(dst->ptr) && aligned16(flt->ptr) && (!b || aligned4(b)),
+                   TinyNN_ERROR_INVALID_LAYOUT, "conv2d: misaligned operand");
+        const size_t inner = round_up256(conv_mfma_workspace_bytes(g1));
+        MG_REQUIRE(workspace && workspace->ptr && workspace->size >= inner + gather_bytes(g) &&
+                           aligned16(workspace->ptr),
+                   TinyNN_ERROR_OUT_OF_RANGE,
+                   "conv2d: a strided 1x1 convolution needs %zu bytes of workspace",
+                   inner + gather_bytes(g));
+        void* gathered = (char*)workspace->ptr + inner;
+        Layout from = {}, to = {};
+        from.nr_dim = to.nr_dim = 3;  // [N * C/4, OH, OW] of 4-byte pixels
+        from.dims[0] = to.dims[0] = (uint32_t)(g.n * (g.ic / 4));
+        from.dims[1] = to.dims[1] = (uint32_t)g.oh;
+        from.dims[2] = to.dims[2] = (uint32_t)g.ow;
+        from.stride[0] = g.ih * g.iw; from.stride[1] = g.sh * g.iw; from.stride[2] = g.sw;
+        to.stride[0] = g.oh * g.ow; to.stride[1] = g.ow; to.stride[2] = 1;
+        st = strided_copy(src->ptr, from, gathered, to, 4, "conv2d (gather of a strided 1x1)");
+        if (st != TinyNN_SUCCESS)
+            return st;
+        Workspace sub = {workspace->ptr, inner, 0};
+        return conv_mfma_launch(g1, gathered, flt->ptr, b, dst->ptr, &sub);
+    }
     if (packed) {
         MG_REQUIRE(q8 && conv_mfma_supported(g), TinyNN_ERROR_INVALID_LAYOUT,
                    "conv2d: a packed filter was passed to a convolution the MFMA kernel does not cover");
@@ -219,6 +269,8 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d_init(
         TinyNNStatus st = make_geom(attr, src, flt, nullptr, false, 0, &g);
         if (st != TinyNN_SUCCESS)
             return st;
+        if (strided_pointwise(g))
+            g = subsampled(g);
         pack = conv_mfma_supported(g);
     }
     if (!out_weights) {  // phase 1: how many
@@ -265,9 +317,12 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d_workspace(
     } else if (is_q8(src) && is_q8(flt) && attr->sparse == MEGCC_SPARSE_DENSE &&
                !is_packed_filter(flt)) {
         // split-K partial sums of the one-stage MFMA kernel (few pixels, long K)
-        if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS &&
-            conv_mfma_supported(g))
-            *workspace = conv_mfma_workspace_bytes(g);
+        if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS) {
+            if (strided_pointwise(g) && conv_mfma_supported(subsampled(g)))
+                *workspace = round_up256(conv_mfma_workspace_bytes(subsampled(g))) + gather_bytes(g);
+            else if (conv_mfma_supported(g))
+                *workspace = conv_mfma_workspace_bytes(g);
+        }
     }
     return TinyNN_SUCCESS;
 }

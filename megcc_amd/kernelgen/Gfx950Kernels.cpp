@@ -270,8 +270,12 @@ struct ConvKernel : KernelFuncBase {
            << "            if (s > stages) s = stages;\n"
            << "            if (s > 16) s = 16;\n"
            << "        }\n"
-           << "        if (s > 1) *workspace = (size_t)s * P * ((oc + 3) & ~3L) * 4;\n"
-           << "    }\n"
+           << "        if (s > 1) *workspace = (size_t)s * P * ((oc + 3) & ~3L) * 4;\n";
+        // a strided 1x1 convolution first gathers the pixels it keeps (conv_api.hip)
+        if (fmt == "NCHW44" && taps == 1 && c->getAttrUInt("pad_h") == 0 && c->getAttrUInt("pad_w") == 0 &&
+            (c->getAttrUInt("stride_h") > 1 || c->getAttrUInt("stride_w") > 1))
+            ss << "        *workspace = ((*workspace + 255) & ~(size_t)255) + (size_t)P * ic;\n";
+        ss << "    }\n"
            << "    return TinyNN_SUCCESS;\n}\n";
         return ss.str();
     }

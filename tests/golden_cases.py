@@ -38,6 +38,8 @@ def golden_cases():
         A.FMT_NCHW44, A.DENSE, 1, 8, 7, 7, 8, 3, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(72)))
     c["conv44_1x1_RELU"] = ConvCase(
         A.FMT_NCHW44, A.DENSE, 2, 16, 5, 7, 24, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(16)))
+    c["conv44_1x1_s2_RELU"] = ConvCase(
+        A.FMT_NCHW44, A.DENSE, 2, 16, 9, 8, 24, 1, 2, 0, A.RELU, scales=(0.02, 0.01, unsat(16)))
     # (a qsi8 conv without bias does not exist in the reference: ConvGeneral::IsAvailable wants
     #  operand:2 to be qsi32, BareMetal/ConvKernel.cpp:25-29)
     # --- qsi8 NCHW dense: FullyConnected (1x1 on [M,K,1,1]) and 3x3

@@ -275,6 +275,23 @@ def test_first_layer_shapes(case):
     compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
 
 
+STRIDED_1X1 = [
+    # projection shortcuts: 1x1 with a stride = the pointwise kernels on the gathered pixels
+    ConvCase(A.FMT_NCHW44, A.DENSE, 4, 64, 56, 56, 128, 1, 2, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(64))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 256, 14, 14, 512, 1, 2, 0, A.RELU, scales=(0.02, 0.01, unsat(256))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 32, 15, 17, 24, 1, 2, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(32))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 1, 1024, 7, 7, 64, 1, 3, 0, A.H_SWISH, scales=(0.02, 0.01, unsat(1024))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 16, 9, 9, 8, 1, 2, 0, A.RELU, scales=(0.02, 0.01, unsat(16))),
+]
+
+
+@pytest.mark.parametrize("case", STRIDED_1X1, ids=[repr(c) for c in STRIDED_1X1])
+def test_strided_pointwise(case):
+    port.set_threads(8)
+    arrays = case.gen(seed=47)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+
+
 RESIZE = [
     # the 2x upsampling of detection necks, a camera frame scaled down to a network input, odd
     # ratios, extent 1 either side, a channel slice with a column step as NEAREST source

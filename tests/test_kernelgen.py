@@ -121,7 +121,7 @@ def test_generated_workspace_functions_agree_with_the_library(shim_library):
         elif desc.kind == 1 and "qsi8" in sym and "_NCHW44_DENSE_" in sym:
             k = desc.attr.conv.kernel_h
             cases_ = [[(64, 256, 7, 7, 4), (256, 256, k, k, 4, 4)], [(2, 8, 20, 24, 4), (12, 8, k, k, 4, 4)],
-                      [(1, 128, 14, 14, 4), (32, 128, k, k, 4, 4)]]
+                      [(1, 128, 14, 14, 4), (32, 128, k, k, 4, 4)], [(8, 64, 56, 56, 4), (128, 64, k, k, 4, 4)]]
         elif desc.kind == 1 and "qsi8" in sym and "_1x1_NCHW_DENSE_p0x0_s1x1" in sym:
             cases_ = [[(64, 1024, 1, 1), (1000, 1024, 1, 1)], [(64, 4096, 1, 1), (4096, 4096, 1, 1)],
                       [(1, 1024, 1, 1), (1000, 1024, 1, 1)], [(4096, 4096, 1, 1), (4096, 4096, 1, 1)]]

@@ -5,6 +5,7 @@
 //   qsi8 NCHW44 depthwise                                           -> dwconv.hip
 //   qsi8 3-channel NCHW -> NCHW44 3x3 stride 2 (first layer)        -> conv_first.hip
 //   qsi8 NCHW -> NCHW44, other filters up to 8x8, stride 1 / 2       -> conv_hybrid_mfma.hip
+//   qsi8 NCHW44 dense, anything else (5x5, 7x7, filter not packed)   -> conv_dot4.hip
 //   f32 NCHW DENSE                                                  -> gemm_f32.hip
 //   everything else ConvGeneral accepts                             -> conv_direct.hip
 #include "common.h"
@@ -19,6 +20,8 @@ TinyNNStatus conv_mfma_launch(const ConvGeom&, const void*, const void*, const v
 size_t conv_mfma_workspace_bytes(const ConvGeom& g);
 bool conv_hybrid_mfma_supported(const ConvGeom& g);
 TinyNNStatus conv_hybrid_mfma_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+bool conv_dot4_supported(const ConvGeom& g);
+TinyNNStatus conv_dot4_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool conv_first_supported(const ConvGeom& g);
 TinyNNStatus conv_first_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool dwconv44_supported(const ConvGeom& g);
@@ -249,6 +252,9 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
     if (q8 && conv_hybrid_mfma_supported(g) && aligned4(dst->ptr) && aligned4(flt->ptr) && (!b || aligned4(b)) &&
         !getenv("MEGCC_NOHYBRID"))
         return conv_hybrid_mfma_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+    if (q8 && conv_dot4_supported(g) && aligned4(src->ptr) && aligned4(dst->ptr) && aligned16(flt->ptr) &&
+        (!b || aligned4(b)) && !getenv("MEGCC_NODOT4"))
+        return conv_dot4_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     if (f32 && conv_f32_small_supported(g) && !getenv("MEGCC_NOF32SMALL"))
         return conv_f32_small_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     if (f32 && conv_f32_gemm_supported(g))

@@ -11,7 +11,6 @@ namespace mg {
 namespace {
 
 enum { FT_VECTOR = 0, FT_SCALAR = 1, FT_BCAST101 = 2, FT_BCAST101x4 = 3 };
-constexpr int FUSED_VALUES = MEGCC_FUSED_MAX_INPUTS + MEGCC_FUSED_MAX_STEPS;
 
 struct FusedArgs {
     const float* in[MEGCC_FUSED_MAX_INPUTS];

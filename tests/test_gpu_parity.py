@@ -292,6 +292,26 @@ def test_strided_pointwise(case):
     compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
 
 
+DOT4 = [
+    # dense NCHW44 layers the matrix-core kernels do not take (more than 9 taps): the dot-product
+    # kernel; both channel-group widths, an odd number of channel groups, stride, dilation,
+    # padding wider than the image edge, every activation
+    ConvCase(A.FMT_NCHW44, A.DENSE, 4, 32, 28, 28, 64, 5, 1, 2, A.RELU, scales=(0.02, 0.01, unsat(800))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 1, 8, 9, 11, 12, 5, 2, 2, A.IDENTITY, scales=(0.02, 0.01, unsat(200))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 16, 23, 19, 20, 7, 2, 3, A.H_SWISH, scales=(0.02, 0.01, unsat(784))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 4, 30, 30, 4, 5, 1, 0, A.SIGMOID, scales=(0.02, 0.01, unsat(100) * 30)),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 12, 17, 17, 28, 4, 1, 3, A.RELU, scales=(0.02, 0.01, unsat(192)), dilate=2),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 40, 8, 20, 20, 40, 6, 3, 1, A.RELU, scales=(0.02, 0.01, unsat(288))),
+]
+
+
+@pytest.mark.parametrize("case", DOT4, ids=[repr(c) for c in DOT4])
+def test_many_tap_dense_conv(case):
+    port.set_threads(8)
+    arrays = case.gen(seed=53)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+
+
 RESIZE = [
     # the 2x upsampling of detection necks, a camera frame scaled down to a network input, odd
     # ratios, extent 1 either side, a channel slice with a column step as NEAREST source

@@ -72,6 +72,18 @@ def make_workload(name):
     from cases import (ConcatCase, ConvCase, FusedCase, MatMulCase, MultiTypeCase, PoolCase,
                        RelayoutCase, ResizeCase, TypeCvtCase)
     from megcc_amd import abi
+    if name == "stem7x7":
+        case = ConvCase(abi.FMT_NCHW_NCHW44, abi.DENSE, 64, 3, 224, 224, 64, 7, 2, 3, abi.RELU,
+                        scales=(0.02, 0.01, 0.05))
+        return case, "qsi8 first layer NCHW->NCHW44 7x7 s2 p3 N=64 3->64 224x224", "hbm"
+    if name == "conv5x5":
+        case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 64, 32, 28, 28, 64, 5, 1, 2, abi.RELU,
+                        scales=(0.02, 0.01, 0.05))
+        return case, "qsi8 conv5x5 s1 p2 NCHW44 N=64 32->64 28x28", "mfma"
+    if name == "pw_s2":
+        case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 64, 256, 56, 56, 512, 1, 2, 0, abi.IDENTITY,
+                        scales=(0.02, 0.01, 0.05))
+        return case, "qsi8 conv1x1 s2 NCHW44 N=64 256->512 56x56 -> 28x28", "mfma"
     if name == "fused":
         return (FusedCase(["I0,SILU,O0", "O0,I1,MUL,O1", "O1,I2,ADD,D"],
                           [(8, 256, 80, 80), (1, 256, 1, 1), (1, 256, 1, 1)]),

@@ -161,6 +161,33 @@ static size_t gather_bytes(const ConvGeom& g) {
     return (size_t)g.n * g.ic * g.oh * g.ow;
 }
 
+// A dense qsi8 convolution with spatial extent on plain NCHW tensors (a model compiled without
+// the NCHW44 layout pass): the matrix-core kernels want 4 channels per pixel next to each other,
+// so the layer runs as relayout NCHW -> NCHW44 into the workspace, the NCHW44 kernel, relayout
+// back. The filter [OC][IC][FH][FW] packs into the same tiles as an NCHW44 one; the bias layouts
+// are the same bytes.
+static bool nchw_spatial(const ConvGeom& g) {
+    return g.fmt == MEGCC_FMT_NCHW && g.groups == 1 && (g.ic & 3) == 0 && (g.oc & 3) == 0 &&
+           !(g.ih == 1 && g.iw == 1 && g.fh == 1 && g.fw == 1);
+}
+static ConvGeom as_nchw44(const ConvGeom& g) {
+    ConvGeom s = g;
+    s.fmt = MEGCC_FMT_NCHW44;
+    return s;
+}
+// [N, C/4, H, W, 4] view (byte strides = element strides) of an NCHW int8 tensor, and the dense one
+static void nchw44_views(int n, int c, int h, int w, Layout* view, Layout* dense) {
+    view->nr_dim = dense->nr_dim = 5;
+    const uint32_t d[5] = {(uint32_t)n, (uint32_t)(c / 4), (uint32_t)h, (uint32_t)w, 4u};
+    const int vs[5] = {c * h * w, 4 * h * w, w, 1, h * w};
+    const int ds[5] = {c * h * w, 4 * h * w, 4 * w, 4, 1};
+    for (int i = 0; i < 5; ++i) {
+        view->dims[i] = dense->dims[i] = d[i];
+        view->stride[i] = vs[i];
+        dense->stride[i] = ds[i];
+    }
+}
+
 }  // namespace mg
 
 using namespace mg;
@@ -233,6 +260,36 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
         Workspace sub = {workspace->ptr, inner, 0};
         return conv_mfma_launch(g1, gathered, flt->ptr, b, dst->ptr, &sub);
     }
+    if (packed && q8 && nchw_spatial(g) && conv_mfma_supported(as_nchw44(g))) {
+        const ConvGeom g1 = as_nchw44(g);
+        MG_REQUIRE(nr_elem(flt->layout) == conv_mfma_packed_bytes(g1), TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: packed filter has %zu bytes, expected %zu", nr_elem(flt->layout),
+                   conv_mfma_packed_bytes(g1));
+        MG_REQUIRE(aligned16(flt->ptr) && (!b || aligned4(b)), TinyNN_ERROR_INVALID_LAYOUT,
+                   "conv2d: misaligned operand");
+        const size_t inner = round_up256(conv_mfma_workspace_bytes(g1));
+        const size_t in44 = round_up256((size_t)g.n * g.ic * g.ih * g.iw);
+        const size_t out44 = (size_t)g.n * g.oc * g.oh * g.ow;
+        MG_REQUIRE(workspace && workspace->ptr && workspace->size >= inner + in44 + out44 &&
+                           aligned16(workspace->ptr),
+                   TinyNN_ERROR_OUT_OF_RANGE,
+                   "conv2d: a dense NCHW convolution needs %zu bytes of workspace", inner + in44 + out44);
+        MG_REQUIRE((long)g.n * g.ic * g.ih * g.iw < (1L << 31) && (long)g.n * g.oc * g.oh * g.ow < (1L << 31),
+                   TinyNN_ERROR_OUT_OF_RANGE, "conv2d: tensor too large");
+        char* src44 = (char*)workspace->ptr + inner;
+        char* dst44 = src44 + in44;
+        Layout view, dense;
+        nchw44_views(g.n, g.ic, g.ih, g.iw, &view, &dense);
+        st = strided_copy(src->ptr, view, src44, dense, 1, "conv2d (NCHW -> NCHW44)");
+        if (st != TinyNN_SUCCESS)
+            return st;
+        Workspace sub = {workspace->ptr, inner, 0};
+        st = conv_mfma_launch(g1, src44, flt->ptr, b, dst44, &sub);
+        if (st != TinyNN_SUCCESS)
+            return st;
+        nchw44_views(g.n, g.oc, g.oh, g.ow, &view, &dense);
+        return strided_copy(dst44, dense, dst->ptr, view, 1, "conv2d (NCHW44 -> NCHW)");
+    }
     if (packed) {
         MG_REQUIRE(q8 && conv_mfma_supported(g), TinyNN_ERROR_INVALID_LAYOUT,
                    "conv2d: a packed filter was passed to a convolution the MFMA kernel does not cover");
@@ -277,7 +334,8 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d_init(
             return st;
         if (strided_pointwise(g))
             g = subsampled(g);
-        pack = conv_mfma_supported(g);
+        // (an NCHW filter packs into the tiles of the NCHW44 kernel: conv_mfma_pack reads g.fmt)
+        pack = nchw_spatial(g) ? conv_mfma_supported(as_nchw44(g)) : conv_mfma_supported(g);
     }
     if (!out_weights) {  // phase 1: how many
         MG_REQUIRE(nr_out_weight, TinyNN_ERROR_NULL_PTR, "conv2d_init: both outputs NULL");
@@ -326,6 +384,10 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d_workspace(
         if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS) {
             if (strided_pointwise(g) && conv_mfma_supported(subsampled(g)))
                 *workspace = round_up256(conv_mfma_workspace_bytes(subsampled(g))) + gather_bytes(g);
+            else if (nchw_spatial(g) && conv_mfma_supported(as_nchw44(g)))
+                *workspace = round_up256(conv_mfma_workspace_bytes(as_nchw44(g))) +
+                             round_up256((size_t)g.n * g.ic * g.ih * g.iw) +
+                             (size_t)g.n * g.oc * g.oh * g.ow;
             else if (conv_mfma_supported(g))
                 *workspace = conv_mfma_workspace_bytes(g);
         }

@@ -255,10 +255,11 @@ struct ConvKernel : KernelFuncBase {
         const int ks = taps <= 2 ? 4 : taps <= 4 ? 2 : 1;
         ss << "    const long P = (long)src.dims[0] * oh * ow, oc = (long)flt.dims[0] * " << r
            << ", ic = (long)src.dims[1] * " << r << ";\n";
+        // NCHW with spatial extent runs as relayout -> NCHW44 kernel -> relayout (conv_api.hip):
+        // both NCHW44 copies live in the workspace, after the split-K room
         if (fmt == "NCHW")
-            ss << "    if (!(src.dims[2] == 1 && src.dims[3] == 1 && " << taps << " == 1 && "
-               << c->getAttrUInt("pad_h") << " == 0 && " << c->getAttrUInt("pad_w")
-               << " == 0)) {\n        *workspace = 0;\n        return TinyNN_SUCCESS;\n    }\n";
+            ss << "    const int spatial = !(src.dims[2] == 1 && src.dims[3] == 1 && " << taps << " == 1);\n"
+               << "    if (spatial && ((ic & 3) || (oc & 3))) {\n        *workspace = 0;\n        return TinyNN_SUCCESS;\n    }\n";
         ss << "    *workspace = 0;\n"
            << "    if ((ic & 3) == 0 && P > 0) {\n"
            << "        const long stages = ((ic + 31) / 32 + " << ks - 1 << ") / " << ks << ";\n"
@@ -275,6 +276,11 @@ struct ConvKernel : KernelFuncBase {
         if (fmt == "NCHW44" && taps == 1 && c->getAttrUInt("pad_h") == 0 && c->getAttrUInt("pad_w") == 0 &&
             (c->getAttrUInt("stride_h") > 1 || c->getAttrUInt("stride_w") > 1))
             ss << "        *workspace = ((*workspace + 255) & ~(size_t)255) + (size_t)P * ic;\n";
+        if (fmt == "NCHW")
+            ss << "        if (spatial)\n"
+               << "            *workspace = ((*workspace + 255) & ~(size_t)255) +\n"
+               << "                         (((size_t)src.dims[0] * ic * src.dims[2] * src.dims[3] + 255) & ~(size_t)255) +\n"
+               << "                         (size_t)P * oc;\n";
         ss << "    }\n"
            << "    return TinyNN_SUCCESS;\n}\n";
         return ss.str();

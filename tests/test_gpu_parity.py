@@ -312,6 +312,25 @@ def test_many_tap_dense_conv(case):
     compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
 
 
+NCHW_SPATIAL = [
+    # dense qsi8 convolutions on plain NCHW tensors (no NCHW44 layout pass): relayout, the NCHW44
+    # matrix-core kernel, relayout back; channel counts that are no multiple of 4 stay on the
+    # one-output-per-thread kernel
+    ConvCase(A.FMT_NCHW, A.DENSE, 2, 16, 20, 24, 12, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(144))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 3, 64, 28, 28, 64, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(576))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 1, 32, 17, 13, 40, 1, 1, 0, A.H_SWISH, scales=(0.02, 0.01, unsat(32))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 2, 8, 15, 15, 8, 3, 1, 2, A.RELU, scales=(0.02, 0.01, unsat(72)), dilate=2),
+    ConvCase(A.FMT_NCHW, A.DENSE, 2, 6, 11, 9, 10, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(54))),
+]
+
+
+@pytest.mark.parametrize("case", NCHW_SPATIAL, ids=[repr(c) for c in NCHW_SPATIAL])
+def test_nchw_spatial_conv(case):
+    port.set_threads(8)
+    arrays = case.gen(seed=59)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+
+
 RESIZE = [
     # the 2x upsampling of detection necks, a camera frame scaled down to a network input, odd
     # ratios, extent 1 either side, a channel slice with a column step as NEAREST source

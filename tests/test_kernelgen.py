@@ -122,6 +122,10 @@ def test_generated_workspace_functions_agree_with_the_library(shim_library):
             k = desc.attr.conv.kernel_h
             cases_ = [[(64, 256, 7, 7, 4), (256, 256, k, k, 4, 4)], [(2, 8, 20, 24, 4), (12, 8, k, k, 4, 4)],
                       [(1, 128, 14, 14, 4), (32, 128, k, k, 4, 4)], [(8, 64, 56, 56, 4), (128, 64, k, k, 4, 4)]]
+        elif desc.kind == 1 and "qsi8" in sym and "_3x3_NCHW_DENSE_" in sym:
+            # plain NCHW with spatial extent: both NCHW44 copies live in the workspace
+            cases_ = [[(2, 8, 20, 24), (12, 8, 3, 3)], [(16, 64, 56, 56), (64, 64, 3, 3)],
+                      [(1, 256, 14, 14), (32, 256, 3, 3)], [(2, 5, 9, 9), (7, 5, 3, 3)]]
         elif desc.kind == 1 and "qsi8" in sym and "_1x1_NCHW_DENSE_p0x0_s1x1" in sym:
             cases_ = [[(64, 1024, 1, 1), (1000, 1024, 1, 1)], [(64, 4096, 1, 1), (4096, 4096, 1, 1)],
                       [(1, 1024, 1, 1), (1000, 1024, 1, 1)], [(4096, 4096, 1, 1), (4096, 4096, 1, 1)]]

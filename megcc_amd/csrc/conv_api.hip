@@ -175,6 +175,17 @@ static ConvGeom as_nchw44(const ConvGeom& g) {
     s.fmt = MEGCC_FMT_NCHW44;
     return s;
 }
+// Channel-wise (depthwise) qsi8 convolution on plain NCHW tensors: the same detour around the
+// NCHW44 depthwise kernel; the filter [G,1,1,FH,FW] becomes [G/4,1,1,FH,FW,4] by a third, tiny
+// relayout. Workspace = [input copy, 256][output copy, 256][filter].
+static bool nchw_depthwise(const ConvGeom& g) {
+    return g.fmt == MEGCC_FMT_NCHW && g.groups > 1 && g.groups == g.ic && g.ic == g.oc && (g.ic & 3) == 0 &&
+           (long)g.n * g.ic * g.ih * g.iw < (1L << 31) && (long)g.n * g.oc * g.oh * g.ow < (1L << 31);
+}
+static size_t nchw_depthwise_bytes(const ConvGeom& g) {
+    return round_up256((size_t)g.n * g.ic * g.ih * g.iw) + round_up256((size_t)g.n * g.oc * g.oh * g.ow) +
+           (size_t)g.ic * g.fh * g.fw;
+}
 // [N, C/4, H, W, 4] view (byte strides = element strides) of an NCHW int8 tensor, and the dense one
 static void nchw44_views(int n, int c, int h, int w, Layout* view, Layout* dense) {
     view->nr_dim = dense->nr_dim = 5;
@@ -301,6 +312,34 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
                    TinyNN_ERROR_INVALID_LAYOUT, "conv2d: misaligned operand");
         return conv_mfma_launch(g, src->ptr, flt->ptr, b, dst->ptr, workspace);
     }
+    if (q8 && nchw_depthwise(g) && dwconv44_supported(as_nchw44(g)) && workspace && workspace->ptr &&
+        workspace->size >= nchw_depthwise_bytes(g) && aligned16(workspace->ptr)) {
+        const ConvGeom g1 = as_nchw44(g);
+        char* src44 = (char*)workspace->ptr;
+        char* dst44 = src44 + round_up256((size_t)g.n * g.ic * g.ih * g.iw);
+        char* flt44 = dst44 + round_up256((size_t)g.n * g.oc * g.oh * g.ow);
+        Layout view, dense;
+        nchw44_views(g.n, g.ic, g.ih, g.iw, &view, &dense);
+        st = strided_copy(src->ptr, view, src44, dense, 1, "conv2d (NCHW -> NCHW44)");
+        if (st != TinyNN_SUCCESS)
+            return st;
+        const int taps = g.fh * g.fw;
+        Layout fv = {}, fd = {};  // [G/4, taps, 4]: channel c = 4 * group + lane
+        fv.nr_dim = fd.nr_dim = 3;
+        fv.dims[0] = fd.dims[0] = (uint32_t)(g.ic / 4);
+        fv.dims[1] = fd.dims[1] = (uint32_t)taps;
+        fv.dims[2] = fd.dims[2] = 4;
+        fv.stride[0] = 4 * taps; fv.stride[1] = 1; fv.stride[2] = taps;
+        fd.stride[0] = 4 * taps; fd.stride[1] = 4; fd.stride[2] = 1;
+        st = strided_copy(flt->ptr, fv, flt44, fd, 1, "conv2d (depthwise filter -> NCHW44)");
+        if (st != TinyNN_SUCCESS)
+            return st;
+        st = dwconv44_launch(g1, src44, flt44, b, dst44);
+        if (st != TinyNN_SUCCESS)
+            return st;
+        nchw44_views(g.n, g.oc, g.oh, g.ow, &view, &dense);
+        return strided_copy(dst44, dense, dst->ptr, view, 1, "conv2d (NCHW44 -> NCHW)");
+    }
     if (q8 && dwconv44_supported(g) && aligned4(src->ptr) && aligned4(flt->ptr) &&
         aligned4(dst->ptr))
         return dwconv44_launch(g, src->ptr, flt->ptr, b, dst->ptr);
@@ -378,6 +417,9 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d_workspace(
         if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS &&
             conv_f32_gemm_supported(g))
             *workspace = conv_f32_gemm_workspace_bytes(g);
+    } else if (is_q8(src) && is_q8(flt) && attr->sparse == MEGCC_SPARSE_GROUP) {
+        if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS && nchw_depthwise(g))
+            *workspace = nchw_depthwise_bytes(g);
     } else if (is_q8(src) && is_q8(flt) && attr->sparse == MEGCC_SPARSE_DENSE &&
                !is_packed_filter(flt)) {
         // split-K partial sums of the one-stage MFMA kernel (few pixels, long K)

@@ -229,6 +229,29 @@ struct ConvKernel : KernelFuncBase {
         const bool dense = c->getAttrStr("sparse") == "DENSE";
         const unsigned taps = c->getAttrUInt("kernel_h") * c->getAttrUInt("kernel_w");
         const bool q8_mfma = !f32 && dense && (fmt == "NCHW44" || fmt == "NCHW") && taps <= 9;
+        if (!f32 && !dense && fmt == "NCHW") {
+            // channel-wise on plain NCHW: NCHW44 copies of input, output and filter (conv_api.hip)
+            std::stringstream ss;
+            ss << "TinyNNStatus " << GetWorkspaceSignature(c) << " {\n"
+               << "    const Layout src = inputs[0]->layout, flt = inputs[1]->layout;\n"
+               << "    const long eh = " << c->getAttrUInt("dilate_h") << " * (" << c->getAttrUInt("kernel_h")
+               << " - 1) + 1, ew = " << c->getAttrUInt("dilate_w") << " * (" << c->getAttrUInt("kernel_w")
+               << " - 1) + 1;\n"
+               << "    const long ih = src.dims[2] + 2 * " << c->getAttrUInt("pad_h")
+               << ", iw = src.dims[3] + 2 * " << c->getAttrUInt("pad_w") << ";\n"
+               << "    const long oh = ih >= eh ? (ih - eh) / " << c->getAttrUInt("stride_h")
+               << " + 1 : 0, ow = iw >= ew ? (iw - ew) / " << c->getAttrUInt("stride_w") << " + 1 : 0;\n"
+               << "    const long n = src.dims[0], ch = src.dims[1];\n"
+               << "    const long in = n * ch * src.dims[2] * src.dims[3], out = n * ch * oh * ow;\n"
+               << "    *workspace = 0;\n"
+               << "    /* one output channel per input channel, a multiple of 4 of them */\n"
+               << "    if (flt.nr_dim == 5 && flt.dims[0] == ch && flt.dims[1] == 1 && flt.dims[2] == 1 && (ch & 3) == 0 &&\n"
+               << "        in < (1L << 31) && out < (1L << 31))\n"
+               << "        *workspace = ((size_t)(in + 255) & ~(size_t)255) + ((size_t)(out + 255) & ~(size_t)255) + (size_t)ch * "
+               << taps << ";\n"
+               << "    return TinyNN_SUCCESS;\n}\n";
+            return ss.str();
+        }
         if (!(f32 && fmt == "NCHW" && dense) && !q8_mfma)
             return "TinyNNStatus " + GetWorkspaceSignature(c) +
                    " {\n    *workspace = 0;\n    return TinyNN_SUCCESS;\n}\n";

@@ -331,6 +331,23 @@ def test_nchw_spatial_conv(case):
     compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
 
 
+NCHW_DW = [
+    # channel-wise qsi8 convolution on plain NCHW tensors: the NCHW44 depthwise kernel between
+    # relayouts (channel counts that are multiples of 4; the others stay on the generic kernel)
+    ConvCase(A.FMT_NCHW, A.GROUP, 4, 32, 56, 56, 32, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW, A.GROUP, 3, 16, 29, 31, 16, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW, A.GROUP, 2, 8, 13, 17, 8, 5, 1, 2, A.H_SWISH, scales=(0.02, 0.01, unsat(25))),
+    ConvCase(A.FMT_NCHW, A.GROUP, 2, 6, 9, 7, 6, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+]
+
+
+@pytest.mark.parametrize("case", NCHW_DW, ids=[repr(c) for c in NCHW_DW])
+def test_nchw_depthwise_conv(case):
+    port.set_threads(8)
+    arrays = case.gen(seed=61)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+
+
 RESIZE = [
     # the 2x upsampling of detection necks, a camera frame scaled down to a network input, odd
     # ratios, extent 1 either side, a channel slice with a column step as NEAREST source

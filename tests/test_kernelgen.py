@@ -122,6 +122,10 @@ def test_generated_workspace_functions_agree_with_the_library(shim_library):
             k = desc.attr.conv.kernel_h
             cases_ = [[(64, 256, 7, 7, 4), (256, 256, k, k, 4, 4)], [(2, 8, 20, 24, 4), (12, 8, k, k, 4, 4)],
                       [(1, 128, 14, 14, 4), (32, 128, k, k, 4, 4)], [(8, 64, 56, 56, 4), (128, 64, k, k, 4, 4)]]
+        elif desc.kind == 1 and "qsi8" in sym and "_NCHW_GROUP_" in sym:
+            k = desc.attr.conv.kernel_h
+            cases_ = [[(64, 32, 112, 112), (32, 1, 1, k, k)], [(2, 8, 9, 7), (8, 1, 1, k, k)],
+                      [(2, 6, 9, 7), (6, 1, 1, k, k)]]
         elif desc.kind == 1 and "qsi8" in sym and "_3x3_NCHW_DENSE_" in sym:
             # plain NCHW with spatial extent: both NCHW44 copies live in the workspace
             cases_ = [[(2, 8, 20, 24), (12, 8, 3, 3)], [(16, 64, 56, 56), (64, 64, 3, 3)],

@@ -133,6 +133,9 @@ LIVE = [
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 30, 34, 8, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),  # generic path (IW % 4 != 0)
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
+    PoolCase(A.FMT_NCHW, A.POOL_MAX, 3, 5, 10, 24, 2, 2, 0),   # 8-byte row pieces, odd plane count
+    PoolCase(A.FMT_NCHW, A.POOL_MAX, 3, 5, 11, 24, 2, 2, 0),   # odd height: the generic kernel
+    PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 7, 10, 20, 2, 2, 0),   # IW % 8 != 0: the generic kernel
     PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE, 5, 1024, 7, 7, 7, 7, 0),
     PoolCase(A.FMT_NCHW, A.POOL_AVERAGE, 5, 1024, 7, 7, 7, 7, 0),
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 3, 64, 13, 13, 13, 13, 0),  # one output pixel per plane

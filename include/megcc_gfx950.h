@@ -230,7 +230,9 @@ typedef enum {
     MEGCC_REDUCE_SUM = 0,
     MEGCC_REDUCE_MEAN = 1,
     MEGCC_REDUCE_MAX = 2,
-    MEGCC_REDUCE_MIN = 3
+    MEGCC_REDUCE_MIN = 3,
+    MEGCC_REDUCE_PRODUCT = 4,
+    MEGCC_REDUCE_SUM_SQR = 5
 } MegccReduceMode;
 
 typedef struct {
@@ -323,8 +325,13 @@ TinyNNStatus megcc_gfx950_elemwise_multitype(
         const MegccMultiTypeMode* mode, Tensor** inputs, int nr_input, Tensor** outputs,
         int nr_output, const Workspace* workspace, const RuntimeOpt* opt);
 
-/* f32 elementwise, unary or binary with the same broadcast rules as above plus a trailing-axis
- * vector ([M,N] op [N], the FullyConnected bias). Replaces GeneralIntrinsic::ElemwiseKernel
+/* f32 elementwise, unary (inputs = {a}) or binary (inputs = {a, b}) over the broadcast of the two
+ * operand shapes: shapes are aligned at their last dim, an extent of 1 stretches, the output has
+ * the broadcast shape. That covers every operand pairing the reference names
+ * (Common/ElemwiseCommon.cpp:47-127: VEC_VEC, VEC_SCALAR, VEC_BCAST101, VEC_BCAST101xX,
+ * VEC_BCAST111C - [M,N] + [N], the FullyConnected bias -, VEC_BV, VEC_BCAST110, their mirrored
+ * forms and NAIVE). More than one merged dim: fewer than 2^31 elements. Replaces
+ * GeneralIntrinsic::ElemwiseKernel
  * (GeneralIntrinsic/Elemwise/Elemwise.cpp:10-36) / BareMetal::ElmwiseKernel
  * (BareMetal/ElemwiseKernel.cpp:35-66,413-431). */
 TinyNNStatus megcc_gfx950_elemwise(
@@ -453,6 +460,18 @@ TinyNNStatus megcc_gfx950_wait(void);
 void* megcc_gfx950_stream(void);
 /* Text of the most recent error on the calling thread ("" if none). */
 const char* megcc_gfx950_last_error(void);
+/* Diagnostics (no counterpart in the reference, whose kernel choice is fixed at compile time):
+ * which kernel variant the calling thread's most recent operator call selected, as
+ * "<kernel>[:n,n,...]" (e.g. "conv_mfma_i8_dma:3,128,512,1024" = variant, oc tile, pixel
+ * sub-tile, patch slots). The text lives until the thread's next call of this function. */
+const char* megcc_gfx950_last_kernel(void);
+/* Kernel-selection overrides, for regression tests of kernels that un-switched shapes only reach
+ * through a fallback: "nopws", "nogevm", "nofcb", "nosmall", "nopm768", "nopm", "nodma512",
+ * "nopm256", "nodma", "nows", "nowide", "nofcs", "nopwshare", "nohybrid", "nodot4", "nof32small",
+ * "dw_generic", "no_graph"; value 1 takes the kernel out of the dispatch, 0 puts it back. The
+ * same names in capitals behind MEGCC_ are read from the environment once, at first use.
+ * Unknown names return TinyNN_ERROR_NO_FOUND. */
+TinyNNStatus megcc_gfx950_set_option(const char* name, int value);
 
 /* ------------------------------------------------------------------------------------------
  * In-memory model runtime: MegCC's static memory plan on one HBM arena. The calls mirror what the

@@ -40,7 +40,8 @@ EW_ADD, EW_SUB, EW_MUL, EW_TRUE_DIV, EW_MAX, EW_MIN, EW_FUSE_ADD_RELU = 16, 17, 
 EW_MODES = {"RELU": 0, "EXP": 1, "SIGMOID": 2, "H_SWISH": 3, "NEGATE": 4, "ADD": 16, "SUB": 17,
             "MUL": 18, "TRUE_DIV": 19, "MAX": 20, "MIN": 21, "FUSE_ADD_RELU": 22}
 # MegccReduceMode
-REDUCE_SUM, REDUCE_MEAN, REDUCE_MAX, REDUCE_MIN = 0, 1, 2, 3
+REDUCE_SUM, REDUCE_MEAN, REDUCE_MAX, REDUCE_MIN, REDUCE_PRODUCT, REDUCE_SUM_SQR = 0, 1, 2, 3, 4, 5
+REDUCE_MODES = {"SUM": 0, "MEAN": 1, "MAX": 2, "MIN": 3, "PRODUCT": 4, "SUM_SQR": 5}
 # MegccKernelKind
 KERN_CONV, KERN_MATMUL, KERN_POOLING, KERN_ELEMWISE_MULTITYPE = 1, 2, 3, 4
 KERN_ELEMWISE, KERN_TYPECVT, KERN_REDUCE = 5, 6, 7

@@ -145,6 +145,8 @@ const ModeName kMultiType[] = {
         {"QRELU", MEGCC_Q_RELU},
 };
 const ModeName kReduce[] = {
+        {"SUM_SQR", MEGCC_REDUCE_SUM_SQR},
+        {"PRODUCT", MEGCC_REDUCE_PRODUCT},
         {"SUM", MEGCC_REDUCE_SUM},
         {"MEAN", MEGCC_REDUCE_MEAN},
         {"MAX", MEGCC_REDUCE_MAX},

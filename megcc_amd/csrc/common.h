@@ -1,5 +1,5 @@
 // Shared host-side helpers of libmegcc_gfx950.so: error reporting, the library stream, Tensor
-// inspection. Everything here is host code; device helpers live in epilogue.cuh.
+// inspection. Everything here is host code; device helpers live in epilogue.h.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -22,6 +22,20 @@ TinyNNStatus fail(TinyNNStatus st, const char* fmt, ...) __attribute__((format(p
         if (!(cond))                       \
             return ::mg::fail(st, __VA_ARGS__); \
     } while (0)
+
+// Kernel-selection overrides: each one takes a kernel (or a variant of one) out of the dispatch so
+// that the regression tests can reach the kernels that serve the shapes behind it. Read from the
+// environment (MEGCC_NOPWS=1, ...) ONCE, when the library first consults them; later changes go
+// through megcc_gfx950_set_option(). Nothing on a launch path scans the environment.
+struct Options {
+    bool no_pws, no_gevm, no_fcb, no_small, no_pm768, no_pm, no_dma512, no_pm256, no_dma, no_ws,
+            no_wide, no_fcs, no_pwshare, no_hybrid, no_dot4, no_f32small, dw_generic, no_graph;
+};
+Options& options();
+
+// Which kernel variant the most recent dispatch on this thread selected: `name` (a string literal)
+// and up to five numbers that identify the instantiation; megcc_gfx950_last_kernel() formats them.
+void note_kernel(const char* name, int a = -1, int b = -1, int c = -1, int d = -1, int e = -1);
 
 // After a kernel launch: surfaces launch-configuration errors as TinyNN_ERROR_RUNTIME.
 TinyNNStatus check_launch(const char* what);

@@ -334,6 +334,7 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
         st = strided_copy(flt->ptr, fv, flt44, fd, 1, "conv2d (depthwise filter -> NCHW44)");
         if (st != TinyNN_SUCCESS)
             return st;
+        note_kernel("dwconv44 between NCHW relayouts");
         st = dwconv44_launch(g1, src44, flt44, b, dst44);
         if (st != TinyNN_SUCCESS)
             return st;
@@ -341,20 +342,33 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
         return strided_copy(dst44, dense, dst->ptr, view, 1, "conv2d (NCHW44 -> NCHW)");
     }
     if (q8 && dwconv44_supported(g) && aligned4(src->ptr) && aligned4(flt->ptr) &&
-        aligned4(dst->ptr))
+        aligned4(dst->ptr)) {
+        note_kernel("dwconv44");
         return dwconv44_launch(g, src->ptr, flt->ptr, b, dst->ptr);
-    if (q8 && conv_first_supported(g) && aligned4(src->ptr) && aligned4(dst->ptr) && (!b || aligned4(b)))
+    }
+    if (q8 && conv_first_supported(g) && aligned4(src->ptr) && aligned4(dst->ptr) && (!b || aligned4(b))) {
+        note_kernel("conv_first_q8");
         return conv_first_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+    }
     if (q8 && conv_hybrid_mfma_supported(g) && aligned4(dst->ptr) && aligned4(flt->ptr) && (!b || aligned4(b)) &&
-        !getenv("MEGCC_NOHYBRID"))
+        !options().no_hybrid) {
+        note_kernel("conv_hybrid_mfma");
         return conv_hybrid_mfma_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+    }
     if (q8 && conv_dot4_supported(g) && aligned4(src->ptr) && aligned4(dst->ptr) && aligned16(flt->ptr) &&
-        (!b || aligned4(b)) && !getenv("MEGCC_NODOT4"))
+        (!b || aligned4(b)) && !options().no_dot4) {
+        note_kernel("conv_dot4");
         return conv_dot4_launch(g, src->ptr, flt->ptr, b, dst->ptr);
-    if (f32 && conv_f32_small_supported(g) && !getenv("MEGCC_NOF32SMALL"))
+    }
+    if (f32 && conv_f32_small_supported(g) && !options().no_f32small) {
+        note_kernel("conv_f32_small");
         return conv_f32_small_launch(g, src->ptr, flt->ptr, b, dst->ptr);
-    if (f32 && conv_f32_gemm_supported(g))
+    }
+    if (f32 && conv_f32_gemm_supported(g)) {
+        note_kernel("conv_f32_gemm");
         return conv_f32_gemm_launch(g, src->ptr, flt->ptr, b, dst->ptr, workspace);
+    }
+    note_kernel("conv_direct");
     return conv_direct_launch(g, f32, src->ptr, flt->ptr, b, dst->ptr);
 }
 

@@ -6,7 +6,7 @@
 // depthwise on dwconv.hip, f32 NCHW dense on gemm_f32.hip.
 #include "common.h"
 #include "conv_geom.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
 
 namespace mg {
 

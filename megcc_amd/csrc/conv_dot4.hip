@@ -12,7 +12,7 @@
 //     one-output-per-thread kernel, far below the matrix cores - a fallback, not a fast path.
 #include "common.h"
 #include "conv_geom.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
 
 namespace mg {
 

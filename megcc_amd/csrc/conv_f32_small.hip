@@ -9,7 +9,7 @@
 // held to the 1e-4 tolerance, not to bit equality).
 #include "common.h"
 #include "conv_geom.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
 
 namespace mg {
 

@@ -16,7 +16,7 @@
 // Only the top row and the left column can be padding for even IH, IW.
 #include "common.h"
 #include "conv_geom.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
 
 namespace mg {
 

@@ -26,7 +26,7 @@
 #include "common.h"
 #include "conv_geom.h"
 #include "conv_mfma_i8.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
 
 namespace mg {
 

@@ -6,7 +6,8 @@
 
 #include "common.h"
 #include "conv_geom.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
+#include "fastdiv.h"
 
 namespace mg {
 
@@ -20,30 +21,6 @@ static constexpr int MAX_TAPS_STAGE = 9;
 static constexpr int MAX_B_ITEMS = 8;  // 16-byte gather items per thread per stage
 static constexpr int OC_PAD = 256;   // packed filter rows are padded to the largest oc tile
 static constexpr int CHUNK_PAD = 4;  // ... and ic chunks to the largest sub-chunk count per stage
-
-// unsigned division by a run-time constant: q = (x * mul) >> (32 + shift), exact for x < 2^31
-struct FastDiv {
-    uint32_t mul, shift, d;
-};
-static inline FastDiv make_fastdiv(uint32_t d) {
-    FastDiv f;
-    f.d = d;
-    if (d == 1) {
-        f.mul = 0;
-        f.shift = 0;
-        return f;
-    }
-    uint32_t s = 0;
-    while ((1u << s) < d)
-        ++s;  // ceil(log2 d)
-    uint64_t m = ((uint64_t(1) << (32 + s - 1)) + d - 1) / d;  // fits 32 bits for x < 2^31
-    f.mul = (uint32_t)m;
-    f.shift = s - 1;
-    return f;
-}
-__device__ __forceinline__ uint32_t fdiv(uint32_t x, const FastDiv& f) {
-    return f.d == 1 ? x : (__umulhi(x, f.mul) >> f.shift);
-}
 
 struct MfmaParams {
     const int8_t* src;
@@ -70,7 +47,7 @@ struct MfmaParams {
     FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
     int G, RG;       // 16-byte gather: pixel groups per row, groups per plane of the largest patch
     FastDiv dG, dRG;
-    // exact requantisation thresholds for IDENTITY / RELU (built on the host, epilogue.cuh); only
+    // exact requantisation thresholds for IDENTITY / RELU (built on the host, epilogue.h); only
     // the kernels that look outputs up in LDS read it
     RequantTable rq_table;
 };

@@ -5,7 +5,7 @@
 // MegCC uses as quantized FullyConnected, the scalar seven-deep loop of BareMetal::ConvGeneral
 // (compiler/lib/KernelGen/BareMetal/ConvKernel.cpp:305-344). int8 x int8 products are summed
 // exactly in int32, so any summation order gives the reference's accumulator; the epilogue is the
-// reference's float sequence (epilogue.cuh).
+// reference's float sequence (epilogue.h).
 //
 // Data movement per workgroup (256 threads = 4 waves in a 2x2 grid, tile BM oc x 128 pixels):
 //   * the filter is pre-packed once by the _init entry point into rows of 32 consecutive input
@@ -491,39 +491,43 @@ TinyNNStatus conv_mfma_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst,
         const Workspace* ws) {
     // pointwise layers with few input channels: the streaming kernel (conv_pw_stream.hip)
-    if (conv_pw_stream_supported(g) && !getenv("MEGCC_NOPWS"))
-        return conv_pw_stream_launch(g, src, packed, bias, dst);
+    if (conv_pw_stream_supported(g) && !options().no_pws)
+        return conv_pw_stream_launch(g, src, packed, bias, dst);  // (notes its own variant)
     // FullyConnected with at most 4 rows: one pass over the weights (fc_gevm_q8.hip)
-    if (is_fc(g) && fc_gevm_q8_supported(g) && !getenv("MEGCC_NOGEVM"))
+    if (is_fc(g) && fc_gevm_q8_supported(g) && !options().no_gevm) {
+        note_kernel("fc_gevm_q8");
         return fc_gevm_q8_launch(g, src, packed, bias, dst);
+    }
     MfmaParams q = {};
     PipeConfig pc;
     const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;
-    const bool b128_ok = ((uintptr_t)src & 15) == 0 && !getenv("MEGCC_NOFCB");
+    const bool b128_ok = ((uintptr_t)src & 15) == 0 && !options().no_fcb;
     // candidates in order of preference; development switches (MEGCC_NO...) skip one
     long range_len = 0;
     TilePlan t;
     bool pipe = false;
+    int picked = -1;  // DMA variant, 100 = producer/consumer kernel, 101 = register-staged kernel
     // DMA kernel variants in order of preference (see conv_mfma_dma_config), then the two older
     // generations
     static const int kDmaVariants[] = {6, 7, 2, 3, 0, 4, 1};
-    static const char* const kDmaSwitch[] = {"MEGCC_NOSMALL", "MEGCC_NOSMALL", "MEGCC_NOPM768", "MEGCC_NOPM",
-                                             "MEGCC_NODMA512", "MEGCC_NOPM256", "MEGCC_NODMA"};
+    const Options& opt = options();
+    const bool dma_off[] = {opt.no_small, opt.no_small, opt.no_pm768, opt.no_pm,
+                            opt.no_dma512, opt.no_pm256, opt.no_dma};
     constexpr int N_DMA_VARIANTS = 7;
     for (int cand = 0; cand < N_DMA_VARIANTS + 2 && !pipe; ++cand) {
         bool have = false;
         if (cand < N_DMA_VARIANTS) {
             const int v = kDmaVariants[cand];
-            have = !getenv("MEGCC_NODMA") && !getenv(kDmaSwitch[cand]) &&
-                   !((v == 2 || v == 4 || v == 6) && getenv("MEGCC_NOPM")) &&
+            have = !opt.no_dma && !dma_off[cand] && !((v == 2 || v == 4 || v == 6) && opt.no_pm) &&
                    conv_mfma_dma_config(g, is_fc(g), v, b128_ok, &pc);
         } else if (cand == N_DMA_VARIANTS) {
-            have = !getenv("MEGCC_NOWS") && conv_mfma_ws_config(g, g4_ok, &pc);
+            have = !opt.no_ws && conv_mfma_ws_config(g, g4_ok, &pc);
         } else {
-            have = !getenv("MEGCC_NOWIDE") && conv_mfma_pipe_config(g, g4_ok, &pc);
+            have = !opt.no_wide && conv_mfma_pipe_config(g, g4_ok, &pc);
         }
         if (!have)
             continue;
+        picked = cand < N_DMA_VARIANTS ? kDmaVariants[cand] : 100 + cand - N_DMA_VARIANTS;
         // one pixel range per free workgroup slot, so that the whole grid is resident at once and
         // every CU finishes at the same time (no partial last round)
         const long P = (long)g.n * g.oh * g.ow;
@@ -617,14 +621,19 @@ TinyNNStatus conv_mfma_launch(
     q.split = 1;
     q.sps = q.stages;
     q.partial = nullptr;
-    if (pipe)
+    if (pipe) {
+        note_kernel(picked >= 100 ? (picked == 100 ? "conv_mfma_i8_ws" : "conv_mfma_i8_wide")
+                                  : "conv_mfma_i8_dma",
+                    picked >= 100 ? -1 : picked, pc.bm, pc.bn, q.Lmax, pc.ks);
         return conv_mfma_pipe_launch(pc, q);
+    }
     const int split = conv_mfma_split(g);
     // FullyConnected with few rows: stream the weights (fc_stream.hip), finish with the reduce
     // kernel below
-    if (fc && split > 1 && ws && ws->ptr && ((uintptr_t)ws->ptr & 15) == 0 && !getenv("MEGCC_NOFCS")) {
+    if (fc && split > 1 && ws && ws->ptr && ((uintptr_t)ws->ptr & 15) == 0 && !options().no_fcs) {
         const int fs = fc_stream_split(g, src, ws->size, split);
         if (fs > 0) {
+            note_kernel("fc_stream", fs);
             TinyNNStatus st = fc_stream_launch(g, src, packed, (int32_t*)ws->ptr, fs);
             if (st != TinyNN_SUCCESS)
                 return st;
@@ -648,6 +657,7 @@ TinyNNStatus conv_mfma_launch(
     }
 
     const int bm = conv_mfma_bm(g);
+    note_kernel("conv_mfma_i8", bm, q.split);
     const size_t lds = (size_t)q.taps * q.KS * bm * KROW + (size_t)q.KS * q.Lmax * KROW;
     MG_REQUIRE(lds <= 160 * 1024, TinyNN_ERROR_OUT_OF_RANGE, "conv_mfma: %zu bytes of LDS", lds);
     dim3 grid((q.P + BN - 1) / BN, (g.oc + bm - 1) / bm, q.split);

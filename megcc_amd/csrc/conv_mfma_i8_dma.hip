@@ -16,7 +16,7 @@
 // One workgroup = 8 waves (2 x 4) on a 128 oc x 256 pixel tile, 64 accumulators per lane. The
 // loads of the next sub-tile's first stages are already in flight while a sub-tile's epilogue runs.
 //
-// Requantisation uses the exact threshold table (epilogue.cuh) built once per workgroup.
+// Requantisation uses the exact threshold table (epilogue.h) built once per workgroup.
 #include <stdlib.h>
 
 #include "conv_mfma_i8.h"

@@ -18,7 +18,7 @@
 // them can be resident and the memory latency is hidden by occupancy.
 //
 // Same arithmetic as the other qsi8 kernels: int32 accumulators starting from the bias, exact
-// requantisation by threshold table (epilogue.cuh). Reference loop: BareMetal/ConvKernel.cpp:305-344.
+// requantisation by threshold table (epilogue.h). Reference loop: BareMetal/ConvKernel.cpp:305-344.
 #include <stdlib.h>
 
 #include <map>
@@ -364,7 +364,7 @@ TinyNNStatus conv_pw_stream_launch(
 #undef MG_PW_PICK
 
     // 512 input channels and more tiles than resident waves: the workgroup-shared form
-    if (g.ic == 512 && (q.groups & 3) == 0 && !getenv("MEGCC_NOPWSHARE")) {
+    if (g.ic == 512 && (q.groups & 3) == 0 && !options().no_pwshare) {
         const void* sk = act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_share_kernel<16, MEGCC_NONLINE_IDENTITY>
                          : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_share_kernel<16, MEGCC_NONLINE_RELU>
                                                        : (const void*)conv_pw_share_kernel<16, -1>;
@@ -377,6 +377,7 @@ TinyNNStatus conv_pw_stream_launch(
             if (runs < 1)
                 runs = 1;
             void* sargs[] = {&q};
+            note_kernel("conv_pw_share", g.ic / 32);
             hipError_t e = hipLaunchKernel(sk, dim3((unsigned)(runs * gblocks)), dim3(PW_THREADS), sargs, 0, stream());
             MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_pw_share: %s", hipGetErrorString(e));
             return check_launch("conv_pw_share");
@@ -399,6 +400,7 @@ TinyNNStatus conv_pw_stream_launch(
     const unsigned blocks = (unsigned)(waves / 4);
 
     void* args[] = {&q};
+    note_kernel("conv_pw_stream", g.ic / 32);
     hipError_t e = hipLaunchKernel(kern, dim3(blocks), dim3(PW_THREADS), args, 0, stream());
     MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_pw_stream: %s", hipGetErrorString(e));
     return check_launch("conv_pw_stream");

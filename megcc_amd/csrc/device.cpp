@@ -3,6 +3,8 @@
 // per-thread error text.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
 
 #include <mutex>
 
@@ -13,6 +15,56 @@ namespace mg {
 static hipStream_t g_stream = nullptr;
 static std::once_flag g_stream_once;
 static thread_local char g_error[512] = "";
+
+namespace {
+struct OptionName {
+    const char* name;  // option name; the environment variable is MEGCC_<NAME in capitals>
+    bool Options::*field;
+};
+const OptionName kOptions[] = {
+        {"nopws", &Options::no_pws},         {"nogevm", &Options::no_gevm},
+        {"nofcb", &Options::no_fcb},         {"nosmall", &Options::no_small},
+        {"nopm768", &Options::no_pm768},     {"nopm", &Options::no_pm},
+        {"nodma512", &Options::no_dma512},   {"nopm256", &Options::no_pm256},
+        {"nodma", &Options::no_dma},         {"nows", &Options::no_ws},
+        {"nowide", &Options::no_wide},       {"nofcs", &Options::no_fcs},
+        {"nopwshare", &Options::no_pwshare}, {"nohybrid", &Options::no_hybrid},
+        {"nodot4", &Options::no_dot4},       {"nof32small", &Options::no_f32small},
+        {"dw_generic", &Options::dw_generic}, {"no_graph", &Options::no_graph},
+};
+struct KernelNote {
+    const char* name;
+    int v[5];
+};
+thread_local KernelNote g_note = {"", {-1, -1, -1, -1, -1}};
+thread_local char g_note_text[160];
+}  // namespace
+
+Options& options() {
+    static Options opt = [] {
+        Options o = {};
+        for (const OptionName& n : kOptions) {
+            char env[48] = "MEGCC_";
+            size_t k = strlen(env);
+            for (const char* c = n.name; *c && k + 1 < sizeof(env); ++c)
+                env[k++] = (*c >= 'a' && *c <= 'z') ? (char)(*c - 'a' + 'A') : *c;
+            env[k] = 0;
+            const char* v = getenv(env);
+            o.*(n.field) = v && *v && strcmp(v, "0") != 0;
+        }
+        return o;
+    }();
+    return opt;
+}
+
+void note_kernel(const char* name, int a, int b, int c, int d, int e) {
+    g_note.name = name;
+    g_note.v[0] = a;
+    g_note.v[1] = b;
+    g_note.v[2] = c;
+    g_note.v[3] = d;
+    g_note.v[4] = e;
+}
 
 hipStream_t stream() {
     std::call_once(g_stream_once, [] {
@@ -134,6 +186,23 @@ void* megcc_gfx950_stream(void) {
 
 const char* megcc_gfx950_last_error(void) {
     return g_error;
+}
+
+const char* megcc_gfx950_last_kernel(void) {
+    int n = snprintf(g_note_text, sizeof(g_note_text), "%s", g_note.name);
+    for (int i = 0; i < 5 && g_note.v[i] != -1 && n > 0 && n < (int)sizeof(g_note_text); ++i)
+        n += snprintf(g_note_text + n, sizeof(g_note_text) - n, "%c%d", i ? ',' : ':', g_note.v[i]);
+    return g_note_text;
+}
+
+TinyNNStatus megcc_gfx950_set_option(const char* name, int value) {
+    MG_REQUIRE(name, TinyNN_ERROR_NULL_PTR, "set_option: NULL name");
+    for (const OptionName& n : kOptions)
+        if (strcmp(n.name, name) == 0) {
+            options().*(n.field) = value != 0;
+            return TinyNN_SUCCESS;
+        }
+    return fail(TinyNN_ERROR_NO_FOUND, "set_option: unknown option '%s'", name);
 }
 
 }  // extern "C"

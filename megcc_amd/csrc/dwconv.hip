@@ -9,7 +9,7 @@
 #include "common.h"
 #include "conv_geom.h"
 #include "conv_mfma_i8.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
 
 namespace mg {
 
@@ -240,7 +240,7 @@ TinyNNStatus dwconv44_launch(
     size_t total = (size_t)g.n * (g.oc >> 2) * g.oh * g.ow;
     if (total == 0)
         return TinyNN_SUCCESS;
-    if (dwconv44_3x3_ok(g, src, dst) && !getenv("MEGCC_DW_GENERIC")) {
+    if (dwconv44_3x3_ok(g, src, dst) && !options().dw_generic) {
         // one thread per R output rows x 4 output pixels x 4 channels
         // (two rows share input rows and the weight set-up: measured faster for stride 1 on
         // large planes only)

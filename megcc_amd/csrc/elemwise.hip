@@ -11,7 +11,8 @@
 //   typecvt (GI)    x * (src_scale/dst_scale), roundf, clamp    GeneralIntrinsic/Typecvt.cpp:173-190,262-281
 //   typecvt q32->q8 x * src_scale / dst_scale, roundf, clamp    BareMetal/Typecvt.cpp:43-105
 #include "common.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
+#include "fastdiv.h"
 
 namespace mg {
 
@@ -107,37 +108,83 @@ __device__ __forceinline__ float ew_one(float x, float y) {
     }
 }
 
-template <int MODE, bool VEC>
-__global__ void __launch_bounds__(256) elemwise_f32_kernel(EwArgs p) {
-    const float* a = (const float*)p.a;
-    const float* b = (const float*)p.b;
-    float* d = (float*)p.d;
+// f32 elementwise over the broadcast of two dense operands (GetBinaryBcastType of the reference,
+// Common/ElemwiseCommon.cpp:47-127: VEC_VEC, VEC_SCALAR, VEC_BCAST101, VEC_BCAST101xX,
+// VEC_BCAST111C, VEC_BV, VEC_BCAST110, their mirrored forms and NAIVE are all one index rule
+// here). The host right-aligns the operand shapes against the output's, gives broadcast dims the
+// stride 0 and merges neighbouring dims that both operands walk densely (or both broadcast), so
+// the common cases arrive with 1-3 dims: [n], [rows, N] + [N], [outer, C, inner] * [C].
+// A work item is one output element, or 4 neighbours of the innermost dim (one 16-byte access per
+// dense operand, one scalar load per broadcast one).
+constexpr int EW_MAX_DIM = MAX_DIM;
+struct EwBcastArgs {
+    const float* a;
+    const float* b;
+    float* d;
+    size_t items;            // work items
+    int nd;                  // merged dims, dims[nd - 1] innermost
+    FastDiv div[EW_MAX_DIM]; // extents (innermost: in work items)
+    int sa[EW_MAX_DIM], sb[EW_MAX_DIM];  // element strides; innermost 0 or 1
+};
+
+template <int MODE, int ND, bool VEC>
+__global__ void __launch_bounds__(256) elemwise_f32_bcast_kernel(EwBcastArgs p) {
     constexpr bool binary = MODE >= MEGCC_EW_ADD;
+    constexpr int W = VEC ? 4 : 1;
     const size_t tid = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
     const size_t nthreads = (size_t)gridDim.x * blockDim.x;
-    size_t done = 0;
-    if (VEC) {
-        const size_t nvec = p.n / 4;
-        const float bs = (binary && p.bcast == BC_SCALAR) ? b[0] : 0.f;
-        for (size_t i = tid; i < nvec; i += nthreads) {
-            float4 x = ((const float4*)a)[i];
-            float4 y = make_float4(bs, bs, bs, bs);
-            if (binary && p.bcast == BC_NONE)
-                y = ((const float4*)b)[i];
+    for (size_t item = tid; item < p.items; item += nthreads) {
+        size_t oa, ob;
+        if (ND == 1) {
+            oa = item * W * p.sa[0];
+            ob = item * W * p.sb[0];
+        } else {
+            // (more than one dim: the host keeps the element count below 2^31)
+            uint32_t k = (uint32_t)item;
+            uint32_t q = fdiv(k, p.div[p.nd - 1]);
+            const uint32_t in = (k - q * p.div[p.nd - 1].d) * W;
+            oa = (size_t)in * p.sa[p.nd - 1];
+            ob = (size_t)in * p.sb[p.nd - 1];
+            k = q;
+#pragma unroll
+            for (int i = (ND < EW_MAX_DIM ? ND : EW_MAX_DIM) - 2; i >= 1; --i) {
+                if (ND < EW_MAX_DIM || i < p.nd - 1) {
+                    q = fdiv(k, p.div[i]);
+                    const uint32_t r = k - q * p.div[i].d;
+                    oa += (size_t)r * p.sa[i];
+                    ob += (size_t)r * p.sb[i];
+                    k = q;
+                }
+            }
+            oa += (size_t)k * p.sa[0];
+            ob += (size_t)k * p.sb[0];
+        }
+        const int li = ND == 1 ? 0 : p.nd - 1;
+        if (VEC) {
+            float4 x, y = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (p.sa[li]) {
+                x = *(const float4*)(p.a + oa);
+            } else {
+                const float v = p.a[oa];
+                x = make_float4(v, v, v, v);
+            }
+            if (binary) {
+                if (p.sb[li]) {
+                    y = *(const float4*)(p.b + ob);
+                } else {
+                    const float v = p.b[ob];
+                    y = make_float4(v, v, v, v);
+                }
+            }
             float4 r;
             r.x = ew_one<MODE>(x.x, y.x);
             r.y = ew_one<MODE>(x.y, y.y);
             r.z = ew_one<MODE>(x.z, y.z);
             r.w = ew_one<MODE>(x.w, y.w);
-            ((float4*)d)[i] = r;
+            ((float4*)p.d)[item] = r;
+        } else {
+            p.d[item] = ew_one<MODE>(p.a[oa], binary ? p.b[ob] : 0.f);
         }
-        done = nvec * 4;
-    }
-    for (size_t i = done + tid; i < p.n; i += nthreads) {
-        float y = 0.f;
-        if (binary)
-            y = p.bcast == BC_NONE ? b[i] : p.bcast == BC_SCALAR ? b[0] : b[(i / p.inner) % p.C];
-        d[i] = ew_one<MODE>(a[i], y);
     }
 }
 
@@ -319,6 +366,57 @@ extern "C" TinyNNStatus megcc_gfx950_elemwise_multitype(
     return check_launch("elemwise_multitype");
 }
 
+namespace {
+
+// Right-aligns `t` against the output dims `od[0..nd)`; fills element strides (0 where the operand
+// has extent 1 and the output more). False when the shapes do not broadcast.
+bool bcast_strides(const Tensor* t, const uint32_t* od, int nd, long* stride) {
+    const Layout& l = t->layout;
+    if (l.nr_dim > nd)
+        return false;
+    long dense = 1;
+    for (int i = nd - 1; i >= 0; --i) {
+        const int j = i - (nd - l.nr_dim);
+        const uint32_t ext = j >= 0 ? l.dims[j] : 1;
+        if (ext == od[i]) {
+            stride[i] = ext == 1 ? 0 : dense;
+        } else if (ext == 1) {
+            stride[i] = 0;
+        } else {
+            return false;
+        }
+        dense *= ext;
+    }
+    return true;
+}
+
+template <int MODE>
+void launch_elemwise_bcast(const EwBcastArgs& p, bool vec) {
+    const dim3 grid(grid_for(p.items)), block(256);
+#define MG_EW_ND(ND)                                                                              \
+    do {                                                                                          \
+        if (vec)                                                                                  \
+            hipLaunchKernelGGL((elemwise_f32_bcast_kernel<MODE, ND, true>), grid, block, 0,       \
+                               stream(), p);                                                      \
+        else                                                                                      \
+            hipLaunchKernelGGL((elemwise_f32_bcast_kernel<MODE, ND, false>), grid, block, 0,      \
+                               stream(), p);                                                      \
+    } while (0)
+    if (p.nd == 1)
+        MG_EW_ND(1);
+    else if (MODE < MEGCC_EW_ADD)
+        return;  // (a unary operator has one dense operand: always one dim)
+    else if (p.nd == 2)
+        MG_EW_ND(2);
+    else if (p.nd == 3)
+        MG_EW_ND(3);
+    else
+        MG_EW_ND(EW_MAX_DIM);
+#undef MG_EW_ND
+}
+
+}  // namespace
+
 extern "C" TinyNNStatus megcc_gfx950_elemwise(
         const MegccElemwiseMode* mode, Tensor** inputs, int nr_input, Tensor** outputs,
         int nr_output, const Workspace*, const RuntimeOpt*) {
@@ -334,29 +432,74 @@ extern "C" TinyNNStatus megcc_gfx950_elemwise(
     MG_REQUIRE(is_f32(a) && (!b || is_f32(b)) && is_f32(d), TinyNN_ERROR_UNSUPPORTED_DTYPE_TYPE,
                "elemwise: only f32 is implemented");
     MG_REQUIRE(is_contiguous(a->layout) && (!b || is_contiguous(b->layout)) &&
-                       is_contiguous(d->layout) && nr_elem(d->layout) == nr_elem(a->layout),
+                       is_contiguous(d->layout),
                TinyNN_ERROR_INVALID_LAYOUT, "elemwise: expects contiguous tensors");
-    EwArgs p;
-    p.a = a->ptr;
-    p.b = b ? b->ptr : nullptr;
-    p.d = d->ptr;
-    p.n = nr_elem(a->layout);
-    p.bcast = BC_NONE;
-    p.C = 1;
-    p.inner = 1;
-    p.s0 = p.s1 = p.sdiv = p.smul = 0.f;
-    if (b) {
-        st = classify_bcast(a, b, &p, "elemwise");
-        if (st != TinyNN_SUCCESS)
-            return st;
-    }
-    if (p.n == 0)
+    const int nd0 = d->layout.nr_dim;
+    MG_REQUIRE(nd0 >= 1 && nd0 <= MAX_DIM, TinyNN_ERROR_INVALID_LAYOUT, "elemwise: %d dims", nd0);
+    uint32_t od[MAX_DIM];
+    long sa[MAX_DIM], sb[MAX_DIM];
+    for (int i = 0; i < nd0; ++i)
+        od[i] = d->layout.dims[i];
+    const size_t n = nr_elem(d->layout);
+    MG_REQUIRE(bcast_strides(a, od, nd0, sa) && (!b || bcast_strides(b, od, nd0, sb)),
+               TinyNN_ERROR_INVALID_LAYOUT,
+               "elemwise: operand shapes do not broadcast to the output's");
+    // the output is the broadcast of the operands, not more
+    for (int i = 0; i < nd0; ++i)
+        MG_REQUIRE(od[i] == 1 || sa[i] != 0 || (b && sb[i] != 0), TinyNN_ERROR_INVALID_LAYOUT,
+                   "elemwise: output dim %d (%u) is larger than both operands'", i, od[i]);
+    if (n == 0)
         return TinyNN_SUCCESS;
-    const bool vec = p.bcast != BC_CHANNEL && aligned16(p.a) && aligned16(p.d) &&
-                     (p.bcast != BC_NONE || !b || aligned16(p.b));
-    const size_t work = vec ? p.n / 4 + 4 : p.n;
+    if (!b)
+        for (int i = 0; i < nd0; ++i)
+            sb[i] = sa[i];
+    // drop dims of extent 1, merge neighbours that both operands walk as one dense (or one
+    // broadcast) run
+    uint32_t md[MAX_DIM];
+    long ma[MAX_DIM], mb[MAX_DIM];
+    int nd = 0;
+    for (int i = 0; i < nd0; ++i) {
+        if (od[i] == 1)
+            continue;
+        if (nd > 0 && ma[nd - 1] == sa[i] * (long)od[i] && mb[nd - 1] == sb[i] * (long)od[i]) {
+            md[nd - 1] *= od[i];
+            ma[nd - 1] = sa[i];
+            mb[nd - 1] = sb[i];
+        } else {
+            md[nd] = od[i];
+            ma[nd] = sa[i];
+            mb[nd] = sb[i];
+            ++nd;
+        }
+    }
+    if (nd == 0) {
+        md[0] = 1;
+        ma[0] = mb[0] = 1;
+        nd = 1;
+    }
+    MG_REQUIRE(nd == 1 || n < (1u << 31), TinyNN_ERROR_OUT_OF_RANGE,
+               "elemwise: a broadcast over %zu elements is beyond the 32-bit index range", n);
+    EwBcastArgs p = {};
+    p.a = (const float*)a->ptr;
+    p.b = b ? (const float*)b->ptr : nullptr;
+    p.d = (float*)d->ptr;
+    p.nd = nd;
+    // 16-byte accesses: whole groups of 4 along the innermost dim, aligned bases; the outer
+    // strides of an operand that is dense along it are multiples of its extent
+    const bool vec = (md[nd - 1] & 3) == 0 && aligned16(p.d) && (ma[nd - 1] == 0 || aligned16(p.a)) &&
+                     (!b || mb[nd - 1] == 0 || aligned16(p.b));
+    bool outer_ok = true;
+    for (int i = 0; i < nd - 1; ++i)
+        outer_ok = outer_ok && (ma[nd - 1] == 0 || (ma[i] & 3) == 0) && (mb[nd - 1] == 0 || (mb[i] & 3) == 0);
+    const bool v4 = vec && outer_ok;
+    for (int i = 0; i < nd; ++i) {
+        p.div[i] = make_fastdiv(i == nd - 1 && v4 ? md[i] / 4 : md[i]);
+        p.sa[i] = (int)ma[i];
+        p.sb[i] = (int)mb[i];
+    }
+    p.items = v4 ? n / 4 : n;
     switch (*mode) {
-#define MG_CASE(M) case M: MG_LAUNCH_EW(elemwise_f32_kernel, M, vec, work, p); break;
+#define MG_CASE(M) case M: launch_elemwise_bcast<M>(p, v4); break;
         MG_CASE(MEGCC_EW_RELU)
         MG_CASE(MEGCC_EW_EXP)
         MG_CASE(MEGCC_EW_SIGMOID)
@@ -372,6 +515,7 @@ extern "C" TinyNNStatus megcc_gfx950_elemwise(
 #undef MG_CASE
         default: return fail(TinyNN_ERROR_NO_IMPLEMENT, "elemwise: mode %d", (int)*mode);
     }
+    note_kernel("elemwise_f32_bcast", nd, v4 ? 4 : 1);
     return check_launch("elemwise");
 }
 

@@ -8,7 +8,7 @@
 // BareMetal/ConvKernel.cpp:305-344,374-380 on the [M,K,1,1] x [N,K,1,1] layer).
 #include "conv_geom.h"
 #include "conv_mfma_i8.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
 
 namespace mg {
 

@@ -11,11 +11,14 @@
 // tiles are K-major with the row padded by 4 floats so both the staging writes and the MFMA
 // operand reads are bank-conflict free.
 // fp32 sums are formed in a different order from the reference's 4x12 micro-kernel; results are
-// held to 1e-4 relative, not bit-exactness.
+// held to 1e-4 relative, not bit-exactness. A float32 running sum over thousands of products
+// drifts from the exact value by more than that (K = 4096, values in [-1, 1]: 1.1e-4 on the worst
+// of 16 M outputs), so a workgroup whose K range is longer than 1024 (LONGK) closes its running
+// sums every 512 steps of K into a second set of registers: 3e-5 at K = 4096.
 #include "common.h"
 #include "gevm_f32.h"
 #include "conv_geom.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
 
 namespace mg {
 
@@ -68,8 +71,9 @@ __device__ __forceinline__ float conv_b(const GemmArgs& q, int k, int p) {
 
 // A_KFAST: A(m,k) has k contiguous (row-major, not transposed) -> lanes walk k when staging.
 // B_NFAST: B(k,n) has n contiguous -> lanes walk n.
-template <bool A_KFAST, bool B_NFAST, bool CONV, int BM>
+template <bool A_KFAST, bool B_NFAST, bool CONV, int BM, bool LONGK = false>
 __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
+    constexpr int KSEG = 512;  // LONGK: steps of K per running sum
     constexpr int BN = GBM * GBN / BM;  // 128 x 128 or 64 x 256
     constexpr int A_IT = BM / 16, B_IT = BN / 16;
     // LDS is double buffered: the global loads of step k+1 are in flight (in registers) while
@@ -80,14 +84,17 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
     const int wm = BM == 128 ? wave >> 1 : 0, wn = BM == 128 ? wave & 1 : wave;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
 
-    v16f acc[2][2];
+    v16f acc[2][2], tot[LONGK ? 2 : 1][LONGK ? 2 : 1];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int e = 0; e < 16; ++e)
+            for (int e = 0; e < 16; ++e) {
                 acc[i][j][e] = 0.f;
+                if (LONGK)
+                    tot[i][j][e] = 0.f;
+            }
 
     const int k_begin = blockIdx.z * q.kchunk;
     const int k_end = min(q.K, k_begin + q.kchunk);
@@ -201,9 +208,29 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
                 for (int j = 0; j < 2; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
         }
+        if (LONGK && ((k0 - k_begin) / GBK) % (KSEG / GBK) == KSEG / GBK - 1) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        tot[i][j][e] += acc[i][j][e];
+                        acc[i][j][e] = 0.f;
+                    }
+        }
         if (more)
             store_tiles(buf ^ 1);
         __syncthreads();
+    }
+    if (LONGK) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    acc[i][j][e] += tot[i][j][e];
     }
 
     // register e of a tile: row 8*(e/4) + 4*(lane/32) + e%4, column lane%32
@@ -339,12 +366,19 @@ TinyNNStatus conv_f32_gemm_launch(
     if (q.M == 0 || q.N == 0)
         return TinyNN_SUCCESS;
     gemm_plan_split(q, ws);
+    const bool longk = q.kchunk > 1024;
     if (q.M <= 64 && (long)((q.N + 255) / 256) * q.split >= 128) {
         dim3 grid((q.N + 255) / 256, 1, q.split);
-        hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 64>), grid, dim3(256), 0, stream(), q);
+        if (longk)
+            hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 64, true>), grid, dim3(256), 0, stream(), q);
+        else
+            hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 64>), grid, dim3(256), 0, stream(), q);
     } else {
         dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM, q.split);
-        hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 128>), grid, dim3(256), 0, stream(), q);
+        if (longk)
+            hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 128, true>), grid, dim3(256), 0, stream(), q);
+        else
+            hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 128>), grid, dim3(256), 0, stream(), q);
     }
     if (q.split > 1)
         gemm_launch_reduce(q);
@@ -399,20 +433,30 @@ extern "C" TinyNNStatus megcc_gfx950_matmul(
     q.is_conv = 0;
     if (q.M == 0 || q.N == 0)
         return TinyNN_SUCCESS;
-    if (q.M <= 4 && q.K > 0 && !getenv("MEGCC_NOGEVM")) {  // the reference's gevm case: one pass over B
+    if (q.M <= 4 && q.K > 0 && !options().no_gevm) {  // the reference's gevm case: one pass over B
         const GevmArgs v = {q.A, q.B, q.C, q.M, q.N, q.K, q.a_rs, q.a_cs, q.b_rs, q.b_cs, q.ldc};
-        if (gevm_f32_supported(v))
+        if (gevm_f32_supported(v)) {
+            note_kernel("gevm_f32");
             return gevm_f32_launch(v);
+        }
     }
     gemm_plan_split(q, ws);
     // 64 x 256 tiles when they still give every CU a workgroup
     const bool skinny = q.M <= 64 && (long)((q.N + 255) / 256) * q.split >= 128;
+    note_kernel("gemm_f32", skinny ? 64 : 128, q.split, q.kchunk > 1024);
     dim3 grid(skinny ? (q.N + 255) / 256 : (q.N + GBN - 1) / GBN, skinny ? 1 : (q.M + GBM - 1) / GBM,
               q.split);
+    const bool longk = q.kchunk > 1024;
 #define MG_GEMM_LAUNCH(AK, BN_)                                                                  \
     do {                                                                                         \
-        if (skinny)                                                                              \
+        if (skinny && longk)                                                                     \
+            hipLaunchKernelGGL((gemm_f32_kernel<AK, BN_, false, 64, true>), grid, dim3(256), 0,  \
+                               stream(), q);                                                     \
+        else if (skinny)                                                                         \
             hipLaunchKernelGGL((gemm_f32_kernel<AK, BN_, false, 64>), grid, dim3(256), 0,        \
+                               stream(), q);                                                     \
+        else if (longk)                                                                          \
+            hipLaunchKernelGGL((gemm_f32_kernel<AK, BN_, false, 128, true>), grid, dim3(256), 0, \
                                stream(), q);                                                     \
         else                                                                                     \
             hipLaunchKernelGGL((gemm_f32_kernel<AK, BN_, false, 128>), grid, dim3(256), 0,       \

@@ -493,7 +493,7 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
     // the first forward runs eagerly (it also warms per-kernel attributes), the second is captured
     if (m->graph_state == 0 && m->forwards >= 2) {
         m->graph_state = -1;
-        if (!getenv("MEGCC_NO_GRAPH") &&
+        if (!options().no_graph &&
             hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal) == hipSuccess) {
             TinyNNStatus st = forward_eager(m);
             hipGraph_t g = nullptr;

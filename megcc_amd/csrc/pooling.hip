@@ -8,7 +8,7 @@
 // NCHW44: one thread per output dword (4 channels of a pixel), lanes walk W -> coalesced dwords.
 // NCHW  : one thread per output byte, lanes walk W.
 #include "common.h"
-#include "epilogue.cuh"
+#include "epilogue.h"
 
 namespace mg {
 

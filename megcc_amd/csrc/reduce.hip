@@ -12,11 +12,22 @@ namespace mg {
 
 template <int MODE>
 __device__ __forceinline__ float red_init() {
-    return MODE == MEGCC_REDUCE_MAX ? -FLT_MAX : MODE == MEGCC_REDUCE_MIN ? FLT_MAX : 0.f;
+    return MODE == MEGCC_REDUCE_MAX       ? -FLT_MAX
+           : MODE == MEGCC_REDUCE_MIN     ? FLT_MAX
+           : MODE == MEGCC_REDUCE_PRODUCT ? 1.f
+                                          : 0.f;
+}
+// an element on its way into the reduction (SUM_SQR squares it once; partial sums then add)
+template <int MODE>
+__device__ __forceinline__ float red_in(float v) {
+    return MODE == MEGCC_REDUCE_SUM_SQR ? v * v : v;
 }
 template <int MODE>
 __device__ __forceinline__ float red_op(float a, float b) {
-    return MODE == MEGCC_REDUCE_MAX ? (a > b ? a : b) : MODE == MEGCC_REDUCE_MIN ? (a < b ? a : b) : a + b;
+    return MODE == MEGCC_REDUCE_MAX       ? (a > b ? a : b)
+           : MODE == MEGCC_REDUCE_MIN     ? (a < b ? a : b)
+           : MODE == MEGCC_REDUCE_PRODUCT ? a * b
+                                          : a + b;
 }
 
 template <int MODE>
@@ -26,7 +37,7 @@ __global__ void __launch_bounds__(256) reduce_rows_kernel(
     const float* row = src + (size_t)blockIdx.x * B;
     float acc = red_init<MODE>();
     for (int j = threadIdx.x; j < B; j += 256)
-        acc = red_op<MODE>(acc, row[j]);
+        acc = red_op<MODE>(acc, red_in<MODE>(row[j]));
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1)
         acc = red_op<MODE>(acc, __shfl_down(acc, off, 64));
@@ -49,7 +60,7 @@ __global__ void __launch_bounds__(256) reduce_strided_kernel(
     const float* p = src + a * B * C + k;
     float acc = red_init<MODE>();
     for (int j = 0; j < B; ++j)
-        acc = red_op<MODE>(acc, p[(size_t)j * C]);
+        acc = red_op<MODE>(acc, red_in<MODE>(p[(size_t)j * C]));
     dst[i] = MODE == MEGCC_REDUCE_MEAN ? acc / (float)B : acc;
 }
 
@@ -102,7 +113,10 @@ extern "C" TinyNNStatus megcc_gfx950_reduce(
         case MEGCC_REDUCE_MEAN: launch_reduce<MEGCC_REDUCE_MEAN>(sp, dp, (int)A, B, (int)C); break;
         case MEGCC_REDUCE_MAX: launch_reduce<MEGCC_REDUCE_MAX>(sp, dp, (int)A, B, (int)C); break;
         case MEGCC_REDUCE_MIN: launch_reduce<MEGCC_REDUCE_MIN>(sp, dp, (int)A, B, (int)C); break;
+        case MEGCC_REDUCE_PRODUCT: launch_reduce<MEGCC_REDUCE_PRODUCT>(sp, dp, (int)A, B, (int)C); break;
+        case MEGCC_REDUCE_SUM_SQR: launch_reduce<MEGCC_REDUCE_SUM_SQR>(sp, dp, (int)A, B, (int)C); break;
         default: return fail(TinyNN_ERROR_NO_IMPLEMENT, "reduce: mode %d", (int)attr->mode);
     }
+    note_kernel(C == 1 ? "reduce_rows" : "reduce_strided", attr->mode);
     return check_launch("reduce");
 }

@@ -30,7 +30,7 @@
 #include <vector>
 
 #include "common.h"
-#include "conv_mfma_i8.h"  // FastDiv
+#include "fastdiv.h"
 
 namespace mg {
 namespace {

@@ -1,4 +1,4 @@
-// Host-side cache of requantisation threshold tables (see epilogue.cuh): one table per
+// Host-side cache of requantisation threshold tables (see epilogue.h): one table per
 // (activation, src scale, filter scale, dst scale), built on first use with the reference's
 // literal float sequence evaluated by the host CPU - the same IEEE single-precision multiply,
 // multiply, divide, roundf the generated C kernels execute - and kept for the life of the process.
@@ -8,7 +8,7 @@
 #include <mutex>
 #include <tuple>
 
-#include "epilogue.cuh"
+#include "epilogue.h"
 
 namespace mg {
 

@@ -439,7 +439,8 @@ struct ReduceKernel : KernelFuncBase {
         const std::string mode = c->getAttrStr("mode");
         return c->getAttrStr("data_type") == "DEFAULT" &&
                is_f32(c->getAttrOprand("operand:0").dtype) &&
-               (mode == "SUM" || mode == "MEAN" || mode == "MAX" || mode == "MIN");
+               (mode == "SUM" || mode == "MEAN" || mode == "MAX" || mode == "MIN" ||
+                mode == "PRODUCT" || mode == "SUM_SQR");
     }
     std::string GetKernelSymbol(TContext* c) const override {
         std::stringstream ss;

@@ -55,6 +55,9 @@ def lib():
         L.megcc_gfx950_stream.restype = C.c_void_p
         L.megcc_gfx950_last_error.argtypes = []
         L.megcc_gfx950_last_error.restype = C.c_char_p
+        L.megcc_gfx950_last_kernel.argtypes = []
+        L.megcc_gfx950_last_kernel.restype = C.c_char_p
+        L.megcc_gfx950_set_option.argtypes = [C.c_char_p, C.c_int]
         L.megcc_gfx950_model_create.argtypes = []
         L.megcc_gfx950_model_create.restype = C.c_void_p
         L.megcc_gfx950_model_destroy.argtypes = [C.c_void_p]
@@ -99,7 +102,8 @@ EXPORTS = [
     "megcc_gfx950_call_init", "megcc_gfx950_call_workspace", "megcc_gfx950_init_device",
     "megcc_gfx950_malloc", "megcc_gfx950_free", "megcc_gfx950_memcpy_h2d",
     "megcc_gfx950_memcpy_d2h", "megcc_gfx950_memset", "megcc_gfx950_wait",
-    "megcc_gfx950_stream", "megcc_gfx950_last_error",
+    "megcc_gfx950_stream", "megcc_gfx950_last_error", "megcc_gfx950_last_kernel",
+    "megcc_gfx950_set_option",
     "megcc_gfx950_model_create", "megcc_gfx950_model_destroy", "megcc_gfx950_model_add_tensor",
     "megcc_gfx950_model_add_weight", "megcc_gfx950_model_add_alias", "megcc_gfx950_model_add_view",
     "megcc_gfx950_model_add_opr", "megcc_gfx950_model_add_opr_desc",
@@ -187,6 +191,16 @@ class DeviceBuffer:
 
 def wait():
     check(lib().megcc_gfx950_wait(), "wait")
+
+
+def last_kernel():
+    """which kernel variant this thread's most recent operator call selected"""
+    return lib().megcc_gfx950_last_kernel().decode()
+
+
+def set_option(name, value):
+    """kernel-selection override (megcc_gfx950_set_option)"""
+    check(lib().megcc_gfx950_set_option(name.encode(), int(value)), "set_option " + name)
 
 
 def parse_symbol(symbol):

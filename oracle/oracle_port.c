@@ -387,19 +387,27 @@ void orc_elemwise_f32(
     }
 }
 
-enum { RED_SUM = 0, RED_MEAN = 1, RED_MAX = 2, RED_MIN = 3 };
+enum { RED_SUM = 0, RED_MEAN = 1, RED_MAX = 2, RED_MIN = 3, RED_PRODUCT = 4, RED_SUM_SQR = 5 };
 
-/* BareMetal/Reduce.cpp:98-131: view as [A,B,C], reduce over B in ascending j. */
+/* BareMetal/Reduce.cpp:11-72,98-131: view as [A,B,C], reduce over B in ascending j; start value
+ * lowest / highest float for MAX / MIN, 1 for PRODUCT, else 0; MEAN divides the sum by B. */
 void orc_reduce_f32(const float* src, float* dst, int mode, int A, int B, int C) {
     for (int i = 0; i < A; ++i)
         for (int k = 0; k < C; ++k) {
-            float acc = mode == RED_MAX ? -__FLT_MAX__ : mode == RED_MIN ? __FLT_MAX__ : 0.f;
+            float acc = mode == RED_MAX       ? -__FLT_MAX__
+                        : mode == RED_MIN     ? __FLT_MAX__
+                        : mode == RED_PRODUCT ? 1.f
+                                              : 0.f;
             for (int j = 0; j < B; ++j) {
                 float v = src[((size_t)i * B + j) * C + k];
                 if (mode == RED_MAX)
                     acc = acc > v ? acc : v;
                 else if (mode == RED_MIN)
                     acc = acc < v ? acc : v;
+                else if (mode == RED_PRODUCT)
+                    acc = acc * v;
+                else if (mode == RED_SUM_SQR)
+                    acc = acc + (v * v);
                 else
                     acc = acc + v;
             }

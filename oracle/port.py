@@ -124,10 +124,16 @@ def multitype_q8(a, b, mode, s0, s1, sd):
 
 
 def elemwise_f32(a, b, mode):
-    dst = np.empty(a.shape, np.float32)
-    bc, c, inner = _bcast(a, b)
-    lib().orc_elemwise_f32(_p(a), _p(b), _p(dst), mode, C.c_size_t(a.size), bc, c,
-                           C.c_size_t(inner))
+    """f32 Elemwise over the broadcast of a and b (right-aligned shapes, extent 1 stretches:
+    numpy's own rule materialises the operands, the per-element expressions are the C port's)."""
+    if b is None:
+        shape = a.shape
+    else:
+        shape = np.broadcast_shapes(a.shape, b.shape)
+        a = np.ascontiguousarray(np.broadcast_to(a, shape))
+        b = np.ascontiguousarray(np.broadcast_to(b, shape))
+    dst = np.empty(shape, np.float32)
+    lib().orc_elemwise_f32(_p(a), _p(b), _p(dst), mode, C.c_size_t(dst.size), 0, 1, C.c_size_t(1))
     return dst
 
 

@@ -364,6 +364,133 @@ class MatMulCase:
         return port.matmul_f32(arrays["a"], arrays["b"], self.trans_a, self.trans_b)
 
 
+def _nelem(shape):
+    return int(np.prod(shape, dtype=np.int64))
+
+
+def binary_bcast_type(s0, s1):
+    """GetBinaryBcastType, Common/ElemwiseCommon.cpp:47-127: the name the reference gives the way
+    two operand shapes meet (part of the GI kernel's symbol)."""
+    s0, s1 = tuple(s0), tuple(s1)
+    n0, n1 = _nelem(s0), _nelem(s1)
+    if n0 == n1:
+        return "VEC_VEC"
+    if n0 == 1:
+        return "SCALAR_VEC"
+    if n1 == 1:
+        return "VEC_SCALAR"
+    if (n0 == s0[-1] or n1 == s1[-1]) and s0[-1] == s1[-1]:
+        return "BCAST111C_VEC" if n0 == s0[-1] else "VEC_BCAST111C"
+    assert len(s0) == len(s1)
+    small, big = (s0, s1) if n0 < n1 else (s1, s0)
+    names = (lambda a, b: a + "_VEC" if n0 < n1 else "VEC_" + a)
+    if all(sm == 1 for sm, bg in zip(small, big) if bg == 1):
+        if len(small) == 4 and small[0] == small[2] == small[3] == 1:
+            return names("BCAST101", None)
+        if len(small) == 5 and small[0] == small[2] == small[3] == 1 and small[4] in (4, 8):
+            return names("BCAST101xX", None)
+        # CalBroadcastElemwise: runs of broadcast / elementwise dims
+        runs, bc = [1], True
+        for sm, bg in zip(small, big):
+            if not bc and sm != bg:
+                bc = True
+                runs.append(1)
+            elif bc and sm != 1:
+                bc = False
+                runs.append(1)
+            runs[-1] *= bg
+        if len(runs) == 2:
+            return names("BV", None)
+        if small[:-1] == big[:-1] and small[-1] == 1 and big[-1] > 1:
+            return names("BCAST110", None)
+    return "NAIVE"
+
+
+class ElemwiseCase:
+    """f32 Elemwise: unary (one shape) or binary over the broadcast of two shapes (right-aligned,
+    extent 1 stretches: megdnn's rule, which is numpy's). `span` = range of the drawn values."""
+
+    GI_MODES = {"RELU", "EXP", "SIGMOID", "H_SWISH", "ADD", "SUB", "MUL", "TRUE_DIV",
+                "FUSE_ADD_RELU", "MAX", "MIN"}
+
+    def __init__(self, mode, shapes, span=(-4.0, 4.0)):
+        self.mode, self.shapes, self.span = mode, [tuple(s) for s in shapes], span
+        assert len(self.shapes) == (2 if abi.EW_MODES[mode] >= abi.EW_ADD else 1)
+        self.out_shape = tuple(np.broadcast_shapes(*self.shapes))
+
+    def __repr__(self):
+        return "elemwise_%s[%s]" % (self.mode, " ".join("x".join(map(str, s)) for s in self.shapes))
+
+    def symbol(self):
+        """GeneralIntrinsic/Elemwise/Elemwise.cpp:38-63 for the modes GI knows (:17-20), else
+        BareMetal/ElemwiseKernel.cpp:433-439"""
+        io = "f32" * (len(self.shapes) + 1)
+        if self.mode not in self.GI_MODES:
+            return "kernel_elementwise_%s_%s" % (self.mode, io)
+        kind = "unary_vec_vec" if len(self.shapes) == 1 else \
+            "binary_" + binary_bcast_type(*self.shapes)
+        return "GI_kernel_elementwise_%s_f32_%s_%s" % (self.mode, kind, io)
+
+    def spec_line(self):
+        ops = [_op(s, "f32") for s in self.shapes] + [_op(self.out_shape, "f32")]
+        return " ".join(["ElemwiseKernel", "mode=s:" + self.mode, "nr_operands=i:%d" % len(ops)] +
+                        ["operand:%d=%s" % (i, o) for i, o in enumerate(ops)])
+
+    def gen(self, seed=0):
+        r = rng(seed)
+        out = {"a": r.uniform(self.span[0], self.span[1], self.shapes[0]).astype(np.float32)}
+        out["b"] = (r.uniform(self.span[0], self.span[1], self.shapes[1]).astype(np.float32)
+                    if len(self.shapes) == 2 else None)
+        return out
+
+    def specs(self, arrays):
+        ins = [TensorSpec(b"a", self.shapes[0], abi.FLOAT, 1.0, arrays["a"])]
+        if len(self.shapes) == 2:
+            ins.append(TensorSpec(b"b", self.shapes[1], abi.FLOAT, 1.0, arrays["b"]))
+        return ins, [TensorSpec(b"dst", self.out_shape, abi.FLOAT, 1.0)]
+
+    def run_port(self, arrays):
+        return port.elemwise_f32(arrays["a"], arrays["b"], abi.EW_MODES[self.mode])
+
+    def min_bytes(self):
+        return 4 * (sum(_nelem(s) for s in self.shapes) + _nelem(self.out_shape))
+
+
+class ReduceCase:
+    """f32 Reduce over one axis (kept with extent 1 in the output, as megdnn deduces it)"""
+
+    def __init__(self, mode, shape, axis):
+        self.mode, self.shape, self.axis = mode, tuple(shape), axis
+        self.out_shape = tuple(1 if i == axis else d for i, d in enumerate(self.shape))
+
+    def __repr__(self):
+        return "reduce_%s_a%d[%s]" % (self.mode, self.axis, "x".join(map(str, self.shape)))
+
+    def symbol(self):
+        """GeneralIntrinsic/Reduce.cpp:615-623 (f32 always resolves to the GI kernel)"""
+        return "GI_kernel_reduce_%s_DEFAULT_f32_a%d" % (self.mode, self.axis)
+
+    def spec_line(self):
+        return " ".join(["ReduceKernel", "mode=s:" + self.mode, "axis=i:%d" % self.axis,
+                         "data_type=s:DEFAULT", "nr_operands=i:2",
+                         "operand:0=" + _op(self.shape, "f32"),
+                         "operand:1=" + _op(self.out_shape, "f32")])
+
+    def attr(self):
+        return abi.ReduceAttr(abi.REDUCE_MODES[self.mode], self.axis)
+
+    def gen(self, seed=0):
+        lo, hi = (0.6, 1.5) if self.mode == "PRODUCT" else (-3.0, 3.0)
+        return {"src": rng(seed).uniform(lo, hi, self.shape).astype(np.float32)}
+
+    def specs(self, arrays):
+        return ([TensorSpec(b"src", self.shape, abi.FLOAT, 1.0, arrays["src"])],
+                [TensorSpec(b"dst", self.out_shape, abi.FLOAT, 1.0)])
+
+    def run_port(self, arrays):
+        return port.reduce_f32(arrays["src"], abi.REDUCE_MODES[self.mode], self.axis)
+
+
 POISON = 0x5A  # byte every output buffer holds before a kernel runs
 
 

@@ -4,8 +4,8 @@ tests/golden/make_golden.py). Shapes follow the reference's own kernel tests
 typecvt.cpp:5-70): odd sizes, k in {1,3}, stride in {1,2}, pad in {0,k/2}, every activation, the
 small-magnitude tie case and the 30..50 overflow case."""
 from megcc_amd import abi
-from cases import (ConcatCase, ConvCase, FusedCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
-                   ResizeCase, TypeCvtCase)
+from cases import (ConcatCase, ConvCase, ElemwiseCase, FusedCase, MatMulCase, MultiTypeCase, PoolCase,
+                   ReduceCase, RelayoutCase, ResizeCase, TypeCvtCase)
 
 A = abi
 
@@ -171,4 +171,33 @@ def golden_cases():
                                              [(2, 3, 4, 5), (2, 3, 4, 5)], positive=(1,))
     c["resize_nearest_nchw_view"] = ResizeCase(A.FMT_NCHW, "NEAREST", 2, 3, 6, 5, 9, 11,
                                                src_strides=(400, 120, 20, 2))
+    # --- f32 elementwise: the shapes of compiler/test/kernel/opr/generalIntrinsic/elementwise.cpp
+    # :7-80 (every way two operands meet: same shape, scalar either side, [1,C,1,1] either side,
+    # a trailing vector either side, a leading run, a kept last axis of extent 1; {2,100,3,96}
+    # cut to {2,10,3,96}), then the NCHW44 channel vector, a general broadcast and the
+    # FullyConnected bias [M,N] + [1,N]
+    for mode in ("RELU", "SIGMOID", "EXP", "H_SWISH", "NEGATE"):
+        c["ew_%s_4d" % mode] = ElemwiseCase(mode, [(1, 10, 12, 13)])
+    c["ew_RELU_1"] = ElemwiseCase("RELU", [(1,)])
+    pairs = [((1,), (1,)), ((1, 10), (1, 10)), ((1, 10), (1, 1)), ((2, 3, 4, 5), (2, 3, 4, 5)),
+             ((2, 3, 4, 5), (1, 3, 1, 1)), ((1, 3, 1, 1), (2, 3, 4, 5)), ((13,), (3, 9, 13)),
+             ((3, 9, 13), (13,)), ((1, 1, 1, 13), (2, 3, 4, 13)), ((2, 10, 3, 96), (1, 1, 1, 96)),
+             ((3, 6, 9, 5), (3, 6, 9, 1)), ((5, 32, 1), (5, 32, 13)),
+             ((2, 3, 4, 5, 4), (1, 3, 1, 1, 4)), ((1, 3, 1, 1, 4), (2, 3, 4, 5, 4)),
+             ((2, 3, 4, 5), (1, 1, 4, 5)), ((2, 3, 4, 5), (2, 1, 4, 1)), ((5, 40), (1, 40))]
+    for i, (s0, s1) in enumerate(pairs):
+        c["ew_ADD_%d" % i] = ElemwiseCase("ADD", [s0, s1])
+    others = ["SUB", "MUL", "FUSE_ADD_RELU", "MAX", "MIN"]
+    for i, (s0, s1) in enumerate(pairs):  # every pairing under two more modes
+        for j in (0, 1):
+            mode = others[(2 * i + j) % len(others)]
+            c["ew_%s_%d" % (mode, i)] = ElemwiseCase(mode, [s0, s1])
+    for i, (s0, s1) in enumerate(pairs + [((2, 3, 4), (1,)), ((1,), (2, 3, 4))]):
+        c["ew_TRUE_DIV_%d" % i] = ElemwiseCase("TRUE_DIV", [s0, s1], span=(3.0, 12.0))
+    # --- f32 reduce: compiler/test/kernel/opr/generalIntrinsic/reduce.cpp:7-27 (every mode, every
+    # axis of a 2-, 3- and 4-d tensor)
+    for mode in ("SUM", "MEAN", "MAX", "MIN", "PRODUCT", "SUM_SQR"):
+        for shape in ((2, 3), (3, 4, 5), (4, 5, 6, 7)):
+            for axis in range(len(shape)):
+                c["reduce_%s_%dd_a%d" % (mode, len(shape), axis)] = ReduceCase(mode, shape, axis)
     return c

@@ -10,8 +10,8 @@ import numpy as np
 import pytest
 
 import cases
-from cases import (ConcatCase, ConvCase, FusedCase, MatMulCase, MultiTypeCase, PoolCase, RelayoutCase,
-                   ResizeCase, TypeCvtCase)
+from cases import (ConcatCase, ConvCase, ElemwiseCase, FusedCase, MatMulCase, MultiTypeCase, PoolCase,
+                   ReduceCase, RelayoutCase, ResizeCase, TypeCvtCase)
 from golden_cases import golden_cases, unsat
 from megcc_amd import abi, runtime
 from oracle import port
@@ -207,6 +207,54 @@ def test_matches_oracle(case):
     compare(got, want, repr(case))
 
 
+F32_POINTWISE = [
+    # f32 elementwise: the FullyConnected bias [M,N] + [N] / [1,N] at the sizes of the MatMul
+    # configurations, the softmax steps ([A,N] op [A,1]), every other way two operands meet
+    # (scalar and [1,C,1,1] either side, NCHW44 channel vector, leading run, general broadcast),
+    # ragged sizes that take the one-element-per-thread path, every mode
+    ElemwiseCase("ADD", [(64, 4096), (4096,)]),
+    ElemwiseCase("ADD", [(64, 4096), (1, 4096)]),
+    ElemwiseCase("ADD", [(1, 1000), (1000,)]),
+    ElemwiseCase("ADD", [(4096, 4096), (1, 4096)]),
+    ElemwiseCase("ADD", [(1, 4096), (4096, 4096)]),
+    ElemwiseCase("SUB", [(64, 1000), (64, 1)]),
+    ElemwiseCase("TRUE_DIV", [(64, 1000), (64, 1)], span=(1.0, 9.0)),
+    ElemwiseCase("TRUE_DIV", [(1,), (5, 1001)], span=(1.0, 9.0)),
+    ElemwiseCase("MUL", [(4, 32, 14, 14), (1, 32, 1, 1)]),
+    ElemwiseCase("MUL", [(1, 32, 1, 1), (4, 32, 14, 14)]),
+    ElemwiseCase("MUL", [(4, 32, 7, 9), (1, 32, 1, 1)]),
+    ElemwiseCase("MAX", [(4, 8, 14, 14, 4), (1, 8, 1, 1, 4)]),
+    ElemwiseCase("MIN", [(3, 1, 5, 1), (3, 4, 5, 6)]),
+    ElemwiseCase("MIN", [(3, 4, 5, 8), (3, 1, 5, 1)]),
+    ElemwiseCase("FUSE_ADD_RELU", [(2, 3, 4, 5), (1, 1, 4, 5)]),
+    ElemwiseCase("FUSE_ADD_RELU", [(64, 1000), (64, 1000)]),
+    ElemwiseCase("SUB", [(100003,), (1,)]),
+    ElemwiseCase("ADD", [(7, 1, 9, 1, 5, 1, 4), (1, 6, 1, 3, 1, 2, 4)]),
+    ElemwiseCase("RELU", [(64, 1000)]),
+    ElemwiseCase("NEGATE", [(5, 1001)]),
+    ElemwiseCase("EXP", [(64, 1000)], span=(-20.0, 0.0)),
+    ElemwiseCase("SIGMOID", [(5, 1001)]),
+    ElemwiseCase("H_SWISH", [(3, 16, 28, 28)], span=(-6.0, 6.0)),
+    # f32 reduce: the softmax steps, a global average written as MEAN, every mode, every position
+    # of the axis (first: C > 1 with A = 1; middle; last: C = 1)
+    ReduceCase("MAX", (64, 1000), 1),
+    ReduceCase("SUM", (64, 1000), 1),
+    ReduceCase("MEAN", (8, 1024, 49), 2),
+    ReduceCase("MEAN", (6, 50, 33), 1),
+    ReduceCase("MIN", (50, 7, 9), 0),
+    ReduceCase("SUM", (3000, 5), 0),
+    ReduceCase("SUM_SQR", (4, 5, 6, 7), 2),
+    ReduceCase("PRODUCT", (3, 40, 5), 1),
+    ReduceCase("MAX", (1, 100003), 1),
+]
+
+
+@pytest.mark.parametrize("case", F32_POINTWISE, ids=[repr(c) for c in F32_POINTWISE])
+def test_f32_elemwise_and_reduce(case):
+    arrays = case.gen(seed=67)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+
+
 def _random_views():
     """seeded random strided views: permuted dims, steps of 2, reversed dims, both sides or one"""
     r = np.random.Generator(np.random.PCG64(77))
@@ -399,35 +447,46 @@ def test_fused_elemwise(case):
 
 
 OLDER = [
-    # shapes the newer kernels take, forced back (development switches of the library) onto the
+    # shapes the newer kernels take, forced back (megcc_gfx950_set_option) onto the
     # kernels that still serve other shapes: one-stage kernel with split-K (slices of 2 stages out
     # of 8: a sixth slice would start past the packed filter), dword activation loads, the
     # 256-pixel variant, the tiled FullyConnected
-    ("MEGCC_NOSMALL", ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 56, 56, 256, 3, 1, 1, A.RELU,
+    ("nosmall", ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 56, 56, 256, 3, 1, 1, A.RELU,
                                scales=(0.02, 0.01, unsat(2304)))),
-    ("MEGCC_NOSMALL", ConvCase(A.FMT_NCHW44, A.DENSE, 3, 256, 14, 14, 256, 3, 1, 1, A.IDENTITY,
+    ("nosmall", ConvCase(A.FMT_NCHW44, A.DENSE, 3, 256, 14, 14, 256, 3, 1, 1, A.IDENTITY,
                                scales=(0.02, 0.01, 0.05))),
-    ("MEGCC_NOPM", ConvCase(A.FMT_NCHW44, A.DENSE, 6, 32, 56, 56, 160, 3, 1, 1, A.RELU,
+    ("nopm", ConvCase(A.FMT_NCHW44, A.DENSE, 6, 32, 56, 56, 160, 3, 1, 1, A.RELU,
                             scales=(0.02, 0.01, unsat(288)))),
-    ("MEGCC_NODMA512", ConvCase(A.FMT_NCHW44, A.DENSE, 6, 64, 56, 56, 128, 3, 1, 1, A.RELU,
+    ("nodma512", ConvCase(A.FMT_NCHW44, A.DENSE, 22, 64, 54, 57, 128, 3, 1, 1, A.RELU,
                                 scales=(0.02, 0.01, unsat(576)))),
-    ("MEGCC_NOGEVM", ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY,
+    ("nogevm", ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY,
                               scales=(0.01, 0.01, unsat(1024) / 2))),
-    ("MEGCC_NOGEVM", MatMulCase(3, 301, 79, trans_b=True)),
-    ("MEGCC_NOF32SMALL", ConvCase(A.FMT_NCHW, A.DENSE, 1, 32, 56, 56, 32, 3, 1, 1, A.RELU, dtype="f32")),
-    ("MEGCC_NOPWSHARE", ConvCase(A.FMT_NCHW44, A.DENSE, 70, 512, 14, 14, 512, 1, 1, 0, A.RELU,
+    ("nogevm", MatMulCase(3, 301, 79, trans_b=True)),
+    ("nof32small", ConvCase(A.FMT_NCHW, A.DENSE, 1, 32, 56, 56, 32, 3, 1, 1, A.RELU, dtype="f32")),
+    ("nopwshare", ConvCase(A.FMT_NCHW44, A.DENSE, 70, 512, 14, 14, 512, 1, 1, 0, A.RELU,
                                  scales=(0.02, 0.01, unsat(512)))),
-    ("MEGCC_NOPWS", ConvCase(A.FMT_NCHW44, A.DENSE, 11, 64, 56, 56, 128, 1, 1, 0, A.IDENTITY,
+    ("nopws", ConvCase(A.FMT_NCHW44, A.DENSE, 11, 64, 56, 56, 128, 1, 1, 0, A.IDENTITY,
                              scales=(0.02, 0.01, unsat(64)))),
 ]
 
 
 @pytest.mark.parametrize("switch,case", OLDER, ids=["%s-%r" % (s, c) for s, c in OLDER])
-def test_older_kernels_still_agree(switch, case, monkeypatch):
-    monkeypatch.setenv(switch, "1")
+def test_older_kernels_still_agree(switch, case):
     port.set_threads(8)
     arrays = case.gen(seed=29)
-    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+    want = case.run_port(arrays)
+    normally = None
+    try:
+        runtime.set_option(switch, 1)
+        got = run_gpu(case, arrays)
+        forced = runtime.last_kernel()
+    finally:
+        runtime.set_option(switch, 0)
+    compare(got, want, repr(case))
+    # the switch must have changed which kernel ran
+    run_gpu(case, arrays)
+    normally = runtime.last_kernel()
+    assert forced != normally, "%s did not change the kernel (%s)" % (switch, forced)
 
 
 def _plane_major_sweep():

@@ -41,7 +41,9 @@ def test_every_layer_is_bit_exact_batch2():
     assert cases.max_rel_err(got, want) <= 1e-4
     assert np.allclose(got.sum(axis=1), 1.0, atol=1e-4)
     # the test images must not collapse to a constant prediction
-    assert len(set(np.argmax(want, axis=1).tolist())) >= 1 and want.max() < 0.999
+    # (with random weights the bias picks the arg-max class; the logits of the two images differ)
+    fc = trace["fc"].reshape(2, 1000)
+    assert np.mean(fc[0] != fc[1]) > 0.5 and len(np.unique(fc)) > 50 and want.max() < 0.999
     model.close()
 
 
@@ -72,7 +74,7 @@ def test_memory_plan_reuses_the_arena_and_keeps_results():
 
 
 @pytest.mark.gpu
-def test_graph_replays_equal_eager_forwards(monkeypatch):
+def test_graph_replays_equal_eager_forwards():
     """The model runtime captures its operator sequence into a HIP graph on the second forward.
     Every replay, with new inputs, host copies and synchronisations in between, must give what an
     eager forward gives (bit for bit: same kernels, same order)."""
@@ -82,11 +84,13 @@ def test_graph_replays_equal_eager_forwards(monkeypatch):
     names = ["conv0", "pw1", "pw13", "fc", "softmax"]
     for it in range(5):
         image = mobilenet.draw_input(2, seed=20 + it)
-        monkeypatch.setenv("MEGCC_NO_GRAPH", "1")
-        eager.set_input(ids["image"], image)
-        eager.forward()
+        runtime.set_option("no_graph", 1)
+        try:
+            eager.set_input(ids["image"], image)
+            eager.forward()
+        finally:
+            runtime.set_option("no_graph", 0)
         want = {k: eager.get(ids[k]).copy() for k in names}
-        monkeypatch.delenv("MEGCC_NO_GRAPH")
         graph.set_input(ids["image"], image)
         graph.forward()  # it == 0: eager, it == 1: capture + first launch, then replays
         for k in names:

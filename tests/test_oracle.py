@@ -283,3 +283,96 @@ def test_port_fused_elemwise_vs_numpy():
     with np.errstate(divide="ignore", invalid="ignore"):
         want = np.floor((t0 < y).astype(np.float32) / t0)
     assert np.array_equal(got, want, equal_nan=True)
+
+
+# ---- f32 elementwise and reduce: what numpy fixes without the reference --------------------------
+EW_PAIRS = [((7, 40), (40,)), ((7, 40), (1, 40)), ((2, 3, 4, 5), (1, 3, 1, 1)), ((1, 3, 1, 1), (2, 3, 4, 5)),
+            ((2, 3, 4, 5), (2, 1, 4, 1)), ((5, 32, 1), (5, 32, 13)), ((6,), (1,)), ((1,), (2, 3, 4)),
+            ((2, 3, 4, 5, 4), (1, 3, 1, 1, 4)), ((9, 11), (9, 11))]
+
+
+@pytest.mark.parametrize("shapes", EW_PAIRS, ids=lambda s: "%sx%s" % s)
+def test_port_elemwise_binary_vs_numpy(shapes):
+    """single IEEE operations under numpy's own broadcasting: results must be identical, bit for
+    bit (a wrong operand order, a transposed broadcast or a dropped operand all show)"""
+    from cases import ElemwiseCase
+    r = np.random.default_rng(11)
+    a = r.uniform(-4, 4, shapes[0]).astype(np.float32)
+    b = r.uniform(0.5, 4, shapes[1]).astype(np.float32)
+    f32 = np.float32
+    want = {"ADD": a + b, "SUB": a - b, "MUL": a * b, "TRUE_DIV": a / b, "MAX": np.maximum(a, b),
+            "MIN": np.minimum(a, b), "FUSE_ADD_RELU": np.maximum(a + b, f32(0))}
+    for mode, w in want.items():
+        got = ElemwiseCase(mode, list(shapes)).run_port({"a": a, "b": b})
+        assert got.dtype == np.float32 and np.array_equal(got, w), mode
+    # not commutative: the operands must not be swapped
+    assert not np.array_equal(ElemwiseCase("SUB", list(shapes)).run_port({"a": a, "b": b}), b - a)
+
+
+def test_port_elemwise_unary_vs_numpy():
+    from cases import ElemwiseCase
+    x = np.random.default_rng(12).uniform(-8, 8, (3, 5, 7)).astype(np.float32)
+    x[0, 0, :4] = [0.0, -3.0, 3.0, -0.0]
+    run = lambda m: ElemwiseCase(m, [x.shape]).run_port({"a": x, "b": None})
+    assert np.array_equal(run("RELU"), np.maximum(x, np.float32(0)))
+    assert np.array_equal(run("NEGATE"), -x)
+    x64 = x.astype(np.float64)
+    np.testing.assert_allclose(run("EXP"), np.exp(x64), rtol=3e-7)
+    np.testing.assert_allclose(run("SIGMOID"), 1 / (1 + np.exp(-x64)), rtol=5e-7)
+    np.testing.assert_allclose(run("H_SWISH"), x64 * np.clip(x64 + 3, 0, 6) / 6, rtol=5e-7, atol=1e-7)
+    # H_SWISH is zero at and below -3 and the identity at and above 3
+    hs = run("H_SWISH")
+    assert hs[0, 0, 1] == 0 and hs[0, 0, 2] == 3.0
+
+
+@pytest.mark.parametrize("shape,axis", [((2, 3), 0), ((2, 3), 1), ((3, 4, 5), 0), ((3, 4, 5), 1),
+                                        ((3, 4, 5), 2), ((4, 5, 6, 7), 2), ((64, 1000), 1)])
+def test_port_reduce_vs_numpy(shape, axis):
+    """MAX / MIN are exact; the sums are the float32 running sum in ascending order along the
+    axis (numpy's accumulate does exactly that), MEAN divides it once by the extent; fp64 numpy
+    bounds all of them"""
+    from cases import ReduceCase
+    x = np.random.default_rng(13).uniform(-3, 3, shape).astype(np.float32)
+    run = lambda m: ReduceCase(m, shape, axis).run_port({"src": x})
+    keep = lambda v: np.expand_dims(v, axis)
+    assert np.array_equal(run("MAX"), keep(x.max(axis)))
+    assert np.array_equal(run("MIN"), keep(x.min(axis)))
+    last = lambda acc: keep(np.take(acc, -1, axis=axis))
+    seq = last(np.add.accumulate(x, axis=axis, dtype=np.float32))
+    assert np.array_equal(run("SUM"), seq)
+    assert np.array_equal(run("MEAN"), seq / np.float32(shape[axis]))
+    assert np.array_equal(run("SUM_SQR"), last(np.add.accumulate(x * x, axis=axis, dtype=np.float32)))
+    assert np.array_equal(run("PRODUCT"), last(np.multiply.accumulate(x, axis=axis, dtype=np.float32)))
+    np.testing.assert_allclose(run("SUM"), keep(x.astype(np.float64).sum(axis)), rtol=1e-4, atol=1e-4)
+    assert run("SUM").shape == tuple(1 if i == axis else d for i, d in enumerate(shape))
+
+
+LIVE_F32 = None
+
+
+def _live_f32():
+    from cases import ElemwiseCase, ReduceCase
+    return [ElemwiseCase("ADD", [(64, 4096), (1, 4096)]), ElemwiseCase("ADD", [(33, 1000), (1000,)]),
+            ElemwiseCase("SUB", [(64, 1000), (64, 1)]), ElemwiseCase("TRUE_DIV", [(64, 1000), (64, 1)], span=(1.0, 9.0)),
+            ElemwiseCase("MUL", [(4, 32, 14, 14), (1, 32, 1, 1)]), ElemwiseCase("EXP", [(64, 1000)], span=(-20.0, 0.0)),
+            ElemwiseCase("SIGMOID", [(5, 1001)]), ElemwiseCase("H_SWISH", [(5, 1001)], span=(-6.0, 6.0)),
+            ElemwiseCase("MAX", [(3, 1, 5, 1), (3, 4, 5, 6)]),
+            ReduceCase("MAX", (64, 1000), 1), ReduceCase("SUM", (64, 1000), 1),
+            ReduceCase("MEAN", (8, 1024, 49), 2), ReduceCase("MEAN", (6, 50, 33), 1),
+            ReduceCase("MIN", (50, 7, 9), 0)]
+
+
+@pytest.mark.skipif(not ref.available(), reason="oracle/_ref not built (needs /root/reference)")
+@pytest.mark.parametrize("idx", range(14))
+def test_port_f32_elemwise_reduce_match_reference_live(idx):
+    """larger shapes through the reference's generated GI kernels (SIMD bodies + scalar tails;
+    their exp is a polynomial, hence the tolerance)"""
+    case = _live_f32()[idx]
+    if not ref.has(case.symbol()):
+        pytest.skip("symbol not in this _ref build")
+    arrays = case.gen(seed=7)
+    want = cases.run_ref(case, arrays)
+    got = case.run_port(arrays)
+    assert got.shape == want.shape
+    tol = 1e-4 if type(case).__name__ == "ReduceCase" else 1e-5  # (SIMD partial sums: another order)
+    assert cases.max_rel_err(got, want) <= tol, repr(case)

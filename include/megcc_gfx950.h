@@ -290,10 +290,21 @@ TinyNNStatus megcc_gfx950_conv2d(
 TinyNNStatus megcc_gfx950_conv2d_init(
         const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor* out_weights,
         int* nr_out_weight, const RuntimeOpt* opt);
-/* Always 0 bytes: padding and im2col are folded into the LDS loads (the reference's optimised
- * paths copy a padded source into workspace, e.g. GeneralIntrinsic/ConvKernel/Im2colCommon.cpp:
- * 326-377). Plain C semantics, no side effects, so the compiler may evaluate it at compile time
- * as compiler/lib/KernelGen/Jit/JitExe.cpp:67-123 does. */
+/* Scratch bytes of the layer; MUST be queried (with the unpacked filter, before the init protocol
+ * replaces it, as the compiler does) and handed to megcc_gfx950_conv2d. Padding and im2col are
+ * folded into the LDS loads (the reference's optimised paths copy a padded source into workspace,
+ * e.g. GeneralIntrinsic/ConvKernel/Im2colCommon.cpp:326-377), so most layers report 0; these do
+ * not:
+ *   - dense qsi8 layers with few output pixels and a long K (batch-1 layers, FullyConnected with
+ *     up to 64 rows) and skinny f32 layers: int32 / f32 partial sums of a split of K. Without the
+ *     workspace the layer still runs, unsplit and slower;
+ *   - a 1x1 NCHW44 convolution with a stride: the gathered pixels. REQUIRED: without it the call
+ *     returns TinyNN_ERROR_OUT_OF_RANGE (the filter was packed for the gathered geometry);
+ *   - a dense qsi8 convolution on plain NCHW tensors: both NCHW44 copies. REQUIRED likewise;
+ *   - a channel-wise qsi8 convolution on plain NCHW tensors: both NCHW44 copies and the filter.
+ *     Without it the layer runs on the generic one-output-per-thread kernel.
+ * Plain C semantics, no side effects, so the compiler may evaluate it at compile time as
+ * compiler/lib/KernelGen/Jit/JitExe.cpp:67-123 does. */
 TinyNNStatus megcc_gfx950_conv2d_workspace(
         const MegccConvAttr* attr, Tensor** inputs, int nr_input, int nr_thread,
         size_t* workspace);

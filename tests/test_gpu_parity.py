@@ -560,3 +560,27 @@ def test_errors_do_not_launch():
     st = runtime.lib().megcc_gfx950_conv2d(
         C.byref(attr), abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1, None, None)
     assert st == abi.ERROR_UNSUPPORTED_DTYPE_TYPE
+
+
+@pytest.mark.parametrize("case", [
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 16, 9, 9, 8, 1, 2, 0, A.RELU, scales=(0.02, 0.01, unsat(16))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 2, 16, 20, 24, 12, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(144))),
+], ids=["strided_1x1", "dense_nchw"])
+def test_layers_that_require_their_workspace_say_so(case):
+    """a strided 1x1 NCHW44 layer and a dense layer on plain NCHW tensors run on copies in the
+    workspace; once the init protocol has packed the filter for that, a call without the
+    workspace (or with a short one) must fail with TinyNN_ERROR_OUT_OF_RANGE and launch nothing"""
+    import ctypes as C
+    arrays = case.gen(5)
+    ins, outs = case.specs(arrays)
+    op = runtime.PreparedOp(runtime.parse_symbol(case.symbol()), ins, outs)
+    assert op.n_processed == 1 and op.ws.size > 0
+    for ws in (None, abi.Workspace(op.ws.ptr, op.ws.size - 1, 0)):
+        st = runtime.lib().megcc_gfx950_call(
+            C.byref(op.desc), op.ins, len(op.in_tensors), op.outs, len(op.out_tensors),
+            C.byref(ws) if ws is not None else None, None)
+        assert st == abi.ERROR_OUT_OF_RANGE
+        assert b"workspace" in runtime.lib().megcc_gfx950_last_error()
+    assert (op.result().view(np.uint8) == cases.POISON).all(), "nothing may have been written"
+    op.launch()
+    compare(op.result(), case.run_port(arrays), repr(case))

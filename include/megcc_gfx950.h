@@ -309,6 +309,23 @@ TinyNNStatus megcc_gfx950_conv2d_workspace(
         const MegccConvAttr* attr, Tensor** inputs, int nr_input, int nr_thread,
         size_t* workspace);
 
+/* megcc_gfx950_conv2d without the workspace argument and without any allocation. No counterpart
+ * in the reference (its kernels get their scratch from the VM's arena); it is for callers that
+ * cannot allocate or plan a workspace: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc. The scratch the layer's kernels need (split-K partial sums,
+ * gathered pixels, NCHW44 copies: see megcc_gfx950_conv2d_workspace) lives in a static device
+ * array of MEGCC_GFX950_NOALLOC_SCRATCH_BYTES that each GPU the library runs on holds until the
+ * process ends. A layer that needs more returns TinyNN_ERROR_OUT_OF_RANGE (use
+ * megcc_gfx950_conv2d). `inputs[1]` is the filter as the init protocol left it. Every call on a
+ * GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race.
+ * Nothing in the array has to start at zero - every byte a kernel reads was written by an
+ * earlier kernel of the same call. Calls no hipMalloc / hipFree; the array's address is looked
+ * up at megcc_gfx950_init_device() or, failing that, on the first call on a device. */
+#define MEGCC_GFX950_NOALLOC_SCRATCH_BYTES (32u << 20)
+TinyNNStatus megcc_gfx950_conv2d_noalloc(
+        const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const RuntimeOpt* opt);
+
 /* f32 MatrixMul, row-major, C = op(A) * op(B), no bias. Replaces GeneralIntrinsic::
  * Fp32MatMulM4N12 (GeneralIntrinsic/MatMulKernel/Fp32MatMulM4N12.cpp:9-158), Fp32GevmKernel
  * (GeneralIntrinsic/MatMulKernel/Fp32Gevm.cpp:50-119) and BareMetal::MatrixMulKernel

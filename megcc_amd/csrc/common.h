@@ -37,6 +37,10 @@ Options& options();
 // and up to five numbers that identify the instantiation; megcc_gfx950_last_kernel() formats them.
 void note_kernel(const char* name, int a = -1, int b = -1, int c = -1, int d = -1, int e = -1);
 
+// conv_api.hip: looks up the address of the static scratch array of
+// megcc_gfx950_conv2d_noalloc on the current device (once per device; later calls return at once).
+TinyNNStatus noalloc_scratch_setup();
+
 // After a kernel launch: surfaces launch-configuration errors as TinyNN_ERROR_RUNTIME.
 TinyNNStatus check_launch(const char* what);
 

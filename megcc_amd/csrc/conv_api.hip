@@ -8,6 +8,8 @@
 //   qsi8 NCHW44 dense, anything else (5x5, 7x7, filter not packed)   -> conv_dot4.hip
 //   f32 NCHW DENSE                                                  -> gemm_f32.hip
 //   everything else ConvGeneral accepts                             -> conv_direct.hip
+#include <mutex>
+
 #include "common.h"
 #include "conv_geom.h"
 
@@ -199,13 +201,66 @@ static void nchw44_views(int n, int c, int h, int w, Layout* view, Layout* dense
     }
 }
 
+// ---- scratch memory of megcc_gfx950_conv2d_noalloc ---------------------------------------------
+// One array per GPU, placed by the loader when the code object is loaded on that GPU; it holds
+// whatever the last call left in it. In host code its NAME is only a handle for
+// hipGetSymbolAddress: every use of the memory goes through the per-device address that call
+// returns.
+static __device__ __align__(256) unsigned char scratch[MEGCC_GFX950_NOALLOC_SCRATCH_BYTES];
+
+static constexpr int MAX_GPUS = 64;
+static void* g_scratch_ptr[MAX_GPUS];  // address of `scratch` on device i, once asked for
+static std::mutex g_scratch_lock;
+
+// Address of the current device's copy of `scratch` (asked for once per device).
+static TinyNNStatus scratch_of_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    MG_REQUIRE(e == hipSuccess && dev >= 0 && dev < MAX_GPUS, TinyNN_ERROR_RUNTIME,
+               "conv2d_noalloc: no current HIP device (%s)", hipGetErrorString(e));
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        MG_REQUIRE(e == hipSuccess && p, TinyNN_ERROR_RUNTIME,
+                   "conv2d_noalloc: address of the scratch array on device %d: %s", dev,
+                   hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return TinyNN_SUCCESS;
+}
+
+TinyNNStatus noalloc_scratch_setup() {
+    void* p = nullptr;
+    return scratch_of_current_device(&p);
+}
+
+// Scratch bytes the kernels of this layer take from the workspace (what
+// megcc_gfx950_conv2d_workspace reports before the filter is packed).
+static size_t conv2d_scratch_bytes(const ConvGeom& g, bool q8, bool f32, bool packed) {
+    if (packed && q8 && strided_pointwise(g) && conv_mfma_supported(subsampled(g)))
+        return round_up256(conv_mfma_workspace_bytes(subsampled(g))) + gather_bytes(g);
+    if (packed && q8 && nchw_spatial(g) && conv_mfma_supported(as_nchw44(g)))
+        return round_up256(conv_mfma_workspace_bytes(as_nchw44(g))) +
+               round_up256((size_t)g.n * g.ic * g.ih * g.iw) + (size_t)g.n * g.oc * g.oh * g.ow;
+    if (packed && q8 && conv_mfma_supported(g))
+        return conv_mfma_workspace_bytes(g);
+    if (!packed && q8 && nchw_depthwise(g) && dwconv44_supported(as_nchw44(g)))
+        return nchw_depthwise_bytes(g);
+    if (f32 && !(conv_f32_small_supported(g) && !options().no_f32small) && conv_f32_gemm_supported(g))
+        return conv_f32_gemm_workspace_bytes(g);
+    return 0;
+}
+
 }  // namespace mg
 
 using namespace mg;
 
-extern "C" TinyNNStatus megcc_gfx950_conv2d(
+// `workspace` from the caller, or (static_scratch) the library's own array of the current GPU.
+static TinyNNStatus conv2d_run(
         const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
-        const Workspace* workspace, const RuntimeOpt*) {
+        const Workspace* workspace, bool static_scratch) {
     MG_REQUIRE(attr, TinyNN_ERROR_NULL_PTR, "conv2d: NULL attr");
     const int want_in = attr->with_bias ? 3 : 2;
     // the test harness of the reference passes an extra empty `z` operand after the bias
@@ -243,6 +298,21 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
     const void* b = bias ? bias->ptr : nullptr;
     if ((size_t)g.n * g.oc * g.oh * g.ow == 0)
         return TinyNN_SUCCESS;
+    Workspace own = {nullptr, 0, 0};
+    if (static_scratch) {
+        const size_t need = conv2d_scratch_bytes(g, q8, f32, packed);
+        MG_REQUIRE(need <= (size_t)MEGCC_GFX950_NOALLOC_SCRATCH_BYTES, TinyNN_ERROR_OUT_OF_RANGE,
+                   "conv2d_noalloc: this layer needs %zu bytes of scratch memory, the static "
+                   "buffer holds %zu; call megcc_gfx950_conv2d with a workspace instead",
+                   need, (size_t)MEGCC_GFX950_NOALLOC_SCRATCH_BYTES);
+        if (need) {
+            st = scratch_of_current_device(&own.ptr);
+            if (st != TinyNN_SUCCESS)
+                return st;
+            own.size = need;
+        }
+        workspace = &own;
+    }
 
     if (packed && q8 && strided_pointwise(g) && conv_mfma_supported(subsampled(g))) {
         const ConvGeom g1 = subsampled(g);
@@ -370,6 +440,18 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d(
     }
     note_kernel("conv_direct");
     return conv_direct_launch(g, f32, src->ptr, flt->ptr, b, dst->ptr);
+}
+
+extern "C" TinyNNStatus megcc_gfx950_conv2d(
+        const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace* workspace, const RuntimeOpt*) {
+    return conv2d_run(attr, inputs, nr_input, outputs, nr_output, workspace, false);
+}
+
+extern "C" TinyNNStatus megcc_gfx950_conv2d_noalloc(
+        const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const RuntimeOpt*) {
+    return conv2d_run(attr, inputs, nr_input, outputs, nr_output, nullptr, true);
 }
 
 extern "C" TinyNNStatus megcc_gfx950_conv2d_init(

@@ -143,6 +143,10 @@ TinyNNStatus megcc_gfx950_init_device(Device* device) {
     int n = 0;
     MG_REQUIRE(hipGetDeviceCount(&n) == hipSuccess && n > 0, TinyNN_ERROR_RUNTIME,
                "init_device: no HIP device");
+    // (so that a first megcc_gfx950_conv2d_noalloc call under stream capture has nothing to set up)
+    TinyNNStatus st = noalloc_scratch_setup();
+    if (st != TinyNN_SUCCESS)
+        return st;
     device->alignment = 256;
     device->device_type = TinyNN_GFX950;
     device->malloc = megcc_gfx950_malloc;

@@ -27,6 +27,7 @@ def lib():
         L.megcc_gfx950_conv2d.argtypes = [C.POINTER(abi.ConvAttr)] + kern
         L.megcc_gfx950_conv2d_init.argtypes = [C.POINTER(abi.ConvAttr)] + abi.INIT_ARGS
         L.megcc_gfx950_conv2d_workspace.argtypes = [C.POINTER(abi.ConvAttr)] + abi.WORKSPACE_ARGS
+        L.megcc_gfx950_conv2d_noalloc.argtypes = [C.POINTER(abi.ConvAttr)] + kern[:4] + kern[5:]
         L.megcc_gfx950_matmul.argtypes = [C.POINTER(abi.MatMulAttr)] + kern
         L.megcc_gfx950_matmul_workspace.argtypes = [C.POINTER(abi.MatMulAttr)] + abi.WORKSPACE_ARGS
         L.megcc_gfx950_pooling.argtypes = [C.POINTER(abi.PoolAttr)] + kern
@@ -95,6 +96,7 @@ def lib():
 
 EXPORTS = [
     "megcc_gfx950_conv2d", "megcc_gfx950_conv2d_init", "megcc_gfx950_conv2d_workspace",
+    "megcc_gfx950_conv2d_noalloc",
     "megcc_gfx950_matmul", "megcc_gfx950_matmul_workspace", "megcc_gfx950_pooling",
     "megcc_gfx950_elemwise_multitype", "megcc_gfx950_elemwise", "megcc_gfx950_typecvt",
     "megcc_gfx950_reduce", "megcc_gfx950_relayout", "megcc_gfx950_concat", "megcc_gfx950_resize", "megcc_gfx950_fused_elemwise",
@@ -268,6 +270,18 @@ class PreparedOp:
     def launch(self):
         check(lib().megcc_gfx950_call(C.byref(self.desc), self.ins, len(self.in_tensors), self.outs,
                                       len(self.out_tensors), C.byref(self.ws), None), "kernel")
+
+    def launch_noalloc(self):
+        """the same convolution through megcc_gfx950_conv2d_noalloc: no workspace argument, the
+        library's static scratch array instead"""
+        assert self.desc.kind == abi.KERN_CONV
+        check(lib().megcc_gfx950_conv2d_noalloc(
+            C.byref(self.desc.attr.conv), self.ins, len(self.in_tensors), self.outs,
+            len(self.out_tensors), None), "conv2d_noalloc")
+
+    def poison_outputs(self):
+        for buf in self.out_bufs:
+            buf.fill(0x5A)
 
     def result(self, i=0):
         s = self.out_specs[i]

@@ -14,7 +14,18 @@ then one kernel call per step with all operands resident in HBM.
   cpu_baseline  the reference's own generated C kernel (oracle/_ref, kind "reference") or our C
              restatement (kind "port") on ONE host core, on a bounded slice of the same layer
 
-Other workloads (--workload dw|fc|chain ...) are for development; the driver uses the default.
+  checked    after the timed region the output of the LAST timed launch is fetched and compared
+             with the CPU oracle (bit for bit for qsi8): images 0, middle and last of a batched
+             convolution (the reference's kernels treat images independently, so the oracle on one
+             image is exact for that image), the whole tensor for small workloads. A mismatch
+             aborts the run: no metric line is printed for wrong results.
+
+Before the W warm-up steps the same operator is launched untimed for --preheat-ms (default 300 ms):
+a cold MI355X takes a few hundred 60 us launches to leave its idle clocks, and 5 warm-up launches
+(1/3 ms) measure that ramp rather than the kernel. The line says how many launches that was.
+
+Other workloads (--workload dw|fc|chain|mobilenet ...) report the other configurations; the driver
+uses the default.
 """
 import argparse
 import ctypes as C
@@ -30,10 +41,25 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
 
 PEAK_INT8_TOPS = 5000.0  # dense int8 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the default workload's kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch, scaled by what a 256 MiB copy reads on the same counters: x2.000 / x1.000);
-# the counter runs and their figures are in profiles/conv_mfma_i8_dma__conv3x3_n32_c256_56x56.txt
-MEASURED_TRAFFIC = {"conv": (37666 * 2.000 + 25088 * 1.000) * 1024}
+# HBM bytes per launch of a workload's dominant kernel come from the committed rocprofv3 --pmc
+# summaries (FETCH_SIZE / WRITE_SIZE in KiB per dispatch, scaled by what a 256 MiB copy reads on
+# the same counters); each summary ends in a line "TRAFFIC_BYTES_PER_LAUNCH=<n>".
+TRAFFIC_FILES = {"conv": "profiles/conv_mfma_i8_dma__conv3x3_n32_c256_56x56.txt"}
+
+
+def measured_traffic(workload):
+    """(bytes per launch, file it was read from) or (None, None)"""
+    rel = TRAFFIC_FILES.get(workload)
+    if not rel:
+        return None, None
+    try:
+        with open(os.path.join(ROOT, rel)) as f:
+            for line in f:
+                if line.startswith("TRAFFIC_BYTES_PER_LAUNCH="):
+                    return int(line.split("=", 1)[1]), rel
+    except OSError:
+        pass
+    return None, None
 
 
 class HipEvents:
@@ -158,6 +184,13 @@ def make_workload(name):
     if name == "conv_f32":
         case = ConvCase(abi.FMT_NCHW, abi.DENSE, 1, 32, 56, 56, 32, 3, 1, 1, abi.RELU, dtype="f32")
         return case, "f32 conv3x3 NCHW N=1 C=32 56x56 +bias +ReLU", "mfma_f32"
+    if name in ("bias64", "bias4096", "bias1"):  # the f32 FullyConnected bias: [M,N] + [N]
+        from cases import ElemwiseCase
+        m, n = {"bias64": (64, 4096), "bias4096": (4096, 4096), "bias1": (1, 1000)}[name]
+        return ElemwiseCase("ADD", [(m, n), (n,)]), "f32 elementwise ADD [%d,%d] + [%d]" % (m, n, n), "hbm"
+    if name == "softmax_max":
+        from cases import ReduceCase
+        return ReduceCase("MAX", (64, 1000), 1), "f32 reduce MAX [64,1000] axis 1", "hbm"
     if name == "copy":  # same-scale requantise = a plain copy: the counter calibration kernel
         return (TypeCvtCase("qsi8", "qsi8", (256, 1024, 1024), src_scale=0.05, dst_scale=0.05),
                 "qsi8->qsi8 typecvt, equal scales, 256 MiB in + 256 MiB out", "hbm")
@@ -207,6 +240,107 @@ def bench_mobilenet(batch, steps, warmup, per_layer=False):
     return out
 
 
+def check_output(case, arrays, got):
+    """Compares the output the timed launches left behind with the CPU oracle. Returns a short
+    description of what was compared; raises SystemExit on a mismatch."""
+    import numpy as np
+    import cases
+    from cases import ConvCase
+    from oracle import port
+    port.set_threads(os.cpu_count() or 8)
+
+    def same(a, b, what):
+        if a.dtype == np.float32:
+            err = cases.max_rel_err(a, b)
+            if err > 1e-4:
+                raise SystemExit("bench.py: %s differs from the oracle (max err %g)" % (what, err))
+        elif not np.array_equal(a, b):
+            raise SystemExit("bench.py: %s differs from the oracle in %d of %d elements" % (
+                what, int((a != b).sum()), a.size))
+
+    if isinstance(case, ConvCase) and case.n > 3 and case.ops() > 4e9:
+        picks = sorted({0, case.n // 2, case.n - 1})
+        import copy
+        one = copy.copy(case)
+        one.n = 1
+        for i in picks:
+            want = one.run_port({"src": arrays["src"][i:i + 1], "flt": arrays["flt"], "bias": arrays["bias"]})
+            same(got[i:i + 1], want, "image / row %d of the output" % i)
+        return "%s %s of %d against the oracle, bit for bit" % (
+            "rows" if case.ih == 1 and case.fmt == 0 else "images", picks, case.n)
+    if hasattr(case, "ops") and case.ops() > 4e10:
+        return None  # (too large for the oracle in a benchmark run; covered by tests/test_full_size.py)
+    same(got, case.run_port(arrays), "the output")
+    return "whole output against the oracle"
+
+
+def bench_chain(c, hw, stride, steps, warmup, batch=64):
+    """BASELINE configs[3]: depthwise 3x3 -> max-pool 2x2 s2 -> add + ReLU with requantisation,
+    three operators of one model on the static arena, replayed as a HIP graph. Bytes = what each
+    operator must read and write once (the pooled map's partner tensor included)."""
+    import numpy as np
+    from cases import ConvCase, MultiTypeCase, PoolCase
+    from megcc_amd import abi, runtime
+    dw = ConvCase(abi.FMT_NCHW44, abi.GROUP, batch, c, hw, hw, c, 3, stride, 1, abi.RELU,
+                  scales=(0.02, 0.01, 0.05))
+    pool = PoolCase(abi.FMT_NCHW44, abi.POOL_MAX, batch, c, dw.oh, dw.ow, 2, 2, 0, scale=0.05)
+    add = MultiTypeCase(abi.Q_FUSE_ADD_RELU, pool.dst_shape(), (0.05, 0.01, 0.05))
+    arrays = dw.gen(0)
+    other = np.random.default_rng(1).integers(-128, 128, pool.dst_shape()).astype(np.int8)
+    m = runtime.Model()
+    x = m.tensor("x", dw.src_shape(), abi.QINT8, 0.02)
+    y = m.tensor("other", pool.dst_shape(), abi.QINT8, 0.01)
+    m.mark_input(x)
+    m.mark_input(y)
+    w = m.weight("dw.w", arrays["flt"], abi.QINT8, 0.01)
+    b = m.weight("dw.b", arrays["bias"], abi.QINT32, float(np.float32(0.02) * np.float32(0.01)))
+    t1 = m.tensor("dw", dw.dst_shape(), abi.QINT8, 0.05)
+    m.opr(dw.symbol(), [x, w, b], [t1])
+    t2 = m.tensor("pool", pool.dst_shape(), abi.QINT8, 0.05)
+    m.opr(pool.symbol(), [t1], [t2])
+    t3 = m.tensor("out", pool.dst_shape(), abi.QINT8, 0.05)
+    m.opr(add.symbol(), [t2, y], [t3])
+    m.mark_output(t3)
+    m.finalize()
+    m.set_input(x, arrays["src"])
+    m.set_input(y, other)
+    ev = HipEvents(runtime.lib().megcc_gfx950_stream())
+    for _ in range(max(warmup, 3)):
+        m.forward()
+    runtime.wait()
+    e0, e1 = ev.new(), ev.new()
+    ev.record(e0)
+    for _ in range(steps):
+        m.forward()
+    ev.record(e1)
+    runtime.wait()
+    ms = ev.elapsed_ms(e0, e1) / steps
+    n_in, n_dw, n_pool = (int(np.prod(sh)) for sh in (dw.src_shape(), dw.dst_shape(), pool.dst_shape()))
+    nbytes = (n_in + n_dw) + (n_dw + n_pool) + 3 * n_pool
+    # what came out, against the oracle on image 0 and the last one
+    from oracle import port
+    port.set_threads(os.cpu_count() or 8)
+    got = m.get(t3)
+    one = ConvCase(abi.FMT_NCHW44, abi.GROUP, 1, c, hw, hw, c, 3, stride, 1, abi.RELU, scales=(0.02, 0.01, 0.05))
+    for i in (0, batch - 1):
+        d = one.run_port({"src": arrays["src"][i:i + 1], "flt": arrays["flt"], "bias": arrays["bias"]})
+        p = port.pool_q8(d, abi.FMT_NCHW44, abi.POOL_MAX, (2, 2), (2, 2), (0, 0))
+        want = port.multitype_q8(p, other[i:i + 1], abi.Q_FUSE_ADD_RELU, 0.05, 0.01, 0.05)
+        if not np.array_equal(got[i:i + 1], want):
+            raise SystemExit("bench.py: chain output of image %d differs from the oracle" % i)
+    m.close()
+    return {"metric": "hbm_gbps", "value": round(nbytes / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+            "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
+            "data": "synthetic",
+            "config": {"workload": "qsi8 depthwise 3x3 s%d -> maxpool 2x2 s2 -> add+ReLU requant, N=%d C=%d %dx%d NCHW44"
+                       % (stride, batch, c, hw, hw)},
+            "roofline": {"bound": "hbm", "achieved": round(nbytes / (ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                         "traffic": None, "algorithmic_per_launch": nbytes},
+            "checked": True, "checked_what": "images 0 and %d of the chain's output, bit for bit" % (batch - 1)}
+
+
 def case_bytes(case):
     ins, outs = case.specs(case.gen(0))
     return sum(s.nbytes for s in ins) + sum(s.nbytes for s in outs)
@@ -248,6 +382,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=500,
                     help="untimed launches first (the GPU takes a few hundred 70 us launches to "
                          "reach its sustained clocks)")
+    ap.add_argument("--preheat-ms", type=float, default=300.0,
+                    help="untimed launches of the same operator before the warm-up steps, for this long")
     ap.add_argument("--workload", default="conv")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--batch", type=int, default=64, help="batch of the mobilenet workload")
@@ -263,6 +399,11 @@ def main():
     if args.workload == "mobilenet":
         print(json.dumps(bench_mobilenet(args.batch, args.steps, args.warmup, args.per_layer)))
         return
+    if args.workload.startswith("chain"):  # chain, chain_s2, chain512, chain512_s2
+        c, hw, st = {"chain": (32, 112, 1), "chain_s2": (32, 112, 2), "chain512": (512, 14, 1),
+                     "chain512_s2": (512, 14, 2)}[args.workload]
+        print(json.dumps(bench_chain(c, hw, st, args.steps, args.warmup)))
+        return
     case, desc, bound = make_workload(args.workload)
     arrays = case.gen(seed=0)
     ins, outs = case.specs(arrays)
@@ -270,6 +411,13 @@ def main():
     op = runtime.PreparedOp(kdesc, ins, outs)
     ev = HipEvents(runtime.lib().megcc_gfx950_stream())
 
+    preheat = 0
+    t_heat = time.perf_counter() + args.preheat_ms * 1e-3
+    while time.perf_counter() < t_heat:
+        for _ in range(50):
+            op.launch()
+        runtime.wait()
+        preheat += 50
     for _ in range(args.warmup):
         op.launch()
     runtime.wait()
@@ -282,8 +430,10 @@ def main():
     runtime.wait()
     wall = time.perf_counter() - t0
     kern_ms = ev.elapsed_ms(e0, e1) / args.steps
+    kernel_name = runtime.last_kernel()
 
-    # spot check of the timed output against the oracle on one image (full check is in tests/)
+    # outside the timed region: what the timed launches computed, against the CPU oracle
+    checked = check_output(case, arrays, op.result())
     ops = case.ops() if hasattr(case, "ops") else 0
     nbytes = case_bytes(case)
     ms = wall * 1e3 / args.steps
@@ -300,8 +450,9 @@ def main():
         value, unit, metric = nbytes / (wall / args.steps) / 1e9, "GB/s", "hbm_gbps"
         roof = {"bound": "hbm", "achieved": round(nbytes / (kern_ms * 1e-3) / 1e9, 2),
                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "traffic": None}
-    if args.workload in MEASURED_TRAFFIC:
-        roof["traffic"] = int(MEASURED_TRAFFIC[args.workload])
+    roof["traffic"], traffic_file = measured_traffic(args.workload)
+    if traffic_file:
+        roof["traffic_source"] = traffic_file
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
     roof["kernel_ms"] = round(kern_ms, 5)
     roof["algorithmic_per_launch"] = ops if bound == "mfma" else nbytes
@@ -311,17 +462,24 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if unit == "TFLOP/s" else "int8", "data": "synthetic",
-        "config": {"workload": desc, "symbol": case.symbol(), "abi": "megcc_gfx950_call"},
+        "config": {"workload": desc, "symbol": case.symbol(), "abi": "megcc_gfx950_call",
+                   "kernel": kernel_name},
         "roofline": roof,
+        "checked": checked is not None, "checked_what": checked,
+        "preheat_launches": preheat,
     }
     if not args.no_cpu and args.workload == "conv":
         out["cpu_baseline"] = cpu_baseline(case)
         op = None
         mb = bench_mobilenet(64, 200, 100)
+        mb1 = bench_mobilenet(1, 300, 100)
+        mb256 = bench_mobilenet(256, 60, 30)
         import mobilenet
         cpu_s, used = mobilenet.Net(1).run_cpu_timed(mobilenet.draw_input(1, seed=1), threads=1)
         out["extra"] = {"mobilenet_v1_int8_images_per_s_batch64": mb["images_per_s"],
                         "mobilenet_v1_int8_ms_per_forward_batch64": mb["ms_per_forward"],
+                        "mobilenet_v1_int8_images_per_s_batch1": mb1["images_per_s"],
+                        "mobilenet_v1_int8_images_per_s_batch256": mb256["images_per_s"],
                         "mobilenet_v1_int8_cpu_images_per_s": round(1.0 / cpu_s, 4),
                         "mobilenet_v1_int8_cpu_note": "1 host core, batch 1, one forward in %.2f s: "
                         "%d operators by MegCC's generated x86 kernels, %d by the C restatement" % (

@@ -1,5 +1,5 @@
-// Definitions shared by the two qsi8 MFMA convolution kernels (conv_mfma_i8.hip: one stage at a time,
-// any shape; conv_mfma_i8_wide.hip and conv_mfma_i8_ws.hip: pipelined, large shapes).
+// Definitions shared by the qsi8 MFMA convolution kernels (conv_mfma_i8.hip: one stage at a time,
+// any shape; conv_mfma_i8_dma.hip: LDS-direct loads, pipelined, large shapes).
 #pragma once
 #include <stddef.h>
 #include <utility>
@@ -45,8 +45,6 @@ struct MfmaParams {
     int split, sps;
     int32_t* partial;
     FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
-    int G, RG;       // 16-byte gather: pixel groups per row, groups per plane of the largest patch
-    FastDiv dG, dRG;
     // exact requantisation thresholds for IDENTITY / RELU (built on the host, epilogue.h); only
     // the kernels that look outputs up in LDS read it
     RequantTable rq_table;
@@ -139,8 +137,7 @@ __device__ __forceinline__ void dma_buffer_b128(v4u rsrc, unsigned voffset, unsi
 }
 
 struct PipeConfig {
-    int bm, bn, ks, maxb, blocks_per_cu, threads, a_bytes, g4;
-    int gather_threads;  // threads that share the activation gather (maxb items each)
+    int bm, bn, ks, blocks_per_cu, threads, a_bytes;
     int nbuf;            // LDS stage buffers
     int extra_lds;       // bytes of LDS beyond the stage buffers
     int fixed_lmax;      // patch slots compiled into the kernel (0: run-time Lmax)

@@ -472,10 +472,26 @@ TinyNNStatus conv_mfma_pack(const ConvGeom& g, const void* flt, void* packed) {
     return check_launch("pack_filter");
 }
 
-bool conv_mfma_pipe_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
-bool conv_mfma_ws_config(const ConvGeom& g, bool g4_ok, PipeConfig* c);
 bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok, PipeConfig* c);
-TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q);
+
+// launches a configuration of the LDS-direct kernel (conv_mfma_i8_dma.hip): one workgroup per
+// pixel range and output-channel tile, the whole grid resident at once
+static TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q) {
+    const size_t lds = c.nbuf * ((size_t)c.a_bytes + (size_t)c.ks * q.Lmax * KROW) + c.extra_lds;
+    MG_REQUIRE(lds <= 160 * 1024, TinyNN_ERROR_OUT_OF_RANGE, "conv_mfma_i8_dma: %zu bytes of LDS", lds);
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(c.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_mfma_i8_dma: LDS attribute: %s",
+                   hipGetErrorString(e));
+    }
+    dim3 grid((q.P + q.range_len - 1) / q.range_len, (q.OC + c.bm - 1) / c.bm);
+    void* args[] = {&q};
+    hipError_t e = hipLaunchKernel(c.kernel, grid, dim3(c.threads), args, lds, stream());
+    MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_mfma_i8_dma: launch: %s", hipGetErrorString(e));
+    return check_launch("conv_mfma_i8_dma");
+}
+
+
 
 int fc_stream_split(const ConvGeom& g, const void* src, size_t ws_bytes, int max_split);
 TinyNNStatus fc_stream_launch(
@@ -500,34 +516,26 @@ TinyNNStatus conv_mfma_launch(
     }
     MfmaParams q = {};
     PipeConfig pc;
-    const bool g4_ok = g.fmt == MEGCC_FMT_NCHW44 && (g.iw & 3) == 0 && ((uintptr_t)src & 15) == 0;
     const bool b128_ok = ((uintptr_t)src & 15) == 0 && !options().no_fcb;
     // candidates in order of preference; development switches (MEGCC_NO...) skip one
     long range_len = 0;
     TilePlan t;
     bool pipe = false;
-    int picked = -1;  // DMA variant, 100 = producer/consumer kernel, 101 = register-staged kernel
-    // DMA kernel variants in order of preference (see conv_mfma_dma_config), then the two older
-    // generations
+    int picked = -1;  // variant of the LDS-direct kernel
+    // variants of the LDS-direct kernel in order of preference (see conv_mfma_dma_config); a
+    // layer none of them takes runs on the one-stage kernel below
     static const int kDmaVariants[] = {6, 7, 2, 3, 0, 4, 1};
     const Options& opt = options();
     const bool dma_off[] = {opt.no_small, opt.no_small, opt.no_pm768, opt.no_pm,
                             opt.no_dma512, opt.no_pm256, opt.no_dma};
     constexpr int N_DMA_VARIANTS = 7;
-    for (int cand = 0; cand < N_DMA_VARIANTS + 2 && !pipe; ++cand) {
-        bool have = false;
-        if (cand < N_DMA_VARIANTS) {
-            const int v = kDmaVariants[cand];
-            have = !opt.no_dma && !dma_off[cand] && !((v == 2 || v == 4 || v == 6) && opt.no_pm) &&
-                   conv_mfma_dma_config(g, is_fc(g), v, b128_ok, &pc);
-        } else if (cand == N_DMA_VARIANTS) {
-            have = !opt.no_ws && conv_mfma_ws_config(g, g4_ok, &pc);
-        } else {
-            have = !opt.no_wide && conv_mfma_pipe_config(g, g4_ok, &pc);
-        }
+    for (int cand = 0; cand < N_DMA_VARIANTS && !pipe; ++cand) {
+        const int v = kDmaVariants[cand];
+        const bool have = !opt.no_dma && !dma_off[cand] && !((v == 2 || v == 4 || v == 6) && opt.no_pm) &&
+                          conv_mfma_dma_config(g, is_fc(g), v, b128_ok, &pc);
         if (!have)
             continue;
-        picked = cand < N_DMA_VARIANTS ? kDmaVariants[cand] : 100 + cand - N_DMA_VARIANTS;
+        picked = v;
         // one pixel range per free workgroup slot, so that the whole grid is resident at once and
         // every CU finishes at the same time (no partial last round)
         const long P = (long)g.n * g.oh * g.ow;
@@ -546,10 +554,7 @@ TinyNNStatus conv_mfma_launch(
                 continue;
             t.Lmax = pc.fixed_lmax;
         }
-        const long gather_items =
-                pc.g4 ? 8L * pc.ks * t.rows_max * (g.iw / 4) : 2L * pc.ks * t.Lmax;
-        pipe = (pc.gather_threads == 0 || gather_items <= (long)pc.maxb * pc.gather_threads) &&
-               ((long)pc.nbuf * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) + pc.extra_lds) * pc.blocks_per_cu <= 160 * 1024;
+        pipe = ((long)pc.nbuf * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) + pc.extra_lds) * pc.blocks_per_cu <= 160 * 1024;
     }
     if (!pipe) {
         range_len = 0;
@@ -613,18 +618,12 @@ TinyNNStatus conv_mfma_launch(
     q.dVH = make_fastdiv(q.VH);
     q.dL = make_fastdiv(q.Lmax);
     q.dOHW = make_fastdiv(q.OHW);
-    q.G = g.iw / 4 > 0 ? g.iw / 4 : 1;
-    q.RG = t.rows_max * q.G;
-    q.dG = make_fastdiv(q.G);
-    q.dRG = make_fastdiv(q.RG);
 
     q.split = 1;
     q.sps = q.stages;
     q.partial = nullptr;
     if (pipe) {
-        note_kernel(picked >= 100 ? (picked == 100 ? "conv_mfma_i8_ws" : "conv_mfma_i8_wide")
-                                  : "conv_mfma_i8_dma",
-                    picked >= 100 ? -1 : picked, pc.bm, pc.bn, q.Lmax, pc.ks);
+        note_kernel("conv_mfma_i8_dma", picked, pc.bm, pc.bn, q.Lmax, pc.ks);
         return conv_mfma_pipe_launch(pc, q);
     }
     const int split = conv_mfma_split(g);

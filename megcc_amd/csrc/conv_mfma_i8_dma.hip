@@ -403,10 +403,7 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.bm = DM_BM;
     c.bn = 128 * NT;
     c.ks = KS;
-    c.maxb = 0;
-    c.g4 = 0;
     c.threads = 256 * WGM;
-    c.gather_threads = 0;
     c.nbuf = DM_NBUF;
     c.blocks_per_cu = BPC;
     c.a_bytes = FH * FW * KS * c.bm * KROW;

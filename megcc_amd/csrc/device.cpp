@@ -26,8 +26,7 @@ const OptionName kOptions[] = {
         {"nofcb", &Options::no_fcb},         {"nosmall", &Options::no_small},
         {"nopm768", &Options::no_pm768},     {"nopm", &Options::no_pm},
         {"nodma512", &Options::no_dma512},   {"nopm256", &Options::no_pm256},
-        {"nodma", &Options::no_dma},         {"nows", &Options::no_ws},
-        {"nowide", &Options::no_wide},       {"nofcs", &Options::no_fcs},
+        {"nodma", &Options::no_dma},         {"nofcs", &Options::no_fcs},
         {"nopwshare", &Options::no_pwshare}, {"nohybrid", &Options::no_hybrid},
         {"nodot4", &Options::no_dot4},       {"nof32small", &Options::no_f32small},
         {"dw_generic", &Options::dw_generic}, {"no_graph", &Options::no_graph},

@@ -91,8 +91,10 @@ int root_of(const Model* m, int id) {
 
 // Offsets for the arena from the tensors' lifetimes: time step = operator index, a tensor is
 // alive from the operator that writes it to one past the last operator that reads it
-// (compiler/lib/Dialect/Kernel/Transforms/StaticMemoryPlanning.cpp:88-96); model inputs are staged
-// into the arena before the first operator and outputs stay valid after forward().
+// (compiler/lib/Dialect/Kernel/Transforms/StaticMemoryPlanning.cpp:88-96). Model inputs are not
+// planned: the compiler plans allocations only and the function arguments are the caller's memory
+// (runtime/src/init.c:456-460); here each input is a device buffer of its own, which keeps what
+// set_input put there across any number of forwards. Outputs stay valid after forward().
 bool plan_memory(Model* m) {
     if (m->preplanned)
         return true;
@@ -100,7 +102,7 @@ bool plan_memory(Model* m) {
     std::vector<int> ids;
     for (size_t i = 0; i < m->tensors.size(); ++i) {
         ModelTensor* t = m->tensors[i];
-        if (t->is_weight || t->alias_of >= 0 || t->def < 0)
+        if (t->is_weight || t->is_input || t->alias_of >= 0 || t->def < 0)
             continue;
         MemInterval iv;
         iv.begin = (size_t)t->def;
@@ -345,7 +347,7 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
     for (auto* t : m->tensors) {
         if (t->is_weight || t->alias_of >= 0)
             continue;
-        if (m->preplanned && t->is_input) {
+        if (t->is_input) {
             // user memory in the TinyNN runtime (runtime/src/init.c:456-460); here a device
             // buffer of its own that set_input fills
             t->owned = m->dev.malloc(t->t.size ? t->t.size : 1);

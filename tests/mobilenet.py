@@ -70,13 +70,13 @@ def draw_input(batch, seed=0):
 class Lifetimes:
     """Stands in for runtime.Model on a machine without a GPU: records tensors and operators and
     derives the memory-plan requests the model runtime makes from them - time step = operator
-    index; a tensor is alive from the operator that writes it (inputs: from step 0) to one past the
-    last operator that touches it (outputs: one past the last operator + 1); views share their
-    root's request; weights are not planned."""
+    index; a tensor is alive from the operator that writes it to one past the last operator that
+    touches it (outputs: one past the last operator + 1); views share their root's request;
+    weights and model inputs (the caller's memory) are not planned."""
 
     def __init__(self):
         self.sizes, self.root, self.first, self.last = [], [], [], []
-        self.is_weight, self.is_output, self.dtype = [], [], []
+        self.is_weight, self.is_output, self.is_input, self.dtype = [], [], [], []
         self.nr_opr = 0
 
     def _add(self, shape, type_enum, root=-1, weight=False):
@@ -86,6 +86,7 @@ class Lifetimes:
         self.last.append(-1)
         self.is_weight.append(weight)
         self.is_output.append(False)
+        self.is_input.append(False)
         self.dtype.append(type_enum)
         return len(self.sizes) - 1
 
@@ -117,6 +118,7 @@ class Lifetimes:
 
     def mark_input(self, t):
         r = self._root(t)
+        self.is_input[r] = True
         self.first[r] = 0
         self.last[r] = max(self.last[r], 0)
 
@@ -129,7 +131,8 @@ class Lifetimes:
     def requests(self):
         """(tensor ids, begin, end, size) in tensor-id order"""
         ids = [t for t in range(len(self.sizes))
-               if not self.is_weight[t] and self.root[t] < 0 and self.first[t] >= 0]
+               if not self.is_weight[t] and not self.is_input[t] and self.root[t] < 0
+               and self.first[t] >= 0]
         begin = [self.first[t] for t in ids]
         end = [self.nr_opr + 1 if self.is_output[t] else self.last[t] + 1 for t in ids]
         return ids, begin, end, [self.sizes[t] for t in ids]

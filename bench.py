@@ -194,6 +194,9 @@ def make_workload(name):
     if name == "copy":  # same-scale requantise = a plain copy: the counter calibration kernel
         return (TypeCvtCase("qsi8", "qsi8", (256, 1024, 1024), src_scale=0.05, dst_scale=0.05),
                 "qsi8->qsi8 typecvt, equal scales, 256 MiB in + 256 MiB out", "hbm")
+    if name == "copy_dw":  # a plain copy of the depthwise workload's size: what that size allows
+        return (TypeCvtCase("qsi8", "qsi8", (64, 32, 112 * 112), src_scale=0.05, dst_scale=0.05),
+                "qsi8->qsi8 typecvt, equal scales, 25.7 MB in + 25.7 MB out", "hbm")
     raise SystemExit("unknown workload " + name)
 
 

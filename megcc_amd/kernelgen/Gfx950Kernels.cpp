@@ -323,6 +323,8 @@ struct PoolingKernel : KernelFuncBase {
         return is_q(src.dtype, 8) && is_q(dst.dtype, 8) && src.scale == dst.scale;
     }
     std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)  // name filtering without a context (KernelGen.cpp:49-53)
+            return "kernel_pooling";
         std::stringstream ss;
         const bool f44 = c->getAttrStr("format") == "NCHW44";
         ss << (f44 ? "GI_" : "") << "kernel_pooling_" << c->getAttrStr("mode") << "_"
@@ -367,6 +369,8 @@ struct ElemwiseMultiTypeKernel : KernelFuncBase {
                 a.shape[1] == b.shape[1] && nb == b.shape[1]);
     }
     std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)  // name filtering without a context (KernelGen.cpp:49-53)
+            return "kernel_elementwise_multitype";
         return "kernel_elementwise_multitype_" + c->getAttrStr("mode") + "_" + io_str(c);
     }
     std::string GetKernelBody(TContext* c) const override {
@@ -398,6 +402,8 @@ struct ElemwiseKernel : KernelFuncBase {
         return ok;
     }
     std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)  // name filtering without a context (KernelGen.cpp:49-53)
+            return "kernel_elementwise";
         return "kernel_elementwise_" + c->getAttrStr("mode") + "_" + io_str(c);
     }
     std::string GetKernelBody(TContext* c) const override {
@@ -423,6 +429,8 @@ struct TypeCvtKernel : KernelFuncBase {
         return (is_f32(s.dtype) || s.scale > 0) && (is_f32(d.dtype) || d.scale > 0);
     }
     std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)  // name filtering without a context (KernelGen.cpp:49-53)
+            return "kernel_typecvt";
         const std::string p = pair(c);
         return std::string(p == "qsi32qsi8" ? "" : "GI_") + "kernel_typecvt_" + p;
     }
@@ -443,6 +451,8 @@ struct ReduceKernel : KernelFuncBase {
                 mode == "PRODUCT" || mode == "SUM_SQR");
     }
     std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)  // name filtering without a context (KernelGen.cpp:49-53)
+            return "kernel_reduce";
         std::stringstream ss;
         ss << "kernel_reduce_" << c->getAttrStr("mode") << "_" << c->getAttrStr("data_type")
            << "_a" << c->getAttrInt("axis") << "_" << io_str(c);
@@ -477,6 +487,8 @@ struct RelayoutKernel : KernelFuncBase {
         return dtype_bytes(d) != 0 && d == c->getAttrOprand("operand:1").dtype;
     }
     std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)  // name filtering without a context (KernelGen.cpp:49-53)
+            return "GI_kernel_relayout";
         return "GI_kernel_relayout_" + valid_dtype(c->getAttrOprand("operand:0").dtype);
     }
     std::string GetKernelBody(TContext* c) const override {
@@ -491,6 +503,8 @@ struct ConcatKernel : KernelFuncBase {
         return dtype_bytes(c->getAttrOprand("operand:0").dtype) != 0 && c->getAttrInt("axis") >= 0;
     }
     std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)  // name filtering without a context (KernelGen.cpp:49-53)
+            return "kernel_concat";
         std::stringstream ss;
         ss << "kernel_concat_byte_" << dtype_bytes(c->getAttrOprand("operand:0").dtype) << "_axis_"
            << c->getAttrInt("axis");
@@ -514,6 +528,8 @@ struct ResizeKernel : KernelFuncBase {
                 (imode == "NEAREST" && fmt == "NCHW"));
     }
     std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)  // name filtering without a context (KernelGen.cpp:49-53)
+            return "kernel_resize_linear";
         const std::string imode = c->getAttrStr("imode");
         return std::string(imode == "LINEAR" ? "GI_" : "") + "kernel_resize_linear_" +
                c->getAttrStr("format") + "_" + imode + "_" + c->getAttrOprand("operand:0").dtype;
@@ -596,6 +612,8 @@ struct FusedElemwiseKernel : KernelFuncBase {
         return true;
     }
     std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)  // name filtering without a context (KernelGen.cpp:49-53)
+            return "kernel_fused_elemwise";
         const int steps = c->getAttrInt("modes:size"), nr = c->getAttrInt("nr_operands");
         const CCOperand dst = c->getAttrOprand("operand:" + std::to_string(nr - 1));
         std::stringstream ss;
@@ -644,6 +662,8 @@ struct MatrixMulKernel : KernelFuncBase {
                (!c->haveAttr("compute_mode") || c->getAttrStr("compute_mode") == "DEFAULT");
     }
     std::string GetKernelSymbol(TContext* c) const override {
+        if (!c)  // name filtering without a context (KernelGen.cpp:49-53)
+            return "kernel_matmul";
         return std::string("kernel_matmul_") + (c->getAttrBool("transposeA") ? "t" : "n") +
                (c->getAttrBool("transposeB") ? "t" : "n") + "_" +
                c->getAttrOprand("operand:0").dtype;

@@ -50,10 +50,6 @@ static CCOperand parse_operand(const std::string& v) {
 }
 
 int main(int argc, char** argv) {
-    if (argc != 3) {
-        fprintf(stderr, "usage: %s <spec-file> <outdir>\n", argv[0]);
-        return 2;
-    }
     static const std::map<std::string, KernType> types = {
             {"ConvKernel", KernType::ConvKernel},
             {"ElemwiseKernel", KernType::ElemwiseKernel},
@@ -67,6 +63,17 @@ int main(int argc, char** argv) {
             {"ResizeKernel", KernType::ResizeKernel},
             {"FusedElemwiseKernel", KernType::FusedElemwiseKernel},
     };
+    if (argc == 2 && std::string(argv[1]) == "--null-symbols") {
+        // what every kernel answers to the exporter's name filter, which has no context
+        for (auto& t : types)
+            for (auto* k : Gfx950KernelPack::GetKernel(t.second))
+                printf("%s\n", k->GetKernelSymbol(nullptr).c_str());
+        return 0;
+    }
+    if (argc != 3) {
+        fprintf(stderr, "usage: %s <spec-file> <outdir> | --null-symbols\n", argv[0]);
+        return 2;
+    }
     std::ifstream spec(argv[1]);
     if (!spec) {
         fprintf(stderr, "cannot read %s\n", argv[1]);

@@ -46,6 +46,42 @@ def test_quantized_symbols_equal_the_reference_registry(emitted):
     assert checked >= 35
 
 
+REFERENCE = "/root/reference"
+
+
+@pytest.mark.skipif(not os.path.isdir(os.path.join(REFERENCE, "compiler", "lib", "KernelGen")),
+                    reason="needs the reference tree (its headers and its KernelGen registry)")
+def test_target_builds_against_the_reference_headers_and_agrees_with_its_registry():
+    """Gfx950Kernels.cpp compiled with -DMEGCC_GFX950_IN_TREE derives from the reference's own
+    KernelFunc and reads its TContext; oracle/ref_intree_check.cpp then asks both registries for
+    every operator of the spec: each gfx950 symbol must be the symbol of an available
+    Arch::BAREMETAL kernel for the same context, the texts must be produced from the reference's
+    attribute bag without a missing key, the workspace text must be self-contained C, and
+    GetKernelSymbol(nullptr) must return for every kernel."""
+    oracle = os.path.join(ROOT, "oracle")
+    subprocess.check_call(["make", "-s", "-C", oracle, "REF=" + REFERENCE, "_ref/intree_check"])
+    r = subprocess.run([os.path.join(oracle, "_ref", "intree_check"),
+                        os.path.join(oracle, "ref_kernels.spec")], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-1000:]
+    summary = dict(kv.split("=") for kv in r.stdout.strip().splitlines()[-1].split()[1:])
+    assert int(summary["failed"]) == 0
+    assert int(summary["lines"]) >= 250
+    # every quantised operator is named exactly as the x86 build's first choice
+    for line in r.stdout.splitlines():
+        f = line.split()
+        if f[0] == "ok" and "qsi" in f[2]:
+            assert f[3] == "first", line
+
+
+def test_symbol_without_a_context(emitted):
+    """The exporter filters kernels by name with a null context (KernelGen.cpp:49-53)."""
+    r = subprocess.run([os.path.join(KG, "kernelgen_tool"), "--null-symbols"],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    names = r.stdout.split()
+    assert len(names) >= 11 and all(n.startswith(("kernel_", "GI_kernel_")) for n in names)
+
+
 def test_library_resolves_every_emitted_symbol(emitted):
     _, manifest = emitted
     for sym in set(manifest.values()):

@@ -28,6 +28,7 @@ bool conv_first_supported(const ConvGeom& g);
 TinyNNStatus conv_first_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool dwconv44_supported(const ConvGeom& g);
 TinyNNStatus dwconv44_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+void dwconv44_note(const ConvGeom&, const void* src, const void* dst);
 bool conv_f32_small_supported(const ConvGeom& g);
 TinyNNStatus conv_f32_small_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool conv_f32_gemm_supported(const ConvGeom& g);
@@ -413,7 +414,7 @@ static TinyNNStatus conv2d_run(
     }
     if (q8 && dwconv44_supported(g) && aligned4(src->ptr) && aligned4(flt->ptr) &&
         aligned4(dst->ptr)) {
-        note_kernel("dwconv44");
+        dwconv44_note(g, src->ptr, dst->ptr);
         return dwconv44_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     }
     if (q8 && conv_first_supported(g) && aligned4(src->ptr) && aligned4(dst->ptr) && (!b || aligned4(b))) {

@@ -108,12 +108,15 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
         const int n = fdiv(r2, d_c4n), c4 = r2 - n * c4n;
         const int plane_off = ((n * c4n + c4) * g.ih) * g.iw * 4;  // bytes
         // weights: per filter row one dword per channel = (w(fw=0), w(fw=1), w(fw=2), 0)
-        unsigned wq[3][4];
+        unsigned wq[3][4], ws[3][4];  // ws: (0, w0, w1, w2), for the odd outputs of stride 2
 #pragma unroll
         for (int fh = 0; fh < 3; ++fh) {
             const uint32_t* f = flt + (size_t)c4 * 9 + fh * 3;
             const dw_v4u fv = {f[0], f[1], f[2], 0u};
             transpose4x4(fv, wq[fh]);
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                ws[fh][c] = wq[fh][c] << 8;
         }
         int acc[R * 16];  // [row][pixel][channel]
         {
@@ -170,10 +173,12 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
                 transpose4x4(l1, t1);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
+                    // outputs 1 and 3 read bytes 1-3 of t0 / t1: they meet the weights moved up a
+                    // byte (SHIFTED below) instead of being shifted themselves
                     win[0][c] = __builtin_amdgcn_perm(t0[c], pv, 0x06050400u | c);
-                    win[1][c] = t0[c] >> 8;
+                    win[1][c] = t0[c];
                     win[2][c] = __builtin_amdgcn_alignbyte(t1[c], t0[c], 3);
-                    win[3][c] = t1[c] >> 8;
+                    win[3][c] = t1[c];
                 }
             }
             // input row ir is filter row ir - orow * S of output row orow
@@ -187,7 +192,8 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
 #pragma unroll
                     for (int c = 0; c < 4; ++c)
                         acc[orow * 16 + j * 4 + c] = __builtin_amdgcn_sdot4(
-                                (int)win[j][c], (int)wq[fh][c], acc[orow * 16 + j * 4 + c], false);
+                                (int)win[j][c], (int)(S == 2 && (j & 1) ? ws[fh][c] : wq[fh][c]),
+                                acc[orow * 16 + j * 4 + c], false);
             }
         }
         if (ACT < 0) {
@@ -235,16 +241,43 @@ bool dwconv44_supported(const ConvGeom& g) {
            (g.ic & 3) == 0;
 }
 
+bool dwconv44_mfma_supported(const ConvGeom& g, const void* src, const void* dst);
+TinyNNStatus dwconv44_mfma_launch(
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, void* dst);
+
+// the matrix-core kernel (dwconv_mfma.hip) for stride 1, where the vector ALU is the limit
+static bool use_mfma(const ConvGeom& g, const void* src, const void* dst) {
+    return dwconv44_mfma_supported(g, src, dst) && !options().no_dwmfma && !options().dw_generic;
+}
+
+// which kernel dwconv44_launch picks: (pixels per thread and row) << 4 | rows per thread
+static int dwconv44_shape(const ConvGeom& g, const void* src, const void* dst) {
+    if (!dwconv44_3x3_ok(g, src, dst) || options().dw_generic)
+        return 1 << 4 | 1;
+    return 4 << 4 | (g.sh == 1 && g.oh >= 28 ? 2 : 1);
+}
+
+// records the kernel dwconv44_launch runs for this layer
+void dwconv44_note(const ConvGeom& g, const void* src, const void* dst) {
+    if (use_mfma(g, src, dst))
+        note_kernel("dwconv44_mfma");
+    else  // pixels per thread and row (4: the 3x3 kernels, 1: the generic one), rows per thread
+        note_kernel("dwconv44", dwconv44_shape(g, src, dst) >> 4, dwconv44_shape(g, src, dst) & 15);
+}
+
 TinyNNStatus dwconv44_launch(
         const ConvGeom& g, const void* src, const void* flt, const void* bias, void* dst) {
     size_t total = (size_t)g.n * (g.oc >> 2) * g.oh * g.ow;
     if (total == 0)
         return TinyNN_SUCCESS;
-    if (dwconv44_3x3_ok(g, src, dst) && !options().dw_generic) {
+    if (use_mfma(g, src, dst))
+        return dwconv44_mfma_launch(g, src, flt, bias, dst);
+    const int shape = dwconv44_shape(g, src, dst);
+    if (shape >> 4 == 4) {
         // one thread per R output rows x 4 output pixels x 4 channels
         // (two rows share input rows and the weight set-up: measured faster for stride 1 on
         // large planes only)
-        const int R = g.sh == 1 && g.oh >= 28 ? 2 : 1;
+        const int R = shape & 15;
         const int groups4 = (int)((long)g.n * (g.oc >> 2) * ((g.oh + R - 1) / R) * ((g.ow + 3) / 4));
         unsigned nb = (unsigned)((groups4 + 255) / 256);
         const RequantFast rq3 = make_requant_fast(g.s_src, g.s_flt, g.s_dst);

@@ -1,0 +1,294 @@
+// qsi8 depthwise 3x3 (pad 1, stride 1 or 2) in NCHW44 on the matrix cores.
+//
+// A depthwise layer moves two bytes per output and has to requantise every output exactly, which
+// costs 7 vector instructions and a table look-up (epilogue.h). Done with v_dot4 the multiply-adds
+// and the byte shuffling in front of them cost another 10 vector instructions per output, and the
+// layer is bound by the vector ALU at a third of the memory rate. Here the multiply-adds go to the
+// MFMA unit, which is otherwise idle, as a product with a banded matrix:
+//
+//   for one group of 4 channels (one NCHW44 plane set) and one filter row dy,
+//     D[(px, ch), col] += A_dy[(px, ch), (ipx, ich)] * B_dy[(ipx, ich), col]
+//   * a column is one group of 8 consecutive output pixels (image n, row y, pixels 8b .. 8b + 7)
+//     of the plane set; the 32 columns of a tile are 32 consecutive groups in (n, y, b) order,
+//     i.e. they walk along the rows;
+//   * K = 32 bytes = 8 consecutive input pixels x 4 channels exactly as they lie in memory, so the
+//     B operand of lane (col, K-half) is ONE aligned 16-byte load from input row y*S - 1 + dy, and
+//     the 64 lanes of a K step read one contiguous kilobyte (stride 1: column c + 1 continues
+//     where column c ends): no transposes, no shuffles, fully coalesced; rows above / below the
+//     image and pixel groups left / right of it are loaded with an out-of-range buffer offset and
+//     read as zero, which is the padding;
+//   * M = 32 = 8 output pixels x 4 channels; A_dy holds weight w[dy][fw][ch] where ich == ch and
+//     fw = ipx - (S * px - 1) is the filter column that connects input pixel ipx with output
+//     pixel px (0 <= fw <= 2), zero elsewhere. It only depends on the DISTANCE between the K
+//     step's first pixel and the tile's first pixel, so S + 1 matrices per filter row serve every
+//     tile of the layer; a wave builds them once from the 36 weight bytes of its plane set and
+//     keeps them in registers.
+//   A group of 8 output pixels from x0 on needs input pixels S*x0 - 1 .. S*x0 + 7*S + 1: S + 1
+//   aligned K steps of 8 pixels starting at S*x0 - 4, i.e. 3 * (S + 1) MFMAs per tile of
+//   32 groups x 8 pixels x 4 channels. The accumulators start from the bias through the MFMA's C
+//   operand.
+//
+// The 1/32 utilisation of the band is irrelevant: 3 * (S + 1) MFMAs per 1024 outputs is 0.2
+// cycles per output and SIMD, against 28 cycles for the exact epilogue.
+//
+// Accumulator register e of lane (col, h) is output pixel 2 * (e / 4) + h, channel e % 4: four
+// consecutive registers pack into the NCHW44 dword of one pixel, and two v_permlane32_swap hand the
+// odd pixels of the lower half wave to the upper one and back, after which every lane owns 4
+// consecutive pixels = one 16-byte store, the 64 stores of a wave again one contiguous kilobyte.
+//
+// Same arithmetic as the reference's loop (BareMetal/ConvKernel.cpp:305-344,374-380): int32
+// accumulators over the in-bounds taps plus the bias, then the exact requantisation (epilogue.h).
+#include "common.h"
+#include "conv_geom.h"
+#include "conv_mfma_i8.h"
+#include "epilogue.h"
+
+namespace mg {
+
+struct DwMfmaParams {
+    const uint32_t* src;
+    const uint32_t* flt;   // [C/4][3][3] dwords of 4 channel bytes
+    const int32_t* bias;   // or nullptr
+    uint32_t* dst;
+    int src_bytes;
+    int c4n, ih, iw, oh, ow;
+    int dst_bytes;
+    int ohp;               // ceil(OH / R): row groups per image
+    int cols;              // N * ohp * xblocks: (row group, 8 output pixels) pairs per plane set
+    int xblocks;           // ceil(OW / 8)
+    int tiles;             // per plane set: ceil(cols / 32)
+    int act;
+    float s_src, s_flt, s_dst, c;
+    FastDiv d_ohp, d_xb;  // division by ohp, by xblocks
+    RequantTable table;
+};
+
+typedef unsigned dwm_v2u __attribute__((ext_vector_type(2)));
+typedef unsigned dw_v4u __attribute__((ext_vector_type(4)));
+// output rows per lane and tile (2 share input rows and index arithmetic but need 200 registers:
+// measured 15.3 us against 14.9 us with 1 on N=64 C=32 112x112)
+static constexpr int DWM_ROWS = 1;
+
+// S: stride (only 1 is instantiated: with stride 2 the layer reads four bytes per byte written and
+// the v_dot4 kernel of dwconv.hip already runs at the rate of a copy - measured 7.8 us against
+// 9.8 us for this one on N=64 C=32 112x112). RAGGED: IW is not a multiple of 4, so the last 16-byte load of a row runs into the
+// next row and is masked. ACT: IDENTITY / RELU use the threshold table, -1 evaluates the literal
+// sequence with the run-time activation.
+template <int S, bool RAGGED, int ACT>
+__global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
+    constexpr int NS = S + 1;            // K steps a group of 8 output pixels reads
+    constexpr int R = DWM_ROWS;          // output rows per lane and tile
+    constexpr int IR = (R - 1) * S + 3;  // input rows they read
+    __shared__ int tbl[REQUANT_TABLE_ENTRIES];
+    const int tid = threadIdx.x, lane = tid & 63;
+    if (ACT >= 0) {
+        tbl[tid] = q.table.t[tid];
+        __syncthreads();
+    }
+    const int col_l = lane & 31, kg = lane >> 5;
+    // wave -> (plane set, first tile, tile step): the grid holds a multiple of c4n waves
+    const int gw = blockIdx.x * 4 + (tid >> 6);
+    const int nw = gridDim.x * 4;
+    const int c4 = gw % q.c4n;
+    const int tstep = nw / q.c4n;
+
+    // ---- the banded weight matrices of this plane set -------------------------------------------
+    // row m = lane & 31 = (output pixel m / 4, channel m % 4); the lane's 16 K bytes are input
+    // pixels 4 * kg + j (j = 0..3) of the K step, 4 channel bytes each. K step s starts 4 pixels
+    // left of S * x0, so input pixel (s, j) meets output pixel px through filter column
+    // fw = 8 * s + 4 * kg + j - 4 - S * px + 1.
+    v4i A[3][NS];
+    {
+        const int px = col_l >> 2, ch = col_l & 3;
+        const unsigned keep = 0xffu << (8 * ch);
+        const uint32_t* w = q.flt + (size_t)c4 * 9;
+#pragma unroll
+        for (int dy = 0; dy < 3; ++dy) {
+            const unsigned w0 = w[dy * 3] & keep, w1 = w[dy * 3 + 1] & keep, w2 = w[dy * 3 + 2] & keep;
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int fw = 8 * s + 4 * kg + j - 3 - S * px;
+                    A[dy][s][j] = (int)(fw == 0 ? w0 : fw == 1 ? w1 : fw == 2 ? w2 : 0u);
+                }
+        }
+    }
+    v16i biasv;
+    {
+        int b4[4] = {0, 0, 0, 0};
+        if (q.bias) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                b4[c] = q.bias[c4 * 4 + c];
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            biasv[e] = b4[e & 3];
+    }
+    const __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc((void*)q.src, 0, q.src_bytes, 0x00020000);
+    const int OOB = (int)0x80000000u;
+
+    const __amdgpu_buffer_rsrc_t rd =
+            __builtin_amdgcn_make_buffer_rsrc((void*)q.dst, 0, q.dst_bytes, 0x00020000);
+    // where a lane's results go: byte offset of its 4 pixels in output row y, pixels left in the
+    // row (<= 0: nothing to store), rows left in the image
+    struct Where {
+        int off, left, rows;
+    };
+    // requests the B operands of a tile: NS aligned 16-byte loads for each of the IR input rows
+    auto request = [&](int tile, v4i (&B)[IR][NS]) __attribute__((always_inline)) -> Where {
+        const int col = tile * 32 + col_l;
+        const bool col_ok = col < q.cols && tile < q.tiles;
+        const int rg = fdiv(col, q.d_xb), x0 = (col - rg * q.xblocks) * 8;
+        const int n = fdiv(rg, q.d_ohp), y = (rg - n * q.ohp) * R;
+        const int pset = n * q.c4n + c4;
+        const int base = pset * q.ih * q.iw;   // first pixel of the input plane set
+        const int ix0 = S * x0 - 4 + 4 * kg;   // this lane's first input pixel of K step 0
+#pragma unroll
+        for (int ir = 0; ir < IR; ++ir) {
+            const int iy = y * S - 1 + ir;
+            const bool row_ok = col_ok && (unsigned)iy < (unsigned)q.ih;
+            const int row_off = base + __mul24(iy, q.iw);
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const int ix = ix0 + 8 * s;
+                const bool ok = row_ok && (unsigned)ix < (unsigned)q.iw;
+                B[ir][s] = __builtin_bit_cast(
+                        v4i, __builtin_amdgcn_raw_buffer_load_b128(rs, ok ? (row_off + ix) * 4 : OOB, 0, 0));
+                if (RAGGED) {
+#pragma unroll
+                    for (int j = 1; j < 4; ++j)
+                        B[ir][s][j] = ix + j < q.iw ? B[ir][s][j] : 0;
+                }
+            }
+        }
+        Where w;
+        const int xo = x0 + 4 * kg;  // after the exchange this lane stores pixels xo .. xo + 3
+        w.off = ((pset * q.oh + y) * q.ow + xo) * 4;
+        w.left = col_ok ? q.ow - xo : 0;
+        w.rows = q.oh - y;
+        return w;
+    };
+
+    v4i B[IR][NS];
+    int tile = gw / q.c4n;
+    Where next = request(tile, B);
+    for (; tile < q.tiles; tile += tstep) {
+        const Where cur = next;
+        v16i acc[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            acc[r] = biasv;
+#pragma unroll
+            for (int dy = 0; dy < 3; ++dy)
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                    acc[r] = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[dy][s], B[r * S + dy][s], acc[r], 0, 0, 0);
+        }
+        // the operands are consumed: the next tile's loads fly while this one is requantised
+        // (past the last tile every offset is out of range and nothing is fetched)
+        next = request(tile + tstep, B);
+        // ---- requantise, pack, exchange, store ---------------------------------------------------
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int o[16];
+            if (ACT < 0) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    o[e] = requant_conv_rt(q.act, acc[r][e], q.s_src, q.s_flt, q.s_dst);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    o[e] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[r][e], q.c, tbl);
+            }
+            unsigned d[4];  // pixel 2 * j + kg
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                d[j] = pack4_perm(o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]);
+            // lower half wave: pixels 0 2 4 6, upper: 1 3 5 7  ->  lower 0 1 2 3, upper 4 5 6 7
+            const dwm_v2u s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+            const dwm_v2u s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+            const dw_v4u px4 = {s02[0], s02[1], s13[0], s13[1]};
+            const int left = r < cur.rows ? cur.left : 0;
+            const int off = cur.off + r * q.ow * 4;
+            if ((q.ow & 3) == 0) {
+                __builtin_amdgcn_raw_buffer_store_b128(px4, rd, left >= 4 ? off : OOB, 0, 0);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    __builtin_amdgcn_raw_buffer_store_b32(px4[j], rd, left > j ? off + 4 * j : OOB, 0, 0);
+            }
+        }
+    }
+}
+
+bool dwconv44_mfma_supported(const ConvGeom& g, const void* src, const void* dst) {
+    const long src_bytes = (long)g.n * g.ic * g.ih * g.iw;
+    return g.fmt == MEGCC_FMT_NCHW44 && g.groups > 1 && g.groups == g.ic && g.ic == g.oc &&
+           (g.ic & 3) == 0 && g.fh == 3 && g.fw == 3 && g.ph == 1 && g.pw == 1 && g.dh == 1 &&
+           g.dw == 1 && g.sh == 1 && g.sw == 1 && ((uintptr_t)src & 15) == 0 &&
+           ((uintptr_t)dst & 15) == 0 && src_bytes < (1L << 31) &&
+           (long)g.n * g.oc * g.oh * g.ow < (1L << 31) && (long)g.n * g.oh * ((g.ow + 7) / 8) < (1L << 30) && (long)g.ih * g.iw < (1L << 24);
+}
+
+TinyNNStatus dwconv44_mfma_launch(
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, void* dst) {
+    DwMfmaParams q = {};
+    q.src = (const uint32_t*)src;
+    q.flt = (const uint32_t*)flt;
+    q.bias = (const int32_t*)bias;
+    q.dst = (uint32_t*)dst;
+    q.src_bytes = (int)((long)g.n * g.ic * g.ih * g.iw);
+    q.c4n = g.ic >> 2;
+    q.ih = g.ih;
+    q.iw = g.iw;
+    q.oh = g.oh;
+    q.ow = g.ow;
+    q.dst_bytes = (int)((long)g.n * g.oc * g.oh * g.ow);
+    q.xblocks = (g.ow + 7) / 8;
+    q.ohp = (g.oh + DWM_ROWS - 1) / DWM_ROWS;
+    q.cols = g.n * q.ohp * q.xblocks;
+    q.tiles = (q.cols + 31) / 32;
+    q.act = g.act;
+    q.s_src = g.s_src;
+    q.s_flt = g.s_flt;
+    q.s_dst = g.s_dst;
+    q.c = make_requant_fast(g.s_src, g.s_flt, g.s_dst).c;
+    q.d_ohp = make_fastdiv(q.ohp);
+    q.d_xb = make_fastdiv(q.xblocks);
+    if ((long)q.tiles * q.c4n == 0)
+        return TinyNN_SUCCESS;
+    const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
+                     requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    if (tab)
+        q.table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
+    const int act = tab ? g.act : -1;
+    const bool ragged = (g.iw & 3) != 0;
+    const void* kern = nullptr;
+#define MG_DWM_ACT(S_, R_)                                                                      \
+    (act == MEGCC_NONLINE_IDENTITY ? (const void*)dwconv44_mfma_kernel<S_, R_, MEGCC_NONLINE_IDENTITY> \
+     : act == MEGCC_NONLINE_RELU   ? (const void*)dwconv44_mfma_kernel<S_, R_, MEGCC_NONLINE_RELU>     \
+                                   : (const void*)dwconv44_mfma_kernel<S_, R_, -1>)
+    kern = ragged ? MG_DWM_ACT(1, true) : MG_DWM_ACT(1, false);
+#undef MG_DWM_ACT
+    // one wave per (plane set, tile) while they are all resident at once, otherwise as many
+    // waves as are resident, each walking over the tiles of its plane set; the wave count is a
+    // multiple of the plane sets and of the 4 waves of a workgroup
+    const long items = (long)q.tiles * q.c4n;
+    const long cap = (long)num_cus() * 16;
+    long per_set = items <= cap ? q.tiles : cap / q.c4n;
+    if (per_set < 1)
+        per_set = 1;
+    long waves = per_set * q.c4n;
+    while (waves & 3) {  // (c4n odd: add whole rounds of plane sets until workgroups are full)
+        waves += q.c4n;
+    }
+    void* args[] = {&q};
+    hipError_t e = hipLaunchKernel(kern, dim3((unsigned)(waves / 4)), dim3(256), args, 0, stream());
+    MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "dwconv44_mfma: %s", hipGetErrorString(e));
+    return check_launch("dwconv44_mfma");
+}
+
+}  // namespace mg

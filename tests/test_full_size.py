@@ -203,7 +203,7 @@ def test_cfg4_chain_n64(c, hw, stride):
     dw = ConvCase(A.FMT_NCHW44, A.GROUP, n, c, hw, hw, c, 3, stride, 1, A.RELU, scales=(0.02, 0.01, 0.05))
     arrays = dw.gen(seed=7)
     y = run_gpu(dw, arrays)
-    assert runtime.last_kernel() == "dwconv44"
+    assert runtime.last_kernel().startswith("dwconv44")
     one = ConvCase(A.FMT_NCHW44, A.GROUP, 1, c, hw, hw, c, 3, stride, 1, A.RELU, scales=(0.02, 0.01, 0.05))
     for i in (0, 31, 63):
         want = one.run_port({"src": arrays["src"][i:i + 1], "flt": arrays["flt"], "bias": arrays["bias"]})

@@ -126,7 +126,15 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 11, 20, 8, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW44, A.GROUP, 2, 24, 13, 12, 24, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW44, A.GROUP, 1, 4, 5, 4, 4, 3, 1, 1, A.SIGMOID, scales=(0.02, 0.01, unsat(9) * 40)),
-    ConvCase(A.FMT_NCHW44, A.GROUP, 5, 12, 7, 7, 12, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),  # generic path
+    ConvCase(A.FMT_NCHW44, A.GROUP, 5, 12, 7, 7, 12, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    # stride 1 on the matrix cores: rows that are not a multiple of 4 / 8 pixels (masked loads,
+    # dword stores), an odd number of plane sets, one pixel group per row, no bias, the literal
+    # epilogue, 13 rows x 3 groups x 2 images = 78 columns (a ragged last tile)
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 20, 13, 18, 20, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 3, 12, 6, 5, 12, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(9)), bias=False),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 1, 36, 17, 33, 36, 3, 1, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 7, 4, 3, 1, 4, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 1, 40, 8, 3, 1, 1, A.IDENTITY, scales=(0.5, 0.5, 0.5)),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 224, 224, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 3, 3, 64, 48, 24, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(27))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 32, 36, 8, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(27))),
@@ -467,6 +475,13 @@ OLDER = [
                                  scales=(0.02, 0.01, unsat(512)))),
     ("nopws", ConvCase(A.FMT_NCHW44, A.DENSE, 11, 64, 56, 56, 128, 1, 1, 0, A.IDENTITY,
                              scales=(0.02, 0.01, unsat(64)))),
+    # stride-1 depthwise on the v_dot4 kernels (two rows per thread on large planes, one on small)
+    ("nodwmfma", ConvCase(A.FMT_NCHW44, A.GROUP, 2, 32, 112, 112, 32, 3, 1, 1, A.RELU,
+                          scales=(0.02, 0.01, unsat(9)))),
+    ("nodwmfma", ConvCase(A.FMT_NCHW44, A.GROUP, 3, 16, 9, 28, 16, 3, 1, 1, A.IDENTITY,
+                          scales=(0.02, 0.01, unsat(9)))),
+    ("nodwmfma", ConvCase(A.FMT_NCHW44, A.GROUP, 5, 12, 7, 7, 12, 3, 1, 1, A.H_SWISH,
+                          scales=(0.02, 0.01, unsat(9)))),
 ]
 
 

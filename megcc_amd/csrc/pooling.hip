@@ -9,6 +9,7 @@
 // NCHW  : one thread per output byte, lanes walk W.
 #include "common.h"
 #include "epilogue.h"
+#include "fastdiv.h"
 
 namespace mg {
 
@@ -167,6 +168,47 @@ __global__ void __launch_bounds__(256) pool_nchw_max2x2_kernel(
     dst[i] = pack4(o[0], o[1], o[2], o[3]);
 }
 
+// MAX 2x2 stride 2 without padding on NCHW44 (the pooling of the depthwise -> pool -> add chain):
+// a thread makes 4 neighbouring output pixels = one 16-byte store from 8 input pixels of each of
+// the two input rows (four 16-byte loads). The maximum per channel byte is taken on packed 16-bit
+// halves: a dword of 4 signed bytes is split into its even bytes (shift left, arithmetic shift
+// right, both packed) and its odd bytes (arithmetic shift right), the four window positions meet
+// in v_pk_max_i16, and one v_perm puts the low bytes of the two results back together:
+// 20 vector instructions per output dword instead of 40 byte extractions and maxima, and no
+// division in the index arithmetic beyond two by run-time constants. Needs IW % 8 == 0.
+typedef short pool_s2 __attribute__((ext_vector_type(2)));
+typedef unsigned pool_v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ unsigned max4_bytes(unsigned a, unsigned b, unsigned c, unsigned d) {
+    auto even = [](unsigned v) { return (__builtin_bit_cast(pool_s2, v) << 8) >> 8; };
+    auto odd = [](unsigned v) { return __builtin_bit_cast(pool_s2, v) >> 8; };
+    const pool_s2 e = __builtin_elementwise_max(__builtin_elementwise_max(even(a), even(b)),
+                                                __builtin_elementwise_max(even(c), even(d)));
+    const pool_s2 o = __builtin_elementwise_max(__builtin_elementwise_max(odd(a), odd(b)),
+                                                __builtin_elementwise_max(odd(c), odd(d)));
+    // bytes: e.lo, o.lo, e.hi, o.hi
+    return __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, o), __builtin_bit_cast(unsigned, e), 0x06020400u);
+}
+
+__global__ void __launch_bounds__(256) pool44_max2x2_kernel(
+        const pool_v4u* __restrict__ src, pool_v4u* __restrict__ dst, unsigned total, FastDiv d_ow4,
+        int ow4) {
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;  // (plane set, oh, group of 4 ow)
+    if (i >= total)
+        return;
+    const unsigned row = fdiv(i, d_ow4), q = i - row * (unsigned)ow4;
+    // an input row is 2 * ow4 16-byte words; output row `row` (over all plane sets: IH = 2 * OH)
+    // reads input rows 2 * row and 2 * row + 1
+    const size_t in = (size_t)row * 4 * ow4 + 2 * q;
+    const pool_v4u a0 = src[in], a1 = src[in + 1], b0 = src[in + 2 * ow4], b1 = src[in + 2 * ow4 + 1];
+    pool_v4u o;
+    o[0] = max4_bytes(a0[0], a0[1], b0[0], b0[1]);
+    o[1] = max4_bytes(a0[2], a0[3], b0[2], b0[3]);
+    o[2] = max4_bytes(a1[0], a1[1], b1[0], b1[1]);
+    o[3] = max4_bytes(a1[2], a1[3], b1[2], b1[3]);
+    dst[i] = o;
+}
+
 }  // namespace mg
 
 using namespace mg;
@@ -222,6 +264,16 @@ extern "C" TinyNNStatus megcc_gfx950_pooling(
             unsigned blocks = min(ceil_div((size_t)planes, 32), 1u << 16);
             hipLaunchKernelGGL(pool44_global_q8_kernel, dim3(blocks), dim3(256), 0, stream(), g,
                                (const uint32_t*)src->ptr, (uint32_t*)dst->ptr, (int)planes);
+            return check_launch("pooling");
+        }
+        if (g.mode == MEGCC_POOL_MAX && g.wh == 2 && g.ww == 2 && g.sh == 2 && g.sw == 2 && g.ph == 0 &&
+            g.pw == 0 && (g.iw & 7) == 0 && (g.ih & 1) == 0 && ((uintptr_t)src->ptr & 15) == 0 &&
+            ((uintptr_t)dst->ptr & 15) == 0 && total / 16 < (1ull << 31)) {
+            const unsigned items = (unsigned)(total / 16);  // 4 pixels x 4 channels each
+            hipLaunchKernelGGL(pool44_max2x2_kernel, dim3((items + 255) / 256), dim3(256), 0, stream(),
+                               (const pool_v4u*)src->ptr, (pool_v4u*)dst->ptr, items,
+                               make_fastdiv(g.ow / 4), g.ow / 4);
+            note_kernel("pool44_max2x2");
             return check_launch("pooling");
         }
         unsigned blocks = min(ceil_div(total / 4, 256), 1u << 20);

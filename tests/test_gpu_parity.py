@@ -140,6 +140,11 @@ LIVE = [
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 32, 36, 8, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(27))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 30, 34, 8, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),  # generic path (IW % 4 != 0)
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
+    # the 2x2 stride-2 maximum on packed halves (rows of 8, 16 pixels), and rows it does not take
+    PoolCase(A.FMT_NCHW44, A.POOL_MAX, 3, 12, 6, 8, 2, 2, 0),
+    PoolCase(A.FMT_NCHW44, A.POOL_MAX, 1, 4, 2, 16, 2, 2, 0),
+    PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 8, 6, 12, 2, 2, 0),
+    PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 8, 7, 16, 2, 2, 0),
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 3, 5, 10, 24, 2, 2, 0),   # 8-byte row pieces, odd plane count
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 3, 5, 11, 24, 2, 2, 0),   # odd height: the generic kernel

@@ -133,6 +133,10 @@ def make_workload(name):
     if name == "concat":
         return (ConcatCase("qsi8", [(32, 32, 56, 56, 4), (32, 32, 56, 56, 4)], 1),
                 "qsi8 concat of two N=32 C=128 56x56 NCHW44 maps along C", "hbm")
+    if name.startswith("conv:"):  # conv:N,C,HW - any shape of the qsi8 3x3 configuration
+        n, c, hw = (int(v) for v in name[5:].split(","))
+        return (headline_case(n, c, hw),
+                "qsi8 conv3x3 s1 p1 NCHW44 N=%d Cin=Cout=%d %dx%d +bias +ReLU requant" % (n, c, hw, hw), "mfma")
     if name == "conv":
         case = headline_case()
         return case, "qsi8 conv3x3 s1 p1 NCHW44 N=32 Cin=Cout=256 56x56 +bias +ReLU requant", "mfma"
@@ -271,6 +275,17 @@ def check_output(case, arrays, got):
             same(got[i:i + 1], want, "image / row %d of the output" % i)
         return "%s %s of %d against the oracle, bit for bit" % (
             "rows" if case.ih == 1 and case.fmt == 0 else "images", picks, case.n)
+    from cases import MatMulCase
+    if isinstance(case, MatMulCase):
+        # f32 MatMul: against the fp64 product of the first 64 rows. (The oracle's float32 running
+        # sum over K = 4096 is itself up to 1.2e-4 from the fp64 result, further than the GPU's
+        # tiled sums; tests/test_full_size.py compares all three.)
+        rows = min(case.m, 64)
+        a = arrays["a"].T if case.trans_a else arrays["a"]
+        b = arrays["b"].T if case.trans_b else arrays["b"]
+        want = (a[:rows].astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+        same(got[:rows], want, "rows 0..%d of the product" % (rows - 1))
+        return "rows 0..%d of %d against the fp64 product, 1e-4" % (rows - 1, case.m)
     if hasattr(case, "ops") and case.ops() > 4e10:
         return None  # (too large for the oracle in a benchmark run; covered by tests/test_full_size.py)
     same(got, case.run_port(arrays), "the output")
@@ -349,31 +364,50 @@ def case_bytes(case):
     return sum(s.nbytes for s in ins) + sum(s.nbytes for s in outs)
 
 
-def cpu_baseline(full_case, budget_s=20.0):
-    """One host core on a bounded slice of the same layer: batch 1 (of 32) of the headline conv."""
+def cpu_baseline(full_case, unit="TOP/s"):
+    """One host core on a bounded sample of the same workload, through the reference's own
+    generated kernel where oracle/_ref has it: batch 1 of a batched convolution, 64 rows of a
+    FullyConnected / MatMul with more (images and rows are independent in the reference's loops,
+    so the time of the whole workload is the sample's time times the stated factor)."""
+    import copy
     from oracle import port, ref
     import cases
-    from cases import ConvCase
-    if not isinstance(full_case, ConvCase) or full_case.sparse != 0 or full_case.fh != 3:
-        return None
-    sample = headline_case(1, full_case.ic, full_case.ih)
+    import config_cases
+    from cases import ConvCase, MatMulCase
+    sample, factor, what = full_case, 1, "the whole workload"
+    if isinstance(full_case, ConvCase):
+        fc = full_case.fmt == 0 and full_case.fh == 1 and full_case.ih == 1
+        keep = 64 if fc else 1
+        if full_case.n > keep:
+            sample = copy.copy(full_case)
+            sample.n = keep
+            factor = full_case.n / keep
+            what = "%s %d of %d" % ("rows" if fc else "batch", keep, full_case.n)
+    elif isinstance(full_case, MatMulCase) and full_case.m > 64:
+        sample = MatMulCase(64, full_case.k, full_case.n, full_case.trans_a, full_case.trans_b)
+        factor = full_case.m / 64
+        what = "rows 64 of %d" % full_case.m
     arrays = sample.gen(seed=0)
-    use_ref = ref.available() and ref.has(sample.symbol())
+    try:
+        symbol = config_cases.ref_symbol(sample)
+    except AssertionError:
+        symbol = sample.symbol()
+    use_ref = ref.available() and ref.has(symbol)
     port.set_threads(1)
     t0 = time.perf_counter()
     if use_ref:
-        cases.run_ref(sample, arrays)
+        cases.run_ref(sample, arrays, symbol)
     else:
         sample.run_port(arrays)
     dt = time.perf_counter() - t0
+    work = sample.ops() if unit != "GB/s" and hasattr(sample, "ops") else case_bytes(sample)
     return {
-        "value": round(sample.ops() / dt / 1e12, 6), "unit": "TOP/s", "cores": 1,
+        "value": round(work / dt / (1e9 if unit == "GB/s" else 1e12), 6), "unit": unit, "cores": 1,
         "kind": "reference" if use_ref else "port",
-        "sample": "batch 1 of 32 of the same layer (N=1 Cin=Cout=%d %dx%d, %.2f GOP) timed once "
-                  "in %.2f s; %s" % (
-                      sample.ic, sample.ih, sample.iw, sample.ops() / 1e9, dt,
-                      "MegCC's generated kernel %s built with -O3 -fno-finite-math-only" %
-                      sample.symbol() if use_ref else "oracle/oracle_port.c built with -O2"),
+        "sample": "%s, timed once in %.3f s (the whole workload at that rate: %.2f s); %s" % (
+            what, dt, dt * factor,
+            "MegCC's generated kernel %s built with -O3 -fno-finite-math-only" % symbol
+            if use_ref else "oracle/oracle_port.c built with -O2"),
         "host_cores": os.cpu_count(),
     }
 
@@ -389,6 +423,8 @@ def main():
                     help="untimed launches of the same operator before the warm-up steps, for this long")
     ap.add_argument("--workload", default="conv")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--cpu", action="store_true",
+                    help="time the CPU baseline for this workload too (the default workload always does)")
     ap.add_argument("--batch", type=int, default=64, help="batch of the mobilenet workload")
     ap.add_argument("--per-layer", action="store_true")
     args = ap.parse_args()
@@ -471,6 +507,8 @@ def main():
         "checked": checked is not None, "checked_what": checked,
         "preheat_launches": preheat,
     }
+    if args.cpu and args.workload != "conv":
+        out["cpu_baseline"] = cpu_baseline(case, unit)
     if not args.no_cpu and args.workload == "conv":
         out["cpu_baseline"] = cpu_baseline(case)
         op = None

@@ -86,8 +86,14 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
         __syncthreads();
     }
     const int col_l = lane & 31, kg = lane >> 5;
+    // Workgroups are handed to the 8 XCDs in turn and every XCD has an L2 of its own: workgroup b
+    // takes the place b % 8 * (blocks / 8) + b / 8 in tile order, so that an XCD walks a contiguous
+    // eighth of the tiles and the input rows that neighbouring tiles share are fetched into one
+    // L2 instead of two or three.
+    const int nb = gridDim.x;
+    const int lb = (nb & 7) == 0 ? (blockIdx.x & 7) * (nb >> 3) + (blockIdx.x >> 3) : blockIdx.x;
     // wave -> (plane set, first tile, tile step): the grid holds a multiple of c4n waves
-    const int gw = blockIdx.x * 4 + (tid >> 6);
+    const int gw = lb * 4 + (tid >> 6);
     const int nw = gridDim.x * 4;
     const int c4 = gw % q.c4n;
     const int tstep = nw / q.c4n;

@@ -43,22 +43,23 @@ PEAK_INT8_TOPS = 5000.0  # dense int8 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of a workload's dominant kernel come from the committed rocprofv3 --pmc
 # summaries (FETCH_SIZE / WRITE_SIZE in KiB per dispatch, scaled by what a 256 MiB copy reads on
-# the same counters); each summary ends in a line "TRAFFIC_BYTES_PER_LAUNCH=<n>".
-TRAFFIC_FILES = {"conv": "profiles/conv_mfma_i8_dma__conv3x3_n32_c256_56x56.txt"}
+# the same counters); a summary holds one line "TRAFFIC_BYTES_PER_LAUNCH[<workload>]=<n>" per
+# workload it covers.
+TRAFFIC_FILES = ["profiles/conv_mfma_i8_dma__conv3x3_n32_c256_56x56.txt",
+                 "profiles/cfg3_fc_matmul__all_shapes.txt", "profiles/cfg4_dw_pool_add__n64.txt"]
 
 
 def measured_traffic(workload):
     """(bytes per launch, file it was read from) or (None, None)"""
-    rel = TRAFFIC_FILES.get(workload)
-    if not rel:
-        return None, None
-    try:
-        with open(os.path.join(ROOT, rel)) as f:
-            for line in f:
-                if line.startswith("TRAFFIC_BYTES_PER_LAUNCH="):
-                    return int(line.split("=", 1)[1]), rel
-    except OSError:
-        pass
+    key = "TRAFFIC_BYTES_PER_LAUNCH[%s]=" % workload
+    for rel in TRAFFIC_FILES:
+        try:
+            with open(os.path.join(ROOT, rel)) as f:
+                for line in f:
+                    if line.startswith(key):
+                        return int(line.split("=", 1)[1]), rel
+        except OSError:
+            pass
     return None, None
 
 
@@ -404,7 +405,7 @@ def cpu_baseline(full_case, unit="TOP/s"):
     return {
         "value": round(work / dt / (1e9 if unit == "GB/s" else 1e12), 6), "unit": unit, "cores": 1,
         "kind": "reference" if use_ref else "port",
-        "sample": "%s, timed once in %.3f s (the whole workload at that rate: %.2f s); %s" % (
+        "sample": "%s, timed once in %.5f s (the whole workload at that rate: %.4g s); %s" % (
             what, dt, dt * factor,
             "MegCC's generated kernel %s built with -O3 -fno-finite-math-only" % symbol
             if use_ref else "oracle/oracle_port.c built with -O2"),

@@ -544,9 +544,15 @@ TinyNNStatus conv_mfma_launch(
         long ranges = slots / oc_tiles > 0 ? slots / oc_tiles : 1;
         range_len = ((P + ranges - 1) / ranges + 31) / 32 * 32;
         if (range_len < pc.bn / 2) {  // too few pixels per workgroup for the tile
-            if (pc.bm != 32)
+            if (pc.bm == 32)
+                range_len = pc.bn;  // the small-layer tiles: one tile per workgroup, not every CU busy
+            else if (pc.bn == 256 && P >= 4096)
+                // between the small-layer tiles and a full grid of 256-pixel tiles: half-filled
+                // tiles on part of the CUs (N=6, 128->128, 56x56: 9.4 us; the one-stage kernel
+                // these layers fell to: 20.8 us)
+                range_len = pc.bn / 2;
+            else
                 continue;
-            range_len = pc.bn;  // the small-layer tiles: one tile per workgroup, not every CU busy
         }
         t = plan_tiles(g, pc.bn, range_len, pc.pm);
         if (pc.fixed_lmax) {

@@ -431,10 +431,12 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok,
         // small 3x3 layers (batch 1): 32 oc x 128 px tiles of four waves, one 32 x 32 MFMA tile
         // each, so that a few thousand pixels still give every CU a workgroup; variant 6 with the
         // plane-major patch
-        // (only while the 128-channel tiles of the other variants would get fewer than 64 pixels per
-        //  CU: measured cross-over between 49 and 98)
+        // (only while the 128-channel tiles of the other variants would get fewer than 32 pixels per
+        //  CU: above that, half-filled 256-pixel tiles on part of the CUs are faster - N=3,
+        //  128->128, 56x56: 8.9 against 9.3 us, N=2, 256->256: 13.1 against 14.5 us; below, N=2,
+        //  128->128: 6.1 against 8.8 us; layers under 4096 pixels keep these tiles up to 64 per CU)
         if (!k3 || fc || g.fmt != MEGCC_FMT_NCHW44 || P < 512 ||
-            P * ((g.oc + 127) / 128) >= 64L * num_cus() || g.oc < 32 || (g.ic & 31) ||
+            P * ((g.oc + 127) / 128) >= (P >= 4096 ? 32L : 64L) * num_cus() || g.oc < 32 || (g.ic & 31) ||
             (long)g.n * g.oc * g.oh * g.ow >= (1L << 31))
             return false;
         const bool okt = requant_table_ok(g.s_src, g.s_flt, g.s_dst);

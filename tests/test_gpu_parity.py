@@ -88,7 +88,7 @@ LIVE = [
     # FullyConnected with an output width that is not a multiple of 4 (byte stores) and K % 128 != 0
     ConvCase(A.FMT_NCHW, A.DENSE, 9000, 160, 1, 1, 130, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(160) / 2)),
     ConvCase(A.FMT_NCHW, A.DENSE, 8300, 260, 1, 1, 256, 1, 1, 0, A.SIGMOID, scales=(0.01, 0.01, unsat(260) / 2)),
-    # few images at 56x56: too few output tiles for the LDS-direct kernel, the one-stage kernel runs
+    # few images at 56x56: between the small-layer tiles and a full grid (half-filled 256-pixel tiles)
     ConvCase(A.FMT_NCHW44, A.DENSE, 3, 64, 56, 56, 128, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(64))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 3, 32, 56, 56, 128, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(288))),
     # MobileNet pointwise shapes

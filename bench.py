@@ -107,6 +107,10 @@ def make_workload(name):
         case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 64, 32, 28, 28, 64, 5, 1, 2, abi.RELU,
                         scales=(0.02, 0.01, 0.05))
         return case, "qsi8 conv5x5 s1 p2 NCHW44 N=64 32->64 28x28", "mfma"
+    if name.startswith("conv_s2:"):  # conv_s2:N,C,HW - 3x3 stride 2 pad 1, Cin = Cout (down-sampling layers)
+        n, c, hw = (int(v) for v in name[8:].split(","))
+        case = ConvCase(abi.FMT_NCHW44, abi.DENSE, n, c, hw, hw, c, 3, 2, 1, abi.RELU, scales=(0.02, 0.01, 0.05))
+        return case, "qsi8 conv3x3 s2 p1 NCHW44 N=%d Cin=Cout=%d %dx%d +bias +ReLU requant" % (n, c, hw, hw), "mfma"
     if name == "pw_s2":
         case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 64, 256, 56, 56, 512, 1, 2, 0, abi.IDENTITY,
                         scales=(0.02, 0.01, 0.05))

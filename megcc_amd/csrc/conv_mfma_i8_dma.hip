@@ -486,6 +486,21 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok,
             *c = make_dma_config<3, 3, 1, 512, false, 2, 3, 2, 1, 2, false, true>(g.act, ok);
         return true;
     }
+    // 3x3 with stride 2 (down-sampling layers): the patch of a sub-tile holds four input pixels per
+    // output pixel, so the sub-tiles are smaller and the patches longer - 256 pixels in 1280 slots
+    // for large layers (variant 0), 128 pixels in 768 slots otherwise (variant 1). N=64, 128->128,
+    // 56x56: 17.1 us (the one-stage kernel: 29.4); 256->256, 28x28: 16.9 (36.9); 512->512, 14x14:
+    // 24.9 (40.9).
+    const bool k3s2 = k3 && g.sh == 2 && g.sw == 2 && !fc;
+    if (k3s2 && (variant == 0 || variant == 1)) {
+        if (g.oc < 128 || (variant == 0 && P < 32768))
+            return false;
+        if (variant == 0)
+            *c = make_dma_config<3, 3, 1, 1280, false, 2, 2>(g.act, ok);
+        else
+            *c = make_dma_config<3, 3, 1, 768, false, 2, 2, 2, 1, 1>(g.act, ok);
+        return true;
+    }
     if (variant == 0) {
         if (!k3)
             return false;

@@ -104,6 +104,12 @@ LIVE = [
     # 3x3 layers with 64..127 output channels on the LDS-direct kernel (64-channel tiles, one of them ragged)
     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 64, 40, 40, 64, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(576))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 9, 32, 31, 29, 96, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(288))),
+    # 3x3 stride 2 on the LDS-direct kernel: 128-pixel sub-tiles (ragged rows, sub-tiles that cross
+    # images), 256-pixel sub-tiles on a large layer, a ragged last channel tile, the literal epilogue
+    ConvCase(A.FMT_NCHW44, A.DENSE, 11, 64, 30, 27, 128, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(576))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 40, 32, 57, 60, 160, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(288))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 16, 96, 28, 28, 136, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(864))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 64, 128, 14, 14, 128, 3, 2, 1, A.RELU, scales=(0.02, 0.01, 0.05)),
     # split-K of the one-stage kernel where the stages do not divide by the split asked for
     # (8 stages, 100 tiles -> 6 slices asked, 4 slices of 2 stages run)
     ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 56, 56, 256, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(2304))),

@@ -175,6 +175,10 @@ def make_workload(name):
         case = ConvCase(abi.FMT_NCHW, abi.DENSE, 64, 4096, 1, 1, 4096, 1, 1, 0, abi.IDENTITY,
                         scales=(0.01, 0.01, 0.1))
         return case, "qsi8 FullyConnected 64x4096x4096", "hbm"
+    if name in ("dw_nchw", "dw_nchw_s2"):  # the depthwise layer of configs[3] on plain NCHW tensors
+        s = 2 if name.endswith("s2") else 1
+        case = ConvCase(abi.FMT_NCHW, abi.GROUP, 64, 32, 112, 112, 32, 3, s, 1, abi.RELU, scales=(0.02, 0.01, 0.05))
+        return case, "qsi8 depthwise 3x3 s%d NCHW N=64 C=32 112x112" % s, "hbm"
     if name.startswith("dw"):
         c, hw, s = {"dw": (32, 112, 1), "dw_s2": (32, 112, 2), "dw512": (512, 14, 1),
                     "dw512_s2": (512, 14, 2)}[name]

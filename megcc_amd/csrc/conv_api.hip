@@ -29,6 +29,8 @@ TinyNNStatus conv_first_launch(const ConvGeom&, const void*, const void*, const 
 bool dwconv44_supported(const ConvGeom& g);
 TinyNNStatus dwconv44_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 void dwconv44_note(const ConvGeom&, const void* src, const void* dst);
+bool dwconv_nchw_supported(const ConvGeom& g, const void* src, const void* dst);
+TinyNNStatus dwconv_nchw_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool conv_f32_small_supported(const ConvGeom& g);
 TinyNNStatus conv_f32_small_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool conv_f32_gemm_supported(const ConvGeom& g);
@@ -301,7 +303,9 @@ static TinyNNStatus conv2d_run(
         return TinyNN_SUCCESS;
     Workspace own = {nullptr, 0, 0};
     if (static_scratch) {
-        const size_t need = conv2d_scratch_bytes(g, q8, f32, packed);
+        // (the native kernel for channel-wise NCHW layers needs none)
+        const bool native_dw = q8 && dwconv_nchw_supported(g, src->ptr, dst->ptr) && !options().no_dwnchw;
+        const size_t need = native_dw ? 0 : conv2d_scratch_bytes(g, q8, f32, packed);
         MG_REQUIRE(need <= (size_t)MEGCC_GFX950_NOALLOC_SCRATCH_BYTES, TinyNN_ERROR_OUT_OF_RANGE,
                    "conv2d_noalloc: this layer needs %zu bytes of scratch memory, the static "
                    "buffer holds %zu; call megcc_gfx950_conv2d with a workspace instead",
@@ -382,6 +386,11 @@ static TinyNNStatus conv2d_run(
                            (!b || aligned4(b)),
                    TinyNN_ERROR_INVALID_LAYOUT, "conv2d: misaligned operand");
         return conv_mfma_launch(g, src->ptr, flt->ptr, b, dst->ptr, workspace);
+    }
+    // channel-wise 3x3 on plain NCHW planes whose rows are a multiple of 4 pixels: native kernel
+    if (q8 && dwconv_nchw_supported(g, src->ptr, dst->ptr) && !options().no_dwnchw) {
+        note_kernel("dwconv_nchw", g.sh);
+        return dwconv_nchw_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     }
     if (q8 && nchw_depthwise(g) && dwconv44_supported(as_nchw44(g)) && workspace && workspace->ptr &&
         workspace->size >= nchw_depthwise_bytes(g) && aligned16(workspace->ptr)) {

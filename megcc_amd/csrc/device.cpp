@@ -30,7 +30,7 @@ const OptionName kOptions[] = {
         {"nopwshare", &Options::no_pwshare}, {"nohybrid", &Options::no_hybrid},
         {"nodot4", &Options::no_dot4},       {"nof32small", &Options::no_f32small},
         {"dw_generic", &Options::dw_generic}, {"no_graph", &Options::no_graph},
-        {"nodwmfma", &Options::no_dwmfma},
+        {"nodwmfma", &Options::no_dwmfma},   {"nodwnchw", &Options::no_dwnchw},
 };
 struct KernelNote {
     const char* name;

@@ -408,6 +408,14 @@ NCHW_DW = [
     ConvCase(A.FMT_NCHW, A.GROUP, 3, 16, 29, 31, 16, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW, A.GROUP, 2, 8, 13, 17, 8, 5, 1, 2, A.H_SWISH, scales=(0.02, 0.01, unsat(25))),
     ConvCase(A.FMT_NCHW, A.GROUP, 2, 6, 9, 7, 6, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    # native NCHW kernel (rows of a multiple of 4 pixels): channel counts that are no multiple of 4,
+    # one group per row, output rows that are no multiple of 4 (byte stores), no bias, literal epilogue
+    ConvCase(A.FMT_NCHW, A.GROUP, 2, 6, 9, 8, 6, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW, A.GROUP, 3, 5, 11, 12, 5, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW, A.GROUP, 1, 3, 4, 4, 3, 3, 1, 1, A.IDENTITY, scales=(0.5, 0.5, 0.5), bias=False),
+    ConvCase(A.FMT_NCHW, A.GROUP, 2, 7, 17, 28, 7, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW, A.GROUP, 2, 33, 30, 44, 33, 3, 1, 1, A.RELU, scales=(0.02, 0.01, 0.05)),
+    ConvCase(A.FMT_NCHW, A.GROUP, 1, 2, 1, 4, 2, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
 ]
 
 
@@ -492,6 +500,9 @@ OLDER = [
     ("nodwmfma", ConvCase(A.FMT_NCHW44, A.GROUP, 3, 16, 9, 28, 16, 3, 1, 1, A.IDENTITY,
                           scales=(0.02, 0.01, unsat(9)))),
     ("nodwmfma", ConvCase(A.FMT_NCHW44, A.GROUP, 5, 12, 7, 7, 12, 3, 1, 1, A.H_SWISH,
+                          scales=(0.02, 0.01, unsat(9)))),
+    # channel-wise NCHW through the NCHW44 detour (what rows that are no multiple of 4 still use)
+    ("nodwnchw", ConvCase(A.FMT_NCHW, A.GROUP, 4, 32, 56, 56, 32, 3, 1, 1, A.RELU,
                           scales=(0.02, 0.01, unsat(9)))),
 ]
 

@@ -264,11 +264,17 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_share_kernel(PwParams q) {
             for (int k = 0; k < 4; ++k)
                 acc[e4 * 4 + k] = bv[k];
         }
+        // two accumulator chains (even and odd chunks): a dependent MFMA can only issue when the one
+        // before it has left the pipe, two chains keep the matrix core busy between them
+        v16i acc1 = {};
 #pragma unroll
-        for (int c = 0; c < KC; ++c) {
-            const v4i b = *(const v4i*)(btile[buf] + c * 1024 + lane * 16);
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[c], b, acc, 0, 0, 0);
+        for (int c = 0; c < KC; c += 2) {
+            const v4i b0 = *(const v4i*)(btile[buf] + c * 1024 + lane * 16);
+            const v4i b1 = *(const v4i*)(btile[buf] + (c + 1) * 1024 + lane * 16);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[c], b0, acc, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[c + 1], b1, acc1, 0, 0, 0);
         }
+        acc += acc1;
         const int p = t * 32 + col;
         const bool ok = p < q.P;
         const int n = fdiv(p, q.dOHW);

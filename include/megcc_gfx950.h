@@ -437,7 +437,8 @@ typedef enum {
     MEGCC_KERN_RELAYOUT = 8,
     MEGCC_KERN_CONCAT = 9,
     MEGCC_KERN_RESIZE = 10,
-    MEGCC_KERN_FUSED_ELEMWISE = 11 /* never produced by parse_symbol; a caller fills the attr */
+    MEGCC_KERN_FUSED_ELEMWISE = 11, /* never produced by parse_symbol; a caller fills the attr */
+    MEGCC_KERN_SOFTMAX = 12         /* never produced by parse_symbol either: see megcc_gfx950_softmax */
 } MegccKernelKind;
 
 typedef struct {
@@ -454,6 +455,22 @@ typedef struct {
         MegccFusedElemwiseAttr fused;
     } attr;
 } MegccKernelDesc;
+
+/* Soft-max over the last axis in ONE kernel. MegCC has no such kernel: its importer decomposes
+ * opr::Softmax into Reduce MAX -> SUB -> EXP -> Reduce SUM -> TRUE_DIV
+ * (compiler/lib/Target/MGB/importer.cpp:987-1016), five kernel calls per forward, usually behind a
+ * typecvt qsi8 -> f32. A kernel boundary costs 3-5 us on this chip, so the model runtime
+ * (megcc_gfx950_model_finalize) replaces that operator chain - and the typecvt in front of it, when
+ * nothing else reads its result - by this entry point; the five kernels stay available under their
+ * own symbols. inputs[0]: f32, or qsi8 (dequantised with its scale first, as
+ * GI_kernel_typecvt_qsi8f32 does); outputs[0]: f32 with as many elements, its last axis is the
+ * soft-max axis; rows of at most
+ * megcc_gfx950_softmax_max_columns() elements; same expressions per element as the five kernels,
+ * only the order of the additions of a row's sum differs (results within 1e-6 relative). */
+TinyNNStatus megcc_gfx950_softmax(
+        Tensor** inputs, int nr_input, Tensor** outputs, int nr_output, const Workspace* workspace,
+        const RuntimeOpt* opt);
+int megcc_gfx950_softmax_max_columns(void);
 
 /* TinyNN_ERROR_NO_FOUND when the symbol is not one of this path's operators. */
 TinyNNStatus megcc_gfx950_parse_symbol(const char* symbol, MegccKernelDesc* desc);

@@ -45,7 +45,7 @@ REDUCE_MODES = {"SUM": 0, "MEAN": 1, "MAX": 2, "MIN": 3, "PRODUCT": 4, "SUM_SQR"
 # MegccKernelKind
 KERN_CONV, KERN_MATMUL, KERN_POOLING, KERN_ELEMWISE_MULTITYPE = 1, 2, 3, 4
 KERN_ELEMWISE, KERN_TYPECVT, KERN_REDUCE = 5, 6, 7
-KERN_RELAYOUT, KERN_CONCAT, KERN_RESIZE, KERN_FUSED_ELEMWISE = 8, 9, 10, 11
+KERN_RELAYOUT, KERN_CONCAT, KERN_RESIZE, KERN_FUSED_ELEMWISE, KERN_SOFTMAX = 8, 9, 10, 11, 12
 IMODE_NEAREST, IMODE_LINEAR = 0, 1
 
 

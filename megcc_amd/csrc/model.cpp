@@ -55,6 +55,10 @@ struct Model {
     RuntimeOpt opt;
     std::vector<ModelTensor*> tensors;
     std::vector<ModelOpr*> oprs;
+    // what forward() launches: the operators in order, with recognised operator chains replaced by
+    // one kernel (`fused` owns the replacements); run_opr, nr_opr and the memory plan keep the
+    // operator list as it was given
+    std::vector<ModelOpr*> schedule, fused;
     void* arena = nullptr;
     size_t arena_bytes = 0;
     // one scratch buffer shared by all operators (they run one after the other on one stream),
@@ -121,6 +125,95 @@ bool plan_memory(Model* m) {
     return true;
 }
 
+// ---- forward schedule ----------------------------------------------------------------------------
+// The importer's decomposition of a soft-max (Reduce MAX over the last axis -> SUB -> EXP -> Reduce
+// SUM -> TRUE_DIV, compiler/lib/Target/MGB/importer.cpp:987-1016), optionally behind the typecvt
+// qsi8 -> f32 that dequantises the logits, is five or six kernel boundaries of 3-5 us each for half
+// a megabyte of data. When the intermediate tensors have no other reader and are no outputs, the
+// chain runs as ONE kernel (softmax.hip). The intermediates keep their place in the memory plan.
+static bool dense_f32(const Tensor& t) {
+    return t.dtype.type_enum == TinyNN_FLOAT && is_contiguous(t.layout);
+}
+static void build_schedule(Model* m) {
+    m->schedule.clear();
+    const int n = (int)m->oprs.size();
+    std::vector<int> readers(m->tensors.size(), 0);
+    for (auto* o : m->oprs)
+        for (int id : o->in)
+            ++readers[root_of(m, id)];
+    // a tensor only this chain touches: its own memory, `nr` readers, neither input, output nor weight
+    auto temp = [&](int id, int nr) {
+        const ModelTensor* t = m->tensors[id];
+        return t->alias_of < 0 && !t->is_input && !t->is_output && !t->is_weight && readers[id] == nr;
+    };
+    auto is_ew = [](const ModelOpr* o, MegccElemwiseMode mode, size_t nin) {
+        return o->desc.kind == MEGCC_KERN_ELEMWISE && o->desc.attr.elemwise == mode &&
+               o->in.size() == nin && o->out.size() == 1;
+    };
+    auto is_red = [&](const ModelOpr* o, MegccReduceMode mode) {
+        if (o->desc.kind != MEGCC_KERN_REDUCE || o->desc.attr.reduce.mode != mode ||
+            o->in.size() != 1 || o->out.size() != 1)
+            return false;
+        const Tensor& s = m->tensors[o->in[0]]->t;
+        return o->desc.attr.reduce.axis == s.layout.nr_dim - 1;
+    };
+    for (int i = 0; i < n; ++i) {
+        ModelOpr* o0 = m->oprs[i];
+        bool fuse = !options().no_fuse_softmax && i + 4 < n && is_red(o0, MEGCC_REDUCE_MAX) &&
+                    is_ew(m->oprs[i + 1], MEGCC_EW_SUB, 2) && is_ew(m->oprs[i + 2], MEGCC_EW_EXP, 1) &&
+                    is_red(m->oprs[i + 3], MEGCC_REDUCE_SUM) && is_ew(m->oprs[i + 4], MEGCC_EW_TRUE_DIV, 2);
+        if (fuse) {
+            ModelOpr *o1 = m->oprs[i + 1], *o2 = m->oprs[i + 2], *o3 = m->oprs[i + 3], *o4 = m->oprs[i + 4];
+            const int x = o0->in[0], mx = o0->out[0], sub = o1->out[0], ex = o2->out[0], sum = o3->out[0],
+                      y = o4->out[0];
+            const Tensor& tx = m->tensors[x]->t;
+            const Tensor& ty = m->tensors[y]->t;
+            const size_t cols = tx.layout.nr_dim ? tx.layout.dims[tx.layout.nr_dim - 1] : 0;
+            fuse = o1->in[0] == x && o1->in[1] == mx && o2->in[0] == sub && o3->in[0] == ex &&
+                   o4->in[0] == ex && o4->in[1] == sum && m->tensors[x]->alias_of < 0 &&
+                   m->tensors[y]->alias_of < 0 && temp(mx, 1) && temp(sub, 1) && temp(ex, 2) &&
+                   temp(sum, 1) && dense_f32(tx) && dense_f32(ty) && dense_f32(m->tensors[mx]->t) &&
+                   dense_f32(m->tensors[sum]->t) && dense_f32(m->tensors[sub]->t) &&
+                   dense_f32(m->tensors[ex]->t) && cols >= 1 &&
+                   cols <= (size_t)megcc_gfx950_softmax_max_columns() &&
+                   nr_elem(ty.layout) == nr_elem(tx.layout) &&
+                   nr_elem(m->tensors[sub]->t.layout) == nr_elem(tx.layout) &&
+                   nr_elem(m->tensors[ex]->t.layout) == nr_elem(tx.layout) &&
+                   nr_elem(m->tensors[mx]->t.layout) * cols == nr_elem(tx.layout) &&
+                   nr_elem(m->tensors[sum]->t.layout) * cols == nr_elem(tx.layout);
+            if (fuse) {
+                int src = x;
+                // the dequantisation in front of it, when the soft-max is all that reads its result
+                if (!m->schedule.empty() && i > 0 && m->schedule.back() == m->oprs[i - 1]) {
+                    const ModelOpr* cv = m->oprs[i - 1];
+                    if (cv->desc.kind == MEGCC_KERN_TYPECVT && cv->in.size() == 1 && cv->out.size() == 1 &&
+                        cv->out[0] == x && temp(x, 2) &&
+                        m->tensors[cv->in[0]]->t.dtype.type_enum == TinyNN_QINT8 &&
+                        is_contiguous(m->tensors[cv->in[0]]->t.layout) &&
+                        nr_elem(m->tensors[cv->in[0]]->t.layout) == nr_elem(tx.layout)) {
+                        src = cv->in[0];
+                        m->schedule.pop_back();
+                    }
+                }
+                ModelOpr* f = new ModelOpr();
+                memset(&f->desc, 0, sizeof(f->desc));
+                f->desc.kind = MEGCC_KERN_SOFTMAX;
+                f->symbol = "softmax (fused)";
+                memset(&f->ws, 0, sizeof(f->ws));
+                f->in.push_back(src);
+                f->out.push_back(y);
+                f->in_ptrs.push_back(&m->tensors[src]->t);
+                f->out_ptrs.push_back(&m->tensors[y]->t);
+                m->fused.push_back(f);
+                m->schedule.push_back(f);
+                i += 4;
+                continue;
+            }
+        }
+        m->schedule.push_back(o0);
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -150,6 +243,8 @@ void megcc_gfx950_model_destroy(void* model) {
             m->dev.free(t->owned);
         delete t;
     }
+    for (auto* o : m->fused)
+        delete o;
     if (m->arena)
         m->dev.free(m->arena);
     if (m->workspace)
@@ -311,7 +406,7 @@ TinyNNStatus megcc_gfx950_model_add_opr_desc(
     Model* m = (Model*)model;
     MG_REQUIRE(m && desc && name && inputs && outputs && !m->finalized, TinyNN_ERROR_NULL_PTR,
                "model_add_opr_desc: bad argument");
-    MG_REQUIRE(desc->kind >= MEGCC_KERN_CONV && desc->kind <= MEGCC_KERN_FUSED_ELEMWISE,
+    MG_REQUIRE(desc->kind >= MEGCC_KERN_CONV && desc->kind <= MEGCC_KERN_SOFTMAX,
                TinyNN_ERROR_OUT_OF_RANGE, "model_add_opr_desc: kind %d", (int)desc->kind);
     return add_opr(m, *desc, name, inputs, nr_input, outputs, nr_output);
 }
@@ -433,6 +528,7 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
         for (auto* o : m->oprs)
             o->ws.ptr = o->ws.size ? m->workspace : nullptr;
     }
+    build_schedule(m);
     m->finalized = true;
     return megcc_gfx950_wait();
 }
@@ -472,7 +568,7 @@ TinyNNStatus megcc_gfx950_model_get_output(void* model, int tensor, void* host, 
 // LITE_forward: one asynchronous kernel launch per Opr, in order, on the library stream; stops at
 // the first failing kernel like network.c:191-194. Results are visible after megcc_gfx950_wait().
 static TinyNNStatus forward_eager(Model* m) {
-    for (auto* o : m->oprs) {
+    for (auto* o : m->schedule) {
         TinyNNStatus st = megcc_gfx950_call(
                 &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), o->out_ptrs.data(),
                 (int)o->out_ptrs.size(), &o->ws, &m->opt);

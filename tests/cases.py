@@ -779,6 +779,49 @@ class FusedCase:
                                    self.types(), self.out_shape)
 
 
+class SoftmaxCase:
+    """soft-max over the last axis in one kernel (megcc_gfx950_softmax): what the importer's
+    decomposition Reduce MAX -> SUB -> EXP -> Reduce SUM -> TRUE_DIV computes
+    (compiler/lib/Target/MGB/importer.cpp:987-1016), optionally from qsi8 logits that
+    GI_kernel_typecvt_qsi8f32 would dequantise first. The oracle is that chain of oracle calls."""
+
+    def __init__(self, shape, quantised=False, scale=0.1, span=(-8.0, 8.0)):
+        self.shape, self.quantised, self.scale, self.span = tuple(shape), quantised, scale, span
+
+    def __repr__(self):
+        return "softmax%s[%s]" % ("_q8" if self.quantised else "", "x".join(map(str, self.shape)))
+
+    def symbol(self):
+        return None  # no reference symbol: the kernel is addressed by a descriptor
+
+    def desc(self):
+        d = abi.KernelDesc()
+        d.kind = abi.KERN_SOFTMAX
+        return d
+
+    def gen(self, seed=0):
+        r = rng(seed)
+        if self.quantised:
+            return {"src": r.integers(-128, 128, self.shape).astype(np.int8)}
+        return {"src": r.uniform(self.span[0], self.span[1], self.shape).astype(np.float32)}
+
+    def specs(self, arrays):
+        if self.quantised:
+            ins = [TensorSpec(b"src", self.shape, abi.QINT8, self.scale, arrays["src"])]
+        else:
+            ins = [TensorSpec(b"src", self.shape, abi.FLOAT, 1.0, arrays["src"])]
+        return ins, [TensorSpec(b"dst", self.shape, abi.FLOAT, 1.0)]
+
+    def run_port(self, arrays):
+        x = arrays["src"]
+        if self.quantised:
+            x = port.typecvt(np.ascontiguousarray(x), "qsi8", "f32", self.scale, 1.0)
+        x2 = np.ascontiguousarray(x.reshape(-1, self.shape[-1]))
+        mx = port.reduce_f32(x2, abi.REDUCE_MAX, 1)
+        e = port.elemwise_f32(port.elemwise_f32(x2, mx, abi.EW_SUB), None, abi.EW_EXP)
+        return port.elemwise_f32(e, port.reduce_f32(e, abi.REDUCE_SUM, 1), abi.EW_TRUE_DIV).reshape(self.shape)
+
+
 def run_ref(case, arrays, symbol=None):
     """Evaluate `case` with the reference's generated C kernel; returns the output array."""
     ins, outs = case.specs(arrays)

@@ -507,6 +507,34 @@ OLDER = [
 ]
 
 
+SOFTMAX = [
+    cases.SoftmaxCase((64, 1000)), cases.SoftmaxCase((64, 1000), quantised=True, scale=0.13),
+    cases.SoftmaxCase((1, 1000), quantised=True, scale=0.05), cases.SoftmaxCase((3, 7, 4096)),
+    cases.SoftmaxCase((5, 1)), cases.SoftmaxCase((2, 3, 257), span=(-60.0, 60.0)),
+    cases.SoftmaxCase((300, 10), quantised=True, scale=1.0),
+]
+
+
+@pytest.mark.parametrize("case", SOFTMAX, ids=[repr(c) for c in SOFTMAX])
+def test_softmax_in_one_kernel_equals_the_five_operator_chain(case):
+    """the fused soft-max against the oracle's chain of the five operators it replaces"""
+    arrays = case.gen(seed=41)
+    ins, outs = case.specs(arrays)
+    got = runtime.PreparedOp(case.desc(), ins, outs)
+    got.launch()
+    out = got.result()
+    want = case.run_port(arrays)
+    assert cases.max_rel_err(out, want) <= 1e-5, repr(case)
+    assert np.allclose(out.reshape(-1, case.shape[-1]).sum(axis=1), 1.0, atol=1e-5)
+
+
+def test_softmax_refuses_rows_beyond_its_limit():
+    case = cases.SoftmaxCase((2, 4097))
+    ins, outs = case.specs(case.gen(seed=1))
+    with pytest.raises(runtime.MegccError):
+        runtime.PreparedOp(case.desc(), ins, outs).launch()
+
+
 @pytest.mark.parametrize("switch,case", OLDER, ids=["%s-%r" % (s, c) for s, c in OLDER])
 def test_older_kernels_still_agree(switch, case):
     port.set_threads(8)

@@ -97,3 +97,37 @@ def test_graph_replays_equal_eager_forwards():
             np.testing.assert_array_equal(graph.get(ids[k]), want[k], err_msg="%s, forward %d" % (k, it))
     eager.close()
     graph.close()
+
+
+@pytest.mark.gpu
+def test_softmax_chain_runs_as_one_kernel_and_gives_the_same_result():
+    """forward() replaces Reduce MAX -> SUB -> EXP -> Reduce SUM -> TRUE_DIV (and the typecvt in
+    front) by one kernel when nothing else reads the intermediates; with every layer's result kept
+    as an output the typecvt stays an operator of its own, with the option off all of them do. Same
+    probabilities either way, on eager forwards and on graph replays."""
+    net = mobilenet.Net(3)
+    image = mobilenet.draw_input(3, seed=33)
+    want, _ = net.run_oracle(image)
+    fused, ids = net.build_gpu()
+    runtime.set_option("nofusesoftmax", 1)
+    try:
+        plain, _ = net.build_gpu()
+    finally:
+        runtime.set_option("nofusesoftmax", 0)
+    kept, kids = net.build_gpu(keep_all=True)
+    results = []
+    for model, mids, last in ((fused, ids, "softmax_rows:1"), (plain, ids, "elemwise_f32_bcast"),
+                              (kept, kids, "softmax_rows:4")):
+        model.set_input(mids["image"], image)
+        for it in range(3):  # eager, capture, replay
+            model.forward()
+            out = model.get(mids["softmax"])
+            assert cases.max_rel_err(out, want) <= 1e-4
+            if it == 0:
+                assert runtime.last_kernel().startswith(last), runtime.last_kernel()
+        results.append(out.copy())
+        assert model.nr_opr == 36
+    assert cases.max_rel_err(results[0], results[1]) <= 1e-6
+    np.testing.assert_array_equal(results[0], results[2])
+    for m in (fused, plain, kept):
+        m.close()

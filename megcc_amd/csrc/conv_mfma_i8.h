@@ -110,6 +110,13 @@ __device__ __forceinline__ void dma_global_b128(const void* gptr, unsigned lds_a
                  : "v"(gptr), "s"(__builtin_amdgcn_readfirstlane(lds_addr))
                  : "memory");
 }
+// the same with a scalar base address and a 32-bit lane offset (no 64-bit address per lane)
+__device__ __forceinline__ void dma_global_saddr_b128(const void* sbase, unsigned voffset, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(voffset), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane(lds_addr))
+                 : "memory");
+}
 // raw buffer (stride 0): offsets at or beyond num_records read as zero
 __device__ __forceinline__ v4u make_raw_buffer(const void* base, unsigned num_records) {
     const unsigned long long a = (unsigned long long)base;

@@ -82,7 +82,11 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     int* const rq_table = (int*)(lds + DM_NBUF * BUF_BYTES);
     int* const bias_lds = rq_table + REQUANT_TABLE_ENTRIES;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // (the wave index through readfirstlane: everything derived from it - which chunks a wave loads,
+    //  ring positions, the column count of a ragged sub-tile, the stage counters updated under it -
+    //  then lives in scalar registers and branches are scalar)
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const unsigned lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds));
     // (waves w and w + 4 share a SIMD: give them different pixel columns, so that the wave with
     //  one column more in a ragged sub-tile does not meet its twin on the same SIMD)
     const int wm = wave / WGN, wn = (wave + wm) % WGN, kg = lane >> 5;
@@ -183,23 +187,24 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     };
     int lp0 = range0, lst = 0, lbuf = 0;  // load cursor: sub-tile, stage in it, LDS buffer
     describe(lp0);
-    auto issue = [&](int8_t* buf) __attribute__((always_inline)) {
+    auto issue = [&](int bufidx) __attribute__((always_inline)) {
+        const unsigned buf = lds0 + bufidx * BUF_BYTES;  // (LDS byte address, scalar)
         const int8_t* abase = q.wp + ((size_t)lst * TS * q.OCP + oc0) * KROW;
 #pragma unroll
         for (int a = 0; a < A_PER_WAVE; ++a)
-            dma_global_b128(abase + ((a_chunk[a] / (DM_BM / 32)) * q.OCP * KROW +
-                                     (a_chunk[a] % (DM_BM / 32)) * 1024) + lane16,
-                            lds_address(buf + a_chunk[a] * 1024));
+            dma_global_saddr_b128(abase + ((size_t)(a_chunk[a] / (DM_BM / 32)) * q.OCP * KROW +
+                                           (a_chunk[a] % (DM_BM / 32)) * 1024),
+                                  lane16, buf + a_chunk[a] * 1024);
         const unsigned poff = (unsigned)(lst * KS * 8) * (unsigned)q.plane_stride;
         static_for<B_PER_WAVE>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             const int u = wave + j * DM_WAVES;
             if constexpr (FCB)
-                dma_global_b128(q.src + (b_goff[j] + poff), lds_address(buf + A_BYTES + u * 1024));
+                dma_global_b128(q.src + (b_goff[j] + poff), buf + A_BYTES + u * 1024);
             else if constexpr (PM)
-                dma_buffer_b128(src_rsrc, b_goff[j] + poff, lds_address(buf + A_BYTES + u * 1024));
+                dma_buffer_b128(src_rsrc, b_goff[j] + poff, buf + A_BYTES + u * 1024);
             else
-                dma_buffer_b32(src_rsrc, b_goff[j] + poff, lds_address(buf + A_BYTES + u * 256));
+                dma_buffer_b32(src_rsrc, b_goff[j] + poff, buf + A_BYTES + u * 256);
         });
         if (++lst == stages) {
             lst = 0;
@@ -219,7 +224,6 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     }
 
     v16i acc[MT][NT];
-    const int kg_plane = kg * q.OHW;
 
     // Epilogue of one 32 oc x 32 pixel MFMA tile (16 outputs per lane = 4 NCHW44 dwords), written
     // as one straight-line block so that its 4 bias reads and 16 table look-ups are in flight
@@ -256,8 +260,10 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
                     continue;
                 const uint32_t w = pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
                 if constexpr (!FC) {
-                    const int o = ob + ((oc0 >> 2) + (wm * MT + mi) * 8 + e4 * 2) * q.OHW + kg_plane;
-                    ((uint32_t*)q.dst)[o] = w;
+                    // scalar base (channel group) + 32-bit lane offset (pixel and K-half's plane)
+                    int8_t* const base =
+                            q.dst + ((size_t)(((oc0 >> 2) + (wm * MT + mi) * 8 + e4 * 2) * q.OHW) << 2);
+                    *(uint32_t*)(base + ((unsigned)ob << 2)) = w;
                 } else {  // ob = pixel (row of the output matrix)
                     int8_t* o = q.dst + (size_t)ob * q.OC + oc;
                     if ((q.OC & 3) == 0) {
@@ -277,7 +283,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
 #pragma unroll
     for (int i = 0; i < DM_NBUF - 1; ++i)
         if (i < G)
-            issue(lds + i * BUF_BYTES);
+            issue(i);
     if (G >= DM_NBUF - 1)
         wait_vmcnt<N_FLIGHT>();
     else
@@ -308,7 +314,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             cur_o[ni] = pc > plast ? -2
                         : p > plast ? -1
                         : FC        ? p
-                                    : pn * (q.OC >> 2) * q.OHW + (p - pn * q.OHW);
+                                    : pn * (q.OC >> 2) * q.OHW + (p - pn * q.OHW) + kg * q.OHW;
         }
         // the accumulators start from the bias of their output channel (register e of a tile:
         // channel 8 * (e / 4) + 4 * kg + e % 4)
@@ -325,7 +331,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
                     acc[mi][ni][e] = bv[e / 4][e % 4];
         }
 
-        auto stage_body = [&](auto cols_c, const int8_t* bufA, int8_t* dma_buf) __attribute__((always_inline)) {
+        auto stage_body = [&](auto cols_c, const int8_t* bufA, int dma_buf) __attribute__((always_inline)) {
             constexpr int COLS = decltype(cols_c)::value;
             if (g + DM_NBUF - 1 < G)
                 issue(dma_buf);
@@ -373,7 +379,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
         };
         auto run_stages = [&](auto cols_c) __attribute__((always_inline)) {
             for (int st = 0; st < stages; ++st, ++g) {
-                stage_body(cols_c, lds + cbuf * BUF_BYTES, lds + lbuf * BUF_BYTES);
+                stage_body(cols_c, lds + cbuf * BUF_BYTES, lbuf);
                 // stage g+1 must have landed; the DM_NBUF - 2 stages issued after it may be in
                 // flight (stores issued in between only make the wait longer, never shorter)
                 if (g + DM_NBUF - 1 < G)

@@ -546,7 +546,7 @@ TinyNNStatus conv_mfma_launch(
         if (range_len < pc.bn / 2) {  // too few pixels per workgroup for the tile
             if (pc.bm == 32)
                 range_len = pc.bn;  // the small-layer tiles: one tile per workgroup, not every CU busy
-            else if (pc.bn <= 256 && P >= 4096)
+            else if (pc.bn <= 256 && (P >= 4096 || (g.fh == 1 && g.fw == 1 && P >= 2048)))
                 // between the small-layer tiles and a full grid of 256- / 128-pixel tiles: half-filled
                 // tiles on part of the CUs (N=6, 128->128, 56x56: 9.4 us; the one-stage kernel
                 // these layers fell to: 20.8 us)

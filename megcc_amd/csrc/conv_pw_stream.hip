@@ -320,8 +320,10 @@ bool conv_pw_stream_supported(const ConvGeom& g) {
     const long P = (long)g.n * g.oh * g.ow;
     return g.fmt == MEGCC_FMT_NCHW44 && g.groups == 1 && g.fh == 1 && g.fw == 1 && g.sh == 1 &&
            g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.ic == 32 || g.ic == 64 || g.ic == 128 || g.ic == 256 || g.ic == 512 ||
-            // (1024: only layers too small for the LDS-staged kernel, where one round trip wins)
-            (g.ic == 1024 && P < 2048)) &&
+            // (1024: layers too small for the LDS-staged kernel, where one round trip wins, and the
+            //  workgroup-shared form up to a few thousand pixels)
+            (g.ic == 1024 && (P < 2048 || (P <= 4096 && (g.oc & 127) == 0 && !options().no_pwshare &&
+                                         (P + 31) / 32 * (g.oc / 128) >= 256)))) &&
            (g.oc & 63) == 0 && g.oc <= PW_MAX_OC && P >= 32 &&
            (long)g.n * g.ic * g.ih * g.iw < (1L << 31) && P * g.oc < (1L << 31);
 }
@@ -370,10 +372,13 @@ TinyNNStatus conv_pw_stream_launch(
 #undef MG_PW_PICK
 
     // 512 input channels and more tiles than resident waves: the workgroup-shared form
-    if (g.ic == 512 && (q.groups & 3) == 0 && !options().no_pwshare) {
-        const void* sk = act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_share_kernel<16, MEGCC_NONLINE_IDENTITY>
-                         : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_share_kernel<16, MEGCC_NONLINE_RELU>
-                                                       : (const void*)conv_pw_share_kernel<16, -1>;
+    if ((g.ic == 512 || g.ic == 1024) && (q.groups & 3) == 0 && !options().no_pwshare) {
+#define MG_PWS_PICK(KC_)                                                                                  \
+    (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_share_kernel<KC_, MEGCC_NONLINE_IDENTITY>         \
+     : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_share_kernel<KC_, MEGCC_NONLINE_RELU>             \
+                                   : (const void*)conv_pw_share_kernel<KC_, -1>)
+        const void* sk = g.ic == 512 ? MG_PWS_PICK(16) : MG_PWS_PICK(32);
+#undef MG_PWS_PICK
         const long gblocks = q.groups / 4;
         const long capb = (long)num_cus() * pw_resident_blocks(sk);
         if ((long)q.tiles * gblocks >= capb / 2) {

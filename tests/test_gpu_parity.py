@@ -147,6 +147,10 @@ LIVE = [
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 30, 34, 8, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),  # generic path (IW % 4 != 0)
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
     # the 2x2 stride-2 maximum on packed halves (rows of 8, 16 pixels), and rows it does not take
+    # 1x1 with 1024 input channels between 2048 and 4096 pixels: the workgroup-shared pointwise
+    # kernel (1024 -> 512), half-filled tiles of the LDS-direct kernel (1024 -> 256)
+    ConvCase(A.FMT_NCHW44, A.DENSE, 64, 1024, 7, 7, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(1024))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 50, 1024, 7, 7, 256, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(1024))),
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 3, 12, 6, 8, 2, 2, 0),
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 1, 4, 2, 16, 2, 2, 0),
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 8, 6, 12, 2, 2, 0),

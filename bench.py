@@ -188,6 +188,10 @@ def make_workload(name):
     if name == "pool":
         return (PoolCase(abi.FMT_NCHW44, abi.POOL_MAX, 64, 32, 112, 112, 2, 2, 0),
                 "qsi8 maxpool 2x2 s2 NCHW44 N=64 C=32 112x112", "hbm")
+    if name in ("pool_nchw", "pool_nchw_s1"):  # the stem pooling of a ResNet-like model kept in NCHW
+        w, s = (3, 2) if name == "pool_nchw" else (3, 1)
+        return (PoolCase(abi.FMT_NCHW, abi.POOL_MAX, 64, 64, 112, 112, w, s, 1),
+                "qsi8 maxpool %dx%d s%d p1 NCHW N=64 C=64 112x112" % (w, w, s), "hbm")
     if name == "add":
         return (MultiTypeCase(abi.Q_FUSE_ADD_RELU, (64, 32, 56, 56), (0.05, 0.01, 0.05)),
                 "qsi8 QFUSE_ADD_RELU 64x32x56x56", "hbm")

@@ -172,13 +172,25 @@ static size_t gather_bytes(const ConvGeom& g) {
 // back. The filter [OC][IC][FH][FW] packs into the same tiles as an NCHW44 one; the bias layouts
 // are the same bytes.
 static bool nchw_spatial(const ConvGeom& g) {
-    return g.fmt == MEGCC_FMT_NCHW && g.groups == 1 && (g.ic & 3) == 0 && (g.oc & 3) == 0 &&
-           !(g.ih == 1 && g.iw == 1 && g.fh == 1 && g.fw == 1);
+    return g.fmt == MEGCC_FMT_NCHW && g.groups == 1 && !(g.ih == 1 && g.iw == 1 && g.fh == 1 && g.fw == 1);
+}
+// (channel counts that are no multiple of 4 are padded: the packed filter holds zeros for channels
+//  beyond IC / OC anyway, so what the padding lanes of the NCHW44 copies hold does not matter)
+static int round_up4(int v) {
+    return (v + 3) & ~3;
 }
 static ConvGeom as_nchw44(const ConvGeom& g) {
     ConvGeom s = g;
     s.fmt = MEGCC_FMT_NCHW44;
+    s.ic = round_up4(g.ic);
+    s.oc = round_up4(g.oc);
     return s;
+}
+// workspace of the detour: [inner kernel's][input copy][output copy][bias copy when OC % 4 != 0]
+static size_t nchw_spatial_bytes(const ConvGeom& g, size_t inner) {
+    const ConvGeom g1 = as_nchw44(g);
+    return round_up256(inner) + round_up256((size_t)g.n * g1.ic * g.ih * g.iw) +
+           round_up256((size_t)g.n * g1.oc * g.oh * g.ow) + (g1.oc != g.oc ? round_up256((size_t)g1.oc * 4) : 0);
 }
 // Channel-wise (depthwise) qsi8 convolution on plain NCHW tensors: the same detour around the
 // NCHW44 depthwise kernel; the filter [G,1,1,FH,FW] becomes [G/4,1,1,FH,FW,4] by a third, tiny
@@ -202,6 +214,35 @@ static void nchw44_views(int n, int c, int h, int w, Layout* view, Layout* dense
         view->stride[i] = vs[i];
         dense->stride[i] = ds[i];
     }
+}
+// NCHW tensor with c channels <-> NCHW44 tensor with round_up4(c) channels: the whole groups of 4
+// in one copy, the last group's c % 4 channels in a second (its other lanes are not touched)
+static TinyNNStatus nchw_nchw44_copy(
+        bool to44, const void* from, void* to, int n, int c, int h, int w, const char* what) {
+    const int c1 = round_up4(c), full = c & ~3, rem = c - full;
+    const char* nchw = (const char*)(to44 ? from : to);
+    const char* n44 = (const char*)(to44 ? to : from);
+    for (int part = 0; part < 2; ++part) {
+        const int groups = part == 0 ? full / 4 : 1, lanes = part == 0 ? 4 : rem;
+        if (groups == 0 || lanes == 0)
+            continue;
+        Layout view = {}, dense = {};
+        view.nr_dim = dense.nr_dim = 5;
+        const uint32_t d[5] = {(uint32_t)n, (uint32_t)groups, (uint32_t)h, (uint32_t)w, (uint32_t)lanes};
+        const int vs[5] = {c * h * w, 4 * h * w, w, 1, h * w};
+        const int ds[5] = {c1 * h * w, 4 * h * w, 4 * w, 4, 1};
+        for (int i = 0; i < 5; ++i) {
+            view.dims[i] = dense.dims[i] = d[i];
+            view.stride[i] = vs[i];
+            dense.stride[i] = ds[i];
+        }
+        const size_t off = part == 0 ? 0 : (size_t)full * h * w;  // first byte of the last group in both
+        TinyNNStatus st = to44 ? strided_copy(nchw + off, view, (char*)n44 + off, dense, 1, what)
+                               : strided_copy(n44 + off, dense, (char*)nchw + off, view, 1, what);
+        if (st != TinyNN_SUCCESS)
+            return st;
+    }
+    return TinyNN_SUCCESS;
 }
 
 // ---- scratch memory of megcc_gfx950_conv2d_noalloc ---------------------------------------------
@@ -245,8 +286,7 @@ static size_t conv2d_scratch_bytes(const ConvGeom& g, bool q8, bool f32, bool pa
     if (packed && q8 && strided_pointwise(g) && conv_mfma_supported(subsampled(g)))
         return round_up256(conv_mfma_workspace_bytes(subsampled(g))) + gather_bytes(g);
     if (packed && q8 && nchw_spatial(g) && conv_mfma_supported(as_nchw44(g)))
-        return round_up256(conv_mfma_workspace_bytes(as_nchw44(g))) +
-               round_up256((size_t)g.n * g.ic * g.ih * g.iw) + (size_t)g.n * g.oc * g.oh * g.ow;
+        return nchw_spatial_bytes(g, conv_mfma_workspace_bytes(as_nchw44(g)));
     if (packed && q8 && conv_mfma_supported(g))
         return conv_mfma_workspace_bytes(g);
     if (!packed && q8 && nchw_depthwise(g) && dwconv44_supported(as_nchw44(g)))
@@ -354,27 +394,36 @@ static TinyNNStatus conv2d_run(
         MG_REQUIRE(aligned16(flt->ptr) && (!b || aligned4(b)), TinyNN_ERROR_INVALID_LAYOUT,
                    "conv2d: misaligned operand");
         const size_t inner = round_up256(conv_mfma_workspace_bytes(g1));
-        const size_t in44 = round_up256((size_t)g.n * g.ic * g.ih * g.iw);
-        const size_t out44 = (size_t)g.n * g.oc * g.oh * g.ow;
-        MG_REQUIRE(workspace && workspace->ptr && workspace->size >= inner + in44 + out44 &&
-                           aligned16(workspace->ptr),
-                   TinyNN_ERROR_OUT_OF_RANGE,
-                   "conv2d: a dense NCHW convolution needs %zu bytes of workspace", inner + in44 + out44);
-        MG_REQUIRE((long)g.n * g.ic * g.ih * g.iw < (1L << 31) && (long)g.n * g.oc * g.oh * g.ow < (1L << 31),
+        const size_t in44 = round_up256((size_t)g.n * g1.ic * g.ih * g.iw);
+        const size_t out44 = round_up256((size_t)g.n * g1.oc * g.oh * g.ow);
+        const size_t need = nchw_spatial_bytes(g, conv_mfma_workspace_bytes(g1));
+        MG_REQUIRE(workspace && workspace->ptr && workspace->size >= need && aligned16(workspace->ptr),
+                   TinyNN_ERROR_OUT_OF_RANGE, "conv2d: a dense NCHW convolution needs %zu bytes of workspace",
+                   need);
+        MG_REQUIRE((long)g.n * g1.ic * g.ih * g.iw < (1L << 31) && (long)g.n * g1.oc * g.oh * g.ow < (1L << 31),
                    TinyNN_ERROR_OUT_OF_RANGE, "conv2d: tensor too large");
         char* src44 = (char*)workspace->ptr + inner;
         char* dst44 = src44 + in44;
-        Layout view, dense;
-        nchw44_views(g.n, g.ic, g.ih, g.iw, &view, &dense);
-        st = strided_copy(src->ptr, view, src44, dense, 1, "conv2d (NCHW -> NCHW44)");
+        st = nchw_nchw44_copy(true, src->ptr, src44, g.n, g.ic, g.ih, g.iw, "conv2d (NCHW -> NCHW44)");
         if (st != TinyNN_SUCCESS)
             return st;
+        const void* b1 = b;
+        if (b && g1.oc != g.oc) {
+            // the kernel reads a bias per (padded) output channel: a copy it may read to the end
+            Layout bl = {};
+            bl.nr_dim = 1;
+            bl.dims[0] = (uint32_t)g.oc;
+            bl.stride[0] = 1;
+            st = strided_copy(b, bl, dst44 + out44, bl, 4, "conv2d (bias)");
+            if (st != TinyNN_SUCCESS)
+                return st;
+            b1 = dst44 + out44;
+        }
         Workspace sub = {workspace->ptr, inner, 0};
-        st = conv_mfma_launch(g1, src44, flt->ptr, b, dst44, &sub);
+        st = conv_mfma_launch(g1, src44, flt->ptr, b1, dst44, &sub);
         if (st != TinyNN_SUCCESS)
             return st;
-        nchw44_views(g.n, g.oc, g.oh, g.ow, &view, &dense);
-        return strided_copy(dst44, dense, dst->ptr, view, 1, "conv2d (NCHW44 -> NCHW)");
+        return nchw_nchw44_copy(false, dst44, dst->ptr, g.n, g.oc, g.oh, g.ow, "conv2d (NCHW44 -> NCHW)");
     }
     if (packed) {
         MG_REQUIRE(q8 && conv_mfma_supported(g), TinyNN_ERROR_INVALID_LAYOUT,
@@ -533,9 +582,7 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d_workspace(
             if (strided_pointwise(g) && conv_mfma_supported(subsampled(g)))
                 *workspace = round_up256(conv_mfma_workspace_bytes(subsampled(g))) + gather_bytes(g);
             else if (nchw_spatial(g) && conv_mfma_supported(as_nchw44(g)))
-                *workspace = round_up256(conv_mfma_workspace_bytes(as_nchw44(g))) +
-                             round_up256((size_t)g.n * g.ic * g.ih * g.iw) +
-                             (size_t)g.n * g.oc * g.oh * g.ow;
+                *workspace = nchw_spatial_bytes(g, conv_mfma_workspace_bytes(as_nchw44(g)));
             else if (conv_mfma_supported(g))
                 *workspace = conv_mfma_workspace_bytes(g);
         }

@@ -6,7 +6,7 @@
 //            QInt8PoolingNCHW44.cpp:34-113): AVERAGE is saturate(round((float)sum * count_div)) with
 //            `float count_div = 1.0 / window_count` (a double quotient rounded to float).
 // NCHW44: one thread per output dword (4 channels of a pixel), lanes walk W -> coalesced dwords.
-// NCHW  : one thread per output byte, lanes walk W.
+// NCHW  : four outputs of a row per thread for the common windows, else one thread per output byte.
 #include "common.h"
 #include "epilogue.h"
 #include "fastdiv.h"
@@ -145,6 +145,112 @@ __global__ void __launch_bounds__(256) pool_nchw_q8_kernel(
     }
 }
 
+// NCHW, any mode, square windows of the common widths and strides: a thread makes 4 neighbouring
+// outputs of a row. Their windows cover 3 * SW + WW consecutive bytes of each input row, which are
+// fetched as the aligned dwords that contain them (only dwords that hold at least one byte of the
+// row: an aligned dword with a byte of the tensor in it lies inside the tensor's page) and shifted
+// into place with v_alignbyte; bytes left or right of the row (padding, outputs beyond the row's
+// end) are replaced by the neutral value through a per-thread byte mask, so that there is ONE code
+// path and no divergence at the borders. The window ROWS are combined first, on whole dwords: a
+// dword of 4 signed bytes is split into its even and its odd bytes as packed 16-bit halves (as in
+// max4_bytes below) and the rows meet in packed max / add (a column sum of up to 255 bytes fits 16
+// bits); only then the WW columns of each output are picked out of the combined row at
+// compile-time positions. All loads of a thread are in flight together.
+typedef short pool_s2 __attribute__((ext_vector_type(2)));
+
+template <int WW, int SW, bool IS_MAX>
+__global__ void __launch_bounds__(256) pool_nchw_rows_kernel(
+        PoolGeom g, const int8_t* __restrict__ src, int8_t* __restrict__ dst, unsigned total, int owg,
+        FastDiv d_owg, FastDiv d_oh, int dword_store) {
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;  // (plane, oh, group of 4 ow)
+    if (i >= total)
+        return;
+    const unsigned row = fdiv(i, d_owg), q = i - row * (unsigned)owg;
+    const unsigned plane = fdiv(row, d_oh), oh = row - plane * (unsigned)g.oh;
+    const int ow0 = (int)q * 4;
+    const int nvalid = min(4, g.ow - ow0);
+    constexpr int SPAN = 3 * SW + WW;
+    constexpr int NA = (SPAN + 3) / 4;  // dwords of the shifted span
+    const int s = ow0 * SW - g.pw;      // input column of span byte 0
+    // span bytes lo .. hi - 1 lie inside the row
+    const int lo = max(0, -s), hi = min(SPAN, g.iw - s);
+    unsigned keep[NA];  // 0xff for every byte of span dword k that lies inside the row
+#pragma unroll
+    for (int k = 0; k < NA; ++k) {
+        const int b0 = min(max(lo - 4 * k, 0), 4), b1 = min(max(hi - 4 * k, 0), 4);
+        const unsigned below1 = b1 >= 4 ? 0xffffffffu : (1u << (8 * b1)) - 1u;
+        const unsigned below0 = b0 >= 4 ? 0xffffffffu : (1u << (8 * b0)) - 1u;
+        keep[k] = below1 & ~below0;
+    }
+    const int8_t* const in_plane = src + (size_t)plane * g.ih * g.iw;
+    const unsigned neutral = IS_MAX ? 0x80808080u : 0u;
+    int rows = 0;
+    uint32_t d[WW][NA + 1];
+    unsigned shift[WW];
+    bool row_ok[WW];
+#pragma unroll
+    for (int fh = 0; fh < WW; ++fh) {
+        const unsigned ih = (unsigned)((int)oh * g.sh + fh - g.ph);
+        row_ok[fh] = ih < (unsigned)g.ih && hi > lo;
+        rows += ih < (unsigned)g.ih ? 1 : 0;
+        const int8_t* a = in_plane + (ptrdiff_t)(row_ok[fh] ? ih : 0u) * g.iw + s;
+        const int sh = (int)((uintptr_t)a & 3u);
+        shift[fh] = (unsigned)sh;
+        const uint32_t* p0 = (const uint32_t*)(a - sh);
+        // loaded dword k holds span bytes 4k - sh .. 4k - sh + 3
+#pragma unroll
+        for (int k = 0; k <= NA; ++k)
+            d[fh][k] = row_ok[fh] && 4 * k - sh + 3 >= lo && 4 * k - sh < hi ? p0[k] : 0u;
+    }
+    pool_s2 ev[NA], od[NA];  // bytes 0 / 2 and 1 / 3 of each span dword, combined over the rows
+    const short init = IS_MAX ? -128 : 0;
+#pragma unroll
+    for (int k = 0; k < NA; ++k)
+        ev[k] = od[k] = pool_s2{init, init};
+#pragma unroll
+    for (int fh = 0; fh < WW; ++fh) {
+        if (!row_ok[fh])
+            continue;
+#pragma unroll
+        for (int k = 0; k < NA; ++k) {
+            unsigned v = __builtin_amdgcn_alignbyte(d[fh][k + 1], d[fh][k], shift[fh]);
+            v = (v & keep[k]) | (neutral & ~keep[k]);
+            const pool_s2 w = __builtin_bit_cast(pool_s2, v);
+            const pool_s2 e = (w << 8) >> 8, odd = w >> 8;
+            ev[k] = IS_MAX ? __builtin_elementwise_max(ev[k], e) : ev[k] + e;
+            od[k] = IS_MAX ? __builtin_elementwise_max(od[k], odd) : od[k] + odd;
+        }
+    }
+    int o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        int acc = IS_MAX ? -128 : 0;
+#pragma unroll
+        for (int fw = 0; fw < WW; ++fw) {
+            const int j = k * SW + fw;  // byte of the span
+            const int v = (j & 1) ? (int)od[j >> 2][(j >> 1) & 1] : (int)ev[j >> 2][(j >> 1) & 1];
+            acc = IS_MAX ? max(acc, v) : acc + v;
+        }
+        if (IS_MAX) {
+            o[k] = acc;
+        } else if (g.mode == MEGCC_POOL_AVERAGE) {
+            o[k] = (int)roundf((float)acc / (float)(g.wh * g.ww));
+        } else {
+            // taps inside the image: `rows` window rows x the window columns inside the row
+            const int c0 = s + k * SW;
+            const int cols = min(g.iw, c0 + WW) - max(0, c0);
+            o[k] = (int)roundf((float)acc / (float)(rows * cols));
+        }
+    }
+    int8_t* out = dst + ((size_t)plane * g.oh + oh) * g.ow + ow0;
+    if (dword_store && nvalid == 4) {
+        *(uint32_t*)out = pack4(o[0], o[1], o[2], o[3]);
+    } else {
+        for (int k = 0; k < nvalid; ++k)
+            out[k] = (int8_t)o[k];
+    }
+}
+
 // MAX 2x2 stride 2 without padding on NCHW (kernel_pooling_MAX_NCHW_p0x0_s2x2_w2x2_qsi8qsi8): a
 // thread makes 4 neighbouring outputs of a row = one dword, from 8 bytes of each of the two input
 // rows (two 8-byte loads instead of 16 single bytes). Needs IW % 8 == 0 and aligned tensors.
@@ -176,7 +282,6 @@ __global__ void __launch_bounds__(256) pool_nchw_max2x2_kernel(
 // in v_pk_max_i16, and one v_perm puts the low bytes of the two results back together:
 // 20 vector instructions per output dword instead of 40 byte extractions and maxima, and no
 // division in the index arithmetic beyond two by run-time constants. Needs IW % 8 == 0.
-typedef short pool_s2 __attribute__((ext_vector_type(2)));
 typedef unsigned pool_v4u __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ unsigned max4_bytes(unsigned a, unsigned b, unsigned c, unsigned d) {
@@ -286,6 +391,31 @@ extern "C" TinyNNStatus megcc_gfx950_pooling(
         hipLaunchKernelGGL(pool_nchw_max2x2_kernel, dim3((items + 255) / 256), dim3(256), 0, stream(),
                            (const uint2*)src->ptr, (uint32_t*)dst->ptr, items, g.oh, g.ow / 4);
     } else {
+        // four outputs of a row per thread for the common window widths and strides
+        const int owg = (g.ow + 3) / 4;
+        const size_t items = (size_t)g.n * g.c * g.oh * owg;
+        void (*rows_kernel)(PoolGeom, const int8_t*, int8_t*, unsigned, int, FastDiv, FastDiv, int) = nullptr;
+        const bool mx = g.mode == MEGCC_POOL_MAX;
+#define MG_POOL_ROWS(W_, S_) (mx ? pool_nchw_rows_kernel<W_, S_, true> : pool_nchw_rows_kernel<W_, S_, false>)
+        if (g.ww == 3 && g.sw == 2)
+            rows_kernel = MG_POOL_ROWS(3, 2);
+        else if (g.ww == 2 && g.sw == 2)
+            rows_kernel = MG_POOL_ROWS(2, 2);
+        else if (g.ww == 3 && g.sw == 1)
+            rows_kernel = MG_POOL_ROWS(3, 1);
+        else if (g.ww == 2 && g.sw == 1)
+            rows_kernel = MG_POOL_ROWS(2, 1);
+        else if (g.ww == 5 && g.sw == 1)
+            rows_kernel = MG_POOL_ROWS(5, 1);
+#undef MG_POOL_ROWS
+        if (rows_kernel && !options().no_poolrows && g.ow >= 8 && g.wh == g.ww && items < (1ull << 31) && (size_t)g.n * g.c * g.oh < (1ull << 31)) {
+            const int dword_store = ((uintptr_t)dst->ptr & 3) == 0 && (g.ow & 3) == 0;
+            hipLaunchKernelGGL(rows_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream(), g,
+                               (const int8_t*)src->ptr, (int8_t*)dst->ptr, (unsigned)items, owg,
+                               make_fastdiv(owg), make_fastdiv(g.oh), dword_store);
+            note_kernel("pool_nchw_rows", g.ww, g.sw);
+            return check_launch("pooling");
+        }
         unsigned blocks = min(ceil_div(total, 256), 1u << 20);
         hipLaunchKernelGGL(pool_nchw_q8_kernel, dim3(blocks), dim3(256), 0, stream(), g,
                            (const int8_t*)src->ptr, (int8_t*)dst->ptr);

@@ -278,23 +278,26 @@ struct ConvKernel : KernelFuncBase {
         const int ks = taps <= 2 ? 4 : taps <= 4 ? 2 : 1;
         ss << "    const long P = (long)src.dims[0] * oh * ow, oc = (long)flt.dims[0] * " << r
            << ", ic = (long)src.dims[1] * " << r << ";\n";
-        // NCHW with spatial extent runs as relayout -> NCHW44 kernel -> relayout (conv_api.hip):
-        // both NCHW44 copies live in the workspace, after the split-K room
+        // NCHW with spatial extent runs as relayout -> NCHW44 kernel -> relayout (conv_api.hip): both
+        // NCHW44 copies live in the workspace, after the split-K room, their channel counts padded to
+        // a multiple of 4 (then the bias gets a padded copy too)
         if (fmt == "NCHW")
             ss << "    const int spatial = !(src.dims[2] == 1 && src.dims[3] == 1 && " << taps << " == 1);\n"
-               << "    if (spatial && ((ic & 3) || (oc & 3))) {\n        *workspace = 0;\n        return TinyNN_SUCCESS;\n    }\n";
+               << "    const long icp = spatial ? (ic + 3) & ~3L : ic, ocp = spatial ? (oc + 3) & ~3L : oc;\n";
+        else
+            ss << "    const long icp = ic, ocp = oc;\n";
         ss << "    *workspace = 0;\n"
-           << "    if ((ic & 3) == 0 && P > 0) {\n"
-           << "        const long stages = ((ic + 31) / 32 + " << ks - 1 << ") / " << ks << ";\n"
-           << "        const long bm = oc <= 64 || ((P + 127) / 128) * ((oc + 127) / 128) < 64 ? 64 : 128;\n"
-           << "        const long tiles = ((P + 127) / 128) * ((oc + bm - 1) / bm);\n"
+           << "    if ((icp & 3) == 0 && P > 0) {\n"
+           << "        const long stages = ((icp + 31) / 32 + " << ks - 1 << ") / " << ks << ";\n"
+           << "        const long bm = ocp <= 64 || ((P + 127) / 128) * ((ocp + 127) / 128) < 64 ? 64 : 128;\n"
+           << "        const long tiles = ((P + 127) / 128) * ((ocp + bm - 1) / bm);\n"
            << "        long s = 1;\n"
            << "        if (tiles < 128 && stages >= 2) {\n"
            << "            s = (512 + tiles - 1) / tiles;\n"
            << "            if (s > stages) s = stages;\n"
            << "            if (s > 16) s = 16;\n"
            << "        }\n"
-           << "        if (s > 1) *workspace = (size_t)s * P * ((oc + 3) & ~3L) * 4;\n";
+           << "        if (s > 1) *workspace = (size_t)s * P * ((ocp + 3) & ~3L) * 4;\n";
         // a strided 1x1 convolution first gathers the pixels it keeps (conv_api.hip)
         if (fmt == "NCHW44" && taps == 1 && c->getAttrUInt("pad_h") == 0 && c->getAttrUInt("pad_w") == 0 &&
             (c->getAttrUInt("stride_h") > 1 || c->getAttrUInt("stride_w") > 1))
@@ -302,8 +305,9 @@ struct ConvKernel : KernelFuncBase {
         if (fmt == "NCHW")
             ss << "        if (spatial)\n"
                << "            *workspace = ((*workspace + 255) & ~(size_t)255) +\n"
-               << "                         (((size_t)src.dims[0] * ic * src.dims[2] * src.dims[3] + 255) & ~(size_t)255) +\n"
-               << "                         (size_t)P * oc;\n";
+               << "                         (((size_t)src.dims[0] * icp * src.dims[2] * src.dims[3] + 255) & ~(size_t)255) +\n"
+               << "                         (((size_t)P * ocp + 255) & ~(size_t)255) +\n"
+               << "                         (ocp != oc ? (((size_t)ocp * 4 + 255) & ~(size_t)255) : 0);\n";
         ss << "    }\n"
            << "    return TinyNN_SUCCESS;\n}\n";
         return ss.str();

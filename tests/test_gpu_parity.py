@@ -147,6 +147,13 @@ LIVE = [
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 30, 34, 8, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),  # generic path (IW % 4 != 0)
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
     # the 2x2 stride-2 maximum on packed halves (rows of 8, 16 pixels), and rows it does not take
+    # dense NCHW layers whose channel counts are no multiple of 4: padded copies around the NCHW44
+    # kernel (input lanes, output lanes and the bias padded independently)
+    ConvCase(A.FMT_NCHW, A.DENSE, 2, 6, 20, 24, 10, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(54))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 3, 3, 31, 17, 8, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(27))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 2, 16, 14, 14, 7, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(16))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 5, 1, 12, 12, 1, 3, 1, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(9))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 4, 33, 28, 28, 65, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(297)), bias=False),
     # 1x1 with 1024 input channels between 2048 and 4096 pixels: the workgroup-shared pointwise
     # kernel (1024 -> 512), half-filled tiles of the LDS-direct kernel (1024 -> 256)
     ConvCase(A.FMT_NCHW44, A.DENSE, 64, 1024, 7, 7, 512, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(1024))),
@@ -159,6 +166,17 @@ LIVE = [
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 3, 5, 10, 24, 2, 2, 0),   # 8-byte row pieces, odd plane count
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 3, 5, 11, 24, 2, 2, 0),   # odd height: the generic kernel
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 7, 10, 20, 2, 2, 0),   # IW % 8 != 0: the generic kernel
+    # four outputs of a row per thread (NCHW): padded and unpadded borders, rows of every alignment
+    # (odd widths), output rows that are no multiple of 4, all three modes, window height != width
+    # is not expressible here but the height is a run-time loop
+    PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 16, 112, 112, 3, 2, 1),
+    PoolCase(A.FMT_NCHW, A.POOL_MAX, 3, 5, 57, 113, 3, 2, 1),
+    PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 3, 30, 41, 3, 2, 0),
+    PoolCase(A.FMT_NCHW, A.POOL_AVERAGE, 2, 7, 28, 35, 3, 1, 1),
+    PoolCase(A.FMT_NCHW, A.POOL_AVERAGE_COUNT_EXCLUDE_PADDING, 2, 7, 28, 35, 3, 1, 1),
+    PoolCase(A.FMT_NCHW, A.POOL_AVERAGE_COUNT_EXCLUDE_PADDING, 3, 4, 19, 50, 2, 2, 1),
+    PoolCase(A.FMT_NCHW, A.POOL_AVERAGE, 1, 9, 33, 47, 2, 1, 0),
+    PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 6, 20, 37, 5, 1, 2),
     PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE, 5, 1024, 7, 7, 7, 7, 0),
     PoolCase(A.FMT_NCHW, A.POOL_AVERAGE, 5, 1024, 7, 7, 7, 7, 0),
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 3, 64, 13, 13, 13, 13, 0),  # one output pixel per plane
@@ -508,6 +526,8 @@ OLDER = [
     # channel-wise NCHW through the NCHW44 detour (what rows that are no multiple of 4 still use)
     ("nodwnchw", ConvCase(A.FMT_NCHW, A.GROUP, 4, 32, 56, 56, 32, 3, 1, 1, A.RELU,
                           scales=(0.02, 0.01, unsat(9)))),
+    # NCHW pooling one output per thread (what windows wider than 5 or non-square ones still use)
+    ("nopoolrows", PoolCase(A.FMT_NCHW, A.POOL_AVERAGE_COUNT_EXCLUDE_PADDING, 2, 5, 29, 37, 3, 2, 1)),
 ]
 
 

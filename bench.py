@@ -188,6 +188,9 @@ def make_workload(name):
     if name == "pool":
         return (PoolCase(abi.FMT_NCHW44, abi.POOL_MAX, 64, 32, 112, 112, 2, 2, 0),
                 "qsi8 maxpool 2x2 s2 NCHW44 N=64 C=32 112x112", "hbm")
+    if name == "pool44_s2":  # the same stem pooling in NCHW44
+        return (PoolCase(abi.FMT_NCHW44, abi.POOL_MAX, 64, 64, 112, 112, 3, 2, 1),
+                "qsi8 maxpool 3x3 s2 p1 NCHW44 N=64 C=64 112x112", "hbm")
     if name in ("pool_nchw", "pool_nchw_s1"):  # the stem pooling of a ResNet-like model kept in NCHW
         w, s = (3, 2) if name == "pool_nchw" else (3, 1)
         return (PoolCase(abi.FMT_NCHW, abi.POOL_MAX, 64, 64, 112, 112, w, s, 1),

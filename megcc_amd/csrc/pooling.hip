@@ -66,6 +66,103 @@ __global__ void __launch_bounds__(256) pool44_q8_kernel(
     }
 }
 
+// NCHW44, square windows of the common widths and strides, rows a multiple of 4 pixels: a thread
+// makes 4 neighbouring output pixels of a row = one 16-byte store. Their windows cover 3 * SW + WW
+// input pixels of each window row, fetched as the aligned 16-byte groups of 4 pixels that contain
+// them (a third of the loads of one dword per tap, and neighbouring lanes 32 or 16 bytes apart
+// instead of every lane on its own stretch; with a row length that is a multiple of 4 a group lies
+// inside the row or outside, so the left / right padding is a group that is not loaded). A
+// pixel's 4 channel bytes are split into even and odd bytes as packed 16-bit halves, the window
+// rows are combined column by column with packed max / add, then the WW columns of each output,
+// and one v_perm puts the bytes back together (MAX). PW: the horizontal padding, which fixes where
+// the span starts inside its first group.
+typedef short pool44_s2 __attribute__((ext_vector_type(2)));
+typedef unsigned pool44_v4u __attribute__((ext_vector_type(4)));
+
+template <int WW, int SW, int PW, bool IS_MAX>
+__global__ void __launch_bounds__(256) pool44_rows_kernel(
+        PoolGeom g, const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, unsigned total, int owg,
+        FastDiv d_owg, FastDiv d_oh, int vec_store) {
+    const unsigned i = blockIdx.x * 256u + threadIdx.x;  // (plane set, oh, group of 4 ow)
+    if (i >= total)
+        return;
+    const unsigned row = fdiv(i, d_owg), q = i - row * (unsigned)owg;
+    const unsigned plane = fdiv(row, d_oh), oh = row - plane * (unsigned)g.oh;
+    const int ow0 = (int)q * 4;
+    const int nvalid = min(4, g.ow - ow0);
+    constexpr int SPAN = 3 * SW + WW;
+    constexpr int SH = (4 - (PW & 3)) & 3;     // span pixel 0 inside its group of 4
+    constexpr int NCH = (SH + SPAN + 3) / 4;   // groups of 4 pixels per window row
+    const int s = ow0 * SW - PW;               // input column of span pixel 0
+    const int c0 = s - SH;                     // first column of the first group (a multiple of 4)
+    const uint32_t* const in_plane = src + (size_t)plane * g.ih * g.iw;
+    const short init = IS_MAX ? -128 : 0;
+    const unsigned neutral = IS_MAX ? 0x80808080u : 0u;
+    int rows = 0;
+    uint32_t d[WW][NCH * 4];
+#pragma unroll
+    for (int fh = 0; fh < WW; ++fh) {
+        const unsigned ih = (unsigned)((int)oh * g.sh + fh - g.ph);
+        const bool row_ok = ih < (unsigned)g.ih;
+        rows += row_ok ? 1 : 0;
+        const uint32_t* in_row = in_plane + (size_t)(row_ok ? ih : 0u) * g.iw;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const bool ok = row_ok && (unsigned)(c0 + 4 * c) < (unsigned)g.iw;
+            pool44_v4u v = {neutral, neutral, neutral, neutral};
+            if (ok)
+                v = *(const pool44_v4u*)(in_row + c0 + 4 * c);
+            d[fh][4 * c] = v.x;
+            d[fh][4 * c + 1] = v.y;
+            d[fh][4 * c + 2] = v.z;
+            d[fh][4 * c + 3] = v.w;
+        }
+    }
+    pool44_s2 ev[SPAN], od[SPAN];  // channels 0 / 2 and 1 / 3 of each span column, combined over the rows
+#pragma unroll
+    for (int j = 0; j < SPAN; ++j)
+        ev[j] = od[j] = pool44_s2{init, init};
+#pragma unroll
+    for (int fh = 0; fh < WW; ++fh)
+#pragma unroll
+        for (int j = 0; j < SPAN; ++j) {
+            const pool44_s2 w = __builtin_bit_cast(pool44_s2, d[fh][j + SH]);
+            const pool44_s2 e = (w << 8) >> 8, odd = w >> 8;
+            ev[j] = IS_MAX ? __builtin_elementwise_max(ev[j], e) : ev[j] + e;
+            od[j] = IS_MAX ? __builtin_elementwise_max(od[j], odd) : od[j] + odd;
+        }
+    uint32_t out[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        pool44_s2 e = ev[k * SW], o = od[k * SW];
+#pragma unroll
+        for (int fw = 1; fw < WW; ++fw) {
+            e = IS_MAX ? __builtin_elementwise_max(e, ev[k * SW + fw]) : e + ev[k * SW + fw];
+            o = IS_MAX ? __builtin_elementwise_max(o, od[k * SW + fw]) : o + od[k * SW + fw];
+        }
+        if (IS_MAX) {
+            // bytes: e.lo, o.lo, e.hi, o.hi
+            out[k] = __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, o), __builtin_bit_cast(unsigned, e), 0x06020400u);
+        } else {
+            float div = g.count_div;
+            if (g.mode != MEGCC_POOL_AVERAGE) {
+                const int x0 = s + k * SW;
+                const int cols = min(g.iw, x0 + WW) - max(0, x0);
+                div = (float)(1.0 / (double)(uint32_t)max(rows * cols, 1));
+            }
+            out[k] = pack4(fp32_to_int8((float)(int)e[0] * div), fp32_to_int8((float)(int)o[0] * div),
+                           fp32_to_int8((float)(int)e[1] * div), fp32_to_int8((float)(int)o[1] * div));
+        }
+    }
+    uint32_t* o = dst + ((size_t)plane * g.oh + oh) * g.ow + ow0;
+    if (vec_store && nvalid == 4) {
+        *(pool44_v4u*)o = pool44_v4u{out[0], out[1], out[2], out[3]};
+    } else {
+        for (int k = 0; k < nvalid; ++k)
+            o[k] = out[k];
+    }
+}
+
 // NCHW44, one output pixel per plane (global pooling, e.g. the 7x7 average in front of a
 // classifier): 8 lanes per plane group instead of one thread, so that a wave reads 8 consecutive
 // planes as one contiguous stretch; integer max / sum are combined across the 8 lanes, the last
@@ -380,6 +477,36 @@ extern "C" TinyNNStatus megcc_gfx950_pooling(
                                make_fastdiv(g.ow / 4), g.ow / 4);
             note_kernel("pool44_max2x2");
             return check_launch("pooling");
+        }
+        {
+            // four output pixels of a row per thread for the common window widths and strides
+            const int owg = (g.ow + 3) / 4;
+            const size_t items = (size_t)planes * g.oh * owg;
+            void (*rk)(PoolGeom, const uint32_t*, uint32_t*, unsigned, int, FastDiv, FastDiv, int) = nullptr;
+            const bool mx = g.mode == MEGCC_POOL_MAX;
+#define MG_POOL44_ROWS(W_, S_)                                                                        \
+    (g.pw == 0   ? (mx ? pool44_rows_kernel<W_, S_, 0, true> : pool44_rows_kernel<W_, S_, 0, false>)     \
+     : g.pw == 1 ? (mx ? pool44_rows_kernel<W_, S_, 1, true> : pool44_rows_kernel<W_, S_, 1, false>)     \
+                 : nullptr)
+            if (g.ww == 3 && g.sw == 2)
+                rk = MG_POOL44_ROWS(3, 2);
+            else if (g.ww == 2 && g.sw == 2)
+                rk = MG_POOL44_ROWS(2, 2);
+            else if (g.ww == 3 && g.sw == 1)
+                rk = MG_POOL44_ROWS(3, 1);
+            else if (g.ww == 2 && g.sw == 1)
+                rk = MG_POOL44_ROWS(2, 1);
+#undef MG_POOL44_ROWS
+            if (rk && !options().no_poolrows && g.wh == g.ww && g.ow >= 4 && (g.iw & 3) == 0 &&
+                ((uintptr_t)src->ptr & 15) == 0 && items < (1ull << 31) &&
+                (size_t)planes * g.oh < (1ull << 31)) {
+                const int vec_store = ((uintptr_t)dst->ptr & 15) == 0 && (g.ow & 3) == 0;
+                hipLaunchKernelGGL(rk, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream(), g,
+                                   (const uint32_t*)src->ptr, (uint32_t*)dst->ptr, (unsigned)items, owg,
+                                   make_fastdiv(owg), make_fastdiv(g.oh), vec_store);
+                note_kernel("pool44_rows", g.ww, g.sw);
+                return check_launch("pooling");
+            }
         }
         unsigned blocks = min(ceil_div(total / 4, 256), 1u << 20);
         hipLaunchKernelGGL(pool44_q8_kernel, dim3(blocks), dim3(256), 0, stream(), g,

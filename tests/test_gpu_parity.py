@@ -166,6 +166,14 @@ LIVE = [
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 3, 5, 10, 24, 2, 2, 0),   # 8-byte row pieces, odd plane count
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 3, 5, 11, 24, 2, 2, 0),   # odd height: the generic kernel
     PoolCase(A.FMT_NCHW, A.POOL_MAX, 2, 7, 10, 20, 2, 2, 0),   # IW % 8 != 0: the generic kernel
+    # four output pixels of a row per thread (NCHW44)
+    PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 16, 57, 44, 3, 2, 1),
+    PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 64, 112, 112, 3, 2, 1),
+    PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE, 2, 8, 14, 16, 3, 1, 1),
+    PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE_COUNT_EXCLUDE_PADDING, 3, 8, 15, 24, 3, 2, 1),
+    PoolCase(A.FMT_NCHW44, A.POOL_AVERAGE_COUNT_EXCLUDE_PADDING, 1, 4, 9, 12, 2, 1, 0),
+    PoolCase(A.FMT_NCHW44, A.POOL_MAX, 3, 12, 10, 20, 2, 2, 1),
+    PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 16, 57, 43, 3, 2, 1),  # rows of 43 pixels: the generic kernel
     # four outputs of a row per thread (NCHW): padded and unpadded borders, rows of every alignment
     # (odd widths), output rows that are no multiple of 4, all three modes, window height != width
     # is not expressible here but the height is a run-time loop
@@ -528,6 +536,7 @@ OLDER = [
                           scales=(0.02, 0.01, unsat(9)))),
     # NCHW pooling one output per thread (what windows wider than 5 or non-square ones still use)
     ("nopoolrows", PoolCase(A.FMT_NCHW, A.POOL_AVERAGE_COUNT_EXCLUDE_PADDING, 2, 5, 29, 37, 3, 2, 1)),
+    ("nopoolrows", PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 16, 57, 44, 3, 2, 1)),
 ]
 
 

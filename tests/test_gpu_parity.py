@@ -143,6 +143,12 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 1, 40, 8, 3, 1, 1, A.IDENTITY, scales=(0.5, 0.5, 0.5)),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 224, 224, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 3, 3, 64, 48, 24, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(27))),
+    # the matrix-core form (32 / 64 output channels): ragged last tile, rows of 4 and 8 columns (first
+    # and last column next to each other), H_SWISH through the literal sequence, no bias
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 3, 3, 18, 28, 64, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(27))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 5, 3, 6, 4, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, 0.05)),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 10, 8, 32, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(27))),
+    ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 224, 224, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27)), bias=False),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 32, 36, 8, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(27))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 30, 34, 8, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),  # generic path (IW % 4 != 0)
     PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 32, 112, 112, 2, 2, 0),
@@ -535,6 +541,8 @@ OLDER = [
     ("nodwnchw", ConvCase(A.FMT_NCHW, A.GROUP, 4, 32, 56, 56, 32, 3, 1, 1, A.RELU,
                           scales=(0.02, 0.01, unsat(9)))),
     # NCHW pooling one output per thread (what windows wider than 5 or non-square ones still use)
+    ("nofirstmfma", ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 224, 224, 32, 3, 2, 1, A.RELU,
+                             scales=(0.02, 0.01, unsat(27)))),
     ("nopoolrows", PoolCase(A.FMT_NCHW, A.POOL_AVERAGE_COUNT_EXCLUDE_PADDING, 2, 5, 29, 37, 3, 2, 1)),
     ("nopoolrows", PoolCase(A.FMT_NCHW44, A.POOL_MAX, 2, 16, 57, 44, 3, 2, 1)),
 ]

@@ -576,6 +576,27 @@ def test_softmax_refuses_rows_beyond_its_limit():
         runtime.PreparedOp(case.desc(), ins, outs).launch()
 
 
+@pytest.mark.parametrize("src_off,dst_off", [(1, 0), (2, 3), (3, 1)])
+@pytest.mark.parametrize("mode", [A.POOL_MAX, A.POOL_AVERAGE_COUNT_EXCLUDE_PADDING])
+def test_nchw_pooling_on_unaligned_tensors(mode, src_off, dst_off):
+    """the row kernel fetches aligned dwords around a window and shifts: tensors that start at any
+    byte, outputs stored byte by byte when their rows cannot be stored as dwords, and not a byte
+    written outside the destination"""
+    case = PoolCase(A.FMT_NCHW, mode, 2, 3, 21, 32, 3, 2, 1)
+    arrays = case.gen(seed=3)
+    want = case.run_port(arrays)
+    src = arrays["src"]
+    flat = np.zeros(src.size + 8, np.int8)
+    flat[src_off:src_off + src.size] = src.ravel()
+    ins = [cases.TensorSpec(b"src", src.shape, A.QINT8, case.scale, flat, offset=src_off)]
+    outs = [cases.TensorSpec(b"dst", want.shape, A.QINT8, case.scale, offset=dst_off,
+                             storage=(want.size + 8,))]
+    got = runtime.run_symbol(case.symbol(), ins, outs)
+    assert runtime.last_kernel().startswith("pool_nchw_rows")
+    np.testing.assert_array_equal(got[dst_off:dst_off + want.size].reshape(want.shape), want)
+    assert (got[:dst_off] == 0x5A).all() and (got[dst_off + want.size:] == 0x5A).all()
+
+
 @pytest.mark.parametrize("switch,case", OLDER, ids=["%s-%r" % (s, c) for s, c in OLDER])
 def test_older_kernels_still_agree(switch, case):
     port.set_threads(8)

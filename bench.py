@@ -380,6 +380,38 @@ def case_bytes(case):
     return sum(s.nbytes for s in ins) + sum(s.nbytes for s in outs)
 
 
+MFMA_OPS = 2 * 32 * 32 * 32  # one v_mfma_i32_32x32x32_i8
+
+
+def bench_mfma_only(mfma_per_simd, launches):
+    """Launches that issue nothing but v_mfma_i32_32x32x32_i8 (operands in registers), timed by the
+    library with HIP events, for three operand distributions: the board is power-limited and the
+    rate depends on the operand values."""
+    import ctypes
+    from megcc_amd import runtime
+    lib = runtime.lib()
+    lib.megcc_gfx950_probe_mfma_i8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                               ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    lib.megcc_gfx950_probe_mfma_i8.restype = ctypes.c_int
+    res = {}
+    for kind, name in ((1, "uniform_int8"), (0, "zeros"), (2, "relu_activations_normal_weights")):
+        us, n = ctypes.c_double(), ctypes.c_double()
+        st = lib.megcc_gfx950_probe_mfma_i8(kind, mfma_per_simd, launches, ctypes.byref(us), ctypes.byref(n))
+        if st != 0:
+            raise SystemExit("megcc_gfx950_probe_mfma_i8: status %d: %s" % (st, lib.megcc_gfx950_last_error().decode()))
+        res[name] = {"us_per_launch": round(us.value, 2), "tops": round(n.value * MFMA_OPS / us.value / 1e6, 1)}
+    v = res["uniform_int8"]
+    return {"metric": "int8_mfma_only_tops", "value": v["tops"], "unit": "TOP/s", "n_gpus": 1, "steps": launches,
+            "warmup": launches, "ms_per_step": round(v["us_per_launch"] * 1e-3, 5), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+            "config": {"workload": "v_mfma_i32_32x32x32_i8 only, %d per SIMD per launch (the default "
+                       "workload's count), operands in registers" % mfma_per_simd,
+                       "abi": "megcc_gfx950_probe_mfma_i8"},
+            "roofline": {"bound": "mfma", "achieved": v["tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                         "frac": round(v["tops"] / PEAK_INT8_TOPS, 4), "traffic": None},
+            **res}
+
+
 def cpu_baseline(full_case, unit="TOP/s"):
     """One host core on a bounded sample of the same workload, through the reference's own
     generated kernel where oracle/_ref has it: batch 1 of a batched convolution, 64 rows of a
@@ -459,6 +491,10 @@ def main():
                      "chain512_s2": (512, 14, 2)}[args.workload]
         print(json.dumps(bench_chain(c, hw, st, args.steps, args.warmup)))
         return
+    if args.workload == "mfma_only":
+        # as many MFMAs per SIMD as the default workload's launch has, spread evenly over 256 CUs
+        print(json.dumps(bench_mfma_only(int(make_workload("conv")[0].ops() / MFMA_OPS / (4 * 256)), args.steps)))
+        return
     case, desc, bound = make_workload(args.workload)
     arrays = case.gen(seed=0)
     ins, outs = case.specs(arrays)
@@ -511,6 +547,11 @@ def main():
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
     roof["kernel_ms"] = round(kern_ms, 5)
     roof["algorithmic_per_launch"] = ops if bound == "mfma" else nbytes
+    if args.workload == "conv":
+        # what the matrix cores alone deliver on this board for the same number of MFMAs per SIMD and
+        # the same operand distribution (uniform random int8): no loads, no LDS, no epilogue
+        mo = bench_mfma_only(int(ops / MFMA_OPS / (4 * 256)), 300)
+        roof["mfma_only_same_operands"] = {k: mo[k] for k in ("uniform_int8", "zeros")}
 
     out = {
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1,

@@ -518,6 +518,14 @@ const char* megcc_gfx950_last_kernel(void);
  * same names in capitals behind MEGCC_ are read from the environment once, at first use.
  * Unknown names return TinyNN_ERROR_NO_FOUND. */
 TinyNNStatus megcc_gfx950_set_option(const char* name, int value);
+/* Measurement aid (no counterpart in the reference): the time of a launch that does nothing but
+ * v_mfma_i32_32x32x32_i8 - operands in registers, `mfma_per_simd` MFMAs on every SIMD of the chip -
+ * averaged over `launches` launches after as many untimed ones. operand_kind 0: zeros, 1: uniform
+ * random int8 (the operand distribution of the reference's benchmarks), 2: ReLU-like activations
+ * against normally distributed weights. The board is power-limited and the rate depends on the
+ * operand values; bench.py --workload mfma_only prints it beside the published peak. */
+TinyNNStatus megcc_gfx950_probe_mfma_i8(
+        int operand_kind, int mfma_per_simd, int launches, double* us_per_launch, double* mfma_per_launch);
 
 /* ------------------------------------------------------------------------------------------
  * In-memory model runtime: MegCC's static memory plan on one HBM arena. The calls mirror what the

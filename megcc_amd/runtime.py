@@ -106,7 +106,7 @@ EXPORTS = [
     "megcc_gfx950_malloc", "megcc_gfx950_free", "megcc_gfx950_memcpy_h2d",
     "megcc_gfx950_memcpy_d2h", "megcc_gfx950_memset", "megcc_gfx950_wait",
     "megcc_gfx950_stream", "megcc_gfx950_last_error", "megcc_gfx950_last_kernel",
-    "megcc_gfx950_set_option",
+    "megcc_gfx950_set_option", "megcc_gfx950_probe_mfma_i8",
     "megcc_gfx950_model_create", "megcc_gfx950_model_destroy", "megcc_gfx950_model_add_tensor",
     "megcc_gfx950_model_add_weight", "megcc_gfx950_model_add_alias", "megcc_gfx950_model_add_view",
     "megcc_gfx950_model_add_opr", "megcc_gfx950_model_add_opr_desc",

@@ -711,3 +711,21 @@ def test_layers_that_require_their_workspace_say_so(case):
     assert (op.result().view(np.uint8) == cases.POISON).all(), "nothing may have been written"
     op.launch()
     compare(op.result(), case.run_port(arrays), repr(case))
+
+
+def test_mfma_only_probe_reports_a_plausible_rate():
+    """the measurement aid behind bench.py's mfma_only figures: argument checks, the MFMA count of
+    a launch, and a rate between a tenth of the published int8 peak and the peak itself"""
+    import ctypes as C
+    lib = runtime.lib()
+    lib.megcc_gfx950_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double),
+                                               C.POINTER(C.c_double)]
+    us, n = C.c_double(), C.c_double()
+    assert lib.megcc_gfx950_probe_mfma_i8(3, 256, 10, C.byref(us), C.byref(n)) == abi.ERROR_OUT_OF_RANGE
+    assert lib.megcc_gfx950_probe_mfma_i8(1, 256, 0, C.byref(us), C.byref(n)) == abi.ERROR_OUT_OF_RANGE
+    assert lib.megcc_gfx950_probe_mfma_i8(1, 256, 10, None, C.byref(n)) == abi.ERROR_OUT_OF_RANGE
+    for kind in (0, 1, 2):
+        assert lib.megcc_gfx950_probe_mfma_i8(kind, 1024, 20, C.byref(us), C.byref(n)) == 0
+        assert n.value == 256 * 4 * 1024, "256 CUs x 4 SIMDs x 1024 MFMAs"
+        tops = n.value * 65536 / us.value / 1e6
+        assert 500 < tops <= 5000, (kind, us.value, tops)

@@ -271,8 +271,7 @@ static TinyNNStatus conv_first_mfma_launch(
     q.c = make_requant_fast(g.s_src, g.s_flt, g.s_dst).c;
     q.dOW = make_fastdiv(q.OW);
     q.dOHW = make_fastdiv(q.OHW);
-    const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
-                     requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    const bool tab = requant_table_act(g.act) && requant_table_ok(g.s_src, g.s_flt, g.s_dst);
     if (tab)
         q.table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
     const int act = tab ? g.act : -1;
@@ -280,6 +279,7 @@ static TinyNNStatus conv_first_mfma_launch(
 #define MG_CFM(MT_)                                                                                     \
     (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_first_mfma_kernel<MT_, MEGCC_NONLINE_IDENTITY>     \
      : act == MEGCC_NONLINE_RELU   ? (const void*)conv_first_mfma_kernel<MT_, MEGCC_NONLINE_RELU>         \
+     : act == MEGCC_NONLINE_H_SWISH ? (const void*)conv_first_mfma_kernel<MT_, MEGCC_NONLINE_H_SWISH>     \
                                    : (const void*)conv_first_mfma_kernel<MT_, -1>)
     kern = g.oc == 32 ? MG_CFM(1) : MG_CFM(2);
 #undef MG_CFM
@@ -316,12 +316,12 @@ TinyNNStatus conv_first_launch(
     const RequantFast rq = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
     // exact thresholds for the monotone activations; anything else (and extreme scales)
     // evaluates the literal sequence per output
-    const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
-                     requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    const bool tab = requant_table_act(g.act) && requant_table_ok(g.s_src, g.s_flt, g.s_dst);
     static const RequantTable no_table = {};
     const RequantTable& table = tab ? requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst) : no_table;
     auto kern = tab && g.act == MEGCC_NONLINE_IDENTITY ? conv_first_q8_kernel<MEGCC_NONLINE_IDENTITY>
               : tab && g.act == MEGCC_NONLINE_RELU     ? conv_first_q8_kernel<MEGCC_NONLINE_RELU>
+              : tab && g.act == MEGCC_NONLINE_H_SWISH  ? conv_first_q8_kernel<MEGCC_NONLINE_H_SWISH>
                                                        : conv_first_q8_kernel<-1>;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(CF_THREADS), 0, stream(), g, rq,
                        (const int8_t*)src, (const int8_t*)flt, (const int32_t*)bias, (uint32_t*)dst,

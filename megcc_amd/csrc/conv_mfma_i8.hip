@@ -615,7 +615,7 @@ TinyNNStatus conv_mfma_launch(
     q.s_flt = g.s_flt;
     q.s_dst = g.s_dst;
     q.rq = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
-    if (pipe && (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
+    if (pipe && requant_table_act(g.act) && !(fc && g.act == MEGCC_NONLINE_H_SWISH) &&
         requant_table_ok(g.s_src, g.s_flt, g.s_dst))
         q.rq_table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
     q.dOW = make_fastdiv(q.OW);

@@ -240,12 +240,10 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             for (int e = 0; e < 16; ++e)
                 r[e] = requant_conv_rt(q.act, acc[mi][ni][e], q.s_src, q.s_flt, q.s_dst);
         } else {
-            constexpr int LO = ACT == MEGCC_NONLINE_RELU ? 0 : -128;
             int m[16], t[16];
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int f = cvt_floor_i32((float)acc[mi][ni][e] * q.rq.c);
-                m[e] = f < LO ? LO : (f > 126 ? 126 : f);
+                m[e] = requant_table_candidate<ACT>(acc[mi][ni][e], q.rq.c);
                 t[e] = tbl[m[e] + 128];
             }
 #pragma unroll
@@ -416,12 +414,15 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.fixed_lmax = LMAX;
     c.pm = PM ? 1 : 0;
     c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + (DM_BM > 128 ? DM_BM : 128) * 4;
+    c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
         c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
     else if (act == MEGCC_NONLINE_RELU && table_ok)
         c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
-    else
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
+    if constexpr (!FC) {  // (FullyConnected with H_SWISH keeps the literal sequence)
+        if (act == MEGCC_NONLINE_H_SWISH && table_ok)
+            c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_H_SWISH, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
+    }
     return c;
 }
 

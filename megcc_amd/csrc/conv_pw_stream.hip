@@ -350,8 +350,7 @@ TinyNNStatus conv_pw_stream_launch(
     q.s_dst = g.s_dst;
     q.c = make_requant_fast(g.s_src, g.s_flt, g.s_dst).c;
     q.dOHW = make_fastdiv(q.OHW);
-    const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
-                     requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    const bool tab = requant_table_act(g.act) && requant_table_ok(g.s_src, g.s_flt, g.s_dst);
     if (tab)
         q.table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
     const int act = tab ? g.act : -1;
@@ -360,6 +359,7 @@ TinyNNStatus conv_pw_stream_launch(
 #define MG_PW_PICK(KC_, MT_)                                                                      \
     (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_IDENTITY> \
      : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_RELU>     \
+     : act == MEGCC_NONLINE_H_SWISH ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_H_SWISH> \
                                    : (const void*)conv_pw_stream_kernel<KC_, MT_, -1>)
     switch (g.ic / 32) {
         case 1: kern = MG_PW_PICK(1, 2); break;
@@ -376,6 +376,7 @@ TinyNNStatus conv_pw_stream_launch(
 #define MG_PWS_PICK(KC_)                                                                                  \
     (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_share_kernel<KC_, MEGCC_NONLINE_IDENTITY>         \
      : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_share_kernel<KC_, MEGCC_NONLINE_RELU>             \
+     : act == MEGCC_NONLINE_H_SWISH ? (const void*)conv_pw_share_kernel<KC_, MEGCC_NONLINE_H_SWISH>         \
                                    : (const void*)conv_pw_share_kernel<KC_, -1>)
         const void* sk = g.ic == 512 ? MG_PWS_PICK(16) : MG_PWS_PICK(32);
 #undef MG_PWS_PICK

@@ -285,13 +285,13 @@ TinyNNStatus dwconv44_launch(
                    FastDiv, FastDiv, FastDiv, RequantTable);
         // exact thresholds for the monotone activations; anything else (and extreme scales)
         // evaluates the literal sequence per output
-        const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
-                         requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+        const bool tab = requant_table_act(g.act) && requant_table_ok(g.s_src, g.s_flt, g.s_dst);
         static const RequantTable no_table = {};
         const RequantTable& table = tab ? requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst) : no_table;
 #define MG_DW_PICK(S_, R_, G_)                                                                      \
     (tab && g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_IDENTITY, R_, G_> \
      : tab && g.act == MEGCC_NONLINE_RELU   ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_RELU, R_, G_>     \
+     : tab && g.act == MEGCC_NONLINE_H_SWISH ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_H_SWISH, R_, G_> \
                                             : dwconv44_3x3_kernel<S_, -1, R_, G_>)
         const bool ragged = (g.iw % (4 * g.sh)) != 0;
         if (g.sh == 1 && R == 2)

@@ -1,4 +1,8 @@
-// qsi8 depthwise 3x3 (pad 1, stride 1 or 2) in NCHW44 on the matrix cores.
+// qsi8 depthwise 3x3 (pad 1, stride 1), 5x5 (pad 2) and 7x7 (pad 3, both stride 1 or 2) in NCHW44 on
+// the matrix cores. The text below describes the 3x3 case; an F x F filter with pad F / 2 has F
+// filter rows, filter columns 0 .. F - 1 in the band, and still fits the same S + 1 aligned K steps
+// (a group of 8 output pixels from x0 on reads input pixels S*x0 - F/2 .. S*x0 + 7*S + F/2, all of
+// them inside S*x0 - 4 .. S*x0 + 8*S + 3 while F/2 <= 3).
 //
 // A depthwise layer moves two bytes per output and has to requantise every output exactly, which
 // costs 7 vector instructions and a table look-up (epilogue.h). Done with v_dot4 the multiply-adds
@@ -47,7 +51,7 @@ namespace mg {
 
 struct DwMfmaParams {
     const uint32_t* src;
-    const uint32_t* flt;   // [C/4][3][3] dwords of 4 channel bytes
+    const uint32_t* flt;   // [C/4][F][F] dwords of 4 channel bytes
     const int32_t* bias;   // or nullptr
     uint32_t* dst;
     int src_bytes;
@@ -72,13 +76,15 @@ static constexpr int DWM_ROWS = 1;
 // S: stride (only 1 is instantiated: with stride 2 the layer reads four bytes per byte written and
 // the v_dot4 kernel of dwconv.hip already runs at the rate of a copy - measured 7.8 us against
 // 9.8 us for this one on N=64 C=32 112x112). RAGGED: IW is not a multiple of 4, so the last 16-byte load of a row runs into the
-// next row and is masked. ACT: IDENTITY / RELU use the threshold table, -1 evaluates the literal
-// sequence with the run-time activation.
-template <int S, bool RAGGED, int ACT>
+// next row and is masked. ACT: IDENTITY / RELU / H_SWISH use the threshold table, -1 evaluates the literal
+// sequence with the run-time activation. F: filter rows = filter columns (3, 5 or 7; pad F / 2).
+template <int S, bool RAGGED, int ACT, int F = 3>
 __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
+    static_assert(F == 3 || F == 5 || F == 7, "the band must fit S + 1 K steps: pad <= 3");
+    constexpr int PAD = F / 2;
     constexpr int NS = S + 1;            // K steps a group of 8 output pixels reads
     constexpr int R = DWM_ROWS;          // output rows per lane and tile
-    constexpr int IR = (R - 1) * S + 3;  // input rows they read
+    constexpr int IR = (R - 1) * S + F;  // input rows they read
     __shared__ int tbl[REQUANT_TABLE_ENTRIES];
     const int tid = threadIdx.x, lane = tid & 63;
     if (ACT >= 0) {
@@ -102,21 +108,28 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
     // row m = lane & 31 = (output pixel m / 4, channel m % 4); the lane's 16 K bytes are input
     // pixels 4 * kg + j (j = 0..3) of the K step, 4 channel bytes each. K step s starts 4 pixels
     // left of S * x0, so input pixel (s, j) meets output pixel px through filter column
-    // fw = 8 * s + 4 * kg + j - 4 - S * px + 1.
-    v4i A[3][NS];
+    // fw = 8 * s + 4 * kg + j - 4 - S * px + PAD.
+    v4i A[F][NS];
     {
         const int px = col_l >> 2, ch = col_l & 3;
         const unsigned keep = 0xffu << (8 * ch);
-        const uint32_t* w = q.flt + (size_t)c4 * 9;
+        const uint32_t* w = q.flt + (size_t)c4 * (F * F);
 #pragma unroll
-        for (int dy = 0; dy < 3; ++dy) {
-            const unsigned w0 = w[dy * 3] & keep, w1 = w[dy * 3 + 1] & keep, w2 = w[dy * 3 + 2] & keep;
+        for (int dy = 0; dy < F; ++dy) {
+            unsigned wr[F];
+#pragma unroll
+            for (int k = 0; k < F; ++k)
+                wr[k] = w[dy * F + k] & keep;
 #pragma unroll
             for (int s = 0; s < NS; ++s)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int fw = 8 * s + 4 * kg + j - 3 - S * px;
-                    A[dy][s][j] = (int)(fw == 0 ? w0 : fw == 1 ? w1 : fw == 2 ? w2 : 0u);
+                    const int fw = 8 * s + 4 * kg + j - 4 + PAD - S * px;
+                    unsigned v = 0;
+#pragma unroll
+                    for (int k = 0; k < F; ++k)
+                        v = fw == k ? wr[k] : v;
+                    A[dy][s][j] = (int)v;
                 }
         }
     }
@@ -154,7 +167,7 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
         const int ix0 = S * x0 - 4 + 4 * kg;   // this lane's first input pixel of K step 0
 #pragma unroll
         for (int ir = 0; ir < IR; ++ir) {
-            const int iy = y * S - 1 + ir;
+            const int iy = y * S - PAD + ir;
             const bool row_ok = col_ok && (unsigned)iy < (unsigned)q.ih;
             const int row_off = base + __mul24(iy, q.iw);
 #pragma unroll
@@ -188,7 +201,7 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
         for (int r = 0; r < R; ++r) {
             acc[r] = biasv;
 #pragma unroll
-            for (int dy = 0; dy < 3; ++dy)
+            for (int dy = 0; dy < F; ++dy)
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
                     acc[r] = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[dy][s], B[r * S + dy][s], acc[r], 0, 0, 0);
@@ -233,8 +246,9 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
 bool dwconv44_mfma_supported(const ConvGeom& g, const void* src, const void* dst) {
     const long src_bytes = (long)g.n * g.ic * g.ih * g.iw;
     return g.fmt == MEGCC_FMT_NCHW44 && g.groups > 1 && g.groups == g.ic && g.ic == g.oc &&
-           (g.ic & 3) == 0 && g.fh == 3 && g.fw == 3 && g.ph == 1 && g.pw == 1 && g.dh == 1 &&
-           g.dw == 1 && g.sh == 1 && g.sw == 1 && ((uintptr_t)src & 15) == 0 &&
+           (g.ic & 3) == 0 && g.fh == g.fw && (g.fh == 3 || g.fh == 5 || g.fh == 7) && g.ph == g.fh / 2 &&
+           g.pw == g.fw / 2 && g.dh == 1 && g.dw == 1 && g.sh == g.sw &&
+           (g.sh == 1 || (g.sh == 2 && g.fh > 3)) && ((uintptr_t)src & 15) == 0 &&
            ((uintptr_t)dst & 15) == 0 && src_bytes < (1L << 31) &&
            (long)g.n * g.oc * g.oh * g.ow < (1L << 31) && (long)g.n * g.oh * ((g.ow + 7) / 8) < (1L << 30) && (long)g.ih * g.iw < (1L << 24);
 }
@@ -266,18 +280,25 @@ TinyNNStatus dwconv44_mfma_launch(
     q.d_xb = make_fastdiv(q.xblocks);
     if ((long)q.tiles * q.c4n == 0)
         return TinyNN_SUCCESS;
-    const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
-                     requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    const bool tab = requant_table_act(g.act) && requant_table_ok(g.s_src, g.s_flt, g.s_dst);
     if (tab)
         q.table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
     const int act = tab ? g.act : -1;
     const bool ragged = (g.iw & 3) != 0;
     const void* kern = nullptr;
-#define MG_DWM_ACT(S_, R_)                                                                      \
-    (act == MEGCC_NONLINE_IDENTITY ? (const void*)dwconv44_mfma_kernel<S_, R_, MEGCC_NONLINE_IDENTITY> \
-     : act == MEGCC_NONLINE_RELU   ? (const void*)dwconv44_mfma_kernel<S_, R_, MEGCC_NONLINE_RELU>     \
-                                   : (const void*)dwconv44_mfma_kernel<S_, R_, -1>)
-    kern = ragged ? MG_DWM_ACT(1, true) : MG_DWM_ACT(1, false);
+#define MG_DWM_ACT(S_, R_, F_)                                                                        \
+    (act == MEGCC_NONLINE_IDENTITY ? (const void*)dwconv44_mfma_kernel<S_, R_, MEGCC_NONLINE_IDENTITY, F_> \
+     : act == MEGCC_NONLINE_RELU   ? (const void*)dwconv44_mfma_kernel<S_, R_, MEGCC_NONLINE_RELU, F_>     \
+     : act == MEGCC_NONLINE_H_SWISH ? (const void*)dwconv44_mfma_kernel<S_, R_, MEGCC_NONLINE_H_SWISH, F_> \
+                                   : (const void*)dwconv44_mfma_kernel<S_, R_, -1, F_>)
+#define MG_DWM_F(S_, F_) (ragged ? MG_DWM_ACT(S_, true, F_) : MG_DWM_ACT(S_, false, F_))
+    if (g.fh == 3)
+        kern = MG_DWM_F(1, 3);
+    else if (g.fh == 5)
+        kern = g.sh == 1 ? MG_DWM_F(1, 5) : MG_DWM_F(2, 5);
+    else
+        kern = g.sh == 1 ? MG_DWM_F(1, 7) : MG_DWM_F(2, 7);
+#undef MG_DWM_F
 #undef MG_DWM_ACT
     // one wave per (plane set, tile) while they are all resident at once, otherwise as many
     // waves as are resident, each walking over the tiles of its plane set; the wave count is a

@@ -33,10 +33,12 @@ __host__ __device__ __forceinline__ float act_apply(float x) {
 }
 
 __host__ __device__ __forceinline__ int fp32_to_int8(float v) {
-    int r = (int)roundf(v);
-    r = r > 127 ? 127 : r;
-    r = r < -128 ? -128 : r;
-    return r;
+    // (clamped as a float: the conversion of an out-of-range float is the saturating one on the
+    //  device but not on the host, where the threshold tables are built)
+    float r = roundf(v);
+    r = r > 127.f ? 127.f : r;
+    r = r < -128.f ? -128.f : r;
+    return (int)r;
 }
 
 // acc already includes the int32 bias.
@@ -163,17 +165,39 @@ struct RequantTable {
     int t[REQUANT_TABLE_ENTRIES];
 };
 
-// host: the table for (act in {IDENTITY, RELU}, scales); the reference stays valid for the life of
-// the process (requant_table.hip)
+// H_SWISH joins the monotone activations: the reference applies it to the value already divided by
+// the output scale, h(v) = v * min(max(v + 3, 0), 6) * (1/6), so its dip (-0.375 at v = -1.5) never
+// reaches -0.5 and F is 0 for every v < 0; for v >= 0 both factors grow with v and every float
+// rounding keeps the order, so F is a non-decreasing step function from 0 to 127 and the same table
+// describes it exactly. The estimate is h(g) itself: |h(g) - h(v)| <= 1.5 * 2^-14, far inside the
+// quarter that the look-up tolerates (m = floor(h(g) + 0.25), F = m or m + 1).
+static inline bool requant_table_act(int act) {
+    return act == MEGCC_NONLINE_IDENTITY || act == MEGCC_NONLINE_RELU || act == MEGCC_NONLINE_H_SWISH;
+}
+
+// host: the table for (act in {IDENTITY, RELU, H_SWISH}, scales); the reference stays valid for the
+// life of the process (requant_table.hip)
 const RequantTable& requant_table_for(int act, float s_src, float s_flt, float s_dst);
 
-// table: pointer to entry 0 (LDS). ACT_LO: lowest output (-128, or 0 with RELU).
+// the lower candidate m (clamped to [lowest output, 126]) of the output for accumulator acc
+template <int ACT>
+__device__ __forceinline__ int requant_table_candidate(int acc, float c) {
+    static_assert(ACT == MEGCC_NONLINE_IDENTITY || ACT == MEGCC_NONLINE_RELU || ACT == MEGCC_NONLINE_H_SWISH,
+                  "monotone only");
+    constexpr int LO = ACT == MEGCC_NONLINE_IDENTITY ? -128 : 0;
+    float g = (float)acc * c;
+    if (ACT == MEGCC_NONLINE_H_SWISH) {
+        const float t = __builtin_fminf(__builtin_fmaxf(g + 3.f, 0.f), 6.f);
+        g = __builtin_fmaf(g * t, 1.f / 6.f, 0.25f);
+    }
+    const int m = cvt_floor_i32(g);  // saturating conversion
+    return m < LO ? LO : (m > 126 ? 126 : m);
+}
+
+// table: pointer to entry 0 (LDS)
 template <int ACT>
 __device__ __forceinline__ int requant_conv_table(int acc, float c, const int* table) {
-    static_assert(ACT == MEGCC_NONLINE_IDENTITY || ACT == MEGCC_NONLINE_RELU, "monotone only");
-    constexpr int LO = ACT == MEGCC_NONLINE_RELU ? 0 : -128;
-    int m = cvt_floor_i32((float)acc * c);  // saturating conversion
-    m = m < LO ? LO : (m > 126 ? 126 : m);
+    const int m = requant_table_candidate<ACT>(acc, c);
     return m + (acc > table[m + 128] ? 1 : 0);
 }
 

@@ -32,6 +32,8 @@ const RequantTable& requant_table_for(int act, float s_src, float s_flt, float s
             t->t[i] = 0;
         else if (act == MEGCC_NONLINE_RELU)
             t->t[i] = requant_threshold<MEGCC_NONLINE_RELU>(i, s_src, s_flt, s_dst, c);
+        else if (act == MEGCC_NONLINE_H_SWISH)
+            t->t[i] = requant_threshold<MEGCC_NONLINE_H_SWISH>(i, s_src, s_flt, s_dst, c);
         else
             t->t[i] = requant_threshold<MEGCC_NONLINE_IDENTITY>(i, s_src, s_flt, s_dst, c);
     }

@@ -141,10 +141,34 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.GROUP, 1, 36, 17, 33, 36, 3, 1, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW44, A.GROUP, 7, 4, 3, 1, 4, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 1, 40, 8, 3, 1, 1, A.IDENTITY, scales=(0.5, 0.5, 0.5)),
+    # H_SWISH through the threshold table in the pointwise kernels (streaming: 64 and 256 input
+    # channels; workgroup-shared: 512) and the plane-major 3x3 kernel
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 64, 28, 28, 128, 1, 1, 0, A.H_SWISH, scales=(0.02, 0.01, unsat(64))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 256, 14, 14, 64, 1, 1, 0, A.H_SWISH, scales=(0.02, 0.01, unsat(256))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 24, 512, 14, 14, 512, 1, 1, 0, A.H_SWISH, scales=(0.02, 0.01, unsat(512))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 4, 64, 56, 56, 128, 3, 1, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(576))),
+    # 5x5 (pad 2) and 7x7 (pad 3) on the matrix cores, stride 1 and 2: rows of whole pixel groups,
+    # ragged rows (masked loads, dword stores), images smaller than the filter, every activation,
+    # no bias, an odd number of plane sets
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 24, 28, 28, 24, 5, 1, 2, A.RELU, scales=(0.02, 0.01, unsat(25))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 16, 56, 56, 16, 5, 2, 2, A.RELU, scales=(0.02, 0.01, 0.05)),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 3, 12, 14, 14, 12, 5, 1, 2, A.H_SWISH, scales=(0.02, 0.01, unsat(25))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 20, 13, 19, 20, 5, 1, 2, A.IDENTITY, scales=(0.02, 0.01, unsat(25))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 17, 21, 8, 5, 2, 2, A.IDENTITY, scales=(0.02, 0.01, unsat(25)), bias=False),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 3, 4, 3, 2, 4, 5, 1, 2, A.RELU, scales=(0.02, 0.01, unsat(25))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 1, 4, 2, 3, 4, 5, 2, 2, A.SIGMOID, scales=(0.02, 0.01, unsat(25) * 40)),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 16, 28, 28, 16, 7, 1, 3, A.RELU, scales=(0.02, 0.01, unsat(49))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 12, 30, 36, 12, 7, 2, 3, A.IDENTITY, scales=(0.02, 0.01, unsat(49))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 11, 13, 8, 7, 1, 3, A.H_SWISH, scales=(0.02, 0.01, unsat(49))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 1, 4, 9, 7, 4, 7, 2, 3, A.RELU, scales=(0.02, 0.01, unsat(49)), bias=False),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 4, 8, 1, 9, 8, 7, 1, 3, A.IDENTITY, scales=(0.5, 0.5, 0.5)),
+    # ... and what keeps the one-output-per-thread kernel: other paddings, dilation
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 12, 16, 8, 5, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(25))),
+    ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 12, 16, 8, 3, 1, 2, A.RELU, scales=(0.02, 0.01, unsat(9)), dilate=2),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 224, 224, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, unsat(27))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 3, 3, 64, 48, 24, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(27))),
     # the matrix-core form (32 / 64 output channels): ragged last tile, rows of 4 and 8 columns (first
-    # and last column next to each other), H_SWISH through the literal sequence, no bias
+    # and last column next to each other), H_SWISH, no bias
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 3, 3, 18, 28, 64, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(27))),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 5, 3, 6, 4, 32, 3, 2, 1, A.RELU, scales=(0.02, 0.01, 0.05)),
     ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 10, 8, 32, 3, 2, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(27))),
@@ -537,6 +561,8 @@ OLDER = [
                           scales=(0.02, 0.01, unsat(9)))),
     ("nodwmfma", ConvCase(A.FMT_NCHW44, A.GROUP, 5, 12, 7, 7, 12, 3, 1, 1, A.H_SWISH,
                           scales=(0.02, 0.01, unsat(9)))),
+    ("nodwmfma", ConvCase(A.FMT_NCHW44, A.GROUP, 2, 24, 28, 28, 24, 5, 1, 2, A.RELU,
+                          scales=(0.02, 0.01, unsat(25)))),
     # channel-wise NCHW through the NCHW44 detour (what rows that are no multiple of 4 still use)
     ("nodwnchw", ConvCase(A.FMT_NCHW, A.GROUP, 4, 32, 56, 56, 32, 3, 1, 1, A.RELU,
                           scales=(0.02, 0.01, unsat(9)))),
@@ -729,3 +755,31 @@ def test_mfma_only_probe_reports_a_plausible_rate():
         assert n.value == 256 * 4 * 1024, "256 CUs x 4 SIMDs x 1024 MFMAs"
         tops = n.value * 65536 / us.value / 1e6
         assert 500 < tops <= 5000, (kind, us.value, tops)
+
+
+@pytest.mark.parametrize("scales", [(0.02, 0.01, 0.025), (0.02, 0.01, 0.05), (0.5, 0.5, 64.0)],
+                         ids=["c0.008", "c0.004_exact_ties", "c_2^-8_exact_ties"])
+@pytest.mark.parametrize("act", [A.IDENTITY, A.RELU, A.H_SWISH], ids=["IDENTITY", "RELU", "H_SWISH"])
+def test_every_accumulator_value_requantises_like_the_literal_sequence(act, scales):
+    """the threshold-table requantisation over a contiguous range of accumulators: a 1x1 layer whose
+    accumulator is 127 * (y - 128) + (x - 128) + bias at pixel (y, x), i.e. every integer in
+    [-16384, 16383] (plus 64 different bias offsets), against the literal float sequence of the
+    oracle - all 127 / 255 thresholds of the first scale triple lie inside that range, the other
+    two put an exact tie at every 125th / 128th accumulator"""
+    case = ConvCase(A.FMT_NCHW44, A.DENSE, 1, 32, 256, 256, 64, 1, 1, 0, act, scales=scales)
+    arrays = case.gen(3)
+    arrays["src"][...] = 0
+    arrays["flt"][...] = 0
+    ramp = np.arange(-128, 128, dtype=np.int8)
+    arrays["src"][0, 0, :, :, 0] = ramp[:, None]
+    arrays["src"][0, 0, :, :, 1] = ramp[None, :]
+    arrays["flt"][:, 0, 0, 0, 0, :] = 127
+    arrays["flt"][:, 0, 0, 0, 1, :] = 1
+    arrays["bias"][...] = (np.arange(64, dtype=np.int32) * 37 - 1000).reshape(arrays["bias"].shape)
+    ins, outs = case.specs(arrays)
+    op = runtime.PreparedOp(runtime.parse_symbol(case.symbol()), ins, outs)
+    op.launch()
+    got, want = op.result(), case.run_port(arrays)
+    if scales[2] == 0.025:
+        assert len(np.unique(want)) == (128 if act != A.IDENTITY else 256), "the range must cover every threshold"
+    compare(got, want, repr(case))

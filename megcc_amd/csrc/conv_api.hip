@@ -172,7 +172,9 @@ static size_t gather_bytes(const ConvGeom& g) {
 // back. The filter [OC][IC][FH][FW] packs into the same tiles as an NCHW44 one; the bias layouts
 // are the same bytes.
 static bool nchw_spatial(const ConvGeom& g) {
-    return g.fmt == MEGCC_FMT_NCHW && g.groups == 1 && !(g.ih == 1 && g.iw == 1 && g.fh == 1 && g.fw == 1);
+    // (at most 9 taps: the generated workspace function sizes the copies for those filters only)
+    return g.fmt == MEGCC_FMT_NCHW && g.groups == 1 && g.fh * g.fw <= 9 &&
+           !(g.ih == 1 && g.iw == 1 && g.fh == 1 && g.fw == 1);
 }
 // (channel counts that are no multiple of 4 are padded: the packed filter holds zeros for channels
 //  beyond IC / OC anyway, so what the padding lanes of the NCHW44 copies hold does not matter)

@@ -149,6 +149,7 @@ struct PipeConfig {
     int extra_lds;       // bytes of LDS beyond the stage buffers
     int fixed_lmax;      // patch slots compiled into the kernel (0: run-time Lmax)
     int pm = 0;          // plane-major activation patch (virtual rows padded to a multiple of 4)
+    int rs = 0;          // a stage is ONE filter row of a 32-channel chunk (filters of more than 9 taps)
     const void* kernel;
 };
 

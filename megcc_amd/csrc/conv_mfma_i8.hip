@@ -432,16 +432,29 @@ static TilePlan plan_tiles_uncached(const ConvGeom& g, int bn, long range_len, i
     return t;
 }
 
+static bool pick_dma(const ConvGeom& g, bool b128_ok, PipeConfig* pc, TilePlan* t, long* range_len, int* picked);
+
 bool conv_mfma_supported(const ConvGeom& g) {
     if (g.groups != 1)
         return false;
     bool fc = is_fc(g);
     if (!(g.fmt == MEGCC_FMT_NCHW44 || fc))
         return false;
-    if ((g.ic & 3) || g.fh * g.fw > MAX_TAPS_STAGE)
+    if (g.ic & 3)
         return false;
     if (g.fmt == MEGCC_FMT_NCHW44 && (g.oc & 3))
         return false;
+    if (g.fh * g.fw > MAX_TAPS_STAGE) {
+        // only the row-split variants of the LDS-direct kernel (no one-stage fallback: that kernel
+        // keeps every tap of a chunk in LDS and registers)
+        PipeConfig pc;
+        TilePlan t;
+        long range_len = 0;
+        int picked = -1;
+        const long slots = ((long)g.n * (g.ih + 2 * g.ph) + 2L * g.fh * g.dh) * (g.iw + 2 * g.pw);
+        return (long)g.n * g.ic * g.ih * g.iw < (1L << 31) && slots < (1L << 31) &&
+               (long)g.n * g.oh * g.ow < (1L << 31) - 512 && pick_dma(g, false, &pc, &t, &range_len, &picked);
+    }
     long P = (long)g.n * g.oh * g.ow;
     long src_bytes = (long)g.n * g.ic * g.ih * g.iw;
     long vmax = ((long)g.n * (g.ih + 2 * g.ph) + 2L * g.fh * g.dh) * (g.iw + 2 * g.pw);
@@ -503,6 +516,57 @@ bool conv_pw_stream_supported(const ConvGeom& g);
 TinyNNStatus conv_pw_stream_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst);
 
+// Picks the variant of the LDS-direct kernel for this layer (in order of preference; development
+// switches skip one) and the pixel range per workgroup; false: none of them takes the layer.
+static bool pick_dma(const ConvGeom& g, bool b128_ok, PipeConfig* pc, TilePlan* t, long* range_len, int* picked) {
+    bool pipe = false;
+    // variants of the LDS-direct kernel in order of preference (see conv_mfma_dma_config); a
+    // layer none of them takes runs on the one-stage kernel below
+    // (8, 9: one filter row per stage, the only ones that take filters of more than 9 taps)
+    static const int kDmaVariants[] = {6, 7, 2, 3, 0, 4, 1, 8, 9};
+    const Options& opt = options();
+    const bool dma_off[] = {opt.no_small, opt.no_small, opt.no_pm768, opt.no_pm,
+                            opt.no_dma512, opt.no_pm256, opt.no_dma, opt.no_rowsplit, opt.no_rowsplit};
+    constexpr int N_DMA_VARIANTS = 9;
+    for (int cand = 0; cand < N_DMA_VARIANTS && !pipe; ++cand) {
+        const int v = kDmaVariants[cand];
+        const bool have = !opt.no_dma && !dma_off[cand] && !((v == 2 || v == 4 || v == 6) && opt.no_pm) &&
+                          conv_mfma_dma_config(g, is_fc(g), v, b128_ok, pc);
+        if (!have)
+            continue;
+        *picked = v;
+        // one pixel range per free workgroup slot, so that the whole grid is resident at once and
+        // every CU finishes at the same time (no partial last round)
+        const long P = (long)g.n * g.oh * g.ow;
+        const long slots = (long)num_cus() * pc->blocks_per_cu;
+        const long oc_tiles = (g.oc + pc->bm - 1) / pc->bm;
+        long ranges = slots / oc_tiles > 0 ? slots / oc_tiles : 1;
+        (*range_len) = ((P + ranges - 1) / ranges + 31) / 32 * 32;
+        if ((*range_len) < pc->bn / 2) {  // too few pixels per workgroup for the tile
+            if (pc->bm == 32)
+                (*range_len) = pc->bn;  // the small-layer tiles: one tile per workgroup, not every CU busy
+            else if (pc->bn <= 256 && (P >= 4096 || (g.fh == 1 && g.fw == 1 && P >= 2048)))
+                // between the small-layer tiles and a full grid of 256- / 128-pixel tiles: half-filled
+                // tiles on part of the CUs (N=6, 128->128, 56x56: 9.4 us; the one-stage kernel
+                // these layers fell to: 20.8 us)
+                (*range_len) = pc->bn / 2;
+            else
+                continue;
+        }
+        ConvGeom gp = g;  // (row split: a stage's patch spans the windows of ONE filter row)
+        if (pc->rs)
+            gp.fh = 1;
+        *t = plan_tiles(gp, pc->bn, (*range_len), pc->pm);
+        if (pc->fixed_lmax) {
+            if (t->Lmax > pc->fixed_lmax)
+                continue;
+            t->Lmax = pc->fixed_lmax;
+        }
+        pipe = ((long)pc->nbuf * (pc->a_bytes + (long)pc->ks * t->Lmax * KROW) + pc->extra_lds) * pc->blocks_per_cu <= 160 * 1024;
+    }
+    return pipe;
+}
+
 TinyNNStatus conv_mfma_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst,
         const Workspace* ws) {
@@ -517,51 +581,10 @@ TinyNNStatus conv_mfma_launch(
     MfmaParams q = {};
     PipeConfig pc;
     const bool b128_ok = ((uintptr_t)src & 15) == 0 && !options().no_fcb;
-    // candidates in order of preference; development switches (MEGCC_NO...) skip one
     long range_len = 0;
     TilePlan t;
-    bool pipe = false;
     int picked = -1;  // variant of the LDS-direct kernel
-    // variants of the LDS-direct kernel in order of preference (see conv_mfma_dma_config); a
-    // layer none of them takes runs on the one-stage kernel below
-    static const int kDmaVariants[] = {6, 7, 2, 3, 0, 4, 1};
-    const Options& opt = options();
-    const bool dma_off[] = {opt.no_small, opt.no_small, opt.no_pm768, opt.no_pm,
-                            opt.no_dma512, opt.no_pm256, opt.no_dma};
-    constexpr int N_DMA_VARIANTS = 7;
-    for (int cand = 0; cand < N_DMA_VARIANTS && !pipe; ++cand) {
-        const int v = kDmaVariants[cand];
-        const bool have = !opt.no_dma && !dma_off[cand] && !((v == 2 || v == 4 || v == 6) && opt.no_pm) &&
-                          conv_mfma_dma_config(g, is_fc(g), v, b128_ok, &pc);
-        if (!have)
-            continue;
-        picked = v;
-        // one pixel range per free workgroup slot, so that the whole grid is resident at once and
-        // every CU finishes at the same time (no partial last round)
-        const long P = (long)g.n * g.oh * g.ow;
-        const long slots = (long)num_cus() * pc.blocks_per_cu;
-        const long oc_tiles = (g.oc + pc.bm - 1) / pc.bm;
-        long ranges = slots / oc_tiles > 0 ? slots / oc_tiles : 1;
-        range_len = ((P + ranges - 1) / ranges + 31) / 32 * 32;
-        if (range_len < pc.bn / 2) {  // too few pixels per workgroup for the tile
-            if (pc.bm == 32)
-                range_len = pc.bn;  // the small-layer tiles: one tile per workgroup, not every CU busy
-            else if (pc.bn <= 256 && (P >= 4096 || (g.fh == 1 && g.fw == 1 && P >= 2048)))
-                // between the small-layer tiles and a full grid of 256- / 128-pixel tiles: half-filled
-                // tiles on part of the CUs (N=6, 128->128, 56x56: 9.4 us; the one-stage kernel
-                // these layers fell to: 20.8 us)
-                range_len = pc.bn / 2;
-            else
-                continue;
-        }
-        t = plan_tiles(g, pc.bn, range_len, pc.pm);
-        if (pc.fixed_lmax) {
-            if (t.Lmax > pc.fixed_lmax)
-                continue;
-            t.Lmax = pc.fixed_lmax;
-        }
-        pipe = ((long)pc.nbuf * (pc.a_bytes + (long)pc.ks * t.Lmax * KROW) + pc.extra_lds) * pc.blocks_per_cu <= 160 * 1024;
-    }
+    const bool pipe = pick_dma(g, b128_ok, &pc, &t, &range_len, &picked);
     if (!pipe) {
         range_len = 0;
         t = plan_tiles(g, BN);
@@ -586,6 +609,10 @@ TinyNNStatus conv_mfma_launch(
     q.FW = g.fw;
     q.KS = pipe ? pc.ks : choose_ks(q.taps);
     q.stages = round_up((g.ic + 31) / 32, q.KS) / q.KS;
+    if (pipe && pc.rs)
+        q.stages *= g.fh;  // one stage per (chunk, filter row)
+    MG_REQUIRE(pipe || q.taps <= MAX_TAPS_STAGE, TinyNN_ERROR_UNSUPPORTED_DTYPE_TYPE,
+               "conv_mfma: %d taps and no row-split variant takes the layer", q.taps);
     q.VW = t.VW;
     q.VH = t.VH;
     q.IH = g.ih;

@@ -53,9 +53,15 @@ static constexpr int ACT_RT = -1;
 // stage together; the eight 16-byte pieces of a row are stored at piece ^ (row & 7) (the load
 // fetches the matching piece), which keeps the MFMA operand reads of 8 consecutive rows on
 // different banks.
-template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT, bool FCB, bool PM>
+// RS: row split for filters of more than 9 taps (5x5, 7x7): FH = 1 here, a stage is ONE filter row
+// (q.FH of them) of one 32-channel chunk - the packed filter keeps the taps of a chunk together, so
+// stage chunk * q.FH + fh finds its FW taps at the same place as a stage of an FW-tap filter would;
+// its patch is the patch of filter row 0 moved down by fh * DH image rows, with the rows that fall
+// off the image read as zeros (every load remembers the image row it fetches for filter row 0).
+template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT, bool FCB, bool PM, bool RS = false>
 __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaParams q) {
     static_assert(!FCB || (FC && KS == 4 && FH * FW == 1), "FCB: FullyConnected, 128 channels per stage");
+    static_assert(!RS || (FH == 1 && KS == 1 && !FC && !FCB && !PM), "RS: one filter row of one chunk per stage");
     constexpr int WGN = 4;
     constexpr int DM_BNP = 32 * NT * WGN;
     constexpr int DM_WAVES = WGM * WGN, DM_THREADS = 64 * DM_WAVES;
@@ -122,6 +128,8 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     // fetches plane (lane & 3) of slot (u % LW) * 16 + (lane >> 2). b_goff = byte offset of that
     // dword in the first plane group of a stage, or 2^31 (out of range -> zero) for padding.
     unsigned b_goff[B_PER_WAVE];
+    int b_ih[RS ? B_PER_WAVE : 1];  // RS: image row of the load for filter row 0 (far below 0: never valid)
+    constexpr int NEVER = -0x40000000;
     // PM: first slot of a sub-tile's patch. Slot space = rows of VW (a multiple of 4) slots per
     // padded image row, image column x at slot x: the left padding of a row is the tail of the
     // row before it. The patch starts PW slots before the first pixel's window, rounded down to 4.
@@ -173,12 +181,22 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             const int u = wave + j * DM_WAVES;
             const int kh = u / LW, slot = (u - kh * LW) * 16 + (lane >> 2);
             unsigned off = 0x80000000u;
+            if constexpr (RS)
+                b_ih[j] = NEVER;
             if (slot < L) {
                 const int vp = vp0 + slot;
                 const int v = fdiv(vp, q.dVW), vc = vp - v * q.VW;
                 const int n = fdiv(v, q.dVH), vh = v - n * q.VH;
                 const int ih = vh - q.PH, iw = vc - q.PW;
-                if (n < q.N && (unsigned)ih < (unsigned)q.IH && (unsigned)iw < (unsigned)q.IW)
+                if constexpr (RS) {
+                    // (the offset of filter row 0 also where that row is above the image: issue()
+                    //  adds fh * DH rows and checks the row it lands on)
+                    if (n < q.N && (unsigned)iw < (unsigned)q.IW) {
+                        b_ih[j] = ih;
+                        off = (unsigned)(n * q.image_stride + ih * q.row_stride + iw * q.pix_stride +
+                                         ((kh >> 1) * 8 + (kh & 1) * 4 + (lane & 3)) * q.plane_stride);
+                    }
+                } else if (n < q.N && (unsigned)ih < (unsigned)q.IH && (unsigned)iw < (unsigned)q.IW)
                     off = n * q.image_stride + ih * q.row_stride + iw * q.pix_stride +
                           ((kh >> 1) * 8 + (kh & 1) * 4 + (lane & 3)) * q.plane_stride;
             }
@@ -186,6 +204,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
         });
     };
     int lp0 = range0, lst = 0, lbuf = 0;  // load cursor: sub-tile, stage in it, LDS buffer
+    int lfh = 0, lchunk = 0;              // RS: filter row and chunk of stage lst
     describe(lp0);
     auto issue = [&](int bufidx) __attribute__((always_inline)) {
         const unsigned buf = lds0 + bufidx * BUF_BYTES;  // (LDS byte address, scalar)
@@ -195,7 +214,9 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             dma_global_saddr_b128(abase + ((size_t)(a_chunk[a] / (DM_BM / 32)) * q.OCP * KROW +
                                            (a_chunk[a] % (DM_BM / 32)) * 1024),
                                   lane16, buf + a_chunk[a] * 1024);
-        const unsigned poff = (unsigned)(lst * KS * 8) * (unsigned)q.plane_stride;
+        const unsigned poff = RS ? (unsigned)(lchunk * 8) * (unsigned)q.plane_stride +
+                                           (unsigned)(lfh * q.DH) * (unsigned)q.row_stride
+                                 : (unsigned)(lst * KS * 8) * (unsigned)q.plane_stride;
         static_for<B_PER_WAVE>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             const int u = wave + j * DM_WAVES;
@@ -203,11 +224,22 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
                 dma_global_b128(q.src + (b_goff[j] + poff), buf + A_BYTES + u * 1024);
             else if constexpr (PM)
                 dma_buffer_b128(src_rsrc, b_goff[j] + poff, buf + A_BYTES + u * 1024);
+            else if constexpr (RS)
+                dma_buffer_b32(src_rsrc,
+                               (unsigned)(b_ih[j] + lfh * q.DH) < (unsigned)q.IH ? b_goff[j] + poff : 0x80000000u,
+                               buf + A_BYTES + u * 256);
             else
                 dma_buffer_b32(src_rsrc, b_goff[j] + poff, buf + A_BYTES + u * 256);
         });
+        if constexpr (RS) {
+            if (++lfh == q.FH) {
+                lfh = 0;
+                ++lchunk;
+            }
+        }
         if (++lst == stages) {
             lst = 0;
+            lchunk = 0;  // (lfh is 0 here: the stages of a sub-tile are whole chunks)
             lp0 += DM_BNP;
             if (lp0 < range1)
                 describe(lp0);
@@ -401,6 +433,33 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
 
 // ---- configurations --------------------------------------------------------------------------
 template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3, int WGM = 2, int BPC = 1, int NT = 2, bool FCB = false, bool PM = false>
+static PipeConfig make_dma_config(int act, bool table_ok);
+
+// row-split configurations (filters of more than 9 taps): 64 * MT oc x 128 * NT px, FW taps per stage
+template <int FW, int LMAX, int MT, int DM_NBUF, int NT>
+static PipeConfig make_rs_config(int act, bool table_ok) {
+    PipeConfig c;
+    c.bm = 64 * MT;
+    c.bn = 128 * NT;
+    c.ks = 1;
+    c.threads = 512;
+    c.nbuf = DM_NBUF;
+    c.blocks_per_cu = 1;
+    c.a_bytes = FW * c.bm * KROW;
+    c.fixed_lmax = LMAX;
+    c.rs = 1;
+    c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + 128 * 4;
+    c.kernel = (const void*)conv_mfma_i8_dma_kernel<1, FW, 1, LMAX, ACT_RT, false, MT, DM_NBUF, 2, 1, NT, false, false, true>;
+    if (act == MEGCC_NONLINE_IDENTITY && table_ok)
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<1, FW, 1, LMAX, MEGCC_NONLINE_IDENTITY, false, MT, DM_NBUF, 2, 1, NT, false, false, true>;
+    else if (act == MEGCC_NONLINE_RELU && table_ok)
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<1, FW, 1, LMAX, MEGCC_NONLINE_RELU, false, MT, DM_NBUF, 2, 1, NT, false, false, true>;
+    else if (act == MEGCC_NONLINE_H_SWISH && table_ok)
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<1, FW, 1, LMAX, MEGCC_NONLINE_H_SWISH, false, MT, DM_NBUF, 2, 1, NT, false, false, true>;
+    return c;
+}
+
+template <int FH, int FW, int KS, int LMAX, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT, bool FCB, bool PM>
 static PipeConfig make_dma_config(int act, bool table_ok) {
     constexpr int DM_BM = 32 * MT * WGM;
     PipeConfig c;
@@ -434,6 +493,25 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
 bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok, PipeConfig* c) {
     const long P = (long)g.n * g.oh * g.ow;
     const bool k3 = g.fh == 3 && g.fw == 3, k1 = g.fh == 1 && g.fw == 1;
+    if (variant == 8 || variant == 9) {
+        // square filters of 5 or 7 columns, one filter row per stage: variant 8 with 256-pixel sub-tiles
+        // and three buffers of 512 patch slots (stride 1), variant 9 with 128-pixel sub-tiles and two
+        // buffers of 1024 slots (stride 2, wide rows, dilation)
+        if (fc || g.fmt != MEGCC_FMT_NCHW44 || !(g.fw == 5 || g.fw == 7) || g.fh != g.fw || g.oc < 32 ||
+            P < 2048 || (long)g.n * g.oc * g.oh * g.ow >= (1L << 31))
+            return false;
+        const bool okt = requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+        const bool wide = g.oc >= 128;
+        if (variant == 8)
+            *c = g.fw == 5 ? (wide ? make_rs_config<5, 512, 2, 3, 2>(g.act, okt) : make_rs_config<5, 512, 1, 3, 2>(g.act, okt))
+                           : (wide ? make_rs_config<7, 512, 2, 3, 2>(g.act, okt) : make_rs_config<7, 512, 1, 3, 2>(g.act, okt));
+        else
+            *c = g.fw == 5 ? (wide ? make_rs_config<5, 1024, 2, 2, 1>(g.act, okt) : make_rs_config<5, 1024, 1, 2, 1>(g.act, okt))
+                           : (wide ? make_rs_config<7, 1024, 2, 2, 1>(g.act, okt) : make_rs_config<7, 1024, 1, 2, 1>(g.act, okt));
+        return true;
+    }
+    if (g.fh * g.fw > MAX_TAPS_STAGE)
+        return false;
     if (variant == 6 || variant == 7) {
         // small 3x3 layers (batch 1): 32 oc x 128 px tiles of four waves, one 32 x 32 MFMA tile
         // each, so that a few thousand pixels still give every CU a workgroup; variant 6 with the

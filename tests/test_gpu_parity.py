@@ -141,6 +141,16 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.GROUP, 1, 36, 17, 33, 36, 3, 1, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW44, A.GROUP, 7, 4, 3, 1, 4, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 1, 40, 8, 3, 1, 1, A.IDENTITY, scales=(0.5, 0.5, 0.5)),
+    # dense 5x5 / 7x7 in NCHW44, one filter row per stage of the LDS-direct kernel: half a chunk of
+    # input channels, two chunks with a ragged second one, stride 2 (128-pixel sub-tiles), dilation,
+    # 64- and 128-channel tiles with ragged channel counts, every activation, no bias
+    ConvCase(A.FMT_NCHW44, A.DENSE, 6, 32, 28, 28, 64, 5, 1, 2, A.RELU, scales=(0.02, 0.01, unsat(800))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 6, 16, 56, 56, 128, 5, 2, 2, A.IDENTITY, scales=(0.02, 0.01, unsat(400))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 5, 40, 30, 34, 136, 7, 1, 3, A.H_SWISH, scales=(0.02, 0.01, unsat(1960))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 6, 64, 57, 55, 72, 7, 2, 3, A.RELU, scales=(0.02, 0.01, unsat(3136)), bias=False),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 5, 32, 31, 33, 36, 5, 1, 4, A.SIGMOID, scales=(0.02, 0.01, unsat(800) * 40), dilate=2),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 8, 40, 300, 32, 5, 1, 2, A.IDENTITY, scales=(0.02, 0.01, unsat(200))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 17, 32, 28, 28, 64, 5, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(800))),
     # H_SWISH through the threshold table in the pointwise kernels (streaming: 64 and 256 input
     # channels; workgroup-shared: 512) and the plane-major 3x3 kernel
     ConvCase(A.FMT_NCHW44, A.DENSE, 3, 64, 28, 28, 128, 1, 1, 0, A.H_SWISH, scales=(0.02, 0.01, unsat(64))),
@@ -563,6 +573,9 @@ OLDER = [
                           scales=(0.02, 0.01, unsat(9)))),
     ("nodwmfma", ConvCase(A.FMT_NCHW44, A.GROUP, 2, 24, 28, 28, 24, 5, 1, 2, A.RELU,
                           scales=(0.02, 0.01, unsat(25)))),
+    # dense 5x5 on the v_dot4 kernel (what layers under 2048 pixels still use)
+    ("norowsplit", ConvCase(A.FMT_NCHW44, A.DENSE, 6, 32, 28, 28, 64, 5, 1, 2, A.RELU,
+                            scales=(0.02, 0.01, unsat(800)))),
     # channel-wise NCHW through the NCHW44 detour (what rows that are no multiple of 4 still use)
     ("nodwnchw", ConvCase(A.FMT_NCHW, A.GROUP, 4, 32, 56, 56, 32, 3, 1, 1, A.RELU,
                           scales=(0.02, 0.01, unsat(9)))),

@@ -471,6 +471,9 @@ size_t conv_mfma_packed_bytes(const ConvGeom& g) {
     int taps = g.fh * g.fw, ks = choose_ks(taps);
     (void)ks;
     int chunks = round_up((g.ic + 31) / 32, CHUNK_PAD);
+    // (pointwise layers of 257 .. 512 input channels: the streaming kernel reads 16 chunks)
+    if (taps == 1 && chunks > 8 && chunks < 16)
+        chunks = 16;
     return (size_t)chunks * taps * round_up(g.oc, OC_PAD) * KROW;
 }
 

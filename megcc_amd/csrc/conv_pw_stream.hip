@@ -37,6 +37,7 @@ struct PwParams {
     const int32_t* bias;
     uint32_t* dst;
     int src_bytes;
+    int IC4;           // input channel planes (IC / 4)
     int P, OHW, OC, OCP;
     int tiles;         // ceil(P / 32)
     int groups;        // OC / channels per wave
@@ -57,7 +58,10 @@ __device__ __forceinline__ int pw_kernarg_table(int i) {
 // KC: 32-channel K chunks (IC = 32 * KC). ACT: IDENTITY / RELU use the table, -1 evaluates the
 // literal sequence with the run-time activation.
 // MT: 32-channel MFMA row tiles per wave (a wave owns 32 * MT output channels).
-template <int KC, int MT, int ACT>
+// RG: ragged channel counts - IC below 32 * KC (the planes beyond IC are not fetched: out-of-range
+// offset, zeros; the packed filter holds zeros there too) and / or OC no multiple of 32 * MT (the last
+// wave's surplus channels are computed from zero filter rows and not stored).
+template <int KC, int MT, int ACT, bool RG = false>
 __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) {
     __shared__ int tbl[REQUANT_TABLE_ENTRIES];
     __shared__ __attribute__((aligned(16))) int bias_lds[PW_MAX_OC];
@@ -103,11 +107,15 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
                        ? (unsigned)(n * q.image_stride + (p - n * q.OHW) * 4 + kg * 4 * q.plane_stride)
                        : 0x80000000u;
     };
+    const int planes_left = q.IC4 - 4 * kg;  // RG: this lane reads plane c * 8 + j while that is below
     auto load_chunk = [&](unsigned base, int c, v4i& dst) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            dst[j] = (int)__builtin_amdgcn_raw_buffer_load_b32(
-                    rs, (int)(base + (unsigned)((c * 8 + j) * q.plane_stride)), 0, 0);
+        for (int j = 0; j < 4; ++j) {
+            unsigned off = base + (unsigned)((c * 8 + j) * q.plane_stride);
+            if (RG)
+                off = c * 8 + j < planes_left ? off : 0x80000000u;
+            dst[j] = (int)__builtin_amdgcn_raw_buffer_load_b32(rs, (int)off, 0, 0);
+        }
     };
 
     v4i ring[RING];
@@ -119,8 +127,8 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
     // threshold table and bias to LDS while those loads are in flight
     if (ACT >= 0)
         tbl[tid] = pw_kernarg_table(tid);
-    for (int i = tid; i < q.OC; i += PW_THREADS)
-        bias_lds[i] = q.bias ? q.bias[i] : 0;
+    for (int i = tid; i < (RG ? q.groups * (32 * MT) : q.OC); i += PW_THREADS)
+        bias_lds[i] = q.bias && i < q.OC ? q.bias[i] : 0;
     __syncthreads();
 
     for (; t < tend; t += U) {
@@ -161,6 +169,8 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
                 const int obase = n * (q.OC >> 2) * q.OHW + (p - n * q.OHW);
 #pragma unroll
                 for (int mi = 0; mi < MT; ++mi) {
+                    if (RG && (og * MT + mi) * 32 >= q.OC)  // (wave-uniform: a tile of surplus channels)
+                        continue;
                     int r[16];
                     if (ACT < 0) {
 #pragma unroll
@@ -175,8 +185,9 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
 #pragma unroll
                         for (int e4 = 0; e4 < 4; ++e4) {
                             const int oc4 = og * (8 * MT) + mi * 8 + e4 * 2 + kg;
-                            q.dst[obase + oc4 * q.OHW] =
-                                    pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
+                            if (!RG || oc4 * 4 < q.OC)
+                                q.dst[obase + oc4 * q.OHW] =
+                                        pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
                         }
                     }
                 }
@@ -319,12 +330,12 @@ static int pw_resident_blocks(const void* kern) {
 bool conv_pw_stream_supported(const ConvGeom& g) {
     const long P = (long)g.n * g.oh * g.ow;
     return g.fmt == MEGCC_FMT_NCHW44 && g.groups == 1 && g.fh == 1 && g.fw == 1 && g.sh == 1 &&
-           g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.ic == 32 || g.ic == 64 || g.ic == 128 || g.ic == 256 || g.ic == 512 ||
+           g.sw == 1 && g.ph == 0 && g.pw == 0 && (g.ic & 3) == 0 && (g.oc & 3) == 0 && (g.ic <= 512 ||
             // (1024: layers too small for the LDS-staged kernel, where one round trip wins, and the
             //  workgroup-shared form up to a few thousand pixels)
             (g.ic == 1024 && (P < 2048 || (P <= 4096 && (g.oc & 127) == 0 && !options().no_pwshare &&
                                          (P + 31) / 32 * (g.oc / 128) >= 256)))) &&
-           (g.oc & 63) == 0 && g.oc <= PW_MAX_OC && P >= 32 &&
+           ((g.oc & 63) == 0 || g.ic <= 512) && g.oc <= PW_MAX_OC && P >= 32 &&
            (long)g.n * g.ic * g.ih * g.iw < (1L << 31) && P * g.oc < (1L << 31);
 }
 
@@ -341,7 +352,14 @@ TinyNNStatus conv_pw_stream_launch(
     q.OC = g.oc;
     q.OCP = (g.oc + OC_PAD - 1) / OC_PAD * OC_PAD;
     q.tiles = (q.P + 31) / 32;
-    q.groups = g.oc / (g.ic > 256 ? 32 : 64);
+    q.IC4 = g.ic >> 2;
+    // (ragged channel counts: IC below the next power of two of 32-channel chunks, OC no multiple of
+    //  a wave's 64 / 32 channels)
+    const int chunks = (g.ic + 31) / 32;
+    const int kc = chunks <= 1 ? 1 : chunks <= 2 ? 2 : chunks <= 4 ? 4 : chunks <= 8 ? 8 : chunks <= 16 ? 16 : 32;
+    const int per_wave = kc > 8 ? 32 : 64;
+    const bool ragged = g.ic != kc * 32 || g.oc % per_wave != 0;
+    q.groups = (g.oc + per_wave - 1) / per_wave;
     q.image_stride = g.ic * q.OHW;
     q.plane_stride = q.OHW * 4;
     q.act = g.act;
@@ -356,23 +374,25 @@ TinyNNStatus conv_pw_stream_launch(
     const int act = tab ? g.act : -1;
 
     const void* kern = nullptr;
-#define MG_PW_PICK(KC_, MT_)                                                                      \
-    (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_IDENTITY> \
-     : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_RELU>     \
-     : act == MEGCC_NONLINE_H_SWISH ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_H_SWISH> \
-                                   : (const void*)conv_pw_stream_kernel<KC_, MT_, -1>)
-    switch (g.ic / 32) {
+#define MG_PW_PICK_RG(KC_, MT_, RG_)                                                                      \
+    (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_IDENTITY, RG_> \
+     : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_RELU, RG_>     \
+     : act == MEGCC_NONLINE_H_SWISH ? (const void*)conv_pw_stream_kernel<KC_, MT_, MEGCC_NONLINE_H_SWISH, RG_> \
+                                   : (const void*)conv_pw_stream_kernel<KC_, MT_, -1, RG_>)
+#define MG_PW_PICK(KC_, MT_) (ragged ? MG_PW_PICK_RG(KC_, MT_, true) : MG_PW_PICK_RG(KC_, MT_, false))
+    switch (kc) {
         case 1: kern = MG_PW_PICK(1, 2); break;
         case 2: kern = MG_PW_PICK(2, 2); break;
         case 4: kern = MG_PW_PICK(4, 2); break;
         case 8: kern = MG_PW_PICK(8, 2); break;
         case 16: kern = MG_PW_PICK(16, 1); break;  // 512 input channels: 32 output channels per wave
-        default: kern = MG_PW_PICK(32, 1); break;  // 1024: the filter rows fill half the registers
+        default: kern = MG_PW_PICK_RG(32, 1, false); break;  // 1024: the filter rows fill half the registers
     }
 #undef MG_PW_PICK
+#undef MG_PW_PICK_RG
 
     // 512 input channels and more tiles than resident waves: the workgroup-shared form
-    if ((g.ic == 512 || g.ic == 1024) && (q.groups & 3) == 0 && !options().no_pwshare) {
+    if ((g.ic == 512 || g.ic == 1024) && !ragged && (q.groups & 3) == 0 && !options().no_pwshare) {
 #define MG_PWS_PICK(KC_)                                                                                  \
     (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_pw_share_kernel<KC_, MEGCC_NONLINE_IDENTITY>         \
      : act == MEGCC_NONLINE_RELU   ? (const void*)conv_pw_share_kernel<KC_, MEGCC_NONLINE_RELU>             \
@@ -412,7 +432,7 @@ TinyNNStatus conv_pw_stream_launch(
     const unsigned blocks = (unsigned)(waves / 4);
 
     void* args[] = {&q};
-    note_kernel("conv_pw_stream", g.ic / 32);
+    note_kernel("conv_pw_stream", kc, ragged);
     hipError_t e = hipLaunchKernel(kern, dim3(blocks), dim3(PW_THREADS), args, 0, stream());
     MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_pw_stream: %s", hipGetErrorString(e));
     return check_launch("conv_pw_stream");

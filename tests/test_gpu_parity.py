@@ -141,6 +141,17 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.GROUP, 1, 36, 17, 33, 36, 3, 1, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW44, A.GROUP, 7, 4, 3, 1, 4, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
     ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 1, 40, 8, 3, 1, 1, A.IDENTITY, scales=(0.5, 0.5, 0.5)),
+    # pointwise layers with any channel counts on the streaming kernel: input channels below the next
+    # power of two of 32-channel chunks (planes beyond IC are not fetched), output channels that do
+    # not fill the last wave's 64 / 32, one channel group in and out, with a stride (gathered pixels)
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 24, 28, 28, 144, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(24))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 144, 28, 28, 24, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(144))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 16, 19, 23, 96, 1, 1, 0, A.H_SWISH, scales=(0.02, 0.01, unsat(16))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 160, 7, 7, 960, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(160))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 384, 14, 14, 68, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(384)), bias=False),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 5, 4, 9, 11, 4, 1, 1, 0, A.SIGMOID, scales=(0.02, 0.01, unsat(4) * 40)),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 40, 31, 29, 80, 1, 2, 0, A.RELU, scales=(0.02, 0.01, unsat(40))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 1, 320, 10, 10, 1024, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(320))),
     # dense 5x5 / 7x7 in NCHW44, one filter row per stage of the LDS-direct kernel: half a chunk of
     # input channels, two chunks with a ragged second one, stride 2 (128-pixel sub-tiles), dilation,
     # 64- and 128-channel tiles with ragged channel counts, every activation, no bias
@@ -564,6 +575,8 @@ OLDER = [
                                  scales=(0.02, 0.01, unsat(512)))),
     ("nopws", ConvCase(A.FMT_NCHW44, A.DENSE, 11, 64, 56, 56, 128, 1, 1, 0, A.IDENTITY,
                              scales=(0.02, 0.01, unsat(64)))),
+    ("nopws", ConvCase(A.FMT_NCHW44, A.DENSE, 3, 24, 28, 28, 144, 1, 1, 0, A.RELU,
+                             scales=(0.02, 0.01, unsat(24)))),
     # stride-1 depthwise on the v_dot4 kernels (two rows per thread on large planes, one on small)
     ("nodwmfma", ConvCase(A.FMT_NCHW44, A.GROUP, 2, 32, 112, 112, 32, 3, 1, 1, A.RELU,
                           scales=(0.02, 0.01, unsat(9)))),

@@ -179,6 +179,16 @@ def make_workload(name):
         s = 2 if name.endswith("s2") else 1
         case = ConvCase(abi.FMT_NCHW, abi.GROUP, 64, 32, 112, 112, 32, 3, s, 1, abi.RELU, scales=(0.02, 0.01, 0.05))
         return case, "qsi8 depthwise 3x3 s%d NCHW N=64 C=32 112x112" % s, "hbm"
+    if name in ("dw5x5", "dw5x5_s2", "dw7x7", "dw_hswish"):  # depthwise layers of MobileNetV3 / EfficientNet style blocks
+        c, hw, k, s, act = {"dw5x5": (240, 28, 5, 1, abi.RELU), "dw5x5_s2": (96, 56, 5, 2, abi.RELU),
+                            "dw7x7": (96, 28, 7, 1, abi.RELU), "dw_hswish": (144, 56, 3, 1, abi.H_SWISH)}[name]
+        case = ConvCase(abi.FMT_NCHW44, abi.GROUP, 64, c, hw, hw, c, k, s, k // 2, act, scales=(0.02, 0.01, 0.05))
+        return case, "qsi8 depthwise %dx%d s%d NCHW44 N=64 C=%d %dx%d %s" % (
+            k, k, s, c, hw, hw, abi.NONLINE_NAMES[act]), "hbm"
+    if name in ("pw_24_144", "pw_144_24"):  # pointwise layers whose channel counts are no multiples of 32
+        ic, oc = (24, 144) if name == "pw_24_144" else (144, 24)
+        case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 64, ic, 56, 56, oc, 1, 1, 0, abi.RELU, scales=(0.02, 0.01, 0.05))
+        return case, "qsi8 conv1x1 NCHW44 N=64 %d->%d 56x56" % (ic, oc), "hbm"
     if name.startswith("dw"):
         c, hw, s = {"dw": (32, 112, 1), "dw_s2": (32, 112, 2), "dw512": (512, 14, 1),
                     "dw512_s2": (512, 14, 2)}[name]

@@ -49,6 +49,29 @@ bool parse_nonline(const std::string& s, MegccNonline* out) {
 }
 
 bool parse_conv(std::string s, MegccConvAttr* a) {
+    // the names of the f32 NCHW44 kernels the reference picks (GeneralIntrinsic/ConvKernel):
+    //   GI_kernel_conv2d_<k>x<k>_NCHW44_DENSE_p.._s.._d.._<io>[_bias][_NONLINE]_winograd_f23 / f43 / f63
+    //   GI_kernel_conv2d_conv1x1_NCHW44_1x1_DENSE_p.._s.._d..[_bias][_NONLINE]
+    for (const char* w : {"_winograd_f23", "_winograd_f43", "_winograd_f63"})
+        if (ends_with(s, w)) {
+            s.erase(s.size() - strlen(w));
+            if (!eat(s, "GI_"))
+                return false;
+        }
+    if (eat(s, "GI_kernel_conv2d_conv1x1_")) {
+        const bool f44 = eat(s, "NCHW44_");
+        if (!f44 && !eat(s, "NCHW_"))
+            return false;
+        if (!eat(s, "1x1_"))
+            return false;
+        s = std::string("kernel_conv2d_1x1_") + (f44 ? "NCHW44_" : "NCHW_") + s;
+        // (no operand types in this name: put them where the common form has them)
+        size_t d = s.find("_d");
+        if (d == std::string::npos)
+            return false;
+        size_t e = s.find('_', d + 1);
+        s.insert(e == std::string::npos ? s.size() : e, "_f32f32f32f32");
+    }
     const bool gi = eat(s, "GI_kernel_conv2d_im2col_");
     if (!gi && !eat(s, "kernel_conv2d_"))
         return false;
@@ -173,7 +196,7 @@ extern "C" TinyNNStatus megcc_gfx950_parse_symbol(const char* symbol, MegccKerne
     memset(desc, 0, sizeof(*desc));
     std::string s(symbol);
     int v = 0;
-    if (starts_with(s, "kernel_conv2d_") || starts_with(s, "GI_kernel_conv2d_im2col_")) {
+    if (starts_with(s, "kernel_conv2d_") || starts_with(s, "GI_kernel_conv2d_")) {
         if (parse_conv(s, &desc->attr.conv)) {
             desc->kind = MEGCC_KERN_CONV;
             return TinyNN_SUCCESS;

@@ -217,6 +217,23 @@ static void nchw44_views(int n, int c, int h, int w, Layout* view, Layout* dense
         dense->stride[i] = ds[i];
     }
 }
+// f32 dense layers in NCHW44 (the layout MegCC gives fp32 models on ARM): the implicit-GEMM kernel
+// works on NCHW, so the layer runs as relayout NCHW44 -> NCHW into the workspace, that kernel,
+// relayout back; the filter [OC/4][IC/4][FH][FW][4 ic][4 oc] becomes [OC][IC][FH][FW] by a third,
+// small relayout. The bias layouts are the same bytes.
+static bool f32_nchw44_dense(const ConvGeom& g) {
+    return g.fmt == MEGCC_FMT_NCHW44 && g.groups == 1 && (g.ic & 3) == 0 && (g.oc & 3) == 0;
+}
+static ConvGeom as_nchw(const ConvGeom& g) {
+    ConvGeom s = g;
+    s.fmt = MEGCC_FMT_NCHW;
+    return s;
+}
+// workspace of that detour: [inner kernel's][input copy][output copy][filter copy]
+static size_t f32_nchw44_bytes(const ConvGeom& g, size_t inner) {
+    return round_up256(inner) + round_up256((size_t)g.n * g.ic * g.ih * g.iw * 4) +
+           round_up256((size_t)g.n * g.oc * g.oh * g.ow * 4) + round_up256((size_t)g.oc * g.ic * g.fh * g.fw * 4);
+}
 // NCHW tensor with c channels <-> NCHW44 tensor with round_up4(c) channels: the whole groups of 4
 // in one copy, the last group's c % 4 channels in a second (its other lanes are not touched)
 static TinyNNStatus nchw_nchw44_copy(
@@ -295,6 +312,8 @@ static size_t conv2d_scratch_bytes(const ConvGeom& g, bool q8, bool f32, bool pa
         return nchw_depthwise_bytes(g);
     if (f32 && !(conv_f32_small_supported(g) && !options().no_f32small) && conv_f32_gemm_supported(g))
         return conv_f32_gemm_workspace_bytes(g);
+    if (f32 && f32_nchw44_dense(g) && conv_f32_gemm_supported(as_nchw(g)))
+        return f32_nchw44_bytes(g, conv_f32_gemm_workspace_bytes(as_nchw(g)));
     return 0;
 }
 
@@ -491,6 +510,41 @@ static TinyNNStatus conv2d_run(
         note_kernel("conv_dot4");
         return conv_dot4_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     }
+    if (f32 && f32_nchw44_dense(g) && conv_f32_gemm_supported(as_nchw(g)) && workspace && workspace->ptr &&
+        aligned16(workspace->ptr) &&
+        workspace->size >= f32_nchw44_bytes(g, conv_f32_gemm_workspace_bytes(as_nchw(g)))) {
+        const ConvGeom g1 = as_nchw(g);
+        const size_t inner = round_up256(conv_f32_gemm_workspace_bytes(g1));
+        char* src_nchw = (char*)workspace->ptr + inner;
+        char* dst_nchw = src_nchw + round_up256((size_t)g.n * g.ic * g.ih * g.iw * 4);
+        char* flt_nchw = dst_nchw + round_up256((size_t)g.n * g.oc * g.oh * g.ow * 4);
+        Layout view, dense;
+        nchw44_views(g.n, g.ic, g.ih, g.iw, &view, &dense);
+        st = strided_copy(src->ptr, dense, src_nchw, view, 4, "conv2d (f32 NCHW44 -> NCHW)");
+        if (st != TinyNN_SUCCESS)
+            return st;
+        const int taps = g.fh * g.fw;
+        Layout fs = {}, fd = {};  // [OC/4][IC/4][taps][4 ic][4 oc] -> oc = 4 * og + o, ic = 4 * ig + i
+        fs.nr_dim = fd.nr_dim = 5;
+        const uint32_t fdim[5] = {(uint32_t)(g.oc / 4), (uint32_t)(g.ic / 4), (uint32_t)taps, 4u, 4u};
+        const int fss[5] = {(g.ic / 4) * taps * 16, taps * 16, 16, 4, 1};
+        const int fds[5] = {4 * g.ic * taps, 4 * taps, 1, taps, g.ic * taps};
+        for (int i = 0; i < 5; ++i) {
+            fs.dims[i] = fd.dims[i] = fdim[i];
+            fs.stride[i] = fss[i];
+            fd.stride[i] = fds[i];
+        }
+        st = strided_copy(flt->ptr, fs, flt_nchw, fd, 4, "conv2d (f32 NCHW44 filter -> NCHW)");
+        if (st != TinyNN_SUCCESS)
+            return st;
+        note_kernel("conv_f32_gemm between NCHW44 relayouts");
+        Workspace sub = {workspace->ptr, inner, 0};
+        st = conv_f32_gemm_launch(g1, src_nchw, flt_nchw, b, dst_nchw, &sub);
+        if (st != TinyNN_SUCCESS)
+            return st;
+        nchw44_views(g.n, g.oc, g.oh, g.ow, &view, &dense);
+        return strided_copy(dst_nchw, view, dst->ptr, dense, 4, "conv2d (f32 NCHW -> NCHW44)");
+    }
     if (f32 && conv_f32_small_supported(g) && !options().no_f32small) {
         note_kernel("conv_f32_small");
         return conv_f32_small_launch(g, src->ptr, flt->ptr, b, dst->ptr);
@@ -571,9 +625,12 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d_workspace(
     const Tensor *src = inputs[0], *flt = inputs[1];
     ConvGeom g;
     if (is_f32(src) && is_f32(flt)) {
-        if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS &&
-            conv_f32_gemm_supported(g))
-            *workspace = conv_f32_gemm_workspace_bytes(g);
+        if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS) {
+            if (conv_f32_gemm_supported(g))
+                *workspace = conv_f32_gemm_workspace_bytes(g);
+            else if (attr->sparse == MEGCC_SPARSE_DENSE && f32_nchw44_dense(g) && conv_f32_gemm_supported(as_nchw(g)))
+                *workspace = f32_nchw44_bytes(g, conv_f32_gemm_workspace_bytes(as_nchw(g)));
+        }
     } else if (is_q8(src) && is_q8(flt) && attr->sparse == MEGCC_SPARSE_GROUP) {
         if (make_geom(attr, src, flt, nullptr, false, 0, &g) == TinyNN_SUCCESS && nchw_depthwise(g))
             *workspace = nchw_depthwise_bytes(g);

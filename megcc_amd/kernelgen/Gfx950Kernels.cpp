@@ -252,6 +252,37 @@ struct ConvKernel : KernelFuncBase {
                << "    return TinyNN_SUCCESS;\n}\n";
             return ss.str();
         }
+        if (f32 && fmt == "NCHW44" && dense) {
+            // f32 dense NCHW44 runs as relayout -> NCHW implicit GEMM -> relayout (conv_api.hip): the
+            // GEMM's split-K room, then NCHW copies of input, output and filter
+            std::stringstream ss;
+            ss << "TinyNNStatus " << GetWorkspaceSignature(c) << " {\n"
+               << "    const Layout src = inputs[0]->layout, flt = inputs[1]->layout;\n"
+               << "    const long eh = " << c->getAttrUInt("dilate_h") << " * (" << c->getAttrUInt("kernel_h")
+               << " - 1) + 1, ew = " << c->getAttrUInt("dilate_w") << " * (" << c->getAttrUInt("kernel_w")
+               << " - 1) + 1;\n"
+               << "    const long ih = src.dims[2] + 2 * " << c->getAttrUInt("pad_h")
+               << ", iw = src.dims[3] + 2 * " << c->getAttrUInt("pad_w") << ";\n"
+               << "    const long oh = ih >= eh ? (ih - eh) / " << c->getAttrUInt("stride_h")
+               << " + 1 : 0, ow = iw >= ew ? (iw - ew) / " << c->getAttrUInt("stride_w") << " + 1 : 0;\n"
+               << "    const long ic = (long)src.dims[1] * 4, oc = (long)flt.dims[0] * 4;\n"
+               << "    const long M = oc, N = (long)src.dims[0] * oh * ow, K = ic * " << taps << ";\n"
+               << "    long tiles = ((M + 127) / 128) * ((N + 127) / 128), s = 1;\n"
+               << "    if (tiles < 192 && K >= 128) {\n"
+               << "        s = (512 + tiles - 1) / tiles;\n"
+               << "        if (s > K / 64) s = K / 64;\n"
+               << "        if (s > 64) s = 64;\n"
+               << "        if (s < 2) s = 1;\n"
+               << "    }\n"
+               << "    *workspace = 0;\n"
+               << "    if (N < (1L << 31) && K < (1L << 31))\n"
+               << "        *workspace = (((s > 1 ? (size_t)s * M * N * 4 : 0) + 255) & ~(size_t)255) +\n"
+               << "                     (((size_t)src.dims[0] * ic * src.dims[2] * src.dims[3] * 4 + 255) & ~(size_t)255) +\n"
+               << "                     (((size_t)N * oc * 4 + 255) & ~(size_t)255) +\n"
+               << "                     (((size_t)oc * K * 4 + 255) & ~(size_t)255);\n"
+               << "    return TinyNN_SUCCESS;\n}\n";
+            return ss.str();
+        }
         if (!(f32 && fmt == "NCHW" && dense) && !q8_mfma)
             return "TinyNNStatus " + GetWorkspaceSignature(c) +
                    " {\n    *workspace = 0;\n    return TinyNN_SUCCESS;\n}\n";

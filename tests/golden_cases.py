@@ -200,4 +200,16 @@ def golden_cases():
         for shape in ((2, 3), (3, 4, 5), (4, 5, 6, 7)):
             for axis in range(len(shape)):
                 c["reduce_%s_%dd_a%d" % (mode, len(shape), axis)] = ReduceCase(mode, shape, axis)
+    # --- later additions (appended: the seed of a case is its position in this dictionary)
+    # f32 dense layers in NCHW44, depthwise 5x5 / 7x7, H_SWISH on a dense 5x5 layer
+    c["conv44_f32_3x3_RELU"] = ConvCase(A.FMT_NCHW44, A.DENSE, 2, 8, 9, 7, 12, 3, 1, 1, A.RELU, dtype="f32")
+    c["conv44_f32_1x1_IDENTITY"] = ConvCase(A.FMT_NCHW44, A.DENSE, 1, 12, 6, 5, 8, 1, 1, 0, A.IDENTITY, dtype="f32")
+    c["dw44_5x5_s1_H_SWISH"] = ConvCase(
+        A.FMT_NCHW44, A.GROUP, 2, 8, 9, 11, 8, 5, 1, 2, A.H_SWISH, scales=(0.02, 0.01, unsat(25)))
+    c["dw44_5x5_s2_RELU"] = ConvCase(
+        A.FMT_NCHW44, A.GROUP, 2, 8, 9, 11, 8, 5, 2, 2, A.RELU, scales=(0.02, 0.01, unsat(25)))
+    c["dw44_7x7_s1_IDENTITY"] = ConvCase(
+        A.FMT_NCHW44, A.GROUP, 1, 4, 10, 9, 4, 7, 1, 3, A.IDENTITY, scales=(0.02, 0.01, unsat(49)))
+    c["conv44_5x5_H_SWISH"] = ConvCase(
+        A.FMT_NCHW44, A.DENSE, 2, 8, 9, 7, 8, 5, 1, 2, A.H_SWISH, scales=(0.02, 0.01, unsat(200)))
     return c

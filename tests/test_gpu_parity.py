@@ -289,6 +289,13 @@ LIVE = [
     # above 2^27 multiply-adds: the implicit GEMM on the matrix cores
     ConvCase(A.FMT_NCHW, A.DENSE, 4, 64, 56, 56, 64, 3, 1, 1, A.RELU, dtype="f32"),
     ConvCase(A.FMT_NCHW, A.DENSE, 3, 40, 57, 55, 72, 3, 2, 1, A.H_SWISH, dtype="f32"),
+    # f32 dense layers in NCHW44: NCHW copies of input, output and filter around the implicit GEMM
+    # (with and without a split of K), stride 2, 1x1, no bias, every activation
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 64, 28, 28, 64, 3, 1, 1, A.RELU, dtype="f32"),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 3, 40, 29, 31, 72, 3, 2, 1, A.H_SWISH, dtype="f32"),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 16, 14, 12, 128, 1, 1, 0, A.IDENTITY, dtype="f32", bias=False),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 7, 7, 32, 3, 1, 1, A.SIGMOID, dtype="f32"),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 2, 8, 12, 10, 8, 5, 1, 2, A.RELU, dtype="f32", dilate=1),
     MatMulCase(1, 1024, 1000),
     MatMulCase(64, 512, 384),
     MatMulCase(130, 77, 259),

@@ -154,6 +154,11 @@ def test_generated_workspace_functions_agree_with_the_library(shim_library):
             k = desc.attr.conv.kernel_h
             cases_ = [[(1, 32, 56, 56), (32, 32, k, k)], [(2, 5, 19, 23), (37, 5, k, k)],
                       [(8, 64, 56, 56), (128, 64, k, k)]]
+        elif desc.kind == 1 and "f32" in sym and "_NCHW44_DENSE_" in sym:
+            # relayout -> NCHW implicit GEMM -> relayout: the GEMM's room plus three NCHW copies
+            k = desc.attr.conv.kernel_h
+            cases_ = [[(2, 2, 9, 7, 4), (3, 2, k, k, 4, 4)], [(8, 16, 56, 56, 4), (16, 16, k, k, 4, 4)],
+                      [(1, 128, 7, 7, 4), (128, 128, k, k, 4, 4)]]
         elif desc.kind == 1 and "qsi8" in sym and "_NCHW44_DENSE_" in sym:
             k = desc.attr.conv.kernel_h
             cases_ = [[(64, 256, 7, 7, 4), (256, 256, k, k, 4, 4)], [(2, 8, 20, 24, 4), (12, 8, k, k, 4, 4)],

@@ -37,6 +37,10 @@ PAIRS = [
     ("dwconv44 between NCHW relayouts",
      ConvCase(A.FMT_NCHW, A.GROUP, 4, 32, 56, 54, 32, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9))),
      ConvCase(A.FMT_NCHW, A.GROUP, 3, 16, 29, 31, 16, 3, 2, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(9)))),
+    # f32 layer in NCHW44: NCHW copies of input, output and filter around the implicit GEMM
+    ("conv_f32_gemm between NCHW44 relayouts",
+     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 64, 28, 28, 64, 3, 1, 1, A.RELU, dtype="f32"),
+     ConvCase(A.FMT_NCHW44, A.DENSE, 1, 16, 9, 7, 8, 1, 1, 0, A.IDENTITY, dtype="f32")),
     # f32 layer with few tiles: f32 partial sums of a split of K
     ("conv_f32_gemm",
      ConvCase(A.FMT_NCHW, A.DENSE, 4, 64, 56, 56, 64, 3, 1, 1, A.RELU, dtype="f32"),

@@ -709,6 +709,60 @@ def test_plane_major_patch_sweep(case):
     compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
 
 
+def _new_kernel_sweep():
+    """seeded random layers for the pointwise kernel with any channel counts, the depthwise 5x5 / 7x7
+    kernels and the dense 5x5 / 7x7 layers with one filter row per stage: random image sizes (rows
+    that are no multiple of 4 or 8 pixels), strides, batches, channel counts, the three activations
+    that go through the threshold table and SIGMOID"""
+    r = np.random.Generator(np.random.PCG64(77))
+    acts = [A.RELU, A.IDENTITY, A.H_SWISH, A.SIGMOID]
+    out = []
+    for _ in range(10):  # pointwise
+        ic, oc = int(r.integers(1, 129)) * 4, int(r.integers(1, 97)) * 4
+        ih, iw, n = int(r.integers(3, 40)), int(r.integers(3, 40)), int(r.integers(1, 6))
+        act = acts[int(r.integers(0, 4))]
+        sc = unsat(ic) * (40 if act == A.SIGMOID else 1)
+        out.append(ConvCase(A.FMT_NCHW44, A.DENSE, n, ic, ih, iw, oc, 1, 1, 0, act, scales=(0.02, 0.01, sc)))
+    for _ in range(10):  # depthwise 5x5 / 7x7
+        k, s = int(r.choice([5, 7])), int(r.integers(1, 3))
+        c = int(r.integers(1, 25)) * 4
+        ih, iw, n = int(r.integers(1, 45)), int(r.integers(1, 45)), int(r.integers(1, 5))
+        act = acts[int(r.integers(0, 4))]
+        sc = unsat(k * k) * (40 if act == A.SIGMOID else 1)
+        out.append(ConvCase(A.FMT_NCHW44, A.GROUP, n, c, ih, iw, c, k, s, k // 2, act, scales=(0.02, 0.01, sc),
+                            bias=bool(r.integers(0, 2))))
+    while len(out) < 28:  # dense 5x5 / 7x7 of at least 4096 pixels
+        k, s = int(r.choice([5, 7])), int(r.integers(1, 3))
+        ic, oc = int(r.integers(1, 13)) * 4, int(r.integers(8, 41)) * 4
+        ih, iw, n = int(r.integers(20, 70)), int(r.integers(20, 70)), int(r.integers(2, 9))
+        pad = int(r.integers(0, k // 2 + 1))
+        oh, ow = (ih + 2 * pad - k) // s + 1, (iw + 2 * pad - k) // s + 1
+        if n * oh * ow < 4096 or n * oh * ow > 30000:
+            continue
+        act = acts[int(r.integers(0, 4))]
+        sc = unsat(k * k * ic) * (40 if act == A.SIGMOID else 1)
+        out.append(ConvCase(A.FMT_NCHW44, A.DENSE, n, ic, ih, iw, oc, k, s, pad, act, scales=(0.02, 0.01, sc)))
+    return out
+
+
+NEW_SWEEP = _new_kernel_sweep()
+
+
+@pytest.mark.parametrize("case", NEW_SWEEP, ids=[repr(c) for c in NEW_SWEEP])
+def test_pointwise_depthwise_and_row_split_sweep(case):
+    port.set_threads(8)
+    arrays = case.gen(seed=29)
+    got = run_gpu(case, arrays)
+    kernel = runtime.last_kernel()
+    if case.sparse == A.GROUP:
+        assert kernel.startswith("dwconv44_mfma"), kernel
+    elif case.fh == 1 and case.ic <= 512:
+        assert kernel.startswith("conv_pw_stream"), kernel
+    elif case.fh >= 5:
+        assert kernel.startswith("conv_mfma_i8_dma:8") or kernel.startswith("conv_mfma_i8_dma:9"), kernel
+    compare(got, case.run_port(arrays), repr(case))
+
+
 def test_direct_kernel_when_filter_was_not_packed():
     """a caller that skips the init protocol still gets the right answer (generic kernel)"""
     import ctypes as C

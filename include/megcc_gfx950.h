@@ -438,8 +438,20 @@ typedef enum {
     MEGCC_KERN_CONCAT = 9,
     MEGCC_KERN_RESIZE = 10,
     MEGCC_KERN_FUSED_ELEMWISE = 11, /* never produced by parse_symbol; a caller fills the attr */
-    MEGCC_KERN_SOFTMAX = 12         /* never produced by parse_symbol either: see megcc_gfx950_softmax */
+    MEGCC_KERN_SOFTMAX = 12,        /* never produced by parse_symbol either: see megcc_gfx950_softmax */
+    MEGCC_KERN_DW_POOL_ADD = 13     /* nor this one: see megcc_gfx950_dw_pool_add */
 } MegccKernelKind;
+
+/* A channel-wise 3x3 convolution, the 2x2 stride-2 maximum pooling of its result and the quantised
+ * addition of the pooled tensor with a second operand, as one operator (megcc_gfx950_dw_pool_add):
+ * the attributes of the three operators and the scale of the two tensors between them (the pooling
+ * keeps its input's scale, BareMetal/Pooling.cpp:22-27). */
+typedef struct {
+    MegccConvAttr conv;
+    MegccPoolAttr pool;
+    MegccMultiTypeMode mode; /* MEGCC_Q_ADD or MEGCC_Q_FUSE_ADD_RELU */
+    float mid_scale;
+} MegccDwPoolAddAttr;
 
 typedef struct {
     MegccKernelKind kind;
@@ -453,8 +465,29 @@ typedef struct {
         int concat_axis;
         MegccResizeAttr resize;
         MegccFusedElemwiseAttr fused;
+        MegccDwPoolAddAttr dw_pool_add;
     } attr;
 } MegccKernelDesc;
+
+/* Depthwise 3x3 -> max-pool 2x2 stride 2 -> QADD / QFUSE_ADD_RELU in ONE kernel. MegCC emits three
+ * kernels for this chain (kernel_conv2d_3x3_NCHW44_GROUP_..., kernel_pooling_MAX_NCHW44_p0x0_s2x2_w2x2_...,
+ * kernel_elementwise_multitype_...: BareMetal/ConvKernel.cpp:144-176, BareMetal/Pooling.cpp:31-44,
+ * BareMetal/ElemwiseMultiType.cpp:39-48); all three are bound by memory traffic, and two thirds of
+ * that traffic is the depthwise result written and read back and the pooled tensor written and read
+ * back. Here a thread keeps the 2 x 4 depthwise outputs of two pooling windows in registers, takes
+ * the maxima, adds the second operand and stores 2 pixels of the final tensor. The model runtime
+ * (megcc_gfx950_model_finalize) launches this entry point instead of the three kernels when the
+ * tensors between them have no other reader; the three kernels stay available under their symbols.
+ * qsi8 NCHW44 only; conv: GROUP (channel-wise) 3x3, pad 1, stride 1 or 2, dilation 1, any
+ * activation; pool: MAX, window 2x2, stride 2, pad 0. inputs: source, filter, bias (when conv has
+ * one), second operand of the addition (shape of the pooled tensor); outputs[0]: the sum. Bit-identical
+ * to the three kernels run in sequence. megcc_gfx950_dw_pool_add_supported returns 1 for operands
+ * this entry point takes. */
+TinyNNStatus megcc_gfx950_dw_pool_add(
+        const MegccDwPoolAddAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace* workspace, const RuntimeOpt* opt);
+int megcc_gfx950_dw_pool_add_supported(
+        const MegccDwPoolAddAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output);
 
 /* Soft-max over the last axis in ONE kernel. MegCC has no such kernel: its importer decomposes
  * opr::Softmax into Reduce MAX -> SUB -> EXP -> Reduce SUM -> TRUE_DIV
@@ -513,7 +546,7 @@ const char* megcc_gfx950_last_kernel(void);
 /* Kernel-selection overrides, for regression tests of kernels that un-switched shapes only reach
  * through a fallback: "nopws", "nogevm", "nofcb", "nosmall", "nopm768", "nopm", "nodma512",
  * "nopm256", "nodma", "nofcs", "nopwshare", "nohybrid", "nodot4", "nof32small",
- * "dw_generic", "nodwmfma", "nodwnchw", "nofusesoftmax", "nopoolrows", "nofirstmfma", "norowsplit", "no_graph"; value 1 takes the kernel out
+ * "dw_generic", "nodwmfma", "nodwnchw", "nofusesoftmax", "nopoolrows", "nofirstmfma", "norowsplit", "nofusechain", "no_graph"; value 1 takes the kernel out
  * of the dispatch, 0 puts it back. The
  * same names in capitals behind MEGCC_ are read from the environment once, at first use.
  * Unknown names return TinyNN_ERROR_NO_FOUND. */

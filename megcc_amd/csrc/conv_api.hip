@@ -28,6 +28,10 @@ bool conv_first_supported(const ConvGeom& g);
 TinyNNStatus conv_first_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool dwconv44_supported(const ConvGeom& g);
 TinyNNStatus dwconv44_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+bool dwconv44_chain_supported(const ConvGeom& g, const void* src, const void* other, const void* dst);
+TinyNNStatus dwconv44_chain_launch(
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, const void* other, void* dst,
+        bool relu_after_add, float s_other, float s_out);
 void dwconv44_note(const ConvGeom&, const void* src, const void* dst);
 bool dwconv_nchw_supported(const ConvGeom& g, const void* src, const void* dst);
 TinyNNStatus dwconv_nchw_launch(const ConvGeom&, const void*, const void*, const void*, void*);
@@ -647,4 +651,78 @@ extern "C" TinyNNStatus megcc_gfx950_conv2d_workspace(
         }
     }
     return TinyNN_SUCCESS;
+}
+
+// ---- depthwise 3x3 -> max-pool 2x2 s2 -> QADD / QFUSE_ADD_RELU as one operator --------------------
+// Fills `g` (the depthwise layer; its s_dst is the scale between the operators) and checks the
+// operands; `why` gets the reason when they are not what the kernel takes.
+static bool dw_pool_add_geom(
+        const MegccDwPoolAddAttr* a, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output, ConvGeom* g,
+        const Tensor** other_out, const char** why) {
+    *why = "NULL argument";
+    if (!a || !inputs || !outputs || nr_output != 1 || !outputs[0])
+        return false;
+    const int want_in = a->conv.with_bias ? 4 : 3;
+    *why = "inputs: source, filter, [bias,] second operand of the addition";
+    if (nr_input != want_in)
+        return false;
+    for (int i = 0; i < nr_input; ++i)
+        if (!inputs[i])
+            return false;
+    const Tensor *src = inputs[0], *flt = inputs[1], *bias = a->conv.with_bias ? inputs[2] : nullptr;
+    const Tensor *other = inputs[want_in - 1], *dst = outputs[0];
+    *why = "operands must be qsi8 (bias qsi32)";
+    if (!is_q8(src) || !is_q8(flt) || !is_q8(other) || !is_q8(dst) || (bias && !is_q32(bias)))
+        return false;
+    *why = "conv: NCHW44 GROUP 3x3, pad 1, stride 1 or 2; pool: MAX 2x2 stride 2 pad 0 NCHW44; mode: QADD or QFUSE_ADD_RELU";
+    if (a->conv.format != MEGCC_FMT_NCHW44 || a->conv.sparse != MEGCC_SPARSE_GROUP || a->pool.format != MEGCC_FMT_NCHW44 ||
+        a->pool.mode != MEGCC_POOL_MAX || a->pool.window_h != 2 || a->pool.window_w != 2 || a->pool.stride_h != 2 ||
+        a->pool.stride_w != 2 || a->pool.pad_h != 0 || a->pool.pad_w != 0 ||
+        !(a->mode == MEGCC_Q_ADD || a->mode == MEGCC_Q_FUSE_ADD_RELU) || !(a->mid_scale > 0.f))
+        return false;
+    *why = "filter / source layout";
+    if (is_packed_filter(flt) || make_geom(&a->conv, src, flt, nullptr, false, 0, g) != TinyNN_SUCCESS)
+        return false;
+    g->s_dst = a->mid_scale;
+    *why = "bias must be per channel";
+    if (bias && !(nr_elem(bias->layout) == (size_t)g->oc && is_contiguous(bias->layout)))
+        return false;
+    *why = "second operand and result must be contiguous [N, C/4, OH/2, OW/2, 4] tensors";
+    const uint32_t want[5] = {(uint32_t)g->n, (uint32_t)(g->oc / 4), (uint32_t)(g->oh / 2), (uint32_t)(g->ow / 2), 4u};
+    for (const Tensor* t : {other, dst}) {
+        if (t->layout.nr_dim != 5 || !is_contiguous(t->layout))
+            return false;
+        for (int i = 0; i < 5; ++i)
+            if (t->layout.dims[i] != want[i])
+                return false;
+    }
+    *why = "alignment, extent or window the kernel does not take";
+    if (!dwconv44_chain_supported(*g, src->ptr, other->ptr, dst->ptr) || !aligned4(flt->ptr) ||
+        (bias && !aligned4(bias->ptr)))
+        return false;
+    *other_out = other;
+    return true;
+}
+
+extern "C" int megcc_gfx950_dw_pool_add_supported(
+        const MegccDwPoolAddAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output) {
+    ConvGeom g;
+    const Tensor* other = nullptr;
+    const char* why = "";
+    return dw_pool_add_geom(attr, inputs, nr_input, outputs, nr_output, &g, &other, &why) ? 1 : 0;
+}
+
+extern "C" TinyNNStatus megcc_gfx950_dw_pool_add(
+        const MegccDwPoolAddAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace*, const RuntimeOpt*) {
+    ConvGeom g;
+    const Tensor* other = nullptr;
+    const char* why = "";
+    MG_REQUIRE(dw_pool_add_geom(attr, inputs, nr_input, outputs, nr_output, &g, &other, &why),
+               TinyNN_ERROR_INVALID_LAYOUT, "dw_pool_add: %s", why);
+    note_kernel("dwconv44_chain", g.sh, attr->mode == MEGCC_Q_FUSE_ADD_RELU);
+    return dwconv44_chain_launch(
+            g, inputs[0]->ptr, inputs[1]->ptr, attr->conv.with_bias ? inputs[2]->ptr : nullptr, other->ptr,
+            outputs[0]->ptr, attr->mode == MEGCC_Q_FUSE_ADD_RELU, other->dtype.param.scale,
+            outputs[0]->dtype.param.scale);
 }

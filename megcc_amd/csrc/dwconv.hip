@@ -85,11 +85,23 @@ __device__ __forceinline__ void transpose4x4(const dw_v4u p, unsigned (&t)[4]) {
 // are rearranged once for 32 outputs.
 // RAGGED: the input width is not a multiple of the pixels a thread loads per row (4, or 8 with
 // stride 2), so the loads of the last group run into the next row and are masked.
-template <int S, int ACT, int R, bool RAGGED>
+// FUSE: what follows the requantised outputs. 0: they are stored. 1 / 2 (R = 2 only): a 2x2 stride-2
+// maximum pooling over them and QADD / QFUSE_ADD_RELU of the pooled value with `other` follow in
+// registers (BareMetal/Pooling.cpp, BareMetal/ElemwiseMultiType.cpp:39-48: the same float sequence
+// as elemwise.hip); the thread's 2 rows x 4 pixels are two pooling windows, and what it stores is
+// 2 pixels of the final tensor - the depthwise result and the pooled one never reach memory.
+struct DwChain {
+    const uint32_t* other;  // the second operand of the addition: [N][C/4][poh][pow] dwords
+    int poh, pow;           // extent of the pooled tensor: floor(OH / 2), floor(OW / 2)
+    float s_a, s_b, sdiv;   // scale of the pooled operand, of `other`, 1 / scale of the result
+};
+
+template <int S, int ACT, int R, bool RAGGED, int FUSE = 0>
 __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
         ConvGeom g, RequantFast rq, const uint32_t* __restrict__ src, const uint32_t* __restrict__ flt,
         const int32_t* __restrict__ bias, uint32_t* __restrict__ dst, int total, int src_bytes,
-        FastDiv d_ogn, FastDiv d_ohn, FastDiv d_c4n, RequantTable table) {
+        FastDiv d_ogn, FastDiv d_ohn, FastDiv d_c4n, RequantTable table, DwChain fz) {
+    static_assert(FUSE == 0 || R == 2, "a pooling window is two output rows");
     __shared__ int tbl[REQUANT_TABLE_ENTRIES];
     if (ACT >= 0) {
         tbl[threadIdx.x] = table.t[threadIdx.x];
@@ -117,6 +129,19 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
 #pragma unroll
             for (int c = 0; c < 4; ++c)
                 ws[fh][c] = wq[fh][c] << 8;
+        }
+        // FUSE: the second operand of the addition for the thread's two pooled pixels, requested before
+        // the input rows (a load issued where its value is needed would wait a round trip to memory)
+        uint32_t other4[2] = {0u, 0u};
+        if (FUSE) {
+            const int py = oh >> 1;  // (oh is even: R = 2)
+            if (py < fz.poh) {
+                const size_t row = ((size_t)(n * c4n + c4) * fz.poh + py) * fz.pow;
+#pragma unroll
+                for (int k = 0; k < 2; ++k)
+                    if (og * 2 + k < fz.pow)
+                        other4[k] = fz.other[row + og * 2 + k];
+            }
         }
         int acc[R * 16];  // [row][pixel][channel]
         {
@@ -196,7 +221,22 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
                                 acc[orow * 16 + j * 4 + c], false);
             }
         }
-        if (ACT < 0) {
+        if (FUSE && ACT >= 0) {
+            // with the threshold table the requantisation is a non-decreasing function of the
+            // accumulator, so max F(a_i) = F(max a_i): pool the int32 accumulators first and requantise
+            // 8 instead of 32 values (the pooled ones land where the code below looks for window k:
+            // row 0, pixel 2 * k; the other three places get the same value)
+#pragma unroll
+            for (int k = 0; k < 2; ++k)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int m = max(max(acc[(2 * k) * 4 + c], acc[(2 * k + 1) * 4 + c]),
+                                      max(acc[16 + (2 * k) * 4 + c], acc[16 + (2 * k + 1) * 4 + c]));
+                    const int f = requant_conv_table<(ACT < 0 ? 0 : ACT)>(m, rq.c, tbl);
+                    acc[(2 * k) * 4 + c] = acc[(2 * k + 1) * 4 + c] = f;
+                    acc[16 + (2 * k) * 4 + c] = acc[16 + (2 * k + 1) * 4 + c] = f;
+                }
+        } else if (ACT < 0) {
 #pragma unroll
             for (int e = 0; e < R * 16; ++e)
                 acc[e] = requant_conv_rt(g.act, acc[e], g.s_src, g.s_flt, g.s_dst);
@@ -204,6 +244,31 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
 #pragma unroll
             for (int e = 0; e < R * 16; ++e)
                 acc[e] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[e], rq.c, tbl);
+        }
+        if (FUSE) {
+            const int py = oh >> 1;  // (oh is even: R = 2)
+            if (py < fz.poh) {
+                const size_t row = ((size_t)(n * c4n + c4) * fz.poh + py) * fz.pow;
+#pragma unroll
+                for (int k = 0; k < 2; ++k) {
+                    const int px = og * 2 + k;
+                    if (px >= fz.pow)
+                        break;
+                    const uint32_t b4 = other4[k];
+                    int r[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const int m0 = max(acc[(2 * k) * 4 + c], acc[(2 * k + 1) * 4 + c]);
+                        const int m1 = max(acc[16 + (2 * k) * 4 + c], acc[16 + (2 * k + 1) * 4 + c]);
+                        const float v0 = fz.s_a * (float)max(m0, m1);
+                        const float v1 = fz.s_b * (float)sbyte(b4, c);
+                        const float sum = v0 + v1;
+                        r[c] = fp32_to_int8((FUSE == 2 ? (sum > 0 ? sum : 0) : sum) * fz.sdiv);
+                    }
+                    dst[row + px] = pack4_perm(r[0], r[1], r[2], r[3]);
+                }
+            }
+            continue;
         }
 #pragma unroll
         for (int orow = 0; orow < R; ++orow) {
@@ -234,6 +299,63 @@ static bool dwconv44_3x3_ok(const ConvGeom& g, const void* src, const void* dst)
            g.sh == g.sw && (g.sh == 1 || g.sh == 2) &&
            ((uintptr_t)src & 3) == 0 && ((uintptr_t)dst & 15) == 0 && src_bytes < (1L << 31) && groups4 < (1L << 31) &&
            (long)g.n * g.oc * g.oh * g.ow < (1L << 31);
+}
+
+// ---- depthwise 3x3 -> 2x2 stride-2 maximum pooling -> QADD / QFUSE_ADD_RELU as one kernel ------------
+// (g.s_dst is the scale of the depthwise result, which the pooling keeps; `other` has the extent of the
+//  pooled tensor)
+bool dwconv44_chain_supported(const ConvGeom& g, const void* src, const void* other, const void* dst) {
+    return g.fmt == MEGCC_FMT_NCHW44 && g.groups > 1 && g.groups == g.ic && g.ic == g.oc && (g.ic & 3) == 0 &&
+           dwconv44_3x3_ok(g, src, dst) && ((uintptr_t)other & 3) == 0 && g.oh >= 2 && g.ow >= 2;
+}
+
+bool dwconv44_mfma_chain_supported(const ConvGeom& g, const void* src, const void* dst);
+TinyNNStatus dwconv44_mfma_chain_launch(
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, const void* other, void* dst,
+        bool relu_after_add, float s_other, float s_out);
+
+TinyNNStatus dwconv44_chain_launch(
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, const void* other, void* dst,
+        bool relu_after_add, float s_other, float s_out) {
+    // stride 1: the multiply-adds on the matrix cores, as for the layer on its own
+    if (dwconv44_mfma_chain_supported(g, src, dst) && !options().no_dwmfma && !options().dw_generic)
+        return dwconv44_mfma_chain_launch(g, src, flt, bias, other, dst, relu_after_add, s_other, s_out);
+    constexpr int R = 2;
+    const int groups4 = (int)((long)g.n * (g.oc >> 2) * ((g.oh + R - 1) / R) * ((g.ow + 3) / 4));
+    if (groups4 == 0)
+        return TinyNN_SUCCESS;
+    const unsigned nb = (unsigned)((groups4 + 255) / 256);
+    const RequantFast rq3 = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
+    const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
+                     requant_table_ok(g.s_src, g.s_flt, g.s_dst);
+    static const RequantTable no_table = {};
+    const RequantTable& table = tab ? requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst) : no_table;
+    DwChain fz;
+    fz.other = (const uint32_t*)other;
+    fz.poh = g.oh / 2;
+    fz.pow = g.ow / 2;
+    fz.s_a = g.s_dst;
+    fz.s_b = s_other;
+    fz.sdiv = 1.f / s_out;
+    void (*k)(ConvGeom, RequantFast, const uint32_t*, const uint32_t*, const int32_t*, uint32_t*, int, int, FastDiv,
+              FastDiv, FastDiv, RequantTable, DwChain);
+#define MG_DWC_ACT(S_, G_, F_)                                                                             \
+    (tab && g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_IDENTITY, 2, G_, F_>     \
+     : tab && g.act == MEGCC_NONLINE_RELU   ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_RELU, 2, G_, F_>         \
+                                            : dwconv44_3x3_kernel<S_, -1, 2, G_, F_>)
+#define MG_DWC_PICK(S_, G_) (relu_after_add ? MG_DWC_ACT(S_, G_, 2) : MG_DWC_ACT(S_, G_, 1))
+    const bool ragged = (g.iw % (4 * g.sh)) != 0;
+    if (g.sh == 1)
+        k = ragged ? MG_DWC_PICK(1, true) : MG_DWC_PICK(1, false);
+    else
+        k = ragged ? MG_DWC_PICK(2, true) : MG_DWC_PICK(2, false);
+#undef MG_DWC_PICK
+#undef MG_DWC_ACT
+    hipLaunchKernelGGL(k, dim3(nb), dim3(256), 0, stream(), g, rq3, (const uint32_t*)src, (const uint32_t*)flt,
+                       (const int32_t*)bias, (uint32_t*)dst, groups4, (int)((long)g.n * g.ic * g.ih * g.iw),
+                       make_fastdiv((g.ow + 3) / 4), make_fastdiv((g.oh + R - 1) / R), make_fastdiv(g.oc >> 2), table,
+                       fz);
+    return check_launch("dwconv44_chain");
 }
 
 bool dwconv44_supported(const ConvGeom& g) {
@@ -282,7 +404,7 @@ TinyNNStatus dwconv44_launch(
         unsigned nb = (unsigned)((groups4 + 255) / 256);
         const RequantFast rq3 = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
         void (*k3)(ConvGeom, RequantFast, const uint32_t*, const uint32_t*, const int32_t*, uint32_t*, int, int,
-                   FastDiv, FastDiv, FastDiv, RequantTable);
+                   FastDiv, FastDiv, FastDiv, RequantTable, DwChain);
         // exact thresholds for the monotone activations; anything else (and extreme scales)
         // evaluates the literal sequence per output
         const bool tab = requant_table_act(g.act) && requant_table_ok(g.s_src, g.s_flt, g.s_dst);
@@ -304,7 +426,7 @@ TinyNNStatus dwconv44_launch(
         hipLaunchKernelGGL(k3, dim3(nb), dim3(256), 0, stream(), g, rq3, (const uint32_t*)src,
                            (const uint32_t*)flt, (const int32_t*)bias, (uint32_t*)dst, groups4,
                            (int)((long)g.n * g.ic * g.ih * g.iw), make_fastdiv((g.ow + 3) / 4),
-                           make_fastdiv((g.oh + R - 1) / R), make_fastdiv(g.oc >> 2), table);
+                           make_fastdiv((g.oh + R - 1) / R), make_fastdiv(g.oc >> 2), table, DwChain{});
         return check_launch("dwconv44_3x3");
     }
     unsigned blocks = (unsigned)((total + 255) / 256);

@@ -64,26 +64,42 @@ struct DwMfmaParams {
     int act;
     float s_src, s_flt, s_dst, c;
     FastDiv d_ohp, d_xb;  // division by ohp, by xblocks
+    // FUSE: the second operand of the addition that follows the pooling ([N][C/4][poh][pow] dwords), the
+    // extent of the pooled tensor, the scales of the pooled operand and of `other`, 1 / the result's
+    const uint32_t* other;
+    int poh, pow;
+    float s_a, s_b, sdiv;
     RequantTable table;
+};
+
+struct DwMfmaChain {
+    const void* other;
+    bool relu_after_add;
+    float s_other, s_out;
 };
 
 typedef unsigned dwm_v2u __attribute__((ext_vector_type(2)));
 typedef unsigned dw_v4u __attribute__((ext_vector_type(4)));
-// output rows per lane and tile (2 share input rows and index arithmetic but need 200 registers:
-// measured 15.3 us against 14.9 us with 1 on N=64 C=32 112x112)
-static constexpr int DWM_ROWS = 1;
+// R: output rows per lane and tile (2 share input rows and index arithmetic but need 200 registers:
+// measured 15.3 us against 14.9 us with 1 on N=64 C=32 112x112; the layer on its own uses 1).
+// FUSE (3x3 stride 1 with R = 2 only): 1 / 2 = a 2x2 stride-2 maximum pooling of the requantised
+// outputs and QADD / QFUSE_ADD_RELU of the pooled value with q.other follow in registers (the same
+// float sequence as elemwise.hip, BareMetal/ElemwiseMultiType.cpp:39-48). A lane's 2 rows x 4 pixels
+// are the halves of four pooling windows whose other halves the lane 32 further on holds: after the
+// vertical maximum the same two v_permlane32_swap that prepare the 16-byte stores of the plain
+// kernel hand each lane both halves of two windows; it stores 2 pixels of the final tensor.
 
 // S: stride (only 1 is instantiated: with stride 2 the layer reads four bytes per byte written and
 // the v_dot4 kernel of dwconv.hip already runs at the rate of a copy - measured 7.8 us against
 // 9.8 us for this one on N=64 C=32 112x112). RAGGED: IW is not a multiple of 4, so the last 16-byte load of a row runs into the
 // next row and is masked. ACT: IDENTITY / RELU / H_SWISH use the threshold table, -1 evaluates the literal
 // sequence with the run-time activation. F: filter rows = filter columns (3, 5 or 7; pad F / 2).
-template <int S, bool RAGGED, int ACT, int F = 3>
+template <int S, bool RAGGED, int ACT, int F = 3, int R = 1, int FUSE = 0>
 __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
+    static_assert(FUSE == 0 || (R == 2 && S == 1 && F == 3), "a pooling window is two output rows");
     static_assert(F == 3 || F == 5 || F == 7, "the band must fit S + 1 K steps: pad <= 3");
     constexpr int PAD = F / 2;
     constexpr int NS = S + 1;            // K steps a group of 8 output pixels reads
-    constexpr int R = DWM_ROWS;          // output rows per lane and tile
     constexpr int IR = (R - 1) * S + F;  // input rows they read
     __shared__ int tbl[REQUANT_TABLE_ENTRIES];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -155,6 +171,11 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
     // row (<= 0: nothing to store), rows left in the image
     struct Where {
         int off, left, rows;
+        // FUSE: dword index of the lane's first pooled pixel in `other` / the result, how many of its 2
+        // pixels exist, and the second operand's 2 dwords (requested with the tile's rows: a load
+        // issued where its value is needed would put a round trip to memory behind every tile)
+        int pidx, pleft;
+        uint32_t b4[2];
     };
     // requests the B operands of a tile: NS aligned 16-byte loads for each of the IR input rows
     auto request = [&](int tile, v4i (&B)[IR][NS]) __attribute__((always_inline)) -> Where {
@@ -188,6 +209,15 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
         w.off = ((pset * q.oh + y) * q.ow + xo) * 4;
         w.left = col_ok ? q.ow - xo : 0;
         w.rows = q.oh - y;
+        if constexpr (FUSE != 0) {
+            const int py = rg - n * q.ohp;  // (R = 2: row group = pooled row)
+            const int px0 = (x0 >> 1) + 2 * kg;
+            w.pidx = (pset * q.poh + py) * q.pow + px0;
+            w.pleft = col_ok && py < q.poh ? q.pow - px0 : 0;
+#pragma unroll
+            for (int k = 0; k < 2; ++k)
+                w.b4[k] = w.pleft > k ? q.other[w.pidx + k] : 0u;
+        }
         return w;
     };
 
@@ -209,6 +239,62 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
         // the operands are consumed: the next tile's loads fly while this one is requantised
         // (past the last tile every offset is out of range and nothing is fetched)
         next = request(tile + tstep, B);
+        if constexpr (FUSE != 0) {
+            // ---- pool, requantise, add, store ----------------------------------------------------
+            // With the threshold table the requantisation F is a non-decreasing function of the
+            // accumulator (epilogue.h), so max F(a_i) = F(max a_i): the maximum is taken over the
+            // int32 accumulators and 8 instead of 32 values per lane are requantised. The literal
+            // sequence (SIGMOID, extreme scales) requantises first.
+            int pooled[2][4];  // [window of this lane][channel], requantised
+            if (ACT >= 0) {
+                int v[16];  // vertical maximum: pixel 2 * (e / 4) + kg, channel e % 4
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    v[e] = max(acc[0][e], acc[1][e]);
+                // lower half wave: both halves of windows 0 and 1; upper: of windows 2 and 3
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const dwm_v2u s02 = __builtin_amdgcn_permlane32_swap((unsigned)v[c], (unsigned)v[8 + c], false, false);
+                    const dwm_v2u s13 = __builtin_amdgcn_permlane32_swap((unsigned)v[4 + c], (unsigned)v[12 + c], false, false);
+                    pooled[0][c] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(max((int)s02[0], (int)s02[1]), q.c, tbl);
+                    pooled[1][c] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(max((int)s13[0], (int)s13[1]), q.c, tbl);
+                }
+            } else {
+                unsigned d[4];  // vertical maximum of pixel 2 * j + kg, 4 requantised channel bytes
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    int o[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        o[c] = max(requant_conv_rt(q.act, acc[0][4 * j + c], q.s_src, q.s_flt, q.s_dst),
+                                   requant_conv_rt(q.act, acc[1][4 * j + c], q.s_src, q.s_flt, q.s_dst));
+                    d[j] = pack4_perm(o[0], o[1], o[2], o[3]);
+                }
+                const dwm_v2u s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+                const dwm_v2u s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    pooled[0][c] = max(sbyte(s02[0], c), sbyte(s02[1], c));
+                    pooled[1][c] = max(sbyte(s13[0], c), sbyte(s13[1], c));
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const bool ok = cur.pleft > k;
+                const uint32_t b4 = cur.b4[k];
+                int r4[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float v0 = q.s_a * (float)pooled[k][c];
+                    const float v1 = q.s_b * (float)sbyte(b4, c);
+                    const float sum = v0 + v1;
+                    r4[c] = fp32_to_int8((FUSE == 2 ? (sum > 0 ? sum : 0) : sum) * q.sdiv);
+                }
+                if (ok)
+                    q.dst[cur.pidx + k] = pack4_perm(r4[0], r4[1], r4[2], r4[3]);
+            }
+            continue;
+        }
         // ---- requantise, pack, exchange, store ---------------------------------------------------
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -253,9 +339,19 @@ bool dwconv44_mfma_supported(const ConvGeom& g, const void* src, const void* dst
            (long)g.n * g.oc * g.oh * g.ow < (1L << 31) && (long)g.n * g.oh * ((g.ow + 7) / 8) < (1L << 30) && (long)g.ih * g.iw < (1L << 24);
 }
 
-TinyNNStatus dwconv44_mfma_launch(
-        const ConvGeom& g, const void* src, const void* flt, const void* bias, void* dst) {
+// chain: the pooling + addition that follow (FUSE), or NULL
+static TinyNNStatus dwconv44_mfma_run(
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, void* dst, const DwMfmaChain* chain) {
+    const int rows = chain ? 2 : 1;
     DwMfmaParams q = {};
+    if (chain) {
+        q.other = (const uint32_t*)chain->other;
+        q.poh = g.oh / 2;
+        q.pow = g.ow / 2;
+        q.s_a = g.s_dst;
+        q.s_b = chain->s_other;
+        q.sdiv = 1.f / chain->s_out;
+    }
     q.src = (const uint32_t*)src;
     q.flt = (const uint32_t*)flt;
     q.bias = (const int32_t*)bias;
@@ -266,9 +362,9 @@ TinyNNStatus dwconv44_mfma_launch(
     q.iw = g.iw;
     q.oh = g.oh;
     q.ow = g.ow;
-    q.dst_bytes = (int)((long)g.n * g.oc * g.oh * g.ow);
+    q.dst_bytes = chain ? (int)((long)g.n * g.oc * (g.oh / 2) * (g.ow / 2)) : (int)((long)g.n * g.oc * g.oh * g.ow);
     q.xblocks = (g.ow + 7) / 8;
-    q.ohp = (g.oh + DWM_ROWS - 1) / DWM_ROWS;
+    q.ohp = (g.oh + rows - 1) / rows;
     q.cols = g.n * q.ohp * q.xblocks;
     q.tiles = (q.cols + 31) / 32;
     q.act = g.act;
@@ -292,7 +388,19 @@ TinyNNStatus dwconv44_mfma_launch(
      : act == MEGCC_NONLINE_H_SWISH ? (const void*)dwconv44_mfma_kernel<S_, R_, MEGCC_NONLINE_H_SWISH, F_> \
                                    : (const void*)dwconv44_mfma_kernel<S_, R_, -1, F_>)
 #define MG_DWM_F(S_, F_) (ragged ? MG_DWM_ACT(S_, true, F_) : MG_DWM_ACT(S_, false, F_))
-    if (g.fh == 3)
+    if (chain) {
+        // (IDENTITY / RELU through the table, anything else the literal sequence)
+        const int a2 = act == MEGCC_NONLINE_H_SWISH ? -1 : act;
+#define MG_DWM_CHAIN(R_, FZ_)                                                                                  \
+    (a2 == MEGCC_NONLINE_IDENTITY ? (const void*)dwconv44_mfma_kernel<1, R_, MEGCC_NONLINE_IDENTITY, 3, 2, FZ_> \
+     : a2 == MEGCC_NONLINE_RELU   ? (const void*)dwconv44_mfma_kernel<1, R_, MEGCC_NONLINE_RELU, 3, 2, FZ_>     \
+                                  : (const void*)dwconv44_mfma_kernel<1, R_, -1, 3, 2, FZ_>)
+        if (chain->relu_after_add)
+            kern = ragged ? MG_DWM_CHAIN(true, 2) : MG_DWM_CHAIN(false, 2);
+        else
+            kern = ragged ? MG_DWM_CHAIN(true, 1) : MG_DWM_CHAIN(false, 1);
+#undef MG_DWM_CHAIN
+    } else if (g.fh == 3)
         kern = MG_DWM_F(1, 3);
     else if (g.fh == 5)
         kern = g.sh == 1 ? MG_DWM_F(1, 5) : MG_DWM_F(2, 5);
@@ -316,6 +424,23 @@ TinyNNStatus dwconv44_mfma_launch(
     hipError_t e = hipLaunchKernel(kern, dim3((unsigned)(waves / 4)), dim3(256), args, 0, stream());
     MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "dwconv44_mfma: %s", hipGetErrorString(e));
     return check_launch("dwconv44_mfma");
+}
+
+TinyNNStatus dwconv44_mfma_launch(
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, void* dst) {
+    return dwconv44_mfma_run(g, src, flt, bias, dst, nullptr);
+}
+
+// 3x3 stride 1 -> max-pool 2x2 stride 2 -> QADD / QFUSE_ADD_RELU in one kernel (g.s_dst: the scale of
+// the depthwise result; dst and other: [N][C/4][OH / 2][OW / 2][4])
+bool dwconv44_mfma_chain_supported(const ConvGeom& g, const void* src, const void* dst) {
+    return dwconv44_mfma_supported(g, src, dst) && g.fh == 3 && g.sh == 1 && g.oh >= 2 && g.ow >= 2;
+}
+TinyNNStatus dwconv44_mfma_chain_launch(
+        const ConvGeom& g, const void* src, const void* flt, const void* bias, const void* other, void* dst,
+        bool relu_after_add, float s_other, float s_out) {
+    const DwMfmaChain chain = {other, relu_after_add, s_other, s_out};
+    return dwconv44_mfma_run(g, src, flt, bias, dst, &chain);
 }
 
 }  // namespace mg

@@ -159,6 +159,45 @@ static void build_schedule(Model* m) {
     };
     for (int i = 0; i < n; ++i) {
         ModelOpr* o0 = m->oprs[i];
+        // A channel-wise 3x3 convolution, the 2x2 stride-2 maximum pooling of its result and the
+        // quantised addition of the pooled tensor with another one: all three are bound by memory
+        // traffic, and two thirds of it is the two tensors in between going out and coming back.
+        // When nothing else reads those, the chain runs as ONE kernel (megcc_gfx950_dw_pool_add).
+        if (!options().no_fuse_chain && i + 2 < n && o0->desc.kind == MEGCC_KERN_CONV && !o0->has_processed &&
+            o0->out.size() == 1) {
+            ModelOpr *o1 = m->oprs[i + 1], *o2 = m->oprs[i + 2];
+            if (o1->desc.kind == MEGCC_KERN_POOLING && o1->in.size() == 1 && o1->out.size() == 1 &&
+                o1->in[0] == o0->out[0] && o2->desc.kind == MEGCC_KERN_ELEMWISE_MULTITYPE && o2->in.size() == 2 &&
+                o2->out.size() == 1 && (o2->in[0] == o1->out[0]) != (o2->in[1] == o1->out[0]) &&
+                temp(o0->out[0], 1) && temp(o1->out[0], 1) &&
+                m->tensors[o0->out[0]]->t.dtype.param.scale == m->tensors[o1->out[0]]->t.dtype.param.scale) {
+                const int other = o2->in[0] == o1->out[0] ? o2->in[1] : o2->in[0];
+                ModelOpr* f = new ModelOpr();
+                memset(&f->desc, 0, sizeof(f->desc));
+                f->desc.kind = MEGCC_KERN_DW_POOL_ADD;
+                f->desc.attr.dw_pool_add.conv = o0->desc.attr.conv;
+                f->desc.attr.dw_pool_add.pool = o1->desc.attr.pool;
+                f->desc.attr.dw_pool_add.mode = o2->desc.attr.multitype;
+                f->desc.attr.dw_pool_add.mid_scale = m->tensors[o0->out[0]]->t.dtype.param.scale;
+                f->symbol = "depthwise 3x3 + max-pool 2x2 + add (fused)";
+                memset(&f->ws, 0, sizeof(f->ws));
+                f->in = o0->in;
+                f->in_ptrs = o0->in_ptrs;
+                f->in.push_back(other);
+                f->in_ptrs.push_back(&m->tensors[other]->t);
+                f->out = o2->out;
+                f->out_ptrs = o2->out_ptrs;
+                if (megcc_gfx950_dw_pool_add_supported(
+                            &f->desc.attr.dw_pool_add, f->in_ptrs.data(), (int)f->in_ptrs.size(), f->out_ptrs.data(),
+                            (int)f->out_ptrs.size())) {
+                    m->fused.push_back(f);
+                    m->schedule.push_back(f);
+                    i += 2;
+                    continue;
+                }
+                delete f;
+            }
+        }
         bool fuse = !options().no_fuse_softmax && i + 4 < n && is_red(o0, MEGCC_REDUCE_MAX) &&
                     is_ew(m->oprs[i + 1], MEGCC_EW_SUB, 2) && is_ew(m->oprs[i + 2], MEGCC_EW_EXP, 1) &&
                     is_red(m->oprs[i + 3], MEGCC_REDUCE_SUM) && is_ew(m->oprs[i + 4], MEGCC_EW_TRUE_DIV, 2);

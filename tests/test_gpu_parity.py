@@ -870,3 +870,112 @@ def test_every_accumulator_value_requantises_like_the_literal_sequence(act, scal
     if scales[2] == 0.025:
         assert len(np.unique(want)) == (128 if act != A.IDENTITY else 256), "the range must cover every threshold"
     compare(got, want, repr(case))
+
+
+# ---- depthwise 3x3 -> max-pool 2x2 s2 -> QADD / QFUSE_ADD_RELU in one kernel ------------------------
+CHAINS = [
+    # (n, c, ih, iw, stride, conv activation, add mode, bias): the four shapes of the bandwidth-bound
+    # configuration at a small batch, odd extents (the pooling drops the last row / column), rows that
+    # are no multiple of 4 / 8 pixels, one pooled pixel, every activation, both additions, no bias
+    (2, 32, 112, 112, 1, A.RELU, A.Q_FUSE_ADD_RELU, True), (2, 32, 112, 112, 2, A.RELU, A.Q_FUSE_ADD_RELU, True),
+    (3, 512, 14, 14, 1, A.RELU, A.Q_FUSE_ADD_RELU, True), (3, 512, 14, 14, 2, A.RELU, A.Q_FUSE_ADD_RELU, True),
+    (2, 8, 13, 19, 1, A.IDENTITY, A.Q_ADD, True), (2, 12, 21, 30, 2, A.H_SWISH, A.Q_ADD, False),
+    (1, 4, 2, 2, 1, A.SIGMOID, A.Q_FUSE_ADD_RELU, True), (3, 20, 9, 6, 1, A.RELU, A.Q_ADD, False),
+    (2, 16, 11, 37, 2, A.IDENTITY, A.Q_FUSE_ADD_RELU, True), (1, 8, 5, 3, 1, A.RELU, A.Q_FUSE_ADD_RELU, True),
+]
+
+
+def _chain_cases(n, c, ih, iw, stride, act, mode, bias):
+    sc = unsat(9) * (40 if act == A.SIGMOID else 1)
+    dw = ConvCase(A.FMT_NCHW44, A.GROUP, n, c, ih, iw, c, 3, stride, 1, act, scales=(0.02, 0.01, sc), bias=bias)
+    pool = PoolCase(A.FMT_NCHW44, A.POOL_MAX, n, c, dw.oh, dw.ow, 2, 2, 0, scale=sc)
+    add = MultiTypeCase(mode, pool.dst_shape(), (sc, 0.013, 0.9 * sc))
+    return dw, pool, add
+
+
+@pytest.mark.parametrize("cfg", CHAINS, ids=["n%d_c%d_%dx%d_s%d_%s_%s%s" % (
+    c[0], c[1], c[2], c[3], c[4], A.NONLINE_NAMES[c[5]], A.MULTITYPE_NAMES[c[6]], "" if c[7] else "_nobias")
+    for c in CHAINS])
+def test_depthwise_pool_add_in_one_kernel_equals_the_three_operator_chain(cfg):
+    """megcc_gfx950_dw_pool_add against the oracle's depthwise convolution, pooling and addition run
+    one after the other, bit for bit"""
+    import ctypes as C
+    dw, pool, add = _chain_cases(*cfg)
+    arrays = dw.gen(11)
+    other = np.random.default_rng(12).integers(-128, 128, pool.dst_shape()).astype(np.int8)
+    want = add.run_port({"a": pool.run_port({"src": dw.run_port(arrays)}), "b": other})
+    attr = abi.DwPoolAddAttr()
+    attr.conv = dw.attr()
+    attr.pool = abi.PoolAttr(2, 2, 2, 2, 0, 0, A.FMT_NCHW44, A.POOL_MAX)
+    attr.mode = cfg[6]
+    attr.mid_scale = dw.scales[2]
+    ins, _ = dw.specs(arrays)
+    bufs = [runtime.DeviceBuffer.from_array(s.array) for s in ins] + [runtime.DeviceBuffer.from_array(other)]
+    out = runtime.DeviceBuffer(want.nbytes)
+    out.fill(cases.POISON)
+    tin = [abi.make_tensor(b.ptr, s.shape, s.type_enum, s.scale, s.name) for b, s in zip(bufs, ins)]
+    tin.append(abi.make_tensor(bufs[-1].ptr, pool.dst_shape(), abi.QINT8, add.scales[1], b"other"))
+    tout = [abi.make_tensor(out.ptr, pool.dst_shape(), abi.QINT8, add.scales[2], b"dst")]
+    L = runtime.lib()
+    L.megcc_gfx950_dw_pool_add_supported.argtypes = [
+        C.POINTER(abi.DwPoolAddAttr), C.POINTER(C.POINTER(abi.Tensor)), C.c_int, C.POINTER(C.POINTER(abi.Tensor)), C.c_int]
+    L.megcc_gfx950_dw_pool_add.argtypes = L.megcc_gfx950_dw_pool_add_supported.argtypes + [C.c_void_p, C.c_void_p]
+    assert L.megcc_gfx950_dw_pool_add_supported(C.byref(attr), abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1) == 1
+    runtime.check(L.megcc_gfx950_dw_pool_add(C.byref(attr), abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1,
+                                             None, None), "dw_pool_add")
+    runtime.wait()
+    got = out.to_array(want.shape, np.int8)
+    compare(got, want, repr(dw))
+    # what the entry point refuses: a 5x5 window, average pooling, a second operand of another shape
+    attr.pool.mode = A.POOL_AVERAGE
+    assert L.megcc_gfx950_dw_pool_add_supported(C.byref(attr), abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1) == 0
+    assert L.megcc_gfx950_dw_pool_add(C.byref(attr), abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1,
+                                      None, None) == abi.ERROR_INVALID_LAYOUT
+    for b in bufs + [out]:
+        b.free()
+
+
+def _chain_model(cfg, fused):
+    dw, pool, add = _chain_cases(*cfg)
+    arrays = dw.gen(11)
+    other = np.random.default_rng(12).integers(-128, 128, pool.dst_shape()).astype(np.int8)
+    runtime.set_option("nofusechain", 0 if fused else 1)
+    try:
+        m = runtime.Model()
+        x = m.tensor("x", dw.src_shape(), abi.QINT8, dw.scales[0])
+        y = m.tensor("other", pool.dst_shape(), abi.QINT8, add.scales[1])
+        m.mark_input(x)
+        m.mark_input(y)
+        ins = [x, m.weight("dw.w", arrays["flt"], abi.QINT8, dw.scales[1])]
+        if dw.bias:
+            ins.append(m.weight("dw.b", arrays["bias"], abi.QINT32, float(np.float32(dw.scales[0]) * np.float32(dw.scales[1]))))
+        t1 = m.tensor("dw", dw.dst_shape(), abi.QINT8, dw.scales[2])
+        m.opr(dw.symbol(), ins, [t1])
+        t2 = m.tensor("pool", pool.dst_shape(), abi.QINT8, dw.scales[2])
+        m.opr(pool.symbol(), [t1], [t2])
+        t3 = m.tensor("out", pool.dst_shape(), abi.QINT8, add.scales[2])
+        m.opr(add.symbol(), [y, t2] if cfg[0] & 1 else [t2, y], [t3])  # (the pooled tensor on either side)
+        m.mark_output(t3)
+        m.finalize()
+    finally:
+        runtime.set_option("nofusechain", 0)
+    m.set_input(x, arrays["src"])
+    m.set_input(y, other)
+    outs = []
+    for _ in range(3):  # eager, captured, replayed
+        m.forward()
+        runtime.wait()
+        outs.append(m.get(t3).copy())
+    kernel = runtime.last_kernel()
+    want = add.run_port({"a": pool.run_port({"src": dw.run_port(arrays)}), "b": other})
+    return outs, kernel, want
+
+
+@pytest.mark.parametrize("cfg", CHAINS[:6], ids=[str(i) for i in range(6)])
+def test_model_runtime_fuses_the_depthwise_pool_add_chain(cfg):
+    fused, kernel, want = _chain_model(cfg, True)
+    assert kernel.startswith("dwconv44_chain"), kernel
+    plain, kernel, _ = _chain_model(cfg, False)
+    assert not kernel.startswith("dwconv44_chain"), kernel
+    for o in fused + plain:
+        compare(o, want, "chain %r" % (cfg,))

@@ -630,7 +630,10 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
     // the first forward runs eagerly (it also warms per-kernel attributes), the second is captured
     if (m->graph_state == 0 && m->forwards >= 2) {
         m->graph_state = -1;
-        if (!options().no_graph &&
+        // (a graph launch costs about 13 us before its first kernel starts, an eager launch 3-4 us
+        //  per kernel: schedules of fewer than 5 kernels stay eager - the depthwise + pooling +
+        //  addition chain as one kernel takes 7.6 us per forward eagerly, 16.2 us as a graph)
+        if (!options().no_graph && m->schedule.size() >= 5 &&
             hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal) == hipSuccess) {
             TinyNNStatus st = forward_eager(m);
             hipGraph_t g = nullptr;

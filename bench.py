@@ -320,8 +320,9 @@ def check_output(case, arrays, got):
 
 def bench_chain(c, hw, stride, steps, warmup, batch=64):
     """BASELINE configs[3]: depthwise 3x3 -> max-pool 2x2 s2 -> add + ReLU with requantisation,
-    three operators of one model on the static arena, replayed as a HIP graph. Bytes = what each
-    operator must read and write once (the pooled map's partner tensor included)."""
+    three operators of one model on the static arena (the model runtime runs the chain as one kernel
+    when nothing else reads the tensors in between). Bytes = what each operator must read and write
+    once (the pooled map's partner tensor included)."""
     import numpy as np
     from cases import ConvCase, MultiTypeCase, PoolCase
     from megcc_amd import abi, runtime

@@ -70,11 +70,18 @@ struct Model {
     // of plan_memory(); model inputs then live outside the arena, as in the TinyNN runtime
     bool preplanned = false;
     // The operator sequence of a finalized model never changes (static shapes, static memory plan),
-    // so after one eager forward it is captured once into a HIP graph and replayed: one launch per
-    // forward instead of one per operator. 0: not tried yet, 1: graph in use, -1: capture failed
-    // or switched off (MEGCC_NO_GRAPH), stay eager.
+    // so it can be captured once into a HIP graph and replayed: one launch per forward instead of one
+    // per operator. 0: not decided yet, 1: graph in use, -1: eager (measured faster, capture failed,
+    // a schedule of fewer than 5 kernels, or switched off by MEGCC_NO_GRAPH).
+    // Whether replaying wins is MEASURED: a graph launch costs about 13 us before its first kernel
+    // starts, eager launches cost the host 3-4 us per kernel, so small batches (host-bound) gain from
+    // the graph and large ones lose its fixed cost. Forward 1 runs eagerly (it warms per-kernel
+    // attributes), 2 and 3 eagerly between two events, 4 captures and launches, 5 and 6 replay between
+    // the events; from forward 7 on the faster way is used.
     int graph_state = 0;
     int forwards = 0;
+    float eager_ms = 1e30f, graph_ms = 1e30f;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
 };
@@ -288,6 +295,10 @@ void megcc_gfx950_model_destroy(void* model) {
         m->dev.free(m->arena);
     if (m->workspace)
         m->dev.free(m->workspace);
+    if (m->ev0)
+        (void)hipEventDestroy(m->ev0);
+    if (m->ev1)
+        (void)hipEventDestroy(m->ev1);
     if (m->graph_exec)
         (void)hipGraphExecDestroy(m->graph_exec);
     if (m->graph)
@@ -621,31 +632,50 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
     Model* m = (Model*)model;
     MG_REQUIRE(m && m->finalized, TinyNN_ERROR_NULL_PTR, "model_forward: model not finalized");
     ++m->forwards;
-    if (m->graph_state == 1) {
+    auto replay = [&]() -> TinyNNStatus {
         hipError_t e = hipGraphLaunch(m->graph_exec, stream());
-        MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "model_forward: graph launch: %s",
-                   hipGetErrorString(e));
+        MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "model_forward: graph launch: %s", hipGetErrorString(e));
         return TinyNN_SUCCESS;
-    }
-    // the first forward runs eagerly (it also warms per-kernel attributes), the second is captured
-    if (m->graph_state == 0 && m->forwards >= 2) {
+    };
+    if (m->graph_state == 1)
+        return replay();
+    if (m->graph_state == -1)
+        return forward_eager(m);
+    // ---- undecided: the first six forwards
+    // (schedules of fewer than 5 kernels stay eager without asking: the depthwise + pooling + addition
+    //  chain as one kernel takes 7.6 us per forward eagerly, 16.2 us as a graph)
+    if (options().no_graph || m->schedule.size() < 5) {
         m->graph_state = -1;
-        // (a graph launch costs about 13 us before its first kernel starts, an eager launch 3-4 us
-        //  per kernel: schedules of fewer than 5 kernels stay eager - the depthwise + pooling +
-        //  addition chain as one kernel takes 7.6 us per forward eagerly, 16.2 us as a graph)
-        if (!options().no_graph && m->schedule.size() >= 5 &&
-            hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal) == hipSuccess) {
+        return forward_eager(m);
+    }
+    if (m->forwards == 1)
+        return forward_eager(m);
+    if (!m->ev0 && (hipEventCreate(&m->ev0) != hipSuccess || hipEventCreate(&m->ev1) != hipSuccess)) {
+        m->graph_state = -1;
+        return forward_eager(m);
+    }
+    // one forward between two events; keeps the shortest time seen
+    auto timed = [&](bool graph, float* best) -> TinyNNStatus {
+        (void)hipEventRecord(m->ev0, stream());
+        TinyNNStatus st = graph ? replay() : forward_eager(m);
+        (void)hipEventRecord(m->ev1, stream());
+        float ms = 0.f;
+        if (st == TinyNN_SUCCESS && hipEventSynchronize(m->ev1) == hipSuccess &&
+            hipEventElapsedTime(&ms, m->ev0, m->ev1) == hipSuccess && ms < *best)
+            *best = ms;
+        return st;
+    };
+    if (m->forwards <= 3)
+        return timed(false, &m->eager_ms);
+    if (m->forwards == 4) {
+        if (hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal) == hipSuccess) {
             TinyNNStatus st = forward_eager(m);
             hipGraph_t g = nullptr;
             hipError_t e = hipStreamEndCapture(stream(), &g);
             if (st == TinyNN_SUCCESS && e == hipSuccess && g &&
                 hipGraphInstantiate(&m->graph_exec, g, nullptr, nullptr, 0) == hipSuccess) {
                 m->graph = g;
-                m->graph_state = 1;
-                e = hipGraphLaunch(m->graph_exec, stream());
-                MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "model_forward: graph launch: %s",
-                           hipGetErrorString(e));
-                return TinyNN_SUCCESS;
+                return replay();
             }
             if (g)
                 (void)hipGraphDestroy(g);
@@ -653,8 +683,13 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
             if (st != TinyNN_SUCCESS)
                 return st;
         }
+        m->graph_state = -1;
+        return forward_eager(m);
     }
-    return forward_eager(m);
+    TinyNNStatus st = timed(true, &m->graph_ms);
+    if (m->forwards >= 6)
+        m->graph_state = m->graph_ms <= m->eager_ms ? 1 : -1;
+    return st;
 }
 
 int megcc_gfx950_model_nr_opr(void* model) {

@@ -78,8 +78,8 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
     constexpr int A_IT = BM / 16, B_IT = BN / 16;
     // LDS is double buffered: the global loads of step k+1 are in flight (in registers) while
     // step k is multiplied out of the other buffer; one barrier per step.
-    __shared__ float As[2][GBK][BM + GPAD];
-    __shared__ float Bs[2][GBK][BN + GPAD];
+    __shared__ __attribute__((aligned(16))) float As[2][GBK][BM + GPAD];
+    __shared__ __attribute__((aligned(16))) float Bs[2][GBK][BN + GPAD];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = BM == 128 ? wave >> 1 : 0, wn = BM == 128 ? wave & 1 : wave;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
@@ -99,6 +99,75 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
     const int k_begin = blockIdx.z * q.kchunk;
     const int k_end = min(q.K, k_begin + q.kchunk);
     float ra[A_IT], rb[B_IT];
+    // MatrixMul tiles that lie inside the matrices are staged with 16-byte loads along each
+    // operand's contiguous axis and no range checks: the checked element-wise loads below are some
+    // 350 instructions per stage, issued while the matrix cores have nothing queued.
+    constexpr bool VEC = !CONV;
+    bool vec_tile = false;
+    if (VEC)  // the strides of the non-contiguous axes: rows of 4n floats from a 16-byte base
+        vec_tile = m0 + BM <= q.M && n0 + BN <= q.N &&
+                   (((A_KFAST ? q.a_rs : q.a_cs) | (B_NFAST ? q.b_rs : q.b_cs)) & 3) == 0 &&
+                   (((uintptr_t)q.A | (uintptr_t)q.B) & 15) == 0;
+    // thread -> (row along the strided axis, first of 4 elements along the contiguous axis) of a
+    // tile of `fast` contiguous elements per row
+    auto vec_pos = [&](int fast, int it, int& slow_i, int& fast_i) {
+        slow_i = tid / (fast / 4) + it * (1024 / fast);
+        fast_i = (tid % (fast / 4)) * 4;
+    };
+    auto load_tiles_vec = [&](int k0) {
+#pragma unroll
+        for (int it = 0; it < A_IT / 4; ++it) {
+            int m, k;
+            if (A_KFAST)
+                vec_pos(GBK, it, m, k);
+            else
+                vec_pos(BM, it, k, m);
+            const float4 v =
+                    *(const float4*)(q.A + (size_t)(m0 + m) * q.a_rs + (size_t)(k0 + k) * q.a_cs);
+            ra[4 * it] = v.x, ra[4 * it + 1] = v.y, ra[4 * it + 2] = v.z, ra[4 * it + 3] = v.w;
+        }
+#pragma unroll
+        for (int it = 0; it < B_IT / 4; ++it) {
+            int k, n;
+            if (B_NFAST)
+                vec_pos(BN, it, k, n);
+            else
+                vec_pos(GBK, it, n, k);
+            const float4 v =
+                    *(const float4*)(q.B + (size_t)(k0 + k) * q.b_rs + (size_t)(n0 + n) * q.b_cs);
+            rb[4 * it] = v.x, rb[4 * it + 1] = v.y, rb[4 * it + 2] = v.z, rb[4 * it + 3] = v.w;
+        }
+    };
+    auto store_tiles_vec = [&](int buf) {
+#pragma unroll
+        for (int it = 0; it < A_IT / 4; ++it) {
+            int m, k;
+            if (A_KFAST) {
+                vec_pos(GBK, it, m, k);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    As[buf][k + j][m] = ra[4 * it + j];
+            } else {
+                vec_pos(BM, it, k, m);
+                *(float4*)&As[buf][k][m] =
+                        make_float4(ra[4 * it], ra[4 * it + 1], ra[4 * it + 2], ra[4 * it + 3]);
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < B_IT / 4; ++it) {
+            int k, n;
+            if (B_NFAST) {
+                vec_pos(BN, it, k, n);
+                *(float4*)&Bs[buf][k][n] =
+                        make_float4(rb[4 * it], rb[4 * it + 1], rb[4 * it + 2], rb[4 * it + 3]);
+            } else {
+                vec_pos(GBK, it, n, k);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    Bs[buf][k + j][n] = rb[4 * it + j];
+            }
+        }
+    };
     // implicit GEMM: with B_NFAST a thread stages the same output pixel in every K step, so its
     // image / row / column are worked out once
     const int cn = n0 + tid % BN;
@@ -129,6 +198,10 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
     };
     // stage A tile (BM x GBK) and B tile (GBK x BN): BM / 16 and BN / 16 elements per thread
     auto load_tiles = [&](int k0) {
+        if (VEC && vec_tile && k0 + GBK <= k_end) {
+            load_tiles_vec(k0);
+            return;
+        }
 #pragma unroll
         for (int it = 0; it < A_IT; ++it) {
             int m, k;
@@ -166,7 +239,11 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
             rb[it] = v;
         }
     };
-    auto store_tiles = [&](int buf) {
+    auto store_tiles = [&](int buf, int k0) {
+        if (VEC && vec_tile && k0 + GBK <= k_end) {
+            store_tiles_vec(buf);
+            return;
+        }
 #pragma unroll
         for (int it = 0; it < A_IT; ++it) {
             if (A_KFAST)
@@ -184,7 +261,7 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
     };
     if (k_begin < k_end) {
         load_tiles(k_begin);
-        store_tiles(0);
+        store_tiles(0, k_begin);
     }
     __syncthreads();
     int buf = 0;
@@ -220,7 +297,7 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
                     }
         }
         if (more)
-            store_tiles(buf ^ 1);
+            store_tiles(buf ^ 1, k0 + GBK);
         __syncthreads();
     }
     if (LONGK) {

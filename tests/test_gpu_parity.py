@@ -302,6 +302,16 @@ LIVE = [
     MatMulCase(33, 65, 70, trans_a=True),
     MatMulCase(33, 65, 70, trans_b=True),
     MatMulCase(33, 65, 70, trans_a=True, trans_b=True),
+    # whole tiles are staged with 16-byte loads, tiles at the edges and the last stage of K element
+    # by element: both in one product, every transposition; then the 64-row tile with split K
+    MatMulCase(192, 100, 320),
+    MatMulCase(192, 100, 320, trans_a=True),
+    MatMulCase(192, 100, 320, trans_b=True),
+    MatMulCase(192, 100, 320, trans_a=True, trans_b=True),
+    MatMulCase(64, 1024, 2048),
+    MatMulCase(64, 1024, 2048, trans_a=True),
+    MatMulCase(64, 1024, 2048, trans_b=True),
+    MatMulCase(64, 1024, 2048, trans_a=True, trans_b=True),
 ]
 
 

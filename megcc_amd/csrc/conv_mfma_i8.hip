@@ -512,6 +512,9 @@ static TinyNNStatus conv_mfma_pipe_launch(const PipeConfig& c, MfmaParams q) {
 int fc_stream_split(const ConvGeom& g, const void* src, size_t ws_bytes, int max_split);
 TinyNNStatus fc_stream_launch(
         const ConvGeom& g, const void* src, const void* packed, int32_t* partial, int split);
+bool fc_one_supported(const ConvGeom& g, const void* src);
+TinyNNStatus fc_one_launch(
+        const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst);
 bool fc_gevm_q8_supported(const ConvGeom& g);
 TinyNNStatus fc_gevm_q8_launch(
         const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst);
@@ -580,6 +583,15 @@ TinyNNStatus conv_mfma_launch(
     if (is_fc(g) && fc_gevm_q8_supported(g) && !options().no_gevm) {
         note_kernel("fc_gevm_q8");
         return fc_gevm_q8_launch(g, src, packed, bias, dst);
+    }
+    // FullyConnected with at most 64 rows: one launch, K slices meet inside the workgroup
+    // (fc_stream.hip). A long K under few output channels is a handful of workgroups with hundreds
+    // of KB each: that shape stays with the K slices in separate workgroups below, if it has the
+    // workspace for them.
+    const bool few_long = g.ic > 8192 && g.oc < 4096 && ws && ws->ptr;
+    if (is_fc(g) && fc_one_supported(g, src) && !few_long && !options().no_fcone && !options().no_fcs) {
+        note_kernel("fc_one", g.n <= 32 ? 1 : 2);
+        return fc_one_launch(g, src, packed, bias, dst);
     }
     MfmaParams q = {};
     PipeConfig pc;

@@ -149,4 +149,161 @@ TinyNNStatus fc_stream_launch(
     return check_launch("fc_stream");
 }
 
+// ---- one launch: the K slices of a 32-channel tile meet inside the workgroup ------------------
+// The split above costs a second launch and a round trip of the int32 partial sums through memory
+// (8 slices of 64 x 4096 sums are half the bytes of the weights themselves). Here a workgroup of 8
+// waves owns 32 output channels for the whole of K: wave w multiplies the 128-byte blocks
+// w, w + 8, ... of K, with every one of its filter chunks (up to 16 KB) requested before the first
+// is used, so a 64 x 4096 x 4096 layer is one memory round trip of 128 KB per workgroup; its
+// activations come from L2 (every workgroup reads the same rows), one block ahead. The eight accumulator sets meet in LDS, and the reference's
+// epilogue (bias, requantisation, activation: BareMetal/ConvKernel.cpp:327-344) runs once.
+struct FcOneParams {
+    const int8_t* src;
+    const int8_t* wp;  // packed filter, as above
+    const int32_t* bias;
+    int8_t* dst;  // [M][OC]
+    int M, K, OC, OCP, act;
+    float s_src, s_flt, s_dst;
+};
+
+static constexpr int FO_WAVES = 8, FO_RING = 16;
+
+template <int NT>
+__global__ void __launch_bounds__(64 * FO_WAVES) fc_one_kernel(FcOneParams q) {
+    __shared__ int32_t red[FO_WAVES][NT * 16][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, kg = lane >> 5;
+    const int oct = blockIdx.x, oc = oct * 32 + col;
+    // chunk j of this wave is chunk (j & 3) of its (j >> 2)-th 128-byte block of K
+    const int blocks = q.K >> 7;
+    const int nj = wave < blocks ? ((blocks - wave + FO_WAVES - 1) / FO_WAVES) * 4 : 0;
+    const size_t astep = (size_t)q.OCP * KROW;
+    const int8_t* arow = q.wp + ((size_t)(wave * 4) * q.OCP + oc) * KROW + (((kg ^ (oc >> 3)) & 1) << 4);
+    auto a_at = [&](int j) { return *(const v4i*)(arow + (size_t)((j >> 2) * (4 * FO_WAVES) + (j & 3)) * astep); };
+    // activations: the wave's 128-byte blocks of K, whole lines at a time (8 lanes per row), through
+    // a staging area of its own: rows of 128 bytes with their 16-byte pieces at piece ^ (row & 7),
+    // so that the B-operand reads of 8 consecutive rows hit different banks. The area is the wave's
+    // slot of `red`: it is free again when the wave's last product has been issued.
+    constexpr int AL = 4 * NT;  // loads per lane and block: rows 8 i + lane / 8
+    int8_t* stage = (int8_t*)&red[wave][0][0];
+    const int srow = lane >> 3, apc = lane & 7, nb = nj >> 2;
+    const int8_t* asrc = q.src + (size_t)srow * q.K + wave * 128 + apc * 16;
+    v4i areg[2][AL];  // two blocks ahead: a block is one L2 round trip
+    auto act_load = [&](int blk, auto par) {
+#pragma unroll
+        for (int i = 0; i < AL; ++i)
+            areg[decltype(par)::value][i] = i * 8 + srow < q.M
+                            ? *(const v4i*)(asrc + (size_t)(i * 8) * q.K + (size_t)blk * (128 * FO_WAVES))
+                            : v4i{0, 0, 0, 0};
+    };
+    auto act_store = [&](auto par) {
+#pragma unroll
+        for (int i = 0; i < AL; ++i)
+            *(v4i*)(stage + (i * 8 + srow) * 128 + ((apc ^ srow) << 4)) = areg[decltype(par)::value][i];
+    };
+    if (nb > 0)
+        act_load(0, std::integral_constant<int, 0>{});
+    if (nb > 1)
+        act_load(1, std::integral_constant<int, 1>{});
+    v4i ring[FO_RING];
+    static_for<FO_RING>([&](auto sc) {
+        constexpr int s = decltype(sc)::value;
+        ring[s] = s < nj ? a_at(s) : v4i{0, 0, 0, 0};
+    });
+    v16i acc[NT];
+#pragma unroll
+    for (int ni = 0; ni < NT; ++ni)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            acc[ni][e] = 0;
+    for (int j0 = 0; j0 < nj; j0 += FO_RING) {
+        static_for<FO_RING / 4>([&](auto bc) {
+            constexpr int bb = decltype(bc)::value;
+            const int blk = (j0 >> 2) + bb;
+            if (blk < nb) {
+                constexpr std::integral_constant<int, bb & 1> par{};
+                act_store(par);  // (LDS operations of one wave execute in order)
+                if (blk + 2 < nb)
+                    act_load(blk + 2, par);
+                static_for<4>([&](auto cc_) {
+                    constexpr int cc = decltype(cc_)::value, s = bb * 4 + cc;
+                    const int j = j0 + s;
+                    const v4i a = ring[s];
+                    if (j + FO_RING < nj)
+                        ring[s] = a_at(j + FO_RING);
+#pragma unroll
+                    for (int ni = 0; ni < NT; ++ni) {
+                        const int row = ni * 32 + col;
+                        const v4i b = *(const v4i*)(stage + row * 128 + (((cc * 2 + kg) ^ (row & 7)) << 4));
+                        acc[ni] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[ni], 0, 0, 0);
+                    }
+                });
+            }
+        });
+    }
+#pragma unroll
+    for (int ni = 0; ni < NT; ++ni)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            red[wave][ni * 16 + e][lane] = acc[ni][e];
+    __syncthreads();
+    // thread -> (row half ni, register quad e4, lane): registers 4 e4 .. 4 e4 + 3 of a lane are the
+    // channels 8 e4 + 4 kg .. + 3 of the tile for row ni * 32 + col
+    const int grp = tid >> 6;
+    if (grp >= NT * 4)
+        return;
+    const int ni = grp >> 2, e4 = grp & 3;
+    const int row = ni * 32 + col, ocb = oct * 32 + e4 * 8 + kg * 4;
+    if (row >= q.M || ocb >= q.OC)
+        return;
+    int r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < FO_WAVES; ++w)
+            sum += red[w][ni * 16 + e4 * 4 + e][lane];
+        const int b = (q.bias && ocb + e < q.OC) ? q.bias[ocb + e] : 0;
+        r[e] = requant_conv_rt(q.act, sum + b, q.s_src, q.s_flt, q.s_dst);
+    }
+    int8_t* o = q.dst + (size_t)row * q.OC + ocb;
+    if ((q.OC & 3) == 0) {
+        *(uint32_t*)o = pack4(r[0], r[1], r[2], r[3]);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (ocb + e < q.OC)
+                o[e] = (int8_t)r[e];
+    }
+}
+
+// M <= 64 rows, K a multiple of 128, 16-byte aligned activations
+bool fc_one_supported(const ConvGeom& g, const void* src) {
+    return g.n >= 1 && g.n <= 64 && g.ic >= 128 && (g.ic & 127) == 0 && ((uintptr_t)src & 15) == 0 &&
+           g.oc >= 1;
+}
+
+TinyNNStatus fc_one_launch(
+        const ConvGeom& g, const void* src, const void* packed, const void* bias, void* dst) {
+    FcOneParams q;
+    q.src = (const int8_t*)src;
+    q.wp = (const int8_t*)packed;
+    q.bias = (const int32_t*)bias;
+    q.dst = (int8_t*)dst;
+    q.M = g.n;
+    q.K = g.ic;
+    q.OC = g.oc;
+    q.OCP = (g.oc + OC_PAD - 1) / OC_PAD * OC_PAD;
+    q.act = g.act;
+    q.s_src = g.s_src;
+    q.s_flt = g.s_flt;
+    q.s_dst = g.s_dst;
+    const int oc_tiles = (g.oc + 31) / 32;
+    if (g.n <= 32)
+        hipLaunchKernelGGL(fc_one_kernel<1>, dim3(oc_tiles), dim3(64 * FO_WAVES), 0, stream(), q);
+    else
+        hipLaunchKernelGGL(fc_one_kernel<2>, dim3(oc_tiles), dim3(64 * FO_WAVES), 0, stream(), q);
+    return check_launch("fc_one");
+}
+
 }  // namespace mg

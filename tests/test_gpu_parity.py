@@ -101,6 +101,15 @@ LIVE = [
     ConvCase(A.FMT_NCHW, A.DENSE, 64, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(1024) / 2)),
     ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, 0.1)),
     ConvCase(A.FMT_NCHW, A.DENSE, 200, 512, 1, 1, 333, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(512) / 2)),
+    # at most 64 rows, K a multiple of 128: one launch, eight K slices per workgroup (one block of
+    # K: seven idle waves; 8192: the ring of filter chunks is refilled; rows short of 32 / 64;
+    # channel counts that are no multiple of 4 or 32; every activation; no bias)
+    ConvCase(A.FMT_NCHW, A.DENSE, 5, 128, 1, 1, 37, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(128) / 2)),
+    ConvCase(A.FMT_NCHW, A.DENSE, 33, 384, 1, 1, 290, 1, 1, 0, A.H_SWISH, scales=(0.01, 0.01, unsat(384) / 2)),
+    ConvCase(A.FMT_NCHW, A.DENSE, 32, 1152, 1, 1, 64, 1, 1, 0, A.SIGMOID, scales=(0.01, 0.01, unsat(1152) / 2)),
+    ConvCase(A.FMT_NCHW, A.DENSE, 61, 8192, 1, 1, 96, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(8192) / 2),
+             bias=False),
+    ConvCase(A.FMT_NCHW, A.DENSE, 17, 2048, 1, 1, 1001, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(2048) / 2)),
     # 3x3 layers with 64..127 output channels on the LDS-direct kernel (64-channel tiles, one of them ragged)
     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 64, 40, 40, 64, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(576))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 9, 32, 31, 29, 96, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(288))),
@@ -587,6 +596,9 @@ OLDER = [
     ("nogevm", ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY,
                               scales=(0.01, 0.01, unsat(1024) / 2))),
     ("nogevm", MatMulCase(3, 301, 79, trans_b=True)),
+    # FullyConnected with few rows as K slices in separate workgroups + the split-K reduction
+    ("nofcone", ConvCase(A.FMT_NCHW, A.DENSE, 40, 1024, 1, 1, 200, 1, 1, 0, A.RELU,
+                         scales=(0.01, 0.01, unsat(1024) / 2))),
     ("nof32small", ConvCase(A.FMT_NCHW, A.DENSE, 1, 32, 56, 56, 32, 3, 1, 1, A.RELU, dtype="f32")),
     ("nopwshare", ConvCase(A.FMT_NCHW44, A.DENSE, 70, 512, 14, 14, 512, 1, 1, 0, A.RELU,
                                  scales=(0.02, 0.01, unsat(512)))),

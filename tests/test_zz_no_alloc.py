@@ -16,10 +16,10 @@ A = abi
 SCRATCH = 32 << 20
 
 PAIRS = [
-    # FullyConnected with 64 rows: K split over ~1000 waves, 8 MiB of int32 partial sums, then a
-    # smaller one
+    # FullyConnected with 64 rows and a long K under few output channels: K slices in separate
+    # workgroups, 1 MiB of int32 partial sums; then a smaller one
     ("fc_stream",
-     ConvCase(A.FMT_NCHW, A.DENSE, 64, 4096, 1, 1, 4096, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(4096) / 2)),
+     ConvCase(A.FMT_NCHW, A.DENSE, 64, 16384, 1, 1, 256, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(16384) / 2)),
      ConvCase(A.FMT_NCHW, A.DENSE, 64, 1024, 1, 1, 1000, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(1024) / 2))),
     # split-K of the one-stage kernel (few pixels, long K)
     ("conv_mfma_i8",

@@ -590,7 +590,6 @@ TinyNNStatus conv_mfma_launch(
     // workspace for them.
     const bool few_long = g.ic > 8192 && g.oc < 4096 && ws && ws->ptr;
     if (is_fc(g) && fc_one_supported(g, src) && !few_long && !options().no_fcone && !options().no_fcs) {
-        note_kernel("fc_one", g.n <= 32 ? 1 : 2);
         return fc_one_launch(g, src, packed, bias, dst);
     }
     MfmaParams q = {};

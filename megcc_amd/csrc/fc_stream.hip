@@ -174,6 +174,7 @@ __global__ void __launch_bounds__(64 * FO_WAVES) fc_one_kernel(FcOneParams q) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, kg = lane >> 5;
     const int oct = blockIdx.x, oc = oct * 32 + col;
+    const int row0 = blockIdx.y * (32 * NT);  // first row of this workgroup
     // chunk j of this wave is chunk (j & 3) of its (j >> 2)-th 128-byte block of K
     const int blocks = q.K >> 7;
     const int nj = wave < blocks ? ((blocks - wave + FO_WAVES - 1) / FO_WAVES) * 4 : 0;
@@ -187,12 +188,12 @@ __global__ void __launch_bounds__(64 * FO_WAVES) fc_one_kernel(FcOneParams q) {
     constexpr int AL = 4 * NT;  // loads per lane and block: rows 8 i + lane / 8
     int8_t* stage = (int8_t*)&red[wave][0][0];
     const int srow = lane >> 3, apc = lane & 7, nb = nj >> 2;
-    const int8_t* asrc = q.src + (size_t)srow * q.K + wave * 128 + apc * 16;
+    const int8_t* asrc = q.src + (size_t)(row0 + srow) * q.K + wave * 128 + apc * 16;
     v4i areg[2][AL];  // two blocks ahead: a block is one L2 round trip
     auto act_load = [&](int blk, auto par) {
 #pragma unroll
         for (int i = 0; i < AL; ++i)
-            areg[decltype(par)::value][i] = i * 8 + srow < q.M
+            areg[decltype(par)::value][i] = row0 + i * 8 + srow < q.M
                             ? *(const v4i*)(asrc + (size_t)(i * 8) * q.K + (size_t)blk * (128 * FO_WAVES))
                             : v4i{0, 0, 0, 0};
     };
@@ -253,7 +254,7 @@ __global__ void __launch_bounds__(64 * FO_WAVES) fc_one_kernel(FcOneParams q) {
     if (grp >= NT * 4)
         return;
     const int ni = grp >> 2, e4 = grp & 3;
-    const int row = ni * 32 + col, ocb = oct * 32 + e4 * 8 + kg * 4;
+    const int row = row0 + ni * 32 + col, ocb = oct * 32 + e4 * 8 + kg * 4;
     if (row >= q.M || ocb >= q.OC)
         return;
     int r[4];
@@ -299,8 +300,14 @@ TinyNNStatus fc_one_launch(
     q.s_flt = g.s_flt;
     q.s_dst = g.s_dst;
     const int oc_tiles = (g.oc + 31) / 32;
-    if (g.n <= 32)
-        hipLaunchKernelGGL(fc_one_kernel<1>, dim3(oc_tiles), dim3(64 * FO_WAVES), 0, stream(), q);
+    // 33..64 rows: two workgroups of 32 rows per channel tile while that still is one workgroup per
+    // CU - what a CU pulls through its L2 port (its share of the weights + the activations of its
+    // rows) bounds the kernel: 64 x 4096 x 4096 8.1 -> 6.6 us. (With a multiple of 8 channel tiles the
+    // two are on the same XCD: the weights still leave HBM once.)
+    const bool rows32 = g.n <= 32 || oc_tiles * 2 <= num_cus();
+    note_kernel("fc_one", rows32 ? 32 : 64);
+    if (rows32)
+        hipLaunchKernelGGL(fc_one_kernel<1>, dim3(oc_tiles, (g.n + 31) / 32), dim3(64 * FO_WAVES), 0, stream(), q);
     else
         hipLaunchKernelGGL(fc_one_kernel<2>, dim3(oc_tiles), dim3(64 * FO_WAVES), 0, stream(), q);
     return check_launch("fc_one");

@@ -110,6 +110,8 @@ LIVE = [
     ConvCase(A.FMT_NCHW, A.DENSE, 61, 8192, 1, 1, 96, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(8192) / 2),
              bias=False),
     ConvCase(A.FMT_NCHW, A.DENSE, 17, 2048, 1, 1, 1001, 1, 1, 0, A.IDENTITY, scales=(0.01, 0.01, unsat(2048) / 2)),
+    # (more channel tiles than half the CUs: one workgroup of 64 rows per tile instead of two of 32)
+    ConvCase(A.FMT_NCHW, A.DENSE, 40, 256, 1, 1, 4200, 1, 1, 0, A.RELU, scales=(0.01, 0.01, unsat(256) / 2)),
     # 3x3 layers with 64..127 output channels on the LDS-direct kernel (64-channel tiles, one of them ragged)
     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 64, 40, 40, 64, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(576))),
     ConvCase(A.FMT_NCHW44, A.DENSE, 9, 32, 31, 29, 96, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(288))),

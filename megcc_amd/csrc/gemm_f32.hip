@@ -54,7 +54,8 @@ __device__ __forceinline__ float act_rt(int act, float x) {
 }
 
 // B(k, p) of the implicit GEMM: source pixel of output pixel p under filter tap k
-__device__ __forceinline__ float conv_b(const GemmArgs& q, int k, int p) {
+// (ok: the tap lies on the image; otherwise element 0 is read and the caller discards it)
+__device__ __forceinline__ float conv_b(const GemmArgs& q, int k, int p, bool& ok) {
     const ConvGeom& g = q.g;
     int taps = g.fh * g.fw;
     int ic = k / taps, t = k - ic * taps;
@@ -64,9 +65,8 @@ __device__ __forceinline__ float conv_b(const GemmArgs& q, int k, int p) {
     int oh = r / g.ow, ow = r - oh * g.ow;
     unsigned ih = (unsigned)(oh * g.sh + fh * g.dh - g.ph);
     unsigned iw = (unsigned)(ow * g.sw + fw * g.dw - g.pw);
-    if (ih >= (unsigned)g.ih || iw >= (unsigned)g.iw)
-        return 0.f;
-    return q.B[(((size_t)n * g.ic + ic) * g.ih + ih) * g.iw + iw];
+    ok = ih < (unsigned)g.ih && iw < (unsigned)g.iw;
+    return q.B[ok ? (((size_t)n * g.ic + ic) * g.ih + ih) * g.iw + iw : 0];
 }
 
 // A_KFAST: A(m,k) has k contiguous (row-major, not transposed) -> lanes walk k when staging.
@@ -186,16 +186,21 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
         c_inv_fw = 1.f / (float)g.fw;
     }
     // B(k, cn): the quotients are exact for k below 2^22 (k + 0.5 keeps them off the boundaries)
-    auto conv_b_col = [&](int k) __attribute__((always_inline)) -> float {
+    auto conv_b_col = [&](int k, bool& ok) __attribute__((always_inline)) -> float {
         const ConvGeom& g = q.g;
         const int taps = g.fh * g.fw;
         const int ic = (int)(((float)k + 0.5f) * c_inv_taps), t = k - ic * taps;
         const int fh = (int)(((float)t + 0.5f) * c_inv_fw), fw = t - fh * g.fw;
         const unsigned ih = (unsigned)(c_ih0 + fh * g.dh), iw = (unsigned)(c_iw0 + fw * g.dw);
-        if (ih >= (unsigned)g.ih || iw >= (unsigned)g.iw)
-            return 0.f;
-        return q.B[c_img + ((size_t)ic * g.ih + ih) * g.iw + iw];
+        ok = ih < (unsigned)g.ih && iw < (unsigned)g.iw;
+        return q.B[ok ? c_img + ((size_t)ic * g.ih + ih) * g.iw + iw : 0];
     };
+    // Loads that are out of range read element 0 instead, and the value is replaced by 0 when it is
+    // written to LDS (the range test is repeated there; a convolution keeps one bit per element of
+    // the stage in flight, tap_ok, for what the gather found). A load under a branch makes the
+    // compiler wait for every outstanding load at the join, and a select right after the load
+    // waits for that load: either turns the loads of a stage into as many round trips.
+    unsigned tap_bits = 0;
     // stage A tile (BM x GBK) and B tile (GBK x BN): BM / 16 and BN / 16 elements per thread
     auto load_tiles = [&](int k0) {
         if (VEC && vec_tile && k0 + GBK <= k_end) {
@@ -212,10 +217,8 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
                 m = tid % BM;
                 k = tid / BM + it * (256 / BM);
             }
-            float v = 0.f;
-            if (m0 + m < q.M && k0 + k < k_end)
-                v = q.A[(size_t)(m0 + m) * q.a_rs + (size_t)(k0 + k) * q.a_cs];
-            ra[it] = v;
+            const bool ok = m0 + m < q.M && k0 + k < k_end;
+            ra[it] = q.A[ok ? (size_t)(m0 + m) * q.a_rs + (size_t)(k0 + k) * q.a_cs : 0];
         }
 #pragma unroll
         for (int it = 0; it < B_IT; ++it) {
@@ -227,16 +230,16 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
                 k = tid & 15;
                 n = (tid >> 4) + it * 16;
             }
-            float v = 0.f;
-            if (n0 + n < q.N && k0 + k < k_end) {
-                if (CONV && B_NFAST)
-                    v = conv_b_col(k0 + k);
-                else if (CONV)
-                    v = conv_b(q, k0 + k, n0 + n);
-                else
-                    v = q.B[(size_t)(k0 + k) * q.b_rs + (size_t)(n0 + n) * q.b_cs];
-            }
-            rb[it] = v;
+            const bool ok = n0 + n < q.N && k0 + k < k_end;
+            bool tap_ok = true;
+            if (CONV && B_NFAST)
+                rb[it] = conv_b_col(min(k0 + k, k_end - 1), tap_ok);
+            else if (CONV)
+                rb[it] = conv_b(q, min(k0 + k, k_end - 1), min(n0 + n, q.N - 1), tap_ok);
+            else
+                rb[it] = q.B[ok ? (size_t)(k0 + k) * q.b_rs + (size_t)(n0 + n) * q.b_cs : 0];
+            if (CONV)
+                tap_bits = (tap_bits & ~(1u << it)) | ((unsigned)tap_ok << it);
         }
     };
     auto store_tiles = [&](int buf, int k0) {
@@ -246,17 +249,16 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
         }
 #pragma unroll
         for (int it = 0; it < A_IT; ++it) {
-            if (A_KFAST)
-                As[buf][tid & 15][(tid >> 4) + it * 16] = ra[it];
-            else
-                As[buf][tid / BM + it * (256 / BM)][tid % BM] = ra[it];
+            const int k = A_KFAST ? tid & 15 : tid / BM + it * (256 / BM);
+            const int m = A_KFAST ? (tid >> 4) + it * 16 : tid % BM;
+            As[buf][k][m] = m0 + m < q.M && k0 + k < k_end ? ra[it] : 0.f;
         }
 #pragma unroll
         for (int it = 0; it < B_IT; ++it) {
-            if (B_NFAST)
-                Bs[buf][tid / BN + it * (256 / BN)][tid % BN] = rb[it];
-            else
-                Bs[buf][tid & 15][(tid >> 4) + it * 16] = rb[it];
+            const int k = B_NFAST ? tid / BN + it * (256 / BN) : tid & 15;
+            const int n = B_NFAST ? tid % BN : (tid >> 4) + it * 16;
+            const bool ok = n0 + n < q.N && k0 + k < k_end && (!CONV || ((tap_bits >> it) & 1));
+            Bs[buf][k][n] = ok ? rb[it] : 0.f;
         }
     };
     if (k_begin < k_end) {
@@ -372,11 +374,16 @@ __global__ void __launch_bounds__(256) gemm_f32_reduce_kernel(GemmArgs q) {
 // Split factor for problems with too few 128 x 128 tiles to fill the chip (skinny M: GEVM,
 // batch-64 FullyConnected, the small f32 convolution). A pure function of the shape, so that the
 // _workspace entry point and the kernel agree.
-static int gemm_split(long M, long N, long K) {
-    const long tiles = ((M + GBM - 1) / GBM) * ((N + GBN - 1) / GBN);
+static int gemm_split(long M, long N, long K, bool conv) {
+    // (at most 64 rows: 64 x 256 tiles)
+    const long tiles = M <= 64 ? (N + 255) / 256 : ((M + GBM - 1) / GBM) * ((N + GBN - 1) / GBN);
     if (tiles >= 192 || K < 128)
         return 1;
-    long s = (512 + tiles - 1) / tiles;
+    // Every split writes M x N partial sums. A MatrixMul of few rows is best at one workgroup per
+    // CU (64 x 4096 x 4096: 37 us with 16 slices, 40 us with 32); the implicit GEMM spends more of a
+    // stage on its gather and gains from a second workgroup per CU that multiplies meanwhile
+    // (N=8, 64 -> 64, 56 x 56, 3x3: 74 us with 3 slices, 64 us with 6; 118 us unsplit).
+    long s = ((M <= 64 && !conv ? 256 : 512) + tiles - 1) / tiles;
     const long max_s = K / 64;
     if (s > max_s)
         s = max_s;
@@ -385,8 +392,8 @@ static int gemm_split(long M, long N, long K) {
     return s < 2 ? 1 : (int)s;
 }
 
-size_t gemm_f32_workspace_bytes(long M, long N, long K) {
-    const int s = gemm_split(M, N, K);
+size_t gemm_f32_workspace_bytes(long M, long N, long K, bool conv) {
+    const int s = gemm_split(M, N, K, conv);
     return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
 }
 
@@ -395,8 +402,8 @@ static void gemm_plan_split(GemmArgs& q, const Workspace* ws) {
     q.split = 1;
     q.kchunk = (q.K + GBK - 1) / GBK * GBK;
     q.partial = nullptr;
-    const int s = gemm_split(q.M, q.N, q.K);
-    if (s > 1 && ws && ws->ptr && ws->size >= gemm_f32_workspace_bytes(q.M, q.N, q.K) &&
+    const int s = gemm_split(q.M, q.N, q.K, q.is_conv != 0);
+    if (s > 1 && ws && ws->ptr && ws->size >= gemm_f32_workspace_bytes(q.M, q.N, q.K, q.is_conv != 0) &&
         ((uintptr_t)ws->ptr & 3) == 0) {
         q.split = s;
         q.kchunk = ((q.K + s - 1) / s + GBK - 1) / GBK * GBK;
@@ -419,7 +426,7 @@ bool conv_f32_gemm_supported(const ConvGeom& g) {
 }
 
 size_t conv_f32_gemm_workspace_bytes(const ConvGeom& g) {
-    return gemm_f32_workspace_bytes(g.oc, (long)g.n * g.oh * g.ow, (long)g.ic * g.fh * g.fw);
+    return gemm_f32_workspace_bytes(g.oc, (long)g.n * g.oh * g.ow, (long)g.ic * g.fh * g.fw, true);
 }
 
 TinyNNStatus conv_f32_gemm_launch(
@@ -568,6 +575,6 @@ extern "C" TinyNNStatus megcc_gfx950_matmul_workspace(
     const long M = ta ? a->layout.dims[1] : a->layout.dims[0];
     const long K = ta ? a->layout.dims[0] : a->layout.dims[1];
     const long N = tb ? b->layout.dims[0] : b->layout.dims[1];
-    *workspace = gemm_f32_workspace_bytes(M, N, K);
+    *workspace = gemm_f32_workspace_bytes(M, N, K, false);
     return TinyNN_SUCCESS;
 }

@@ -81,18 +81,20 @@ std::string KernelFuncBase::GetWorkspaceBody(TContext* c) const {
 
 namespace {
 
-static const char* kSplitBody =
-        "    /* room for the split-K partial sums of problems with too few 128 x 128 tiles to fill\n"
-        "       the chip; the same formula as the library (gemm_f32.hip, gemm_split) */\n"
-        "    long tiles = ((M + 127) / 128) * ((N + 127) / 128), s = 1;\n"
+static std::string split_body(bool conv) {
+    return std::string(
+        "    /* room for the split-K partial sums of problems with too few 128 x 128 tiles (64 x 256\n"
+        "       for at most 64 rows) to fill the chip; the same formula as the library (gemm_f32.hip, gemm_split) */\n"
+        "    long tiles = M <= 64 ? (N + 255) / 256 : ((M + 127) / 128) * ((N + 127) / 128), s = 1;\n"
         "    if (tiles < 192 && K >= 128) {\n"
-        "        s = (512 + tiles - 1) / tiles;\n"
+        "        s = (") + (conv ? "512" : "(M <= 64 ? 256 : 512)") + std::string(" + tiles - 1) / tiles;\n"
         "        if (s > K / 64) s = K / 64;\n"
         "        if (s > 64) s = 64;\n"
         "        if (s < 2) s = 1;\n"
         "    }\n"
         "    *workspace = s > 1 ? (size_t)s * M * N * 4 : 0;\n"
-        "    return TinyNN_SUCCESS;\n}\n";
+        "    return TinyNN_SUCCESS;\n}\n");
+}
 
 
 // ---- dtype helpers (Utils/Utils.h:41-140, Utils/SymbolHelper.h:9-23) ---------------------------
@@ -267,7 +269,7 @@ struct ConvKernel : KernelFuncBase {
                << " + 1 : 0, ow = iw >= ew ? (iw - ew) / " << c->getAttrUInt("stride_w") << " + 1 : 0;\n"
                << "    const long ic = (long)src.dims[1] * 4, oc = (long)flt.dims[0] * 4;\n"
                << "    const long M = oc, N = (long)src.dims[0] * oh * ow, K = ic * " << taps << ";\n"
-               << "    long tiles = ((M + 127) / 128) * ((N + 127) / 128), s = 1;\n"
+               << "    long tiles = M <= 64 ? (N + 255) / 256 : ((M + 127) / 128) * ((N + 127) / 128), s = 1;\n"
                << "    if (tiles < 192 && K >= 128) {\n"
                << "        s = (512 + tiles - 1) / tiles;\n"
                << "        if (s > K / 64) s = K / 64;\n"
@@ -300,7 +302,7 @@ struct ConvKernel : KernelFuncBase {
         if (f32) {
             ss << "    const long M = flt.dims[0], N = (long)src.dims[0] * oh * ow, K = (long)src.dims[1] * "
                << c->getAttrUInt("kernel_h") << " * " << c->getAttrUInt("kernel_w") << ";\n"
-               << kSplitBody;
+               << split_body(true);
             return ss.str();
         }
         // qsi8 dense / FullyConnected: split-K partial sums of the one-stage MFMA kernel
@@ -718,7 +720,7 @@ struct MatrixMulKernel : KernelFuncBase {
            << "    const Layout a = inputs[0]->layout, b = inputs[1]->layout;\n"
            << "    const long M = a.dims[" << (ta ? 1 : 0) << "], K = a.dims[" << (ta ? 0 : 1)
            << "], N = b.dims[" << (tb ? 0 : 1) << "];\n"
-           << kSplitBody;
+           << split_body(false);
         return ss.str();
     }
 };

@@ -278,6 +278,102 @@ __global__ void __launch_bounds__(64 * FO_WAVES) fc_one_kernel(FcOneParams q) {
     }
 }
 
+// The same workgroup for K <= 4096 (at most NB = 4 blocks of K per wave) and 32 rows: every global
+// load of the wave - its activations and its filter chunks - is issued at the top, without a
+// condition. A load that is issued under a condition (a prefetch inside `if (block + 2 < blocks)`,
+// a row test around the load) leaves the compiler unable to count how many loads are outstanding
+// behind an earlier one, and it then waits for ALL of them before the first use: each prefetch
+// became a round trip of its own. Here a wave with fewer blocks than NB, or none, fetches a block it
+// has a right to read again and multiplies it with zeros; rows beyond M read row M - 1 and are
+// zeroed on their way into LDS.
+template <int NB>
+__global__ void __launch_bounds__(64 * FO_WAVES) fc_one32_kernel(FcOneParams q) {
+    __shared__ int32_t red[FO_WAVES][16][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, kg = lane >> 5;
+    const int oct = blockIdx.x, oc = oct * 32 + col;
+    const int row0 = blockIdx.y * 32;
+    const int blocks = q.K >> 7;
+    const int myb = wave < blocks ? (blocks - wave + FO_WAVES - 1) / FO_WAVES : 0;  // <= NB
+    const int wv = myb ? wave : 0;
+    const size_t astep = (size_t)q.OCP * KROW;
+    const int8_t* arow = q.wp + ((size_t)(wv * 4) * q.OCP + oc) * KROW + (((kg ^ (oc >> 3)) & 1) << 4);
+    int8_t* stage = (int8_t*)&red[wave][0][0];  // 4 KB: 32 rows of 128 bytes, pieces at piece ^ (row & 7)
+    const int srow = lane >> 3, apc = lane & 7;
+    v4i areg[NB][4], ring[NB * 4];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const int bc = b < myb ? b : 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = min(row0 + i * 8 + srow, q.M - 1);
+            areg[b][i] = *(const v4i*)(q.src + (size_t)row * q.K + (wv + FO_WAVES * bc) * 128 + apc * 16);
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const int bc = b < myb ? b : 0;
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc)
+            ring[b * 4 + cc] = *(const v4i*)(arow + (size_t)(bc * (4 * FO_WAVES) + cc) * astep);
+    }
+    // (the scheduler otherwise moves each load down to a few instructions before its use)
+    __builtin_amdgcn_sched_barrier(0);
+    v16i acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+        acc[e] = 0;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool ok = row0 + i * 8 + srow < q.M && b < myb;
+            v4i v = areg[b][i];
+            v.x = ok ? v.x : 0, v.y = ok ? v.y : 0, v.z = ok ? v.z : 0, v.w = ok ? v.w : 0;
+            *(v4i*)(stage + (i * 8 + srow) * 128 + ((apc ^ srow) << 4)) = v;  // (a wave's LDS operations execute in order)
+        }
+        // (no `if (b < myb)` here: the compiler would sink the block's filter loads into it, next to
+        //  their use, one round trip each; a block the wave does not own multiplies zeros)
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) {
+            const v4i bo = *(const v4i*)(stage + col * 128 + (((cc * 2 + kg) ^ (col & 7)) << 4));
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[b * 4 + cc], bo, acc, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+        red[wave][e][lane] = acc[e];
+    __syncthreads();
+    const int e4 = tid >> 6;
+    if (e4 >= 4)
+        return;
+    const int row = row0 + col, ocb = oct * 32 + e4 * 8 + kg * 4;
+    if (row >= q.M || ocb >= q.OC)
+        return;
+    int bias[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        bias[e] = q.bias ? q.bias[min(ocb + e, q.OC - 1)] : 0;
+    int r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < FO_WAVES; ++w)
+            sum += red[w][e4 * 4 + e][lane];
+        r[e] = requant_conv_rt(q.act, sum + bias[e], q.s_src, q.s_flt, q.s_dst);
+    }
+    int8_t* o = q.dst + (size_t)row * q.OC + ocb;
+    if ((q.OC & 3) == 0) {
+        *(uint32_t*)o = pack4(r[0], r[1], r[2], r[3]);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (ocb + e < q.OC)
+                o[e] = (int8_t)r[e];
+    }
+}
+
 // M <= 64 rows, K a multiple of 128, 16-byte aligned activations
 bool fc_one_supported(const ConvGeom& g, const void* src) {
     return g.n >= 1 && g.n <= 64 && g.ic >= 128 && (g.ic & 127) == 0 && ((uintptr_t)src & 15) == 0 &&
@@ -305,8 +401,16 @@ TinyNNStatus fc_one_launch(
     // rows) bounds the kernel: 64 x 4096 x 4096 8.1 -> 6.6 us. (With a multiple of 8 channel tiles the
     // two are on the same XCD: the weights still leave HBM once.)
     const bool rows32 = g.n <= 32 || oc_tiles * 2 <= num_cus();
-    note_kernel("fc_one", rows32 ? 32 : 64);
-    if (rows32)
+    const int nb = rows32 && g.ic <= 4096 ? (g.ic / 128 + FO_WAVES - 1) / FO_WAVES : 0;  // blocks per wave
+    note_kernel("fc_one", rows32 ? 32 : 64, nb);
+    const dim3 grid32(oc_tiles, (g.n + 31) / 32), block(64 * FO_WAVES);
+    if (nb == 1)
+        hipLaunchKernelGGL(fc_one32_kernel<1>, grid32, block, 0, stream(), q);
+    else if (nb == 2)
+        hipLaunchKernelGGL(fc_one32_kernel<2>, grid32, block, 0, stream(), q);
+    else if (nb >= 3)
+        hipLaunchKernelGGL(fc_one32_kernel<4>, grid32, block, 0, stream(), q);
+    else if (rows32)
         hipLaunchKernelGGL(fc_one_kernel<1>, dim3(oc_tiles, (g.n + 31) / 32), dim3(64 * FO_WAVES), 0, stream(), q);
     else
         hipLaunchKernelGGL(fc_one_kernel<2>, dim3(oc_tiles), dim3(64 * FO_WAVES), 0, stream(), q);

@@ -117,7 +117,7 @@ def test_cfg3_fc_q8_1x1024x1000(scale_name, dst_scale):
 
 @pytest.mark.parametrize("scale_name,dst_scale", FC_SCALES, ids=[s for s, _ in FC_SCALES])
 def test_cfg3_fc_q8_64x4096x4096(scale_name, dst_scale):
-    assert fc_rows(64, 4096, 4096, scale_name, dst_scale, list(range(64))) == "fc_one:32"
+    assert fc_rows(64, 4096, 4096, scale_name, dst_scale, list(range(64))) == "fc_one:32,4"
 
 
 @pytest.mark.parametrize("scale_name,dst_scale", FC_SCALES, ids=[s for s, _ in FC_SCALES])

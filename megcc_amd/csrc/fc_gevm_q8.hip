@@ -22,7 +22,7 @@ struct FcGevmArgs {
     float s_src, s_flt, s_dst;
 };
 
-static constexpr int FG_SLICES = 16;
+static constexpr int FG_SLICES = 16, FG_PRE = 2;
 
 template <int M>
 __global__ void __launch_bounds__(64 * FG_SLICES) fc_gevm_q8_kernel(FcGevmArgs q) {
@@ -31,22 +31,58 @@ __global__ void __launch_bounds__(64 * FG_SLICES) fc_gevm_q8_kernel(FcGevmArgs q
     const int kpad = q.nchunks * 32;
     int8_t* const act = (int8_t*)fg_lds;                 // [M][kpad], zero beyond K
     int* const red = fg_lds + (M * kpad) / 4;            // [slice][M][64]
-    for (int i = tid; i < M * kpad; i += 64 * FG_SLICES) {
+    // The first 1024 bytes of the activations, then the filter rows: all loads of the common case
+    // (M * K <= 1024) are unconditional and go out together.
+    const int first_m = tid / kpad, first_k = tid - first_m * kpad;
+    const bool first_ok = tid < M * kpad && first_k < q.K;
+    const int8_t first = q.src[first_ok ? (size_t)first_m * q.K + first_k : 0];
+    // The filter rows of the slice's first FG_PRE chunks are requested before the activations are
+    // staged: they do not depend on LDS, and behind the barrier they would be a second memory
+    // round trip of a kernel that is little more than one. (Unconditional loads: a chunk beyond the
+    // end reads the last chunk again and is not used.)
+    const int oc = blockIdx.x * 64 + lane;  // < OCP: rows beyond OC are zero in the packed filter
+    const int sw = ((oc >> 3) & 1) << 4;
+    const int8_t* row = q.wp + (size_t)oc * KROW;
+    const size_t cstep = (size_t)q.OCP * KROW;
+    v4i pre[FG_PRE][2];
+#pragma unroll
+    for (int i = 0; i < FG_PRE; ++i) {
+        const int8_t* r = row + (size_t)min(sl + i * FG_SLICES, q.nchunks - 1) * cstep;
+        pre[i][0] = *(const v4i*)(r + sw);
+        pre[i][1] = *(const v4i*)(r + (sw ^ 16));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // (every thread stores, the surplus ones into a byte of `red` that is written again later: a
+    //  store under a condition would take its load with it, behind the filter rows)
+    *(tid < M * kpad ? act + tid : (int8_t*)red) = first_ok ? first : (int8_t)0;
+    for (int i = tid + 64 * FG_SLICES; i < M * kpad; i += 64 * FG_SLICES) {
         const int m = i / kpad, k = i - m * kpad;
         act[i] = k < q.K ? q.src[(size_t)m * q.K + k] : (int8_t)0;
     }
     __syncthreads();
 
-    const int oc = blockIdx.x * 64 + lane;  // < OCP: rows beyond OC are zero in the packed filter
-    const int sw = ((oc >> 3) & 1) << 4;
-    const int8_t* row = q.wp + (size_t)oc * KROW;
-    const size_t cstep = (size_t)q.OCP * KROW;
     int acc[M];
 #pragma unroll
     for (int m = 0; m < M; ++m)
         acc[m] = 0;
+#pragma unroll
+    for (int i = 0; i < FG_PRE; ++i) {
+        const int c = sl + i * FG_SLICES;
+        if (c < q.nchunks) {
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const v4i a0 = *(const v4i*)(act + m * kpad + c * 32);
+                const v4i a1 = *(const v4i*)(act + m * kpad + c * 32 + 16);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[m] = __builtin_amdgcn_sdot4(pre[i][0][j], a0[j], acc[m], false);
+                    acc[m] = __builtin_amdgcn_sdot4(pre[i][1][j], a1[j], acc[m], false);
+                }
+            }
+        }
+    }
 #pragma unroll 4
-    for (int c = sl; c < q.nchunks; c += FG_SLICES) {
+    for (int c = sl + FG_PRE * FG_SLICES; c < q.nchunks; c += FG_SLICES) {
         const int8_t* r = row + (size_t)c * cstep;
         const v4i w0 = *(const v4i*)(r + sw), w1 = *(const v4i*)(r + (sw ^ 16));
 #pragma unroll

@@ -33,38 +33,34 @@ __global__ void __launch_bounds__(256) gevm_f32_cols_kernel(GevmArgs q) {
             acc[m][j] = 0.f;
     if (n0 < q.N) {
         for (int k0 = kg; k0 < q.K; k0 += 64 * GV_UNROLL) {
-            float b[GV_UNROLL][4];
+            // No load stands under a condition (the compiler would wait for every outstanding
+            // load at each join, one round trip per row): rows beyond K read row K - 1, columns
+            // beyond N column N - 1, and their products are replaced by 0.
+            float b[GV_UNROLL][4], a[GV_UNROLL][M];
 #pragma unroll
             for (int u = 0; u < GV_UNROLL; ++u) {
-                const int k = k0 + u * 64;
+                const int k = min(k0 + u * 64, q.K - 1);
                 const float* p = q.B + (size_t)k * q.b_rs + n0;
-                if (k < q.K) {
-                    if (VEC) {
-                        const float4 v = *(const float4*)p;
-                        b[u][0] = v.x; b[u][1] = v.y; b[u][2] = v.z; b[u][3] = v.w;
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            b[u][j] = n0 + j < q.N ? p[j] : 0.f;
-                    }
+                if (VEC) {
+                    const float4 v = *(const float4*)p;
+                    b[u][0] = v.x; b[u][1] = v.y; b[u][2] = v.z; b[u][3] = v.w;
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        b[u][j] = 0.f;
+                        b[u][j] = p[min(j, q.N - 1 - n0)];
                 }
+#pragma unroll
+                for (int m = 0; m < M; ++m)
+                    a[u][m] = q.A[(size_t)m * q.a_rs + (size_t)k * q.a_cs];
             }
 #pragma unroll
             for (int u = 0; u < GV_UNROLL; ++u) {
-                const int k = k0 + u * 64;
-                if (k < q.K) {
+                const bool ok = k0 + u * 64 < q.K;
 #pragma unroll
-                    for (int m = 0; m < M; ++m) {
-                        const float a = q.A[(size_t)m * q.a_rs + (size_t)k * q.a_cs];
+                for (int m = 0; m < M; ++m)
 #pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            acc[m][j] += a * b[u][j];
-                    }
-                }
+                    for (int j = 0; j < 4; ++j)
+                        acc[m][j] += ok ? a[u][m] * b[u][j] : 0.f;
             }
         }
     }
@@ -101,39 +97,40 @@ __global__ void __launch_bounds__(256) gevm_f32_rows_kernel(GevmArgs q) {
         for (int r = 0; r < 4; ++r)
             acc[m][r] = 0.f;
     for (int k0 = lane * 4; k0 < q.K; k0 += 256 * 2) {
-        float b[2][4][4];
+        // (no load under a condition, as above: rows beyond N read row N - 1, elements beyond K
+        //  element K - 1, and their products are replaced by 0)
+        float b[2][4][4], a[2][M][4];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int k = k0 + u * 256;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float* p = q.B + (size_t)(n0 + r) * q.b_cs + k;
-                const bool row = n0 + r < q.N;
-                if (VEC && row && k < q.K) {  // K % 4 == 0: the piece is whole
-                    const float4 v = *(const float4*)p;
+                const float* row = q.B + (size_t)min(n0 + r, q.N - 1) * q.b_cs;
+                if (VEC) {  // K % 4 == 0: a piece is whole or beyond K
+                    const float4 v = *(const float4*)(row + min(k, q.K - 4));
                     b[u][r][0] = v.x; b[u][r][1] = v.y; b[u][r][2] = v.z; b[u][r][3] = v.w;
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        b[u][r][j] = !VEC && row && k + j < q.K ? p[j] : 0.f;
+                        b[u][r][j] = row[min(k + j, q.K - 1)];
                 }
             }
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    a[u][m][j] = q.A[(size_t)m * q.a_rs + (size_t)min(k + j, q.K - 1) * q.a_cs];
         }
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int k = k0 + u * 256;
 #pragma unroll
-            for (int m = 0; m < M; ++m) {
-                float a[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    a[j] = k + j < q.K ? q.A[(size_t)m * q.a_rs + (size_t)(k + j) * q.a_cs] : 0.f;
+            for (int m = 0; m < M; ++m)
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        acc[m][r] += a[j] * b[u][r][j];
-            }
+                        acc[m][r] += k + j < q.K ? a[u][m][j] * b[u][r][j] : 0.f;
         }
     }
 #pragma unroll

@@ -313,6 +313,12 @@ LIVE = [
     MatMulCase(33, 65, 70, trans_a=True),
     MatMulCase(33, 65, 70, trans_b=True),
     MatMulCase(33, 65, 70, trans_a=True, trans_b=True),
+    # at most 4 rows (the one-pass kernels): B as it lies and transposed, sizes that allow 16-byte
+    # loads and sizes that do not, K short of a whole step
+    MatMulCase(2, 130, 45),
+    MatMulCase(3, 301, 79, trans_b=True),
+    MatMulCase(4, 1024, 1000, trans_b=True),
+    MatMulCase(4, 100, 64),
     # whole tiles are staged with 16-byte loads, tiles at the edges and the last stage of K element
     # by element: both in one product, every transposition; then the 64-row tile with split K
     MatMulCase(192, 100, 320),

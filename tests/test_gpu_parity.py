@@ -793,6 +793,47 @@ def test_pointwise_depthwise_and_row_split_sweep(case):
     compare(got, case.run_port(arrays), repr(case))
 
 
+def _fully_connected_sweep():
+    """seeded random FullyConnected layers of at most 64 rows (K a multiple of 128: 1..4 blocks of K
+    per wave, more than 4096, long K under few channels) and f32 products of at most 4 rows with B
+    as it lies and transposed"""
+    r = np.random.Generator(np.random.PCG64(77))
+    acts = [A.IDENTITY, A.RELU, A.H_SWISH, A.SIGMOID]
+    out = []
+    for i in range(18):
+        m, k, oc = int(r.integers(1, 65)), int(r.integers(1, 33)) * 128, int(r.integers(1, 500))
+        if i % 6 == 0:
+            k, oc = int(r.choice([8192, 12288])), int(r.integers(1, 160))
+        act = acts[int(r.integers(0, 4))]
+        sc = unsat(k) / 2 * (40 if act == A.SIGMOID else 1)
+        out.append(ConvCase(A.FMT_NCHW, A.DENSE, m, k, 1, 1, oc, 1, 1, 0, act, scales=(0.01, 0.01, sc),
+                            bias=bool(r.integers(0, 2))))
+    for _ in range(8):
+        out.append(MatMulCase(int(r.integers(1, 5)), int(r.integers(1, 1500)), int(r.integers(1, 1200)),
+                              trans_b=bool(r.integers(0, 2))))
+    return out
+
+
+FC_SWEEP = _fully_connected_sweep()
+
+
+@pytest.mark.parametrize("case", FC_SWEEP, ids=[repr(c) for c in FC_SWEEP])
+def test_fully_connected_sweep(case):
+    port.set_threads(8)
+    arrays = case.gen(seed=31)
+    got = run_gpu(case, arrays)
+    kernel = runtime.last_kernel()
+    if isinstance(case, MatMulCase):
+        assert kernel == "gevm_f32", kernel
+    elif case.n <= 4:
+        assert kernel == "fc_gevm_q8", kernel
+    elif case.ic > 8192:
+        assert kernel.startswith("fc_stream"), kernel
+    else:
+        assert kernel.startswith("fc_one"), kernel
+    compare(got, case.run_port(arrays), repr(case))
+
+
 def test_direct_kernel_when_filter_was_not_packed():
     """a caller that skips the init protocol still gets the right answer (generic kernel)"""
     import ctypes as C

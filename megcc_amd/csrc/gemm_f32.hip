@@ -170,7 +170,9 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
     };
     // implicit GEMM: with B_NFAST a thread stages the same output pixel in every K step, so its
     // image / row / column are worked out once
-    const int cn = n0 + tid % BN;
+    // (a column beyond N takes the last column's pixel: its loads are issued like all others,
+    //  unconditionally, and must stay inside the tensor; its values are never stored)
+    const int cn = min(n0 + tid % BN, q.N - 1);
     long c_img = 0;
     int c_ih0 = 0, c_iw0 = 0;
     float c_inv_taps = 0.f, c_inv_fw = 0.f;

@@ -307,6 +307,10 @@ LIVE = [
     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 16, 14, 12, 128, 1, 1, 0, A.IDENTITY, dtype="f32", bias=False),
     ConvCase(A.FMT_NCHW44, A.DENSE, 1, 256, 7, 7, 32, 3, 1, 1, A.SIGMOID, dtype="f32"),
     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 8, 12, 10, 8, 5, 1, 2, A.RELU, dtype="f32", dilate=1),
+    # the last tile of output pixels is ragged (1584 = 12 x 128 + 48): its surplus columns must
+    # gather inside the tensor; padding wider than half the filter, no bias, split K
+    ConvCase(A.FMT_NCHW, A.DENSE, 3, 86, 45, 42, 117, 5, 2, 3, A.SIGMOID, dtype="f32", bias=False),
+    ConvCase(A.FMT_NCHW, A.DENSE, 1, 40, 9, 11, 30, 3, 1, 1, A.RELU, dtype="f32", dilate=2),
     MatMulCase(1, 1024, 1000),
     MatMulCase(64, 512, 384),
     MatMulCase(130, 77, 259),

@@ -50,17 +50,47 @@ TRAFFIC_FILES = ["profiles/conv_mfma_i8_dma__conv3x3_n32_c256_56x56.txt",
 
 
 def measured_traffic(workload):
-    """(bytes per launch, file it was read from) or (None, None)"""
-    key = "TRAFFIC_BYTES_PER_LAUNCH[%s]=" % workload
+    """(bytes read per launch, bytes written per launch, file) from the committed counter summaries,
+    or (None, None, None). A summary holds "TRAFFIC_READ_BYTES_PER_LAUNCH[<workload>]=<n>" and
+    "TRAFFIC_WRITE_BYTES_PER_LAUNCH[<workload>]=<n>" (older ones one line with the sum:
+    "TRAFFIC_BYTES_PER_LAUNCH[...]", returned as reads with writes unknown)."""
+    keys = ["TRAFFIC_%sBYTES_PER_LAUNCH[%s]=" % (k, workload) for k in ("READ_", "WRITE_", "")]
     for rel in TRAFFIC_FILES:
+        found = {}
         try:
             with open(os.path.join(ROOT, rel)) as f:
                 for line in f:
-                    if line.startswith(key):
-                        return int(line.split("=", 1)[1]), rel
+                    for k in keys:
+                        if line.startswith(k):
+                            found[k] = int(line.split("=", 1)[1])
         except OSError:
-            pass
-    return None, None
+            continue
+        if keys[0] in found:
+            return found[keys[0]], found.get(keys[1]), rel
+        if keys[2] in found:
+            return found[keys[2]], None, rel
+    return None, None, None
+
+
+def traffic_fields(workload, algorithmic_bytes, output_bytes):
+    """roofline.traffic and what it is made of. WRITE_SIZE reads (close to) nothing for some kernels
+    that do write - their dirty lines are still in L2 when the dispatch ends and leave it during the
+    next one - so where the counter shows less than half of the bytes the kernel must write, the
+    output bytes are counted instead and the line says so."""
+    rd, wr, rel = measured_traffic(workload)
+    if rd is None:
+        return {"traffic": None}
+    out = {"traffic_source": rel, "traffic_read": rd}
+    if wr is None:
+        out.update(traffic=rd, traffic_note="reads and writes as summed in the summary")
+    elif wr < 0.5 * output_bytes:
+        out.update(traffic=rd + output_bytes, traffic_write=output_bytes,
+                   traffic_note="WRITE_SIZE showed %d bytes for a kernel that writes %d (dirty lines still in L2 "
+                                "at dispatch end): the output bytes are counted instead" % (wr, output_bytes))
+    else:
+        out.update(traffic=rd + wr, traffic_write=wr)
+    out["traffic_over_algorithmic"] = round(out["traffic"] / algorithmic_bytes, 3)
+    return out
 
 
 class HipEvents:
@@ -189,9 +219,9 @@ def make_workload(name):
         ic, oc = (24, 144) if name == "pw_24_144" else (144, 24)
         case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 64, ic, 56, 56, oc, 1, 1, 0, abi.RELU, scales=(0.02, 0.01, 0.05))
         return case, "qsi8 conv1x1 NCHW44 N=64 %d->%d 56x56" % (ic, oc), "hbm"
-    if name.startswith("dw"):
-        c, hw, s = {"dw": (32, 112, 1), "dw_s2": (32, 112, 2), "dw512": (512, 14, 1),
-                    "dw512_s2": (512, 14, 2)}[name]
+    if name.startswith("dw"):  # dw:C,HW,S - any shape of the depthwise layer of configs[3]
+        c, hw, s = [int(v) for v in name[3:].split(",")] if name.startswith("dw:") else {
+            "dw": (32, 112, 1), "dw_s2": (32, 112, 2), "dw512": (512, 14, 1), "dw512_s2": (512, 14, 2)}[name]
         case = ConvCase(abi.FMT_NCHW44, abi.GROUP, 64, c, hw, hw, c, 3, s, 1, abi.RELU,
                         scales=(0.02, 0.01, 0.05))
         return case, "qsi8 depthwise 3x3 s%d NCHW44 N=64 C=%d %dx%d" % (s, c, hw, hw), "hbm"
@@ -254,6 +284,15 @@ def bench_mobilenet(batch, steps, warmup, per_layer=False):
            "ms_per_forward": round(wall * 1e3 / steps, 4), "device_ms_per_forward": round(dev_ms, 4),
            "arena_bytes": model.arena_bytes, "nr_opr": model.nr_opr,
            "int8_tops": round(2 * mobilenet.macs_per_image() * batch / (dev_ms * 1e-3) / 1e12, 2)}
+    # the network is bandwidth-bound at these batches (1.14 GOP against 11 MB of activations and
+    # weights per image): priced against HBM on the bytes its operators read and write once each
+    moved = mobilenet.algorithmic_bytes(batch)
+    out["nr_kernel"] = model.nr_kernel
+    out["launch_mode"] = {1: "graph", -1: "eager", 0: "undecided"}[model.launch_mode()[0]]
+    out["roofline"] = {"bound": "hbm", "achieved": round(moved / (dev_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                       "unit": "GB/s", "frac": round(moved / (dev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                       "traffic": None, "algorithmic_per_launch": moved,
+                       "mfma_frac": round(out["int8_tops"] / PEAK_INT8_TOPS, 4)}
     if per_layer:
         names = [n for _, n, _, _ in net.steps] + ["sm.max", "sm.sub", "sm.exp", "sm.sum", "softmax"]
         layers = []
@@ -318,7 +357,7 @@ def check_output(case, arrays, got):
     return "whole output against the oracle"
 
 
-def bench_chain(c, hw, stride, steps, warmup, batch=64):
+def bench_chain(c, hw, stride, steps, warmup, batch=64, cpu=False):
     """BASELINE configs[3]: depthwise 3x3 -> max-pool 2x2 s2 -> add + ReLU with requantisation,
     three operators of one model on the static arena (the model runtime runs the chain as one kernel
     when nothing else reads the tensors in between). Bytes = what each operator must read and write
@@ -378,7 +417,21 @@ def bench_chain(c, hw, stride, steps, warmup, batch=64):
         if not np.array_equal(got[i:i + 1], want):
             raise SystemExit("bench.py: chain output of image %d differs from the oracle" % i)
     m.close()
-    return {"metric": "hbm_gbps", "value": round(nbytes / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+    cpu_leg = {}
+    if cpu:
+        # the three operators through the C restatement on ONE host core, image 0 only
+        port.set_threads(1)
+        t0 = time.perf_counter()
+        d = one.run_port({"src": arrays["src"][:1], "flt": arrays["flt"], "bias": arrays["bias"]})
+        p = port.pool_q8(d, abi.FMT_NCHW44, abi.POOL_MAX, (2, 2), (2, 2), (0, 0))
+        port.multitype_q8(p, other[:1], abi.Q_FUSE_ADD_RELU, 0.05, 0.01, 0.05)
+        dt = time.perf_counter() - t0
+        cpu_leg = {"cpu_baseline": {
+            "value": round(nbytes / batch / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "batch 1 of %d, timed once in %.5f s (the whole workload at that rate: %.4g s); "
+                      "oracle/oracle_port.c built with -O2" % (batch, dt, dt * batch),
+            "host_cores": os.cpu_count()}}
+    return {**cpu_leg, "metric": "hbm_gbps", "value": round(nbytes / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
             "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
             "data": "synthetic",
@@ -404,17 +457,20 @@ def bench_mfma_only(mfma_per_simd, launches):
     library with HIP events, for three operand distributions: the board is power-limited and the
     rate depends on the operand values."""
     import ctypes
-    from megcc_amd import runtime
-    lib = runtime.lib()
-    lib.megcc_gfx950_probe_mfma_i8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                               ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
-    lib.megcc_gfx950_probe_mfma_i8.restype = ctypes.c_int
+    import megcc_amd
+    path = os.path.join(megcc_amd.PKG_DIR, "libmegcc_bench_probe.so")  # bench-only, not the product library
+    if not os.path.exists(path):
+        raise SystemExit("%s is missing: run __graft_entry__.build()" % path)
+    lib = ctypes.CDLL(path)
+    lib.megcc_bench_probe_mfma_i8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                              ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
+    lib.megcc_bench_probe_mfma_i8.restype = ctypes.c_int
     res = {}
     for kind, name in ((1, "uniform_int8"), (0, "zeros"), (2, "relu_activations_normal_weights")):
         us, n = ctypes.c_double(), ctypes.c_double()
-        st = lib.megcc_gfx950_probe_mfma_i8(kind, mfma_per_simd, launches, ctypes.byref(us), ctypes.byref(n))
+        st = lib.megcc_bench_probe_mfma_i8(kind, mfma_per_simd, launches, ctypes.byref(us), ctypes.byref(n))
         if st != 0:
-            raise SystemExit("megcc_gfx950_probe_mfma_i8: status %d: %s" % (st, lib.megcc_gfx950_last_error().decode()))
+            raise SystemExit("megcc_bench_probe_mfma_i8: status %d" % st)
         res[name] = {"us_per_launch": round(us.value, 2), "tops": round(n.value * MFMA_OPS / us.value / 1e6, 1)}
     v = res["uniform_int8"]
     return {"metric": "int8_mfma_only_tops", "value": v["tops"], "unit": "TOP/s", "n_gpus": 1, "steps": launches,
@@ -422,7 +478,7 @@ def bench_mfma_only(mfma_per_simd, launches):
             "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
             "config": {"workload": "v_mfma_i32_32x32x32_i8 only, %d per SIMD per launch (the default "
                        "workload's count), operands in registers" % mfma_per_simd,
-                       "abi": "megcc_gfx950_probe_mfma_i8"},
+                       "abi": "megcc_bench_probe_mfma_i8 (libmegcc_bench_probe.so, not the product library)"},
             "roofline": {"bound": "mfma", "achieved": v["tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                          "frac": round(v["tops"] / PEAK_INT8_TOPS, 4), "traffic": None},
             **res}
@@ -502,10 +558,11 @@ def main():
     if args.workload == "mobilenet":
         print(json.dumps(bench_mobilenet(args.batch, args.steps, args.warmup, args.per_layer)))
         return
-    if args.workload.startswith("chain"):  # chain, chain_s2, chain512, chain512_s2
-        c, hw, st = {"chain": (32, 112, 1), "chain_s2": (32, 112, 2), "chain512": (512, 14, 1),
-                     "chain512_s2": (512, 14, 2)}[args.workload]
-        print(json.dumps(bench_chain(c, hw, st, args.steps, args.warmup)))
+    if args.workload.startswith("chain"):  # chain, chain_s2, chain512, chain512_s2, chain:C,HW,S
+        c, hw, st = [int(v) for v in args.workload[6:].split(",")] if args.workload.startswith("chain:") else {
+            "chain": (32, 112, 1), "chain_s2": (32, 112, 2), "chain512": (512, 14, 1),
+            "chain512_s2": (512, 14, 2)}[args.workload]
+        print(json.dumps(bench_chain(c, hw, st, args.steps, args.warmup, cpu=args.cpu)))
         return
     if args.workload == "mfma_only":
         # as many MFMAs per SIMD as the default workload's launch has, spread evenly over 256 CUs
@@ -557,9 +614,7 @@ def main():
         value, unit, metric = nbytes / (wall / args.steps) / 1e9, "GB/s", "hbm_gbps"
         roof = {"bound": "hbm", "achieved": round(nbytes / (kern_ms * 1e-3) / 1e9, 2),
                 "peak": PEAK_HBM_GBS, "unit": "GB/s", "traffic": None}
-    roof["traffic"], traffic_file = measured_traffic(args.workload)
-    if traffic_file:
-        roof["traffic_source"] = traffic_file
+    roof.update(traffic_fields(args.workload, nbytes, sum(sp.nbytes for sp in outs)))
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
     roof["kernel_ms"] = round(kern_ms, 5)
     roof["algorithmic_per_launch"] = ops if bound == "mfma" else nbytes
@@ -590,6 +645,8 @@ def main():
         mb256 = bench_mobilenet(256, 60, 30)
         import mobilenet
         cpu_s, used = mobilenet.Net(1).run_cpu_timed(mobilenet.draw_input(1, seed=1), threads=1)
+        out["mobilenet_roofline"] = dict(mb["roofline"], workload="MobileNetV1-int8 batch 64, one forward = %d kernels (%s)" % (
+            mb["nr_kernel"], mb["launch_mode"]), images_per_s=mb["images_per_s"])
         out["extra"] = {"mobilenet_v1_int8_images_per_s_batch64": mb["images_per_s"],
                         "mobilenet_v1_int8_ms_per_forward_batch64": mb["ms_per_forward"],
                         "mobilenet_v1_int8_images_per_s_batch1": mb1["images_per_s"],

@@ -315,12 +315,17 @@ TinyNNStatus megcc_gfx950_conv2d_workspace(
  * harnesses that forbid hipMalloc. The scratch the layer's kernels need (split-K partial sums,
  * gathered pixels, NCHW44 copies: see megcc_gfx950_conv2d_workspace) lives in a static device
  * array of MEGCC_GFX950_NOALLOC_SCRATCH_BYTES that each GPU the library runs on holds until the
- * process ends. A layer that needs more returns TinyNN_ERROR_OUT_OF_RANGE (use
- * megcc_gfx950_conv2d). `inputs[1]` is the filter as the init protocol left it. Every call on a
+ * process ends. A layer whose REQUIRED scratch (the strided 1x1 and dense plain-NCHW cases of
+ * megcc_gfx950_conv2d_workspace) exceeds the array returns TinyNN_ERROR_OUT_OF_RANGE (use
+ * megcc_gfx950_conv2d); a layer whose optional scratch exceeds it runs as megcc_gfx950_conv2d runs
+ * it without a workspace (unsplit, or on the generic kernel: qsi8 results identical, f32 results
+ * within the 1e-4 tolerance of another summation order). `inputs[1]` is the filter as the init protocol left it. Every call on a
  * GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race.
  * Nothing in the array has to start at zero - every byte a kernel reads was written by an
  * earlier kernel of the same call. Calls no hipMalloc / hipFree; the array's address is looked
- * up at megcc_gfx950_init_device() or, failing that, on the first call on a device. */
+ * up at megcc_gfx950_init_device() or, failing that, on the first call on a device - so a caller
+ * that captures this entry point into a HIP graph calls megcc_gfx950_init_device() (or this entry
+ * point once) on the device BEFORE the capture begins: the look-up is not a stream operation. */
 #define MEGCC_GFX950_NOALLOC_SCRATCH_BYTES (32u << 20)
 TinyNNStatus megcc_gfx950_conv2d_noalloc(
         const MegccConvAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
@@ -551,14 +556,6 @@ const char* megcc_gfx950_last_kernel(void);
  * same names in capitals behind MEGCC_ are read from the environment once, at first use.
  * Unknown names return TinyNN_ERROR_NO_FOUND. */
 TinyNNStatus megcc_gfx950_set_option(const char* name, int value);
-/* Measurement aid (no counterpart in the reference): the time of a launch that does nothing but
- * v_mfma_i32_32x32x32_i8 - operands in registers, `mfma_per_simd` MFMAs on every SIMD of the chip -
- * averaged over `launches` launches after as many untimed ones. operand_kind 0: zeros, 1: uniform
- * random int8 (the operand distribution of the reference's benchmarks), 2: ReLU-like activations
- * against normally distributed weights. The board is power-limited and the rate depends on the
- * operand values; bench.py --workload mfma_only prints it beside the published peak. */
-TinyNNStatus megcc_gfx950_probe_mfma_i8(
-        int operand_kind, int mfma_per_simd, int launches, double* us_per_launch, double* mfma_per_launch);
 
 /* ------------------------------------------------------------------------------------------
  * In-memory model runtime: MegCC's static memory plan on one HBM arena. The calls mirror what the
@@ -607,7 +604,25 @@ TinyNNStatus megcc_gfx950_model_add_opr_desc(
         void* model, const MegccKernelDesc* desc, const char* name, const int* inputs, int nr_input,
         const int* outputs, int nr_output);
 TinyNNStatus megcc_gfx950_model_mark_io(void* model, int tensor, int is_output);
+/* The compiler's static memory plan for a model built in memory: offsets[i] = byte offset of
+ * tensor i in one arena of arena_bytes bytes (entries of weights, model inputs and views are
+ * ignored), what a `.tiny` file carries as Tensor.offset / DeviceModel.tensor_memory
+ * (runtime/schema/model.fbs:63-124, used by runtime/src/init.c:437-487). finalize then keeps these
+ * offsets instead of planning. TinyNN_ERROR_INVALID_LAYOUT for an offset that is not a multiple of
+ * the device alignment or a tensor that leaves the arena. Call after the last add_* / mark_io. */
+TinyNNStatus megcc_gfx950_model_set_plan(
+        void* model, const size_t* offsets, int nr_tensor, size_t arena_bytes);
 TinyNNStatus megcc_gfx950_model_finalize(void* model);
+/* No counterpart in the reference (its VM runs one kernel per Opr, synchronously): the number of
+ * kernels one forward launches (an operator chain that runs as one kernel counts once; a chain is
+ * only replaced when its result shares no byte with anything the one kernel reads), and how they
+ * are launched: 1 = HIP-graph replay, -1 = one launch per kernel, 0 = still measuring. forward()
+ * 2, 3, 5 and 6 of a model with at least 5 kernels each block the host until that forward has
+ * finished (they time the two ways between events on the library stream; *eager_ms / *graph_ms
+ * receive the shortest of two samples each, -1 when not measured); every other forward is
+ * asynchronous. */
+int megcc_gfx950_model_nr_kernel(void* model);
+int megcc_gfx950_model_launch_mode(void* model, float* eager_ms, float* graph_ms);
 size_t megcc_gfx950_model_arena_bytes(void* model);
 void* megcc_gfx950_model_tensor_ptr(void* model, int tensor);
 TinyNNStatus megcc_gfx950_model_set_input(void* model, int tensor, const void* host, size_t bytes);

@@ -50,14 +50,37 @@ bool parse_nonline(const std::string& s, MegccNonline* out) {
 
 bool parse_conv(std::string s, MegccConvAttr* a) {
     // the names of the f32 NCHW44 kernels the reference picks (GeneralIntrinsic/ConvKernel):
-    //   GI_kernel_conv2d_<k>x<k>_NCHW44_DENSE_p.._s.._d.._<io>[_bias][_NONLINE]_winograd_f23 / f43 / f63
+    //   GI_kernel_conv2d_<k>x<k>_NCHW44_DENSE_p.._s.._d.._<io>[_bias][_NONLINE]_winograd_f23
+    //       ... _winograd_f43_fp32 / _winograd_f63_fp32   (Fp32WinogradNchw44.cpp:83,157,231; F63
+    //       is the registry's first choice for 3x3 stride 1, GeneralIntrinsic/KernelPack.cpp:54-56)
     //   GI_kernel_conv2d_conv1x1_NCHW44_1x1_DENSE_p.._s.._d..[_bias][_NONLINE]
-    for (const char* w : {"_winograd_f23", "_winograd_f43", "_winograd_f63"})
+    //   GI_kernel_conv2d_<k>x<k>_NCHW44_DENSE_..._<io>[_bias][_NONLINE]_nchw_nchw44_oc<n>_ic<n>
+    //       (first layer: 4-dim source, 5-dim result; Fp32ConvNchwNchw44.cpp:37-55)
+    //   GI_chanwise_kernel_conv2d_<k>x<k>_NCHW44_GROUP_..._<io>[_bias][_NONLINE]
+    //       (ConvKernel.h:24-32,63-65)
+    bool first_layer = false;
+    for (const char* w : {"_winograd_f23", "_winograd_f43_fp32", "_winograd_f63_fp32"})
         if (ends_with(s, w)) {
             s.erase(s.size() - strlen(w));
             if (!eat(s, "GI_"))
                 return false;
         }
+    {
+        const size_t at = s.rfind("_nchw_nchw44_oc");
+        unsigned oc, ic;
+        int used = 0;
+        if (at != std::string::npos && sscanf(s.c_str() + at, "_nchw_nchw44_oc%u_ic%u%n", &oc, &ic, &used) == 2 &&
+            at + used == s.size()) {
+            s.erase(at);
+            if (!eat(s, "GI_"))
+                return false;
+            first_layer = true;
+        }
+    }
+    if (eat(s, "GI_chanwise_")) {
+        if (s.find("_NCHW44_GROUP_") == std::string::npos)
+            return false;
+    }
     if (eat(s, "GI_kernel_conv2d_conv1x1_")) {
         const bool f44 = eat(s, "NCHW44_");
         if (!f44 && !eat(s, "NCHW_"))
@@ -83,10 +106,12 @@ bool parse_conv(std::string s, MegccConvAttr* a) {
     if (eat(s, "NCHW_NCHW44_"))
         a->format = MEGCC_FMT_NCHW_NCHW44;
     else if (eat(s, "NCHW44_"))
-        a->format = MEGCC_FMT_NCHW44;
+        a->format = first_layer ? MEGCC_FMT_NCHW_NCHW44 : MEGCC_FMT_NCHW44;
     else if (eat(s, "NCHW_"))
         a->format = MEGCC_FMT_NCHW;
     else
+        return false;
+    if (first_layer && a->format != MEGCC_FMT_NCHW_NCHW44)
         return false;
     if (eat(s, "DENSE_"))
         a->sparse = MEGCC_SPARSE_DENSE;
@@ -196,7 +221,8 @@ extern "C" TinyNNStatus megcc_gfx950_parse_symbol(const char* symbol, MegccKerne
     memset(desc, 0, sizeof(*desc));
     std::string s(symbol);
     int v = 0;
-    if (starts_with(s, "kernel_conv2d_") || starts_with(s, "GI_kernel_conv2d_")) {
+    if (starts_with(s, "kernel_conv2d_") || starts_with(s, "GI_kernel_conv2d_") ||
+        starts_with(s, "GI_chanwise_kernel_conv2d_")) {
         if (parse_conv(s, &desc->attr.conv)) {
             desc->kind = MEGCC_KERN_CONV;
             return TinyNN_SUCCESS;

@@ -371,11 +371,18 @@ static TinyNNStatus conv2d_run(
         // (the native kernel for channel-wise NCHW layers needs none)
         const bool native_dw = q8 && dwconv_nchw_supported(g, src->ptr, dst->ptr) && !options().no_dwnchw;
         const size_t need = native_dw ? 0 : conv2d_scratch_bytes(g, q8, f32, packed);
-        MG_REQUIRE(need <= (size_t)MEGCC_GFX950_NOALLOC_SCRATCH_BYTES, TinyNN_ERROR_OUT_OF_RANGE,
+        // Only two paths cannot run without their scratch: a strided 1x1 layer (gathered pixels) and
+        // a dense layer on plain NCHW tensors (NCHW44 copies), both behind a packed filter. Every
+        // other request is an optimisation (split-K partial sums, relayout detours) that
+        // megcc_gfx950_conv2d also does without when it gets no workspace: same result, other kernel.
+        const bool strict = packed && q8 &&
+                            ((strided_pointwise(g) && conv_mfma_supported(subsampled(g))) ||
+                             (nchw_spatial(g) && conv_mfma_supported(as_nchw44(g))));
+        MG_REQUIRE(need <= (size_t)MEGCC_GFX950_NOALLOC_SCRATCH_BYTES || !strict, TinyNN_ERROR_OUT_OF_RANGE,
                    "conv2d_noalloc: this layer needs %zu bytes of scratch memory, the static "
                    "buffer holds %zu; call megcc_gfx950_conv2d with a workspace instead",
                    need, (size_t)MEGCC_GFX950_NOALLOC_SCRATCH_BYTES);
-        if (need) {
+        if (need && need <= (size_t)MEGCC_GFX950_NOALLOC_SCRATCH_BYTES) {
             st = scratch_of_current_device(&own.ptr);
             if (st != TinyNN_SUCCESS)
                 return st;

@@ -141,6 +141,18 @@ bool plan_memory(Model* m) {
 static bool dense_f32(const Tensor& t) {
     return t.dtype.type_enum == TinyNN_FLOAT && is_contiguous(t.layout);
 }
+// [ptr, ptr + bytes) of a dense tensor against another's: the kernels that replace an operator chain
+// read their inputs while other workgroups already write the chain's output, which is only safe
+// when the two ranges share no byte. A memory plan made for the unfused operators (the compiler's,
+// or plan_memory() above) may well put the chain's output into bytes an input of the chain's first
+// operator has just freed.
+static bool shares_bytes(const Tensor& a, const Tensor& b) {
+    const char *a0 = (const char*)a.ptr, *b0 = (const char*)b.ptr;
+    const size_t an = tensor_bytes(a), bn = tensor_bytes(b);
+    if (!a0 || !b0 || !an || !bn)
+        return false;
+    return a0 < b0 + bn && b0 < a0 + an;
+}
 static void build_schedule(Model* m) {
     m->schedule.clear();
     const int n = (int)m->oprs.size();
@@ -194,7 +206,11 @@ static void build_schedule(Model* m) {
                 f->in_ptrs.push_back(&m->tensors[other]->t);
                 f->out = o2->out;
                 f->out_ptrs = o2->out_ptrs;
-                if (megcc_gfx950_dw_pool_add_supported(
+                // the kernel reads src (with halos) and `other` while it writes the output
+                bool apart = true;
+                for (const Tensor* t : f->in_ptrs)
+                    apart = apart && !shares_bytes(*t, *f->out_ptrs[0]);
+                if (apart && megcc_gfx950_dw_pool_add_supported(
                             &f->desc.attr.dw_pool_add, f->in_ptrs.data(), (int)f->in_ptrs.size(), f->out_ptrs.data(),
                             (int)f->out_ptrs.size())) {
                     m->fused.push_back(f);
@@ -236,10 +252,21 @@ static void build_schedule(Model* m) {
                         cv->out[0] == x && temp(x, 2) &&
                         m->tensors[cv->in[0]]->t.dtype.type_enum == TinyNN_QINT8 &&
                         is_contiguous(m->tensors[cv->in[0]]->t.layout) &&
-                        nr_elem(m->tensors[cv->in[0]]->t.layout) == nr_elem(tx.layout)) {
+                        nr_elem(m->tensors[cv->in[0]]->t.layout) == nr_elem(tx.layout) &&
+                        // (only when the qsi8 logits and the result share no byte: a row of the
+                        //  result covers four rows' worth of logit bytes)
+                        !shares_bytes(m->tensors[cv->in[0]]->t, ty)) {
                         src = cv->in[0];
                         m->schedule.pop_back();
                     }
+                }
+                // A row is read whole before it is written, by one workgroup, so a result that
+                // starts exactly where its f32 source starts is fine; any other overlap would let
+                // one row's stores land in another row's unread source.
+                const Tensor& ts = m->tensors[src]->t;
+                if (shares_bytes(ts, ty) && !(src == x && ts.ptr == ty.ptr)) {
+                    m->schedule.push_back(o0);
+                    continue;
                 }
                 ModelOpr* f = new ModelOpr();
                 memset(&f->desc, 0, sizeof(f->desc));
@@ -583,6 +610,50 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
     return megcc_gfx950_wait();
 }
 
+// The compiler's static memory plan for a model built in memory: what a `.tiny` file carries as
+// Tensor.offset and DeviceModel.tensor_memory (runtime/schema/model.fbs:63-124, consumed by
+// runtime/src/init.c:437-487). finalize() then uses these offsets instead of planning.
+TinyNNStatus megcc_gfx950_model_set_plan(
+        void* model, const size_t* offsets, int nr_tensor, size_t arena_bytes) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && offsets && !m->finalized, TinyNN_ERROR_NULL_PTR, "model_set_plan: bad argument");
+    MG_REQUIRE(nr_tensor == (int)m->tensors.size(), TinyNN_ERROR_OUT_OF_RANGE,
+               "model_set_plan: %d offsets for %zu tensors", nr_tensor, m->tensors.size());
+    for (int i = 0; i < nr_tensor; ++i) {
+        ModelTensor* t = m->tensors[i];
+        if (t->is_weight || t->is_input || t->alias_of >= 0)
+            continue;
+        MG_REQUIRE(offsets[i] % m->dev.alignment == 0 && offsets[i] <= arena_bytes &&
+                           t->t.size <= arena_bytes - offsets[i],
+                   TinyNN_ERROR_INVALID_LAYOUT,
+                   "model_set_plan: tensor %d: %zu bytes at offset %zu of a %zu byte arena (alignment %zu)",
+                   i, (size_t)t->t.size, offsets[i], arena_bytes, (size_t)m->dev.alignment);
+    }
+    for (int i = 0; i < nr_tensor; ++i)
+        m->tensors[i]->t.offset = offsets[i];
+    m->arena_bytes = arena_bytes;
+    m->preplanned = true;
+    return TinyNN_SUCCESS;
+}
+
+// What forward() does with the model: the number of kernels of its schedule (operator chains that
+// run as one kernel count once), and how it launches them.
+int megcc_gfx950_model_nr_kernel(void* model) {
+    Model* m = (Model*)model;
+    return m && m->finalized ? (int)m->schedule.size() : 0;
+}
+
+int megcc_gfx950_model_launch_mode(void* model, float* eager_ms, float* graph_ms) {
+    Model* m = (Model*)model;
+    if (!m)
+        return 0;
+    if (eager_ms)
+        *eager_ms = m->eager_ms < 1e29f ? m->eager_ms : -1.f;
+    if (graph_ms)
+        *graph_ms = m->graph_ms < 1e29f ? m->graph_ms : -1.f;
+    return m->graph_state;
+}
+
 size_t megcc_gfx950_model_arena_bytes(void* model) {
     return model ? ((Model*)model)->arena_bytes : 0;
 }
@@ -688,7 +759,7 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
     }
     TinyNNStatus st = timed(true, &m->graph_ms);
     if (m->forwards >= 6)
-        m->graph_state = m->graph_ms <= m->eager_ms ? 1 : -1;
+        m->graph_state = m->graph_ms < 0.95f * m->eager_ms ? 1 : -1;  // (a tie keeps the plain launches)
     return st;
 }
 

@@ -4,13 +4,16 @@
 // power-limited, and uniform random int8 operands (the reference benchmark's distribution,
 // compiler/test/kernel/opr/arm/benchmark_conv.cpp:198) toggle the multipliers far more than zeros or
 // small values do. bench.py --workload mfma_only reports it next to the published peak.
+//
+// Built into a library of its own (libmegcc_bench_probe.so) that only bench.py and one test load:
+// the product library neither contains nor exports it. Self-contained: its own stream-less
+// launches on the null stream, no dependency on the product's sources.
+#include <hip/hip_runtime.h>
 #include <stdlib.h>
 
 #include <vector>
 
-#include "common.h"
-
-namespace mg {
+namespace {
 
 typedef int probe_v4i __attribute__((ext_vector_type(4)));
 typedef int probe_v16i __attribute__((ext_vector_type(16)));
@@ -39,18 +42,18 @@ __global__ void __launch_bounds__(512) probe_mfma_kernel(
         out[tid] = s;
 }
 
-}  // namespace mg
+}  // namespace
 
 // operand_kind 0: zeros; 1: uniform random int8 in [-127, 127]; 2: activations max(0, x) with x normal
 // (sigma 20) against weights normal (sigma 30), both clipped to int8. Runs `launches` launches of one
 // workgroup per CU with `mfma_per_simd` MFMAs per SIMD each (after as many untimed ones) and
 // returns the average time of a launch in microseconds and the MFMAs a launch issued.
-extern "C" TinyNNStatus megcc_gfx950_probe_mfma_i8(
+// Status: 0 = measured, 1 = bad argument, 2 = device memory, 3 = a HIP call failed.
+extern "C" int megcc_bench_probe_mfma_i8(
         int operand_kind, int mfma_per_simd, int launches, double* us_per_launch, double* mfma_per_launch) {
-    using namespace mg;
-    MG_REQUIRE(us_per_launch && mfma_per_launch && launches > 0 && mfma_per_simd >= 16 && operand_kind >= 0 &&
-                       operand_kind <= 2,
-               TinyNN_ERROR_OUT_OF_RANGE, "probe_mfma_i8: bad argument");
+    if (!(us_per_launch && mfma_per_launch && launches > 0 && mfma_per_simd >= 16 && operand_kind >= 0 &&
+          operand_kind <= 2))
+        return 1;
     const int nvar = 1 << 16;
     std::vector<int> h((size_t)nvar * 4);
     unsigned long long state = 88172645463325252ull;
@@ -84,29 +87,37 @@ extern "C" TinyNNStatus megcc_gfx950_probe_mfma_i8(
         }
         h[i] = (int)w;
     }
-    const int cus = num_cus();
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        return 3;
     const int iters = (mfma_per_simd / 2 + 7) / 8;  // 2 waves per SIMD, 8 MFMAs per iteration
     void* d = nullptr;
     void* out = nullptr;
-    MG_REQUIRE(hipMalloc(&d, (size_t)nvar * 16) == hipSuccess && hipMalloc(&out, (size_t)cus * 512 * 4) == hipSuccess,
-               TinyNN_ERROR_MEMORY_MALLOC, "probe_mfma_i8: device memory");
+    if (hipMalloc(&d, (size_t)nvar * 16) != hipSuccess)
+        return 2;
+    if (hipMalloc(&out, (size_t)cus * 512 * 4) != hipSuccess) {
+        (void)hipFree(d);
+        return 2;
+    }
     hipEvent_t e0 = nullptr, e1 = nullptr;
-    TinyNNStatus st = TinyNN_SUCCESS;
+    int st = 0;
     float ms = 0;
+    hipStream_t strm = nullptr;  // the null stream
     if (hipMemcpy(d, h.data(), (size_t)nvar * 16, hipMemcpyHostToDevice) != hipSuccess ||
         hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
-        st = TinyNN_ERROR_RUNTIME;
+        st = 3;
     } else {
         for (int w = 0; w < launches; ++w)
-            hipLaunchKernelGGL(probe_mfma_kernel, dim3(cus), dim3(512), 0, stream(), (const probe_v4i*)d, (int*)out,
+            hipLaunchKernelGGL(probe_mfma_kernel, dim3(cus), dim3(512), 0, strm, (const probe_v4i*)d, (int*)out,
                                iters, nvar);
-        (void)hipEventRecord(e0, stream());
+        (void)hipEventRecord(e0, strm);
         for (int w = 0; w < launches; ++w)
-            hipLaunchKernelGGL(probe_mfma_kernel, dim3(cus), dim3(512), 0, stream(), (const probe_v4i*)d, (int*)out,
+            hipLaunchKernelGGL(probe_mfma_kernel, dim3(cus), dim3(512), 0, strm, (const probe_v4i*)d, (int*)out,
                                iters, nvar);
-        (void)hipEventRecord(e1, stream());
+        (void)hipEventRecord(e1, strm);
         if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(&ms, e0, e1) != hipSuccess)
-            st = TinyNN_ERROR_RUNTIME;
+            st = 3;
     }
     if (e0)
         (void)hipEventDestroy(e0);
@@ -114,8 +125,9 @@ extern "C" TinyNNStatus megcc_gfx950_probe_mfma_i8(
         (void)hipEventDestroy(e1);
     (void)hipFree(d);
     (void)hipFree(out);
-    MG_REQUIRE(st == TinyNN_SUCCESS, st, "probe_mfma_i8: %s", hipGetErrorString(hipGetLastError()));
+    if (st)
+        return st;
     *us_per_launch = (double)ms / launches * 1e3;
     *mfma_per_launch = (double)cus * 8 * 8 * iters;
-    return TinyNN_SUCCESS;
+    return 0;
 }

@@ -107,11 +107,12 @@ EXPORTS = [
     "megcc_gfx950_malloc", "megcc_gfx950_free", "megcc_gfx950_memcpy_h2d",
     "megcc_gfx950_memcpy_d2h", "megcc_gfx950_memset", "megcc_gfx950_wait",
     "megcc_gfx950_stream", "megcc_gfx950_last_error", "megcc_gfx950_last_kernel",
-    "megcc_gfx950_set_option", "megcc_gfx950_probe_mfma_i8",
+    "megcc_gfx950_set_option",
     "megcc_gfx950_model_create", "megcc_gfx950_model_destroy", "megcc_gfx950_model_add_tensor",
     "megcc_gfx950_model_add_weight", "megcc_gfx950_model_add_alias", "megcc_gfx950_model_add_view",
     "megcc_gfx950_model_add_opr", "megcc_gfx950_model_add_opr_desc",
     "megcc_gfx950_model_mark_io", "megcc_gfx950_model_finalize", "megcc_gfx950_model_arena_bytes",
+    "megcc_gfx950_model_set_plan", "megcc_gfx950_model_nr_kernel", "megcc_gfx950_model_launch_mode",
     "megcc_gfx950_model_tensor_ptr", "megcc_gfx950_model_set_input",
     "megcc_gfx950_model_get_output", "megcc_gfx950_model_forward", "megcc_gfx950_model_nr_opr",
     "megcc_gfx950_model_run_opr", "megcc_gfx950_plan_memory", "megcc_gfx950_model_load",
@@ -374,8 +375,31 @@ class Model:
     def mark_output(self, tid):
         check(lib().megcc_gfx950_model_mark_io(self.h, tid, 1), "mark_io")
 
+    def set_plan(self, offsets, arena_bytes):
+        """the compiler's static memory plan: byte offset per tensor id (entries of weights, inputs
+        and views are ignored) and the arena size; finalize() then keeps it instead of planning"""
+        L = lib()
+        L.megcc_gfx950_model_set_plan.argtypes = [C.c_void_p, C.POINTER(C.c_size_t), C.c_int, C.c_size_t]
+        arr = (C.c_size_t * len(offsets))(*[int(o) for o in offsets])
+        check(L.megcc_gfx950_model_set_plan(self.h, arr, len(offsets), int(arena_bytes)), "set_plan")
+
     def finalize(self):
         check(lib().megcc_gfx950_model_finalize(self.h), "finalize")
+
+    @property
+    def nr_kernel(self):
+        """kernels one forward launches (an operator chain run as one kernel counts once)"""
+        L = lib()
+        L.megcc_gfx950_model_nr_kernel.argtypes = [C.c_void_p]
+        return L.megcc_gfx950_model_nr_kernel(self.h)
+
+    def launch_mode(self):
+        """(mode, eager_ms, graph_ms): 1 = graph replay, -1 = one launch per kernel, 0 = undecided"""
+        L = lib()
+        L.megcc_gfx950_model_launch_mode.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+        e, g = C.c_float(), C.c_float()
+        mode = L.megcc_gfx950_model_launch_mode(self.h, C.byref(e), C.byref(g))
+        return mode, e.value, g.value
 
     @property
     def arena_bytes(self):

@@ -46,6 +46,21 @@ def macs_per_image():
     return sum(c.ops() // 2 for _, c in conv_layers(1))
 
 
+def algorithmic_bytes(batch):
+    """bytes one forward must move when every operator reads its inputs and writes its result once
+    (activations in, weights, bias, activations out; the f32 image, the typecvts, the pooling and
+    the five soft-max operators included): the figure a bandwidth roofline of the whole network is
+    priced against"""
+    n = lambda shape: int(np.prod(shape))
+    total = batch * 3 * 224 * 224 * (4 + 1)  # quantise the f32 image
+    for _, c in conv_layers(batch):
+        total += n(c.src_shape()) + n(c.flt_shape()) + 4 * n(c.bias_shape()) + n(c.dst_shape())
+    total += batch * 1024 * (49 + 1)  # global average pooling
+    total += batch * 1000 * (1 + 4)  # dequantise the logits
+    total += batch * 1000 * 4 * (1 + 2 + 2 + 1 + 2) + batch * 4 * (1 + 1 + 1 + 1)  # max, sub, exp, sum, div
+    return total
+
+
 def draw_weights(seed=0):
     """{layer: (filter int8, bias int32, filter scale)} -- independent of the batch size"""
     r = np.random.Generator(np.random.PCG64(seed))

@@ -68,6 +68,32 @@ def test_parse_conv_symbol_fields():
     assert (d.attr.conv.with_bias, d.attr.conv.nonline) == (0, abi.IDENTITY)
 
 
+def test_parse_f32_nchw44_symbols_of_the_general_intrinsic_pack():
+    """the names MegCC's GI pack gives the f32 NCHW44 layers: all three Winograd variants (F63 is
+    the first choice of a 3x3 stride-1 layer, GeneralIntrinsic/KernelPack.cpp:54-56; F43 and F63
+    end in _fp32, Fp32WinogradNchw44.cpp:157,231), the NCHW -> NCHW44 first layer
+    (Fp32ConvNchwNchw44.cpp:37-55) and the channel-wise kernel (ConvKernel.h:63-65)"""
+    base = "GI_kernel_conv2d_3x3_NCHW44_DENSE_p1x1_s1x1_d1x1_f32f32f32f32_bias_RELU"
+    for tail in ("_winograd_f23", "_winograd_f43_fp32", "_winograd_f63_fp32"):
+        a = runtime.parse_symbol(base + tail).attr.conv
+        assert (a.format, a.sparse, a.kernel_h, a.with_bias, a.nonline) == (abi.FMT_NCHW44, abi.DENSE, 3, 1, abi.RELU)
+    for bad in ("_winograd_f43", "_winograd_f63", "_winograd_f23_fp32"):
+        with pytest.raises(runtime.MegccError):
+            runtime.parse_symbol(base + bad)
+    a = runtime.parse_symbol(
+        "GI_kernel_conv2d_3x3_NCHW44_DENSE_p1x1_s2x2_d1x1_f32f32f32f32_bias_H_SWISH_nchw_nchw44_oc32_ic3").attr.conv
+    assert (a.format, a.stride_h, a.pad_w, a.nonline, a.with_bias) == (abi.FMT_NCHW_NCHW44, 2, 1, abi.H_SWISH, 1)
+    a = runtime.parse_symbol("GI_kernel_conv2d_5x5_NCHW44_DENSE_p2x2_s1x1_d1x1_f32f32f32f32_nchw_nchw44_oc8_ic1").attr.conv
+    assert (a.format, a.kernel_w, a.with_bias, a.nonline) == (abi.FMT_NCHW_NCHW44, 5, 0, abi.IDENTITY)
+    a = runtime.parse_symbol("GI_chanwise_kernel_conv2d_5x5_NCHW44_GROUP_p2x2_s2x2_d1x1_f32f32f32f32_bias_RELU").attr.conv
+    assert (a.format, a.sparse, a.kernel_h, a.stride_w, a.nonline) == (abi.FMT_NCHW44, abi.GROUP, 5, 2, abi.RELU)
+    for bad in ("GI_chanwise_kernel_conv2d_3x3_NCHW44_DENSE_p1x1_s1x1_d1x1_f32f32f32f32",
+                "kernel_conv2d_3x3_NCHW44_DENSE_p1x1_s2x2_d1x1_f32f32f32f32_nchw_nchw44_oc32_ic3",
+                "GI_kernel_conv2d_3x3_NCHW_DENSE_p1x1_s2x2_d1x1_f32f32f32f32_nchw_nchw44_oc32_ic3"):
+        with pytest.raises(runtime.MegccError):
+            runtime.parse_symbol(bad)
+
+
 def test_parse_other_symbols():
     d = runtime.parse_symbol("kernel_pooling_AVERAGE_COUNT_EXCLUDE_PADDING_NCHW_p1x1_s2x2_w3x3_qsi8qsi8")
     assert d.kind == abi.KERN_POOLING and d.attr.pool.mode == abi.POOL_AVERAGE_COUNT_EXCLUDE_PADDING

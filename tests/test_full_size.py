@@ -190,7 +190,7 @@ def test_cfg1_conv_f32():
 
 
 # ---- configs[3]: the bandwidth-bound chain at N = 64 ---------------------------------------------
-CFG4 = [(32, 112, 1), (32, 112, 2), (512, 14, 1), (512, 14, 2)]
+CFG4 = [(32, 112, 1), (32, 112, 2), (512, 14, 1), (512, 14, 2), (512, 112, 1), (512, 112, 2), (32, 14, 1), (32, 14, 2)]
 
 
 @pytest.mark.parametrize("c,hw,stride", CFG4, ids=["c%d_%dx%d_s%d" % (c, hw, hw, st) for c, hw, st in CFG4])

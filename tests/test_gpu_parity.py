@@ -905,15 +905,16 @@ def test_mfma_only_probe_reports_a_plausible_rate():
     """the measurement aid behind bench.py's mfma_only figures: argument checks, the MFMA count of
     a launch, and a rate between a tenth of the published int8 peak and the peak itself"""
     import ctypes as C
-    lib = runtime.lib()
-    lib.megcc_gfx950_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double),
-                                               C.POINTER(C.c_double)]
+    import megcc_amd
+    lib = C.CDLL(os.path.join(megcc_amd.PKG_DIR, "libmegcc_bench_probe.so"))
+    lib.megcc_bench_probe_mfma_i8.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double),
+                                              C.POINTER(C.c_double)]
     us, n = C.c_double(), C.c_double()
-    assert lib.megcc_gfx950_probe_mfma_i8(3, 256, 10, C.byref(us), C.byref(n)) == abi.ERROR_OUT_OF_RANGE
-    assert lib.megcc_gfx950_probe_mfma_i8(1, 256, 0, C.byref(us), C.byref(n)) == abi.ERROR_OUT_OF_RANGE
-    assert lib.megcc_gfx950_probe_mfma_i8(1, 256, 10, None, C.byref(n)) == abi.ERROR_OUT_OF_RANGE
+    assert lib.megcc_bench_probe_mfma_i8(3, 256, 10, C.byref(us), C.byref(n)) == 1
+    assert lib.megcc_bench_probe_mfma_i8(1, 256, 0, C.byref(us), C.byref(n)) == 1
+    assert lib.megcc_bench_probe_mfma_i8(1, 256, 10, None, C.byref(n)) == 1
     for kind in (0, 1, 2):
-        assert lib.megcc_gfx950_probe_mfma_i8(kind, 1024, 20, C.byref(us), C.byref(n)) == 0
+        assert lib.megcc_bench_probe_mfma_i8(kind, 1024, 20, C.byref(us), C.byref(n)) == 0
         assert n.value == 256 * 4 * 1024, "256 CUs x 4 SIMDs x 1024 MFMAs"
         tops = n.value * 65536 / us.value / 1e6
         assert 500 < tops <= 5000, (kind, us.value, tops)
@@ -1054,3 +1055,129 @@ def test_model_runtime_fuses_the_depthwise_pool_add_chain(cfg):
     assert not kernel.startswith("dwconv44_chain"), kernel
     for o in fused + plain:
         compare(o, want, "chain %r" % (cfg,))
+
+
+# ---- operator chains that run as one kernel, under memory plans made for the separate operators ----
+# A static plan gives a tensor's bytes to the next tensor born after its last reader. For the chain
+# depthwise -> pool -> add that is the add's result over the depthwise INPUT (dead after operator i,
+# result born at i + 2); for the soft-max chain the result over the logits. The one-kernel forms read
+# those inputs while they write the result, so the model runtime must keep the operators apart when
+# the plan it was given overlaps them.
+def _planned_chain(out_offset):
+    n, c, hw = 2, 16, 12
+    dw, pool, add = _chain_cases(n, c, hw, hw, 1, A.RELU, A.Q_FUSE_ADD_RELU, True)
+    arrays = dw.gen(21)
+    x0 = np.random.default_rng(22).integers(-128, 128, dw.src_shape()).astype(np.int8)
+    other = np.random.default_rng(23).integers(-128, 128, pool.dst_shape()).astype(np.int8)
+    pre = MultiTypeCase(A.Q_RELU, dw.src_shape(), (0.03, 0.01, dw.scales[0]))
+    m = runtime.Model()
+    t_in = m.tensor("x0", dw.src_shape(), abi.QINT8, 0.03)
+    t_other = m.tensor("other", pool.dst_shape(), abi.QINT8, add.scales[1])
+    m.mark_input(t_in)
+    m.mark_input(t_other)
+    t_x = m.tensor("x", dw.src_shape(), abi.QINT8, dw.scales[0])  # an arena tensor that dies at the depthwise layer
+    m.opr(pre.symbol(), [t_in], [t_x])
+    w = m.weight("dw.w", arrays["flt"], abi.QINT8, dw.scales[1])
+    b = m.weight("dw.b", arrays["bias"], abi.QINT32, float(np.float32(dw.scales[0]) * np.float32(dw.scales[1])))
+    t1 = m.tensor("dw", dw.dst_shape(), abi.QINT8, dw.scales[2])
+    m.opr(dw.symbol(), [t_x, w, b], [t1])
+    t2 = m.tensor("pool", pool.dst_shape(), abi.QINT8, dw.scales[2])
+    m.opr(pool.symbol(), [t1], [t2])
+    t3 = m.tensor("out", pool.dst_shape(), abi.QINT8, add.scales[2])
+    m.opr(add.symbol(), [t2, t_other], [t3])
+    m.mark_output(t3)
+    nx = int(np.prod(dw.src_shape()))
+    up = lambda v: (v + 255) // 256 * 256
+    offs = [0] * 8
+    offs[t_x], offs[t1] = 0, up(nx)
+    offs[t2] = offs[t1] + up(nx)
+    offs[t3] = out_offset if out_offset is not None else offs[t2] + up(nx)
+    m.set_plan(offs[:t3 + 1], offs[t2] + 2 * up(nx))
+    m.finalize()
+    m.set_input(t_in, x0)
+    m.set_input(t_other, other)
+    outs = []
+    for _ in range(3):
+        m.forward()
+        runtime.wait()
+        outs.append(m.get(t3).copy())
+    x = pre.run_port({"a": x0, "b": None})
+    arrays["src"] = x
+    want = add.run_port({"a": pool.run_port({"src": dw.run_port(arrays)}), "b": other})
+    nk = m.nr_kernel
+    m.close()
+    return outs, nk, want
+
+
+@pytest.mark.parametrize("out_offset,kernels", [(None, 2), (0, 4), (256, 4), (4352, 4)],
+                         ids=["apart", "result_on_the_input", "result_256_bytes_into_the_input", "result_over_the_input_tail"])
+def test_chain_is_one_kernel_only_when_its_result_shares_no_byte_with_its_inputs(out_offset, kernels):
+    outs, nk, want = _planned_chain(out_offset)
+    assert nk == kernels
+    for o in outs:
+        compare(o, want, "planned chain, result at %r" % (out_offset,))
+
+
+def _planned_softmax(front, y_on):
+    """soft-max chain behind `front`: "cvt" = f32 -> qsi8 -> f32 typecvts (the dequantising one can join
+    the one-kernel form, which then reads the qsi8 logits), "neg" = an f32 NEGATE (the kernel reads
+    the f32 logits x); the result y is planned apart, or over q / x"""
+    rows, cols = 8, 1000
+    rng = np.random.default_rng(31)
+    logits = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+    big = 32768  # rows * cols * 4 rounded up to 256
+    m = runtime.Model()
+    t_in = m.tensor("in", (rows, cols), abi.FLOAT)
+    m.mark_input(t_in)
+    place = {}
+    if front == "cvt":
+        q = m.tensor("q", (rows, cols), abi.QINT8, 0.1)
+        m.opr("GI_kernel_typecvt_f32qsi8", [t_in], [q])
+        x = m.tensor("x", (rows, cols), abi.FLOAT)
+        m.opr("GI_kernel_typecvt_qsi8f32", [q], [x])
+        place[q] = 0
+        xv = np.clip(np.round(logits / np.float32(0.1)), -128, 127).astype(np.float32) * np.float32(0.1)
+    else:
+        x = m.tensor("x", (rows, cols), abi.FLOAT)
+        m.opr("kernel_elementwise_NEGATE_f32f32", [t_in], [x])
+        xv = -logits
+    mx = m.tensor("sm.max", (rows, 1), abi.FLOAT)
+    m.opr("kernel_reduce_MAX_DEFAULT_a1_f32f32", [x], [mx])
+    sub = m.tensor("sm.sub", (rows, cols), abi.FLOAT)
+    m.opr("kernel_elementwise_SUB_f32f32f32", [x, mx], [sub])
+    ex = m.tensor("sm.exp", (rows, cols), abi.FLOAT)
+    m.opr("kernel_elementwise_EXP_f32f32", [sub], [ex])
+    sm = m.tensor("sm.sum", (rows, 1), abi.FLOAT)
+    m.opr("kernel_reduce_SUM_DEFAULT_a1_f32f32", [ex], [sm])
+    y = m.tensor("softmax", (rows, cols), abi.FLOAT)
+    m.opr("kernel_elementwise_TRUE_DIV_f32f32f32", [ex, sm], [y])
+    m.mark_output(y)
+    place.update({x: big, mx: 2 * big, sub: 3 * big, ex: 4 * big, sm: 5 * big})
+    place[y] = {"apart": 6 * big, "q_shifted": 256, "x_exact": big, "x_shifted": big + 4096}[y_on]
+    m.set_plan([place.get(t, 0) for t in range(y + 1)], 8 * big)
+    m.finalize()
+    m.set_input(t_in, logits)
+    outs = []
+    for _ in range(3):
+        m.forward()
+        runtime.wait()
+        outs.append(m.get(y).copy())
+    nk = m.nr_kernel
+    m.close()
+    e = np.exp(xv.astype(np.float64) - xv.max(axis=1, keepdims=True))
+    return outs, nk, (e / e.sum(axis=1, keepdims=True)).astype(np.float32)
+
+
+@pytest.mark.parametrize("front,y_on,kernels", [
+    ("cvt", "apart", 2), ("cvt", "q_shifted", 3), ("cvt", "x_shifted", 2),
+    ("neg", "apart", 2), ("neg", "x_exact", 2), ("neg", "x_shifted", 6)])
+def test_softmax_is_one_kernel_only_when_its_result_cannot_overwrite_unread_logits(front, y_on, kernels):
+    """cvt/apart: the dequantising typecvt and the five operators are one kernel reading the qsi8
+    logits; result over the qsi8 logits: that typecvt stays an operator and the kernel reads the f32
+    logits; result over the f32 logits while the kernel reads the qsi8 ones: nothing it reads is
+    touched. neg: the kernel reads the f32 logits x; a result exactly on x is fine (a row is read
+    whole before it is written), a result shifted into x is not: the five operators run one by one"""
+    outs, nk, want = _planned_softmax(front, y_on)
+    assert nk == kernels
+    for o in outs:
+        assert cases.max_rel_err(o, want) <= 1e-5, (front, y_on)

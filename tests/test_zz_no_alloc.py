@@ -92,6 +92,31 @@ def test_noalloc_rejects_layers_beyond_the_array():
     runtime.wait()
 
 
+def test_noalloc_runs_layers_whose_optional_scratch_exceeds_the_array_without_it():
+    """scratch that only buys speed (relayout detour of a channel-wise NCHW layer, split-K partial
+    sums of a skinny f32 layer) is done without when it does not fit, like megcc_gfx950_conv2d does
+    when it gets no workspace"""
+    # rows of 110 pixels: the detour would need two 18.9 MB NCHW44 copies
+    case = ConvCase(A.FMT_NCHW, A.GROUP, 48, 32, 112, 110, 32, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(9)))
+    op = prepared(case, 75)
+    assert op.ws.size > SCRATCH
+    op.launch()
+    want = op.result().copy()
+    op.poison_outputs()
+    op.launch_noalloc()
+    assert np.array_equal(op.result(), want)
+    # 10 tiles x 52 K slices x 64 KiB of f32 partial sums = 34 MB
+    case = ConvCase(A.FMT_NCHW, A.DENSE, 1, 512, 14, 14, 640, 3, 1, 1, A.RELU, dtype="f32")
+    op = prepared(case, 76)
+    assert op.ws.size > SCRATCH
+    op.launch()
+    want = op.result().copy()
+    op.poison_outputs()
+    op.launch_noalloc()
+    import cases
+    assert cases.max_rel_err(op.result(), want) <= 1e-4
+
+
 def test_noalloc_layers_without_scratch_run_as_before():
     case = ConvCase(A.FMT_NCHW44, A.DENSE, 8, 64, 56, 56, 128, 3, 1, 1, A.RELU, scales=(0.02, 0.01, unsat(576)))
     op = prepared(case, 74)

@@ -11,14 +11,22 @@
 // HIP kernels behind libmegcc_gfx950.so (include/megcc_gfx950.h).
 //
 // The attribute bag is MegCC's `TContext` (compiler/include/compiler/Common/TContext.h:177-243).
-// Inside a MegCC tree define MEGCC_GFX950_IN_TREE: the reference's own headers are used and
-// the classes below derive from its KernelFunc. Stand-alone (this repository: tests, the
-// kernelgen tool) a minimal mirror with the same method names is declared here.
+// Inside a MegCC tree (this file and Gfx950Kernels.cpp dropped into compiler/lib/KernelGen/Gfx950/,
+// where "compiler/KernelGen/KernelGen.h" is on the include path, or MEGCC_GFX950_IN_TREE defined)
+// the reference's own headers are used and the classes below derive from its KernelFunc.
+// Stand-alone (this repository: tests, the kernelgen tool) a minimal mirror with the same method
+// names is declared here.
 #pragma once
 #include <cstdint>
 #include <string>
 #include <unordered_map>
 #include <vector>
+
+#if !defined(MEGCC_GFX950_IN_TREE) && defined(__has_include)
+#if __has_include("compiler/KernelGen/KernelGen.h")
+#define MEGCC_GFX950_IN_TREE 1
+#endif
+#endif
 
 #ifdef MEGCC_GFX950_IN_TREE
 #include "compiler/KernelGen/KernelGen.h"

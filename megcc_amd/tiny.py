@@ -254,8 +254,18 @@ class ModelBuilder:
     MemForward instruction per view. The plan is the PUSHDOWN plan of the operators' lifetimes
     (time step = Opr index; outputs stay alive to the end); model inputs are not in the arena."""
 
-    def __init__(self, name="model", device=DEVICE_BARE_METAL, alignment=64):
+    def __init__(self, name="model", device=DEVICE_BARE_METAL, alignment=64, kernel_table=None):
+        """kernel_table: {symbol: (kernel_id, init_id, workspace_id)}, the indices of the kernel
+        tables the TinyNN runtime was built with (kernels[] / init_kernels[] / workspace_func[] of
+        the exporter's kernels.c, compiler/lib/Target/TinyNN/KernelExporter.cpp:15-66). With a
+        table every Opr carries those ids and a workspace sized by the kernel's own _workspace
+        function, planned into the arena for the one step the Opr runs (the compiler evaluates
+        that function at compile time, compiler/lib/KernelGen/Jit/JitExe.cpp:67-123; the runtime
+        points Opr.workspace at arena + offset, runtime/src/init.c:478-484). Without a table
+        kernel_id is the Opr's position and no workspace is planned (the model runtime of this
+        library binds kernels by symbol and keeps one workspace of its own)."""
         self.name, self.device, self.alignment = name, device, alignment
+        self.kernel_table = kernel_table
         self.tensors, self.weights, self.instructions = [], [], []
         self.inputs, self.outputs = [], []
         self._root, self._first, self._last = [], [], []
@@ -317,11 +327,35 @@ class ModelBuilder:
             if self._first[r] < 0:
                 self._first[r] = k
             self._last[r] = max(self._last[r], k)
-        self.instructions.append(("Opr", dict(
+        fields = dict(
             name="%s:%d" % (symbol, k), type=symbol, inputs=[int(t) for t in inputs],
             input_types=[WEIGHT if isinstance(t, _WeightId) else TENSOR for t in inputs],
-            outputs=list(outputs), kernel_id=k)))
+            outputs=list(outputs), kernel_id=k)
+        if self.kernel_table is not None:
+            if symbol not in self.kernel_table:
+                raise KeyError("the runtime's kernel tables hold no %s" % symbol)
+            fields["kernel_id"], fields["init_id"], fields["workspace_id"] = self.kernel_table[symbol]
+            fields["workspace_size"] = self._workspace_bytes(symbol, inputs)
+        self.instructions.append(("Opr", fields))
         self._nr_opr += 1
+
+    def _workspace_bytes(self, symbol, inputs):
+        """what the kernel's _workspace function answers for these operands (shapes, dtypes and
+        scales only: no tensor memory is touched)"""
+        import ctypes as C
+
+        from . import abi, runtime
+        tensors = []
+        for t in inputs:
+            info = self.weights[t] if isinstance(t, _WeightId) else self.tensors[t]
+            kind, scale = info["dtype"]
+            tensors.append(abi.make_tensor(None, info["dims"], kind, scale if scale is not None else 1.0,
+                                           info["name"].encode(), info.get("stride")))
+        size = C.c_size_t(0)
+        desc = runtime.parse_symbol(symbol)
+        runtime.check(runtime.lib().megcc_gfx950_call_workspace(
+            C.byref(desc), abi.tensor_array(tensors), len(tensors), 1, C.byref(size)), "workspace of " + symbol)
+        return size.value
 
     def mark_input(self, t):
         self.inputs.append(t)
@@ -344,9 +378,18 @@ class ModelBuilder:
         for t in planned:
             info = self.tensors[t]
             size.append(int(np.prod(info["dims"])) * _ITEMSIZE[info["dtype"][0]])
+        # workspaces: alive for the one step of their Opr
+        with_ws = [(k, f) for k, f in enumerate(f for kind, f in self.instructions if kind == "Opr")
+                   if f.get("workspace_size", 0) > 0]
+        for k, f in with_ws:
+            begin.append(k)
+            end.append(k + 1)
+            size.append(f["workspace_size"])
         offsets, arena, _ = runtime.plan_memory(begin, end, size, self.alignment)
         for t, off in zip(planned, offsets):
             self.tensors[t]["offset"] = int(off)
+        for (k, f), off in zip(with_ws, offsets[len(planned):]):
+            f["workspace_offset"] = int(off)
         for t in range(len(self.tensors)):  # views report their root's offset
             if self._root[t] >= 0:
                 self.tensors[t]["offset"] = self.tensors[self._root_of(t)]["offset"]

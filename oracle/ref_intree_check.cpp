@@ -1,12 +1,14 @@
 // TEST INFRASTRUCTURE ONLY -- never linked into or called by the product library.
 //
-// The gfx950 KernelGen target (megcc_amd/kernelgen/Gfx950Kernels.cpp) built with
-// -DMEGCC_GFX950_IN_TREE, i.e. deriving from the reference's own KernelGen::KernelFunc
+// The gfx950 KernelGen target (megcc_amd/kernelgen/Gfx950Kernels.cpp) built in-tree, i.e.
+// deriving from the reference's own KernelGen::KernelFunc
 // (compiler/include/compiler/KernelGen/KernelGen.h:75-136) and reading the reference's own
 // TContext (compiler/include/compiler/Common/TContext.h:177-243), linked with the reference's
-// KernelGen registry compiled from the sources where they lie (oracle/Makefile). For every line
-// of a spec file (format: oracle/ref_dump.cpp) it checks what a maintainer adding
-// `Arch::GFX950` to KernelPack::GetKernel (compiler/lib/KernelGen/KernelGen.cpp:100-125) relies on:
+// KernelGen registry compiled from the sources where they lie (oracle/Makefile) - except
+// KernelGen.h / KernelGen.cpp, of which scratch copies with
+// megcc_amd/upstream/kernelgen_arch_gfx950.patch applied are compiled, so that every pack below
+// comes from the reference's own KernelPack::GetKernel(type, Arch::GFX950). For every line
+// of a spec file (format: oracle/ref_dump.cpp) it checks what that registry branch relies on:
 //   1. a gfx950 kernel is available for the context, through the reference's CodeGenContext;
 //   2. its symbol is the symbol of an available kernel of the reference's Arch::BAREMETAL list
 //      for the same context ("first" = the one the x86 build would select, "later" = a lower
@@ -96,7 +98,7 @@ int main(int argc, char** argv) {
     megcc::setAssertThrow(true);
     int bad = 0, n_first = 0, n_later = 0, n_lines = 0;
     for (auto& kv : kTypes) {
-        for (auto* k : megcc_gfx950::Gfx950KernelPack::GetKernel(kv.second)) {
+        for (auto* k : KernelGen::KernelPack::GetKernel(kv.second, KernelGen::Arch::GFX950).first) {
             std::string s = k->GetKernelSymbol(nullptr);
             if (s.empty()) {
                 printf("FAIL %s: empty symbol for a null context\n", kv.first.c_str());
@@ -144,7 +146,7 @@ int main(int argc, char** argv) {
             if (available(k, &ctx))
                 ref_syms.push_back(k->GetKernelSymbol(&ctx));
         const KernelGen::KernelFunc* mine = nullptr;
-        for (auto* k : megcc_gfx950::Gfx950KernelPack::GetKernel(it->second))
+        for (auto* k : KernelGen::KernelPack::GetKernel(it->second, KernelGen::Arch::GFX950).first)
             if (available(k, &ctx)) {
                 mine = k;
                 break;

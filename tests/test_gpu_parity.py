@@ -838,6 +838,49 @@ def test_fully_connected_sweep(case):
     compare(got, case.run_port(arrays), repr(case))
 
 
+def _f32_sweep():
+    """seeded random f32 convolutions (NCHW and NCHW44; 1x1, 3x3 with and without dilation, 5x5;
+    stride 1 / 2; any padding up to k/2 + 1; ragged channel counts and pixel counts, so that the
+    implicit GEMM's edge tiles, its last partial stage of K and the small-layer kernel's clamped
+    taps all occur) and f32 products of 5..300 rows in all four transpositions, a third of them
+    with at most 64 rows and K, N multiples of 64 / 256 (the 64 x 256 tiles with split K)"""
+    r = np.random.Generator(np.random.PCG64(99))
+    acts = [A.IDENTITY, A.RELU, A.H_SWISH, A.SIGMOID]
+    out = []
+    for i in range(50):
+        k = int(r.choice([1, 3, 3, 5]))
+        s = int(r.integers(1, 3))
+        dil = int(r.integers(1, 3)) if k == 3 else 1
+        ic, oc = int(r.integers(1, 90)), int(r.integers(1, 200))
+        ih, iw, n = int(r.integers(5, 60)), int(r.integers(5, 60)), int(r.integers(1, 9))
+        pad = int(r.integers(0, k // 2 + 2))
+        eh = dil * (k - 1) + 1
+        if ih + 2 * pad < eh or iw + 2 * pad < eh:
+            continue
+        fmt = A.FMT_NCHW
+        if i % 5 == 0:
+            ic, oc, fmt = (ic + 3) // 4 * 4, (oc + 3) // 4 * 4, A.FMT_NCHW44
+        act, bias = acts[int(r.integers(0, 4))], bool(r.integers(0, 2))
+        out.append((500 + i, ConvCase(fmt, A.DENSE, n, ic, ih, iw, oc, k, s, pad, act, dtype="f32", bias=bias,
+                                      dilate=dil)))
+    for i in range(30):
+        m, k, n = int(r.integers(5, 300)), int(r.integers(1, 700)), int(r.integers(1, 700))
+        if i % 3 == 0:
+            m, k, n = int(r.integers(5, 65)), int(r.integers(1, 40)) * 64, int(r.integers(1, 20)) * 256
+        out.append((700 + i, MatMulCase(m, k, n, trans_a=bool(r.integers(0, 2)), trans_b=bool(r.integers(0, 2)))))
+    return out
+
+
+F32_SWEEP = _f32_sweep()
+
+
+@pytest.mark.parametrize("seed,case", F32_SWEEP, ids=["%d_%r" % (s, c) for s, c in F32_SWEEP])
+def test_f32_convolution_and_matmul_sweep(seed, case):
+    port.set_threads(16)
+    arrays = case.gen(seed=seed)
+    compare(run_gpu(case, arrays), case.run_port(arrays), repr(case))
+
+
 def test_direct_kernel_when_filter_was_not_packed():
     """a caller that skips the init protocol still gets the right answer (generic kernel)"""
     import ctypes as C

@@ -37,6 +37,10 @@ bool dwconv_nchw_supported(const ConvGeom& g, const void* src, const void* dst);
 TinyNNStatus dwconv_nchw_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool conv_f32_small_supported(const ConvGeom& g);
 TinyNNStatus conv_f32_small_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+bool dwconv44_f32_supported(const ConvGeom&);
+TinyNNStatus dwconv44_f32_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+bool conv_first_f32_supported(const ConvGeom&);
+TinyNNStatus conv_first_f32_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool conv_f32_gemm_supported(const ConvGeom& g);
 TinyNNStatus conv_f32_gemm_launch(const ConvGeom&, const void*, const void*, const void*, void*,
                                   const Workspace*);
@@ -563,6 +567,16 @@ static TinyNNStatus conv2d_run(
     if (f32 && conv_f32_gemm_supported(g)) {
         note_kernel("conv_f32_gemm");
         return conv_f32_gemm_launch(g, src->ptr, flt->ptr, b, dst->ptr, workspace);
+    }
+    if (f32 && dwconv44_f32_supported(g) && aligned16(src->ptr) && aligned16(flt->ptr) && aligned16(dst->ptr) &&
+        (!b || aligned16(b))) {
+        note_kernel("dwconv44_f32", g.fh, g.sh);
+        return dwconv44_f32_launch(g, src->ptr, flt->ptr, b, dst->ptr);
+    }
+    if (f32 && conv_first_f32_supported(g) && aligned4(src->ptr) && aligned16(flt->ptr) && aligned16(dst->ptr) &&
+        (!b || aligned16(b))) {
+        note_kernel("conv_first_f32", g.fh, g.sh);
+        return conv_first_f32_launch(g, src->ptr, flt->ptr, b, dst->ptr);
     }
     note_kernel("conv_direct");
     return conv_direct_launch(g, f32, src->ptr, flt->ptr, b, dst->ptr);

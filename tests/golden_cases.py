@@ -212,4 +212,18 @@ def golden_cases():
         A.FMT_NCHW44, A.GROUP, 1, 4, 10, 9, 4, 7, 1, 3, A.IDENTITY, scales=(0.02, 0.01, unsat(49)))
     c["conv44_5x5_H_SWISH"] = ConvCase(
         A.FMT_NCHW44, A.DENSE, 2, 8, 9, 7, 8, 5, 1, 2, A.H_SWISH, scales=(0.02, 0.01, unsat(200)))
+    # f32 first layers (NCHW source, NCHW44 result: GeneralIntrinsic/ConvKernel/Fp32ConvNchwNchw44.cpp)
+    # and f32 channel-wise layers in NCHW44 (Fp32ChannelWiseMk4.cpp: 3x3 and 5x5, stride 1 and 2)
+    c["conv_hybrid_f32_3x3_s2_RELU"] = ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 11, 9, 8, 3, 2, 1, A.RELU, dtype="f32")
+    c["conv_hybrid_f32_3x3_s1_H_SWISH"] = ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 9, 8, 12, 3, 1, 1, A.H_SWISH,
+                                                   dtype="f32")
+    c["conv_hybrid_f32_5x5_s2_IDENTITY"] = ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 1, 12, 10, 4, 5, 2, 2, A.IDENTITY,
+                                                    dtype="f32")
+    c["conv_hybrid_f32_7x7_s2_RELU_nobias"] = ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 3, 17, 15, 8, 7, 2, 3, A.RELU,
+                                                       dtype="f32", bias=False)
+    c["dw44_f32_3x3_s1_RELU"] = ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 9, 7, 8, 3, 1, 1, A.RELU, dtype="f32")
+    c["dw44_f32_3x3_s2_IDENTITY"] = ConvCase(A.FMT_NCHW44, A.GROUP, 2, 8, 9, 7, 8, 3, 2, 1, A.IDENTITY, dtype="f32")
+    c["dw44_f32_5x5_s1_H_SWISH"] = ConvCase(A.FMT_NCHW44, A.GROUP, 1, 12, 10, 11, 12, 5, 1, 2, A.H_SWISH, dtype="f32")
+    c["dw44_f32_5x5_s2_RELU_nobias"] = ConvCase(A.FMT_NCHW44, A.GROUP, 2, 4, 11, 13, 4, 5, 2, 2, A.RELU, dtype="f32",
+                                                bias=False)
     return c

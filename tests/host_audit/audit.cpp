@@ -12,6 +12,8 @@
 //   mm     M K N ta tb lda_pad ldb_pad ws     f32 MatMul through megcc_gfx950_matmul (gemm / gevm); ws = 1: with split-K room
 //   conv   n ic ih iw oc k s p d bias ws      f32 NCHW convolution through the implicit GEMM
 //   small  n ic ih iw oc k s p d bias         f32 NCHW convolution through conv_f32_small (k = 1 or 3)
+//   dwf32  n c ih iw k s p bias               f32 channel-wise layer in NCHW44
+//   first  n ic ih iw oc k s p bias           f32 first layer, NCHW source -> NCHW44 result
 //   fcone  M K OC packed_bytes bias           qsi8 FullyConnected, M <= 64, one launch
 //   fcgevm M K OC packed_bytes bias           qsi8 FullyConnected, M <= 4
 #include <hip/hip_runtime.h>
@@ -62,6 +64,10 @@ size_t conv_f32_gemm_workspace_bytes(const ConvGeom& g);
 TinyNNStatus conv_f32_gemm_launch(const ConvGeom&, const void*, const void*, const void*, void*, const Workspace*);
 bool conv_f32_small_supported(const ConvGeom& g);
 TinyNNStatus conv_f32_small_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+bool dwconv44_f32_supported(const ConvGeom&);
+TinyNNStatus dwconv44_f32_launch(const ConvGeom&, const void*, const void*, const void*, void*);
+bool conv_first_f32_supported(const ConvGeom&);
+TinyNNStatus conv_first_f32_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool fc_one_supported(const ConvGeom& g, const void* src);
 TinyNNStatus fc_one_launch(const ConvGeom&, const void*, const void*, const void*, void*);
 bool fc_gevm_q8_supported(const ConvGeom& g);
@@ -170,6 +176,38 @@ static bool run_case(const std::string& line, bool at_end) {
         Fenced W(wsb ? wsb : 16, at_end, 16);
         Workspace w = {wsb ? W.ptr : nullptr, wsb, 0};
         return conv_f32_gemm_launch(g, src.ptr, flt.ptr, bias ? b.ptr : nullptr, dst.ptr, &w) == TinyNN_SUCCESS;
+    }
+    if (kind == "dwf32" || kind == "first") {
+        ConvGeom g;
+        memset(&g, 0, sizeof(g));
+        int k, s, p, bias;
+        ss >> g.n >> g.ic >> g.ih >> g.iw;
+        if (kind == "first")
+            ss >> g.oc;
+        else
+            g.oc = g.ic;
+        ss >> k >> s >> p >> bias;
+        g.fh = g.fw = k, g.sh = g.sw = s, g.ph = g.pw = p, g.dh = g.dw = 1;
+        g.oh = (g.ih + 2 * p - k) / s + 1;
+        g.ow = (g.iw + 2 * p - k) / s + 1;
+        g.groups = kind == "first" ? 1 : g.ic;
+        g.fmt = kind == "first" ? MEGCC_FMT_NCHW_NCHW44 : MEGCC_FMT_NCHW44;
+        g.act = MEGCC_NONLINE_H_SWISH, g.has_bias = bias;
+        const size_t taps = (size_t)k * k * (kind == "first" ? (size_t)g.ic * g.oc : (size_t)g.ic);
+        Fenced src((size_t)g.n * g.ic * g.ih * g.iw * 4, at_end, 16), flt(taps * 4, at_end, 16),
+                b((size_t)g.oc * 4, at_end, 16), dst((size_t)g.n * g.oc * g.oh * g.ow * 4, at_end, 16);
+        if (kind == "first") {
+            if (!conv_first_f32_supported(g)) {
+                fprintf(stderr, "not a conv_first_f32 layer: %s\n", line.c_str());
+                return false;
+            }
+            return conv_first_f32_launch(g, src.ptr, flt.ptr, bias ? b.ptr : nullptr, dst.ptr) == TinyNN_SUCCESS;
+        }
+        if (!dwconv44_f32_supported(g)) {
+            fprintf(stderr, "not a dwconv44_f32 layer: %s\n", line.c_str());
+            return false;
+        }
+        return dwconv44_f32_launch(g, src.ptr, flt.ptr, bias ? b.ptr : nullptr, dst.ptr) == TinyNN_SUCCESS;
     }
     if (kind == "fcone" || kind == "fcgevm") {
         ConvGeom g;

@@ -81,9 +81,9 @@ def test_parse_f32_nchw44_symbols_of_the_general_intrinsic_pack():
         with pytest.raises(runtime.MegccError):
             runtime.parse_symbol(base + bad)
     a = runtime.parse_symbol(
-        "GI_kernel_conv2d_3x3_NCHW44_DENSE_p1x1_s2x2_d1x1_f32f32f32f32_bias_H_SWISH_nchw_nchw44_oc32_ic3").attr.conv
+        "GI_kernel_conv2d_3x3_NCHW_NCHW44_DENSE_p1x1_s2x2_d1x1_f32f32f32f32_bias_H_SWISH_nchw_nchw44_oc32_ic3").attr.conv
     assert (a.format, a.stride_h, a.pad_w, a.nonline, a.with_bias) == (abi.FMT_NCHW_NCHW44, 2, 1, abi.H_SWISH, 1)
-    a = runtime.parse_symbol("GI_kernel_conv2d_5x5_NCHW44_DENSE_p2x2_s1x1_d1x1_f32f32f32f32_nchw_nchw44_oc8_ic1").attr.conv
+    a = runtime.parse_symbol("GI_kernel_conv2d_5x5_NCHW_NCHW44_DENSE_p2x2_s1x1_d1x1_f32f32f32_nchw_nchw44_oc8_ic1").attr.conv
     assert (a.format, a.kernel_w, a.with_bias, a.nonline) == (abi.FMT_NCHW_NCHW44, 5, 0, abi.IDENTITY)
     a = runtime.parse_symbol("GI_chanwise_kernel_conv2d_5x5_NCHW44_GROUP_p2x2_s2x2_d1x1_f32f32f32f32_bias_RELU").attr.conv
     assert (a.format, a.sparse, a.kernel_h, a.stride_w, a.nonline) == (abi.FMT_NCHW44, abi.GROUP, 5, 2, abi.RELU)

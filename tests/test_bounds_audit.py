@@ -1,6 +1,6 @@
 """Host-side bounds audit of the kernels that issue their loads unconditionally from clamped
-indices (gemm_f32: all four transpositions and the implicit-GEMM gather; gevm_f32; conv_f32_small;
-fc_one32 / fc_one; fc_gevm_q8). tests/host_audit/audit.cpp links the library's own kernel sources,
+indices (gemm_f32: all four transpositions and the implicit-GEMM gather; gevm_f32; conv_f32_small; the
+f32 NCHW44 channel-wise and first-layer kernels; fc_one32 / fc_one; fc_gevm_q8). tests/host_audit/audit.cpp links the library's own kernel sources,
 compiled as host C++ against a stand-in HIP header that runs every thread of every workgroup on
 the CPU, and fences each operand buffer with inaccessible pages: one element outside a tensor ends
 the run. No GPU involved; the shapes are every case of the GPU sweeps plus a seeded sweep of ragged
@@ -20,7 +20,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 AUDIT_DIR = os.path.join(HERE, "host_audit")
 CSRC = os.path.join(os.path.dirname(HERE), "megcc_amd", "csrc")
 CLANG = "/opt/rocm/llvm/bin/clang++"
-SOURCES = ["gemm_f32", "gevm_f32", "conv_f32_small", "fc_stream", "fc_gevm_q8"]
+SOURCES = ["gemm_f32", "gevm_f32", "conv_f32_small", "conv_f32_nchw44", "fc_stream", "fc_gevm_q8"]
 
 pytestmark = pytest.mark.skipif(not os.path.exists(CLANG), reason="needs ROCm's clang++ for the kernels' vector types")
 
@@ -120,6 +120,30 @@ def audit_lines():
                                             (1, 32, 56, 56, 32, 3, 1, 1, 1), (3, 7, 9, 11, 13, 3, 1, 2, 2), (1, 5, 2, 2, 3, 3, 1, 1, 1),
                                             (4, 9, 17, 3, 6, 1, 2, 0, 1), (1, 64, 13, 13, 66, 3, 1, 0, 1), (5, 2, 8, 64, 3, 3, 2, 1, 2)]:
         lines.append("small %d %d %d %d %d %d %d %d %d 1" % (n, ic, ih, iw, oc, k, s, p, d))
+    # f32 NCHW44: channel-wise tiles of 4 x 64 pixels with halos, first layers of 256-pixel blocks
+    for _, case in gp.F32_NCHW44:
+        if case.sparse == abi.GROUP and case.fh in (3, 5):
+            lines.append("dwf32 %d %d %d %d %d %d %d %d" % (case.n, case.ic, case.ih, case.iw, case.fh, case.sh,
+                                                          case.ph, int(case.bias)))
+        elif case.fmt == abi.FMT_NCHW_NCHW44:
+            lines.append("first %d %d %d %d %d %d %d %d %d" % (case.n, case.ic, case.ih, case.iw, case.oc, case.fh,
+                                                             case.sh, case.ph, int(case.bias)))
+    for i in range(16):
+        k, s = int(r.choice([3, 5])), int(r.integers(1, 3))
+        ih, iw = int(r.integers(1, 20)), int(r.choice([1, 2, 63, 64, 65, 127, 129, 200]))
+        p = int(r.integers(0, k // 2 + 2))
+        if ih + 2 * p < k or iw + 2 * p < k:
+            continue
+        lines.append("dwf32 %d %d %d %d %d %d %d %d" % (r.integers(1, 4), 4 * r.integers(1, 5), ih, iw, k, s, p,
+                                                      r.integers(0, 2)))
+    for i in range(12):
+        k, s = int(r.choice([3, 5, 7])), int(r.integers(1, 3))
+        ih, iw = int(r.integers(3, 40)), int(r.integers(3, 70))
+        p = int(r.integers(0, k // 2 + 2))
+        if ih + 2 * p < k or iw + 2 * p < k:
+            continue
+        lines.append("first %d %d %d %d %d %d %d %d %d" % (r.integers(1, 4), r.integers(1, 5), ih, iw,
+                                                         4 * r.choice([1, 2, 8, 9, 16]), k, s, p, r.integers(0, 2)))
     # qsi8 FullyConnected: 1..64 rows, K = 1..32 blocks of 128 (and beyond 4096), channel counts off every tile size
     for i in range(24):
         m = int(r.choice([1, 2, 3, 4, 5, 31, 32, 33, 63, 64]))

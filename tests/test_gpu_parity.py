@@ -345,6 +345,39 @@ def test_matches_oracle(case):
     compare(got, want, repr(case))
 
 
+F32_NCHW44 = [
+    # f32 channel-wise layers in NCHW44 (the reference's GI_chanwise kernels: 3x3 / 5x5, stride 1 / 2):
+    # tiles of 4 x 64 pixels - extents below, at and above a tile, padding 0 .. k/2 + 1, every activation
+    ("dwconv44_f32", ConvCase(A.FMT_NCHW44, A.GROUP, 3, 32, 56, 56, 32, 3, 1, 1, A.RELU, dtype="f32")),
+    ("dwconv44_f32", ConvCase(A.FMT_NCHW44, A.GROUP, 2, 16, 57, 131, 16, 3, 2, 1, A.IDENTITY, dtype="f32")),
+    ("dwconv44_f32", ConvCase(A.FMT_NCHW44, A.GROUP, 2, 24, 28, 28, 24, 5, 1, 2, A.H_SWISH, dtype="f32")),
+    ("dwconv44_f32", ConvCase(A.FMT_NCHW44, A.GROUP, 1, 8, 30, 65, 8, 5, 2, 2, A.SIGMOID, dtype="f32", bias=False)),
+    ("dwconv44_f32", ConvCase(A.FMT_NCHW44, A.GROUP, 5, 4, 3, 2, 4, 3, 1, 1, A.RELU, dtype="f32")),
+    ("dwconv44_f32", ConvCase(A.FMT_NCHW44, A.GROUP, 2, 12, 9, 70, 12, 3, 1, 0, A.RELU, dtype="f32")),
+    ("dwconv44_f32", ConvCase(A.FMT_NCHW44, A.GROUP, 2, 12, 13, 64, 12, 5, 1, 3, A.IDENTITY, dtype="f32")),
+    ("dwconv44_f32", ConvCase(A.FMT_NCHW44, A.GROUP, 1, 8, 1, 1, 8, 3, 2, 1, A.RELU, dtype="f32")),
+    # (a 7x7 window is none of the reference's four variants: the one-output-per-thread kernel)
+    ("conv_direct", ConvCase(A.FMT_NCHW44, A.GROUP, 1, 8, 12, 11, 8, 7, 1, 3, A.RELU, dtype="f32")),
+    # f32 first layers, NCHW source -> NCHW44 result (the reference's GI nchw_nchw44 kernel)
+    ("conv_first_f32", ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 64, 64, 32, 3, 2, 1, A.RELU, dtype="f32")),
+    ("conv_first_f32", ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 37, 41, 64, 7, 2, 3, A.RELU, dtype="f32")),
+    ("conv_first_f32", ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 1, 30, 29, 8, 5, 1, 2, A.H_SWISH, dtype="f32")),
+    ("conv_first_f32", ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 3, 4, 17, 300, 40, 3, 1, 0, A.IDENTITY, dtype="f32",
+                                bias=False)),
+    ("conv_first_f32", ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 1, 2, 5, 4, 4, 3, 2, 2, A.SIGMOID, dtype="f32")),
+    ("conv_first_f32", ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 20, 20, 36, 3, 1, 1, A.RELU, dtype="f32")),
+]
+
+
+@pytest.mark.parametrize("kernel,case", F32_NCHW44, ids=[repr(c) for _, c in F32_NCHW44])
+def test_f32_channel_wise_and_first_layers_in_nchw44(kernel, case):
+    port.set_threads(8)
+    arrays = case.gen(seed=13)
+    got = run_gpu(case, arrays)
+    assert runtime.last_kernel().startswith(kernel), runtime.last_kernel()
+    compare(got, case.run_port(arrays), repr(case))
+
+
 F32_POINTWISE = [
     # f32 elementwise: the FullyConnected bias [M,N] + [N] / [1,N] at the sizes of the MatMul
     # configurations, the softmax steps ([A,N] op [A,1]), every other way two operands meet

@@ -52,7 +52,12 @@ def test_port_matches_golden(name):
 def test_symbol_mirror(name):
     """our reading of the reference's symbol scheme against what its registry actually chose"""
     case = CASES[name]
-    if isinstance(case, ConvCase) and case.dtype == "f32" and case.fmt == abi.FMT_NCHW44:
+    if isinstance(case, ConvCase) and case.dtype == "f32" and case.fmt == abi.FMT_NCHW_NCHW44:
+        # the GI first-layer kernel: our reading of the name + its own suffix
+        assert SYMBOLS[name] == "GI_%s_nchw_nchw44_oc%d_ic%d" % (case.symbol(), case.oc, case.ic)
+    elif isinstance(case, ConvCase) and case.dtype == "f32" and case.sparse == abi.GROUP:
+        assert SYMBOLS[name] == "GI_chanwise_" + case.symbol()
+    elif isinstance(case, ConvCase) and case.dtype == "f32" and case.fmt == abi.FMT_NCHW44:
         # the registry's first choice for f32 NCHW44: Winograd F(2,3) for 3x3, the 1x1 kernel
         assert SYMBOLS[name].startswith(("GI_kernel_conv2d_3x3_NCHW44_DENSE", "GI_kernel_conv2d_conv1x1_NCHW44"))
     elif isinstance(case, ConvCase) and case.dtype == "f32":

@@ -114,11 +114,18 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
     // L2 instead of two or three.
     const int nb = gridDim.x;
     const int lb = (nb & 7) == 0 ? (blockIdx.x & 7) * (nb >> 3) + (blockIdx.x >> 3) : blockIdx.x;
-    // wave -> (plane set, first tile, tile step): the grid holds a multiple of c4n waves
+    // wave -> (plane set, a run of consecutive tiles): the grid holds a multiple of c4n waves. A
+    // tile is 256 output pixels along the rows - 2.3 rows of a 112-pixel map - and reads one row
+    // more above and below, which the tile after it reads again: walking its run tile by tile, a
+    // wave finds those rows in its XCD's L2 two microseconds after it fetched them. (Tiles dealt
+    // round-robin to the waves of a plane set left the re-read to another wave at another time:
+    // on N=64 C=512 112x112, whose 411 MB no cache holds, 1.82 times the input came from HBM.)
     const int gw = lb * 4 + (tid >> 6);
     const int nw = gridDim.x * 4;
     const int c4 = gw % q.c4n;
-    const int tstep = nw / q.c4n;
+    const int wps = nw / q.c4n;                     // waves per plane set
+    const int run = (q.tiles + wps - 1) / wps;      // tiles per wave
+    const int t_end = min((gw / q.c4n + 1) * run, q.tiles);
 
     // ---- the banded weight matrices of this plane set -------------------------------------------
     // row m = lane & 31 = (output pixel m / 4, channel m % 4); the lane's 16 K bytes are input
@@ -222,9 +229,9 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
     };
 
     v4i B[IR][NS];
-    int tile = gw / q.c4n;
-    Where next = request(tile, B);
-    for (; tile < q.tiles; tile += tstep) {
+    int tile = (gw / q.c4n) * run;
+    Where next = request(tile < t_end ? tile : q.tiles, B);
+    for (; tile < t_end; ++tile) {
         const Where cur = next;
         v16i acc[R];
 #pragma unroll
@@ -238,7 +245,7 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
         }
         // the operands are consumed: the next tile's loads fly while this one is requantised
         // (past the last tile every offset is out of range and nothing is fetched)
-        next = request(tile + tstep, B);
+        next = request(tile + 1 < t_end ? tile + 1 : q.tiles, B);
         if constexpr (FUSE != 0) {
             // ---- pool, requantise, add, store ----------------------------------------------------
             // With the threshold table the requantisation F is a non-decreasing function of the

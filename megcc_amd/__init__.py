@@ -9,7 +9,8 @@ import os
 import subprocess
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(PKG_DIR, "libmegcc_gfx950.so")
+# (MEGCC_GFX950_LIB: another build of the same library, e.g. one made with EXTRA_FLAGS for an experiment)
+LIB_PATH = os.environ.get("MEGCC_GFX950_LIB") or os.path.join(PKG_DIR, "libmegcc_gfx950.so")
 
 
 def build(jobs=8):

@@ -670,7 +670,7 @@ TinyNNStatus conv_mfma_launch(
     q.sps = q.stages;
     q.partial = nullptr;
     if (pipe) {
-        note_kernel("conv_mfma_i8_dma", picked, pc.bm, pc.bn, q.Lmax, pc.ks);
+        note_kernel(pc.m16 ? "conv_mfma_i8_dma_m16" : "conv_mfma_i8_dma", picked, pc.bm, pc.bn, q.Lmax, pc.ks);
         return conv_mfma_pipe_launch(pc, q);
     }
     const int split = conv_mfma_split(g);

@@ -636,6 +636,12 @@ OLDER = [
                                scales=(0.02, 0.01, 0.05))),
     ("nopm", ConvCase(A.FMT_NCHW44, A.DENSE, 6, 32, 56, 56, 160, 3, 1, 1, A.RELU,
                             scales=(0.02, 0.01, unsat(288)))),
+    # the 32 x 32 x 32 MFMA form of the plane-major 3x3 kernel (the default is 16 x 16 x 64):
+    # ragged channel tile, three chunks of input channels, rows of 60 pixels
+    ("nom16", ConvCase(A.FMT_NCHW44, A.DENSE, 9, 96, 56, 60, 200, 3, 1, 1, A.H_SWISH,
+                       scales=(0.02, 0.01, unsat(864)))),
+    ("nom16", ConvCase(A.FMT_NCHW44, A.DENSE, 16, 64, 56, 56, 128, 3, 1, 1, A.IDENTITY,
+                       scales=(0.02, 0.01, unsat(576)))),
     ("nodma512", ConvCase(A.FMT_NCHW44, A.DENSE, 22, 64, 54, 57, 128, 3, 1, 1, A.RELU,
                                 scales=(0.02, 0.01, unsat(576)))),
     ("nogevm", ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY,

@@ -1,5 +1,5 @@
 // Shared host-side helpers of libmegcc_gfx950.so: error reporting, the library stream, Tensor
-// inspection. Everything here is host code; device helpers live in epilogue.h.
+// inspection. Host code, plus the tile-order helper the tiled kernels share; the other device helpers live in epilogue.h.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -23,12 +23,46 @@ TinyNNStatus fail(TinyNNStatus st, const char* fmt, ...) __attribute__((format(p
             return ::mg::fail(st, __VA_ARGS__); \
     } while (0)
 
+// Tile order of a 2-D grid of gx x gy workgroups for the chip's eight XCDs. Workgroups are handed to
+// the XCDs in turn (workgroup i runs on XCD i % 8) and every XCD has an L2 of its own, so with the
+// plain order each XCD touches every row panel of one operand. Here workgroup i takes place
+// (i % 8) * (gx * gy / 8) + i / 8 in an order that walks the grid in strips of `w` columns, row by
+// row inside a strip: the eighth of the tiles one XCD owns is then a compact rectangle and each
+// operand panel is fetched by the one or two XCDs that need it. w = 0 (or a tile count that is no
+// multiple of 8) keeps the plain order. Any w >= 1 gives a bijection.
+struct XcdOrder {
+    int w;
+};
+inline XcdOrder make_xcd_order(int gx, int gy) {
+    const long nb = (long)gx * gy;
+    if (nb < 64 || (nb & 7) != 0)
+        return {0};
+    // w ~ sqrt(tiles per XCD / 2): the half of its share an XCD has resident at a time is about square
+    // (a round of workgroups streams its panels through the 4 MB L2 once; the next round starts over)
+    int w = 1;
+    while ((long)w * w * 8 <= nb / 8)
+        w *= 2;
+    return {w < gx ? w : gx};
+}
+__device__ __forceinline__ void xcd_tile(XcdOrder o, int bx, int by, int gx, int gy, int& tx, int& ty) {
+    tx = bx;
+    ty = by;
+    if (o.w == 0)
+        return;
+    const int nb = gx * gy, lb = by * gx + bx;
+    const int place = (lb & 7) * (nb >> 3) + (lb >> 3);
+    const int strip = place / (o.w * gy), rem = place - strip * (o.w * gy);
+    const int w = min(o.w, gx - strip * o.w);
+    ty = rem / w;
+    tx = strip * o.w + rem - ty * w;
+}
+
 // Kernel-selection overrides: each one takes a kernel (or a variant of one) out of the dispatch so
 // that the regression tests can reach the kernels that serve the shapes behind it. Read from the
 // environment (MEGCC_NOPWS=1, ...) ONCE, when the library first consults them; later changes go
 // through megcc_gfx950_set_option(). Nothing on a launch path scans the environment.
 struct Options {
-    bool no_pws, no_gevm, no_fcb, no_small, no_pm768, no_pm, no_dma512, no_pm256, no_dma, no_fcs, no_pwshare, no_hybrid, no_dot4, no_f32small, dw_generic, no_dwmfma, no_dwnchw, no_fuse_softmax, no_graph, no_poolrows, no_firstmfma, no_rowsplit, no_fuse_chain, no_fcone, no_m16;
+    bool no_pws, no_gevm, no_fcb, no_small, no_pm768, no_pm, no_dma512, no_pm256, no_dma, no_fcs, no_pwshare, no_hybrid, no_dot4, no_f32small, dw_generic, no_dwmfma, no_dwnchw, no_fuse_softmax, no_graph, no_poolrows, no_firstmfma, no_rowsplit, no_fuse_chain, no_fcone, no_m16, no_xcdorder;
 };
 Options& options();
 

@@ -44,6 +44,7 @@ struct MfmaParams {
     // int32 sums to partial[z][P][round_up(OC,4)]; conv_mfma_reduce_kernel finishes
     int split, sps;
     int32_t* partial;
+    XcdOrder xo;  // FullyConnected tiles of the LDS-direct kernel: tile order (set at launch)
     FastDiv dOW, dOH, dVW, dVH, dL, dOHW;
     // exact requantisation thresholds for IDENTITY / RELU (built on the host, epilogue.h); only
     // the kernels that look outputs up in LDS read it
@@ -151,6 +152,7 @@ struct PipeConfig {
     int pm = 0;          // plane-major activation patch (virtual rows padded to a multiple of 4)
     int rs = 0;          // a stage is ONE filter row of a 32-channel chunk (filters of more than 9 taps)
     int m16 = 0;         // 16 x 16 x 64 MFMA tiles (3x3 layers with the plane-major patch)
+    int fcb = 0;         // FullyConnected with 16-byte activation loads (K a multiple of 128)
     const void* kernel;
 };
 

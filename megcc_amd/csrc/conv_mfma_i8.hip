@@ -670,7 +670,12 @@ TinyNNStatus conv_mfma_launch(
     q.sps = q.stages;
     q.partial = nullptr;
     if (pipe) {
-        note_kernel(pc.m16 ? "conv_mfma_i8_dma_m16" : "conv_mfma_i8_dma", picked, pc.bm, pc.bn, q.Lmax, pc.ks);
+        // (FullyConnected tiles: each XCD a compact rectangle of the tile grid, common.h)
+        q.xo = pc.fcb && !options().no_xcdorder
+                       ? make_xcd_order((q.P + q.range_len - 1) / q.range_len, (q.OC + pc.bm - 1) / pc.bm)
+                       : XcdOrder{0};
+        note_kernel(pc.m16 ? "conv_mfma_i8_dma_m16" : q.xo.w ? "conv_mfma_i8_dma_xo" : "conv_mfma_i8_dma", picked,
+                    pc.bm, pc.bn, q.Lmax, pc.ks);
         return conv_mfma_pipe_launch(pc, q);
     }
     const int split = conv_mfma_split(g);

@@ -109,8 +109,13 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     // (waves w and w + 4 share a SIMD: give them different pixel columns, so that the wave with
     //  one column more in a ragged sub-tile does not meet its twin on the same SIMD)
     const int wm = wave / WGN, wn = (wave + wm) % WGN, kg = lane >> 5;
-    const int oc0 = blockIdx.y * DM_BM;
-    const int range0 = blockIdx.x * q.range_len;
+    // (FCB: both operands are matrices of many panels, so each XCD gets a compact rectangle of
+    //  tiles; for convolutions the order made no difference - two or four channel tiles per range)
+    int tile_x = blockIdx.x, tile_y = blockIdx.y;
+    if constexpr (FCB)
+        xcd_tile(q.xo, blockIdx.x, blockIdx.y, gridDim.x, gridDim.y, tile_x, tile_y);
+    const int oc0 = tile_y * DM_BM;
+    const int range0 = tile_x * q.range_len;
     const int range1 = min(range0 + q.range_len, q.P);
     const int stages = q.stages;
     const int n_tiles = (range1 - range0 + DM_BNP - 1) / DM_BNP;
@@ -635,6 +640,7 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.pm = PM ? 1 : 0;
     c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + (DM_BM > 128 ? DM_BM : 128) * 4 + (M16 ? 64 * DM_NBUF : 0);
     c.m16 = M16 ? 1 : 0;
+    c.fcb = FCB ? 1 : 0;
     c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM, false, M16>;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
         c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM, false, M16>;

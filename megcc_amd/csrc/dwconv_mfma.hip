@@ -103,10 +103,6 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
     constexpr int IR = (R - 1) * S + F;  // input rows they read
     __shared__ int tbl[REQUANT_TABLE_ENTRIES];
     const int tid = threadIdx.x, lane = tid & 63;
-    if (ACT >= 0) {
-        tbl[tid] = q.table.t[tid];
-        __syncthreads();
-    }
     const int col_l = lane & 31, kg = lane >> 5;
     // Workgroups are handed to the 8 XCDs in turn and every XCD has an L2 of its own: workgroup b
     // takes the place b % 8 * (blocks / 8) + b / 8 in tile order, so that an XCD walks a contiguous
@@ -120,54 +116,13 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
     // wave finds those rows in its XCD's L2 two microseconds after it fetched them. (Tiles dealt
     // round-robin to the waves of a plane set left the re-read to another wave at another time:
     // on N=64 C=512 112x112, whose 411 MB no cache holds, 1.82 times the input came from HBM.)
-    const int gw = lb * 4 + (tid >> 6);
+    const int gw = lb * 4 + __builtin_amdgcn_readfirstlane(tid >> 6);  // (scalar: the plane set's weights and bias come through the scalar cache)
     const int nw = gridDim.x * 4;
     const int c4 = gw % q.c4n;
     const int wps = nw / q.c4n;                     // waves per plane set
     const int run = (q.tiles + wps - 1) / wps;      // tiles per wave
     const int t_end = min((gw / q.c4n + 1) * run, q.tiles);
 
-    // ---- the banded weight matrices of this plane set -------------------------------------------
-    // row m = lane & 31 = (output pixel m / 4, channel m % 4); the lane's 16 K bytes are input
-    // pixels 4 * kg + j (j = 0..3) of the K step, 4 channel bytes each. K step s starts 4 pixels
-    // left of S * x0, so input pixel (s, j) meets output pixel px through filter column
-    // fw = 8 * s + 4 * kg + j - 4 - S * px + PAD.
-    v4i A[F][NS];
-    {
-        const int px = col_l >> 2, ch = col_l & 3;
-        const unsigned keep = 0xffu << (8 * ch);
-        const uint32_t* w = q.flt + (size_t)c4 * (F * F);
-#pragma unroll
-        for (int dy = 0; dy < F; ++dy) {
-            unsigned wr[F];
-#pragma unroll
-            for (int k = 0; k < F; ++k)
-                wr[k] = w[dy * F + k] & keep;
-#pragma unroll
-            for (int s = 0; s < NS; ++s)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int fw = 8 * s + 4 * kg + j - 4 + PAD - S * px;
-                    unsigned v = 0;
-#pragma unroll
-                    for (int k = 0; k < F; ++k)
-                        v = fw == k ? wr[k] : v;
-                    A[dy][s][j] = (int)v;
-                }
-        }
-    }
-    v16i biasv;
-    {
-        int b4[4] = {0, 0, 0, 0};
-        if (q.bias) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                b4[c] = q.bias[c4 * 4 + c];
-        }
-#pragma unroll
-        for (int e = 0; e < 16; ++e)
-            biasv[e] = b4[e & 3];
-    }
     const __amdgpu_buffer_rsrc_t rs =
             __builtin_amdgcn_make_buffer_rsrc((void*)q.src, 0, q.src_bytes, 0x00020000);
     const int OOB = (int)0x80000000u;
@@ -228,9 +183,57 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
         return w;
     };
 
+    // The first tile's rows are requested before anything else is fetched: the threshold table, the
+    // weights and the bias then travel in the same memory round trip instead of one each in front
+    // of it (a 14 x 14 layer gives a wave two tiles, so the set-up is a third of its life).
     v4i B[IR][NS];
     int tile = (gw / q.c4n) * run;
     Where next = request(tile < t_end ? tile : q.tiles, B);
+    if (ACT >= 0) {
+        tbl[tid] = q.table.t[tid];
+        __syncthreads();
+    }
+    // ---- the banded weight matrices of this plane set -------------------------------------------
+    // row m = lane & 31 = (output pixel m / 4, channel m % 4); the lane's 16 K bytes are input
+    // pixels 4 * kg + j (j = 0..3) of the K step, 4 channel bytes each. K step s starts 4 pixels
+    // left of S * x0, so input pixel (s, j) meets output pixel px through filter column
+    // fw = 8 * s + 4 * kg + j - 4 - S * px + PAD.
+    v4i A[F][NS];
+    {
+        const int px = col_l >> 2, ch = col_l & 3;
+        const unsigned keep = 0xffu << (8 * ch);
+        const uint32_t* w = q.flt + (size_t)c4 * (F * F);
+#pragma unroll
+        for (int dy = 0; dy < F; ++dy) {
+            unsigned wr[F];
+#pragma unroll
+            for (int k = 0; k < F; ++k)
+                wr[k] = w[dy * F + k] & keep;
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int fw = 8 * s + 4 * kg + j - 4 + PAD - S * px;
+                    unsigned v = 0;
+#pragma unroll
+                    for (int k = 0; k < F; ++k)
+                        v = fw == k ? wr[k] : v;
+                    A[dy][s][j] = (int)v;
+                }
+        }
+    }
+    v16i biasv;
+    {
+        int b4[4] = {0, 0, 0, 0};
+        if (q.bias) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                b4[c] = q.bias[c4 * 4 + c];
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            biasv[e] = b4[e & 3];
+    }
     for (; tile < t_end; ++tile) {
         const Where cur = next;
         v16i acc[R];
@@ -423,6 +426,9 @@ static TinyNNStatus dwconv44_mfma_run(
     long per_set = items <= cap ? q.tiles : cap / q.c4n;
     if (per_set < 1)
         per_set = 1;
+    // (no more waves than have a run of tiles: 56 tiles over 32 waves are runs of 2 for 28 of them)
+    const long run = (q.tiles + per_set - 1) / per_set;
+    per_set = (q.tiles + run - 1) / run;
     long waves = per_set * q.c4n;
     while (waves & 3) {  // (c4n odd: add whole rounds of plane sets until workgroups are full)
         waves += q.c4n;

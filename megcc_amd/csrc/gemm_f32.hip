@@ -42,6 +42,7 @@ struct GemmArgs {
     // partial[z][M][N]; gemm_f32_reduce_kernel adds them in z order (deterministic) and stores
     int split, kchunk;
     float* partial;
+    XcdOrder xo;  // tile order (set at launch from the grid)
 };
 
 __device__ __forceinline__ float act_rt(int act, float x) {
@@ -82,7 +83,11 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(GemmArgs q) {
     __shared__ __attribute__((aligned(16))) float Bs[2][GBK][BN + GPAD];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = BM == 128 ? wave >> 1 : 0, wn = BM == 128 ? wave & 1 : wave;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    // (each XCD owns a compact rectangle of tiles: with the plain order every XCD fetched every
+    //  row panel of A - 3.7 times the matrices' bytes from memory for 4096 x 4096 x 4096)
+    int tile_x, tile_y;
+    xcd_tile(q.xo, blockIdx.x, blockIdx.y, gridDim.x, gridDim.y, tile_x, tile_y);
+    const int m0 = tile_y * BM, n0 = tile_x * BN;
 
     v16f acc[2][2], tot[LONGK ? 2 : 1][LONGK ? 2 : 1];
 #pragma unroll
@@ -500,12 +505,14 @@ TinyNNStatus conv_f32_gemm_launch(
     const bool longk = q.kchunk > 1024;
     if (q.M <= 64 && (long)((q.N + 255) / 256) * q.split >= 128) {
         dim3 grid((q.N + 255) / 256, 1, q.split);
+        q.xo = options().no_xcdorder ? XcdOrder{0} : make_xcd_order((int)grid.x, (int)grid.y);
         if (longk)
             hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 64, true>), grid, dim3(256), 0, stream(), q);
         else
             hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 64>), grid, dim3(256), 0, stream(), q);
     } else {
         dim3 grid((q.N + GBN - 1) / GBN, (q.M + GBM - 1) / GBM, q.split);
+        q.xo = options().no_xcdorder ? XcdOrder{0} : make_xcd_order((int)grid.x, (int)grid.y);
         if (longk)
             hipLaunchKernelGGL((gemm_f32_kernel<true, true, true, 128, true>), grid, dim3(256), 0, stream(), q);
         else
@@ -574,9 +581,10 @@ extern "C" TinyNNStatus megcc_gfx950_matmul(
     gemm_plan_split(q, ws);
     // 64 x 256 tiles when they still give every CU a workgroup
     const bool skinny = q.M <= 64 && (long)((q.N + 255) / 256) * q.split >= 128;
-    note_kernel("gemm_f32", skinny ? 64 : 128, q.split, q.kchunk > 1024);
     dim3 grid(skinny ? (q.N + 255) / 256 : (q.N + GBN - 1) / GBN, skinny ? 1 : (q.M + GBM - 1) / GBM,
               q.split);
+    q.xo = options().no_xcdorder ? XcdOrder{0} : make_xcd_order((int)grid.x, (int)grid.y);
+    note_kernel("gemm_f32", skinny ? 64 : 128, q.split, q.kchunk > 1024, q.xo.w);
     const bool longk = q.kchunk > 1024;
 #define MG_GEMM_LAUNCH(AK, BN_)                                                                  \
     do {                                                                                         \

@@ -124,7 +124,7 @@ def test_cfg3_fc_q8_64x4096x4096(scale_name, dst_scale):
 def test_cfg3_fc_q8_4096x4096x4096(scale_name, dst_scale):
     rows = sorted(set(range(64)) | set(np.random.default_rng(8).integers(64, 4096, 64).tolist()) | {4095})
     kernel = fc_rows(4096, 4096, 4096, scale_name, dst_scale, rows)
-    assert kernel == "conv_mfma_i8_dma:1,256,256,256,4", kernel  # the 256 x 256 FullyConnected tile
+    assert kernel == "conv_mfma_i8_dma_xo:1,256,256,256,4", kernel  # the 256 x 256 FullyConnected tile, XCD-aware tile order
 
 
 def matmul_rows(m, k, n, rows):

@@ -640,8 +640,18 @@ OLDER = [
     # ragged channel tile, three chunks of input channels, rows of 60 pixels
     ("nom16", ConvCase(A.FMT_NCHW44, A.DENSE, 9, 96, 56, 60, 200, 3, 1, 1, A.H_SWISH,
                        scales=(0.02, 0.01, unsat(864)))),
-    ("nom16", ConvCase(A.FMT_NCHW44, A.DENSE, 16, 64, 56, 56, 128, 3, 1, 1, A.IDENTITY,
-                       scales=(0.02, 0.01, unsat(576)))),
+    # the plain tile order of the tiled GEMMs (the default gives each XCD a compact rectangle of
+    # tiles): f32 MatMul with a ragged 9 x 8 grid of 128 x 128 tiles, all four transpositions,
+    # FullyConnected with 256 x 256 tiles (8 x 8)
+    ("noxcdorder", MatMulCase(1100, 40, 1000)),
+    ("noxcdorder", MatMulCase(1024, 24, 1030, trans_a=True)),
+    ("noxcdorder", MatMulCase(1024, 24, 1030, trans_b=True)),
+    ("noxcdorder", MatMulCase(1030, 24, 1024, trans_a=True, trans_b=True)),
+    ("noxcdorder", ConvCase(A.FMT_NCHW, A.DENSE, 2048, 128, 1, 1, 2040, 1, 1, 0, A.IDENTITY,
+                            scales=(0.02, 0.01, unsat(128)))),
+    # (one channel tile: 512-pixel sub-tiles from 57 600 pixels on)
+    ("nom16", ConvCase(A.FMT_NCHW44, A.DENSE, 20, 32, 56, 56, 128, 3, 1, 1, A.IDENTITY,
+                       scales=(0.02, 0.01, unsat(288)))),
     ("nodma512", ConvCase(A.FMT_NCHW44, A.DENSE, 22, 64, 54, 57, 128, 3, 1, 1, A.RELU,
                                 scales=(0.02, 0.01, unsat(576)))),
     ("nogevm", ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY,

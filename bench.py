@@ -288,7 +288,9 @@ def bench_mobilenet(batch, steps, warmup, per_layer=False):
     # weights per image): priced against HBM on the bytes its operators read and write once each
     moved = mobilenet.algorithmic_bytes(batch)
     out["nr_kernel"] = model.nr_kernel
-    out["launch_mode"] = {1: "graph", -1: "eager", 0: "undecided"}[model.launch_mode()[0]]
+    mode, eager_ms, graph_ms = model.launch_mode()
+    out["launch_mode"] = {1: "graph", -1: "eager", 0: "undecided"}[mode]
+    out["launch_mode_measured_ms"] = {"eager": round(eager_ms, 4), "graph": round(graph_ms, 4)}
     out["roofline"] = {"bound": "hbm", "achieved": round(moved / (dev_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
                        "unit": "GB/s", "frac": round(moved / (dev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                        "traffic": None, "algorithmic_per_launch": moved,

@@ -546,12 +546,22 @@ const char* megcc_gfx950_last_error(void);
 /* Diagnostics (no counterpart in the reference, whose kernel choice is fixed at compile time):
  * which kernel variant the calling thread's most recent operator call selected, as
  * "<kernel>[:n,n,...]" (e.g. "conv_mfma_i8_dma:3,128,512,1024" = variant, oc tile, pixel
- * sub-tile, patch slots). The text lives until the thread's next call of this function. */
+ * sub-tile, patch slots); "+affine" at the end: the kernel requantised by the one fused multiply-add
+ * the host proved exact for the layer's scales instead of the threshold table. The text lives until
+ * the thread's next call of this function. */
 const char* megcc_gfx950_last_kernel(void);
+/* Diagnostics (no counterpart in the reference): the constants of the one-multiply-add
+ * requantisation for a convolution's activation and scales, as the qsi8 kernels would use them:
+ * out = clamp(floor(fma((float)acc, *c, *d)), activation's lowest output, 127) equals the
+ * reference's fp32_to_int8(act(acc * s_src * s_flt / s_dst)) (BareMetal/Activation.cpp:47-56,
+ * 105-114) for EVERY int32 accumulator. Returns 1 and the pair when the host search finds one
+ * (IDENTITY / RELU only), else 0 - such layers requantise by threshold table. Host arithmetic only:
+ * needs no device. */
+int megcc_gfx950_requant_affine(int nonline_mode, float s_src, float s_flt, float s_dst, float* c, float* d);
 /* Kernel-selection overrides, for regression tests of kernels that un-switched shapes only reach
  * through a fallback: "nopws", "nogevm", "nofcb", "nosmall", "nopm768", "nopm", "nodma512",
  * "nopm256", "nodma", "nofcs", "nopwshare", "nohybrid", "nodot4", "nof32small",
- * "dw_generic", "nodwmfma", "nodwnchw", "nofusesoftmax", "nopoolrows", "nofirstmfma", "norowsplit", "nofusechain", "nofcone", "nom16", "noxcdorder", "no_graph"; value 1 takes the kernel out
+ * "dw_generic", "nodwmfma", "nodwnchw", "nofusesoftmax", "nopoolrows", "nofirstmfma", "norowsplit", "nofusechain", "nofcone", "nom16", "noxcdorder", "noaffine", "no_graph"; value 1 takes the kernel out
  * of the dispatch, 0 puts it back. The
  * same names in capitals behind MEGCC_ are read from the environment once, at first use.
  * Unknown names return TinyNN_ERROR_NO_FOUND. */
@@ -617,10 +627,10 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model);
  * kernels one forward launches (an operator chain that runs as one kernel counts once; a chain is
  * only replaced when its result shares no byte with anything the one kernel reads), and how they
  * are launched: 1 = HIP-graph replay, -1 = one launch per kernel, 0 = still measuring. forward()
- * 2, 3, 5 and 6 of a model with at least 5 kernels each block the host until that forward has
+ * 2, 3 and 5 to 10 of a model with at least 5 kernels each block the host until that forward has
  * finished (they time the two ways between events on the library stream; *eager_ms / *graph_ms
- * receive the shortest of two samples each, -1 when not measured); every other forward is
- * asynchronous. */
+ * receive the shortest of four samples each, -1 when not measured; the replay is kept when it is
+ * at least 2 % faster); every other forward is asynchronous. */
 int megcc_gfx950_model_nr_kernel(void* model);
 int megcc_gfx950_model_launch_mode(void* model, float* eager_ms, float* graph_ms);
 size_t megcc_gfx950_model_arena_bytes(void* model);

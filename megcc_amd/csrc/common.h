@@ -62,13 +62,17 @@ __device__ __forceinline__ void xcd_tile(XcdOrder o, int bx, int by, int gx, int
 // environment (MEGCC_NOPWS=1, ...) ONCE, when the library first consults them; later changes go
 // through megcc_gfx950_set_option(). Nothing on a launch path scans the environment.
 struct Options {
-    bool no_pws, no_gevm, no_fcb, no_small, no_pm768, no_pm, no_dma512, no_pm256, no_dma, no_fcs, no_pwshare, no_hybrid, no_dot4, no_f32small, dw_generic, no_dwmfma, no_dwnchw, no_fuse_softmax, no_graph, no_poolrows, no_firstmfma, no_rowsplit, no_fuse_chain, no_fcone, no_m16, no_xcdorder;
+    bool no_pws, no_gevm, no_fcb, no_small, no_pm768, no_pm, no_dma512, no_pm256, no_dma, no_fcs, no_pwshare, no_hybrid, no_dot4, no_f32small, dw_generic, no_dwmfma, no_dwnchw, no_fuse_softmax, no_graph, no_poolrows, no_firstmfma, no_rowsplit, no_fuse_chain, no_fcone, no_m16, no_xcdorder, no_affine;
 };
 Options& options();
 
 // Which kernel variant the most recent dispatch on this thread selected: `name` (a string literal)
 // and up to five numbers that identify the instantiation; megcc_gfx950_last_kernel() formats them.
 void note_kernel(const char* name, int a = -1, int b = -1, int c = -1, int d = -1, int e = -1);
+
+// A kernel that requantises by the proven fused multiply-add (epilogue.h) says so after its
+// note_kernel(): megcc_gfx950_last_kernel() then ends in "+affine".
+void note_requant_affine(bool on);
 
 // conv_api.hip: looks up the address of the static scratch array of
 // megcc_gfx950_conv2d_noalloc on the current device (once per device; later calls return at once).

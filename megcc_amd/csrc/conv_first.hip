@@ -130,6 +130,7 @@ struct ConvFirstMfmaParams {
     int N, IH, IW, OH, OW, OHW, P, tiles, OC;
     int act;
     float s_src, s_flt, s_dst, c;
+    float aff_c, aff_d;  // requantisation by one fused multiply-add (epilogue.h); aff_d == 0: table
     FastDiv dOW, dOHW;
     RequantTable table;
 };
@@ -231,12 +232,18 @@ __global__ void __launch_bounds__(256) conv_first_mfma_kernel(ConvFirstMfmaParam
 #pragma unroll
         for (int mi = 0; mi < MT; ++mi) {
             int r[16];
+            if (ACT >= 0 && q.aff_d != 0.f) {  // (uniform)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                if (ACT < 0)
-                    r[e] = requant_conv_rt(q.act, acc[mi][e], q.s_src, q.s_flt, q.s_dst);
-                else
-                    r[e] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[mi][e], q.c, tbl);
+                for (int e = 0; e < 16; ++e)
+                    r[e] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(acc[mi][e], q.aff_c, q.aff_d);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    if (ACT < 0)
+                        r[e] = requant_conv_rt(q.act, acc[mi][e], q.s_src, q.s_flt, q.s_dst);
+                    else
+                        r[e] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[mi][e], q.c, tbl);
+                }
             }
             if (cur.ok) {
 #pragma unroll
@@ -275,6 +282,9 @@ static TinyNNStatus conv_first_mfma_launch(
     if (tab)
         q.table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
     const int act = tab ? g.act : -1;
+    const RequantAffine aff = requant_affine_pick(tab, g.act, g.s_src, g.s_flt, g.s_dst);
+    q.aff_c = aff.c;
+    q.aff_d = aff.d;
     const void* kern;
 #define MG_CFM(MT_)                                                                                     \
     (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_first_mfma_kernel<MT_, MEGCC_NONLINE_IDENTITY>     \

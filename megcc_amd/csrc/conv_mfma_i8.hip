@@ -676,6 +676,11 @@ TinyNNStatus conv_mfma_launch(
                        : XcdOrder{0};
         note_kernel(pc.m16 ? "conv_mfma_i8_dma_m16" : q.xo.w ? "conv_mfma_i8_dma_xo" : "conv_mfma_i8_dma", picked,
                     pc.bm, pc.bn, q.Lmax, pc.ks);
+        const RequantAffine aff = requant_affine_pick(
+                requant_table_act(g.act) && requant_table_ok(g.s_src, g.s_flt, g.s_dst), g.act, g.s_src, g.s_flt,
+                g.s_dst);
+        q.rq.aff_c = aff.c;
+        q.rq.aff_d = aff.d;
         return conv_mfma_pipe_launch(pc, q);
     }
     const int split = conv_mfma_split(g);

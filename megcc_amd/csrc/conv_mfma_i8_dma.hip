@@ -311,6 +311,10 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
 #pragma unroll
             for (int e = 0; e < 16; ++e)
                 r[e] = requant_conv_rt(q.act, acc[mi][ni][e], q.s_src, q.s_flt, q.s_dst);
+        } else if (ACT != MEGCC_NONLINE_H_SWISH && q.rq.aff_d != 0.f) {  // (uniform)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                r[e] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(acc[mi][ni][e], q.rq.aff_c, q.rq.aff_d);
         } else {
             int m[16], t[16];
 #pragma unroll
@@ -568,6 +572,13 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                             r[ni][e] = requant_conv_rt(q.act, acc16[mi][ni][e], q.s_src, q.s_flt, q.s_dst);
+                } else if (ACT != MEGCC_NONLINE_H_SWISH && q.rq.aff_d != 0.f) {  // (uniform)
+#pragma unroll
+                    for (int ni = 0; ni < NT16; ++ni)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            r[ni][e] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(
+                                    acc16[mi][ni][e], q.rq.aff_c, q.rq.aff_d);
                 } else {
                     int m[NT16][4], t[NT16][4];
 #pragma unroll

@@ -45,6 +45,7 @@ struct PwParams {
     int plane_stride;  // bytes
     int act;
     float s_src, s_flt, s_dst, c;
+    float aff_c, aff_d;  // requantisation by one fused multiply-add (epilogue.h); aff_d == 0: table
     FastDiv dOHW;
     RequantTable table;
 };
@@ -176,6 +177,10 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_stream_kernel(PwParams q) 
 #pragma unroll
                         for (int e = 0; e < 16; ++e)
                             r[e] = requant_conv_rt(q.act, acc[mi][e], q.s_src, q.s_flt, q.s_dst);
+                    } else if (q.aff_d != 0.f) {  // (uniform)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e)
+                            r[e] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(acc[mi][e], q.aff_c, q.aff_d);
                     } else {
 #pragma unroll
                         for (int e = 0; e < 16; ++e)
@@ -295,6 +300,10 @@ __global__ void __launch_bounds__(PW_THREADS) conv_pw_share_kernel(PwParams q) {
 #pragma unroll
             for (int e = 0; e < 16; ++e)
                 r[e] = requant_conv_rt(q.act, acc[e], q.s_src, q.s_flt, q.s_dst);
+        } else if (q.aff_d != 0.f) {  // (uniform)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                r[e] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(acc[e], q.aff_c, q.aff_d);
         } else {
 #pragma unroll
             for (int e = 0; e < 16; ++e)
@@ -410,6 +419,9 @@ TinyNNStatus conv_pw_stream_launch(
                 runs = 1;
             void* sargs[] = {&q};
             note_kernel("conv_pw_share", g.ic / 32);
+            const RequantAffine aff = requant_affine_pick(tab, g.act, g.s_src, g.s_flt, g.s_dst);
+            q.aff_c = aff.c;
+            q.aff_d = aff.d;
             hipError_t e = hipLaunchKernel(sk, dim3((unsigned)(runs * gblocks)), dim3(PW_THREADS), sargs, 0, stream());
             MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_pw_share: %s", hipGetErrorString(e));
             return check_launch("conv_pw_share");
@@ -431,8 +443,11 @@ TinyNNStatus conv_pw_stream_launch(
     waves = (waves + unit - 1) / unit * unit;
     const unsigned blocks = (unsigned)(waves / 4);
 
-    void* args[] = {&q};
     note_kernel("conv_pw_stream", kc, ragged);
+    const RequantAffine aff = requant_affine_pick(tab, g.act, g.s_src, g.s_flt, g.s_dst);
+    q.aff_c = aff.c;
+    q.aff_d = aff.d;
+    void* args[] = {&q};
     hipError_t e = hipLaunchKernel(kern, dim3(blocks), dim3(PW_THREADS), args, 0, stream());
     MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "conv_pw_stream: %s", hipGetErrorString(e));
     return check_launch("conv_pw_stream");

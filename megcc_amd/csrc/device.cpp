@@ -9,6 +9,7 @@
 #include <mutex>
 
 #include "common.h"
+#include "epilogue.h"
 
 namespace mg {
 
@@ -31,7 +32,7 @@ const OptionName kOptions[] = {
         {"nodot4", &Options::no_dot4},       {"nof32small", &Options::no_f32small},
         {"dw_generic", &Options::dw_generic}, {"no_graph", &Options::no_graph},
         {"nodwmfma", &Options::no_dwmfma},   {"nodwnchw", &Options::no_dwnchw},
-        {"nofusesoftmax", &Options::no_fuse_softmax}, {"nopoolrows", &Options::no_poolrows}, {"nofirstmfma", &Options::no_firstmfma}, {"norowsplit", &Options::no_rowsplit}, {"nofusechain", &Options::no_fuse_chain}, {"nofcone", &Options::no_fcone}, {"nom16", &Options::no_m16}, {"noxcdorder", &Options::no_xcdorder},
+        {"nofusesoftmax", &Options::no_fuse_softmax}, {"nopoolrows", &Options::no_poolrows}, {"nofirstmfma", &Options::no_firstmfma}, {"norowsplit", &Options::no_rowsplit}, {"nofusechain", &Options::no_fuse_chain}, {"nofcone", &Options::no_fcone}, {"nom16", &Options::no_m16}, {"noxcdorder", &Options::no_xcdorder}, {"noaffine", &Options::no_affine},
 };
 struct KernelNote {
     const char* name;
@@ -39,6 +40,7 @@ struct KernelNote {
 };
 thread_local KernelNote g_note = {"", {-1, -1, -1, -1, -1}};
 thread_local char g_note_text[160];
+thread_local bool g_note_affine = false;  // the noted kernel requantises by the proven multiply-add
 }  // namespace
 
 Options& options() {
@@ -65,6 +67,11 @@ void note_kernel(const char* name, int a, int b, int c, int d, int e) {
     g_note.v[2] = c;
     g_note.v[3] = d;
     g_note.v[4] = e;
+    g_note_affine = false;
+}
+
+void note_requant_affine(bool on) {
+    g_note_affine = on;
 }
 
 hipStream_t stream() {
@@ -197,7 +204,18 @@ const char* megcc_gfx950_last_kernel(void) {
     int n = snprintf(g_note_text, sizeof(g_note_text), "%s", g_note.name);
     for (int i = 0; i < 5 && g_note.v[i] != -1 && n > 0 && n < (int)sizeof(g_note_text); ++i)
         n += snprintf(g_note_text + n, sizeof(g_note_text) - n, "%c%d", i ? ',' : ':', g_note.v[i]);
+    if (g_note_affine && n > 0 && n < (int)sizeof(g_note_text))
+        snprintf(g_note_text + n, sizeof(g_note_text) - n, "+affine");
     return g_note_text;
+}
+
+int megcc_gfx950_requant_affine(int nonline_mode, float s_src, float s_flt, float s_dst, float* c, float* d) {
+    const RequantAffine a = requant_affine_for(nonline_mode, s_src, s_flt, s_dst);
+    if (c)
+        *c = a.c;
+    if (d)
+        *d = a.d;
+    return a.d != 0.f;
 }
 
 TinyNNStatus megcc_gfx950_set_option(const char* name, int value) {

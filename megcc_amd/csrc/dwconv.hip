@@ -232,7 +232,9 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
                 for (int c = 0; c < 4; ++c) {
                     const int m = max(max(acc[(2 * k) * 4 + c], acc[(2 * k + 1) * 4 + c]),
                                       max(acc[16 + (2 * k) * 4 + c], acc[16 + (2 * k + 1) * 4 + c]));
-                    const int f = requant_conv_table<(ACT < 0 ? 0 : ACT)>(m, rq.c, tbl);
+                    const int f = rq.aff_d != 0.f
+                                          ? requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(m, rq.aff_c, rq.aff_d)
+                                          : requant_conv_table<(ACT < 0 ? 0 : ACT)>(m, rq.c, tbl);
                     acc[(2 * k) * 4 + c] = acc[(2 * k + 1) * 4 + c] = f;
                     acc[16 + (2 * k) * 4 + c] = acc[16 + (2 * k + 1) * 4 + c] = f;
                 }
@@ -240,6 +242,10 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
 #pragma unroll
             for (int e = 0; e < R * 16; ++e)
                 acc[e] = requant_conv_rt(g.act, acc[e], g.s_src, g.s_flt, g.s_dst);
+        } else if (rq.aff_d != 0.f) {  // (uniform)
+#pragma unroll
+            for (int e = 0; e < R * 16; ++e)
+                acc[e] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(acc[e], rq.aff_c, rq.aff_d);
         } else {
 #pragma unroll
             for (int e = 0; e < R * 16; ++e)
@@ -325,11 +331,14 @@ TinyNNStatus dwconv44_chain_launch(
     if (groups4 == 0)
         return TinyNN_SUCCESS;
     const unsigned nb = (unsigned)((groups4 + 255) / 256);
-    const RequantFast rq3 = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
+    RequantFast rq3 = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
     const bool tab = (g.act == MEGCC_NONLINE_IDENTITY || g.act == MEGCC_NONLINE_RELU) &&
                      requant_table_ok(g.s_src, g.s_flt, g.s_dst);
     static const RequantTable no_table = {};
     const RequantTable& table = tab ? requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst) : no_table;
+    const RequantAffine aff = requant_affine_pick(tab, g.act, g.s_src, g.s_flt, g.s_dst);
+    rq3.aff_c = aff.c;
+    rq3.aff_d = aff.d;
     DwChain fz;
     fz.other = (const uint32_t*)other;
     fz.poh = g.oh / 2;
@@ -402,7 +411,7 @@ TinyNNStatus dwconv44_launch(
         const int R = shape & 15;
         const int groups4 = (int)((long)g.n * (g.oc >> 2) * ((g.oh + R - 1) / R) * ((g.ow + 3) / 4));
         unsigned nb = (unsigned)((groups4 + 255) / 256);
-        const RequantFast rq3 = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
+        RequantFast rq3 = make_requant_fast(g.s_src, g.s_flt, g.s_dst);
         void (*k3)(ConvGeom, RequantFast, const uint32_t*, const uint32_t*, const int32_t*, uint32_t*, int, int,
                    FastDiv, FastDiv, FastDiv, RequantTable, DwChain);
         // exact thresholds for the monotone activations; anything else (and extreme scales)
@@ -410,6 +419,9 @@ TinyNNStatus dwconv44_launch(
         const bool tab = requant_table_act(g.act) && requant_table_ok(g.s_src, g.s_flt, g.s_dst);
         static const RequantTable no_table = {};
         const RequantTable& table = tab ? requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst) : no_table;
+        const RequantAffine aff = requant_affine_pick(tab, g.act, g.s_src, g.s_flt, g.s_dst);
+        rq3.aff_c = aff.c;
+        rq3.aff_d = aff.d;
 #define MG_DW_PICK(S_, R_, G_)                                                                      \
     (tab && g.act == MEGCC_NONLINE_IDENTITY ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_IDENTITY, R_, G_> \
      : tab && g.act == MEGCC_NONLINE_RELU   ? dwconv44_3x3_kernel<S_, MEGCC_NONLINE_RELU, R_, G_>     \

@@ -63,6 +63,7 @@ struct DwMfmaParams {
     int tiles;             // per plane set: ceil(cols / 32)
     int act;
     float s_src, s_flt, s_dst, c;
+    float aff_c, aff_d;   // requantisation by one fused multiply-add (epilogue.h); aff_d == 0: table
     FastDiv d_ohp, d_xb;  // division by ohp, by xblocks
     // FUSE: the second operand of the addition that follows the pooling ([N][C/4][poh][pow] dwords), the
     // extent of the pooled tensor, the scales of the pooled operand and of `other`, 1 / the result's
@@ -266,8 +267,14 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
                 for (int c = 0; c < 4; ++c) {
                     const dwm_v2u s02 = __builtin_amdgcn_permlane32_swap((unsigned)v[c], (unsigned)v[8 + c], false, false);
                     const dwm_v2u s13 = __builtin_amdgcn_permlane32_swap((unsigned)v[4 + c], (unsigned)v[12 + c], false, false);
-                    pooled[0][c] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(max((int)s02[0], (int)s02[1]), q.c, tbl);
-                    pooled[1][c] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(max((int)s13[0], (int)s13[1]), q.c, tbl);
+                    const int w0 = max((int)s02[0], (int)s02[1]), w1 = max((int)s13[0], (int)s13[1]);
+                    if (q.aff_d != 0.f) {  // (uniform)
+                        pooled[0][c] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(w0, q.aff_c, q.aff_d);
+                        pooled[1][c] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(w1, q.aff_c, q.aff_d);
+                    } else {
+                        pooled[0][c] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(w0, q.c, tbl);
+                        pooled[1][c] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(w1, q.c, tbl);
+                    }
                 }
             } else {
                 unsigned d[4];  // vertical maximum of pixel 2 * j + kg, 4 requantised channel bytes
@@ -313,6 +320,10 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     o[e] = requant_conv_rt(q.act, acc[r][e], q.s_src, q.s_flt, q.s_dst);
+            } else if (q.aff_d != 0.f) {  // (uniform)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    o[e] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(acc[r][e], q.aff_c, q.aff_d);
             } else {
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
@@ -390,6 +401,10 @@ static TinyNNStatus dwconv44_mfma_run(
     if (tab)
         q.table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
     const int act = tab ? g.act : -1;
+    // (the chain kernel has no table instantiation for H_SWISH: the pair is only asked for where one runs)
+    const RequantAffine aff = requant_affine_pick(tab, g.act, g.s_src, g.s_flt, g.s_dst);
+    q.aff_c = aff.c;
+    q.aff_d = aff.d;
     const bool ragged = (g.iw & 3) != 0;
     const void* kern = nullptr;
 #define MG_DWM_ACT(S_, R_, F_)                                                                        \

@@ -62,6 +62,7 @@ __host__ __device__ __forceinline__ int requant_conv(int acc, float s_src, float
 struct RequantFast {
     float c;       // fl(fl(s_src*s_flt)/s_dst); 0 disables the fast path (extreme scales)
     float s_src, s_flt, s_dst;
+    float aff_c, aff_d;  // requant_conv_affine's pair when the launch picked one (below); aff_d == 0: none
 };
 
 // host side: c, or 0 when a scale is so extreme that the error bound above does not hold
@@ -75,6 +76,7 @@ static inline RequantFast make_requant_fast(float s_src, float s_flt, float s_ds
     auto mid = [](float x) { return x > 1e-30f && x < 1e30f; };
     const bool sane = mid(s_src) && mid(s_flt) && mid(p) && mid(s_dst) && mid(c);
     q.c = sane ? c : 0.f;
+    q.aff_c = q.aff_d = 0.f;
     return q;
 }
 
@@ -199,6 +201,38 @@ template <int ACT>
 __device__ __forceinline__ int requant_conv_table(int acc, float c, const int* table) {
     const int m = requant_table_candidate<ACT>(acc, c);
     return m + (acc > table[m + 128] ? 1 : 0);
+}
+
+// ---- exact requantisation by ONE fused multiply-add, where the host can prove it ----------------
+// The table look-up costs 7-8 vector instructions and an LDS read per output, and layers with few
+// multiply-adds per output (pointwise with 32..128 input channels, depthwise) are bound by exactly
+// that. For IDENTITY and RELU the candidate
+//     F'(a) = clamp(floor(fma((float)a, c', d)), lo, 127)
+// is a non-decreasing step function of a like F itself, so F' == F on all of int32 iff the two
+// agree on both sides of every step of F - 2 x 255 evaluations. The host looks for a pair (c', d)
+// near (c, 0.5) that passes that check against the reference's literal float sequence (for each
+// c' within a few ulps of c the feasible d form an interval; its middle is then verified with the
+// exact fmaf) and caches the answer per (activation, scales). Scales with exact ties whose
+// roundings land on either side (0.02 * 0.01 / 0.05 ...) have no such pair and keep the table;
+// calibrated scales of real networks almost always have one. 4 instructions per output, no LDS.
+struct RequantAffine {
+    float c, d;  // d == 0: no exact pair exists (or the activation is not IDENTITY / RELU)
+};
+RequantAffine requant_affine_for(int act, float s_src, float s_flt, float s_dst);
+// what a launch uses: the pair (and the launch is noted as "+affine") when `table` - the kernel is the
+// table instantiation for IDENTITY / RELU - and the switch "noaffine" is off; else d == 0. Call it
+// after note_kernel().
+RequantAffine requant_affine_pick(bool table, int act, float s_src, float s_flt, float s_dst);
+
+template <int ACT>
+__host__ __device__ __forceinline__ int requant_affine_lo() {
+    return ACT == MEGCC_NONLINE_RELU ? 0 : -128;
+}
+template <int ACT>
+__device__ __forceinline__ int requant_conv_affine(int acc, float c, float d) {
+    constexpr int LO = ACT == MEGCC_NONLINE_RELU ? 0 : -128;
+    const int m = cvt_floor_i32(__builtin_fmaf((float)acc, c, d));  // saturating conversion
+    return m < LO ? LO : (m > 127 ? 127 : m);
 }
 
 // host side: the estimate above is valid (else kernels use the literal sequence per element)

@@ -712,7 +712,8 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
         return replay();
     if (m->graph_state == -1)
         return forward_eager(m);
-    // ---- undecided: the first six forwards
+    // ---- undecided: the first ten forwards (1: plain; 2, 3, 7, 8: timed plain launches; 4: the capture
+    //      and its first replay; 5, 6, 9, 10: timed replays)
     // (schedules of fewer than 5 kernels stay eager without asking: the depthwise + pooling + addition
     //  chain as one kernel takes 7.6 us per forward eagerly, 16.2 us as a graph)
     if (options().no_graph || m->schedule.size() < 5) {
@@ -736,7 +737,7 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
             *best = ms;
         return st;
     };
-    if (m->forwards <= 3)
+    if (m->forwards <= 3 || (m->graph_exec && (m->forwards == 7 || m->forwards == 8)))
         return timed(false, &m->eager_ms);
     if (m->forwards == 4) {
         if (hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal) == hipSuccess) {
@@ -758,8 +759,10 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
         return forward_eager(m);
     }
     TinyNNStatus st = timed(true, &m->graph_ms);
-    if (m->forwards >= 6)
-        m->graph_state = m->graph_ms < 0.95f * m->eager_ms ? 1 : -1;  // (a tie keeps the plain launches)
+    // (the shortest of four each: a single sample of a 0.12 ms forward is off by several percent, which
+    //  flipped the choice for batch-1 networks from run to run; a tie keeps the plain launches)
+    if (m->forwards >= 10)
+        m->graph_state = m->graph_ms < 0.98f * m->eager_ms ? 1 : -1;
     return st;
 }
 

@@ -107,7 +107,7 @@ EXPORTS = [
     "megcc_gfx950_malloc", "megcc_gfx950_free", "megcc_gfx950_memcpy_h2d",
     "megcc_gfx950_memcpy_d2h", "megcc_gfx950_memset", "megcc_gfx950_wait",
     "megcc_gfx950_stream", "megcc_gfx950_last_error", "megcc_gfx950_last_kernel",
-    "megcc_gfx950_set_option",
+    "megcc_gfx950_set_option", "megcc_gfx950_requant_affine",
     "megcc_gfx950_model_create", "megcc_gfx950_model_destroy", "megcc_gfx950_model_add_tensor",
     "megcc_gfx950_model_add_weight", "megcc_gfx950_model_add_alias", "megcc_gfx950_model_add_view",
     "megcc_gfx950_model_add_opr", "megcc_gfx950_model_add_opr_desc",
@@ -201,6 +201,15 @@ def wait():
 def last_kernel():
     """which kernel variant this thread's most recent operator call selected"""
     return lib().megcc_gfx950_last_kernel().decode()
+
+
+def requant_affine(act, s_src, s_flt, s_dst):
+    """(c, d) of the one-multiply-add requantisation the host proved exact for these scales, or None"""
+    c, d = C.c_float(), C.c_float()
+    f = lib().megcc_gfx950_requant_affine
+    f.argtypes = [C.c_int, C.c_float, C.c_float, C.c_float, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    f.restype = C.c_int
+    return (c.value, d.value) if f(act, s_src, s_flt, s_dst, C.byref(c), C.byref(d)) else None
 
 
 def set_option(name, value):

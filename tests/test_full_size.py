@@ -70,7 +70,7 @@ def test_cfg2_conv3x3_n32(c, hw, act, dst_scale):
     assert kernel.startswith("conv_mfma_i8_dma"), kernel
     if c == 256 and hw == 56:
         # the instantiation bench.py times: plane-major patch of 1024 slots, 128 oc x 512 px
-        assert kernel == "conv_mfma_i8_dma_m16:3,128,512,1024,1", kernel
+        assert kernel.split("+")[0] == "conv_mfma_i8_dma_m16:3,128,512,1024,1", kernel
     one = ConvCase(A.FMT_NCHW44, A.DENSE, 1, c, hw, hw, c, 3, 1, 1, act, scales=scales)
     for i in (0, 17, 31):
         want = one.run_port({"src": arrays["src"][i:i + 1], "flt": arrays["flt"], "bias": arrays["bias"]})
@@ -124,7 +124,7 @@ def test_cfg3_fc_q8_64x4096x4096(scale_name, dst_scale):
 def test_cfg3_fc_q8_4096x4096x4096(scale_name, dst_scale):
     rows = sorted(set(range(64)) | set(np.random.default_rng(8).integers(64, 4096, 64).tolist()) | {4095})
     kernel = fc_rows(4096, 4096, 4096, scale_name, dst_scale, rows)
-    assert kernel == "conv_mfma_i8_dma_xo:1,256,256,256,4", kernel  # the 256 x 256 FullyConnected tile, XCD-aware tile order
+    assert kernel.split("+")[0] == "conv_mfma_i8_dma_xo:1,256,256,256,4", kernel  # the 256 x 256 FullyConnected tile, XCD-aware tile order
 
 
 def matmul_rows(m, k, n, rows):

@@ -649,6 +649,25 @@ OLDER = [
     ("noxcdorder", MatMulCase(1030, 24, 1024, trans_a=True, trans_b=True)),
     ("noxcdorder", ConvCase(A.FMT_NCHW, A.DENSE, 2048, 128, 1, 1, 2040, 1, 1, 0, A.IDENTITY,
                             scales=(0.02, 0.01, unsat(128)))),
+    # the threshold table where the default is the one-multiply-add requantisation the host proved
+    # exact for the layer's scales (scales without exact ties; "+affine" in the kernel's name):
+    # pointwise streaming and workgroup-shared kernels, depthwise on the matrix cores and by v_dot4,
+    # the matrix-core first layer, the LDS-direct 3x3 kernel in both MFMA shapes
+    ("noaffine", ConvCase(A.FMT_NCHW44, A.DENSE, 4, 32, 56, 56, 64, 1, 1, 0, A.RELU,
+                          scales=(0.0213, 0.0097, unsat(32) * 1.0371))),
+    ("noaffine", ConvCase(A.FMT_NCHW44, A.DENSE, 64, 512, 14, 14, 512, 1, 1, 0, A.RELU,
+                          scales=(0.015522320754826069, 0.0012519484153017402, 0.015279783867299557),
+                          src_range=(-40, 40), flt_range=(-40, 40))),
+    ("noaffine", ConvCase(A.FMT_NCHW44, A.GROUP, 3, 64, 28, 28, 64, 3, 1, 1, A.RELU,
+                          scales=(0.0213, 0.0097, unsat(9) * 1.0371))),
+    ("noaffine", ConvCase(A.FMT_NCHW44, A.GROUP, 3, 64, 28, 28, 64, 3, 2, 1, A.IDENTITY,
+                          scales=(0.0213, 0.0097, unsat(9) * 1.0371))),
+    ("noaffine", ConvCase(A.FMT_NCHW_NCHW44, A.DENSE, 2, 3, 64, 64, 32, 3, 2, 1, A.RELU,
+                          scales=(0.0213, 0.0097, unsat(27) * 1.0371))),
+    ("noaffine", ConvCase(A.FMT_NCHW44, A.DENSE, 6, 32, 56, 56, 160, 3, 1, 1, A.RELU,
+                          scales=(0.0213, 0.0097, unsat(288) * 1.0371))),
+    ("noaffine", ConvCase(A.FMT_NCHW44, A.DENSE, 20, 32, 56, 56, 128, 3, 1, 1, A.RELU,
+                          scales=(0.0213, 0.0097, unsat(288) * 1.0371))),
     # (one channel tile: 512-pixel sub-tiles from 57 600 pixels on)
     ("nom16", ConvCase(A.FMT_NCHW44, A.DENSE, 20, 32, 56, 56, 128, 3, 1, 1, A.IDENTITY,
                        scales=(0.02, 0.01, unsat(288)))),
@@ -1055,7 +1074,12 @@ CHAINS = [
 
 def _chain_cases(n, c, ih, iw, stride, act, mode, bias):
     sc = unsat(9) * (40 if act == A.SIGMOID else 1)
-    dw = ConvCase(A.FMT_NCHW44, A.GROUP, n, c, ih, iw, c, 3, stride, 1, act, scales=(0.02, 0.01, sc), bias=bias)
+    s_src, s_flt = 0.02, 0.01
+    if n % 2 == 0:
+        # scales without exact ties: IDENTITY / RELU then requantise by the proven multiply-add, the
+        # odd batches (0.02 * 0.01 / ...: ties at every 125th accumulator or so) by threshold table
+        s_src, s_flt, sc = 0.0213, 0.0097, sc * 1.0371
+    dw = ConvCase(A.FMT_NCHW44, A.GROUP, n, c, ih, iw, c, 3, stride, 1, act, scales=(s_src, s_flt, sc), bias=bias)
     pool = PoolCase(A.FMT_NCHW44, A.POOL_MAX, n, c, dw.oh, dw.ow, 2, 2, 0, scale=sc)
     add = MultiTypeCase(mode, pool.dst_shape(), (sc, 0.013, 0.9 * sc))
     return dw, pool, add

@@ -76,14 +76,14 @@ def test_memory_plan_reuses_the_arena_and_keeps_results():
 @pytest.mark.gpu
 def test_graph_replays_equal_eager_forwards():
     """The model runtime captures its operator sequence into a HIP graph on the fourth forward, replays
-    it on the fifth and sixth and then keeps whichever of eager launches and replays it measured
-    faster. Every forward, with new inputs, host copies and synchronisations in between, must give
+    it on the fifth and sixth, ninth and tenth (plain launches again in between) and then keeps
+    whichever of eager launches and replays it measured faster. Every forward, with new inputs, host copies and synchronisations in between, must give
     what an eager forward gives (bit for bit: same kernels, same order)."""
     net = mobilenet.Net(2)
     eager, ids = net.build_gpu(keep_all=True)
     graph, _ = net.build_gpu(keep_all=True)
     names = ["conv0", "pw1", "pw13", "fc", "softmax"]
-    for it in range(9):
+    for it in range(13):
         image = mobilenet.draw_input(2, seed=20 + it)
         runtime.set_option("no_graph", 1)
         try:
@@ -93,7 +93,7 @@ def test_graph_replays_equal_eager_forwards():
             runtime.set_option("no_graph", 0)
         want = {k: eager.get(ids[k]).copy() for k in names}
         graph.set_input(ids["image"], image)
-        graph.forward()  # it 0-2: eager, 3: capture + first launch, 4-5: replays, then the faster way
+        graph.forward()  # it 0-2: eager, 3: capture + first launch, 4-5: replays, 6-7: eager, 8-9: replays, then the faster way
         for k in names:
             np.testing.assert_array_equal(graph.get(ids[k]), want[k], err_msg="%s, forward %d" % (k, it))
     eager.close()

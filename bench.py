@@ -534,6 +534,63 @@ def cpu_baseline(full_case, unit="TOP/s"):
     }
 
 
+def bench_sustained(op, seconds):
+    """Back-to-back launches for `seconds`, 2000 per interval: time per launch of each interval next
+    to the GPU clock and board power the driver reports meanwhile (pp_dpm_sclk's current level,
+    hwmon power1_average / power1_input, sampled every 0.2 s from sysfs; None where the files are
+    not readable). Says whether a kernel's rate is held back by the power cap."""
+    import glob
+    import threading
+    from megcc_amd import runtime
+    samples, stop = [], [False]
+
+    def read(path):
+        try:
+            with open(path) as f:
+                return f.read().strip()
+        except OSError:
+            return None
+
+    def sampler():
+        cards = glob.glob("/sys/class/drm/card*/device")
+        t0 = time.perf_counter()
+        while not stop[0]:
+            mhz, watts = None, None
+            for c in cards:
+                levels = read(c + "/pp_dpm_sclk")
+                cur = [l for l in (levels or "").splitlines() if l.endswith("*")]
+                if cur:
+                    mhz = max(mhz or 0, int("".join(ch for ch in cur[0].split(":")[1] if ch.isdigit())))
+                for h in glob.glob(c + "/hwmon/hwmon*/power1_average") + glob.glob(c + "/hwmon/hwmon*/power1_input"):
+                    v = read(h)
+                    if v and v.isdigit():
+                        watts = max(watts or 0, int(v) / 1e6)
+            samples.append((time.perf_counter() - t0, mhz, watts))
+            time.sleep(0.2)
+
+    th = threading.Thread(target=sampler)
+    th.start()
+    ev = HipEvents(runtime.lib().megcc_gfx950_stream())
+    rows, t0 = [], time.perf_counter()
+    try:
+        while time.perf_counter() - t0 < seconds:
+            e0, e1 = ev.new(), ev.new()
+            ev.record(e0)
+            for _ in range(2000):
+                op.launch()
+            ev.record(e1)
+            runtime.wait()
+            t = time.perf_counter() - t0
+            near = [x for x in samples if abs(x[0] - t) < 0.3]
+            rows.append({"t_s": round(t, 2), "us_per_launch": round(ev.elapsed_ms(e0, e1) / 2, 2),
+                         "sclk_mhz": near[-1][1] if near else None,
+                         "power_w": round(near[-1][2], 0) if near and near[-1][2] else None})
+    finally:
+        stop[0] = True
+        th.join()
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -549,6 +606,9 @@ def main():
                     help="time the CPU baseline for this workload too (the default workload always does)")
     ap.add_argument("--batch", type=int, default=64, help="batch of the mobilenet workload")
     ap.add_argument("--per-layer", action="store_true")
+    ap.add_argument("--sustain", type=float, default=0.0,
+                    help="instead of the timed steps: launch the workload back to back for this many "
+                         "seconds and print time per launch, GPU clock and board power over time")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (the path shards over the batch "
@@ -576,6 +636,9 @@ def main():
     kdesc = case.desc() if hasattr(case, "desc") else runtime.parse_symbol(case.symbol())
     op = runtime.PreparedOp(kdesc, ins, outs)
     ev = HipEvents(runtime.lib().megcc_gfx950_stream())
+    if args.sustain > 0:
+        print(json.dumps({"workload": desc, "kernel": None, "sustained": bench_sustained(op, args.sustain)}))
+        return
 
     preheat = 0
     t_heat = time.perf_counter() + args.preheat_ms * 1e-3

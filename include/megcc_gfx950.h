@@ -561,7 +561,7 @@ int megcc_gfx950_requant_affine(int nonline_mode, float s_src, float s_flt, floa
 /* Kernel-selection overrides, for regression tests of kernels that un-switched shapes only reach
  * through a fallback: "nopws", "nogevm", "nofcb", "nosmall", "nopm768", "nopm", "nodma512",
  * "nopm256", "nodma", "nofcs", "nopwshare", "nohybrid", "nodot4", "nof32small",
- * "dw_generic", "nodwmfma", "nodwnchw", "nofusesoftmax", "nopoolrows", "nofirstmfma", "norowsplit", "nofusechain", "nofcone", "nom16", "noxcdorder", "noaffine", "no_graph"; value 1 takes the kernel out
+ * "dw_generic", "nodwmfma", "nodwnchw", "nofusesoftmax", "nopoolrows", "nofirstmfma", "norowsplit", "nofusechain", "nofcone", "noxcdorder", "noaffine", "no_graph"; value 1 takes the kernel out
  * of the dispatch, 0 puts it back. The
  * same names in capitals behind MEGCC_ are read from the environment once, at first use.
  * Unknown names return TinyNN_ERROR_NO_FOUND. */

@@ -57,6 +57,7 @@ struct ChParams {
     float inv_pitch4, inv_rp;  // 4 / pitch, 1 / RP
     int act;
     float s_src, s_flt, s_dst, c;
+    float aff_c, aff_d;  // requantisation by one fused multiply-add (epilogue.h); aff_d == 0: table
     RequantTable table;
 };
 
@@ -247,6 +248,10 @@ __global__ void __launch_bounds__(CH_THREADS, OT == 1 ? 3 : 2) conv_hybrid_mfma_
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     r[e] = requant_conv_rt(q.act, acc[t][e], q.s_src, q.s_flt, q.s_dst);
+            } else if (q.aff_d != 0.f) {  // (uniform)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    r[e] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(acc[t][e], q.aff_c, q.aff_d);
             } else {
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
@@ -312,6 +317,9 @@ TinyNNStatus conv_hybrid_mfma_launch(
     if (tab)
         q.table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
     const int act = tab ? g.act : -1;
+    const RequantAffine aff = requant_affine_pick(tab, g.act, g.s_src, g.s_flt, g.s_dst);
+    q.aff_c = aff.c;
+    q.aff_d = aff.d;
     const void* kern = nullptr;
 #define MG_CH_PICK(S_, OT_)                                                                             \
     (act == MEGCC_NONLINE_IDENTITY ? (const void*)conv_hybrid_mfma_kernel<S_, MEGCC_NONLINE_IDENTITY, OT_> \

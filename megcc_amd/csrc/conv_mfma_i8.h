@@ -151,7 +151,6 @@ struct PipeConfig {
     int fixed_lmax;      // patch slots compiled into the kernel (0: run-time Lmax)
     int pm = 0;          // plane-major activation patch (virtual rows padded to a multiple of 4)
     int rs = 0;          // a stage is ONE filter row of a 32-channel chunk (filters of more than 9 taps)
-    int m16 = 0;         // 16 x 16 x 64 MFMA tiles (3x3 layers with the plane-major patch)
     int fcb = 0;         // FullyConnected with 16-byte activation loads (K a multiple of 128)
     const void* kernel;
 };

@@ -674,7 +674,7 @@ TinyNNStatus conv_mfma_launch(
         q.xo = pc.fcb && !options().no_xcdorder
                        ? make_xcd_order((q.P + q.range_len - 1) / q.range_len, (q.OC + pc.bm - 1) / pc.bm)
                        : XcdOrder{0};
-        note_kernel(pc.m16 ? "conv_mfma_i8_dma_m16" : q.xo.w ? "conv_mfma_i8_dma_xo" : "conv_mfma_i8_dma", picked,
+        note_kernel(q.xo.w ? "conv_mfma_i8_dma_xo" : "conv_mfma_i8_dma", picked,
                     pc.bm, pc.bn, q.Lmax, pc.ks);
         const RequantAffine aff = requant_affine_pick(
                 requant_table_act(g.act) && requant_table_ok(g.s_src, g.s_flt, g.s_dst), g.act, g.s_src, g.s_flt,

@@ -58,23 +58,10 @@ static constexpr int ACT_RT = -1;
 // stage chunk * q.FH + fh finds its FW taps at the same place as a stage of an FW-tap filter would;
 // its patch is the patch of filter row 0 moved down by fh * DH image rows, with the rows that fall
 // off the image read as zeros (every load remembers the image row it fetches for filter row 0).
-// M16 (3x3 layers with the plane-major patch): the products run as v_mfma_i32_16x16x64_i8 on 16 x 16
-// tiles instead of v_mfma_i32_32x32x32_i8 on 32 x 32 tiles. On this power-limited board a launch of
-// nothing but MFMAs on uniformly random int8 operands delivers 3.5 POP/s with the 16 x 16 x 64 form
-// against 3.0 POP/s with the 32 x 32 x 32 form (a quarter of the accumulator traffic per
-// multiply-add), and the matrix cores' energy is what bounds this kernel. K = 64 of one instruction
-// = two taps x 32 channels: lane group g = lane / 16 holds the 16 channels of half g & 1 of tap
-// 2j + g / 2; the ninth tap goes through v_mfma_i32_16x16x32_i8 (8 channels per lane group), whose
-// result tile has the same layout. A wave's 64 * MT / 2 oc x 32 * NT px are MT * 2 x NT * 2 tiles
-// of four accumulators per lane: register e of lane (g, i) is channel 4 g + e of pixel i - one
-// NCHW44 dword. The patch's planes 4..7 sit 64 bytes further on in LDS so that the two channel
-// halves a 32-lane pass of an operand read touches fall on different banks.
-template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT, bool FCB, bool PM, bool RS = false, bool M16 = false>
+template <int FH, int FW, int KS, int LMAX, int ACT, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT, bool FCB, bool PM, bool RS = false>
 __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaParams q) {
     static_assert(!FCB || (FC && KS == 4 && FH * FW == 1), "FCB: FullyConnected, 128 channels per stage");
     static_assert(!RS || (FH == 1 && KS == 1 && !FC && !FCB && !PM), "RS: one filter row of one chunk per stage");
-    static_assert(!M16 || (PM && FH == 3 && FW == 3 && KS == 1), "M16: 3x3, plane-major patch, one chunk per stage");
-    constexpr int HALF_SKEW = M16 ? 64 : 0;
     constexpr int WGN = 4;
     constexpr int DM_BNP = 32 * NT * WGN;
     constexpr int DM_WAVES = WGM * WGN, DM_THREADS = 64 * DM_WAVES;
@@ -84,8 +71,8 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     constexpr int A_BYTES = TS * DM_BM * KROW;
     constexpr int A_CHUNKS = A_BYTES / 1024;
     constexpr int A_PER_WAVE = (A_CHUNKS + DM_WAVES - 1) / DM_WAVES;
-    constexpr int B_BYTES = KS * 2 * LMAX * 16 + HALF_SKEW;
-    constexpr int B_WL = (B_BYTES - HALF_SKEW) / (FCB || PM ? 1024 : 256);
+    constexpr int B_BYTES = KS * 2 * LMAX * 16;
+    constexpr int B_WL = B_BYTES / (FCB || PM ? 1024 : 256);
     static_assert(B_WL % DM_WAVES == 0 && LMAX % 16 == 0, "whole wave-loads");
     static_assert(!PM || (!FC && LMAX % 256 == 0), "PM: planes of whole 1 KB wave-loads");
     constexpr int PM_PARTS = LMAX / 256;  // wave-loads per plane
@@ -241,8 +228,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             if constexpr (FCB)
                 dma_global_b128(q.src + (b_goff[j] + poff), buf + A_BYTES + u * 1024);
             else if constexpr (PM)
-                dma_buffer_b128(src_rsrc, b_goff[j] + poff,
-                                buf + A_BYTES + u * 1024 + (M16 && u / PM_PARTS >= 4 ? HALF_SKEW : 0));
+                dma_buffer_b128(src_rsrc, b_goff[j] + poff, buf + A_BYTES + u * 1024);
             else if constexpr (RS)
                 dma_buffer_b32(src_rsrc,
                                (unsigned)(b_ih[j] + lfh * q.DH) < (unsigned)q.IH ? b_goff[j] + poff : 0x80000000u,
@@ -274,28 +260,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
         a_off[mi] = r * KROW + (((kg ^ (r >> 3)) & 1) << 4);
     }
 
-    v16i acc[M16 ? 1 : MT][M16 ? 1 : NT];
-    // M16: lane = (pixel or row i16 of a 16 x 16 tile, lane group g4); MT16 x NT16 tiles per wave
-    constexpr int MT16 = 2 * MT, NT16 = 2 * NT;
-    const int i16 = lane & 15, g4 = lane >> 4, half16 = g4 & 1, tsel = g4 >> 1;
-    int a_off16[M16 ? MT16 : 1], a_off8[M16 ? MT16 : 1];
-    int boff16[4];  // byte offset of tap 2j + tsel in the patch
-    v4i acc16[M16 ? MT16 : 1][M16 ? NT16 : 1];
-    if constexpr (M16) {
-#pragma unroll
-        for (int mi = 0; mi < MT16; ++mi) {
-            const int r = wm * MT * 32 + mi * 16 + i16;
-            // K = 64: the 16 channels of half16 of tap 2j + tsel (2j: an immediate of the read)
-            a_off16[mi] = r * KROW + (((half16 ^ (r >> 3)) & 1) << 4) + tsel * (DM_BM * KROW);
-            // K = 32 (the ninth tap): channels 8 g4 .. 8 g4 + 7 = half tsel, 8-byte piece half16
-            a_off8[mi] = r * KROW + (((tsel ^ (r >> 3)) & 1) << 4) + half16 * 8 + 8 * (DM_BM * KROW);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int t = 2 * j + tsel;
-            boff16[j] = ((t / 3) * q.DH * q.VW + (t % 3) * q.DW) * 4;
-        }
-    }
+    v16i acc[MT][NT];
 
     // Epilogue of one 32 oc x 32 pixel MFMA tile (16 outputs per lane = 4 NCHW44 dwords), written
     // as one straight-line block so that its 4 bias reads and 16 table look-ups are in flight
@@ -371,27 +336,8 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
         int b_byte[NT];  // LDS byte offset of this lane's 16 channels at tap (0,0)
         int cur_o[NT];
         int cols = 0;    // wave-uniform: 32-pixel columns of this wave with pixels of the sub-tile
-        int b_byte16[M16 ? NT16 : 1];  // M16: the same for the lane's pixel of each 16-pixel tile (half16's planes)
-        if constexpr (M16) {
 #pragma unroll
-            for (int ni = 0; ni < NT16; ++ni) {
-                const int pc = p0 + ((ni >> 1) * WGN + wn) * 32;  // the 32-pixel column of the tile
-                const int p = pc + (ni & 1) * 16 + i16;
-                b_byte16[ni] = (half16 * 4 * LMAX + (p <= plast ? vp_of(q, p) - vp0 : 0)) * 4 + half16 * HALF_SKEW;
-                if (ni & 1)
-                    cols += pc <= plast ? 1 : 0;
-            }
-#pragma unroll
-            for (int mi = 0; mi < MT16; ++mi) {
-                // register e of a tile: channel 4 * g4 + e of the tile's 16
-                const v4i bv = *(const v4i*)(bias_lds + wm * MT * 32 + mi * 16 + 4 * g4);
-#pragma unroll
-                for (int ni = 0; ni < NT16; ++ni)
-                    acc16[mi][ni] = bv;
-            }
-        }
-#pragma unroll
-        for (int ni = 0; ni < (M16 ? 0 : NT); ++ni) {
+        for (int ni = 0; ni < NT; ++ni) {
             // columns are dealt round-robin to the 4 pixel waves, so a partial sub-tile keeps
             // all of them busy
             const int pc = p0 + (ni * WGN + wn) * 32;
@@ -412,7 +358,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
         // the accumulators start from the bias of their output channel (register e of a tile:
         // channel 8 * (e / 4) + 4 * kg + e % 4)
 #pragma unroll
-        for (int mi = 0; mi < (M16 ? 0 : MT); ++mi) {
+        for (int mi = 0; mi < MT; ++mi) {
             v4i bv[4];
 #pragma unroll
             for (int e4 = 0; e4 < 4; ++e4)
@@ -429,69 +375,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             if (g + DM_NBUF - 1 < G)
                 issue(dma_buf);
             const int8_t* bufB = bufA + A_BYTES;
-            if constexpr (M16 && COLS > 0) {
-                // COLS 32-pixel columns = 2 COLS tiles of 16 pixels, multiplied in two halves of COLS
-                // tiles. Sub-step s = 2 j + h: operand pair j (taps 2j, 2j + 1; j = 4: the ninth tap
-                // alone, K = 32) against half h of the tiles; the reads of sub-step s + 1 are issued
-                // before the MFMAs of sub-step s.
-                typedef long v1l;
-                v4i fa[2][MT16], fb[2][COLS];
-                v1l fa8[MT16], fb8[2][COLS];
-                // planes 2 g4, 2 g4 + 1 of the ninth tap, relative to b_byte16 (half16's planes)
-                const int d8 = (2 * g4 - 4 * half16) * LMAX * 4 + (tsel - half16) * HALF_SKEW +
-                               (2 * q.DH * q.VW + 2 * q.DW) * 4;
-                auto fetch_a = [&](auto jc) __attribute__((always_inline)) {
-                    constexpr int j = decltype(jc)::value;
-                    if constexpr (j < 4) {
-#pragma unroll
-                        for (int mi = 0; mi < MT16; ++mi)
-                            fa[j & 1][mi] = *(const v4i*)(bufA + 2 * j * (DM_BM * KROW) + a_off16[mi]);
-                    } else {
-#pragma unroll
-                        for (int mi = 0; mi < MT16; ++mi)
-                            fa8[mi] = *(const v1l*)(bufA + a_off8[mi]);
-                    }
-                };
-                auto fetch_b = [&](auto sc) __attribute__((always_inline)) {
-                    constexpr int s = decltype(sc)::value, j = s >> 1, h = s & 1;
-#pragma unroll
-                    for (int t = 0; t < COLS; ++t) {
-                        const int ni = h * COLS + t;
-                        if constexpr (j < 4) {
-                            const int8_t* b0 = bufB + b_byte16[ni] + boff16[j];
-#pragma unroll
-                            for (int i = 0; i < 4; ++i)
-                                fb[s & 1][t][i] = *(const int*)(b0 + i * (LMAX * 4));
-                        } else {
-                            const int8_t* b0 = bufB + b_byte16[ni] + d8;
-                            const unsigned lo = *(const unsigned*)b0, hi = *(const unsigned*)(b0 + LMAX * 4);
-                            fb8[s & 1][t] = (v1l)(((unsigned long)hi << 32) | lo);
-                        }
-                    }
-                };
-                fetch_a(std::integral_constant<int, 0>{});
-                fetch_b(std::integral_constant<int, 0>{});
-                static_for<10>([&](auto sc) {
-                    constexpr int s = decltype(sc)::value, j = s >> 1, h = s & 1;
-                    if constexpr (s + 1 < 10) {
-                        if constexpr (h == 1)
-                            fetch_a(std::integral_constant<int, j + 1>{});
-                        fetch_b(std::integral_constant<int, s + 1>{});
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int t = 0; t < COLS; ++t)
-#pragma unroll
-                        for (int mi = 0; mi < MT16; ++mi) {
-                            if constexpr (j < 4)
-                                acc16[mi][h * COLS + t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-                                        fa[j & 1][mi], fb[s & 1][t], acc16[mi][h * COLS + t], 0, 0, 0);
-                            else
-                                acc16[mi][h * COLS + t] = __builtin_amdgcn_mfma_i32_16x16x32_i8(
-                                        fa8[mi], fb8[s & 1][t], acc16[mi][h * COLS + t], 0, 0, 0);
-                        }
-                });
-            } else if constexpr (COLS > 0) {
+            if constexpr (COLS > 0) {
                 v4i fa[2][MT], fb[2][NT];
                 auto fetch = [&](auto tc) __attribute__((always_inline)) {
                     constexpr int t = decltype(tc)::value;
@@ -550,66 +434,14 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
                 run_stages(cc);
         });
 
-        if constexpr (M16) {
-            // where each of the lane's pixels goes (worked out after the stages, so that it does not
-            // occupy registers during them): dword index of pixel p in channel group g4 of a tile,
-            // -1 for a lane beyond the sub-tile
-            int ob16[NT16];
-#pragma unroll
-            for (int ni = 0; ni < NT16; ++ni) {
-                const int p = p0 + ((ni >> 1) * WGN + wn) * 32 + (ni & 1) * 16 + i16;
-                const int pn = (int)fdiv(p, q.dOHW);
-                ob16[ni] = p > plast ? -1 : pn * (q.OC >> 2) * q.OHW + (p - pn * q.OHW) + g4 * q.OHW;
-            }
-            static_for<MT16>([&](auto mic) {
-                constexpr int mi = decltype(mic)::value;
-                const int oc = oc0 + wm * MT * 32 + mi * 16 + 4 * g4;
-                int8_t* const base = q.dst + ((size_t)(((oc0 + wm * MT * 32 + mi * 16) >> 2) * q.OHW) << 2);
-                int r[NT16][4];
-                if constexpr (ACT == ACT_RT) {
-#pragma unroll
-                    for (int ni = 0; ni < NT16; ++ni)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            r[ni][e] = requant_conv_rt(q.act, acc16[mi][ni][e], q.s_src, q.s_flt, q.s_dst);
-                } else if (ACT != MEGCC_NONLINE_H_SWISH && q.rq.aff_d != 0.f) {  // (uniform)
-#pragma unroll
-                    for (int ni = 0; ni < NT16; ++ni)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            r[ni][e] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(
-                                    acc16[mi][ni][e], q.rq.aff_c, q.rq.aff_d);
-                } else {
-                    int m[NT16][4], t[NT16][4];
-#pragma unroll
-                    for (int ni = 0; ni < NT16; ++ni)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            m[ni][e] = requant_table_candidate<ACT>(acc16[mi][ni][e], q.rq.c);
-                            t[ni][e] = rq_table[m[ni][e] + 128];
-                        }
-#pragma unroll
-                    for (int ni = 0; ni < NT16; ++ni)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            r[ni][e] = m[ni][e] + (acc16[mi][ni][e] > t[ni][e] ? 1 : 0);
-                }
-#pragma unroll
-                for (int ni = 0; ni < NT16; ++ni)
-                    if (ob16[ni] >= 0 && oc < q.OC)
-                        *(uint32_t*)(base + ((unsigned)ob16[ni] << 2)) =
-                                pack4_perm(r[ni][0], r[ni][1], r[ni][2], r[ni][3]);
-            });
-        } else {
-            static_for<MT>([&](auto mic) {
-                static_for<NT>([&](auto nic) { emit_tile(mic, nic, cur_o[decltype(nic)::value], rq_table); });
-            });
-        }
+        static_for<MT>([&](auto mic) {
+            static_for<NT>([&](auto nic) { emit_tile(mic, nic, cur_o[decltype(nic)::value], rq_table); });
+        });
     }
 }
 
 // ---- configurations --------------------------------------------------------------------------
-template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3, int WGM = 2, int BPC = 1, int NT = 2, bool FCB = false, bool PM = false, bool M16 = false>
+template <int FH, int FW, int KS, int LMAX, bool FC, int MT = 2, int DM_NBUF = 3, int WGM = 2, int BPC = 1, int NT = 2, bool FCB = false, bool PM = false>
 static PipeConfig make_dma_config(int act, bool table_ok);
 
 // row-split configurations (filters of more than 9 taps): 64 * MT oc x 128 * NT px, FW taps per stage
@@ -636,7 +468,7 @@ static PipeConfig make_rs_config(int act, bool table_ok) {
     return c;
 }
 
-template <int FH, int FW, int KS, int LMAX, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT, bool FCB, bool PM, bool M16>
+template <int FH, int FW, int KS, int LMAX, bool FC, int MT, int DM_NBUF, int WGM, int BPC, int NT, bool FCB, bool PM>
 static PipeConfig make_dma_config(int act, bool table_ok) {
     constexpr int DM_BM = 32 * MT * WGM;
     PipeConfig c;
@@ -649,17 +481,16 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     c.fixed_lmax = LMAX;
     c.pm = PM ? 1 : 0;
-    c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + (DM_BM > 128 ? DM_BM : 128) * 4 + (M16 ? 64 * DM_NBUF : 0);
-    c.m16 = M16 ? 1 : 0;
+    c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + (DM_BM > 128 ? DM_BM : 128) * 4;
     c.fcb = FCB ? 1 : 0;
-    c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM, false, M16>;
+    c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM, false, M16>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_IDENTITY, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
     else if (act == MEGCC_NONLINE_RELU && table_ok)
-        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM, false, M16>;
+        c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_RELU, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
     if constexpr (!FC) {  // (FullyConnected with H_SWISH keeps the literal sequence)
         if (act == MEGCC_NONLINE_H_SWISH && table_ok)
-            c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_H_SWISH, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM, false, M16>;
+            c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, MEGCC_NONLINE_H_SWISH, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
     }
     return c;
 }
@@ -734,10 +565,6 @@ bool conv_mfma_dma_config(const ConvGeom& g, bool fc, int variant, bool b128_ok,
             *c = make_dma_config<3, 3, 1, 768, false, 1, 2, 2, 1, 4, false, true>(g.act, ok);
         else if (g.oc < 128)
             *c = make_dma_config<3, 3, 1, 1024, false, 1, 2, 2, 1, 4, false, true>(g.act, ok);
-        else if (variant == 2 && !options().no_m16)
-            *c = make_dma_config<3, 3, 1, 768, false, 2, 2, 2, 1, 4, false, true, true>(g.act, ok);
-        else if (!options().no_m16)
-            *c = make_dma_config<3, 3, 1, 1024, false, 2, 2, 2, 1, 4, false, true, true>(g.act, ok);
         else if (variant == 2)
             *c = make_dma_config<3, 3, 1, 768, false, 2, 2, 2, 1, 4, false, true>(g.act, ok);
         else

@@ -35,6 +35,7 @@ struct DwNchwParams {
     int total;  // threads: planes * ohn * ogn
     int act;
     float s_src, s_flt, s_dst, cf;
+    float aff_c, aff_d;  // requantisation by one fused multiply-add (epilogue.h); aff_d == 0: table
     FastDiv d_ogn, d_oh, d_c;  // by ogn, ohn, c
     RequantTable table;
 };
@@ -126,6 +127,8 @@ __global__ void __launch_bounds__(256) dwconv_nchw_3x3_kernel(DwNchwParams q) {
 #pragma unroll
         for (int e = 0; e < G * 4; ++e)
             o[e] = ACT < 0 ? requant_conv_rt(q.act, acc[r][e], q.s_src, q.s_flt, q.s_dst)
+                   : q.aff_d != 0.f
+                           ? requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(acc[r][e], q.aff_c, q.aff_d)
                            : requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[r][e], q.cf, tbl);
         const int x0 = og * (G * 4);
         const int out = (plane * q.oh + oy + r) * q.ow + x0;
@@ -189,6 +192,9 @@ TinyNNStatus dwconv_nchw_launch(
     if (tab)
         q.table = requant_table_for(g.act, g.s_src, g.s_flt, g.s_dst);
     const int act = tab ? g.act : -1;
+    const RequantAffine aff = requant_affine_pick(tab, g.act, g.s_src, g.s_flt, g.s_dst);
+    q.aff_c = aff.c;
+    q.aff_d = aff.d;
     void (*kern)(DwNchwParams);
 #define MG_DWN_PICK(S_)                                                                         \
     (act == MEGCC_NONLINE_IDENTITY ? dwconv_nchw_3x3_kernel<S_, MEGCC_NONLINE_IDENTITY, G, R>    \

@@ -70,7 +70,7 @@ def test_cfg2_conv3x3_n32(c, hw, act, dst_scale):
     assert kernel.startswith("conv_mfma_i8_dma"), kernel
     if c == 256 and hw == 56:
         # the instantiation bench.py times: plane-major patch of 1024 slots, 128 oc x 512 px
-        assert kernel.split("+")[0] == "conv_mfma_i8_dma_m16:3,128,512,1024,1", kernel
+        assert kernel.split("+")[0] == "conv_mfma_i8_dma:3,128,512,1024,1", kernel
     one = ConvCase(A.FMT_NCHW44, A.DENSE, 1, c, hw, hw, c, 3, 1, 1, act, scales=scales)
     for i in (0, 17, 31):
         want = one.run_port({"src": arrays["src"][i:i + 1], "flt": arrays["flt"], "bias": arrays["bias"]})

@@ -63,6 +63,10 @@ def test_matches_reference_golden(name, golden):
 
 A = abi
 LIVE = [
+    # 512-pixel sub-tiles of the plane-major 3x3 kernel: ragged channel tile, three chunks of input
+    # channels, rows of 60 pixels; one channel tile (512-pixel sub-tiles from 57 600 pixels on)
+    ConvCase(A.FMT_NCHW44, A.DENSE, 9, 96, 56, 60, 200, 3, 1, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(864))),
+    ConvCase(A.FMT_NCHW44, A.DENSE, 20, 32, 56, 56, 128, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(288))),
     # headline kernel at its real channel counts (spatial size cut so the oracle stays fast)
     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 64, 56, 56, 64, 3, 1, 1, A.RELU, scales=(0.02, 0.01, 0.05)),
     ConvCase(A.FMT_NCHW44, A.DENSE, 2, 64, 56, 56, 64, 3, 1, 1, A.IDENTITY, scales=(0.02, 0.01, unsat(576))),
@@ -636,10 +640,6 @@ OLDER = [
                                scales=(0.02, 0.01, 0.05))),
     ("nopm", ConvCase(A.FMT_NCHW44, A.DENSE, 6, 32, 56, 56, 160, 3, 1, 1, A.RELU,
                             scales=(0.02, 0.01, unsat(288)))),
-    # the 32 x 32 x 32 MFMA form of the plane-major 3x3 kernel (the default is 16 x 16 x 64):
-    # ragged channel tile, three chunks of input channels, rows of 60 pixels
-    ("nom16", ConvCase(A.FMT_NCHW44, A.DENSE, 9, 96, 56, 60, 200, 3, 1, 1, A.H_SWISH,
-                       scales=(0.02, 0.01, unsat(864)))),
     # the plain tile order of the tiled GEMMs (the default gives each XCD a compact rectangle of
     # tiles): f32 MatMul with a ragged 9 x 8 grid of 128 x 128 tiles, all four transpositions,
     # FullyConnected with 256 x 256 tiles (8 x 8)
@@ -652,7 +652,7 @@ OLDER = [
     # the threshold table where the default is the one-multiply-add requantisation the host proved
     # exact for the layer's scales (scales without exact ties; "+affine" in the kernel's name):
     # pointwise streaming and workgroup-shared kernels, depthwise on the matrix cores and by v_dot4,
-    # the matrix-core first layer, the LDS-direct 3x3 kernel in both MFMA shapes
+    # the matrix-core first layer, the LDS-direct 3x3 kernel with 256- and 512-pixel sub-tiles
     ("noaffine", ConvCase(A.FMT_NCHW44, A.DENSE, 4, 32, 56, 56, 64, 1, 1, 0, A.RELU,
                           scales=(0.0213, 0.0097, unsat(32) * 1.0371))),
     ("noaffine", ConvCase(A.FMT_NCHW44, A.DENSE, 64, 512, 14, 14, 512, 1, 1, 0, A.RELU,
@@ -668,9 +668,6 @@ OLDER = [
                           scales=(0.0213, 0.0097, unsat(288) * 1.0371))),
     ("noaffine", ConvCase(A.FMT_NCHW44, A.DENSE, 20, 32, 56, 56, 128, 3, 1, 1, A.RELU,
                           scales=(0.0213, 0.0097, unsat(288) * 1.0371))),
-    # (one channel tile: 512-pixel sub-tiles from 57 600 pixels on)
-    ("nom16", ConvCase(A.FMT_NCHW44, A.DENSE, 20, 32, 56, 56, 128, 3, 1, 1, A.IDENTITY,
-                       scales=(0.02, 0.01, unsat(288)))),
     ("nodma512", ConvCase(A.FMT_NCHW44, A.DENSE, 22, 64, 54, 57, 128, 3, 1, 1, A.RELU,
                                 scales=(0.02, 0.01, unsat(576)))),
     ("nogevm", ConvCase(A.FMT_NCHW, A.DENSE, 1, 1024, 1, 1, 1000, 1, 1, 0, A.IDENTITY,

@@ -193,6 +193,12 @@ def make_workload(name):
         case = ConvCase(abi.FMT_NCHW44, abi.DENSE, 64, ic, hw, hw, oc, 1, 1, 0, abi.RELU,
                         scales=(0.02, 0.01, 0.05))
         return case, "qsi8 conv1x1 NCHW44 N=64 %d->%d %dx%d" % (ic, oc, hw, hw), "hbm"
+    if name.startswith("mb:"):  # mb:<layer> - a convolution of MobileNetV1 at batch 64 with its calibrated scales
+        import mobilenet
+        for kind, lname, case, _ in mobilenet.Net(64).steps:
+            if kind == "conv" and lname == name[3:]:
+                return case, "MobileNetV1 batch 64, layer %s: %s" % (lname, case.symbol()), "hbm"
+        raise SystemExit("bench.py: MobileNetV1 has no convolution called %r" % name[3:])
     if name == "fc":
         case = ConvCase(abi.FMT_NCHW, abi.DENSE, 4096, 4096, 1, 1, 4096, 1, 1, 0, abi.IDENTITY,
                         scales=(0.01, 0.01, 0.1))

@@ -226,17 +226,28 @@ __global__ void __launch_bounds__(256) dwconv44_3x3_kernel(
             // accumulator, so max F(a_i) = F(max a_i): pool the int32 accumulators first and requantise
             // 8 instead of 32 values (the pooled ones land where the code below looks for window k:
             // row 0, pixel 2 * k; the other three places get the same value)
+            int m[8], f[8];
+#pragma unroll
+            for (int k = 0; k < 2; ++k)
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    m[k * 4 + c] = max(max(acc[(2 * k) * 4 + c], acc[(2 * k + 1) * 4 + c]),
+                                       max(acc[16 + (2 * k) * 4 + c], acc[16 + (2 * k + 1) * 4 + c]));
+            if (rq.aff_d != 0.f) {  // (uniform; one branch around all eight)
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    f[i] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(m[i], rq.aff_c, rq.aff_d);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    f[i] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(m[i], rq.c, tbl);
+            }
 #pragma unroll
             for (int k = 0; k < 2; ++k)
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    const int m = max(max(acc[(2 * k) * 4 + c], acc[(2 * k + 1) * 4 + c]),
-                                      max(acc[16 + (2 * k) * 4 + c], acc[16 + (2 * k + 1) * 4 + c]));
-                    const int f = rq.aff_d != 0.f
-                                          ? requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(m, rq.aff_c, rq.aff_d)
-                                          : requant_conv_table<(ACT < 0 ? 0 : ACT)>(m, rq.c, tbl);
-                    acc[(2 * k) * 4 + c] = acc[(2 * k + 1) * 4 + c] = f;
-                    acc[16 + (2 * k) * 4 + c] = acc[16 + (2 * k + 1) * 4 + c] = f;
+                    acc[(2 * k) * 4 + c] = acc[(2 * k + 1) * 4 + c] = f[k * 4 + c];
+                    acc[16 + (2 * k) * 4 + c] = acc[16 + (2 * k + 1) * 4 + c] = f[k * 4 + c];
                 }
         } else if (ACT < 0) {
 #pragma unroll

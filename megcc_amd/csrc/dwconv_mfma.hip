@@ -120,9 +120,14 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
     const int gw = lb * 4 + __builtin_amdgcn_readfirstlane(tid >> 6);  // (scalar: the plane set's weights and bias come through the scalar cache)
     const int nw = gridDim.x * 4;
     const int c4 = gw % q.c4n;
+    // (runs of floor(tiles / waves) tiles, the first tiles % waves of them one longer: with runs of
+    //  the rounded-up length the last waves of a plane set had nothing to do - an eighth of them on
+    //  N=64 C=32 112x112, which cost that layer 5 % and its fused chain 14 %)
     const int wps = nw / q.c4n;                     // waves per plane set
-    const int run = (q.tiles + wps - 1) / wps;      // tiles per wave
-    const int t_end = min((gw / q.c4n + 1) * run, q.tiles);
+    const int wi = gw / q.c4n;                      // this wave's place among them
+    const int run_q = q.tiles / wps, run_r = q.tiles - run_q * wps;
+    const int t_begin = wi * run_q + min(wi, run_r);
+    const int t_end = t_begin + run_q + (wi < run_r ? 1 : 0);
 
     const __amdgpu_buffer_rsrc_t rs =
             __builtin_amdgcn_make_buffer_rsrc((void*)q.src, 0, q.src_bytes, 0x00020000);
@@ -184,16 +189,17 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
         return w;
     };
 
-    // The first tile's rows are requested before anything else is fetched: the threshold table, the
-    // weights and the bias then travel in the same memory round trip instead of one each in front
-    // of it (a 14 x 14 layer gives a wave two tiles, so the set-up is a third of its life).
+    // Order of the set-up: threshold table to LDS (one barrier), then the first tile's rows are
+    // requested, then the banded matrices are built while those loads fly. (Requesting the rows
+    // before the table copy made the barrier wait for them: 5 - 8 % slower on 14 x 14 and 112 x 112
+    // maps alike.)
     v4i B[IR][NS];
-    int tile = (gw / q.c4n) * run;
-    Where next = request(tile < t_end ? tile : q.tiles, B);
+    int tile = t_begin;
     if (ACT >= 0) {
         tbl[tid] = q.table.t[tid];
         __syncthreads();
     }
+    Where next = request(tile < t_end ? tile : q.tiles, B);
     // ---- the banded weight matrices of this plane set -------------------------------------------
     // row m = lane & 31 = (output pixel m / 4, channel m % 4); the lane's 16 K bytes are input
     // pixels 4 * kg + j (j = 0..3) of the K step, 4 channel bytes each. K step s starts 4 pixels
@@ -263,17 +269,27 @@ __global__ void __launch_bounds__(256) dwconv44_mfma_kernel(DwMfmaParams q) {
                 for (int e = 0; e < 16; ++e)
                     v[e] = max(acc[0][e], acc[1][e]);
                 // lower half wave: both halves of windows 0 and 1; upper: of windows 2 and 3
+                int w0[4], w1[4];  // the windows' maxima over the accumulators
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const dwm_v2u s02 = __builtin_amdgcn_permlane32_swap((unsigned)v[c], (unsigned)v[8 + c], false, false);
                     const dwm_v2u s13 = __builtin_amdgcn_permlane32_swap((unsigned)v[4 + c], (unsigned)v[12 + c], false, false);
-                    const int w0 = max((int)s02[0], (int)s02[1]), w1 = max((int)s13[0], (int)s13[1]);
-                    if (q.aff_d != 0.f) {  // (uniform)
-                        pooled[0][c] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(w0, q.aff_c, q.aff_d);
-                        pooled[1][c] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(w1, q.aff_c, q.aff_d);
-                    } else {
-                        pooled[0][c] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(w0, q.c, tbl);
-                        pooled[1][c] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(w1, q.c, tbl);
+                    w0[c] = max((int)s02[0], (int)s02[1]);
+                    w1[c] = max((int)s13[0], (int)s13[1]);
+                }
+                // (one uniform branch around all eight, so that the look-ups of the table form stay in
+                //  flight together)
+                if (q.aff_d != 0.f) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        pooled[0][c] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(w0[c], q.aff_c, q.aff_d);
+                        pooled[1][c] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(w1[c], q.aff_c, q.aff_d);
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        pooled[0][c] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(w0[c], q.c, tbl);
+                        pooled[1][c] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(w1[c], q.c, tbl);
                     }
                 }
             } else {
@@ -441,9 +457,6 @@ static TinyNNStatus dwconv44_mfma_run(
     long per_set = items <= cap ? q.tiles : cap / q.c4n;
     if (per_set < 1)
         per_set = 1;
-    // (no more waves than have a run of tiles: 56 tiles over 32 waves are runs of 2 for 28 of them)
-    const long run = (q.tiles + per_set - 1) / per_set;
-    per_set = (q.tiles + run - 1) / run;
     long waves = per_set * q.c4n;
     while (waves & 3) {  // (c4n odd: add whole rounds of plane sets until workgroups are full)
         waves += q.c4n;

@@ -124,12 +124,19 @@ __global__ void __launch_bounds__(256) dwconv_nchw_3x3_kernel(DwNchwParams q) {
         if (oy + r >= q.oh)
             break;
         int o[G * 4];
+        if (ACT < 0) {
 #pragma unroll
-        for (int e = 0; e < G * 4; ++e)
-            o[e] = ACT < 0 ? requant_conv_rt(q.act, acc[r][e], q.s_src, q.s_flt, q.s_dst)
-                   : q.aff_d != 0.f
-                           ? requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(acc[r][e], q.aff_c, q.aff_d)
-                           : requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[r][e], q.cf, tbl);
+            for (int e = 0; e < G * 4; ++e)
+                o[e] = requant_conv_rt(q.act, acc[r][e], q.s_src, q.s_flt, q.s_dst);
+        } else if (q.aff_d != 0.f) {  // (uniform)
+#pragma unroll
+            for (int e = 0; e < G * 4; ++e)
+                o[e] = requant_conv_affine<(ACT == MEGCC_NONLINE_RELU ? ACT : 0)>(acc[r][e], q.aff_c, q.aff_d);
+        } else {
+#pragma unroll
+            for (int e = 0; e < G * 4; ++e)
+                o[e] = requant_conv_table<(ACT < 0 ? 0 : ACT)>(acc[r][e], q.cf, tbl);
+        }
         const int x0 = og * (G * 4);
         const int out = (plane * q.oh + oy + r) * q.ow + x0;
 #pragma unroll

@@ -34,7 +34,8 @@ struct MfmaParams {
     int VW, VH, IH, IW, PH, PW, SH, SW, DH, DW;
     int image_stride, plane_stride, row_stride, pix_stride;  // bytes
     int Lmax;    // LDS patch slots (multiple of 64)
-    int dst_fc;  // 0: NCHW44, 1: [P][OC] row-major
+    int dst_fc;  // 0: NCHW44, 1: [P][OC] row-major, 2: the same with OC a multiple of 32 and a 16-byte aligned base,
+                 // 3: 2 and the LDS-direct kernel's FullyConnected tile (rows leave through LDS)
     int bias_vec4;  // bias pointer is 16-byte aligned
     int range_len;  // pixels per workgroup of the pipelined kernel (multiple of 32)
     int act;

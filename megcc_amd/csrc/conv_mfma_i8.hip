@@ -649,7 +649,7 @@ TinyNNStatus conv_mfma_launch(
         q.pix_stride = 4;
     }
     q.Lmax = t.Lmax;
-    q.dst_fc = fc ? 1 : 0;
+    q.dst_fc = fc ? ((g.oc & 31) == 0 && ((uintptr_t)dst & 15) == 0 ? 2 : 1) : 0;
     q.bias_vec4 = bias && ((uintptr_t)bias & 15) == 0;
     q.act = g.act;
     q.s_src = g.s_src;
@@ -674,6 +674,8 @@ TinyNNStatus conv_mfma_launch(
         q.xo = pc.fcb && !options().no_xcdorder
                        ? make_xcd_order((q.P + q.range_len - 1) / q.range_len, (q.OC + pc.bm - 1) / pc.bm)
                        : XcdOrder{0};
+        if (pc.fcb && pc.bm == 256 && q.dst_fc == 2)
+            q.dst_fc = 3;  // rows leave through the kernel's staging area in LDS
         note_kernel(q.xo.w ? "conv_mfma_i8_dma_xo" : "conv_mfma_i8_dma", picked,
                     pc.bm, pc.bn, q.Lmax, pc.ks);
         const RequantAffine aff = requant_affine_pick(

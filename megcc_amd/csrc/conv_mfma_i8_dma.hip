@@ -63,6 +63,7 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     static_assert(!FCB || (FC && KS == 4 && FH * FW == 1), "FCB: FullyConnected, 128 channels per stage");
     static_assert(!RS || (FH == 1 && KS == 1 && !FC && !FCB && !PM), "RS: one filter row of one chunk per stage");
     constexpr int WGN = 4;
+    constexpr int FC_STAGE_ROW = 80, FC_STAGE_BYTES = 32 * FC_STAGE_ROW;  // (FCB: a wave's staging rows)
     constexpr int DM_BNP = 32 * NT * WGN;
     constexpr int DM_WAVES = WGM * WGN, DM_THREADS = 64 * DM_WAVES;
     constexpr int DM_BM = 32 * MT * WGM;
@@ -266,12 +267,9 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
     // as one straight-line block so that its 4 bias reads and 16 table look-ups are in flight
     // together. ob: dword index in dst of this lane's pixel in oc-group 0 (-1: lane beyond the
     // sub-tile, -2: whole 32-pixel column beyond it, wave-uniform).
-    auto emit_tile = [&](auto mic, auto nic, const int ob, const int* tbl) __attribute__((always_inline)) {
+    // the 16 requantised outputs of this lane in tile (mi, ni)
+    auto requant_tile = [&](auto mic, auto nic, int (&r)[16], const int* tbl) __attribute__((always_inline)) {
         constexpr int mi = decltype(mic)::value, ni = decltype(nic)::value;
-        if (ob < -1)
-            return;
-        const int ocl = (wm * MT + mi) * 32 + kg * 4;
-        int r[16];
         if constexpr (ACT == ACT_RT) {
 #pragma unroll
             for (int e = 0; e < 16; ++e)
@@ -291,6 +289,41 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
             for (int e = 0; e < 16; ++e)
                 r[e] = m[e] + (acc[mi][ni][e] > t[e] ? 1 : 0);
         }
+    };
+    // (FC, dst_fc >= 2) the lane's 16 bytes of tile (mi, ni): channels 16 kg .. + 15 of the tile, row =
+    // the lane's column. A lane's four dwords are channels 8 e4 + 4 kg .. + 3, so lanes l and l + 32
+    // (same row, the two K-halves) together own 32 consecutive bytes; two v_permlane32_swap give the
+    // lower lane the first 16 of them and the upper lane the rest.
+    auto fc_piece = [&](auto mic, auto nic, const int* tbl) __attribute__((always_inline)) -> v4u {
+        typedef unsigned v2u_t __attribute__((ext_vector_type(2)));
+        int r[16];
+        requant_tile(mic, nic, r, tbl);
+        uint32_t w[4];
+#pragma unroll
+        for (int e4 = 0; e4 < 4; ++e4)
+            w[e4] = pack4_perm(r[e4 * 4], r[e4 * 4 + 1], r[e4 * 4 + 2], r[e4 * 4 + 3]);
+        const v2u_t s02 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
+        const v2u_t s13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+        return v4u{s02[0], s02[1], s13[0], s13[1]};
+    };
+    auto emit_tile = [&](auto mic, auto nic, const int ob, const int* tbl) __attribute__((always_inline)) {
+        constexpr int mi = decltype(mic)::value;
+        if (ob < -1)
+            return;
+        const int ocl = (wm * MT + mi) * 32 + kg * 4;
+        if constexpr (FC) {
+            // Row-major [row][OC] output with whole 32-channel tiles and 16-byte alignment: one 16-byte
+            // store per lane instead of four dword stores 4096 bytes apart from their neighbours' (the
+            // dword stores were half of the 4096 x 4096 x 4096 layer's time).
+            if (q.dst_fc >= 2) {  // (uniform)
+                const v4u px = fc_piece(mic, nic, tbl);
+                if (ob >= 0 && oc0 + (wm * MT + mi) * 32 < q.OC)  // (whole tiles: OC is a multiple of 32)
+                    *(v4u*)(q.dst + (size_t)ob * q.OC + oc0 + (wm * MT + mi) * 32 + kg * 16) = px;
+                return;
+            }
+        }
+        int r[16];
+        requant_tile(mic, nic, r, tbl);
         if (ob >= 0) {
 #pragma unroll
             for (int e4 = 0; e4 < 4; ++e4) {
@@ -434,6 +467,37 @@ __global__ void __launch_bounds__(256 * WGM, BPC) conv_mfma_i8_dma_kernel(MfmaPa
                 run_stages(cc);
         });
 
+        if constexpr (FCB && MT == 4) {  // (the 256-channel tile: its two stage buffers leave room for the staging area)
+            // dst_fc == 3: the rows leave through a staging area in LDS (this wave's own 32 rows x 64
+            // bytes, rows 80 bytes apart): the lanes park the 16-byte pieces of two neighbouring tiles
+            // and read them back four lanes to a row, so that a store instruction writes 64 contiguous
+            // bytes of each of 16 rows instead of 32 bytes of each of 32.
+            if (q.dst_fc == 3) {  // (uniform)
+                int8_t* const stage = (int8_t*)(bias_lds + (DM_BM > 128 ? DM_BM : 128)) + wave * FC_STAGE_BYTES;
+                static_for<NT>([&](auto nic) {
+                    constexpr int ni = decltype(nic)::value;
+                    if (cur_o[ni] < -1)
+                        return;
+                    const int row0 = p0 + (ni * WGN + wn) * 32;  // first row of this 32-row column
+                    static_for<MT / 2>([&](auto hc) {
+                        constexpr int h = decltype(hc)::value;
+                        const v4u pa = fc_piece(std::integral_constant<int, 2 * h>{}, nic, rq_table);
+                        const v4u pb = fc_piece(std::integral_constant<int, 2 * h + 1>{}, nic, rq_table);
+                        *(v4u*)(stage + (lane & 31) * FC_STAGE_ROW + kg * 16) = pa;
+                        *(v4u*)(stage + (lane & 31) * FC_STAGE_ROW + 32 + kg * 16) = pb;
+                        const int ocb = oc0 + (wm * MT + 2 * h) * 32;  // (64 channels from here on)
+#pragma unroll
+                        for (int it = 0; it < 2; ++it) {
+                            const int rr = (lane >> 2) + 16 * it, piece = lane & 3;
+                            const v4u v = *(const v4u*)(stage + rr * FC_STAGE_ROW + piece * 16);
+                            if (row0 + rr <= plast && ocb + piece * 16 < q.OC)
+                                *(v4u*)(q.dst + (size_t)(row0 + rr) * q.OC + ocb + piece * 16) = v;
+                        }
+                    });
+                });
+                continue;
+            }
+        }
         static_for<MT>([&](auto mic) {
             static_for<NT>([&](auto nic) { emit_tile(mic, nic, cur_o[decltype(nic)::value], rq_table); });
         });
@@ -481,7 +545,8 @@ static PipeConfig make_dma_config(int act, bool table_ok) {
     c.a_bytes = FH * FW * KS * c.bm * KROW;
     c.fixed_lmax = LMAX;
     c.pm = PM ? 1 : 0;
-    c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + (DM_BM > 128 ? DM_BM : 128) * 4;
+    c.extra_lds = REQUANT_TABLE_ENTRIES * 4 + (DM_BM > 128 ? DM_BM : 128) * 4 +
+                  (FCB && MT == 4 ? 4 * WGM * 32 * 80 : 0);  // (32 rows x 80 bytes of staging per wave)
     c.fcb = FCB ? 1 : 0;
     c.kernel = (const void*)conv_mfma_i8_dma_kernel<FH, FW, KS, LMAX, ACT_RT, FC, MT, DM_NBUF, WGM, BPC, NT, FCB, PM>;
     if (act == MEGCC_NONLINE_IDENTITY && table_ok)

@@ -63,6 +63,13 @@ def test_matches_reference_golden(name, golden):
 
 A = abi
 LIVE = [
+    # FullyConnected on the LDS-direct kernel, row-major output in 16-byte pieces: the 256 x 256 tile whose
+    # rows leave through LDS (ragged rows, a partial channel tile of 32), the 128-channel tile, and a K
+    # that is no multiple of 128 (dword activation loads); 2040 outputs (no multiple of 32): dword stores
+    ConvCase(A.FMT_NCHW, A.DENSE, 2100, 256, 1, 1, 288, 1, 1, 0, A.RELU, scales=(0.02, 0.01, unsat(256))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 2100, 256, 1, 1, 160, 1, 1, 0, A.IDENTITY, scales=(0.0213, 0.0097, unsat(256) * 1.0371)),
+    ConvCase(A.FMT_NCHW, A.DENSE, 2100, 160, 1, 1, 320, 1, 1, 0, A.IDENTITY, scales=(0.02, 0.01, unsat(160))),
+    ConvCase(A.FMT_NCHW, A.DENSE, 2100, 256, 1, 1, 2040, 1, 1, 0, A.H_SWISH, scales=(0.02, 0.01, unsat(256))),
     # 512-pixel sub-tiles of the plane-major 3x3 kernel: ragged channel tile, three chunks of input
     # channels, rows of 60 pixels; one channel tile (512-pixel sub-tiles from 57 600 pixels on)
     ConvCase(A.FMT_NCHW44, A.DENSE, 9, 96, 56, 60, 200, 3, 1, 1, A.H_SWISH, scales=(0.02, 0.01, unsat(864))),

@@ -628,9 +628,12 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model);
  * only replaced when its result shares no byte with anything the one kernel reads), and how they
  * are launched: 1 = HIP-graph replay, -1 = one launch per kernel, 0 = still measuring. forward()
  * 2, 3 and 5 to 10 of a model with at least 5 kernels each block the host until that forward has
- * finished (they time the two ways between events on the library stream; *eager_ms / *graph_ms
- * receive the shortest of four samples each, -1 when not measured; the replay is kept when it is
- * at least 2 % faster); every other forward is asynchronous. */
+ * finished (they time the two ways between events on the library stream; a sample is the time on
+ * the device or the time the host took to enqueue the forward, whichever is longer - what limits
+ * back-to-back forwards; *eager_ms / *graph_ms receive the shortest of four samples each, -1 when
+ * not measured; the replay is kept when it is at least 2 % faster, or not more than 5 % slower
+ * when the kernels average under 6 us each - back-to-back plain launches of such a model are bound
+ * by the host); every other forward is asynchronous. */
 int megcc_gfx950_model_nr_kernel(void* model);
 int megcc_gfx950_model_launch_mode(void* model, float* eager_ms, float* graph_ms);
 size_t megcc_gfx950_model_arena_bytes(void* model);

@@ -444,7 +444,8 @@ typedef enum {
     MEGCC_KERN_RESIZE = 10,
     MEGCC_KERN_FUSED_ELEMWISE = 11, /* never produced by parse_symbol; a caller fills the attr */
     MEGCC_KERN_SOFTMAX = 12,        /* never produced by parse_symbol either: see megcc_gfx950_softmax */
-    MEGCC_KERN_DW_POOL_ADD = 13     /* nor this one: see megcc_gfx950_dw_pool_add */
+    MEGCC_KERN_DW_POOL_ADD = 13,    /* nor this one: see megcc_gfx950_dw_pool_add */
+    MEGCC_KERN_PW_DW = 14           /* nor this one: see megcc_gfx950_pw_dw */
 } MegccKernelKind;
 
 /* A channel-wise 3x3 convolution, the 2x2 stride-2 maximum pooling of its result and the quantised
@@ -457,6 +458,14 @@ typedef struct {
     MegccMultiTypeMode mode; /* MEGCC_Q_ADD or MEGCC_Q_FUSE_ADD_RELU */
     float mid_scale;
 } MegccDwPoolAddAttr;
+
+/* A pointwise (1x1) convolution and the channel-wise 3x3 convolution of its result as one operator
+ * (megcc_gfx950_pw_dw): the attributes of the two and the scale of the tensor between them. */
+typedef struct {
+    MegccConvAttr pw;
+    MegccConvAttr dw;
+    float mid_scale;
+} MegccPwDwAttr;
 
 typedef struct {
     MegccKernelKind kind;
@@ -471,6 +480,7 @@ typedef struct {
         MegccResizeAttr resize;
         MegccFusedElemwiseAttr fused;
         MegccDwPoolAddAttr dw_pool_add;
+        MegccPwDwAttr pw_dw;
     } attr;
 } MegccKernelDesc;
 
@@ -493,6 +503,27 @@ TinyNNStatus megcc_gfx950_dw_pool_add(
         const Workspace* workspace, const RuntimeOpt* opt);
 int megcc_gfx950_dw_pool_add_supported(
         const MegccDwPoolAddAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output);
+
+/* Pointwise 1x1 convolution -> channel-wise 3x3 convolution in ONE kernel, for images of at most 31
+ * pixels a row. MegCC emits two kernels for the pair (kernel_conv2d_1x1_NCHW44_DENSE_... and
+ * kernel_conv2d_3x3_NCHW44_GROUP_..., BareMetal/ConvKernel.cpp:144-176, loops :305-344); on the 14 x 14
+ * and 7 x 7 images at the end of a MobileNet each of them is over before the chip is filled, so
+ * their cost is launches and the trip of the tensor in between through memory. Here a workgroup
+ * owns one image and 64 or 128 output channels, keeps its slice of the pointwise filter and the
+ * pointwise result (channel-planar, zero border included) in LDS and runs the 3x3 window from
+ * there. The model runtime launches this entry point instead of the two kernels when nothing else
+ * reads the tensor between them; the two kernels stay available under their symbols.
+ * qsi8 NCHW44 only. pw: DENSE 1x1, stride 1, pad 0, 128 / 256 / 512 input channels, output
+ * channels a multiple of 64; dw: GROUP (channel-wise) 3x3, pad 1, stride 1 or 2, dilation 1; both with
+ * IDENTITY or RELU; image width 4..31. inputs: source, the pointwise filter as megcc_gfx950_conv2d_init
+ * returns it for `pw`, pointwise bias (when pw has one), channel-wise filter, channel-wise bias (when dw
+ * has one); outputs[0]: the channel-wise layer's result. Bit-identical to the two kernels run in
+ * sequence. megcc_gfx950_pw_dw_supported returns 1 for operands this entry point takes. */
+TinyNNStatus megcc_gfx950_pw_dw(
+        const MegccPwDwAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace* workspace, const RuntimeOpt* opt);
+int megcc_gfx950_pw_dw_supported(
+        const MegccPwDwAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output);
 
 /* Soft-max over the last axis in ONE kernel. MegCC has no such kernel: its importer decomposes
  * opr::Softmax into Reduce MAX -> SUB -> EXP -> Reduce SUM -> TRUE_DIV
@@ -561,8 +592,9 @@ int megcc_gfx950_requant_affine(int nonline_mode, float s_src, float s_flt, floa
 /* Kernel-selection overrides, for regression tests of kernels that un-switched shapes only reach
  * through a fallback: "nopws", "nogevm", "nofcb", "nosmall", "nopm768", "nopm", "nodma512",
  * "nopm256", "nodma", "nofcs", "nopwshare", "nohybrid", "nodot4", "nof32small",
- * "dw_generic", "nodwmfma", "nodwnchw", "nofusesoftmax", "nopoolrows", "nofirstmfma", "norowsplit", "nofusechain", "nofcone", "noxcdorder", "noaffine", "no_graph"; value 1 takes the kernel out
- * of the dispatch, 0 puts it back. The
+ * "dw_generic", "nodwmfma", "nodwnchw", "nofusesoftmax", "nopoolrows", "nofirstmfma", "norowsplit", "nofusechain", "nofusepwdw", "fusepwdw", "nofcone", "noxcdorder", "noaffine", "no_graph"; value 1 takes the kernel out
+ * of the dispatch, 0 puts it back ("fusepwdw": 1 makes the model runtime take the one-kernel form of a
+ * pointwise / channel-wise pair wherever it applies instead of timing both forms). The
  * same names in capitals behind MEGCC_ are read from the environment once, at first use.
  * Unknown names return TinyNN_ERROR_NO_FOUND. */
 TinyNNStatus megcc_gfx950_set_option(const char* name, int value);

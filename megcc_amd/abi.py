@@ -47,6 +47,7 @@ KERN_CONV, KERN_MATMUL, KERN_POOLING, KERN_ELEMWISE_MULTITYPE = 1, 2, 3, 4
 KERN_ELEMWISE, KERN_TYPECVT, KERN_REDUCE = 5, 6, 7
 KERN_RELAYOUT, KERN_CONCAT, KERN_RESIZE, KERN_FUSED_ELEMWISE, KERN_SOFTMAX = 8, 9, 10, 11, 12
 KERN_DW_POOL_ADD = 13
+KERN_PW_DW = 14
 IMODE_NEAREST, IMODE_LINEAR = 0, 1
 
 
@@ -180,12 +181,16 @@ class DwPoolAddAttr(C.Structure):
     _fields_ = [("conv", ConvAttr), ("pool", PoolAttr), ("mode", C.c_int), ("mid_scale", C.c_float)]
 
 
+class PwDwAttr(C.Structure):
+    _fields_ = [("pw", ConvAttr), ("dw", ConvAttr), ("mid_scale", C.c_float)]
+
+
 class _KernelAttrUnion(C.Union):
     _fields_ = [
         ("conv", ConvAttr), ("matmul", MatMulAttr), ("pool", PoolAttr),
         ("multitype", C.c_int), ("elemwise", C.c_int), ("reduce", ReduceAttr),
         ("concat_axis", C.c_int), ("resize", ResizeAttr), ("fused", FusedElemwiseAttr),
-        ("dw_pool_add", DwPoolAddAttr),
+        ("dw_pool_add", DwPoolAddAttr), ("pw_dw", PwDwAttr),
     ]
 
 

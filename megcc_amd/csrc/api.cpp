@@ -332,6 +332,8 @@ extern "C" TinyNNStatus megcc_gfx950_call(
             return megcc_gfx950_softmax(inputs, nr_input, outputs, nr_output, ws, opt);
         case MEGCC_KERN_DW_POOL_ADD:
             return megcc_gfx950_dw_pool_add(&d->attr.dw_pool_add, inputs, nr_input, outputs, nr_output, ws, opt);
+        case MEGCC_KERN_PW_DW:
+            return megcc_gfx950_pw_dw(&d->attr.pw_dw, inputs, nr_input, outputs, nr_output, ws, opt);
         case MEGCC_KERN_CONCAT:
             return megcc_gfx950_concat(&d->attr.concat_axis, inputs, nr_input, outputs, nr_output,
                                        ws, opt);

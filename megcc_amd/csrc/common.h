@@ -62,7 +62,7 @@ __device__ __forceinline__ void xcd_tile(XcdOrder o, int bx, int by, int gx, int
 // environment (MEGCC_NOPWS=1, ...) ONCE, when the library first consults them; later changes go
 // through megcc_gfx950_set_option(). Nothing on a launch path scans the environment.
 struct Options {
-    bool no_pws, no_gevm, no_fcb, no_small, no_pm768, no_pm, no_dma512, no_pm256, no_dma, no_fcs, no_pwshare, no_hybrid, no_dot4, no_f32small, dw_generic, no_dwmfma, no_dwnchw, no_fuse_softmax, no_graph, no_poolrows, no_firstmfma, no_rowsplit, no_fuse_chain, no_fcone, no_xcdorder, no_affine;
+    bool no_pws, no_gevm, no_fcb, no_small, no_pm768, no_pm, no_dma512, no_pm256, no_dma, no_fcs, no_pwshare, no_hybrid, no_dot4, no_f32small, dw_generic, no_dwmfma, no_dwnchw, no_fuse_softmax, no_graph, no_poolrows, no_firstmfma, no_rowsplit, no_fuse_chain, no_fuse_pwdw, fuse_pwdw, no_fcone, no_xcdorder, no_affine;
 };
 Options& options();
 

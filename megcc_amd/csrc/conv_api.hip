@@ -46,6 +46,10 @@ TinyNNStatus conv_f32_gemm_launch(const ConvGeom&, const void*, const void*, con
                                   const Workspace*);
 size_t conv_f32_gemm_workspace_bytes(const ConvGeom& g);
 TinyNNStatus conv_direct_launch(const ConvGeom&, bool, const void*, const void*, const void*, void*);
+bool conv_pw_dw_supported(const ConvGeom& pw, const ConvGeom& dw, const void* src, const void* dst);
+TinyNNStatus conv_pw_dw_launch(
+        const ConvGeom& pw, const ConvGeom& dw, const void* src, const void* packed, const void* pw_bias,
+        const void* dw_flt, const void* dw_bias, void* dst);
 
 // A filter that went through megcc_gfx950_conv2d_init is a 1-d byte tensor.
 static bool is_packed_filter(const Tensor* flt) {
@@ -746,4 +750,98 @@ extern "C" TinyNNStatus megcc_gfx950_dw_pool_add(
             g, inputs[0]->ptr, inputs[1]->ptr, attr->conv.with_bias ? inputs[2]->ptr : nullptr, other->ptr,
             outputs[0]->ptr, attr->mode == MEGCC_Q_FUSE_ADD_RELU, other->dtype.param.scale,
             outputs[0]->dtype.param.scale);
+}
+
+// ---- pointwise 1x1 -> channel-wise 3x3 as one operator -------------------------------------------
+// Fills the two layers' geometries (pw.s_dst = dw.s_src = the scale in between) and checks the
+// operands; `why` gets the reason when they are not what the kernel takes.
+struct PwDwOperands {
+    const Tensor *src, *packed, *pw_bias, *dw_flt, *dw_bias, *dst;
+};
+static bool pw_dw_geom(
+        const MegccPwDwAttr* a, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output, ConvGeom* pw,
+        ConvGeom* dw, PwDwOperands* t, const char** why) {
+    *why = "NULL argument";
+    if (!a || !inputs || !outputs || nr_output != 1 || !outputs[0])
+        return false;
+    *why = "inputs: source, packed pointwise filter, [pointwise bias,] channel-wise filter [, channel-wise bias]";
+    if (nr_input != 3 + (a->pw.with_bias ? 1 : 0) + (a->dw.with_bias ? 1 : 0))
+        return false;
+    for (int i = 0; i < nr_input; ++i)
+        if (!inputs[i])
+            return false;
+    int k = 0;
+    t->src = inputs[k++];
+    t->packed = inputs[k++];
+    t->pw_bias = a->pw.with_bias ? inputs[k++] : nullptr;
+    t->dw_flt = inputs[k++];
+    t->dw_bias = a->dw.with_bias ? inputs[k++] : nullptr;
+    t->dst = outputs[0];
+    *why = "operands must be qsi8 (biases qsi32)";
+    if (!is_q8(t->src) || !is_q8(t->packed) || !is_q8(t->dw_flt) || !is_q8(t->dst) ||
+        (t->pw_bias && !is_q32(t->pw_bias)) || (t->dw_bias && !is_q32(t->dw_bias)))
+        return false;
+    *why = "pw: NCHW44 DENSE 1x1 with the filter from megcc_gfx950_conv2d_init; dw: NCHW44 GROUP 3x3";
+    if (a->pw.format != MEGCC_FMT_NCHW44 || a->pw.sparse != MEGCC_SPARSE_DENSE || a->dw.format != MEGCC_FMT_NCHW44 ||
+        a->dw.sparse != MEGCC_SPARSE_GROUP || !is_packed_filter(t->packed) || is_packed_filter(t->dw_flt) ||
+        !(a->mid_scale > 0.f) || t->dw_flt->layout.nr_dim < 1)
+        return false;
+    *why = "source / filter / destination layout";
+    const int oc = (int)t->dw_flt->layout.dims[0] * 4;
+    if (make_geom(&a->pw, t->src, t->packed, nullptr, true, oc, pw) != TinyNN_SUCCESS || pw->oh <= 0 || pw->ow <= 0)
+        return false;
+    pw->s_dst = a->mid_scale;
+    Tensor mid = {};
+    mid.dtype.type_enum = TinyNN_QINT8;
+    mid.dtype.param.scale = a->mid_scale;
+    mid.layout.nr_dim = 5;
+    const uint32_t md[5] = {(uint32_t)pw->n, (uint32_t)(oc / 4), (uint32_t)pw->oh, (uint32_t)pw->ow, 4u};
+    int stride = 1;
+    for (int i = 4; i >= 0; --i) {
+        mid.layout.dims[i] = md[i];
+        mid.layout.stride[i] = stride;
+        stride *= (int)md[i];
+    }
+    if (make_geom(&a->dw, &mid, t->dw_flt, t->dst, false, 0, dw) != TinyNN_SUCCESS)
+        return false;
+    *why = "packed filter size";
+    if (!conv_mfma_supported(*pw) || nr_elem(t->packed->layout) != conv_mfma_packed_bytes(*pw))
+        return false;
+    *why = "biases must be per channel, with the scale source scale * filter scale";
+    for (const Tensor* b : {t->pw_bias, t->dw_bias}) {
+        if (!b)
+            continue;
+        if (!(nr_elem(b->layout) == (size_t)oc && is_contiguous(b->layout) && aligned4(b->ptr)))
+            return false;
+        // ConvGeneral::IsAvailable, BareMetal/ConvKernel.cpp:37-42
+        const ConvGeom& g = b == t->pw_bias ? *pw : *dw;
+        const float d = g.s_src * g.s_flt - b->dtype.param.scale;
+        if (!((d < 0 ? -d : d) < 1e-5f))
+            return false;
+    }
+    *why = "shape, activation, alignment or extent the kernel does not take";
+    return conv_pw_dw_supported(*pw, *dw, t->src->ptr, t->dst->ptr) && aligned16(t->packed->ptr) &&
+           aligned4(t->dw_flt->ptr);
+}
+
+extern "C" int megcc_gfx950_pw_dw_supported(
+        const MegccPwDwAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output) {
+    ConvGeom pw, dw;
+    PwDwOperands t;
+    const char* why = "";
+    return pw_dw_geom(attr, inputs, nr_input, outputs, nr_output, &pw, &dw, &t, &why) ? 1 : 0;
+}
+
+extern "C" TinyNNStatus megcc_gfx950_pw_dw(
+        const MegccPwDwAttr* attr, Tensor** inputs, int nr_input, Tensor** outputs, int nr_output,
+        const Workspace*, const RuntimeOpt*) {
+    ConvGeom pw, dw;
+    PwDwOperands t;
+    const char* why = "";
+    MG_REQUIRE(pw_dw_geom(attr, inputs, nr_input, outputs, nr_output, &pw, &dw, &t, &why),
+               TinyNN_ERROR_INVALID_LAYOUT, "pw_dw: %s", why);
+    note_kernel("conv_pw_dw", pw.ic / 32, dw.sh);
+    return conv_pw_dw_launch(
+            pw, dw, t.src->ptr, t.packed->ptr, t.pw_bias ? t.pw_bias->ptr : nullptr, t.dw_flt->ptr,
+            t.dw_bias ? t.dw_bias->ptr : nullptr, t.dst->ptr);
 }

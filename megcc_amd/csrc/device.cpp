@@ -32,7 +32,7 @@ const OptionName kOptions[] = {
         {"nodot4", &Options::no_dot4},       {"nof32small", &Options::no_f32small},
         {"dw_generic", &Options::dw_generic}, {"no_graph", &Options::no_graph},
         {"nodwmfma", &Options::no_dwmfma},   {"nodwnchw", &Options::no_dwnchw},
-        {"nofusesoftmax", &Options::no_fuse_softmax}, {"nopoolrows", &Options::no_poolrows}, {"nofirstmfma", &Options::no_firstmfma}, {"norowsplit", &Options::no_rowsplit}, {"nofusechain", &Options::no_fuse_chain}, {"nofcone", &Options::no_fcone}, {"noxcdorder", &Options::no_xcdorder}, {"noaffine", &Options::no_affine},
+        {"nofusesoftmax", &Options::no_fuse_softmax}, {"nopoolrows", &Options::no_poolrows}, {"nofirstmfma", &Options::no_firstmfma}, {"norowsplit", &Options::no_rowsplit}, {"nofusechain", &Options::no_fuse_chain}, {"nofusepwdw", &Options::no_fuse_pwdw}, {"fusepwdw", &Options::fuse_pwdw}, {"nofcone", &Options::no_fcone}, {"noxcdorder", &Options::no_xcdorder}, {"noaffine", &Options::no_affine},
 };
 struct KernelNote {
     const char* name;

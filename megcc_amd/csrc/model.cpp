@@ -110,6 +110,32 @@ int root_of(const Model* m, int id) {
 bool plan_memory(Model* m) {
     if (m->preplanned)
         return true;
+    // A pointwise convolution followed by the channel-wise 3x3 convolution of its result may run
+    // as one kernel (build_schedule), which reads the pointwise layer's source while it writes the
+    // channel-wise layer's result: that source stays alive one operator longer, as it would in a
+    // plan made for the one operator.
+    std::vector<int> keep_until(m->tensors.size(), -1);
+    for (size_t i = 0; !options().no_fuse_pwdw && i + 1 < m->oprs.size(); ++i) {
+        const ModelOpr *o0 = m->oprs[i], *o1 = m->oprs[i + 1];
+        if (o0->desc.kind != MEGCC_KERN_CONV || o1->desc.kind != MEGCC_KERN_CONV || o0->in.empty() ||
+            o1->in.empty() || o0->out.size() != 1 || o1->in[0] != o0->out[0])
+            continue;
+        const MegccConvAttr &a = o0->desc.attr.conv, &b = o1->desc.attr.conv;
+        if (a.format == MEGCC_FMT_NCHW44 && a.sparse == MEGCC_SPARSE_DENSE && a.kernel_h == 1 && a.kernel_w == 1 &&
+            a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 0 && a.pad_w == 0 && b.format == MEGCC_FMT_NCHW44 &&
+            b.sparse == MEGCC_SPARSE_GROUP && b.kernel_h == 3 && b.kernel_w == 3 && b.pad_h == 1 && b.pad_w == 1) {
+            // ... where the one kernel can win at all: shapes it takes, and no more images than give
+            // every CU a workgroup or two (beyond that the two kernels are faster, and a longer
+            // lifetime only costs arena and cache reuse)
+            const Layout& sl = m->tensors[o0->in[0]]->t.layout;
+            const Layout& ml = m->tensors[o0->out[0]]->t.layout;
+            if (sl.nr_dim != 5 || ml.nr_dim != 5)
+                continue;
+            const long n = sl.dims[0], ic = 4L * sl.dims[1], w = sl.dims[3], oc = 4L * ml.dims[1];
+            if ((ic == 128 || ic == 256 || ic == 512) && oc % 64 == 0 && w >= 4 && w <= 31 && n * (oc / 64) <= 512)
+                keep_until[root_of(m, o0->in[0])] = (int)i + 1;
+        }
+    }
     std::vector<MemInterval> intervals;
     std::vector<int> ids;
     for (size_t i = 0; i < m->tensors.size(); ++i) {
@@ -118,7 +144,7 @@ bool plan_memory(Model* m) {
             continue;
         MemInterval iv;
         iv.begin = (size_t)t->def;
-        iv.end = t->is_output ? m->oprs.size() + 1 : (size_t)t->last + 1;
+        iv.end = t->is_output ? m->oprs.size() + 1 : (size_t)std::max(t->last, keep_until[i]) + 1;
         iv.size = tensor_bytes(t->t);
         intervals.push_back(iv);
         ids.push_back((int)i);
@@ -154,6 +180,44 @@ static bool shares_bytes(const Tensor& a, const Tensor& b) {
         return false;
     return a0 < b0 + bn && b0 < a0 + an;
 }
+// Milliseconds `iters` back-to-back rounds of the operators in `ops` take on the library stream
+// (after one untimed round), or a negative value when a launch fails or an operand has no memory
+// yet (a model input before set_input).
+static float time_oprs(Model* m, const std::vector<ModelOpr*>& ops, int iters) {
+    for (const ModelOpr* o : ops) {
+        for (const Tensor* t : o->in_ptrs)
+            if (!t->ptr)
+                return -1.f;
+        for (const Tensor* t : o->out_ptrs)
+            if (!t->ptr)
+                return -1.f;
+    }
+    auto round = [&]() {
+        for (ModelOpr* o : ops)
+            if (megcc_gfx950_call(
+                        &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), o->out_ptrs.data(),
+                        (int)o->out_ptrs.size(), &o->ws, &m->opt) != TinyNN_SUCCESS)
+                return false;
+        return true;
+    };
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        if (e0)
+            (void)hipEventDestroy(e0);
+        return -1.f;
+    }
+    float ms = -1.f;
+    bool ok = round();
+    ok = ok && hipEventRecord(e0, stream()) == hipSuccess;
+    for (int i = 0; ok && i < iters; ++i)
+        ok = round();
+    ok = ok && hipEventRecord(e1, stream()) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+         hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return ok ? ms : -1.f;
+}
+
 static void build_schedule(Model* m) {
     m->schedule.clear();
     const int n = (int)m->oprs.size();
@@ -217,6 +281,55 @@ static void build_schedule(Model* m) {
                     m->fused.push_back(f);
                     m->schedule.push_back(f);
                     i += 2;
+                    continue;
+                }
+                delete f;
+            }
+        }
+        // A pointwise convolution and the channel-wise 3x3 convolution of its result, on images small
+        // enough for a workgroup to hold one: one kernel (megcc_gfx950_pw_dw) when nothing else reads
+        // the tensor in between.
+        if (!options().no_fuse_pwdw && i + 1 < n && o0->desc.kind == MEGCC_KERN_CONV && o0->has_processed &&
+            o0->out.size() == 1 && o0->in.size() == (o0->desc.attr.conv.with_bias ? 3u : 2u)) {
+            ModelOpr* o1 = m->oprs[i + 1];
+            if (o1->desc.kind == MEGCC_KERN_CONV && !o1->has_processed && o1->out.size() == 1 &&
+                o1->in.size() == (o1->desc.attr.conv.with_bias ? 3u : 2u) && o1->in[0] == o0->out[0] &&
+                o1->desc.attr.conv.sparse == MEGCC_SPARSE_GROUP && temp(o0->out[0], 1)) {
+                ModelOpr* f = new ModelOpr();
+                memset(&f->desc, 0, sizeof(f->desc));
+                f->desc.kind = MEGCC_KERN_PW_DW;
+                f->desc.attr.pw_dw.pw = o0->desc.attr.conv;
+                f->desc.attr.pw_dw.dw = o1->desc.attr.conv;
+                f->desc.attr.pw_dw.mid_scale = m->tensors[o0->out[0]]->t.dtype.param.scale;
+                f->symbol = "pointwise 1x1 + depthwise 3x3 (fused)";
+                memset(&f->ws, 0, sizeof(f->ws));
+                f->in = o0->in;
+                f->in_ptrs = o0->in_ptrs;
+                for (size_t k = 1; k < o1->in.size(); ++k) {
+                    f->in.push_back(o1->in[k]);
+                    f->in_ptrs.push_back(o1->in_ptrs[k]);
+                }
+                f->out = o1->out;
+                f->out_ptrs = o1->out_ptrs;
+                // a workgroup reads its whole image before it stores, but other images' workgroups
+                // run at the same time: source and result must share no byte
+                bool take = !shares_bytes(*f->in_ptrs[0], *f->out_ptrs[0]) &&
+                            megcc_gfx950_pw_dw_supported(
+                                    &f->desc.attr.pw_dw, f->in_ptrs.data(), (int)f->in_ptrs.size(),
+                                    f->out_ptrs.data(), (int)f->out_ptrs.size());
+                // The one kernel saves a launch and the tensor's round trip, but its three phases run
+                // one after the other on a CU, so which form is faster depends on how many images
+                // there are per CU: both forms are run a few times on the tensors as they are (their
+                // contents do not matter before the first forward) and the faster one is kept. The
+                // switch "fusepwdw" takes the one kernel without measuring.
+                if (take && !options().fuse_pwdw) {
+                    const float one = time_oprs(m, {f}, 20), two = time_oprs(m, {o0, o1}, 20);
+                    take = one > 0.f && two > 0.f && one < 0.97f * two;
+                }
+                if (take) {
+                    m->fused.push_back(f);
+                    m->schedule.push_back(f);
+                    i += 1;
                     continue;
                 }
                 delete f;

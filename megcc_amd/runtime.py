@@ -101,6 +101,7 @@ EXPORTS = [
     "megcc_gfx950_elemwise_multitype", "megcc_gfx950_elemwise", "megcc_gfx950_typecvt",
     "megcc_gfx950_softmax", "megcc_gfx950_softmax_max_columns",
     "megcc_gfx950_dw_pool_add", "megcc_gfx950_dw_pool_add_supported",
+    "megcc_gfx950_pw_dw", "megcc_gfx950_pw_dw_supported",
     "megcc_gfx950_reduce", "megcc_gfx950_relayout", "megcc_gfx950_concat", "megcc_gfx950_resize", "megcc_gfx950_fused_elemwise",
     "megcc_gfx950_parse_symbol", "megcc_gfx950_call",
     "megcc_gfx950_call_init", "megcc_gfx950_call_workspace", "megcc_gfx950_init_device",

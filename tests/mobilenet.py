@@ -89,12 +89,17 @@ class Lifetimes:
     touches it (outputs: one past the last operator + 1); views share their root's request;
     weights and model inputs (the caller's memory) are not planned."""
 
-    def __init__(self):
+    def __init__(self, keep_pointwise_sources=False):
+        """keep_pointwise_sources: what the model runtime's own plan adds to the reference's rule - the
+        source of a pointwise convolution whose result feeds a channel-wise 3x3 convolution lives one
+        operator longer (the pair may run as one kernel that reads it while it writes the result)"""
         self.sizes, self.root, self.first, self.last = [], [], [], []
         self.is_weight, self.is_output, self.is_input, self.dtype = [], [], [], []
         self.nr_opr = 0
+        self.keep, self.prev, self.shapes = keep_pointwise_sources, None, []
 
     def _add(self, shape, type_enum, root=-1, weight=False):
+        self.shapes.append(tuple(shape))
         self.sizes.append(int(np.prod(shape)) * abi.np_dtype(type_enum).itemsize)
         self.root.append(root)
         self.first.append(-1)
@@ -129,6 +134,14 @@ class Lifetimes:
             if self.first[r] < 0:
                 self.first[r] = k
             self.last[r] = max(self.last[r], k)
+        if (self.keep and self.prev and "_conv2d_1x1_NCHW44_DENSE_p0x0_s1x1_" in self.prev[0]
+                and "_conv2d_3x3_NCHW44_GROUP_p1x1_" in symbol and inputs[0] == self.prev[2][0]):
+            n, ic4, _, w, _ = self.shapes[self.prev[1][0]]
+            oc4 = self.shapes[self.prev[2][0]][1]
+            if ic4 * 4 in (128, 256, 512) and oc4 % 16 == 0 and 4 <= w <= 31 and n * (oc4 // 16) <= 512:
+                r = self._root(self.prev[1][0])
+                self.last[r] = max(self.last[r], k)
+        self.prev = (symbol, list(inputs), list(outputs))
         self.nr_opr += 1
 
     def mark_input(self, t):

@@ -57,7 +57,8 @@ def test_memory_plan_reuses_the_arena_and_keeps_results():
     assert model.arena_bytes < total / 3, "tensors with disjoint lifetimes must share memory"
     # the arena is the reference allocator's plan for this model's lifetimes (stored answer for
     # batch 1 and 64 in golden/memplan.json; here the same planner on batch 3)
-    lt = mobilenet.Lifetimes()
+    # (... plus the one rule the runtime's own plan adds: see Lifetimes)
+    lt = mobilenet.Lifetimes(keep_pointwise_sources=True)
     net.build_gpu(model=lt)
     tids, begin, end, size = lt.requests()
     off, arena, _ = runtime.plan_memory(begin, end, size, 256)

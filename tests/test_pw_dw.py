@@ -1,0 +1,212 @@
+"""megcc_gfx950_pw_dw: a pointwise 1x1 convolution and the channel-wise 3x3 convolution of its result
+in one kernel, against the oracle's two convolutions run one after the other, bit for bit; and the
+model runtime's use of it."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import cases
+from cases import ConvCase
+from megcc_amd import abi, runtime
+from megcc_amd import abi as A
+
+pytestmark = pytest.mark.gpu
+
+TIES = (0.02, 0.01)        # source and filter scale whose product over the output scale has exact ties
+GENERIC = (0.0213, 0.0097)  # ... and without: IDENTITY / RELU requantise by the proven multiply-add
+
+PAIRS = [
+    # (n, ic, oc, h, w, stride of the 3x3, pointwise act, channel-wise act, pw bias, dw bias, scales)
+    # the pairs of a MobileNetV1 at 224 x 224 from 28 x 28 down, at a small batch ...
+    (2, 128, 256, 28, 28, 1, A.RELU, A.RELU, True, True, GENERIC),
+    (2, 256, 256, 28, 28, 2, A.RELU, A.RELU, True, True, TIES),
+    (3, 256, 512, 14, 14, 1, A.RELU, A.RELU, True, True, GENERIC),
+    (2, 512, 512, 14, 14, 1, A.RELU, A.RELU, True, True, TIES),
+    (3, 512, 512, 14, 14, 2, A.RELU, A.RELU, True, True, GENERIC),
+    (2, 512, 1024, 7, 7, 1, A.RELU, A.RELU, True, True, GENERIC),
+    # ... and at batches where a workgroup takes 128 channels instead of 64
+    (64, 512, 512, 14, 14, 1, A.RELU, A.RELU, True, True, GENERIC),
+    (32, 512, 1024, 7, 7, 1, A.RELU, A.IDENTITY, True, True, TIES),
+    # rows of 4, 5, 13, 31 pixels, one row, more rows than pixels a row, IDENTITY on either side, no bias
+    (2, 128, 64, 9, 5, 1, A.IDENTITY, A.RELU, False, True, GENERIC),
+    (1, 128, 128, 6, 13, 2, A.RELU, A.IDENTITY, True, False, TIES),
+    (2, 256, 64, 3, 31, 1, A.IDENTITY, A.IDENTITY, False, False, GENERIC),
+    (3, 128, 192, 5, 4, 2, A.RELU, A.RELU, True, True, GENERIC),
+    (2, 128, 64, 1, 8, 1, A.RELU, A.RELU, True, True, TIES),
+    (1, 128, 64, 33, 7, 2, A.RELU, A.RELU, True, True, GENERIC),
+    (5, 256, 320, 8, 16, 1, A.RELU, A.RELU, True, True, TIES),
+]
+
+
+def pair_cases(n, ic, oc, h, w, stride, act0, act1, bias0, bias1, scales):
+    mid = 0.0371 if scales is GENERIC else 0.05
+    pw = ConvCase(A.FMT_NCHW44, A.DENSE, n, ic, h, w, oc, 1, 1, 0, act0, scales=scales + (mid,), bias=bias0)
+    # (filter values of the 3x3 small enough that its output uses the whole int8 range without saturating everywhere)
+    dw = ConvCase(A.FMT_NCHW44, A.GROUP, n, oc, h, w, oc, 3, stride, 1, act1,
+                  scales=(mid, 0.0131 if scales is GENERIC else 0.01, 0.0689 if scales is GENERIC else 0.05),
+                  bias=bias1, flt_range=(-40, 40))
+    return pw, dw
+
+
+def ident(cfg):
+    return "n%d_c%d-%d_%dx%d_s%d_%s_%s%s%s_%s" % (
+        cfg[0], cfg[1], cfg[2], cfg[3], cfg[4], cfg[5], A.NONLINE_NAMES[cfg[6]], A.NONLINE_NAMES[cfg[7]],
+        "" if cfg[8] else "_nopwbias", "" if cfg[9] else "_nodwbias", "ties" if cfg[10] is TIES else "generic")
+
+
+def fused_call(pw, dw, a0, a1):
+    """-> (status, result or None, `supported` answer) of the pair through megcc_gfx950_call"""
+    L = runtime.lib()
+    # the pointwise operator's own init protocol packs its filter
+    ins0, outs0 = pw.specs(a0)
+    op0 = runtime.PreparedOp(runtime.parse_symbol(pw.symbol()), ins0, outs0)
+    assert op0.n_processed == 1
+    ins1, outs1 = dw.specs(a1)
+    bufs = [runtime.DeviceBuffer.from_array(s.array) for s in ins1[1:]]
+    tin = list(op0.in_tensors) + [
+        abi.make_tensor(b.ptr, s.shape, s.type_enum, s.scale, s.name) for b, s in zip(bufs, ins1[1:])]
+    out = runtime.DeviceBuffer(int(np.prod(dw.dst_shape())))
+    out.fill(cases.POISON)
+    tout = [abi.make_tensor(out.ptr, dw.dst_shape(), abi.QINT8, dw.scales[2], b"dst")]
+    desc = abi.KernelDesc()
+    desc.kind = abi.KERN_PW_DW
+    desc.attr.pw_dw.pw = pw.attr()
+    desc.attr.pw_dw.dw = dw.attr()
+    desc.attr.pw_dw.mid_scale = pw.scales[2]
+    L.megcc_gfx950_pw_dw_supported.argtypes = [
+        C.POINTER(abi.PwDwAttr), C.POINTER(C.POINTER(abi.Tensor)), C.c_int, C.POINTER(C.POINTER(abi.Tensor)), C.c_int]
+    ok = L.megcc_gfx950_pw_dw_supported(
+        C.byref(desc.attr.pw_dw), abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1)
+    st = L.megcc_gfx950_call(C.byref(desc), abi.tensor_array(tin), len(tin), abi.tensor_array(tout), 1, None, None)
+    got = None
+    if st == abi.SUCCESS:
+        runtime.wait()
+        got = out.to_array(dw.dst_shape(), np.int8)
+    for b in bufs + [out]:
+        b.free()
+    return st, got, ok
+
+
+def oracle_pair(pw, dw, a0, a1):
+    mid = pw.run_port(a0)
+    return mid, dw.run_port({"src": mid, "flt": a1["flt"], "bias": a1["bias"]})
+
+
+@pytest.mark.parametrize("cfg", PAIRS, ids=[ident(c) for c in PAIRS])
+def test_pointwise_and_depthwise_in_one_kernel_equal_the_two_layers(cfg):
+    pw, dw = pair_cases(*cfg)
+    print("GPU case:", repr(pw), repr(dw), flush=True)
+    a0, a1 = pw.gen(31), dw.gen(32)
+    mid, want = oracle_pair(pw, dw, a0, a1)
+    # the data must exercise both layers: the tensor in between and the result use most of their range
+    assert len(np.unique(mid)) > (100 if cfg[6] == A.RELU else 200), len(np.unique(mid))
+    assert len(np.unique(want)) > (60 if cfg[7] == A.RELU else 120), len(np.unique(want))
+    st, got, ok = fused_call(pw, dw, a0, a1)
+    assert ok == 1 and st == abi.SUCCESS, runtime.lib().megcc_gfx950_last_error().decode()
+    kernel = runtime.last_kernel()
+    assert kernel.startswith("conv_pw_dw:"), kernel
+    assert kernel.endswith("+affine") == (cfg[10] is GENERIC), kernel
+    bad = np.flatnonzero(got.reshape(-1) != want.reshape(-1))
+    assert bad.size == 0, "%r: %d of %d differ, first at %d: got %d want %d" % (
+        cfg, bad.size, got.size, bad[0], got.reshape(-1)[bad[0]], want.reshape(-1)[bad[0]])
+
+
+@pytest.mark.parametrize("cfg,why", [
+    ((2, 128, 64, 8, 32, 1, A.RELU, A.RELU, True, True, GENERIC), "rows of 32 pixels"),
+    ((2, 64, 64, 8, 8, 1, A.RELU, A.RELU, True, True, GENERIC), "64 input channels"),
+    ((2, 128, 32, 8, 8, 1, A.RELU, A.RELU, True, True, GENERIC), "32 output channels"),
+    ((2, 128, 64, 8, 8, 1, A.H_SWISH, A.RELU, True, True, GENERIC), "H_SWISH"),
+    ((2, 128, 64, 8, 8, 1, A.RELU, A.SIGMOID, True, True, GENERIC), "SIGMOID"),
+    ((1, 512, 128, 64, 31, 1, A.RELU, A.RELU, True, True, GENERIC), "an image beyond the LDS"),
+], ids=lambda v: v.replace(" ", "_") if isinstance(v, str) else "")
+def test_what_the_entry_point_refuses(cfg, why):
+    pw, dw = pair_cases(*cfg)
+    st, got, ok = fused_call(pw, dw, pw.gen(1), dw.gen(2))
+    assert ok == 0 and st == abi.ERROR_INVALID_LAYOUT and got is None, why
+
+
+def _pair_model(cfg, fused, second_reader=False):
+    pw, dw = pair_cases(*cfg)
+    a0, a1 = pw.gen(31), dw.gen(32)
+    # (left alone the runtime times both forms and keeps the faster one: the two switches pin it)
+    runtime.set_option("nofusepwdw", 0 if fused else 1)
+    runtime.set_option("fusepwdw", 1 if fused else 0)
+    try:
+        m = runtime.Model()
+        x = m.tensor("x", pw.src_shape(), abi.QINT8, pw.scales[0])
+        m.mark_input(x)
+        ins = [x, m.weight("pw.w", a0["flt"], abi.QINT8, pw.scales[1])]
+        if pw.bias:
+            ins.append(m.weight("pw.b", a0["bias"], abi.QINT32, float(np.float32(pw.scales[0]) * np.float32(pw.scales[1]))))
+        t1 = m.tensor("mid", pw.dst_shape(), abi.QINT8, pw.scales[2])
+        m.opr(pw.symbol(), ins, [t1])
+        ins = [t1, m.weight("dw.w", a1["flt"], abi.QINT8, dw.scales[1])]
+        if dw.bias:
+            ins.append(m.weight("dw.b", a1["bias"], abi.QINT32, float(np.float32(dw.scales[0]) * np.float32(dw.scales[1]))))
+        t2 = m.tensor("out", dw.dst_shape(), abi.QINT8, dw.scales[2])
+        m.opr(dw.symbol(), ins, [t2])
+        m.mark_output(t2)
+        if second_reader:
+            m.mark_output(t1)
+        m.finalize()
+    finally:
+        runtime.set_option("nofusepwdw", 0)
+        runtime.set_option("fusepwdw", 0)
+    m.set_input(x, a0["src"])
+    outs = []
+    for _ in range(3):  # eager, captured, replayed
+        m.forward()
+        runtime.wait()
+        outs.append(m.get(t2).copy())
+    mid = m.get(t1).copy() if second_reader else None
+    return outs, m.nr_kernel, oracle_pair(pw, dw, a0, a1), mid
+
+
+@pytest.mark.parametrize("cfg", [PAIRS[2], PAIRS[4], PAIRS[5], PAIRS[9]], ids=[ident(c) for c in (PAIRS[2], PAIRS[4], PAIRS[5], PAIRS[9])])
+def test_model_runtime_runs_the_pair_as_one_kernel(cfg):
+    fused, nk, (_, want), _ = _pair_model(cfg, True)
+    assert nk == 1, nk
+    plain, nk, _, _ = _pair_model(cfg, False)
+    assert nk == 2, nk
+    for o in fused + plain:
+        assert np.array_equal(o, want), cfg
+
+
+def test_model_runtime_keeps_the_pair_apart_when_the_tensor_between_is_read_elsewhere():
+    outs, nk, (mid_want, want), mid = _pair_model(PAIRS[2], True, second_reader=True)
+    assert nk == 2, nk
+    assert np.array_equal(mid, mid_want)
+    for o in outs:
+        assert np.array_equal(o, want)
+
+
+def test_model_runtime_left_alone_keeps_whichever_form_it_measures_faster():
+    """no switch: one kernel or two, and the same bytes either way"""
+    pw, dw = pair_cases(*PAIRS[2])
+    a0, a1 = pw.gen(31), dw.gen(32)
+    m = runtime.Model()
+    x0 = m.tensor("x0", pw.src_shape(), abi.QINT8, 0.03)
+    m.mark_input(x0)
+    # (the pair's source is an arena tensor, like inside a network: a model input has no memory yet
+    #  when the runtime decides, and such a pair stays two kernels)
+    pre = cases.MultiTypeCase(A.Q_RELU, pw.src_shape(), (0.03, 0.01, pw.scales[0]))
+    x = m.tensor("x", pw.src_shape(), abi.QINT8, pw.scales[0])
+    m.opr(pre.symbol(), [x0], [x])
+    bias_scale = lambda c: float(np.float32(c.scales[0]) * np.float32(c.scales[1]))
+    t1 = m.tensor("mid", pw.dst_shape(), abi.QINT8, pw.scales[2])
+    m.opr(pw.symbol(), [x, m.weight("pw.w", a0["flt"], abi.QINT8, pw.scales[1]),
+                        m.weight("pw.b", a0["bias"], abi.QINT32, bias_scale(pw))], [t1])
+    t2 = m.tensor("out", dw.dst_shape(), abi.QINT8, dw.scales[2])
+    m.opr(dw.symbol(), [t1, m.weight("dw.w", a1["flt"], abi.QINT8, dw.scales[1]),
+                        m.weight("dw.b", a1["bias"], abi.QINT32, bias_scale(dw))], [t2])
+    m.mark_output(t2)
+    m.finalize()
+    assert m.nr_kernel in (2, 3), m.nr_kernel
+    src0 = np.random.default_rng(5).integers(-128, 128, pw.src_shape()).astype(np.int8)
+    m.set_input(x0, src0)
+    m.forward()
+    runtime.wait()
+    a0["src"] = pre.run_port({"a": src0, "b": None})
+    _, want = oracle_pair(pw, dw, a0, a1)
+    assert np.array_equal(m.get(t2), want)

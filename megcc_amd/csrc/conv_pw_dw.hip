@@ -114,8 +114,17 @@ __global__ void __launch_bounds__(PWDW_THREADS) conv_pw_dw_kernel(PwDwParams q) 
                         rs, (int)(base + (unsigned)((c * 8 + j) * q.HW * 4)), 0, 0);
     };
     // ---- 0. filter slice, tables, bias; clear the planes -----------------------------------------
-    // (the filter is what the barrier waits for: its loads go first, the first job's activations
-    //  behind them, and the LDS is written while both are in flight)
+    // Loads return in the order they were issued and the barrier below waits for the filter: the
+    // tables and biases go first, then the filter, then the first job's activations (which are
+    // still in flight while the LDS is written).
+    const int tbl_word = tid < REQUANT_TABLE_ENTRIES
+                                 ? pwdw_kernarg((int)offsetof(PwDwParams, pw_table) + 4 * tid)
+                                 : pwdw_kernarg((int)offsetof(PwDwParams, dw_table) + 4 * (tid - REQUANT_TABLE_ENTRIES));
+    int bias_word = 0;
+    if (tid < OCS)
+        bias_word = q.pw_bias ? q.pw_bias[oc0 + tid] : 0;
+    else if (tid < 2 * OCS)
+        bias_word = q.dw_bias ? q.dw_bias[oc0 + tid - OCS] : 0;
     constexpr int PIECES = KC * OCS * 2;  // 16-byte pieces of the slice
     static_assert(PIECES % PWDW_THREADS == 0, "whole rounds");
     v4i piece[PIECES / PWDW_THREADS];
@@ -127,19 +136,13 @@ __global__ void __launch_bounds__(PWDW_THREADS) conv_pw_dw_kernel(PwDwParams q) 
     }
     v4i bufA[KC], bufB[KC];
     request(wave, bufA);
-    if (tid < REQUANT_TABLE_ENTRIES)
-        tbl_pw[tid] = pwdw_kernarg((int)offsetof(PwDwParams, pw_table) + 4 * tid);
-    else
-        tbl_dw[tid - REQUANT_TABLE_ENTRIES] =
-                pwdw_kernarg((int)offsetof(PwDwParams, dw_table) + 4 * (tid - REQUANT_TABLE_ENTRIES));
-    if (tid < OCS)
-        bias_pw[tid] = q.pw_bias ? q.pw_bias[oc0 + tid] : 0;
-    else if (tid < 2 * OCS)
-        bias_dw[tid - OCS] = q.dw_bias ? q.dw_bias[oc0 + tid - OCS] : 0;
     {
         const int plane_bytes = OCS * q.plane_stride + 16;  // (a multiple of 16 by construction)
         for (int i = tid * 16; i < plane_bytes; i += PWDW_THREADS * 16)
             *(v4i*)(planes + i) = v4i{0, 0, 0, 0};
+        tbl_pw[tid] = tbl_word;  // (tbl_dw follows tbl_pw)
+        if (tid < 2 * OCS)
+            bias_pw[tid] = bias_word;  // (bias_dw follows bias_pw)
 #pragma unroll
         for (int k = 0; k < PIECES / PWDW_THREADS; ++k)
             *(v4i*)(flt + (tid + k * PWDW_THREADS) * 16) = piece[k];

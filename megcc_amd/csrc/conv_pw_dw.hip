@@ -99,19 +99,21 @@ __global__ void __launch_bounds__(PWDW_THREADS) conv_pw_dw_kernel(PwDwParams q) 
             __builtin_amdgcn_make_buffer_rsrc((void*)q.src, 0, q.src_bytes, 0x00020000);
     const int jobs = q.tiles * OT;
     // the A operand of a job: this lane's pixel (row col >> lgP, column col & (P - 1)) of tile t,
-    // planes c * 8 + kg * 4 + j
-    auto request = [&](int job, v4i (&buf)[KC]) __attribute__((always_inline)) {
+    // planes c * 8 + kg * 4 + j; a wave keeps a ring of R chunks in flight, the next job's first
+    // chunks behind the current job's last
+    constexpr int R = KC < 8 ? KC : 8;
+    auto job_base = [&](int job) __attribute__((always_inline)) -> unsigned {
         const int t = job / OT;
         const int y = t * rpt + (col >> q.lgP), x = col & (P - 1);
-        const unsigned base = job < jobs && y < q.H && x < q.W
-                                      ? (unsigned)((((n * q.IC4 + kg * 4) * q.HW) + y * q.W + x) * 4)
-                                      : 0x80000000u;
+        return job < jobs && y < q.H && x < q.W
+                       ? (unsigned)((((n * q.IC4 + kg * 4) * q.HW) + y * q.W + x) * 4)
+                       : 0x80000000u;
+    };
+    auto load_chunk = [&](unsigned base, int c, v4i& dst) __attribute__((always_inline)) {
 #pragma unroll
-        for (int c = 0; c < KC; ++c)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                buf[c][j] = (int)__builtin_amdgcn_raw_buffer_load_b32(
-                        rs, (int)(base + (unsigned)((c * 8 + j) * q.HW * 4)), 0, 0);
+        for (int j = 0; j < 4; ++j)
+            dst[j] = (int)__builtin_amdgcn_raw_buffer_load_b32(
+                    rs, (int)(base + (unsigned)((c * 8 + j) * q.HW * 4)), 0, 0);
     };
     // ---- 0. filter slice, tables, bias; clear the planes -----------------------------------------
     // Loads return in the order they were issued and the barrier below waits for the filter: the
@@ -134,8 +136,11 @@ __global__ void __launch_bounds__(PWDW_THREADS) conv_pw_dw_kernel(PwDwParams q) 
         const int c = idx / (OCS * 2), r = idx - c * (OCS * 2);
         piece[k] = *(const v4i*)(q.wp + ((size_t)c * q.OCP + oc0) * KROW + r * 16);
     }
-    v4i bufA[KC], bufB[KC];
-    request(wave, bufA);
+    v4i ring[R];
+    unsigned base = job_base(wave);
+#pragma unroll
+    for (int c = 0; c < R; ++c)
+        load_chunk(base, c, ring[c]);
     {
         const int plane_bytes = OCS * q.plane_stride + 16;  // (a multiple of 16 by construction)
         for (int i = tid * 16; i < plane_bytes; i += PWDW_THREADS * 16)
@@ -150,7 +155,8 @@ __global__ void __launch_bounds__(PWDW_THREADS) conv_pw_dw_kernel(PwDwParams q) 
     __syncthreads();
 
     // ---- 1. pointwise -----------------------------------------------------------------------------
-    auto compute = [&](int job, const v4i (&buf)[KC]) __attribute__((always_inline)) {
+    for (int job = wave; job < jobs; job += NW) {
+        const unsigned next_base = job_base(job + NW);
         const int t = job / OT, ot = (job - t * OT) * JT;
         v16i acc[JT], acc1 = {};
         const int8_t* frow[JT];
@@ -163,25 +169,30 @@ __global__ void __launch_bounds__(PWDW_THREADS) conv_pw_dw_kernel(PwDwParams q) 
                 acc[jt][e] = b;
             frow[jt] = flt + ocl * KROW + (((kg ^ (ocl >> 3)) & 1) << 4);
         }
-        if (JT == 1) {
-            // two accumulator chains (even and odd chunks) keep the matrix core busy between them
-#pragma unroll
-            for (int c = 0; c < KC; c += 2) {
-                const v4i f0 = *(const v4i*)(frow[0] + c * (OCS * KROW));
-                const v4i f1 = *(const v4i*)(frow[0] + (c + 1) * (OCS * KROW));
-                acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(buf[c], f0, acc[0], 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(buf[c + 1], f1, acc1, 0, 0, 0);
-            }
-            acc[0] += acc1;
-        } else {
-#pragma unroll
-            for (int c = 0; c < KC; ++c)
+        static_for<KC>([&](auto cc) {
+            constexpr int c = decltype(cc)::value;
+            if (JT == 1) {
+                // two accumulator chains (even and odd chunks) keep the matrix core busy between them
+                const v4i f = *(const v4i*)(frow[0] + c * (OCS * KROW));
+                if (c & 1)
+                    acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[c % R], f, acc1, 0, 0, 0);
+                else
+                    acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[c % R], f, acc[0], 0, 0, 0);
+            } else {
 #pragma unroll
                 for (int jt = 0; jt < JT; ++jt) {
                     const v4i f = *(const v4i*)(frow[jt] + c * (OCS * KROW));
-                    acc[jt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(buf[c], f, acc[jt], 0, 0, 0);
+                    acc[jt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[c % R], f, acc[jt], 0, 0, 0);
                 }
-        }
+            }
+            if (c + R < KC)
+                load_chunk(base, c + R, ring[c % R]);
+            else
+                load_chunk(next_base, c + R - KC, ring[c % R]);
+        });
+        base = next_base;
+        if (JT == 1)
+            acc[0] += acc1;
 #pragma unroll
         for (int jt = 0; jt < JT; ++jt) {
             int r[16];
@@ -208,14 +219,6 @@ __global__ void __launch_bounds__(PWDW_THREADS) conv_pw_dw_kernel(PwDwParams q) 
                     *(uint32_t*)(plane + (y + 1) * P + x0) = w;
             }
         }
-    };
-    for (int job = wave; job < jobs; job += 2 * NW) {
-        request(job + NW, bufB);
-        compute(job, bufA);
-        if (job + NW >= jobs)
-            break;
-        request(job + 2 * NW, bufA);
-        compute(job + NW, bufB);
     }
     __syncthreads();
 
@@ -317,9 +320,17 @@ static int pwdw_plane_stride(int h, int w) {
         bytes += 4;  // an odd number of dwords: the planes of 32 lanes start in 32 different banks
     return bytes;
 }
-// channels per workgroup: 128 when that still gives every CU a workgroup, else 64
+// Channels per workgroup. Two workgroups fit a CU while one stays under half the LDS and 128 vector
+// registers, and the three phases of one then overlap the other's: 64 channels do (a pointwise job
+// then holds 2 x 16 accumulators); 128 only for images of a few 32-pixel tiles, where a job is one
+// 32-channel tile and 128 channels give every wave one.
+static size_t pwdw_lds_bytes(const ConvGeom& pw, int ocs);
+static int pwdw_tiles(const ConvGeom& pw) {
+    const int rpt = 32 >> pwdw_lgp(pw.iw);
+    return (pw.ih + rpt - 1) / rpt;
+}
 static int pwdw_slice(const ConvGeom& pw) {
-    return (pw.oc & 127) == 0 && (long)pw.n * (pw.oc / 128) >= 256 ? 128 : 64;
+    return (pw.oc & 127) == 0 && pwdw_tiles(pw) < 6 && pwdw_lds_bytes(pw, 128) <= 80 * 1024 ? 128 : 64;
 }
 static size_t pwdw_lds_bytes(const ConvGeom& pw, int ocs) {
     return (size_t)pw.ic * ocs + 2 * REQUANT_TABLE_ENTRIES * 4 + 2 * ocs * 4 +
@@ -391,17 +402,17 @@ TinyNNStatus conv_pw_dw_launch(
     q.dw_ad = a1.d;
     note_requant_affine(a0.d != 0.f && a1.d != 0.f);  // (the kernel's name says so when both layers use it)
     const int kc = pw.ic / 32;
-    const bool whole = q.tiles >= 6;  // enough 32-pixel tiles for every wave: a job takes the whole slice
+    // enough 32-pixel tiles for every wave: a job takes the whole slice (64 channels then, see pwdw_slice)
+    const bool whole = q.tiles >= 6;
     const void* kern = nullptr;
-#define MG_PWDW_PICK(KC_, OCS_)                                                                       \
-    (whole ? (dw.sh == 1 ? (const void*)conv_pw_dw_kernel<KC_, OCS_, 1, OCS_ / 32>                    \
-                         : (const void*)conv_pw_dw_kernel<KC_, OCS_, 2, OCS_ / 32>)                   \
-           : (dw.sh == 1 ? (const void*)conv_pw_dw_kernel<KC_, OCS_, 1, 1>                            \
-                         : (const void*)conv_pw_dw_kernel<KC_, OCS_, 2, 1>))
+#define MG_PWDW_PICK(KC_, OCS_, JT_)                                          \
+    (dw.sh == 1 ? (const void*)conv_pw_dw_kernel<KC_, OCS_, 1, JT_> : (const void*)conv_pw_dw_kernel<KC_, OCS_, 2, JT_>)
     if (ocs == 128)
-        kern = kc == 4 ? MG_PWDW_PICK(4, 128) : kc == 8 ? MG_PWDW_PICK(8, 128) : MG_PWDW_PICK(16, 128);
+        kern = kc == 4 ? MG_PWDW_PICK(4, 128, 1) : kc == 8 ? MG_PWDW_PICK(8, 128, 1) : MG_PWDW_PICK(16, 128, 1);
+    else if (whole)
+        kern = kc == 4 ? MG_PWDW_PICK(4, 64, 2) : kc == 8 ? MG_PWDW_PICK(8, 64, 2) : MG_PWDW_PICK(16, 64, 2);
     else
-        kern = kc == 4 ? MG_PWDW_PICK(4, 64) : kc == 8 ? MG_PWDW_PICK(8, 64) : MG_PWDW_PICK(16, 64);
+        kern = kc == 4 ? MG_PWDW_PICK(4, 64, 1) : kc == 8 ? MG_PWDW_PICK(8, 64, 1) : MG_PWDW_PICK(16, 64, 1);
 #undef MG_PWDW_PICK
     const size_t lds = pwdw_lds_bytes(pw, ocs);
     MG_REQUIRE(lds <= 160 * 1024, TinyNN_ERROR_OUT_OF_RANGE, "conv_pw_dw: %zu bytes of LDS", lds);

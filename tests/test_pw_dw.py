@@ -25,7 +25,7 @@ PAIRS = [
     (2, 512, 512, 14, 14, 1, A.RELU, A.RELU, True, True, TIES),
     (3, 512, 512, 14, 14, 2, A.RELU, A.RELU, True, True, GENERIC),
     (2, 512, 1024, 7, 7, 1, A.RELU, A.RELU, True, True, GENERIC),
-    # ... and at batches where a workgroup takes 128 channels instead of 64
+    # ... and at the batches of the benchmark (14 x 14: 64 channels per workgroup, 7 x 7: 128)
     (64, 512, 512, 14, 14, 1, A.RELU, A.RELU, True, True, GENERIC),
     (32, 512, 1024, 7, 7, 1, A.RELU, A.IDENTITY, True, True, TIES),
     # rows of 4, 5, 13, 31 pixels, one row, more rows than pixels a row, IDENTITY on either side, no bias
@@ -36,6 +36,9 @@ PAIRS = [
     (2, 128, 64, 1, 8, 1, A.RELU, A.RELU, True, True, TIES),
     (1, 128, 64, 33, 7, 2, A.RELU, A.RELU, True, True, GENERIC),
     (5, 256, 320, 8, 16, 1, A.RELU, A.RELU, True, True, TIES),
+    (5, 512, 128, 7, 7, 2, A.RELU, A.IDENTITY, True, True, GENERIC),
+    (3, 256, 64, 4, 6, 1, A.IDENTITY, A.RELU, True, True, TIES),
+    (1, 512, 1024, 7, 7, 1, A.RELU, A.RELU, True, True, GENERIC),
 ]
 
 

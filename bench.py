@@ -452,6 +452,87 @@ def bench_chain(c, hw, stride, steps, warmup, batch=64, cpu=False):
             "checked": True, "checked_what": "images 0 and %d of the chain's output, bit for bit" % (batch - 1)}
 
 
+def bench_pwdw(batch, ic, oc, hw, stride, steps, warmup):
+    """A pointwise 1x1 layer and the channel-wise 3x3 layer behind it as a two-operator model on the
+    static arena, three ways: as the model runtime decides (it times both forms at finalize), as one
+    kernel (megcc_gfx950_pw_dw) and as the two kernels. Scales with an exact multiply-add
+    requantisation, like a calibrated network's."""
+    import numpy as np
+    from cases import ConvCase, MultiTypeCase
+    from megcc_amd import abi, runtime
+    pw = ConvCase(abi.FMT_NCHW44, abi.DENSE, batch, ic, hw, hw, oc, 1, 1, 0, abi.RELU, scales=(0.0213, 0.0097, 0.0371))
+    dw = ConvCase(abi.FMT_NCHW44, abi.GROUP, batch, oc, hw, hw, oc, 3, stride, 1, abi.RELU,
+                  scales=(0.0371, 0.0131, 0.0689), flt_range=(-40, 40))
+    a0, a1 = pw.gen(31), dw.gen(32)
+    src0 = np.random.default_rng(5).integers(-128, 128, pw.src_shape()).astype(np.int8)
+    pre = MultiTypeCase(abi.Q_RELU, pw.src_shape(), (0.03, 0.01, pw.scales[0]))
+    bias_scale = lambda c: float(np.float32(c.scales[0]) * np.float32(c.scales[1]))
+    ev = HipEvents(runtime.lib().megcc_gfx950_stream())
+    out, results = {}, {}
+    for mode in ("runtime", "one", "two"):
+        runtime.set_option("nofusepwdw", 1 if mode == "two" else 0)
+        runtime.set_option("fusepwdw", 1 if mode == "one" else 0)
+        m = runtime.Model()
+        x0 = m.tensor("x0", pw.src_shape(), abi.QINT8, 0.03)
+        m.mark_input(x0)
+        # (the pair's source is an arena tensor, as inside a network; it is an output as well, so that
+        #  no memory plan lays the pair's result over it and the one kernel can run at every batch)
+        x = m.tensor("x", pw.src_shape(), abi.QINT8, pw.scales[0])
+        m.opr(pre.symbol(), [x0], [x])
+        m.mark_output(x)
+        t1 = m.tensor("mid", pw.dst_shape(), abi.QINT8, pw.scales[2])
+        m.opr(pw.symbol(), [x, m.weight("pw.w", a0["flt"], abi.QINT8, pw.scales[1]),
+                            m.weight("pw.b", a0["bias"], abi.QINT32, bias_scale(pw))], [t1])
+        t2 = m.tensor("out", dw.dst_shape(), abi.QINT8, dw.scales[2])
+        m.opr(dw.symbol(), [t1, m.weight("dw.w", a1["flt"], abi.QINT8, dw.scales[1]),
+                            m.weight("dw.b", a1["bias"], abi.QINT32, bias_scale(dw))], [t2])
+        m.mark_output(t2)
+        m.finalize()
+        runtime.set_option("nofusepwdw", 0)
+        runtime.set_option("fusepwdw", 0)
+        m.set_input(x0, src0)
+        m.forward()
+        runtime.wait()
+        results[mode] = m.get(t2).copy()
+        # the pair alone: operators 1.. of the schedule cannot be run apart from operator 0 through
+        # forward(), so the ReLU in front is timed too and subtracted (its own model below)
+        for _ in range(max(warmup, 3)):
+            m.forward()
+        runtime.wait()
+        e0, e1 = ev.new(), ev.new()
+        ev.record(e0)
+        for _ in range(steps):
+            m.forward()
+        ev.record(e1)
+        runtime.wait()
+        out[mode] = {"us_per_forward": round(ev.elapsed_ms(e0, e1) / steps * 1e3, 2), "nr_kernel": m.nr_kernel}
+        m.close()
+    if not (np.array_equal(results["one"], results["two"]) and np.array_equal(results["runtime"], results["two"])):
+        raise SystemExit("bench.py: the one-kernel pair and the two kernels differ")
+    # image 0 against the oracle
+    from oracle import port
+    port.set_threads(os.cpu_count() or 8)
+    one0 = ConvCase(abi.FMT_NCHW44, abi.DENSE, 1, ic, hw, hw, oc, 1, 1, 0, abi.RELU, scales=pw.scales)
+    one1 = ConvCase(abi.FMT_NCHW44, abi.GROUP, 1, oc, hw, hw, oc, 3, stride, 1, abi.RELU, scales=dw.scales)
+    mid = one0.run_port({"src": pre.run_port({"a": src0[:1], "b": None}), "flt": a0["flt"], "bias": a0["bias"]})
+    want = one1.run_port({"src": mid, "flt": a1["flt"], "bias": a1["bias"]})
+    if not np.array_equal(results["one"][:1], want):
+        raise SystemExit("bench.py: pair output of image 0 differs from the oracle")
+    n_in, n_mid, n_out = (int(np.prod(sh)) for sh in (pw.src_shape(), pw.dst_shape(), dw.dst_shape()))
+    ms = out["runtime"]["us_per_forward"] * 1e-3
+    moved = 2 * n_in + n_in + n_out + ic * oc + (0 if out["runtime"]["nr_kernel"] == 2 else 2 * n_mid)
+    return {"metric": "hbm_gbps", "value": round(moved / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+            "config": {"workload": "qsi8 ReLU -> pointwise %d->%d -> depthwise 3x3 s%d, N=%d %dx%d NCHW44 (three "
+                                   "operators; the last two are the pair)" % (ic, oc, stride, batch, hw, hw)},
+            "forms": out,
+            "roofline": {"bound": "hbm", "achieved": round(moved / (ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": round(moved / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None,
+                         "algorithmic_per_launch": moved},
+            "checked": True, "checked_what": "one kernel == two kernels on every image; image 0 == oracle"}
+
+
 def case_bytes(case):
     ins, outs = case.specs(case.gen(0))
     return sum(s.nbytes for s in ins) + sum(s.nbytes for s in outs)
@@ -625,6 +706,10 @@ def main():
 
     if args.workload == "mobilenet":
         print(json.dumps(bench_mobilenet(args.batch, args.steps, args.warmup, args.per_layer)))
+        return
+    if args.workload.startswith("pwdw:"):  # pwdw:N,IC,OC,HW,S
+        n, ic, oc, hw, st = [int(v) for v in args.workload[5:].split(",")]
+        print(json.dumps(bench_pwdw(n, ic, oc, hw, st, args.steps, args.warmup)))
         return
     if args.workload.startswith("chain"):  # chain, chain_s2, chain512, chain512_s2, chain:C,HW,S
         c, hw, st = [int(v) for v in args.workload[6:].split(",")] if args.workload.startswith("chain:") else {

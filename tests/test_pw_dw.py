@@ -213,3 +213,59 @@ def test_model_runtime_left_alone_keeps_whichever_form_it_measures_faster():
     a0["src"] = pre.run_port({"a": src0, "b": None})
     _, want = oracle_pair(pw, dw, a0, a1)
     assert np.array_equal(m.get(t2), want)
+
+
+# A memory plan made for the two operators gives the depthwise result the bytes of the pointwise
+# layer's source (dead after the pointwise layer). The one kernel reads that source while other
+# workgroups already write the result, so under such a plan the pair must stay two kernels.
+def _planned_pair(out_offset):
+    cfg = (3, 256, 128, 9, 12, 1, A.RELU, A.RELU, True, True, GENERIC)
+    pw, dw = pair_cases(*cfg)
+    a0, a1 = pw.gen(41), dw.gen(42)
+    x0 = np.random.default_rng(43).integers(-128, 128, pw.src_shape()).astype(np.int8)
+    pre = cases.MultiTypeCase(A.Q_RELU, pw.src_shape(), (0.03, 0.01, pw.scales[0]))
+    bias_scale = lambda c: float(np.float32(c.scales[0]) * np.float32(c.scales[1]))
+    runtime.set_option("fusepwdw", 1)  # (no timing: the one kernel wherever it may run)
+    try:
+        m = runtime.Model()
+        t_in = m.tensor("x0", pw.src_shape(), abi.QINT8, 0.03)
+        m.mark_input(t_in)
+        t_x = m.tensor("x", pw.src_shape(), abi.QINT8, pw.scales[0])  # an arena tensor that dies at the pointwise layer
+        m.opr(pre.symbol(), [t_in], [t_x])
+        w0 = m.weight("pw.w", a0["flt"], abi.QINT8, pw.scales[1])
+        b0 = m.weight("pw.b", a0["bias"], abi.QINT32, bias_scale(pw))
+        t1 = m.tensor("mid", pw.dst_shape(), abi.QINT8, pw.scales[2])
+        m.opr(pw.symbol(), [t_x, w0, b0], [t1])
+        w1 = m.weight("dw.w", a1["flt"], abi.QINT8, dw.scales[1])
+        b1 = m.weight("dw.b", a1["bias"], abi.QINT32, bias_scale(dw))
+        t2 = m.tensor("out", dw.dst_shape(), abi.QINT8, dw.scales[2])
+        m.opr(dw.symbol(), [t1, w1, b1], [t2])
+        m.mark_output(t2)
+        up = lambda v: (v + 255) // 256 * 256
+        nx, nmid, nout = (int(np.prod(s)) for s in (pw.src_shape(), pw.dst_shape(), dw.dst_shape()))
+        offs = [0] * (t2 + 1)
+        offs[t_x], offs[t1] = 0, up(nx)
+        offs[t2] = out_offset if out_offset is not None else offs[t1] + up(nmid)
+        m.set_plan(offs, offs[t1] + up(nmid) + up(nout))
+        m.finalize()
+    finally:
+        runtime.set_option("fusepwdw", 0)
+    m.set_input(t_in, x0)
+    outs = []
+    for _ in range(3):
+        m.forward()
+        runtime.wait()
+        outs.append(m.get(t2).copy())
+    nk = m.nr_kernel
+    m.close()
+    a0["src"] = pre.run_port({"a": x0, "b": None})
+    return outs, nk, oracle_pair(pw, dw, a0, a1)[1]
+
+
+@pytest.mark.parametrize("out_offset,kernels", [(None, 2), (0, 3), (256, 3), (41472, 3)],
+                         ids=["apart", "result_on_the_source", "result_256_bytes_into_the_source", "result_over_the_source_tail"])
+def test_pair_is_one_kernel_only_when_its_result_shares_no_byte_with_its_source(out_offset, kernels):
+    outs, nk, want = _planned_pair(out_offset)
+    assert nk == kernels
+    for o in outs:
+        assert np.array_equal(o, want)

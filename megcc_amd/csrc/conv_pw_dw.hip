@@ -128,13 +128,15 @@ __global__ void __launch_bounds__(PWDW_THREADS) conv_pw_dw_kernel(PwDwParams q) 
     else if (tid < 2 * OCS)
         bias_word = q.dw_bias ? q.dw_bias[oc0 + tid - OCS] : 0;
     constexpr int PIECES = KC * OCS * 2;  // 16-byte pieces of the slice
-    static_assert(PIECES % PWDW_THREADS == 0, "whole rounds");
-    v4i piece[PIECES / PWDW_THREADS];
+    constexpr int PPT = (PIECES + PWDW_THREADS - 1) / PWDW_THREADS;  // per thread
+    static_assert(PIECES % PWDW_THREADS == 0 || PIECES < PWDW_THREADS, "whole rounds, or part of one");
+    v4i piece[PPT];
 #pragma unroll
-    for (int k = 0; k < PIECES / PWDW_THREADS; ++k) {
+    for (int k = 0; k < PPT; ++k) {
         const int idx = tid + k * PWDW_THREADS;
         const int c = idx / (OCS * 2), r = idx - c * (OCS * 2);
-        piece[k] = *(const v4i*)(q.wp + ((size_t)c * q.OCP + oc0) * KROW + r * 16);
+        if (PIECES % PWDW_THREADS == 0 || idx < PIECES)
+            piece[k] = *(const v4i*)(q.wp + ((size_t)c * q.OCP + oc0) * KROW + r * 16);
     }
     v4i ring[R];
     unsigned base = job_base(wave);
@@ -149,8 +151,9 @@ __global__ void __launch_bounds__(PWDW_THREADS) conv_pw_dw_kernel(PwDwParams q) 
         if (tid < 2 * OCS)
             bias_pw[tid] = bias_word;  // (bias_dw follows bias_pw)
 #pragma unroll
-        for (int k = 0; k < PIECES / PWDW_THREADS; ++k)
-            *(v4i*)(flt + (tid + k * PWDW_THREADS) * 16) = piece[k];
+        for (int k = 0; k < PPT; ++k)
+            if (PIECES % PWDW_THREADS == 0 || tid + k * PWDW_THREADS < PIECES)
+                *(v4i*)(flt + (tid + k * PWDW_THREADS) * 16) = piece[k];
     }
     __syncthreads();
 
@@ -330,7 +333,11 @@ static int pwdw_tiles(const ConvGeom& pw) {
     return (pw.ih + rpt - 1) / rpt;
 }
 static int pwdw_slice(const ConvGeom& pw) {
-    return (pw.oc & 127) == 0 && pwdw_tiles(pw) < 6 && pwdw_lds_bytes(pw, 128) <= 80 * 1024 ? 128 : 64;
+    if ((pw.oc & 127) == 0 && pwdw_tiles(pw) < 6 && pwdw_lds_bytes(pw, 128) <= 80 * 1024)
+        return 128;
+    // a batch that leaves CUs without a workgroup at 64 channels: 32; also when 64 planes of a large
+    // image do not fit the LDS (32 always do: at most 64 rows of 32 bytes and 512 input channels)
+    return (long)pw.n * (pw.oc / 64) < 256 || pwdw_lds_bytes(pw, 64) > 160 * 1024 ? 32 : 64;
 }
 static size_t pwdw_lds_bytes(const ConvGeom& pw, int ocs) {
     return (size_t)pw.ic * ocs + 2 * REQUANT_TABLE_ENTRIES * 4 + 2 * ocs * 4 +
@@ -409,6 +416,8 @@ TinyNNStatus conv_pw_dw_launch(
     (dw.sh == 1 ? (const void*)conv_pw_dw_kernel<KC_, OCS_, 1, JT_> : (const void*)conv_pw_dw_kernel<KC_, OCS_, 2, JT_>)
     if (ocs == 128)
         kern = kc == 4 ? MG_PWDW_PICK(4, 128, 1) : kc == 8 ? MG_PWDW_PICK(8, 128, 1) : MG_PWDW_PICK(16, 128, 1);
+    else if (ocs == 32)
+        kern = kc == 4 ? MG_PWDW_PICK(4, 32, 1) : kc == 8 ? MG_PWDW_PICK(8, 32, 1) : MG_PWDW_PICK(16, 32, 1);
     else if (whole)
         kern = kc == 4 ? MG_PWDW_PICK(4, 64, 2) : kc == 8 ? MG_PWDW_PICK(8, 64, 2) : MG_PWDW_PICK(16, 64, 2);
     else

@@ -39,6 +39,11 @@ PAIRS = [
     (5, 512, 128, 7, 7, 2, A.RELU, A.IDENTITY, True, True, GENERIC),
     (3, 256, 64, 4, 6, 1, A.IDENTITY, A.RELU, True, True, TIES),
     (1, 512, 1024, 7, 7, 1, A.RELU, A.RELU, True, True, GENERIC),
+    # small batches run 32 channels per workgroup, batches that fill the chip 64: the latter with every
+    # K, both strides, and an image of few tiles
+    (64, 128, 256, 14, 14, 2, A.RELU, A.RELU, True, True, TIES),
+    (32, 256, 512, 14, 14, 1, A.RELU, A.IDENTITY, True, True, GENERIC),
+    (128, 128, 192, 5, 4, 2, A.IDENTITY, A.RELU, True, True, GENERIC),
 ]
 
 
@@ -121,7 +126,7 @@ def test_pointwise_and_depthwise_in_one_kernel_equal_the_two_layers(cfg):
     ((2, 128, 32, 8, 8, 1, A.RELU, A.RELU, True, True, GENERIC), "32 output channels"),
     ((2, 128, 64, 8, 8, 1, A.H_SWISH, A.RELU, True, True, GENERIC), "H_SWISH"),
     ((2, 128, 64, 8, 8, 1, A.RELU, A.SIGMOID, True, True, GENERIC), "SIGMOID"),
-    ((1, 512, 128, 64, 31, 1, A.RELU, A.RELU, True, True, GENERIC), "an image beyond the LDS"),
+    ((1, 128, 64, 65, 8, 1, A.RELU, A.RELU, True, True, GENERIC), "65 rows"),
 ], ids=lambda v: v.replace(" ", "_") if isinstance(v, str) else "")
 def test_what_the_entry_point_refuses(cfg, why):
     pw, dw = pair_cases(*cfg)
@@ -174,6 +179,42 @@ def test_model_runtime_runs_the_pair_as_one_kernel(cfg):
     assert nk == 2, nk
     for o in fused + plain:
         assert np.array_equal(o, want), cfg
+
+
+def test_large_image_at_a_large_batch():
+    """64 planes of 60 x 31 pixels and 512 x 64 filter bytes do not fit the LDS: 32 channels per
+    workgroup although the batch would fill the chip at 64. Against the two kernels (which the other
+    tests hold against the oracle) - the oracle would take a minute here."""
+    cfg = (16, 512, 1024, 60, 31, 1, A.RELU, A.RELU, True, True, GENERIC)
+    pw, dw = pair_cases(*cfg)
+    a0, a1 = pw.gen(31), dw.gen(32)
+    outs = []
+    for fused in (True, False):
+        runtime.set_option("nofusepwdw", 0 if fused else 1)
+        runtime.set_option("fusepwdw", 1 if fused else 0)
+        try:
+            m = runtime.Model()
+            x = m.tensor("x", pw.src_shape(), abi.QINT8, pw.scales[0])
+            m.mark_input(x)
+            bias_scale = lambda c: float(np.float32(c.scales[0]) * np.float32(c.scales[1]))
+            t1 = m.tensor("mid", pw.dst_shape(), abi.QINT8, pw.scales[2])
+            m.opr(pw.symbol(), [x, m.weight("pw.w", a0["flt"], abi.QINT8, pw.scales[1]),
+                                m.weight("pw.b", a0["bias"], abi.QINT32, bias_scale(pw))], [t1])
+            t2 = m.tensor("out", dw.dst_shape(), abi.QINT8, dw.scales[2])
+            m.opr(dw.symbol(), [t1, m.weight("dw.w", a1["flt"], abi.QINT8, dw.scales[1]),
+                                m.weight("dw.b", a1["bias"], abi.QINT32, bias_scale(dw))], [t2])
+            m.mark_output(t2)
+            m.finalize()
+        finally:
+            runtime.set_option("nofusepwdw", 0)
+            runtime.set_option("fusepwdw", 0)
+        assert m.nr_kernel == (1 if fused else 2)
+        m.set_input(x, a0["src"])
+        m.forward()
+        runtime.wait()
+        outs.append(m.get(t2).copy())
+        m.close()
+    assert len(np.unique(outs[0])) > 100 and np.array_equal(outs[0], outs[1])
 
 
 def test_model_runtime_keeps_the_pair_apart_when_the_tensor_between_is_read_elsewhere():

@@ -117,11 +117,10 @@ class HipEvents:
         return ms.value
 
 
-def headline_case(n=32, c=256, hw=56):
+def headline_case(n=32, c=256, hw=56, scales=(0.02, 0.01, 0.05)):
     from cases import ConvCase
     from megcc_amd import abi
-    return ConvCase(abi.FMT_NCHW44, abi.DENSE, n, c, hw, hw, c, 3, 1, 1, abi.RELU,
-                    scales=(0.02, 0.01, 0.05))
+    return ConvCase(abi.FMT_NCHW44, abi.DENSE, n, c, hw, hw, c, 3, 1, 1, abi.RELU, scales=scales)
 
 
 def make_workload(name):
@@ -175,6 +174,12 @@ def make_workload(name):
     if name == "conv":
         case = headline_case()
         return case, "qsi8 conv3x3 s1 p1 NCHW44 N=32 Cin=Cout=256 56x56 +bias +ReLU requant", "mfma"
+    if name == "conv_cal":
+        # The default scales (0.02 * 0.01 / 0.05 = 1 / 250) make every 125th accumulator an exact tie, the
+        # worst case for the requantisation (threshold table). Scales without ties, as a calibrated
+        # network has them, requantise by one multiply-add; the output then also uses the whole range.
+        return (headline_case(scales=(0.0213, 0.0097, 0.517)),
+                "qsi8 conv3x3 s1 p1 NCHW44 N=32 Cin=Cout=256 56x56 +bias +ReLU requant, scales without exact ties", "mfma")
     if name == "conv_c64":
         return headline_case(32, 64, 56), "qsi8 conv3x3 NCHW44 N=32 C=64 56x56", "mfma"
     if name == "conv_c256_28":

@@ -592,7 +592,7 @@ int megcc_gfx950_requant_affine(int nonline_mode, float s_src, float s_flt, floa
 /* Kernel-selection overrides, for regression tests of kernels that un-switched shapes only reach
  * through a fallback: "nopws", "nogevm", "nofcb", "nosmall", "nopm768", "nopm", "nodma512",
  * "nopm256", "nodma", "nofcs", "nopwshare", "nohybrid", "nodot4", "nof32small",
- * "dw_generic", "nodwmfma", "nodwnchw", "nofusesoftmax", "nopoolrows", "nofirstmfma", "norowsplit", "nofusechain", "nofusepwdw", "fusepwdw", "nofcone", "noxcdorder", "noaffine", "no_graph"; value 1 takes the kernel out
+ * "dw_generic", "nodwmfma", "nodwnchw", "nofusesoftmax", "nopoolrows", "nofirstmfma", "norowsplit", "nofusechain", "nofusepwdw", "fusepwdw", "nofcone", "noxcdorder", "noaffine", "nopipeline", "no_graph"; value 1 takes the kernel out
  * of the dispatch, 0 puts it back ("fusepwdw": 1 makes the model runtime take the one-kernel form of a
  * pointwise / channel-wise pair wherever it applies instead of timing both forms). The
  * same names in capitals behind MEGCC_ are read from the environment once, at first use.
@@ -673,6 +673,27 @@ void* megcc_gfx950_model_tensor_ptr(void* model, int tensor);
 TinyNNStatus megcc_gfx950_model_set_input(void* model, int tensor, const void* host, size_t bytes);
 TinyNNStatus megcc_gfx950_model_get_output(void* model, int tensor, void* host, size_t bytes);
 TinyNNStatus megcc_gfx950_model_forward(void* model);
+/* No counterpart in the reference either. With plain launches (launch mode -1) the last operators
+ * of a forward - the suffix of operators whose tensors are at most 8 MB each, a classifier head for
+ * instance - are launched on a second stream, ordered behind the rest by an event, so that they
+ * overlap the first operators of the NEXT forward, which do not depend on them (the runtime's own
+ * memory plan gives what they touch bytes of its own; under any other plan the next forward waits
+ * for them before it writes bytes they use). megcc_gfx950_wait(), megcc_gfx950_model_get_output()
+ * and megcc_gfx950_model_set_input() (for an input those operators read) take that into account.
+ * A caller that orders work of its own on megcc_gfx950_stream() behind a forward - an event, a
+ * copy - calls megcc_gfx950_model_join() first: it makes the library stream wait (on the device,
+ * not the host) for everything the model's forwards have launched. Switch "nopipeline"
+ * (MEGCC_NOPIPELINE=1) keeps every operator on the library stream. */
+TinyNNStatus megcc_gfx950_model_join(void* model);
+/* how many of megcc_gfx950_model_nr_kernel's kernels those last operators are (0: none) */
+int megcc_gfx950_model_nr_tail_kernel(void* model);
+/* megcc_gfx950_model_get_output without the host waiting: the copy is enqueued behind the forward
+ * that produced the tensor (on the second stream when that forward's last operators are there) and
+ * the bytes are in `host` - pinned memory, for the copy to be asynchronous - after
+ * megcc_gfx950_wait(). The loop forward(i), get_output_async(i), set_input(i + 1), forward(i + 1)
+ * keeps forward i's last operators overlapped with forward i + 1's first, which the blocking call
+ * cannot: the host would not enqueue forward i + 1 before forward i is over. */
+TinyNNStatus megcc_gfx950_model_get_output_async(void* model, int tensor, void* host, size_t bytes);
 int megcc_gfx950_model_nr_opr(void* model);
 /* one instruction only: per-layer timing / tensor dumps (the TINYNN_PROFILE_KERNEL and
  * TINYNN_DUMP_TENSOR hooks of runtime/src/lite/network.c:187-224) */

@@ -10,6 +10,14 @@ namespace mg {
 
 // One stream for every launch and copy, default priority, created on first use.
 hipStream_t stream();
+// The library stream itself, whatever stream() currently answers.
+hipStream_t main_stream();
+// While `on`, stream() answers `s` on this thread: the model runtime launches the last operators of a
+// forward on a second stream this way (model.cpp). The kernels' launch code is unchanged.
+void set_stream_override(hipStream_t s, bool on);
+// Streams megcc_gfx950_wait() synchronises besides the library stream.
+void register_aux_stream(hipStream_t s);
+void unregister_aux_stream(hipStream_t s);
 
 // Compute units of the current device (256 when the query fails).
 int num_cus();
@@ -62,7 +70,7 @@ __device__ __forceinline__ void xcd_tile(XcdOrder o, int bx, int by, int gx, int
 // environment (MEGCC_NOPWS=1, ...) ONCE, when the library first consults them; later changes go
 // through megcc_gfx950_set_option(). Nothing on a launch path scans the environment.
 struct Options {
-    bool no_pws, no_gevm, no_fcb, no_small, no_pm768, no_pm, no_dma512, no_pm256, no_dma, no_fcs, no_pwshare, no_hybrid, no_dot4, no_f32small, dw_generic, no_dwmfma, no_dwnchw, no_fuse_softmax, no_graph, no_poolrows, no_firstmfma, no_rowsplit, no_fuse_chain, no_fuse_pwdw, fuse_pwdw, no_fcone, no_xcdorder, no_affine;
+    bool no_pws, no_gevm, no_fcb, no_small, no_pm768, no_pm, no_dma512, no_pm256, no_dma, no_fcs, no_pwshare, no_hybrid, no_dot4, no_f32small, dw_generic, no_dwmfma, no_dwnchw, no_fuse_softmax, no_graph, no_poolrows, no_firstmfma, no_rowsplit, no_fuse_chain, no_fuse_pwdw, fuse_pwdw, no_fcone, no_xcdorder, no_affine, no_pipeline;
 };
 Options& options();
 

@@ -7,6 +7,7 @@
 #include <string.h>
 
 #include <mutex>
+#include <vector>
 
 #include "common.h"
 #include "epilogue.h"
@@ -32,7 +33,7 @@ const OptionName kOptions[] = {
         {"nodot4", &Options::no_dot4},       {"nof32small", &Options::no_f32small},
         {"dw_generic", &Options::dw_generic}, {"no_graph", &Options::no_graph},
         {"nodwmfma", &Options::no_dwmfma},   {"nodwnchw", &Options::no_dwnchw},
-        {"nofusesoftmax", &Options::no_fuse_softmax}, {"nopoolrows", &Options::no_poolrows}, {"nofirstmfma", &Options::no_firstmfma}, {"norowsplit", &Options::no_rowsplit}, {"nofusechain", &Options::no_fuse_chain}, {"nofusepwdw", &Options::no_fuse_pwdw}, {"fusepwdw", &Options::fuse_pwdw}, {"nofcone", &Options::no_fcone}, {"noxcdorder", &Options::no_xcdorder}, {"noaffine", &Options::no_affine},
+        {"nofusesoftmax", &Options::no_fuse_softmax}, {"nopoolrows", &Options::no_poolrows}, {"nofirstmfma", &Options::no_firstmfma}, {"norowsplit", &Options::no_rowsplit}, {"nofusechain", &Options::no_fuse_chain}, {"nofusepwdw", &Options::no_fuse_pwdw}, {"fusepwdw", &Options::fuse_pwdw}, {"nofcone", &Options::no_fcone}, {"noxcdorder", &Options::no_xcdorder}, {"noaffine", &Options::no_affine}, {"nopipeline", &Options::no_pipeline},
 };
 struct KernelNote {
     const char* name;
@@ -74,12 +75,40 @@ void note_requant_affine(bool on) {
     g_note_affine = on;
 }
 
-hipStream_t stream() {
+static thread_local hipStream_t g_stream_override = nullptr;
+static thread_local bool g_stream_override_on = false;
+static std::mutex g_aux_lock;
+static std::vector<hipStream_t> g_aux_streams;
+
+hipStream_t main_stream() {
     std::call_once(g_stream_once, [] {
         if (hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking) != hipSuccess)
             g_stream = nullptr;  // falls back to the null stream; launches still work
     });
     return g_stream;
+}
+
+hipStream_t stream() {
+    return g_stream_override_on ? g_stream_override : main_stream();
+}
+
+void set_stream_override(hipStream_t s, bool on) {
+    g_stream_override = s;
+    g_stream_override_on = on;
+}
+
+void register_aux_stream(hipStream_t s) {
+    std::lock_guard<std::mutex> guard(g_aux_lock);
+    g_aux_streams.push_back(s);
+}
+
+void unregister_aux_stream(hipStream_t s) {
+    std::lock_guard<std::mutex> guard(g_aux_lock);
+    for (size_t i = 0; i < g_aux_streams.size(); ++i)
+        if (g_aux_streams[i] == s) {
+            g_aux_streams.erase(g_aux_streams.begin() + (long)i);
+            break;
+        }
 }
 
 TinyNNStatus fail(TinyNNStatus st, const char* fmt, ...) {
@@ -187,13 +216,23 @@ TinyNNStatus megcc_gfx950_memset(void* dst, int value, size_t length) {
 }
 
 TinyNNStatus megcc_gfx950_wait(void) {
-    hipError_t e = hipStreamSynchronize(stream());
+    hipError_t e = hipStreamSynchronize(main_stream());
     MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "wait: %s", hipGetErrorString(e));
+    // (the streams on which models run the last operators of their forwards)
+    std::vector<hipStream_t> aux;
+    {
+        std::lock_guard<std::mutex> guard(g_aux_lock);
+        aux = g_aux_streams;
+    }
+    for (hipStream_t s : aux) {
+        e = hipStreamSynchronize(s);
+        MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "wait: %s", hipGetErrorString(e));
+    }
     return TinyNN_SUCCESS;
 }
 
 void* megcc_gfx950_stream(void) {
-    return (void*)stream();
+    return (void*)main_stream();
 }
 
 const char* megcc_gfx950_last_error(void) {

@@ -49,6 +49,7 @@ struct ModelOpr {
     bool has_processed = false;
     void* processed_mem = nullptr;
     Workspace ws;
+    int first_index = -1;  // index in Model::oprs of the (first) operator this schedule entry stands for
 };
 
 struct Model {
@@ -85,6 +86,21 @@ struct Model {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
+    // Consecutive forwards overlap: the last operators of a network are small (a few megabytes, a
+    // launch floor each) and the first operators of the next forward do not depend on them, so with
+    // plain launches the schedule from `tail_begin` on runs on a second stream, ordered behind the head
+    // by an event, while the library stream is free for the next forward's head. `tail_opr_begin` is
+    // the same boundary in `oprs` (chosen before the memory plan, which then gives every tensor the
+    // tail touches bytes of its own); `waits_tail[i]`: head entry i writes bytes the previous
+    // forward's tail may still be using and waits for it first (under the runtime's own plan that is
+    // only the entry that produces the tail's input). The tail has its own workspace.
+    int tail_opr_begin = -1, tail_begin = -1;
+    hipStream_t tail_stream = nullptr;
+    hipEvent_t ev_head = nullptr, ev_tail = nullptr;
+    bool tail_pending = false, tail_reads_input = false;
+    std::vector<char> waits_tail;
+    std::vector<const Tensor*> tail_writes;  // tensors the tail's operators write
+    void* tail_workspace = nullptr;
 };
 
 size_t tensor_bytes(const Tensor& t) {
@@ -107,6 +123,47 @@ int root_of(const Model* m, int id) {
 // planned: the compiler plans allocations only and the function arguments are the caller's memory
 // (runtime/src/init.c:456-460); here each input is a device buffer of its own, which keeps what
 // set_input put there across any number of forwards. Outputs stay valid after forward().
+// The suffix of the operator list that may run on the tail stream: operators whose tensors (weights
+// apart) are at most 8 MB each - far too little to fill the chip, so they overlap the next forward's
+// first operators at no cost to them - behind a head of at least four operators.
+static void choose_tail(Model* m) {
+    m->tail_opr_begin = -1;
+    if (options().no_pipeline)
+        return;
+    const int n = (int)m->oprs.size();
+    auto small = [&](const ModelOpr* o) {
+        size_t bytes = 0;
+        for (int id : o->in)
+            if (!m->tensors[id]->is_weight)
+                bytes += tensor_bytes(m->tensors[id]->t);
+        for (int id : o->out)
+            bytes += tensor_bytes(m->tensors[id]->t);
+        return bytes <= (size_t)8 << 20;
+    };
+    // (what the tail touches gets bytes of its own in the memory plan: at most 64 MB of them)
+    std::vector<char> seen(m->tensors.size(), 0);
+    size_t own = 0;
+    int k = n;
+    while (k > 0 && small(m->oprs[k - 1])) {
+        const ModelOpr* o = m->oprs[k - 1];
+        size_t more = 0;
+        for (const std::vector<int>* ids : {&o->in, &o->out})
+            for (int id : *ids) {
+                const int r = root_of(m, id);
+                if (!seen[r] && !m->tensors[r]->is_weight && !m->tensors[r]->is_input) {
+                    seen[r] = 1;
+                    more += tensor_bytes(m->tensors[r]->t);
+                }
+            }
+        if (own + more > (size_t)64 << 20)
+            break;
+        own += more;
+        --k;
+    }
+    if (k >= 4 && n - k >= 2)
+        m->tail_opr_begin = k;
+}
+
 bool plan_memory(Model* m) {
     if (m->preplanned)
         return true;
@@ -136,6 +193,15 @@ bool plan_memory(Model* m) {
                 keep_until[root_of(m, o0->in[0])] = (int)i + 1;
         }
     }
+    // What the tail of a forward touches shares no byte with anything else: the head of the next
+    // forward runs while the tail is still at work.
+    std::vector<char> pinned(m->tensors.size(), 0);
+    for (size_t i = m->tail_opr_begin < 0 ? m->oprs.size() : (size_t)m->tail_opr_begin; i < m->oprs.size(); ++i) {
+        for (int id : m->oprs[i]->in)
+            pinned[root_of(m, id)] = 1;
+        for (int id : m->oprs[i]->out)
+            pinned[root_of(m, id)] = 1;
+    }
     std::vector<MemInterval> intervals;
     std::vector<int> ids;
     for (size_t i = 0; i < m->tensors.size(); ++i) {
@@ -143,8 +209,8 @@ bool plan_memory(Model* m) {
         if (t->is_weight || t->is_input || t->alias_of >= 0 || t->def < 0)
             continue;
         MemInterval iv;
-        iv.begin = (size_t)t->def;
-        iv.end = t->is_output ? m->oprs.size() + 1 : (size_t)std::max(t->last, keep_until[i]) + 1;
+        iv.begin = pinned[i] ? 0 : (size_t)t->def;
+        iv.end = t->is_output || pinned[i] ? m->oprs.size() + 1 : (size_t)std::max(t->last, keep_until[i]) + 1;
         iv.size = tensor_bytes(t->t);
         intervals.push_back(iv);
         ids.push_back((int)i);
@@ -221,6 +287,8 @@ static float time_oprs(Model* m, const std::vector<ModelOpr*>& ops, int iters) {
 static void build_schedule(Model* m) {
     m->schedule.clear();
     const int n = (int)m->oprs.size();
+    for (int i = 0; i < n; ++i)
+        m->oprs[i]->first_index = i;
     std::vector<int> readers(m->tensors.size(), 0);
     for (auto* o : m->oprs)
         for (int id : o->in)
@@ -257,6 +325,7 @@ static void build_schedule(Model* m) {
                 m->tensors[o0->out[0]]->t.dtype.param.scale == m->tensors[o1->out[0]]->t.dtype.param.scale) {
                 const int other = o2->in[0] == o1->out[0] ? o2->in[1] : o2->in[0];
                 ModelOpr* f = new ModelOpr();
+                f->first_index = i;
                 memset(&f->desc, 0, sizeof(f->desc));
                 f->desc.kind = MEGCC_KERN_DW_POOL_ADD;
                 f->desc.attr.dw_pool_add.conv = o0->desc.attr.conv;
@@ -296,6 +365,7 @@ static void build_schedule(Model* m) {
                 o1->in.size() == (o1->desc.attr.conv.with_bias ? 3u : 2u) && o1->in[0] == o0->out[0] &&
                 o1->desc.attr.conv.sparse == MEGCC_SPARSE_GROUP && temp(o0->out[0], 1)) {
                 ModelOpr* f = new ModelOpr();
+                f->first_index = i;
                 memset(&f->desc, 0, sizeof(f->desc));
                 f->desc.kind = MEGCC_KERN_PW_DW;
                 f->desc.attr.pw_dw.pw = o0->desc.attr.conv;
@@ -383,9 +453,12 @@ static void build_schedule(Model* m) {
                     continue;
                 }
                 ModelOpr* f = new ModelOpr();
+                f->first_index = i;
                 memset(&f->desc, 0, sizeof(f->desc));
                 f->desc.kind = MEGCC_KERN_SOFTMAX;
                 f->symbol = "softmax (fused)";
+                if (src != x)
+                    f->first_index = i - 1;  // (the dequantisation in front joined)
                 memset(&f->ws, 0, sizeof(f->ws));
                 f->in.push_back(src);
                 f->out.push_back(y);
@@ -398,6 +471,67 @@ static void build_schedule(Model* m) {
             }
         }
         m->schedule.push_back(o0);
+    }
+}
+
+// The tail stream, its events and workspace, and which head entries must wait for the previous
+// forward's tail (see Model::tail_begin). Leaves tail_begin at -1 when there is nothing to overlap.
+static void setup_tail(Model* m) {
+    m->tail_begin = -1;
+    if (m->tail_opr_begin < 0)
+        return;
+    const int n = (int)m->schedule.size();
+    int tb = -1;
+    for (int s = 0; s < n; ++s)
+        if (m->schedule[s]->first_index >= m->tail_opr_begin) {
+            tb = s;
+            break;
+        }
+    if (tb < 1 || tb >= n)
+        return;
+    // every tensor the tail reads or writes (weights are never written by anyone)
+    std::vector<const Tensor*> touched;
+    size_t ws_bytes = 0;
+    for (int s = tb; s < n; ++s) {
+        const ModelOpr* o = m->schedule[s];
+        for (const Tensor* t : o->in_ptrs)
+            if (!t->is_weight) {
+                touched.push_back(t);
+                m->tail_reads_input = m->tail_reads_input || t->is_input;
+            }
+        for (const Tensor* t : o->out_ptrs) {
+            touched.push_back(t);
+            m->tail_writes.push_back(t);
+        }
+        ws_bytes = std::max(ws_bytes, (size_t)o->ws.size);
+    }
+    if (hipStreamCreateWithFlags(&m->tail_stream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&m->ev_head, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&m->ev_tail, hipEventDisableTiming) != hipSuccess)
+        return;
+    if (ws_bytes) {
+        m->tail_workspace = m->dev.malloc(ws_bytes);
+        if (!m->tail_workspace)
+            return;
+        for (int s = tb; s < n; ++s)
+            if (m->schedule[s]->ws.size)
+                m->schedule[s]->ws.ptr = m->tail_workspace;
+    }
+    m->waits_tail.assign((size_t)tb, 0);
+    for (int s = 0; s < tb; ++s)
+        for (const Tensor* w : m->schedule[s]->out_ptrs)
+            for (const Tensor* t : touched)
+                if (shares_bytes(*w, *t))
+                    m->waits_tail[(size_t)s] = 1;
+    register_aux_stream(m->tail_stream);
+    m->tail_begin = tb;
+}
+
+// Makes the library stream wait for the tail of the last forward (nothing to do when there is none).
+static void join_tail(Model* m) {
+    if (m->tail_pending) {
+        (void)hipStreamWaitEvent(main_stream(), m->ev_tail, 0);
+        m->tail_pending = false;
     }
 }
 
@@ -420,6 +554,17 @@ void megcc_gfx950_model_destroy(void* model) {
     if (!m)
         return;
     (void)hipStreamSynchronize(stream());
+    if (m->tail_stream) {
+        (void)hipStreamSynchronize(m->tail_stream);
+        unregister_aux_stream(m->tail_stream);
+        (void)hipStreamDestroy(m->tail_stream);
+    }
+    if (m->ev_head)
+        (void)hipEventDestroy(m->ev_head);
+    if (m->ev_tail)
+        (void)hipEventDestroy(m->ev_tail);
+    if (m->tail_workspace)
+        m->dev.free(m->tail_workspace);
     for (auto* o : m->oprs) {
         if (o->processed_mem)
             m->dev.free(o->processed_mem);
@@ -625,6 +770,7 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
     for (auto* t : m->tensors)
         if (t->is_input && t->def != 0)
             t->def = 0;
+    choose_tail(m);
     MG_REQUIRE(plan_memory(m), TinyNN_ERROR_INVALID_LAYOUT,
                "model_finalize: memory plan (alignment %zu)", (size_t)m->dev.alignment);
     m->arena = m->dev.malloc(m->arena_bytes ? m->arena_bytes : 1);
@@ -720,6 +866,7 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
             o->ws.ptr = o->ws.size ? m->workspace : nullptr;
     }
     build_schedule(m);
+    setup_tail(m);
     m->finalized = true;
     return megcc_gfx950_wait();
 }
@@ -787,6 +934,8 @@ TinyNNStatus megcc_gfx950_model_set_input(void* model, int tensor, const void* h
     Tensor& t = m->tensors[tensor]->t;
     MG_REQUIRE(bytes == tensor_bytes(t), TinyNN_ERROR_INVALID_LAYOUT,
                "model_set_input: %zu bytes given, tensor has %zu", bytes, tensor_bytes(t));
+    if (m->tail_reads_input)
+        join_tail(m);  // (the last forward's tail may still be reading a model input)
     return megcc_gfx950_memcpy_h2d(t.ptr, host, bytes);
 }
 
@@ -797,20 +946,61 @@ TinyNNStatus megcc_gfx950_model_get_output(void* model, int tensor, void* host, 
     Tensor& t = m->tensors[tensor]->t;
     MG_REQUIRE(bytes == tensor_bytes(t), TinyNN_ERROR_INVALID_LAYOUT,
                "model_get_output: %zu bytes asked, tensor has %zu", bytes, tensor_bytes(t));
+    join_tail(m);
     return megcc_gfx950_memcpy_d2h(host, t.ptr, bytes);
+}
+
+// The copy is enqueued behind the forward that produced the tensor - on the tail stream when the last
+// forward left its tail there - and the host does not wait: a caller that enqueues forward i, this
+// copy, the next input and forward i + 1 keeps the overlap of forward i's tail with forward i + 1's
+// head, which the blocking get_output cannot (the host would not enqueue forward i + 1 before
+// forward i is over). `host` should be pinned memory; the bytes are there after megcc_gfx950_wait().
+TinyNNStatus megcc_gfx950_model_get_output_async(void* model, int tensor, void* host, size_t bytes) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && m->finalized && host && tensor >= 0 && tensor < (int)m->tensors.size(),
+               TinyNN_ERROR_OUT_OF_RANGE, "model_get_output_async: bad argument");
+    Tensor& t = m->tensors[tensor]->t;
+    MG_REQUIRE(bytes == tensor_bytes(t), TinyNN_ERROR_INVALID_LAYOUT,
+               "model_get_output_async: %zu bytes asked, tensor has %zu", bytes, tensor_bytes(t));
+    // a tensor the tail writes: behind the tail, on its stream (the next forward's tail follows the
+    // copy there); any other: on the library stream, between this forward's head and the next one's
+    bool by_tail = false;
+    for (const Tensor* w : m->tail_writes)
+        by_tail = by_tail || shares_bytes(*w, t);
+    hipStream_t s = m->tail_pending && by_tail ? m->tail_stream : main_stream();
+    hipError_t e = hipMemcpyAsync(host, t.ptr, bytes, hipMemcpyDeviceToHost, s);
+    MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "model_get_output_async: %s", hipGetErrorString(e));
+    return TinyNN_SUCCESS;
 }
 
 // LITE_forward: one asynchronous kernel launch per Opr, in order, on the library stream; stops at
 // the first failing kernel like network.c:191-194. Results are visible after megcc_gfx950_wait().
-static TinyNNStatus forward_eager(Model* m) {
-    for (auto* o : m->schedule) {
-        TinyNNStatus st = megcc_gfx950_call(
+// `overlap`: the entries from tail_begin on go to the tail stream (plain launches of a model whose way
+// of launching is decided; never under capture or between timing events).
+static TinyNNStatus forward_eager(Model* m, bool overlap = false) {
+    const int tb = overlap ? m->tail_begin : -1;
+    if (tb < 0)
+        join_tail(m);
+    TinyNNStatus st = TinyNN_SUCCESS;
+    for (int idx = 0; idx < (int)m->schedule.size() && st == TinyNN_SUCCESS; ++idx) {
+        ModelOpr* o = m->schedule[(size_t)idx];
+        if (idx == tb) {
+            (void)hipEventRecord(m->ev_head, main_stream());
+            (void)hipStreamWaitEvent(m->tail_stream, m->ev_head, 0);
+            set_stream_override(m->tail_stream, true);
+        } else if (idx < tb && m->tail_pending && m->waits_tail[(size_t)idx]) {
+            join_tail(m);
+        }
+        st = megcc_gfx950_call(
                 &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), o->out_ptrs.data(),
                 (int)o->out_ptrs.size(), &o->ws, &m->opt);
-        if (st != TinyNN_SUCCESS)
-            return st;
     }
-    return TinyNN_SUCCESS;
+    if (tb >= 0) {
+        set_stream_override(nullptr, false);
+        (void)hipEventRecord(m->ev_tail, m->tail_stream);
+        m->tail_pending = true;
+    }
+    return st;
 }
 
 TinyNNStatus megcc_gfx950_model_forward(void* model) {
@@ -825,7 +1015,7 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
     if (m->graph_state == 1)
         return replay();
     if (m->graph_state == -1)
-        return forward_eager(m);
+        return forward_eager(m, true);
     // ---- undecided: the first ten forwards (1: plain; 2, 3, 7, 8: timed plain launches; 4: the capture
     //      and its first replay; 5, 6, 9, 10: timed replays)
     // (schedules of fewer than 5 kernels stay eager without asking: the depthwise + pooling + addition
@@ -893,6 +1083,21 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
     return st;
 }
 
+// Kernels of one forward that go to the second stream under plain launches (0: none).
+int megcc_gfx950_model_nr_tail_kernel(void* model) {
+    Model* m = (Model*)model;
+    return m && m->finalized && m->tail_begin >= 0 ? (int)m->schedule.size() - m->tail_begin : 0;
+}
+
+// Orders the library stream behind everything the model's forwards have launched (the last
+// operators of a forward may run on a second stream; see Model::tail_begin).
+TinyNNStatus megcc_gfx950_model_join(void* model) {
+    Model* m = (Model*)model;
+    MG_REQUIRE(m && m->finalized, TinyNN_ERROR_NULL_PTR, "model_join: model not finalized");
+    join_tail(m);
+    return TinyNN_SUCCESS;
+}
+
 int megcc_gfx950_model_nr_opr(void* model) {
     return model ? (int)((Model*)model)->oprs.size() : 0;
 }
@@ -904,6 +1109,7 @@ TinyNNStatus megcc_gfx950_model_run_opr(void* model, int index) {
     MG_REQUIRE(m && m->finalized && index >= 0 && index < (int)m->oprs.size(),
                TinyNN_ERROR_OUT_OF_RANGE, "model_run_opr: index %d", index);
     ModelOpr* o = m->oprs[index];
+    join_tail(m);
     return megcc_gfx950_call(
             &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), o->out_ptrs.data(),
             (int)o->out_ptrs.size(), &o->ws, &m->opt);

@@ -82,6 +82,8 @@ def lib():
         L.megcc_gfx950_model_set_input.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t]
         L.megcc_gfx950_model_get_output.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t]
         L.megcc_gfx950_model_forward.argtypes = [C.c_void_p]
+        L.megcc_gfx950_model_join.argtypes = [C.c_void_p]
+        L.megcc_gfx950_model_get_output_async.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_size_t]
         L.megcc_gfx950_model_nr_opr.argtypes = [C.c_void_p]
         L.megcc_gfx950_model_run_opr.argtypes = [C.c_void_p, C.c_int]
         L.megcc_gfx950_model_load.argtypes = [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]
@@ -115,7 +117,7 @@ EXPORTS = [
     "megcc_gfx950_model_mark_io", "megcc_gfx950_model_finalize", "megcc_gfx950_model_arena_bytes",
     "megcc_gfx950_model_set_plan", "megcc_gfx950_model_nr_kernel", "megcc_gfx950_model_launch_mode",
     "megcc_gfx950_model_tensor_ptr", "megcc_gfx950_model_set_input",
-    "megcc_gfx950_model_get_output", "megcc_gfx950_model_forward", "megcc_gfx950_model_nr_opr",
+    "megcc_gfx950_model_get_output", "megcc_gfx950_model_forward", "megcc_gfx950_model_join", "megcc_gfx950_model_nr_tail_kernel", "megcc_gfx950_model_get_output_async", "megcc_gfx950_model_nr_opr",
     "megcc_gfx950_model_run_opr", "megcc_gfx950_plan_memory", "megcc_gfx950_model_load",
     "megcc_gfx950_tiny_describe",
 ]
@@ -403,6 +405,14 @@ class Model:
         L.megcc_gfx950_model_nr_kernel.argtypes = [C.c_void_p]
         return L.megcc_gfx950_model_nr_kernel(self.h)
 
+    @property
+    def nr_tail_kernel(self):
+        """how many of those kernels run on the second stream under plain launches (they overlap the
+        next forward's first kernels)"""
+        L = lib()
+        L.megcc_gfx950_model_nr_tail_kernel.argtypes = [C.c_void_p]
+        return L.megcc_gfx950_model_nr_tail_kernel(self.h)
+
     def launch_mode(self):
         """(mode, eager_ms, graph_ms): 1 = graph replay, -1 = one launch per kernel, 0 = undecided"""
         L = lib()
@@ -426,6 +436,11 @@ class Model:
     def forward(self):
         check(lib().megcc_gfx950_model_forward(self.h), "forward")
 
+    def join(self):
+        """orders the library stream behind everything forward() has launched (the last operators of
+        a forward may run on a second stream)"""
+        check(lib().megcc_gfx950_model_join(self.h), "join")
+
     def run_opr(self, index):
         check(lib().megcc_gfx950_model_run_opr(self.h, index), "run_opr")
 
@@ -434,6 +449,13 @@ class Model:
         out = np.empty(shape, abi.np_dtype(type_enum))
         check(lib().megcc_gfx950_model_get_output(self.h, tid, out.ctypes.data, out.nbytes), "get_output")
         return out
+
+    def get_async(self, tid, out):
+        """enqueues the copy of tensor `tid` into the array `out` behind the forward that produced it;
+        the bytes are there after wait()"""
+        shape, type_enum = self.shapes[tid]
+        assert out.shape == tuple(shape) and out.dtype == abi.np_dtype(type_enum) and out.flags["C_CONTIGUOUS"]
+        check(lib().megcc_gfx950_model_get_output_async(self.h, tid, out.ctypes.data, out.nbytes), "get_output_async")
 
     def close(self):
         if self.h:

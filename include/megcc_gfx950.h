@@ -658,14 +658,16 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model);
 /* No counterpart in the reference (its VM runs one kernel per Opr, synchronously): the number of
  * kernels one forward launches (an operator chain that runs as one kernel counts once; a chain is
  * only replaced when its result shares no byte with anything the one kernel reads), and how they
- * are launched: 1 = HIP-graph replay, -1 = one launch per kernel, 0 = still measuring. forward()
- * 2, 3 and 5 to 10 of a model with at least 5 kernels each block the host until that forward has
- * finished (they time the two ways between events on the library stream; a sample is the time on
- * the device or the time the host took to enqueue the forward, whichever is longer - what limits
- * back-to-back forwards; *eager_ms / *graph_ms receive the shortest of four samples each, -1 when
- * not measured; the replay is kept when it is at least 2 % faster, or not more than 5 % slower
- * when the kernels average under 6 us each - back-to-back plain launches of such a model are bound
- * by the host); every other forward is asynchronous. */
+ * are launched: 1 = HIP-graph replay, -1 = one launch per kernel, 0 = still measuring. The first ten
+ * forwards of a model with at least 5 kernels measure: 2 + 3 and 7 + 8 are pairs of plain-launch
+ * forwards between two events on the library stream, 5 + 6 and 9 + 10 pairs of replays (4 captures);
+ * the second forward of a pair blocks the host until both are done. A pair's cost is the time on
+ * the device from the end of its first forward to the end of its second - the first forward's last
+ * operators overlapping the second one's first where plain launches allow it
+ * (megcc_gfx950_model_join below) - or the time the host took to enqueue the second forward,
+ * whichever is longer: what limits back-to-back forwards. *eager_ms /
+ * *graph_ms receive the lower of the two pairs each, -1 when not measured; the replay is kept when
+ * it is at least 2 % faster. Every other forward is asynchronous. */
 int megcc_gfx950_model_nr_kernel(void* model);
 int megcc_gfx950_model_launch_mode(void* model, float* eager_ms, float* graph_ms);
 size_t megcc_gfx950_model_arena_bytes(void* model);
@@ -674,8 +676,8 @@ TinyNNStatus megcc_gfx950_model_set_input(void* model, int tensor, const void* h
 TinyNNStatus megcc_gfx950_model_get_output(void* model, int tensor, void* host, size_t bytes);
 TinyNNStatus megcc_gfx950_model_forward(void* model);
 /* No counterpart in the reference either. With plain launches (launch mode -1) the last operators
- * of a forward - the suffix of operators whose tensors are at most 8 MB each, a classifier head for
- * instance - are launched on a second stream, ordered behind the rest by an event, so that they
+ * of a forward - the longest suffix estimated to take no longer than the operators before it - are
+ * launched on a second stream, ordered behind the rest by an event, so that they
  * overlap the first operators of the NEXT forward, which do not depend on them (the runtime's own
  * memory plan gives what they touch bytes of its own; under any other plan the next forward waits
  * for them before it writes bytes they use). megcc_gfx950_wait(), megcc_gfx950_model_get_output()

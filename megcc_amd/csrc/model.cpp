@@ -123,28 +123,34 @@ int root_of(const Model* m, int id) {
 // planned: the compiler plans allocations only and the function arguments are the caller's memory
 // (runtime/src/init.c:456-460); here each input is a device buffer of its own, which keeps what
 // set_input put there across any number of forwards. Outputs stay valid after forward().
-// The suffix of the operator list that may run on the tail stream: operators whose tensors (weights
-// apart) are at most 8 MB each - far too little to fill the chip, so they overlap the next forward's
-// first operators at no cost to them - behind a head of at least four operators.
+// Where the tail of a forward may begin (see Model::tail_begin): the longest suffix of the operator
+// list estimated to take at most 55 % of the forward - the two streams should end up with about the
+// same amount of work, which is where back-to-back forwards gain most (MobileNetV1: the split falls
+// behind the 28 x 28 layers at every batch from 16 to 128); setup_tail() shortens it to the measured
+// balance - with a head of at least four operators, a tail of at least two, and at most 128 MB of
+// tensors in the tail (they get bytes of their own in the memory plan). The estimate is a launch
+// floor plus the operator's tensors at half the memory bandwidth.
 static void choose_tail(Model* m) {
     m->tail_opr_begin = -1;
     if (options().no_pipeline)
         return;
     const int n = (int)m->oprs.size();
-    auto small = [&](const ModelOpr* o) {
+    std::vector<double> us((size_t)n);
+    double total = 0;
+    for (int i = 0; i < n; ++i) {
         size_t bytes = 0;
-        for (int id : o->in)
-            if (!m->tensors[id]->is_weight)
-                bytes += tensor_bytes(m->tensors[id]->t);
-        for (int id : o->out)
+        for (int id : m->oprs[i]->in)
             bytes += tensor_bytes(m->tensors[id]->t);
-        return bytes <= (size_t)8 << 20;
-    };
-    // (what the tail touches gets bytes of its own in the memory plan: at most 64 MB of them)
+        for (int id : m->oprs[i]->out)
+            bytes += tensor_bytes(m->tensors[id]->t);
+        us[(size_t)i] = 3.8 + (double)bytes / 4.0e6;
+        total += us[(size_t)i];
+    }
     std::vector<char> seen(m->tensors.size(), 0);
     size_t own = 0;
+    double tail = 0;
     int k = n;
-    while (k > 0 && small(m->oprs[k - 1])) {
+    while (k > 4 && tail + us[(size_t)k - 1] <= 0.55 * total) {
         const ModelOpr* o = m->oprs[k - 1];
         size_t more = 0;
         for (const std::vector<int>* ids : {&o->in, &o->out})
@@ -155,12 +161,13 @@ static void choose_tail(Model* m) {
                     more += tensor_bytes(m->tensors[r]->t);
                 }
             }
-        if (own + more > (size_t)64 << 20)
+        if (own + more > (size_t)128 << 20)
             break;
         own += more;
+        tail += us[(size_t)k - 1];
         --k;
     }
-    if (k >= 4 && n - k >= 2)
+    if (n - k >= 2)
         m->tail_opr_begin = k;
 }
 
@@ -489,6 +496,41 @@ static void setup_tail(Model* m) {
         }
     if (tb < 1 || tb >= n)
         return;
+    // The boundary the memory plan was made for came from an estimate; with the kernels at hand each
+    // entry is timed (a few launches on the tensors as they are; the estimate stands in for an entry
+    // that reads a model input, which has no memory yet) and the tail is shortened until it takes no
+    // longer than the head: one fused pair too many on the tail costs MobileNetV1 batch 64 3 %.
+    {
+        std::vector<double> us((size_t)n);
+        double total = 0;
+        for (int s = 0; s < n; ++s) {
+            ModelOpr* o = m->schedule[(size_t)s];
+            const float ms = time_oprs(m, {o}, 8);
+            if (ms > 0.f) {
+                us[(size_t)s] = ms * 1e3 / 8;
+            } else {
+                size_t bytes = 0;
+                for (const Tensor* t : o->in_ptrs)
+                    bytes += tensor_bytes(*t);
+                for (const Tensor* t : o->out_ptrs)
+                    bytes += tensor_bytes(*t);
+                us[(size_t)s] = 3.8 + (double)bytes / 4.0e6;
+            }
+            total += us[(size_t)s];
+        }
+        // A network whose kernels average under 6 us is bound by launches, not by the device: two
+        // streams then gain or lose a quarter from run to run (MobileNetV1 batch 1: 7.2 k ... 9.9 k
+        // img/s) where one stream or a graph replay is steady. One stream.
+        if (total < 6.0 * n)
+            return;
+        double tail = 0;
+        for (int s = tb; s < n; ++s)
+            tail += us[(size_t)s];
+        while (tb < n - 2 && tail > total - tail) {
+            tail -= us[(size_t)tb];
+            ++tb;
+        }
+    }
     // every tensor the tail reads or writes (weights are never written by anyone)
     std::vector<const Tensor*> touched;
     size_t ws_bytes = 0;
@@ -977,7 +1019,8 @@ TinyNNStatus megcc_gfx950_model_get_output_async(void* model, int tensor, void* 
 // the first failing kernel like network.c:191-194. Results are visible after megcc_gfx950_wait().
 // `overlap`: the entries from tail_begin on go to the tail stream (plain launches of a model whose way
 // of launching is decided; never under capture or between timing events).
-static TinyNNStatus forward_eager(Model* m, bool overlap = false) {
+// `done`: an event recorded behind the forward's last operator, on whichever stream that is.
+static TinyNNStatus forward_eager(Model* m, bool overlap = false, hipEvent_t done = nullptr) {
     const int tb = overlap ? m->tail_begin : -1;
     if (tb < 0)
         join_tail(m);
@@ -1000,6 +1043,8 @@ static TinyNNStatus forward_eager(Model* m, bool overlap = false) {
         (void)hipEventRecord(m->ev_tail, m->tail_stream);
         m->tail_pending = true;
     }
+    if (done)
+        (void)hipEventRecord(done, tb >= 0 ? m->tail_stream : main_stream());
     return st;
 }
 
@@ -1030,16 +1075,26 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
         m->graph_state = -1;
         return forward_eager(m);
     }
-    // One forward between two events; keeps the shortest cost seen. The cost of a way of launching is
-    // what limits back-to-back forwards: the time on the device or, when that is longer, the time the
-    // host needs to enqueue one forward (31 plain launches of a batch-1 network take the host longer
-    // than the device takes to run them, which a single forward between events does not show).
-    auto timed = [&](bool graph, float* best) -> TinyNNStatus {
-        (void)hipEventRecord(m->ev0, stream());
+    // Two consecutive forwards, an event behind the last operator of each; keeps the shortest cost
+    // seen. The cost of a way of launching is what limits back-to-back forwards: the time from the end
+    // of one forward to the end of the next on the device - under plain launches the second one's
+    // first operators overlap the first one's last, which are on the second stream - or, when that
+    // is longer, the time the host needs to enqueue a forward behind another (26 plain launches of a
+    // batch-1 network take the host longer than the device takes to run them). The first forward of a
+    // pair returns at once, the second one blocks until both are done.
+    auto timed = [&](bool graph, bool second, float* best) -> TinyNNStatus {
+        hipEvent_t done = second ? m->ev1 : m->ev0;
         const auto h0 = std::chrono::steady_clock::now();
-        TinyNNStatus st = graph ? replay() : forward_eager(m);
+        TinyNNStatus st;
+        if (graph) {
+            st = replay();
+            (void)hipEventRecord(done, main_stream());
+        } else {
+            st = forward_eager(m, true, done);
+        }
         const float host_ms = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - h0).count();
-        (void)hipEventRecord(m->ev1, stream());
+        if (!second)
+            return st;
         float ms = 0.f;
         if (st == TinyNN_SUCCESS && hipEventSynchronize(m->ev1) == hipSuccess &&
             hipEventElapsedTime(&ms, m->ev0, m->ev1) == hipSuccess) {
@@ -1050,7 +1105,7 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
         return st;
     };
     if (m->forwards <= 3 || (m->graph_exec && (m->forwards == 7 || m->forwards == 8)))
-        return timed(false, &m->eager_ms);
+        return timed(false, m->forwards == 3 || m->forwards == 8, &m->eager_ms);
     if (m->forwards == 4) {
         if (hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal) == hipSuccess) {
             TinyNNStatus st = forward_eager(m);
@@ -1070,16 +1125,11 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
         m->graph_state = -1;
         return forward_eager(m);
     }
-    TinyNNStatus st = timed(true, &m->graph_ms);
-    // (the shortest of four each: a single sample of a 0.12 ms forward is off by several percent, which
-    //  flipped the choice for batch-1 networks from run to run; a tie keeps the plain launches)
-    // Kernels that average under 6 us are launched faster than the host can enqueue them one by
-    // one once forwards follow each other without a pause (4.4 us per launch then, less into an empty
-    // queue, which is all a single timed forward sees): there a replay that is not slower wins.
-    if (m->forwards >= 10) {
-        const bool host_bound = m->eager_ms < 0.006f * (float)m->schedule.size();
-        m->graph_state = m->graph_ms < (host_bound ? 1.05f : 0.98f) * m->eager_ms ? 1 : -1;
-    }
+    TinyNNStatus st = timed(true, m->forwards == 6 || m->forwards == 10, &m->graph_ms);
+    // (the shorter of two pairs each: a single sample of a 0.12 ms forward is off by several percent,
+    //  which flipped the choice for batch-1 networks from run to run; a tie keeps the plain launches)
+    if (m->forwards >= 10)
+        m->graph_state = m->graph_ms < 0.98f * m->eager_ms ? 1 : -1;
     return st;
 }
 

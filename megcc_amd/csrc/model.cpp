@@ -291,7 +291,7 @@ static float time_oprs(Model* m, const std::vector<ModelOpr*>& ops, int iters) {
     return ok ? ms : -1.f;
 }
 
-static void build_schedule(Model* m) {
+static void build_schedule(Model* m, bool allow_pw_dw = true) {
     m->schedule.clear();
     const int n = (int)m->oprs.size();
     for (int i = 0; i < n; ++i)
@@ -365,7 +365,7 @@ static void build_schedule(Model* m) {
         // A pointwise convolution and the channel-wise 3x3 convolution of its result, on images small
         // enough for a workgroup to hold one: one kernel (megcc_gfx950_pw_dw) when nothing else reads
         // the tensor in between.
-        if (!options().no_fuse_pwdw && i + 1 < n && o0->desc.kind == MEGCC_KERN_CONV && o0->has_processed &&
+        if (allow_pw_dw && !options().no_fuse_pwdw && i + 1 < n && o0->desc.kind == MEGCC_KERN_CONV && o0->has_processed &&
             o0->out.size() == 1 && o0->in.size() == (o0->desc.attr.conv.with_bias ? 3u : 2u)) {
             ModelOpr* o1 = m->oprs[i + 1];
             if (o1->desc.kind == MEGCC_KERN_CONV && !o1->has_processed && o1->out.size() == 1 &&
@@ -483,7 +483,8 @@ static void build_schedule(Model* m) {
 
 // The tail stream, its events and workspace, and which head entries must wait for the previous
 // forward's tail (see Model::tail_begin). Leaves tail_begin at -1 when there is nothing to overlap.
-static void setup_tail(Model* m) {
+// `forced`: the boundary to use (a schedule index; finalize tries the neighbours of the balanced one).
+static void setup_tail(Model* m, int forced = -1) {
     m->tail_begin = -1;
     if (m->tail_opr_begin < 0)
         return;
@@ -496,6 +497,11 @@ static void setup_tail(Model* m) {
         }
     if (tb < 1 || tb >= n)
         return;
+    if (forced >= 0) {
+        if (forced < 1 || forced > n - 2)
+            return;
+        tb = forced;
+    } else
     // The boundary the memory plan was made for came from an estimate; with the kernels at hand each
     // entry is timed (a few launches on the tensors as they are; the estimate stands in for an entry
     // that reads a model input, which has no memory yet) and the tail is shortened until it takes no
@@ -575,6 +581,86 @@ static void join_tail(Model* m) {
         (void)hipStreamWaitEvent(main_stream(), m->ev_tail, 0);
         m->tail_pending = false;
     }
+}
+
+// Undoes setup_tail (the schedule is about to be rebuilt).
+static void reset_tail(Model* m) {
+    if (m->tail_stream) {
+        (void)hipStreamSynchronize(m->tail_stream);
+        unregister_aux_stream(m->tail_stream);
+        (void)hipStreamDestroy(m->tail_stream);
+        m->tail_stream = nullptr;
+    }
+    if (m->ev_head)
+        (void)hipEventDestroy(m->ev_head);
+    if (m->ev_tail)
+        (void)hipEventDestroy(m->ev_tail);
+    m->ev_head = m->ev_tail = nullptr;
+    if (m->tail_workspace)
+        m->dev.free(m->tail_workspace);
+    m->tail_workspace = nullptr;
+    for (auto* o : m->oprs)
+        o->ws.ptr = o->ws.size ? m->workspace : nullptr;
+    m->waits_tail.clear();
+    m->tail_writes.clear();
+    m->tail_reads_input = m->tail_pending = false;
+    m->tail_begin = -1;
+}
+
+// LITE_forward: one asynchronous kernel launch per Opr, in order, on the library stream; stops at
+// the first failing kernel like network.c:191-194. Results are visible after megcc_gfx950_wait().
+// `overlap`: the entries from tail_begin on go to the tail stream (plain launches of a model whose way
+// of launching is decided; never under capture or between timing events).
+// `done`: an event recorded behind the forward's last operator, on whichever stream that is.
+static TinyNNStatus forward_eager(Model* m, bool overlap = false, hipEvent_t done = nullptr) {
+    const int tb = overlap ? m->tail_begin : -1;
+    if (tb < 0)
+        join_tail(m);
+    TinyNNStatus st = TinyNN_SUCCESS;
+    for (int idx = 0; idx < (int)m->schedule.size() && st == TinyNN_SUCCESS; ++idx) {
+        ModelOpr* o = m->schedule[(size_t)idx];
+        if (idx == tb) {
+            (void)hipEventRecord(m->ev_head, main_stream());
+            (void)hipStreamWaitEvent(m->tail_stream, m->ev_head, 0);
+            set_stream_override(m->tail_stream, true);
+        } else if (idx < tb && m->tail_pending && m->waits_tail[(size_t)idx]) {
+            join_tail(m);
+        }
+        st = megcc_gfx950_call(
+                &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), o->out_ptrs.data(),
+                (int)o->out_ptrs.size(), &o->ws, &m->opt);
+    }
+    if (tb >= 0) {
+        set_stream_override(nullptr, false);
+        (void)hipEventRecord(m->ev_tail, m->tail_stream);
+        m->tail_pending = true;
+    }
+    if (done)
+        (void)hipEventRecord(done, tb >= 0 ? m->tail_stream : main_stream());
+    return st;
+}
+
+// Milliseconds per forward of six plain-launch forwards enqueued back to back, the way a finalized
+// model runs them (two streams where the schedule has a tail); negative when something fails.
+static float time_forwards(Model* m) {
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        if (e0)
+            (void)hipEventDestroy(e0);
+        return -1.f;
+    }
+    float ms = -1.f;
+    bool ok = forward_eager(m) == TinyNN_SUCCESS;
+    join_tail(m);
+    ok = ok && hipEventRecord(e0, main_stream()) == hipSuccess;
+    for (int i = 0; ok && i < 6; ++i)
+        ok = forward_eager(m, true) == TinyNN_SUCCESS;
+    join_tail(m);
+    ok = ok && hipEventRecord(e1, main_stream()) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+         hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return ok ? ms / 6 : -1.f;
 }
 
 }  // namespace
@@ -909,6 +995,53 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
     }
     build_schedule(m);
     setup_tail(m);
+    // The balance of measured kernel times is only a starting point: one kernel more or less on the
+    // tail moves MobileNetV1 batch 64 by 3 %. The boundary and its two neighbours are timed as whole
+    // forwards and the best one kept.
+    auto tune_tail = [&]() -> float {
+        if (m->tail_begin < 0)
+            return -1.f;
+        int best_tb = m->tail_begin;
+        float best = time_forwards(m);
+        for (int cand : {best_tb + 1, best_tb - 1}) {
+            reset_tail(m);
+            setup_tail(m, cand);
+            if (m->tail_begin != cand)
+                continue;
+            const float t = time_forwards(m);
+            if (t > 0.f && (best <= 0.f || t < best)) {
+                best = t;
+                best_tb = cand;
+            }
+        }
+        if (m->tail_begin != best_tb) {
+            reset_tail(m);
+            setup_tail(m, best_tb);
+        }
+        return best;
+    };
+    const float with = tune_tail();
+    // Pointwise -> depthwise pairs were judged one by one, kernel behind kernel on one stream. With
+    // two streams the launch floors they save are hidden anyway and their one-workgroup-per-image
+    // form fills the chip worse (MobileNetV1 batch 64: 248 k img/s with the pairs as one kernel, 263 k
+    // as two; batch 32 the other way round): the whole forward is timed both ways and the faster
+    // schedule kept.
+    bool has_pair = false;
+    for (const ModelOpr* o : m->schedule)
+        has_pair = has_pair || o->desc.kind == MEGCC_KERN_PW_DW;
+    if (with > 0.f && has_pair && !options().fuse_pwdw) {
+        const std::vector<ModelOpr*> fused_schedule = m->schedule;
+        const int fused_tb = m->tail_begin;
+        reset_tail(m);
+        build_schedule(m, false);
+        setup_tail(m);
+        const float without = tune_tail();
+        if (!(without > 0.f && without < 0.98f * with)) {
+            reset_tail(m);
+            m->schedule = fused_schedule;
+            setup_tail(m, fused_tb);
+        }
+    }
     m->finalized = true;
     return megcc_gfx950_wait();
 }
@@ -1013,39 +1146,6 @@ TinyNNStatus megcc_gfx950_model_get_output_async(void* model, int tensor, void* 
     hipError_t e = hipMemcpyAsync(host, t.ptr, bytes, hipMemcpyDeviceToHost, s);
     MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "model_get_output_async: %s", hipGetErrorString(e));
     return TinyNN_SUCCESS;
-}
-
-// LITE_forward: one asynchronous kernel launch per Opr, in order, on the library stream; stops at
-// the first failing kernel like network.c:191-194. Results are visible after megcc_gfx950_wait().
-// `overlap`: the entries from tail_begin on go to the tail stream (plain launches of a model whose way
-// of launching is decided; never under capture or between timing events).
-// `done`: an event recorded behind the forward's last operator, on whichever stream that is.
-static TinyNNStatus forward_eager(Model* m, bool overlap = false, hipEvent_t done = nullptr) {
-    const int tb = overlap ? m->tail_begin : -1;
-    if (tb < 0)
-        join_tail(m);
-    TinyNNStatus st = TinyNN_SUCCESS;
-    for (int idx = 0; idx < (int)m->schedule.size() && st == TinyNN_SUCCESS; ++idx) {
-        ModelOpr* o = m->schedule[(size_t)idx];
-        if (idx == tb) {
-            (void)hipEventRecord(m->ev_head, main_stream());
-            (void)hipStreamWaitEvent(m->tail_stream, m->ev_head, 0);
-            set_stream_override(m->tail_stream, true);
-        } else if (idx < tb && m->tail_pending && m->waits_tail[(size_t)idx]) {
-            join_tail(m);
-        }
-        st = megcc_gfx950_call(
-                &o->desc, o->in_ptrs.data(), (int)o->in_ptrs.size(), o->out_ptrs.data(),
-                (int)o->out_ptrs.size(), &o->ws, &m->opt);
-    }
-    if (tb >= 0) {
-        set_stream_override(nullptr, false);
-        (void)hipEventRecord(m->ev_tail, m->tail_stream);
-        m->tail_pending = true;
-    }
-    if (done)
-        (void)hipEventRecord(done, tb >= 0 ? m->tail_stream : main_stream());
-    return st;
 }
 
 TinyNNStatus megcc_gfx950_model_forward(void* model) {

@@ -254,8 +254,7 @@ static bool shares_bytes(const Tensor& a, const Tensor& b) {
     return a0 < b0 + bn && b0 < a0 + an;
 }
 // Milliseconds `iters` back-to-back rounds of the operators in `ops` take on the library stream
-// (after one untimed round), or a negative value when a launch fails or an operand has no memory
-// yet (a model input before set_input).
+// (after one untimed round), or a negative value when a launch fails or an operand has no memory.
 static float time_oprs(Model* m, const std::vector<ModelOpr*>& ops, int iters) {
     for (const ModelOpr* o : ops) {
         for (const Tensor* t : o->in_ptrs)
@@ -504,7 +503,7 @@ static void setup_tail(Model* m, int forced = -1) {
     } else
     // The boundary the memory plan was made for came from an estimate; with the kernels at hand each
     // entry is timed (a few launches on the tensors as they are; the estimate stands in for an entry
-    // that reads a model input, which has no memory yet) and the tail is shortened until it takes no
+    // that cannot be run) and the tail is shortened until it takes no
     // longer than the head: one fused pair too many on the tail costs MobileNetV1 batch 64 3 %.
     {
         std::vector<double> us((size_t)n);

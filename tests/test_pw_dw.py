@@ -232,8 +232,7 @@ def test_model_runtime_left_alone_keeps_whichever_form_it_measures_faster():
     m = runtime.Model()
     x0 = m.tensor("x0", pw.src_shape(), abi.QINT8, 0.03)
     m.mark_input(x0)
-    # (the pair's source is an arena tensor, like inside a network: a model input has no memory yet
-    #  when the runtime decides, and such a pair stays two kernels)
+    # (the pair's source is an arena tensor, like inside a network)
     pre = cases.MultiTypeCase(A.Q_RELU, pw.src_shape(), (0.03, 0.01, pw.scales[0]))
     x = m.tensor("x", pw.src_shape(), abi.QINT8, pw.scales[0])
     m.opr(pre.symbol(), [x0], [x])

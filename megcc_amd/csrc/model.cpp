@@ -1152,6 +1152,7 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
     MG_REQUIRE(m && m->finalized, TinyNN_ERROR_NULL_PTR, "model_forward: model not finalized");
     ++m->forwards;
     auto replay = [&]() -> TinyNNStatus {
+        join_tail(m);  // (a plain-launch forward before this one may have left its tail on the second stream)
         hipError_t e = hipGraphLaunch(m->graph_exec, stream());
         MG_REQUIRE(e == hipSuccess, TinyNN_ERROR_RUNTIME, "model_forward: graph launch: %s", hipGetErrorString(e));
         return TinyNN_SUCCESS;
@@ -1206,6 +1207,7 @@ TinyNNStatus megcc_gfx950_model_forward(void* model) {
     if (m->forwards <= 3 || (m->graph_exec && (m->forwards == 7 || m->forwards == 8)))
         return timed(false, m->forwards == 3 || m->forwards == 8, &m->eager_ms);
     if (m->forwards == 4) {
+        join_tail(m);  // (before the capture begins: the wait refers to an event outside of it)
         if (hipStreamBeginCapture(stream(), hipStreamCaptureModeThreadLocal) == hipSuccess) {
             TinyNNStatus st = forward_eager(m);
             hipGraph_t g = nullptr;

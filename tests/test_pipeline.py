@@ -140,3 +140,32 @@ def test_a_network_of_a_few_operators_keeps_one_stream():
         runtime.set_option("no_graph", 0)
     assert m.nr_kernel == 5 and m.nr_tail_kernel == 0
     m.close()
+
+
+def test_the_measuring_forwards_of_a_two_stream_model():
+    """default options: forwards 2 + 3 and 7 + 8 are plain launches on two streams, 4 captures a graph
+    (the tail of forward 3 still pending when the capture begins), 5 + 6 and 9 + 10 replay it, then the
+    faster way runs. Same bytes throughout."""
+    net = mobilenet.Net(BATCH)
+    images = [mobilenet.draw_input(BATCH, seed=s) for s in (11, 12)]
+    model, ids = build(net, False)
+    serial, _ = build(net, False, no_graph=1, nopipeline=1)
+    assert model.nr_tail_kernel >= 2
+    want = []
+    for img in images:
+        serial.set_input(ids["image"], img)
+        serial.forward()
+        want.append(serial.get(ids["softmax"]).copy())
+    model.set_input(ids["image"], images[0])
+    for k in range(1, 13):
+        model.forward()
+        if k >= 4 and k % 2 == 0:
+            np.testing.assert_array_equal(model.get(ids["softmax"]), want[0], err_msg="forward %d" % k)
+    assert model.launch_mode()[0] in (1, -1)
+    for img, w in zip(images[::-1], want[::-1]):
+        model.set_input(ids["image"], img)
+        model.forward()
+        model.forward()
+        np.testing.assert_array_equal(model.get(ids["softmax"]), w)
+    model.close()
+    serial.close()

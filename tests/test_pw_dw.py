@@ -309,3 +309,17 @@ def test_pair_is_one_kernel_only_when_its_result_shares_no_byte_with_its_source(
     assert nk == kernels
     for o in outs:
         assert np.array_equal(o, want)
+
+
+@pytest.mark.parametrize("w", range(4, 32))
+def test_every_row_width(w):
+    """the planes' pitch is the power of two above the width and a pixel group's window reaches one
+    dword past either end of a row: every width the entry point takes, both strides, odd heights"""
+    for stride, h in ((1, 3 + w % 4), (2, 2 + w % 5)):
+        cfg = (2, 128, 64, h, w, stride, A.RELU, A.IDENTITY, True, True, GENERIC if w & 1 else TIES)
+        pw, dw = pair_cases(*cfg)
+        a0, a1 = pw.gen(100 + w), dw.gen(200 + w)
+        _, want = oracle_pair(pw, dw, a0, a1)
+        st, got, ok = fused_call(pw, dw, a0, a1)
+        assert ok == 1 and st == abi.SUCCESS, runtime.lib().megcc_gfx950_last_error().decode()
+        assert np.array_equal(got, want), cfg

@@ -127,10 +127,10 @@ int root_of(const Model* m, int id) {
 // list estimated to take at most 55 % of the forward - the two streams should end up with about the
 // same amount of work, which is where back-to-back forwards gain most (MobileNetV1: the split falls
 // behind the 28 x 28 layers at every batch from 16 to 128); setup_tail() shortens it to the measured
-// balance - with a head of at least four operators, a tail of at least two, and at most 128 MB of
-// tensors in the tail (they get bytes of their own in the memory plan). The estimate is a launch
+// balance - with a head of at least four operators, a tail of at least two, and at most `own_cap`
+// bytes of tensors in the tail (they get bytes of their own in the memory plan). The estimate is a launch
 // floor plus the operator's tensors at half the memory bandwidth.
-static void choose_tail(Model* m) {
+static void choose_tail(Model* m, size_t own_cap) {
     m->tail_opr_begin = -1;
     if (options().no_pipeline)
         return;
@@ -161,7 +161,7 @@ static void choose_tail(Model* m) {
                     more += tensor_bytes(m->tensors[r]->t);
                 }
             }
-        if (own + more > (size_t)128 << 20)
+        if (own + more > own_cap)
             break;
         own += more;
         tail += us[(size_t)k - 1];
@@ -639,8 +639,9 @@ static TinyNNStatus forward_eager(Model* m, bool overlap = false, hipEvent_t don
     return st;
 }
 
-// Milliseconds per forward of six plain-launch forwards enqueued back to back, the way a finalized
-// model runs them (two streams where the schedule has a tail); negative when something fails.
+// Milliseconds per forward of eight plain-launch forwards enqueued back to back, the way a finalized
+// model runs them (two streams where the schedule has a tail) - the shorter of two such runs;
+// negative when something fails.
 static float time_forwards(Model* m) {
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
@@ -648,18 +649,23 @@ static float time_forwards(Model* m) {
             (void)hipEventDestroy(e0);
         return -1.f;
     }
-    float ms = -1.f;
+    float best = -1.f;
     bool ok = forward_eager(m) == TinyNN_SUCCESS;
-    join_tail(m);
-    ok = ok && hipEventRecord(e0, main_stream()) == hipSuccess;
-    for (int i = 0; ok && i < 6; ++i)
-        ok = forward_eager(m, true) == TinyNN_SUCCESS;
-    join_tail(m);
-    ok = ok && hipEventRecord(e1, main_stream()) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
-         hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+    for (int rep = 0; ok && rep < 2; ++rep) {
+        float ms = -1.f;
+        join_tail(m);
+        ok = hipEventRecord(e0, main_stream()) == hipSuccess;
+        for (int i = 0; ok && i < 8; ++i)
+            ok = forward_eager(m, true) == TinyNN_SUCCESS;
+        join_tail(m);
+        ok = ok && hipEventRecord(e1, main_stream()) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+             hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+        if (ok && (best < 0.f || ms / 8 < best))
+            best = ms / 8;
+    }
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
-    return ok ? ms / 6 : -1.f;
+    return ok ? best : -1.f;
 }
 
 }  // namespace
@@ -897,7 +903,13 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
     for (auto* t : m->tensors)
         if (t->is_input && t->def != 0)
             t->def = 0;
-    choose_tail(m);
+    // (planned twice: the arena of the operators as they are says how many bytes the tail's tensors
+    //  may get for themselves - 128 MB or 85 % of that arena, whichever is more: the balanced tail of a
+    //  MobileNetV1 needs about that at every batch, and more only cost cache reuse)
+    m->tail_opr_begin = -1;
+    MG_REQUIRE(plan_memory(m), TinyNN_ERROR_INVALID_LAYOUT,
+               "model_finalize: memory plan");
+    choose_tail(m, std::max((size_t)128 << 20, (size_t)(0.85 * (double)m->arena_bytes)));
     MG_REQUIRE(plan_memory(m), TinyNN_ERROR_INVALID_LAYOUT,
                "model_finalize: memory plan (alignment %zu)", (size_t)m->dev.alignment);
     m->arena = m->dev.malloc(m->arena_bytes ? m->arena_bytes : 1);
@@ -995,14 +1007,15 @@ TinyNNStatus megcc_gfx950_model_finalize(void* model) {
     build_schedule(m);
     setup_tail(m);
     // The balance of measured kernel times is only a starting point: one kernel more or less on the
-    // tail moves MobileNetV1 batch 64 by 3 %. The boundary and its two neighbours are timed as whole
-    // forwards and the best one kept.
+    // tail moves MobileNetV1 batch 64 by 3 %. The boundary and its three neighbours on either side are
+    // timed as whole forwards and the best one kept.
     auto tune_tail = [&]() -> float {
         if (m->tail_begin < 0)
             return -1.f;
         int best_tb = m->tail_begin;
         float best = time_forwards(m);
-        for (int cand : {best_tb + 1, best_tb - 1}) {
+        const int tb0 = best_tb;
+        for (int cand : {tb0 + 1, tb0 - 1, tb0 + 2, tb0 - 2, tb0 + 3, tb0 - 3}) {
             reset_tail(m);
             setup_tail(m, cand);
             if (m->tail_begin != cand)

@@ -169,3 +169,29 @@ def test_the_measuring_forwards_of_a_two_stream_model():
         np.testing.assert_array_equal(model.get(ids["softmax"]), w)
     model.close()
     serial.close()
+
+
+@pytest.mark.parametrize("planned", [False, True], ids=["own_plan", "reference_plan"])
+def test_two_hundred_overlapped_forwards(planned):
+    """three inputs in rotation, every result copied out asynchronously, the host waits once at the
+    end: each of the 200 results is the one of its input"""
+    net = mobilenet.Net(BATCH)
+    images = [mobilenet.draw_input(BATCH, seed=s) for s in (21, 22, 23)]
+    pipe, ids = build(net, planned, no_graph=1)
+    serial, _ = build(net, planned, no_graph=1, nopipeline=1)
+    assert pipe.nr_tail_kernel >= 2
+    want = []
+    for img in images:
+        serial.set_input(ids["image"], img)
+        serial.forward()
+        want.append(serial.get(ids["softmax"]).copy())
+    outs = [np.zeros((BATCH, 1000), np.float32) for _ in range(200)]
+    for k, out in enumerate(outs):
+        pipe.set_input(ids["image"], images[k % 3])
+        pipe.forward()
+        pipe.get_async(ids["softmax"], out)
+    runtime.wait()
+    bad = [k for k, out in enumerate(outs) if not np.array_equal(out, want[k % 3])]
+    assert not bad, bad[:10]
+    pipe.close()
+    serial.close()
